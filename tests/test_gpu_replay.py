@@ -1,0 +1,201 @@
+"""Replay on the GPU against the plain implementation: the same requests whole, with the last 32
+tokens decoded one by one, in portions of changing size, and mixed with other requests on so few
+pages that pages are used again; in float32 and in bfloat16."""
+
+from __future__ import annotations
+
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from tests.helpers import CONFIGS, make_folder, prompt
+from tests.plain.llama import PlainLlama
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LENGTHS = {"A": [5, 17, 33, 100], "B": [1, 40, 70, 129]}
+
+# float32 engine against the float64 oracle: only the engine's own 32-bit rounding separates them.
+# bfloat16 engine against the float64 oracle on bfloat16-rounded weights: activations are rounded
+# to 8 bits of mantissa a few dozen times on the way to a logit.
+TOL = {"float32": dict(atol=2e-5, rtol=1e-4), "bfloat16": dict(atol=3e-2, rtol=5e-2)}
+
+
+@pytest.fixture(scope="module", params=["A", "B"])
+def case(request, tmp_path_factory):
+    name = request.param
+    folder = make_folder(tmp_path_factory, name)
+    config = CONFIGS[name][0]
+    prompts = [prompt(100 + i, n, config.vocab_size) for i, n in enumerate(LENGTHS[name])]
+    oracles = {}
+    for dtype, stored in (("float32", None), ("bfloat16", torch.bfloat16)):
+        plain = PlainLlama(folder, torch.float64, weights_as=stored)
+        oracles[dtype] = [plain.logits(p) for p in prompts]
+    return name, folder, config, prompts, oracles
+
+
+def replayer(folder, dtype, max_tokens):
+    from tinyserve_llm_amd.engine.replay import Replay
+    return Replay(folder, dtype, max_tokens)
+
+
+def check(got: dict[tuple[int, int], torch.Tensor], oracle, dtype: str):
+    """got maps (request, position) to a logits row."""
+    assert got, "nothing was compared"
+    worst = 0.0
+    for (r, pos), row in got.items():
+        want = oracle[r][pos]
+        torch.testing.assert_close(row.double().cpu(), want, **TOL[dtype], msg=lambda m: f"request {r} position {pos}: {m}")
+        worst = max(worst, float((row.double().cpu() - want).abs().max()))
+    return worst
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_whole_requests_alone(case, dtype):
+    name, folder, config, prompts, oracles = case
+    rep = replayer(folder, dtype, 256)
+    got = {}
+    for r, p in enumerate(prompts):
+        logits = rep.step([{"id": f"r{r}", "tokens": p, "want": list(range(len(p)))}], [f"r{r}"])
+        assert logits.shape == (len(p), config.vocab_size) and logits.dtype == torch.float32
+        for pos in range(len(p)):
+            got[(r, pos)] = logits[pos]
+    check(got, oracles[dtype], dtype)
+    assert rep.manager.num_available_blocks() == rep.manager.num_blocks, "every page came back"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_last_32_tokens_one_by_one(case, dtype):
+    name, folder, config, prompts, oracles = case
+    rep = replayer(folder, dtype, 256)
+    got = {}
+    for r, p in enumerate(prompts):
+        head = max(0, len(p) - 32)
+        if head:
+            logits = rep.step([{"id": f"r{r}", "tokens": p[:head], "want": [head - 1]}], [])
+            got[(r, head - 1)] = logits[0]
+        for pos in range(head, len(p)):
+            logits = rep.step([{"id": f"r{r}", "tokens": [p[pos]], "want": [0]}], [f"r{r}"] if pos == len(p) - 1 else [])
+            got[(r, pos)] = logits[0]
+    check(got, oracles[dtype], dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_portions_of_changing_size(case, dtype):
+    name, folder, config, prompts, oracles = case
+    rep = replayer(folder, dtype, 256)
+    sizes = [2, 7, 3, 16, 2, 5, 31, 2, 64, 9]
+    got = {}
+    for r, p in enumerate(prompts):
+        pos, i = 0, r
+        while pos < len(p):
+            n = min(sizes[i % len(sizes)], len(p) - pos)
+            i += 1
+            want = sorted({0, n - 1})
+            logits = rep.step([{"id": f"r{r}", "tokens": p[pos:pos + n], "want": want}],
+                              [f"r{r}"] if pos + n == len(p) else [])
+            for j, w in enumerate(want):
+                got[(r, pos + w)] = logits[j]
+            pos += n
+    check(got, oracles[dtype], dtype)
+
+
+def mixed_schedule(prompts):
+    """Steps that keep up to four requests live: while one decodes token by token, others feed
+    portions. Returns a list of (entries, end) with entries (request, start, count, want)."""
+    cursors = [0] * len(prompts)
+    order = sorted(range(len(prompts)), key=lambda r: -len(prompts[r]))
+    chunk = [13, 2, 1, 7, 1, 1, 30, 1, 3, 1]
+    steps, tick = [], 0
+    while any(cursors[r] < len(prompts[r]) for r in order):
+        entries, end = [], []
+        for k, r in enumerate(order):
+            left = len(prompts[r]) - cursors[r]
+            if left == 0:
+                continue
+            if tick < 2 * k:            # staggered starts
+                continue
+            n = min(left, chunk[(tick + 3 * k) % len(chunk)])
+            entries.append((r, cursors[r], n, [n - 1] if n > 1 else [0]))
+            cursors[r] += n
+            if cursors[r] == len(prompts[r]):
+                end.append(r)
+        steps.append((entries, end))
+        tick += 1
+    return steps
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mixed_requests_on_few_pages(case, dtype):
+    """The pool holds exactly what the four requests need at once (each rounded up to pages of
+    64); a second round of the same requests then has to run on pages that were used before."""
+    name, folder, config, prompts, oracles = case
+    need = sum(-(-len(p) // 64) * 64 for p in prompts)
+    rep = replayer(folder, dtype, need)
+    assert rep.manager.num_blocks == need // 64
+    for round_ in range(2):
+        got = {}
+        for entries, end in mixed_schedule(prompts):
+            batch = [{"id": f"q{round_}_{r}", "tokens": prompts[r][s:s + n], "want": w} for r, s, n, w in entries]
+            logits = rep.step(batch, [f"q{round_}_{r}" for r in end])
+            row = 0
+            for r, s, n, w in entries:
+                for j in w:
+                    got[(r, s + j)] = logits[row]
+                    row += 1
+            assert row == logits.shape[0]
+        check(got, oracles[dtype], dtype)
+        assert rep.manager.num_available_blocks() == rep.manager.num_blocks
+
+
+def test_float32_logits_do_not_depend_on_the_cut(case):
+    """In float32 every kernel fixes the order of its sums per row, so logits are bit-equal
+    however the tokens were cut into steps and whatever else was in the batch."""
+    name, folder, config, prompts, oracles = case
+    rep = replayer(folder, "float32", 512)
+    p = prompts[-1]
+    whole = rep.step([{"id": "w", "tokens": p, "want": list(range(len(p)))}], ["w"])
+    other = prompts[-2]
+    pos, got = 0, []
+    rep.step([{"id": "o", "tokens": other[:3], "want": []}], [])
+    for n in [1, 2, 9, 1, 30, 64, 2, 1000]:
+        n = min(n, len(p) - pos)
+        if n == 0:
+            break
+        batch = [{"id": "c", "tokens": p[pos:pos + n], "want": list(range(n))}]
+        if pos % 2:
+            batch.insert(0, {"id": "o", "tokens": [other[3 + pos % 5]], "want": [0]})
+        logits = rep.step(batch, [])
+        got.append(logits[-n:])
+        pos += n
+    assert torch.equal(torch.cat(got), whole)
+
+
+def test_trace_run_program(case, tmp_path):
+    """bin/trace_run as a user runs it: JSON lines in, `done <step>` lines and .f32 files out."""
+    name, folder, config, prompts, oracles = case
+    p = prompts[2]
+    lines = [
+        {"step": 0, "entries": [{"id": "a", "tokens": p[:10], "want": [0, 9]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": p[10:12], "want": []}], "end": []},
+        {"step": 2, "entries": [{"id": "a", "tokens": p[12:], "want": [len(p) - 13]},
+                                {"id": "b", "tokens": prompts[1], "want": [len(prompts[1]) - 1]}], "end": ["a", "b"]},
+    ]
+    out = tmp_path / "out"
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
+                        "--out", str(out), "--max-tokens", "128"],
+                       input="\n".join(json.dumps(x) for x in lines) + "\n", capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr
+    assert r.stdout.split() == ["done", "0", "done", "1", "done", "2"]
+    assert not (out / "1.f32").exists()
+    s0 = np.fromfile(out / "0.f32", dtype="<f4").reshape(2, config.vocab_size)
+    s2 = np.fromfile(out / "2.f32", dtype="<f4").reshape(2, config.vocab_size)
+    got = {(2, 0): torch.from_numpy(s0[0]), (2, 9): torch.from_numpy(s0[1]),
+           (2, len(p) - 1): torch.from_numpy(s2[0]), (1, len(prompts[1]) - 1): torch.from_numpy(s2[1])}
+    check(got, oracles["float32"], "float32")

@@ -1,0 +1,105 @@
+"""Device memory of the cache: key and value pools in pages, grouped by what layers need, and the
+slots of fixed-size per-request state (tinyserve_llm/kvcache/storage.py:5-49 has one pool pair
+for all layers).
+
+Layers are grouped by the rows they cache (kv heads, head size) and by whether they keep every key
+or a window. A group's pools are laid out [pages, layers of the group, page_size, kv_heads,
+head_dim], page first, so one page of every layer of the group is one contiguous region. All
+full-history groups share page space 0: a page id addresses the pools of each of them. Every
+window group has a page space of its own.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from tinyserve_llm_amd.cache.manager import SpaceSpec
+from tinyserve_llm_amd.ops import hip
+from tinyserve_llm_amd.parts.base import KVSpec, StateSpec
+
+
+@dataclass
+class LayerGroup:
+    kv: KVSpec
+    space: int
+    owners: list[int]                 # run-order indices of the layer runs whose caches live here
+    k_pool: torch.Tensor              # [pages, len(owners), page_size, kv_heads, head_dim]
+    v_pool: torch.Tensor
+
+
+def plan_spaces(kv_specs: list[KVSpec]) -> tuple[list[tuple[KVSpec, int]], int]:
+    """Assigns each distinct KVSpec a page space: window 0 -> space 0, every window size a space of
+    its own. Returns ([(spec, space)], number of spaces)."""
+    distinct: list[KVSpec] = []
+    for kv in kv_specs:
+        if kv not in distinct:
+            distinct.append(kv)
+    windows = sorted({kv.window for kv in distinct if kv.window})
+    has_full = any(kv.window == 0 for kv in distinct)
+    base = 1 if has_full or not windows else 0
+    space_of_window = {w: base + i for i, w in enumerate(windows)}
+    return [(kv, 0 if kv.window == 0 else space_of_window[kv.window]) for kv in distinct], max(1, base + len(windows))
+
+
+def bytes_per_page(cache_plan, page_size: int, dtype: torch.dtype, space: int = 0) -> int:
+    """Bytes that one page id of `space` occupies over all layers (keys and values)."""
+    assigned, _ = plan_spaces([e.kv for e in cache_plan])
+    lookup = dict((kv, s) for kv, s in assigned)
+    return sum(2 * page_size * e.kv.num_kv_heads * e.kv.head_dim * dtype.itemsize
+               for e in cache_plan if lookup[e.kv] == space)
+
+
+class KVStorage:
+    def __init__(self, cache_plan, state_plan, num_pages: int | list[int], page_size: int, dtype: torch.dtype,
+                 device: torch.device | str, num_state_slots: int) -> None:
+        self.page_size = page_size
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.num_state_slots = num_state_slots
+        assigned, num_spaces = plan_spaces([e.kv for e in cache_plan])
+        pages = num_pages if isinstance(num_pages, (list, tuple)) else [num_pages] * num_spaces
+        if len(pages) != num_spaces:
+            raise ValueError(f"{num_spaces} page spaces but {len(pages)} page counts")
+        windows = [0] * num_spaces
+        for kv, s in assigned:
+            windows[s] = kv.window
+        self.spaces = [SpaceSpec(n, w) for n, w in zip(pages, windows)]
+        self.groups: list[LayerGroup] = []
+        self._where: dict[int, tuple[int, int]] = {}       # owner run -> (group, layer within group)
+        for kv, s in assigned:
+            owners = [e.owner for e in cache_plan if e.kv == kv]
+            shape = (pages[s], len(owners), page_size, kv.num_kv_heads, kv.head_dim)
+            group = LayerGroup(kv, s, owners, torch.zeros(shape, dtype=dtype, device=self.device),
+                               torch.zeros(shape, dtype=dtype, device=self.device))
+            for j, owner in enumerate(owners):
+                self._where[owner] = (len(self.groups), j)
+            self.groups.append(group)
+        self.states: dict[int, torch.Tensor] = {
+            e.run: torch.zeros((num_state_slots, *e.state.shape), dtype=e.state.dtype, device=self.device)
+            for e in state_plan}
+
+    def layer_cache(self, owner: int) -> tuple[torch.Tensor, torch.Tensor, int]:
+        """(k view, v view, page space) of the cache that run `owner` of the order owns; the views
+        are [pages, page_size, kv_heads, head_dim], strided over pages."""
+        g, j = self._where[owner]
+        group = self.groups[g]
+        return group.k_pool[:, j], group.v_pool[:, j], group.space
+
+    def state(self, run: int) -> torch.Tensor | None:
+        return self.states.get(run)
+
+    def copy_slots(self, space: int, src: int, dst: int, num_slots: int) -> None:
+        for group in self.groups:
+            if group.space == space:
+                hip.copy_slots(group.k_pool, src, dst, num_slots)
+                hip.copy_slots(group.v_pool, src, dst, num_slots)
+
+    def copy_state(self, src_slot: int, dst_slot: int) -> None:
+        for t in self.states.values():
+            t[dst_slot].copy_(t[src_slot])
+
+    def reset_state(self, slot: int) -> None:
+        for t in self.states.values():
+            t[slot].zero_()

@@ -1,0 +1,64 @@
+// Token choice from 32-bit logits, one block per row: the highest logit at temperature 0, else a
+// draw from softmax(logits / temperature) by the exponential race
+//     argmax_i  softmax_i / E_i   =   argmax_i  logit_i / t - log(E_i),   E_i ~ Exp(1), E_i >= 1e-10
+// (tinyserve_llm/engine/sampler.py:13-23). The noise of element i of a row comes from a counter
+// hash of (seed, the row's key, i), where the key names request, sample and output position: a
+// draw does not depend on the row's place in the batch. Ties go to the lowest index.
+#include "common.h"
+
+#define SAMPLE_THREADS 1024
+
+__device__ __forceinline__ uint64_t mix64(uint64_t x) {
+  x ^= x >> 30; x *= 0xBF58476D1CE4E5B9ull;
+  x ^= x >> 27; x *= 0x94D049BB133111EBull;
+  x ^= x >> 31;
+  return x;
+}
+
+__device__ __forceinline__ float exp1_noise(uint64_t seed, uint64_t key, uint32_t i) {
+  const uint64_t x = mix64(mix64(seed ^ (key * 0x9E3779B97F4A7C15ull)) + (uint64_t)i * 0xD1342543DE82EF95ull);
+  const float u = (float)((x >> 40) + 1) * (1.0f / 16777216.0f);  // (0, 1]
+  const float e = -logf(u);
+  return e < 1e-10f ? 1e-10f : e;
+}
+
+__device__ __forceinline__ bool better(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
+
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_kernel(int32_t* __restrict__ out, const float* __restrict__ logits, const float* __restrict__ temps,
+              const int64_t* __restrict__ keys, uint64_t seed, int vocab, int64_t ld) {
+  __shared__ float sv[SAMPLE_THREADS / TS_WAVE];
+  __shared__ int si[SAMPLE_THREADS / TS_WAVE];
+  const int r = blockIdx.x;
+  const float* row = logits + (int64_t)r * ld;
+  const float t = temps[r];
+  const uint64_t key = (uint64_t)keys[r];
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
+    float v = row[i];
+    if (t > 0.f) v = v / t - logf(exp1_noise(seed, key, (uint32_t)i));
+    if (better(v, i, bv, bi)) { bv = v; bi = i; }
+  }
+#pragma unroll
+  for (int off = TS_WAVE / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, TS_WAVE);
+    const int oi = __shfl_xor(bi, off, TS_WAVE);
+    if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+  }
+  if ((threadIdx.x & (TS_WAVE - 1)) == 0) { sv[threadIdx.x / TS_WAVE] = bv; si[threadIdx.x / TS_WAVE] = bi; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < SAMPLE_THREADS / TS_WAVE; ++w)
+      if (better(sv[w], si[w], bv, bi)) { bv = sv[w]; bi = si[w]; }
+    out[r] = bi == 0x7fffffff ? 0 : bi;
+  }
+}
+
+extern "C" int ts_sample(int32_t* out, const float* logits, const float* temps, const int64_t* keys,
+                         uint64_t seed, int rows, int vocab, int64_t ld, hipStream_t stream) {
+  if (rows <= 0) return TS_OK;
+  if (vocab <= 0 || ld < vocab) return TS_BAD_SHAPE;
+  sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(out, logits, temps, keys, seed, vocab, ld);
+  return ts_check_launch();
+}

@@ -1,0 +1,263 @@
+"""Python side of the HIP kernels: loads the library, checks every operand on the host, launches.
+
+Every function takes torch tensors that live on the GPU and launches on torch's current stream.
+There is no CPU path: a call with a CPU tensor, or without the library, raises. Operand shapes,
+strides and storage types are checked here, before a launch, because a kernel that reads out of
+bounds takes the GPU down with it.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import threading
+
+import torch
+
+from tinyserve_llm_amd.csrc import build as _build
+
+_lib = None
+_lock = threading.Lock()
+
+_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+_ERRORS = {1: "unsupported storage type", 2: "unsupported shape or stride", 3: "the kernel launch failed"}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def library() -> ctypes.CDLL:
+    """The kernel library; built on first use if no current build exists. Never a fallback."""
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                path = _build.find_current() or _build.build(force=True)
+                lib = ctypes.CDLL(path)
+                _declare(lib)
+                _lib = lib
+    return _lib
+
+
+def _declare(lib: ctypes.CDLL) -> None:
+    p, i, i64, f, u64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_uint64
+    sig = {
+        "ts_embedding": [p, p, p, i, i, i, p],
+        "ts_rmsnorm": [p, p, p, p, p, p, i, i, f, i, i, p],
+        "ts_rope_store": [p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i, p],
+        "ts_silu_mul": [p, p, i, i, i, p],
+        "ts_copy_slots": [p, i, i, i64, i, i, i, p],
+        "ts_paged_attention_wave": [p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i, f, i, i, p],
+        "ts_gemm_exact": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
+        "ts_sample": [p, p, p, p, u64, i, i, i64, p],
+    }
+    for name, args in sig.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = ctypes.c_int
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def _code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise KernelError(f"kernels exist for float32 and bfloat16, not {dtype}") from None
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _gpu(*tensors: torch.Tensor | None) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise KernelError("the HIP kernels take GPU tensors only; there is no CPU path")
+
+
+def _run(name: str, rc: int) -> None:
+    if rc:
+        raise KernelError(f"{name}: {_ERRORS.get(rc, rc)}")
+
+
+# ---------------------------------------------------------------------------------------------
+
+def embedding(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+    """out[t] = table[ids[t]]; ids int32 and already checked against the vocabulary on the host."""
+    _gpu(table, ids)
+    _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be contiguous [vocab, hidden]")
+    _need(ids.dtype == torch.int32 and ids.dim() == 1 and ids.is_contiguous(), "ids must be int32 [tokens]")
+    out = torch.empty((ids.shape[0], table.shape[1]), dtype=table.dtype, device=table.device)
+    _run("embedding", library().ts_embedding(_ptr(out), _ptr(table), _ptr(ids), ids.shape[0], table.shape[1],
+                                             _code(table.dtype), _stream()))
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.Tensor | None = None,
+            rows: torch.Tensor | None = None, want_residual: bool = True
+            ) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """(norm(x + residual) * weight, x + residual). With `rows` (int32) only those rows are
+    normalised, in that order, and no residual is returned."""
+    _gpu(x, weight, residual, rows)
+    _need(x.dim() == 2 and x.is_contiguous(), "rmsnorm input must be contiguous [rows, hidden]")
+    hidden = x.shape[1]
+    _need(weight.shape == (hidden,) and weight.is_contiguous(), "rmsnorm weight must be [hidden]")
+    if residual is not None:
+        _need(residual.shape == x.shape and residual.dtype == x.dtype and residual.is_contiguous(),
+              "residual must match the input")
+    n = x.shape[0]
+    if rows is not None:
+        _need(rows.dtype == torch.int32 and rows.dim() == 1 and rows.is_contiguous(), "rows must be int32")
+        n = rows.shape[0]
+    out = torch.empty((n, hidden), dtype=x.dtype, device=x.device)
+    res_out = None
+    if rows is None and want_residual:
+        res_out = x if residual is None else torch.empty_like(x)
+    write_res = res_out if (residual is not None and res_out is not None) else None
+    _run("rmsnorm", library().ts_rmsnorm(_ptr(out), _ptr(write_res), _ptr(x), _ptr(residual), _ptr(weight),
+                                         _ptr(rows), n, hidden, float(eps), _code(x.dtype), _code(weight.dtype),
+                                         _stream()))
+    return out, res_out
+
+
+def rope_store(qkv: torch.Tensor, cos_sin: torch.Tensor | None, positions: torch.Tensor,
+               slots: torch.Tensor | None, k_cache: torch.Tensor | None, v_cache: torch.Tensor | None,
+               num_heads: int, num_kv_heads: int, head_dim: int) -> torch.Tensor:
+    """Rotates q and k of `qkv` [tokens, (nh + 2 nkv) hd] by the table rows of `positions`, returns q
+    [tokens, nh, hd] and writes rotated k and v to the cache slots. `k_cache`/`v_cache` are one
+    layer's view [pages, page_size, nkv, hd] (may be strided over pages and slots); None = no write.
+    `cos_sin` None = no rotation."""
+    _gpu(qkv, cos_sin, positions, slots, k_cache, v_cache)
+    T = qkv.shape[0]
+    row = (num_heads + 2 * num_kv_heads) * head_dim
+    _need(qkv.dim() == 2 and qkv.shape[1] == row and qkv.is_contiguous(), f"qkv must be contiguous [tokens, {row}]")
+    _need(positions.dtype == torch.int32 and positions.shape == (T,) and positions.is_contiguous(),
+          "positions must be int32 [tokens]")
+    if cos_sin is not None:
+        _need(cos_sin.dtype == torch.float32 and cos_sin.dim() == 2 and cos_sin.shape[1] == head_dim
+              and cos_sin.is_contiguous(), "the rotation table must be float32 [positions, head_dim]")
+    page_size, page_stride, slot_stride = 1, 0, 0
+    if k_cache is not None:
+        _need(v_cache is not None and slots is not None, "a cache write needs k, v and the slots")
+        _need(slots.dtype == torch.int64 and slots.shape == (T,) and slots.is_contiguous(), "slots must be int64 [tokens]")
+        _check_cache(k_cache, v_cache, qkv.dtype, num_kv_heads, head_dim)
+        page_size, page_stride, slot_stride = k_cache.shape[1], k_cache.stride(0), k_cache.stride(1)
+    q = torch.empty((T, num_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
+    _run("rope_store", library().ts_rope_store(
+        _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(qkv), _ptr(cos_sin), _ptr(positions), _ptr(slots), T, num_heads,
+        num_kv_heads, head_dim, int(cos_sin is not None), page_size, page_stride, slot_stride, _code(qkv.dtype),
+        _stream()))
+    return q
+
+
+def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, dtype: torch.dtype, nkv: int, hd: int) -> None:
+    _need(k_cache.dim() == 4 and k_cache.shape[2] == nkv and k_cache.shape[3] == hd,
+          f"cache view must be [pages, page_size, {nkv}, {hd}], got {tuple(k_cache.shape)}")
+    _need(k_cache.dtype == dtype and v_cache.dtype == dtype, "cache and activations differ in storage type")
+    _need(k_cache.shape == v_cache.shape and k_cache.stride() == v_cache.stride(), "k and v caches must be laid out alike")
+    _need(k_cache.stride(3) == 1 and k_cache.stride(2) == hd, "a token's heads must be contiguous in the cache")
+    _need(k_cache.stride(1) >= nkv * hd and k_cache.stride(0) >= k_cache.shape[1] * k_cache.stride(1),
+          "cache slots overlap")
+
+
+def paged_attention_wave(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                         block_tables: torch.Tensor, seq_of_token: torch.Tensor, positions: torch.Tensor,
+                         scale: float, window: int = 0) -> torch.Tensor:
+    """Attention of each token (at its position, causal, optionally windowed) over the cache
+    pages that its request's row of `block_tables` names."""
+    _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions)
+    _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
+    T, nh, hd = q.shape
+    nkv = k_cache.shape[2]
+    _check_cache(k_cache, v_cache, q.dtype, nkv, hd)
+    _need(hd % 16 == 0 and hd <= 256, f"head_dim {hd} is not a multiple of 16 up to 256")
+    _need(nh % nkv == 0, f"{nh} heads do not divide into {nkv} key/value heads")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
+          "block_tables must be contiguous int32 [requests, pages]")
+    for name, t in (("seq_of_token", seq_of_token), ("positions", positions)):
+        _need(t.dtype == torch.int32 and t.shape == (T,) and t.is_contiguous(), f"{name} must be int32 [tokens]")
+    out = torch.empty_like(q)
+    _run("paged_attention_wave", library().ts_paged_attention_wave(
+        _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_of_token), _ptr(positions),
+        T, nh, nkv, hd, k_cache.shape[1], k_cache.stride(0), k_cache.stride(1), block_tables.shape[1], float(scale),
+        int(window), _code(q.dtype), _stream()))
+    return out
+
+
+def gemm_exact(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """a [M, K] · w [N, K]^T with 32-bit multiply-adds in ascending k."""
+    _gpu(a, w)
+    _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], f"shapes {tuple(a.shape)} x {tuple(w.shape)}^T")
+    _need(a.dtype == w.dtype, "activations and weights differ in storage type")
+    _need(a.stride(1) == 1 and w.stride(1) == 1, "rows must be contiguous")
+    out_dtype = out_dtype or a.dtype
+    out = torch.empty((a.shape[0], w.shape[0]), dtype=out_dtype, device=a.device)
+    _run("gemm_exact", library().ts_gemm_exact(_ptr(out), _ptr(a), _ptr(w), a.shape[0], w.shape[0], a.shape[1],
+                                               a.stride(0), w.stride(0), out.stride(0), _code(a.dtype),
+                                               _code(out_dtype), _stream()))
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    """silu(gate) * up for rows laid out [gate | up]."""
+    _gpu(gate_up)
+    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0 and gate_up.is_contiguous(),
+          "gate_up must be contiguous [tokens, 2 * intermediate]")
+    inter = gate_up.shape[1] // 2
+    out = torch.empty((gate_up.shape[0], inter), dtype=gate_up.dtype, device=gate_up.device)
+    _run("silu_mul", library().ts_silu_mul(_ptr(out), _ptr(gate_up), gate_up.shape[0], inter, _code(gate_up.dtype),
+                                           _stream()))
+    return out
+
+
+def copy_slots(pool: torch.Tensor, src: int, dst: int, num_slots: int) -> None:
+    """pool[dst, :, :num_slots] = pool[src, :, :num_slots] for a contiguous pool
+    [pages, layers, page_size, kv_heads, head_dim]."""
+    _gpu(pool)
+    _need(pool.dim() == 5 and pool.is_contiguous(), "pool must be contiguous [pages, layers, page_size, heads, dim]")
+    pages, layers, page_size = pool.shape[:3]
+    _need(0 <= src < pages and 0 <= dst < pages and src != dst, f"pages {src}->{dst} outside 0..{pages - 1}")
+    _need(0 <= num_slots <= page_size, f"{num_slots} slots do not fit a page of {page_size}")
+    row_bytes = pool.shape[3] * pool.shape[4] * pool.element_size()
+    _run("copy_slots", library().ts_copy_slots(_ptr(pool), layers, page_size, row_bytes, src, dst, num_slots, _stream()))
+
+
+def sample(logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor, seed: int) -> torch.Tensor:
+    """One token per row of float32 `logits`: argmax where the temperature is 0, else a draw whose
+    noise is a function of (seed, keys[row], vocabulary index) alone."""
+    _gpu(logits, temperatures, keys)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.stride(1) == 1, "logits must be float32 [rows, vocab]")
+    R = logits.shape[0]
+    _need(temperatures.dtype == torch.float32 and temperatures.shape == (R,) and temperatures.is_contiguous(),
+          "temperatures must be float32 [rows]")
+    _need(keys.dtype == torch.int64 and keys.shape == (R,) and keys.is_contiguous(), "keys must be int64 [rows]")
+    out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    _run("sample", library().ts_sample(_ptr(out), _ptr(logits), _ptr(temperatures), _ptr(keys),
+                                       seed & 0xFFFFFFFFFFFFFFFF, R, logits.shape[1], logits.stride(0), _stream()))
+    return out
+
+
+# ---- dispatchers ---------------------------------------------------------------------------------
+
+def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx, space: int,
+                    scale: float, window: int = 0) -> torch.Tensor:
+    """Attention of a packed step over the cache; picks the kernel for the storage type and shape."""
+    return paged_attention_wave(q, k_cache, v_cache, ctx.block_tables[space], ctx.seq_of_token, ctx.positions,
+                                scale, window)
+
+
+def linear_bf16(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """bfloat16 x [M, K] · weight [N, K]^T through the vendor matrix library."""
+    _gpu(x, weight)
+    _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "linear_bf16 takes bfloat16")
+    _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
+          f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
+    return torch.matmul(x, weight.t())

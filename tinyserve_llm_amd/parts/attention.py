@@ -1,0 +1,58 @@
+"""Grouped-query attention over the paged cache (tinyserve_llm/model/llama.py:189-212,
+tinyserve_llm/engine/model_runner.py:100-108, tinyserve_llm/attention/torch_paged.py:15-46).
+
+One fused projection gives q | k | v; q and k are rotated by the named position encoding; k and v
+of the step's tokens are written to their cache slots; then every token attends, causally, over
+the cache pages of its request (its own key included), and the output projection follows.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from tinyserve_llm_amd.ops import hip
+from tinyserve_llm_amd.parts.base import KVSpec, LayerMemory, Mixer, ParamSpec, StepContext, register
+from tinyserve_llm_amd.parts.linear import linear
+
+
+@register("mixer", "attention")
+class Attention(Mixer):
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 position: str | None = "rope", scale: float | None = None, window: int = 0) -> None:
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads do not divide into {num_kv_heads} key/value heads")
+        if head_dim % 16 or head_dim > 256:
+            raise ValueError(f"head_dim {head_dim}: the attention kernels take multiples of 16 up to 256")
+        self.hidden_size = hidden_size
+        self.num_heads = num_heads
+        self.num_kv_heads = num_kv_heads
+        self.head_dim = head_dim
+        self.position = position
+        self.scale = scale if scale is not None else head_dim ** -0.5
+        self.window = window
+        self.qkv: torch.Tensor | None = None
+        self.o: torch.Tensor | None = None
+
+    @property
+    def q_size(self) -> int:
+        return self.num_heads * self.head_dim
+
+    @property
+    def kv_size(self) -> int:
+        return self.num_kv_heads * self.head_dim
+
+    def param_specs(self) -> dict[str, ParamSpec]:
+        return {"qkv": ParamSpec((self.q_size + 2 * self.kv_size, self.hidden_size)),
+                "o": ParamSpec((self.hidden_size, self.q_size))}
+
+    def kv_spec(self) -> KVSpec:
+        return KVSpec(self.num_kv_heads, self.head_dim, self.window)
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, mem: LayerMemory) -> torch.Tensor:
+        qkv = linear(x, self.qkv)
+        table = ctx.position_encodings[self.position].rotary_table() if self.position else None
+        q = hip.rope_store(qkv, table, ctx.positions, ctx.slot_mapping[mem.space] if mem.store else None,
+                           mem.k_cache if mem.store else None, mem.v_cache if mem.store else None,
+                           self.num_heads, self.num_kv_heads, self.head_dim)
+        o = hip.paged_attention(q, mem.k_cache, mem.v_cache, ctx, mem.space, self.scale, self.window)
+        return linear(o.view(ctx.num_tokens, self.q_size), self.o)

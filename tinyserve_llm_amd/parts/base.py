@@ -1,0 +1,176 @@
+"""What a part of a layer is, and the registries that a configuration picks parts from.
+
+A layer is assembled from four parts (a mixer, a feed-forward, two norms) in an arrangement
+(a block); position encodings are shared parts that mixers refer to by name. Each part is built
+from explicit sizes and constants, declares the parameters it needs, receives them once, and then
+works on flat batches of tokens. No part knows which model or which layer it is in.
+
+The reference passes its config object into attention and decoder layer
+(tinyserve_llm/model/llama.py:191,230) and hands attention an injected backend
+(tinyserve_llm/model/attention.py:13-26); here the seam is wider: every kind of part sits behind an
+interface and a name, so that one model may use different mixers and feed-forwards layer by layer.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable
+
+import torch
+
+
+# ---- declarations ---------------------------------------------------------------------------
+
+@dataclass(frozen=True)
+class ParamSpec:
+    """One parameter of a part. `storage`: "compute" = the engine's dtype (bfloat16 or float32),
+    "float32" = kept in 32-bit whatever the engine's dtype, "int32" = an integer table.
+    `init` = (mean, std) of the normal distribution that the random-weights mode draws from."""
+
+    shape: tuple[int, ...]
+    storage: str = "compute"
+    init: tuple[float, float] = (0.0, 0.02)
+
+
+@dataclass(frozen=True)
+class KVSpec:
+    """A mixer that caches a key and a value row per token. `window` 0 = every key is kept;
+    W > 0 = only the last W positions are ever read, so older pages can be given back."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: int = 0
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """Fixed-size state that a mixer keeps per request (one slot per live request)."""
+
+    shape: tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class LayerMemory:
+    """What one run of a layer may touch of the engine's memory."""
+
+    k_cache: torch.Tensor | None = None   # [pages, page_size, kv_heads, head_dim] view of this run's cache
+    v_cache: torch.Tensor | None = None
+    space: int = 0                        # which page space's block tables and slots address it
+    store: bool = True                    # False: read another run's cache, write nothing
+    state: torch.Tensor | None = None     # [slots, *StateSpec.shape]
+
+
+@dataclass
+class StepContext:
+    """One step's batch, packed: tokens of several requests back to back, portions of prompts
+    beside single decoded tokens. Index tensors live on the device; the lists mirror them on the
+    host. `slot_mapping[s]` and `block_tables[s]` belong to page space s."""
+
+    num_tokens: int
+    num_seqs: int
+    token_ids: torch.Tensor               # [T] int32
+    positions: torch.Tensor               # [T] int32, absolute position of each token in its request
+    seq_of_token: torch.Tensor            # [T] int32, row of the batch each token belongs to
+    cu_seqlens: torch.Tensor              # [S+1] int32
+    context_lens: torch.Tensor            # [S] int32, keys of each request after this step's writes
+    state_slots: torch.Tensor             # [S] int32
+    slot_mapping: list[torch.Tensor]      # per space: [T] int64, page * page_size + offset
+    block_tables: list[torch.Tensor]      # per space: [S, max_pages] int32
+    host_cu_seqlens: list[int] = field(default_factory=list)
+    host_starts: list[int] = field(default_factory=list)      # first position fed, per request
+    host_context_lens: list[int] = field(default_factory=list)
+    host_state_slots: list[int] = field(default_factory=list)
+    position_encodings: dict[str, "PositionEncoding"] = field(default_factory=dict)
+
+    @property
+    def max_query_len(self) -> int:
+        c = self.host_cu_seqlens
+        return max((b - a for a, b in zip(c, c[1:])), default=0)
+
+
+# ---- interfaces -----------------------------------------------------------------------------
+
+class Part:
+    """Base of every part: declares parameters, receives them."""
+
+    def param_specs(self) -> dict[str, ParamSpec]:
+        return {}
+
+    def bind(self, params: dict[str, torch.Tensor]) -> None:
+        for name, tensor in params.items():
+            setattr(self, name, tensor)
+
+
+class Norm(Part):
+    def __call__(self, x: torch.Tensor, residual: torch.Tensor | None = None,
+                 rows: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor | None]:
+        """(normalised(x + residual), x + residual); `rows` restricts the output to some rows."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def prepare(self, device: torch.device) -> None:
+        """Build tables on the device (called once, after bind)."""
+
+    def rotary_table(self) -> torch.Tensor | None:
+        """float32 [positions, head_dim] = [cos | sin] for rotate-half mixers, or None."""
+        return None
+
+    def on_embedding(self, hidden: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        """Hook for encodings that act on the embedded tokens."""
+        return hidden
+
+
+class Mixer(Part):
+    def kv_spec(self) -> KVSpec | None:
+        return None
+
+    def state_spec(self) -> StateSpec | None:
+        return None
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, mem: LayerMemory) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+
+# ---- registries -----------------------------------------------------------------------------
+
+MIXERS: dict[str, Callable[..., Mixer]] = {}
+FEED_FORWARDS: dict[str, Callable[..., FeedForward]] = {}
+NORMS: dict[str, Callable[..., Norm]] = {}
+POSITION_ENCODINGS: dict[str, Callable[..., PositionEncoding]] = {}
+BLOCKS: dict[str, Callable[..., Any]] = {}
+
+_TABLES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS,
+           "position_encoding": POSITION_ENCODINGS, "block": BLOCKS}
+
+
+def register(family: str, name: str) -> Callable:
+    """`@register("mixer", "my_mixer")` above a class (or, for blocks, a function)."""
+    table = _TABLES[family]
+
+    def deco(obj):
+        table[name] = obj
+        return obj
+
+    return deco
+
+
+@dataclass(frozen=True)
+class PartSpec:
+    """A part chosen by name with its constructor arguments (sizes and constants only)."""
+
+    kind: str
+    args: dict[str, Any] = field(default_factory=dict)
+
+
+def make(family: str, spec: PartSpec):
+    table = _TABLES[family]
+    if spec.kind not in table:
+        raise KeyError(f"no {family} named {spec.kind!r}; registered: {sorted(table)}")
+    return table[spec.kind](**spec.args)

@@ -1,0 +1,28 @@
+"""SiLU-gated feed-forward (tinyserve_llm/model/llama.py:77-83,215-225): one fused projection gives
+[gate | up], then silu(gate) * up, then the down projection."""
+
+from __future__ import annotations
+
+import torch
+
+from tinyserve_llm_amd.ops import hip
+from tinyserve_llm_amd.parts.base import FeedForward, ParamSpec, StepContext, register
+from tinyserve_llm_amd.parts.linear import linear
+
+
+@register("feed_forward", "gated_mlp")
+class GatedMLP(FeedForward):
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu") -> None:
+        if activation != "silu":
+            raise ValueError(f"activation {activation!r}: the gated feed-forward kernel computes silu")
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.gate_up: torch.Tensor | None = None
+        self.down: torch.Tensor | None = None
+
+    def param_specs(self) -> dict[str, ParamSpec]:
+        return {"gate_up": ParamSpec((2 * self.intermediate_size, self.hidden_size)),
+                "down": ParamSpec((self.hidden_size, self.intermediate_size))}
+
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        return linear(hip.silu_mul(linear(x, self.gate_up)), self.down)

@@ -1,0 +1,27 @@
+"""RMSNorm with the residual add folded in (tinyserve_llm/model/llama.py:39-74).
+
+`norm(x, residual)` returns (normalise(x + residual) * weight, x + residual): the sum, its mean
+square, the rsqrt and the scaling are 32-bit; the returned residual is the sum rounded to the
+storage type, while the normalisation uses the unrounded sum (llama.py:63-67).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from tinyserve_llm_amd.ops import hip
+from tinyserve_llm_amd.parts.base import Norm, ParamSpec, register
+
+
+@register("norm", "rmsnorm")
+class RMSNorm(Norm):
+    def __init__(self, hidden_size: int, eps: float) -> None:
+        self.hidden_size = hidden_size
+        self.eps = eps
+        self.weight: torch.Tensor | None = None
+
+    def param_specs(self) -> dict[str, ParamSpec]:
+        return {"weight": ParamSpec((self.hidden_size,), init=(1.0, 0.1))}
+
+    def __call__(self, x, residual=None, rows=None):
+        return hip.rmsnorm(x, self.weight, self.eps, residual, rows)
