@@ -24,7 +24,7 @@ LENGTHS = {"A": [5, 17, 33, 100], "B": [1, 40, 70, 129]}
 # float32 engine against the float64 oracle: only the engine's own 32-bit rounding separates them.
 # bfloat16 engine against the float64 oracle on bfloat16-rounded weights: activations are rounded
 # to 8 bits of mantissa a few dozen times on the way to a logit.
-TOL = {"float32": dict(atol=2e-5, rtol=1e-4), "bfloat16": dict(atol=3e-2, rtol=5e-2)}
+TOL = {"float32": dict(atol=5e-6, rtol=1e-5), "bfloat16": dict(atol=1.5e-2, rtol=2e-2)}
 
 
 @pytest.fixture(scope="module", params=["A", "B"])
@@ -53,6 +53,7 @@ def check(got: dict[tuple[int, int], torch.Tensor], oracle, dtype: str):
         want = oracle[r][pos]
         torch.testing.assert_close(row.double().cpu(), want, **TOL[dtype], msg=lambda m: f"request {r} position {pos}: {m}")
         worst = max(worst, float((row.double().cpu() - want).abs().max()))
+    print(f"[{dtype}] worst absolute logit error {worst:.3e} over {len(got)} rows")
     return worst
 
 
@@ -189,7 +190,7 @@ def test_trace_run_program(case, tmp_path):
     ]
     out = tmp_path / "out"
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
-                        "--out", str(out), "--max-tokens", "128"],
+                        "--out", str(out), "--max-tokens", str(-(-len(p) // 64) * 64 + -(-len(prompts[1]) // 64) * 64)],
                        input="\n".join(json.dumps(x) for x in lines) + "\n", capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stderr
     assert r.stdout.split() == ["done", "0", "done", "1", "done", "2"]

@@ -1,0 +1,313 @@
+"""The scheduler: admits requests by cache hit and age, cuts prompts into portions under a token
+budget, decodes, forks parallel samples, finishes and frees, and preempts when pages run out
+(tinyserve_llm/scheduler/scheduler.py:12-267). It is host code and talks to the cache manager only.
+
+Beyond the reference: a prompt need not fit one step. An admission feeds the first portion of the
+uncached tokens (as much as the step's budget and `max_prefill_chunk` allow); a sequence that is
+still inside its prompt feeds the next portion each step, after the decodes and before new
+admissions; only the final portion yields a token.
+
+When pages run out: a running sequence that cannot get the page it needs makes the lowest-ranked
+sequences not yet scheduled in this step give up theirs (preemption: pages released, which keeps
+them in the prefix cache while nobody else needs them; the sequence returns to the waiting queue
+with its outputs and its arrival time); if none is left it gives up its own and this kind of
+scheduling stops for the step.
+"""
+
+from __future__ import annotations
+
+import itertools
+import math
+from dataclasses import dataclass, replace
+from typing import Literal, NamedTuple
+
+from tinyserve_llm_amd.cache.manager import AdmissionCost, KVCacheManager
+from tinyserve_llm_amd.engine.sequence import SamplingParams, Sequence, SequenceStatus
+
+
+@dataclass(frozen=True)
+class SchedulerConfig:
+    max_model_len: int = 4096
+    max_num_seqs: int = 512
+    max_num_batched_tokens: int = 16384
+    eos_token_id: int = -1
+    wait_weight: float = 0.1            # score = hit + wait_weight * seconds waited
+    hit_mode: Literal["absolute", "ratio"] = "absolute"
+    max_skip_wait: float = 5.0          # a misfit that waited this long stops admission behind it
+    watermark: float = 0.01             # fraction of pages kept free at admission
+    step_mode: Literal["mixed", "prefill_first"] = "mixed"
+    max_prefill_chunk: int = 0          # most prompt tokens of one sequence per step; 0 = the budget
+
+    def __post_init__(self) -> None:
+        # every running sequence decodes first; one more token must remain for a prompt portion
+        assert self.max_num_batched_tokens >= self.max_num_seqs + 1, \
+            "the token budget could be used up by decodes alone"
+        assert self.max_prefill_chunk >= 0
+
+
+@dataclass
+class SchedulerStats:
+    admissions: int = 0
+    readmissions: int = 0
+    preemptions: int = 0
+    cached_tokens: int = 0
+    prefill_tokens: int = 0
+    decode_tokens: int = 0
+    num_waiting: int = 0
+    num_running: int = 0
+
+
+class ScheduledSeq(NamedTuple):
+    seq: Sequence
+    token_ids: list[int]      # fed this step, at positions start .. start + len - 1
+    num_samples: int = 1      # 0 for a portion that does not end the prompt; n on a group's first token
+    start: int = 0
+
+
+class RequestOutput(NamedTuple):
+    request_id: int
+    sequences: list[Sequence]
+
+
+class Scheduler:
+    def __init__(self, config: SchedulerConfig, kv: KVCacheManager) -> None:
+        self.config = config
+        self.kv = kv
+        self.waiting: list[Sequence] = []
+        self.running: list[Sequence] = []
+        self.groups: dict[int, list[Sequence]] = {}
+        self.watermark_blocks = math.ceil(config.watermark * kv.num_blocks)
+        self._seq_ids = itertools.count()
+        self._request_ids = itertools.count()
+        self.counters = SchedulerStats()
+
+    def has_unfinished(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    # ---- arrival ----------------------------------------------------------------------------
+    def add_request(self, prompt_token_ids: list[int], params: SamplingParams, arrival_time: float) -> int:
+        """Queues a request; refuses one that could never run (scheduler.py:67-87)."""
+        assert prompt_token_ids and params.max_tokens >= 1 and params.n >= 1
+        longest = len(prompt_token_ids) + params.max_tokens
+        if longest > self.config.max_model_len:
+            raise ValueError(f"prompt + max_tokens = {longest} exceeds max_model_len")
+        # one sequence at full length, a page per further sample, the watermark, and one page for
+        # the source of a partial-page copy that must exist beside its destination
+        worst = -(-longest // self.kv.block_size) + (params.n - 1) + self.watermark_blocks + 1
+        if worst > self.kv.num_blocks:
+            raise ValueError(f"needs up to {worst} blocks; the KV cache has {self.kv.num_blocks}")
+        if params.n > self.config.max_num_seqs:
+            raise ValueError(f"n = {params.n} samples exceed max_num_seqs")
+        request_id = next(self._request_ids)
+        seq = Sequence(next(self._seq_ids), request_id, tuple(prompt_token_ids), params, arrival_time)
+        self.groups[request_id] = [seq]
+        self.waiting.append(seq)
+        return request_id
+
+    # ---- ranking ----------------------------------------------------------------------------
+    def _hit(self, num_tokens: int, cost: AdmissionCost) -> float:
+        cached = num_tokens - cost.prefill_tokens
+        return cached / (self.config.max_model_len if self.config.hit_mode == "absolute" else num_tokens)
+
+    def _score(self, hit: float, seq: Sequence, now: float) -> float:
+        return hit + self.config.wait_weight * (now - seq.arrival_time)
+
+    def _ranked_waiting(self, now: float) -> list[tuple[Sequence, float]]:
+        ranked = []
+        for seq in self.waiting:
+            tokens = seq.all_token_ids
+            hit = self._hit(len(tokens), self.kv.calculate_admission_cost(tokens))
+            ranked.append((self._score(hit, seq, now), seq))
+        ranked.sort(key=lambda r: r[0], reverse=True)
+        return [(seq, score) for score, seq in ranked]
+
+    def _chunk(self, left: int, budget: int) -> int:
+        cap = self.config.max_prefill_chunk or budget
+        return max(0, min(left, budget, cap))
+
+    # ---- one step ---------------------------------------------------------------------------
+    def schedule(self, now: float) -> list[ScheduledSeq]:
+        budget = self.config.max_num_batched_tokens
+        if self.config.step_mode == "prefill_first":
+            prompts = self._schedule_running(now, budget, want_prefill=True)
+            prompts += self._admit(now, budget - sum(len(s.token_ids) for s in prompts))
+            return prompts or self._schedule_running(now, budget, want_prefill=False)
+        decodes = self._schedule_running(now, budget, want_prefill=False)
+        budget -= len(decodes)
+        portions = self._schedule_running(now, budget, want_prefill=True)
+        budget -= sum(len(s.token_ids) for s in portions)
+        return decodes + portions + self._admit(now, budget)
+
+    def _schedule_running(self, now: float, budget: int, want_prefill: bool) -> list[ScheduledSeq]:
+        """Feeds running sequences of one kind (inside their prompt, or decoding), best score
+        first. Victims of a page shortage are the lowest-ranked sequences of either kind that
+        this step has not scheduled."""
+        mine = [s for s in self.running if s.in_prefill == want_prefill and not s.in_step]
+        mine.sort(key=lambda s: self._score(s.admission_hit, s, now))       # lowest first
+        scheduled: list[ScheduledSeq] = []
+        gone: set[int] = set()
+        while mine:
+            seq = mine.pop()
+            if want_prefill:
+                n = self._chunk(seq.prefill_target - seq.num_computed, budget)
+                if n == 0:
+                    continue                       # no budget left for it this step; it keeps its pages
+                tokens = seq.all_token_ids[seq.num_computed:seq.num_computed + n]
+            else:
+                if budget <= 0:
+                    continue
+                tokens = [seq.pending_token]
+            while not self.kv.can_append(seq.seq_id, len(tokens)):
+                victim = self._lowest_unscheduled(now, exclude=seq, gone=gone)
+                if victim is None:
+                    break
+                self._preempt(victim)
+                gone.add(victim.seq_id)
+                if victim in mine:
+                    mine.remove(victim)
+            if not self.kv.can_append(seq.seq_id, len(tokens)):
+                self._preempt(seq)
+                gone.add(seq.seq_id)
+                break
+            self.kv.append_slots(seq.seq_id, tokens)
+            final = seq.num_computed + len(tokens) >= seq.prefill_target
+            samples = 1
+            if want_prefill:
+                samples = 0 if not final else (seq.params.n if self._first_of_group(seq) else 1)
+                self.counters.prefill_tokens += len(tokens)
+            else:
+                self.counters.decode_tokens += 1
+            seq.in_step = True
+            scheduled.append(ScheduledSeq(seq, tokens, samples, seq.num_computed))
+            budget -= len(tokens)
+        return scheduled
+
+    def _lowest_unscheduled(self, now: float, exclude: Sequence, gone: set[int]) -> Sequence | None:
+        pool = [s for s in self.running if s is not exclude and s.seq_id not in gone
+                and not s.in_step]
+        return min(pool, key=lambda s: self._score(s.admission_hit, s, now), default=None)
+
+    def _preempt(self, seq: Sequence) -> None:
+        """Pages go back (staying in the prefix cache while nobody needs them); the sequence
+        waits again with its outputs and its original arrival time (scheduler.py:152-158)."""
+        self.kv.release(seq.seq_id)
+        seq.status = SequenceStatus.WAITING
+        seq.num_preemptions += 1
+        seq.num_computed = 0
+        seq.prefill_target = 0
+        self.counters.preemptions += 1
+        self.running.remove(seq)
+        self.waiting.append(seq)
+
+    @staticmethod
+    def _first_of_group(seq: Sequence) -> bool:
+        return seq.params.n > 1 and not seq.output_token_ids
+
+    def _owed_forks(self) -> int:
+        """Samples that running groups will still fork off when their prompts end."""
+        return sum(s.params.n - 1 for s in self.running if self._first_of_group(s))
+
+    def _admit(self, now: float, budget: int) -> list[ScheduledSeq]:
+        """Admits waiting sequences, best score first, within the token budget, the sequence cap
+        and the watermark. A candidate that does not fit is skipped, unless it has waited
+        `max_skip_wait`: then admission stops so that what frees up goes to it
+        (scheduler.py:160-204)."""
+        admitted: list[ScheduledSeq] = []
+        if budget <= 0:
+            return admitted
+        for seq, _ in self._ranked_waiting(now):
+            if budget <= 0:
+                break
+            tokens = seq.all_token_ids
+            whole = self.kv.calculate_admission_cost(tokens)      # fresh: earlier admissions may have evicted
+            feed = self._chunk(whole.prefill_tokens, budget)
+            cost = self.kv.calculate_admission_cost(tokens, feed)
+            hit = self._hit(len(tokens), whole)
+            forks = seq.params.n - 1 if self._first_of_group(seq) else 0
+            owed = self._owed_forks()
+            fits = (feed >= 1
+                    and len(self.running) + owed + 1 + forks <= self.config.max_num_seqs
+                    and self.kv.fits(cost.per_space, owed + forks + self.watermark_blocks))
+            if not fits:
+                if now - seq.arrival_time >= self.config.max_skip_wait:
+                    break
+                continue
+            assert self.kv.allocate(seq.seq_id, tokens, feed) is not None
+            cached = self.kv.num_cached_tokens(seq.seq_id)
+            fed = tokens[cached:cached + feed]
+            if seq.num_preemptions:
+                self.counters.readmissions += 1
+            else:
+                self.counters.admissions += 1
+            self.counters.cached_tokens += cached
+            self.counters.prefill_tokens += len(fed)
+            budget -= len(fed)
+            seq.status = SequenceStatus.RUNNING
+            seq.admission_hit = hit
+            seq.prefill_target = len(tokens)
+            seq.num_computed = cached
+            final = cached + len(fed) >= len(tokens)
+            samples = 0 if not final else (seq.params.n if forks else 1)
+            self.running.append(seq)
+            seq.in_step = True
+            admitted.append(ScheduledSeq(seq, fed, samples, cached))
+        if admitted:
+            chosen = {s.seq.seq_id for s in admitted}
+            self.waiting = [s for s in self.waiting if s.seq_id not in chosen]
+        return admitted
+
+    # ---- after the model ran ----------------------------------------------------------------
+    def _fork(self, parent: Sequence, index: int) -> Sequence:
+        assert not parent.output_token_ids
+        child = Sequence(next(self._seq_ids), parent.request_id, parent.prompt_token_ids, parent.params,
+                         parent.arrival_time, status=SequenceStatus.RUNNING, sample_index=index,
+                         admission_hit=parent.admission_hit, prefill_target=parent.prefill_target,
+                         num_computed=parent.num_computed)
+        self.kv.fork(parent.seq_id, child.seq_id)
+        self.running.append(child)
+        self.groups[parent.request_id].append(child)
+        return child
+
+    def _finish_reason(self, seq: Sequence, token: int) -> Literal["eos", "length"] | None:
+        if token == self.config.eos_token_id and not seq.params.ignore_eos:
+            return "eos"
+        if len(seq.output_token_ids) >= seq.params.max_tokens:
+            return "length"
+        return None
+
+    def postprocess(self, scheduled: list[ScheduledSeq], sampled: list[list[int]], now: float) -> list[RequestOutput]:
+        """Commits each sequence's slots, forks a group after its prompt, records new tokens,
+        releases what finished (scheduler.py:236-263)."""
+        finished: list[Sequence] = []
+        for (seq, token_ids, num_samples, _), tokens in zip(scheduled, sampled, strict=True):
+            assert len(tokens) == num_samples
+            seq.in_step = False
+            self.kv.commit(seq.seq_id, len(token_ids))
+            seq.num_computed += len(token_ids)
+            if num_samples == 0:
+                continue
+            samples = [seq] + [self._fork(seq, k) for k in range(1, num_samples)]
+            for sample, token in zip(samples, tokens):
+                sample.output_token_ids.append(token)
+                sample.prefill_target = sample.num_computed      # from here on it decodes
+                if sample.first_token_time is None:
+                    sample.first_token_time = now
+                reason = self._finish_reason(sample, token)
+                if reason is not None:
+                    self.kv.release(sample.seq_id)
+                    sample.status = SequenceStatus.FINISHED
+                    sample.finish_reason = reason
+                    sample.finish_time = now
+                    finished.append(sample)
+        if finished:
+            done = {s.seq_id for s in finished}
+            self.running = [s for s in self.running if s.seq_id not in done]
+        outputs = []
+        for request_id in dict.fromkeys(s.request_id for s in finished):
+            group = self.groups[request_id]
+            if all(s.status is SequenceStatus.FINISHED for s in group):
+                outputs.append(RequestOutput(request_id, self.groups.pop(request_id)))
+        return outputs
+
+    def stats(self) -> SchedulerStats:
+        return replace(self.counters, num_waiting=len(self.waiting), num_running=len(self.running))
