@@ -67,7 +67,7 @@ def main() -> int:
     kv_bytes_per_token = 2 * args.layers * c.kv_size * itemsize
 
     def engine(batch: int, steps: int) -> LLM:
-        pages = batch * (-(-(PROMPT_LEN + steps + batch + 16) // PAGE) + 1) + 4
+        pages = batch * (MAX_MODEL_LEN // PAGE) + 2
         sc = SchedulerConfig(max_model_len=MAX_MODEL_LEN, max_num_seqs=max(batch, 1),
                              max_num_batched_tokens=max(PROMPT_LEN, batch + 1) + batch, watermark=0.0)
         return LLM(None, sc, CacheConfig(block_size=PAGE, caching=False), dtype=dtype, num_blocks=pages, seed=0,
