@@ -1,0 +1,206 @@
+"""Generation through the entry point on the GPU: greedy tokens against the plain
+implementation; nothing the cache or the scheduler does (prefix hits, portions, preemption,
+forks, caching off) may change what is generated; long decoding; the first tokens of a sequence."""
+
+from __future__ import annotations
+
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from tests.helpers import CONFIGS, make_folder, prompt
+from tests.plain.llama import PlainLlama
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def folder_a(tmp_path_factory):
+    return make_folder(tmp_path_factory, "A")
+
+
+@pytest.fixture(scope="module")
+def folder_b(tmp_path_factory):
+    return make_folder(tmp_path_factory, "B")
+
+
+def engine(folder, dtype=torch.float32, num_blocks=64, block_size=4, caching=True, seed=None, **over):
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    sc = SchedulerConfig(**{**dict(max_model_len=96, max_num_seqs=8, max_num_batched_tokens=104), **over})
+    return LLM(folder, sc, CacheConfig(block_size=block_size, caching=caching), dtype=dtype, num_blocks=num_blocks,
+               seed=seed)
+
+
+def greedy(max_tokens=12, **kw):
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+    return SamplingParams(max_tokens=max_tokens, temperature=0.0, ignore_eos=True, **kw)
+
+
+PREFIX = [5, 17, 3, 99, 42, 8, 61, 23, 7]     # two full pages of 4 and a partial one
+PROMPTS = [PREFIX + [11, 12], PREFIX + [30], [77, 2, 9], PREFIX + [11, 12, 13, 14, 15], [64] * 6]
+
+
+def test_greedy_equals_the_plain_implementation_and_prefixes_are_reused(folder_a):
+    """tests/test_engine.py:142-154 of the reference, against our own oracle."""
+    plain = PlainLlama(folder_a, torch.float64)
+    llm = engine(folder_a)
+    results = llm.generate(PROMPTS, greedy())
+    for p, r in zip(PROMPTS, results):
+        assert r.token_ids == [plain.greedy(p, 12)] and r.finish_reasons == ["length"]
+        assert r.prompt_token_ids == p and r.texts is None
+    assert llm.scheduler.stats().cached_tokens == 0, "all admitted in one step, nothing was committed yet"
+    later = PREFIX + [11, 40]
+    (r,) = llm.generate([later], greedy())
+    assert r.token_ids == [plain.greedy(later, 12)]
+    assert llm.scheduler.stats().cached_tokens == len(PREFIX) + 1, "the released prefix pages were found again"
+    assert llm.manager.stats().blocks_in_use == 0
+
+
+@pytest.mark.parametrize("caching", [True, False])
+def test_preemption_portions_and_caching_do_not_change_the_output(folder_a, caching):
+    """tests/test_engine.py:157-166: a pool too small for all five forces preemption."""
+    expected = [r.token_ids for r in engine(folder_a).generate(PROMPTS, greedy())]
+    small = engine(folder_a, num_blocks=14, caching=caching)
+    assert [r.token_ids for r in small.generate(PROMPTS, greedy())] == expected
+    st = small.scheduler.stats()
+    assert st.preemptions > 0 and (st.cached_tokens > 0) == caching
+    cut = engine(folder_a, caching=caching, max_num_batched_tokens=9, max_prefill_chunk=3)
+    assert [r.token_ids for r in cut.generate(PROMPTS, greedy())] == expected
+    assert max(s.num_tokens for s in cut.steps) <= 9
+    first = engine(folder_a, caching=caching, step_mode="prefill_first", max_prefill_chunk=5)
+    assert [r.token_ids for r in first.generate(PROMPTS, greedy())] == expected
+
+
+def test_parallel_samples_fork_and_greedy_samples_agree(folder_b):
+    plain = PlainLlama(folder_b, torch.float64)
+    llm = engine(folder_b)
+    p = prompt(1, 13, 384)
+    (r,) = llm.generate([p], greedy(6, n=3))
+    assert r.token_ids == [plain.greedy(p, 6)] * 3
+    st = llm.manager.stats()
+    assert st.blocks_in_use == 0 and st.cow_copies >= 2, "the shared tail page was copied by the writers"
+
+
+def test_sampling_is_seeded_and_does_not_depend_on_the_batch(folder_b):
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+    sp = SamplingParams(max_tokens=10, temperature=0.7, n=2, ignore_eos=True)
+    prompts = [prompt(i, n, 384) for i, n in enumerate((1, 40, 70, 29))]
+    a = [r.token_ids for r in engine(folder_b, seed=3).generate(prompts, sp)]
+    b = [r.token_ids for r in engine(folder_b, seed=3).generate(prompts, sp)]
+    c = [r.token_ids for r in engine(folder_b, seed=4).generate(prompts, sp)]
+    assert a == b and a != c
+    assert all(x[0] != x[1] for x in a), "the two samples of a request draw different noise"
+    # the same requests in portions, on a pool that forces preemption: same draws, since the
+    # noise is keyed by (request, sample, output position) and float32 logits do not depend on the cut
+    d = [r.token_ids for r in engine(folder_b, seed=3, num_blocks=50, max_num_batched_tokens=24,
+                                     max_prefill_chunk=16).generate(prompts, sp)]
+    assert d == a
+
+
+def test_the_end_token_stops_generation(folder_a):
+    plain = PlainLlama(folder_a, torch.float64)
+    full = plain.greedy(PROMPTS[0], 12)
+    eos = full[2]
+    llm = engine(folder_a, eos_token_id=eos)
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+    (r,) = llm.generate(PROMPTS[:1], SamplingParams(max_tokens=12, temperature=0.0))
+    assert r.token_ids == [full[:full.index(eos) + 1]] and r.finish_reasons == ["eos"]
+
+
+def test_step_records_requests_by_hand_and_timing(folder_a):
+    llm = engine(folder_a)
+    (r,) = llm.generate([PROMPTS[0]], greedy(3))
+    assert [s.num_tokens for s in llm.steps] == [len(PROMPTS[0]), 1, 1] and all(s.start <= s.end for s in llm.steps)
+    assert llm.steps[-1].scheduler.decode_tokens == 2 and llm.steps[-1].cache.publishes > 0
+    assert r.arrival_time <= r.first_token_time <= r.finish_time
+    rid = llm.add_request([1, 2, 3], greedy(2))
+    outs = []
+    while llm.scheduler.has_unfinished():
+        outs += llm.step()
+    assert [o.request_id for o in outs] == [rid]
+    with pytest.raises(ValueError, match="vocabulary"):
+        llm.add_request([1, 256], greedy(2))
+    with pytest.raises(ValueError, match="tokenizer"):
+        llm.add_request("text", greedy(2))
+    with pytest.raises(ValueError, match="max_model_len"):
+        llm.add_request([1] * 90, greedy(12))
+
+
+def test_pool_sized_from_free_memory(folder_a):
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    sc = SchedulerConfig(max_model_len=96, max_num_seqs=8, max_num_batched_tokens=104)
+    llm = LLM(folder_a, sc, CacheConfig(block_size=16), dtype=torch.float32)
+    assert llm.manager.num_blocks >= 8 * 7
+    (r,) = llm.generate([PROMPTS[2]], greedy(4))
+    assert len(r.token_ids[0]) == 4
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_bfloat16_generation_stays_within_the_logit_gap(name, folder_a, folder_b):
+    """In bfloat16 near-ties may flip a token, so tokens are judged by the oracle's logits: every
+    generated token must be within a small gap of the oracle's best for the same history
+    (the reference judges real-weight runs the same way, scripts/check_real_model.py:59-78)."""
+    folder = folder_a if name == "A" else folder_b
+    vocab = CONFIGS[name][0].vocab_size
+    plain = PlainLlama(folder, torch.float64, weights_as=torch.bfloat16)
+    llm = engine(folder, dtype=torch.bfloat16, block_size=16, num_blocks=32)
+    prompts = [prompt(20 + i, n, vocab) for i, n in enumerate((5, 33, 60))]
+    results = llm.generate(prompts, greedy(10))
+    agree = total = 0
+    for p, r in zip(prompts, results):
+        ids = list(p)
+        for tok in r.token_ids[0]:
+            row = plain.logits(ids)[-1]
+            assert float(row.max() - row[tok]) <= 0.03, "a token far from the oracle's best"
+            agree += int(tok == int(row.argmax()))
+            total += 1
+            ids.append(tok)
+    assert agree / total >= 0.8
+
+
+def test_long_decoding_keeps_matching(folder_b):
+    """150 tokens decoded one by one over five pages of 32: logits checked along the way."""
+    from tinyserve_llm_amd.engine.replay import Replay
+    ids = prompt(77, 200, 384)
+    want = PlainLlama(folder_b, torch.float64).logits(ids)
+    rep = Replay(folder_b, "float32", 256, page_size=32)
+    rep.step([{"id": "x", "tokens": ids[:50], "want": []}], [])
+    for pos in range(50, 200):
+        row = rep.step([{"id": "x", "tokens": [ids[pos]], "want": [0]}], [])[0]
+        if pos % 7 == 0 or pos in (63, 64, 95, 96, 127, 128, 199):
+            torch.testing.assert_close(row.double().cpu(), want[pos], rtol=1e-5, atol=5e-6, msg=lambda m: f"position {pos}: {m}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_of_a_sequence(folder_a, dtype):
+    """Positions 0, 1, 2 fed one at a time: the first key alone, then two, then three."""
+    from tinyserve_llm_amd.engine.replay import Replay
+    ids = prompt(5, 4, 256)
+    want = PlainLlama(folder_a, torch.float64, weights_as=torch.bfloat16 if dtype == "bfloat16" else None).logits(ids)
+    rep = Replay(folder_a, dtype, 64)
+    tol = dict(rtol=1e-5, atol=5e-6) if dtype == "float32" else dict(rtol=2e-2, atol=1.5e-2)
+    for pos in range(4):
+        row = rep.step([{"id": "f", "tokens": [ids[pos]], "want": [0]}], [])[0]
+        torch.testing.assert_close(row.double().cpu(), want[pos], **tol)
+
+
+def test_command_line_writes_one_record(folder_a, tmp_path):
+    out = tmp_path / "result.json"
+    r = subprocess.run([sys.executable, "-m", "tinyserve_llm_amd.generate", "--model", folder_a, "--prompt-ids", "5,17,3",
+                        "--prompt-ids", "77,2,9", "--max-tokens", "5", "--temperature", "0", "--ignore-eos", "--dtype",
+                        "float32", "--block-size", "16", "--num-blocks", "16", "--max-model-len", "64", "--max-num-seqs", "4",
+                        "--max-num-batched-tokens", "64", "--out", str(out)],
+                       capture_output=True, text=True, cwd=ROOT, timeout=600)
+    assert r.returncode == 0, r.stderr
+    record = json.loads(out.read_text())
+    plain = PlainLlama(folder_a, torch.float64)
+    assert [c["token_ids"][0] for c in record["completions"]] == [plain.greedy([5, 17, 3], 5), plain.greedy([77, 2, 9], 5)]
+    assert record["output_tokens"] == 10 and "wrote" in r.stdout

@@ -1,0 +1,335 @@
+"""Each HIP kernel alone against a plain float64/float32 formula, at sizes other than the engine's
+tiny models use: widths and vocabularies that are no power of two, head sizes from 16 to 256, odd
+head groupings, several page sizes, strided cache views, out-of-order block tables."""
+
+from __future__ import annotations
+
+import math
+
+import pytest
+import torch
+
+from tests.plain import llama as P
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def hip():
+    from tinyserve_llm_amd.ops import hip as h
+    return h
+
+
+def tol(dtype):
+    return dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def test_missing_gpu_tensor_is_refused_not_run_on_the_cpu():
+    with pytest.raises(hip().KernelError, match="GPU"):
+        hip().silu_mul(torch.zeros(2, 4))
+    with pytest.raises(hip().KernelError, match="float32 and bfloat16"):
+        hip().silu_mul(torch.zeros(2, 4, dtype=torch.float16, device=dev()))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding(dtype):
+    table = torch.randn(1000, 72, generator=gen(0)).to(dtype)
+    ids = torch.tensor([999, 0, 17, 17, 500], dtype=torch.int32)
+    out = hip().embedding(table.to(dev()), ids.to(dev()))
+    assert torch.equal(out.cpu(), table[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden", [200, 72, 2048, 3000])
+def test_rmsnorm_forms(dtype, hidden):
+    g = gen(hidden)
+    x, r = torch.randn(7, hidden, generator=g).to(dtype), torch.randn(7, hidden, generator=g).to(dtype)
+    w = (1 + 0.1 * torch.randn(hidden, generator=g)).to(dtype)
+    eps = 1e-5
+    out, res = hip().rmsnorm(x.to(dev()), w.to(dev()), eps)
+    want = P.rms_norm(x.double(), w.double(), eps)
+    torch.testing.assert_close(out.double().cpu(), want, **tol(dtype))
+    assert res.data_ptr() != 0 and torch.equal(res.cpu(), x), "without a residual the input is the residual"
+    out, res = hip().rmsnorm(x.to(dev()), w.to(dev()), eps, r.to(dev()))
+    want, s = P.add_rms_norm(x.double(), r.double(), w.double(), eps)
+    torch.testing.assert_close(out.double().cpu(), want, **tol(dtype))
+    assert torch.equal(res.cpu(), (x.float() + r.float()).to(dtype)), "the residual is the sum, rounded once"
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32)
+    out, res = hip().rmsnorm(x.to(dev()), w.to(dev()), eps, r.to(dev()), rows.to(dev()))
+    assert res is None
+    torch.testing.assert_close(out.double().cpu(), want[rows.long()], **tol(dtype))
+
+
+def test_rmsnorm_bfloat16_rounds_before_the_weight():
+    """tinyserve_llm/model/llama.py:58,67: the normalised value is cast to the storage type and
+    then multiplied by the weight in that type."""
+    x = torch.randn(3, 96, generator=gen(1)).bfloat16()
+    w = (1 + 0.1 * torch.randn(96, generator=gen(2))).bfloat16()
+    out, _ = hip().rmsnorm(x.to(dev()), w.to(dev()), 1e-6)
+    xf = x.float()
+    y = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16() * w
+    assert (out.cpu().float() - y.float()).abs().max() <= 2 ** -7 * y.float().abs().max()
+    assert (out.cpu() == y).float().mean() > 0.98, "same two roundings nearly everywhere"
+
+
+def test_rmsnorm_row_does_not_depend_on_the_batch():
+    x = torch.randn(9, 1000, generator=gen(3)).to(dev())
+    w = torch.randn(1000, generator=gen(4)).to(dev())
+    a, _ = hip().rmsnorm(x, w, 1e-5)
+    b, _ = hip().rmsnorm(x[4:5].contiguous(), w, 1e-5)
+    assert torch.equal(a[4:5], b)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rope_and_cache_write_on_a_strided_layer_view(dtype):
+    """Slots [12,13,14,15,4,5,6] on pages of 4, a skipped row (-1), other layers untouched: the
+    vectors of the reference's store tests (tests/test_attention.py:21-101), with rotation."""
+    nh, nkv, hd, T, page = 5, 1, 48, 8, 4
+    g = gen(5)
+    qkv = torch.randn(T, (nh + 2 * nkv) * hd, generator=g).to(dtype)
+    positions = torch.tensor([30, 31, 32, 33, 0, 1, 2, 7], dtype=torch.int32)
+    slots = torch.tensor([12, 13, 14, 15, 4, 5, 6, -1], dtype=torch.int64)
+    cos, sin = P.rope_tables(hd, 10000.0, None, 64, 64, torch.float64)
+    table = torch.cat((cos, sin), -1).float()
+    k_pool = torch.zeros(6, 3, page, nkv, hd, dtype=dtype, device=dev())
+    v_pool = torch.zeros_like(k_pool)
+    q = hip().rope_store(qkv.to(dev()), table.to(dev()), positions.to(dev()), slots.to(dev()), k_pool[:, 1],
+                         v_pool[:, 1], nh, nkv, hd)
+    x = qkv.double()
+    qs, ks, vs = x[:, :nh * hd].view(T, nh, hd), x[:, nh * hd:(nh + nkv) * hd].view(T, nkv, hd), x[:, (nh + nkv) * hd:].view(T, nkv, hd)
+    pos = positions.long()
+    torch.testing.assert_close(q.double().cpu(), P.apply_rope(qs, cos[pos], sin[pos]), **tol(dtype))
+    kr = P.apply_rope(ks, cos[pos], sin[pos])
+    for t in range(T - 1):
+        b, o = int(slots[t]) // page, int(slots[t]) % page
+        torch.testing.assert_close(k_pool[b, 1, o].double().cpu(), kr[t], **tol(dtype))
+        assert torch.equal(v_pool[b, 1, o].cpu(), qkv[t, (nh + nkv) * hd:].view(nkv, hd))
+    assert k_pool[:, 0].eq(0).all() and k_pool[:, 2].eq(0).all() and v_pool[:, 0].eq(0).all(), "other layers untouched"
+    assert int(k_pool.ne(0).any(dim=(-1, -2)).sum()) == 7, "exactly seven slots written; the -1 row skipped"
+    # no table: q passes through, k is stored as it is
+    q2 = hip().rope_store(qkv.to(dev()), None, positions.to(dev()), slots.to(dev()), k_pool[:, 2], v_pool[:, 2], nh, nkv, hd)
+    assert torch.equal(q2.cpu(), qkv[:, :nh * hd].view(T, nh, hd))
+    assert torch.equal(k_pool[3, 2, 0].cpu(), qkv[0, nh * hd:(nh + nkv) * hd].view(nkv, hd))
+
+
+def scattered(k, v, table, page, pages, dtype, layers=2, layer=1):
+    """A pool full of junk with k/v of positions 0.. written to the pages `table` names."""
+    g = gen(9)
+    kp = torch.randn(pages, layers, page, k.shape[1], k.shape[2], generator=g).to(dtype)
+    vp = torch.randn(pages, layers, page, k.shape[1], k.shape[2], generator=g).to(dtype)
+    for p in range(k.shape[0]):
+        kp[table[p // page], layer, p % page] = k[p]
+        vp[table[p // page], layer, p % page] = v[p]
+    return kp.to(dev())[:, layer], vp.to(dev())[:, layer]
+
+
+def run_attention(q, kc, vc, tables, seq_of, positions, scale, window=0):
+    return hip().paged_attention_wave(
+        q.to(dev()), kc, vc, torch.tensor(tables, dtype=torch.int32, device=dev()),
+        torch.tensor(seq_of, dtype=torch.int32, device=dev()), torch.tensor(positions, dtype=torch.int32, device=dev()),
+        scale, window)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv,hd,page", [(4, 2, 16, 4), (3, 1, 32, 16), (6, 2, 48, 8), (8, 8, 64, 256),
+                                              (5, 5, 128, 32), (2, 1, 256, 16)])
+def test_paged_attention_prefill_prefix_and_decode_in_one_batch(dtype, heads, kv, hd, page):
+    """A whole prompt, its last 4 tokens over a cached prefix and its last token as a decode, in
+    one batch, through an out-of-order block table padded with zeros
+    (tests/test_engine.py:69-82 of the reference)."""
+    n = 11 if page <= 8 else 75
+    g = gen(hd)
+    q = torch.randn(n, heads, hd, generator=g).to(dtype)
+    k, v = torch.randn(n, kv, hd, generator=g).to(dtype), torch.randn(n, kv, hd, generator=g).to(dtype)
+    need = -(-n // page)
+    table = [6, 1, 4, 9, 2, 7, 3, 8, 5, 0][:need]
+    kc, vc = scattered(k, v, table, page, 10, dtype)
+    dense = P.causal_attention(q.double(), k.double(), v.double())
+    queries = torch.cat([q, q[n - 4:], q[n - 1:]])
+    seq_of = [0] * n + [1] * 4 + [2]
+    positions = list(range(n)) + list(range(n - 4, n)) + [n - 1]
+    out = run_attention(queries, kc, vc, [table + [0], table + [0], table + [0]], seq_of, positions, hd ** -0.5)
+    out = out.double().cpu()
+    torch.testing.assert_close(out[:n], dense, **tol(dtype))
+    torch.testing.assert_close(out[n:n + 4], dense[n - 4:], **tol(dtype))
+    torch.testing.assert_close(out[n + 4:], dense[n - 1:], **tol(dtype))
+    if dtype == torch.float32:
+        assert torch.equal(out[n:n + 4], out[n - 4:n]) and torch.equal(out[n + 4:], out[n - 1:n]), \
+            "a row's sums do not depend on the portion it came in"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_finds_a_far_key_among_hundreds(dtype):
+    """Random keys hide a lost page or a wrong offset: here one key, far back, is made to win
+    every score, so the output must be that key's value."""
+    n, heads, kv, hd, page = 700, 4, 2, 64, 64
+    g = gen(11)
+    q = torch.randn(n, heads, hd, generator=g) * 0.1
+    k, v = torch.randn(n, kv, hd, generator=g) * 0.1, torch.randn(n, kv, hd, generator=g)
+    for target in (0, 63, 64, 389, 640):
+        kk = k.clone()
+        kk[target] = 0
+        kk[target, :, 5] = 40.0
+        qq = q.clone()
+        qq[:, :, 5] = 40.0
+        table = list(range(10, -1, -1))
+        kc, vc = scattered(kk.to(dtype), v.to(dtype), table, page, 11, dtype)
+        rows = [target, target + 1 if target + 1 < n else target, n - 1]
+        out = run_attention(qq[rows].to(dtype), kc, vc, [table], [0, 0, 0], rows, hd ** -0.5).float().cpu()
+        for i, r in enumerate(rows):
+            for h in range(heads):
+                torch.testing.assert_close(out[i, h], v[target, h // 2].to(dtype).float(), rtol=1e-3, atol=1e-3)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_window_edge(dtype):
+    n, heads, kv, hd, page, window = 200, 2, 1, 32, 16, 37
+    g = gen(12)
+    q, k, v = torch.randn(n, heads, hd, generator=g), torch.randn(n, kv, hd, generator=g), torch.randn(n, kv, hd, generator=g)
+    table = list(range(12, -1, -1))
+    kc, vc = scattered(k.to(dtype), v.to(dtype), table, page, 13, dtype)
+    want = P.causal_attention(q.to(dtype).double(), k.to(dtype).double(), v.to(dtype).double(), window=window)
+    out = run_attention(q.to(dtype), kc, vc, [table], [0] * n, list(range(n)), hd ** -0.5, window).double().cpu()
+    torch.testing.assert_close(out, want, **tol(dtype))
+    # the key just inside the window wins, the key just outside must not be seen at all
+    pos = 150
+    for off, seen in ((window - 1, True), (window, False)):
+        kk = k.clone()
+        kk[pos - off] = 0
+        kk[pos - off, 0, 3] = 50.0
+        qq = q[pos:pos + 1].clone()
+        qq[0, :, 3] = 50.0
+        kc, vc = scattered(kk.to(dtype), v.to(dtype), table, page, 13, dtype)
+        out = run_attention(qq.to(dtype), kc, vc, [table], [0], [pos], hd ** -0.5, window).float().cpu()
+        is_it = torch.allclose(out[0, 0], v[pos - off, 0].to(dtype).float(), rtol=1e-2, atol=1e-2)
+        assert is_it == seen
+
+
+def test_attention_refuses_sizes_it_cannot_take():
+    kc = torch.zeros(2, 4, 1, 24, device=dev())
+    with pytest.raises(hip().KernelError, match="multiple of 16"):
+        hip().paged_attention_wave(torch.zeros(1, 1, 24, device=dev()), kc, kc, torch.zeros(1, 1, dtype=torch.int32, device=dev()),
+                                   torch.zeros(1, dtype=torch.int32, device=dev()), torch.zeros(1, dtype=torch.int32, device=dev()), 1.0)
+    kc = torch.zeros(2, 4, 2, 16, device=dev())
+    with pytest.raises(hip().KernelError, match="divide"):
+        hip().paged_attention_wave(torch.zeros(1, 3, 16, device=dev()), kc, kc, torch.zeros(1, 1, dtype=torch.int32, device=dev()),
+                                   torch.zeros(1, dtype=torch.int32, device=dev()), torch.zeros(1, dtype=torch.int32, device=dev()), 1.0)
+
+
+@pytest.mark.parametrize("m,n,k", [(70, 130, 50), (1, 384, 96), (3, 5, 7), (129, 64, 160), (33, 1000, 2048)])
+def test_gemm_exact(m, n, k):
+    g = gen(m * n)
+    a, w = torch.randn(m, k, generator=g), torch.randn(n, k, generator=g)
+    out = hip().gemm_exact(a.to(dev()), w.to(dev()))
+    torch.testing.assert_close(out.double().cpu(), a.double() @ w.double().T, rtol=1e-5, atol=1e-5 * math.sqrt(k))
+    one = hip().gemm_exact(a[m // 2:m // 2 + 1].contiguous().to(dev()), w.to(dev()))
+    assert torch.equal(one, out[m // 2:m // 2 + 1]), "a row's result does not depend on the other rows"
+    a16, w16 = a.bfloat16(), w.bfloat16()
+    out = hip().gemm_exact(a16.to(dev()), w16.to(dev()), torch.float32)
+    torch.testing.assert_close(out.double().cpu(), a16.double() @ w16.double().T, rtol=1e-5, atol=1e-5 * math.sqrt(k))
+    out = hip().gemm_exact(a16.to(dev()), w16.to(dev()))
+    assert out.dtype == torch.bfloat16
+    torch.testing.assert_close(out.double().cpu(), a16.double() @ w16.double().T, rtol=1e-2, atol=1e-2 * math.sqrt(k))
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 384, 96), (8, 3072, 2048), (64, 2048, 8192), (200, 1000, 160), (2048, 512, 2048)])
+def test_linear_bfloat16(m, n, k):
+    from tinyserve_llm_amd.parts.linear import linear
+    g = gen(m + n)
+    a, w = torch.randn(m, k, generator=g).bfloat16(), (torch.randn(n, k, generator=g) * 0.05).bfloat16()
+    out = linear(a.to(dev()), w.to(dev()))
+    want = a.double() @ w.double().T
+    assert out.dtype == torch.bfloat16 and out.shape == (m, n)
+    torch.testing.assert_close(out.double().cpu(), want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
+    f = linear(a.to(dev()), w.to(dev()), out_dtype=torch.float32)
+    assert f.dtype == torch.float32
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul(dtype):
+    gu = torch.randn(9, 2 * 150, generator=gen(13)).to(dtype)
+    out = hip().silu_mul(gu.to(dev()))
+    torch.testing.assert_close(out.double().cpu(), P.silu_mul(gu.double()), **tol(dtype))
+    gu[:, :150] = 0
+    assert float(hip().silu_mul(gu.to(dev())).abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_copy_slots_copies_the_leading_slots_of_every_layer(dtype):
+    pool = torch.randn(5, 3, 8, 2, 16, generator=gen(14)).to(dtype).to(dev())
+    before = pool.clone()
+    hip().copy_slots(pool, 3, 1, 5)
+    assert torch.equal(pool[1, :, :5], before[3, :, :5]) and torch.equal(pool[1, :, 5:], before[1, :, 5:])
+    keep = [0, 2, 3, 4]
+    assert torch.equal(pool[keep], before[keep])
+    with pytest.raises(hip().KernelError):
+        hip().copy_slots(pool, 3, 3, 2)
+    with pytest.raises(hip().KernelError):
+        hip().copy_slots(pool, 0, 5, 2)
+
+
+def exp_noise(seed, key, n):
+    """The kernel's counter hash, written out with Python integers."""
+    M = (1 << 64) - 1
+
+    def mix(x):
+        x ^= x >> 30
+        x = (x * 0xBF58476D1CE4E5B9) & M
+        x ^= x >> 27
+        x = (x * 0x94D049BB133111EB) & M
+        return x ^ (x >> 31)
+
+    out = []
+    for i in range(n):
+        x = mix((mix(seed ^ ((key * 0x9E3779B97F4A7C15) & M)) + i * 0xD1342543DE82EF95) & M)
+        u = ((x >> 40) + 1) / 16777216.0
+        out.append(max(-math.log(u), 1e-10))
+    return torch.tensor(out, dtype=torch.float64)
+
+
+def test_sampler_greedy_vector_frequencies_and_seeds():
+    """The cases of the reference's sampler test (tests/test_engine.py:121-129)."""
+    from tinyserve_llm_amd.sampling.sampler import row_key, sample
+    logits = torch.tensor([[0.0, 5.0, 1.0], [3.0, 0.0, 0.0]], device=dev())
+    assert sample(logits, [0.0, 0.0], [1, 2], seed=0).tolist() == [1, 0]
+    assert sample(torch.tensor([[2.0, 7.0, 7.0, 1.0]], device=dev()), [0.0], [1], 0).tolist() == [1], "ties: lowest index"
+    rows = 20000
+    keys = [row_key(3, 0, i) for i in range(rows)]
+    draws = sample(logits[:1].expand(rows, 3).contiguous(), [1.0] * rows, keys, seed=0)
+    freq = torch.bincount(draws.long().cpu(), minlength=3).double() / rows
+    torch.testing.assert_close(freq, torch.softmax(logits[0].double().cpu(), -1), atol=0.01, rtol=0)
+    cold = sample(logits[:1].expand(rows, 3).contiguous(), [0.25] * rows, keys, seed=0)
+    freq = torch.bincount(cold.long().cpu(), minlength=3).double() / rows
+    torch.testing.assert_close(freq, torch.softmax(logits[0].double().cpu() / 0.25, -1), atol=0.01, rtol=0)
+    again = sample(logits[:1].expand(rows, 3).contiguous(), [1.0] * rows, keys, seed=0)
+    other = sample(logits[:1].expand(rows, 3).contiguous(), [1.0] * rows, keys, seed=1)
+    assert torch.equal(draws, again) and not torch.equal(draws, other)
+
+
+def test_sampler_draw_is_the_exponential_race_and_ignores_the_row_order():
+    """argmax(softmax(logits / t) / E) with the kernel's own noise, computed here in float64
+    (tinyserve_llm/engine/sampler.py:18-23); and a row's draw depends on its key, not its place."""
+    from tinyserve_llm_amd.sampling.sampler import sample
+    vocab, rows = 1500, 12
+    logits = torch.randn(rows, vocab, generator=gen(15)) * 3
+    temps = [0.7, 1.0, 0.0, 1.3] * 3
+    keys = [1000 + 17 * r for r in range(rows)]
+    got = sample(logits.to(dev()), temps, keys, seed=42).tolist()
+    for r in range(rows):
+        if temps[r] == 0:
+            assert got[r] == int(logits[r].argmax())
+            continue
+        p = torch.softmax(logits[r].double() / temps[r], -1)
+        assert got[r] == int((p / exp_noise(42, keys[r], vocab)).argmax())
+    perm = torch.randperm(rows, generator=gen(16)).tolist()
+    shuffled = sample(logits[perm].contiguous().to(dev()), [temps[i] for i in perm], [keys[i] for i in perm], seed=42).tolist()
+    assert shuffled == [got[i] for i in perm]

@@ -1,0 +1,337 @@
+"""Each part of a layer alone on the GPU against its plain counterpart, built from explicit sizes
+that no model of the tests uses; then parts the framework does not have (a mixer with state of its
+own, a routed feed-forward, another position encoding) registered from here and stepped through
+the unchanged engine; then the run order as data (a layer named twice, a layer reading another
+layer's cache)."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+from tests.plain import llama as P
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+DEV = "cuda:0"
+
+
+def tol(dtype):
+    return dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=3e-2, atol=3e-2)
+
+
+def context(lengths, starts, page, tables, encodings=None):
+    """A StepContext by hand: requests with `lengths[i]` tokens starting at `starts[i]`."""
+    from tinyserve_llm_amd.parts.base import StepContext
+    pos, seq_of, slots, cu = [], [], [], [0]
+    for s, (n, st) in enumerate(zip(lengths, starts)):
+        pos += list(range(st, st + n))
+        seq_of += [s] * n
+        slots += [tables[s][p // page] * page + p % page for p in range(st, st + n)]
+        cu.append(cu[-1] + n)
+    width = max(len(t) for t in tables)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    return StepContext(
+        num_tokens=len(pos), num_seqs=len(lengths), token_ids=i32([0] * len(pos)), positions=i32(pos),
+        seq_of_token=i32(seq_of), cu_seqlens=i32(cu), context_lens=i32([a + b for a, b in zip(lengths, starts)]),
+        state_slots=i32(list(range(len(lengths)))), slot_mapping=[torch.tensor(slots, dtype=torch.int64, device=DEV)],
+        block_tables=[i32([t + [0] * (width - len(t)) for t in tables])], host_cu_seqlens=cu, host_starts=list(starts),
+        host_context_lens=[a + b for a, b in zip(lengths, starts)], host_state_slots=list(range(len(lengths))),
+        position_encodings=encodings or {})
+
+
+def bound(part, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    params = {}
+    for name, ps in part.param_specs().items():
+        mean, std = ps.init
+        params[name] = (torch.randn(ps.shape, generator=g) * max(std, 0.05) + mean).to(dtype)
+    part.bind({k: v.to(DEV) for k, v in params.items()})
+    return {k: v.double() for k, v in params.items()}
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_part(dtype):
+    from tinyserve_llm_amd.parts.norm import RMSNorm
+    part = RMSNorm(hidden_size=176, eps=3e-6)
+    w = bound(part, dtype, 0)["weight"]
+    x, r = torch.randn(5, 176).to(dtype), torch.randn(5, 176).to(dtype)
+    out, res = part(x.to(DEV), r.to(DEV))
+    want, s = P.add_rms_norm(x.double(), r.double(), w, 3e-6)
+    torch.testing.assert_close(out.double().cpu(), want, **tol(dtype))
+    torch.testing.assert_close(res.double().cpu(), s, **tol(dtype))
+
+
+def test_rope_part_table_is_the_reference_table():
+    from tinyserve_llm_amd.parts.rope import Rope
+    scaling = dict(factor=4.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=32)
+    part = Rope(head_dim=48, max_position=200, theta=12345.0, scaling=scaling)
+    part.prepare(torch.device(DEV))
+    cos, sin = P.rope_tables(48, 12345.0, scaling, 200, 200, torch.float32)
+    assert torch.equal(part.rotary_table().cpu(), torch.cat((cos, sin), -1)), "bit-equal: same float32 operations"
+    assert torch.equal(Rope(48, 200, 12345.0).inv_freq, P.rope_inv_freq(48, 12345.0, None, 200))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_part_over_two_steps(dtype):
+    """A prompt portion then the rest beside a second request: projections, rotation, cache
+    write, attention over the pages and output projection against the plain parts."""
+    from tinyserve_llm_amd.parts.attention import Attention
+    from tinyserve_llm_amd.parts.base import LayerMemory
+    from tinyserve_llm_amd.parts.rope import Rope
+    hidden, heads, kv, hd, page = 80, 6, 2, 48, 8
+    part = Attention(hidden_size=hidden, num_heads=heads, num_kv_heads=kv, head_dim=hd, position="rope")
+    w = bound(part, dtype, 1)
+    rope = Rope(hd, 64, 10000.0)
+    rope.prepare(torch.device(DEV))
+    mem = LayerMemory(k_cache=torch.zeros(6, page, kv, hd, dtype=dtype, device=DEV),
+                      v_cache=torch.zeros(6, page, kv, hd, dtype=dtype, device=DEV))
+    xa, xb = torch.randn(19, hidden).to(dtype), torch.randn(5, hidden).to(dtype)
+    ta, tb = [4, 0, 2], [5]
+    part.forward(xa[:11].to(DEV), context([11], [0], page, [ta], {"rope": rope}), mem)
+    out = part.forward(torch.cat([xa[11:], xb]).to(DEV), context([8, 5], [11, 0], page, [ta, tb], {"rope": rope}), mem)
+
+    def plain(x):
+        n = x.shape[0]
+        qkv = x.double() @ w["qkv"].T
+        q, k, v = qkv[:, :heads * hd], qkv[:, heads * hd:(heads + kv) * hd], qkv[:, (heads + kv) * hd:]
+        cos, sin = P.rope_tables(hd, 10000.0, None, 64, n, torch.float64)
+        q, k = P.apply_rope(q.view(n, heads, hd), cos, sin), P.apply_rope(k.view(n, kv, hd), cos, sin)
+        return P.causal_attention(q, k, v.view(n, kv, hd)).reshape(n, heads * hd) @ w["o"].T
+
+    want = torch.cat([plain(xa)[11:], plain(xb)])
+    torch.testing.assert_close(out.double().cpu(), want, **tol(dtype))
+    assert part.kv_spec().num_kv_heads == kv and part.kv_spec().head_dim == hd and part.state_spec() is None
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gated_mlp_part(dtype):
+    from tinyserve_llm_amd.parts.mlp import GatedMLP
+    part = GatedMLP(hidden_size=72, intermediate_size=200)
+    w = bound(part, dtype, 2)
+    x = torch.randn(9, 72).to(dtype)
+    out = part.forward(x.to(DEV), None)
+    want = P.silu_mul(x.double() @ w["gate_up"].T) @ w["down"].T
+    torch.testing.assert_close(out.double().cpu(), want, **tol(dtype))
+    with pytest.raises(ValueError, match="silu"):
+        GatedMLP(8, 8, activation="gelu")
+
+
+# ---- parts from outside the framework --------------------------------------------------------------
+
+def register_toy_parts():
+    from tinyserve_llm_amd.parts.base import (FeedForward, Mixer, ParamSpec, PositionEncoding, StateSpec, register)
+
+    @register("mixer", "toy_running_mean")
+    class RunningMean(Mixer):
+        """y_t = W · mean(x_0..x_t): no keys, only a per-request state (sum, count)."""
+
+        def __init__(self, hidden_size):
+            self.hidden_size = hidden_size
+
+        def param_specs(self):
+            return {"w": ParamSpec((self.hidden_size, self.hidden_size), init=(0.0, 0.1))}
+
+        def state_spec(self):
+            return StateSpec((self.hidden_size + 1,), torch.float32)
+
+        def forward(self, x, ctx, mem):
+            out = torch.empty_like(x)
+            for s in range(ctx.num_seqs):
+                a, b = ctx.host_cu_seqlens[s], ctx.host_cu_seqlens[s + 1]
+                state = mem.state[ctx.host_state_slots[s]]
+                if ctx.host_starts[s] == 0:
+                    state.zero_()
+                sums = state[:-1] + torch.cumsum(x[a:b].float(), 0)
+                counts = state[-1] + torch.arange(1, b - a + 1, device=x.device)
+                out[a:b] = ((sums / counts[:, None]).to(x.dtype) @ self.w.T)
+                state[:-1] = sums[-1]
+                state[-1] = counts[-1]
+            return out
+
+    @register("feed_forward", "toy_routed")
+    class Routed(FeedForward):
+        """Top-1 of E small experts, chosen by a 32-bit router."""
+
+        def __init__(self, hidden_size, experts):
+            self.hidden_size, self.experts = hidden_size, experts
+
+        def param_specs(self):
+            return {"router": ParamSpec((self.experts, self.hidden_size), storage="float32", init=(0.0, 0.5)),
+                    "w": ParamSpec((self.experts * self.hidden_size, self.hidden_size), init=(0.0, 0.1))}
+
+        def forward(self, x, ctx):
+            choice = (x.float() @ self.router.T).argmax(-1)
+            w = self.w.view(self.experts, self.hidden_size, self.hidden_size)[choice]
+            return torch.einsum("toh,th->to", w.float(), x.float()).to(x.dtype)
+
+    @register("position_encoding", "toy_learned")
+    class Learned(PositionEncoding):
+        """A learned vector per position, added to the embedded tokens."""
+
+        def __init__(self, hidden_size, max_position):
+            self.hidden_size, self.max_position = hidden_size, max_position
+
+        def param_specs(self):
+            return {"table": ParamSpec((self.max_position, self.hidden_size), init=(0.0, 0.3))}
+
+        def on_embedding(self, hidden, ctx):
+            return hidden + self.table[ctx.positions.long()]
+
+
+def toy_spec(hidden=48, vocab=97):
+    from tinyserve_llm_amd.models.spec import LayerRun, LayerSpec, ModelSpec
+    from tinyserve_llm_amd.parts.base import PartSpec
+    norm = PartSpec("rmsnorm", dict(hidden_size=hidden, eps=1e-5))
+    mlp = PartSpec("gated_mlp", dict(hidden_size=hidden, intermediate_size=64))
+    attn = PartSpec("attention", dict(hidden_size=hidden, num_heads=3, num_kv_heads=1, head_dim=16, position=None))
+    layers = [LayerSpec(PartSpec("toy_running_mean", dict(hidden_size=hidden)), mlp, norm, norm),
+              LayerSpec(attn, PartSpec("toy_routed", dict(hidden_size=hidden, experts=3)), norm, norm)]
+    return ModelSpec(architecture="Toy", vocab_size=vocab, hidden_size=hidden, max_position=128, layers=layers,
+                     order=[LayerRun(0), LayerRun(1), LayerRun(0)], final_norm=norm,
+                     position_encodings={"learned": PartSpec("toy_learned", dict(hidden_size=hidden, max_position=128))},
+                     tie_word_embeddings=True)
+
+
+def toy_engine(dtype, seed=0, pages=24, page=8):
+    from tinyserve_llm_amd.cache.manager import KVCacheManager
+    from tinyserve_llm_amd.cache.storage import KVStorage
+    from tinyserve_llm_amd.engine.runner import ModelRunner
+    from tinyserve_llm_amd.models.decoder import DecoderModel
+    from tinyserve_llm_amd.weights.random_init import random_params
+    register_toy_parts()
+    model = DecoderModel(toy_spec())
+    params = random_params(model, seed, dtype, "cpu")
+    model.bind({k: v.to(DEV) for k, v in params.items()}, dtype, torch.device(DEV))
+    storage = KVStorage(model.cache_plan(), model.state_plan(), pages, page, dtype, DEV, num_state_slots=4)
+    manager = KVCacheManager(storage, caching=False)
+    return model, {k: v.double() for k, v in params.items()}, storage, manager, ModelRunner(model, storage, manager)
+
+
+def toy_plain(p, ids):
+    """The toy model whole, in float64, from its definition."""
+    n = len(ids)
+    h = p["embed.weight"][torch.tensor(ids)] + p["positions.learned.table"][:n]
+
+    def mean_mixer(x, w):
+        return (torch.cumsum(x, 0) / torch.arange(1, n + 1)[:, None].double()) @ w.T
+
+    def layer0(h):
+        x = P.rms_norm(h, p["layers.0.mixer_norm.weight"], 1e-5)
+        h = h + mean_mixer(x, p["layers.0.mixer.w"])
+        x = P.rms_norm(h, p["layers.0.ff_norm.weight"], 1e-5)
+        return h + P.silu_mul(x @ p["layers.0.ff.gate_up"].T) @ p["layers.0.ff.down"].T
+
+    h = layer0(h)
+    x = P.rms_norm(h, p["layers.1.mixer_norm.weight"], 1e-5)
+    qkv = x @ p["layers.1.mixer.qkv"].T
+    o = P.causal_attention(qkv[:, :48].reshape(n, 3, 16), qkv[:, 48:64].reshape(n, 1, 16), qkv[:, 64:].reshape(n, 1, 16))
+    h = h + o.reshape(n, 48) @ p["layers.1.mixer.o"].T
+    x = P.rms_norm(h, p["layers.1.ff_norm.weight"], 1e-5)
+    choice = (x @ p["layers.1.ff.router"].T).argmax(-1)
+    w = p["layers.1.ff.w"].view(3, 48, 48)[choice]
+    h = h + torch.einsum("toh,th->to", w, x)
+    h = layer0(h)                                     # the same layer, named twice in the order
+    return P.rms_norm(h, p["final_norm.weight"], 1e-5) @ p["embed.weight"].T
+
+
+def test_toy_parts_register_build_and_step_without_touching_the_framework():
+    """A mixer with state of its own, a routed feed-forward and a learned position encoding,
+    defined above, run through the framework's model, cache manager, storage and step function
+    in portions and beside another request; layer 0 is named twice in the run order and has a
+    state slot per run."""
+    from tinyserve_llm_amd.engine.runner import StepEntry
+    model, p, storage, manager, runner = toy_engine(torch.float32)
+    assert [e.run for e in model.state_plan()] == [0, 2] and [e.owner for e in model.cache_plan()] == [1]
+    assert storage.state(0).shape == (4, 49) and storage.state(1) is None
+    a, b = [3, 50, 7, 7, 96, 1, 0, 22, 41, 5, 88, 13, 2], [9, 8, 7, 6, 5]
+    want_a, want_b = toy_plain(p, a), toy_plain(p, b)
+    got = {}
+    manager.allocate(0, a[:4])
+    out = runner.step([StepEntry(0, a[:4], 0, [0, 3])])
+    got[("a", 0)], got[("a", 3)] = out[0], out[1]
+    manager.commit(0, 4)
+    manager.allocate(1, b)
+    manager.append_slots(0, a[4:6])
+    out = runner.step([StepEntry(1, b, 0, [4]), StepEntry(0, a[4:6], 4, [1])])
+    got[("b", 4)], got[("a", 5)] = out[0], out[1]
+    manager.commit(0, 2)
+    manager.commit(1, 5)
+    manager.release(1)
+    for pos in range(6, len(a)):
+        manager.append_slots(0, [a[pos]])
+        got[("a", pos)] = runner.step([StepEntry(0, [a[pos]], pos, [0])])[0]
+        manager.commit(0, 1)
+    for (name, pos), row in got.items():
+        want = (want_a if name == "a" else want_b)[pos]
+        torch.testing.assert_close(row.double().cpu(), want, rtol=1e-4, atol=1e-5, msg=lambda m: f"{name}{pos}: {m}")
+    manager.release(0)
+    assert manager.num_available_blocks() == manager.num_blocks and len(manager.free_state_slots) == 4
+
+
+def test_a_layer_can_read_another_layers_cache():
+    """order = [layer 0 (owns a cache), layer 1 reading layer 0's cache without writing]:
+    layer 1's queries attend over layer 0's keys and values."""
+    from tinyserve_llm_amd.cache.manager import KVCacheManager
+    from tinyserve_llm_amd.cache.storage import KVStorage
+    from tinyserve_llm_amd.engine.runner import ModelRunner, StepEntry
+    from tinyserve_llm_amd.models.decoder import DecoderModel
+    from tinyserve_llm_amd.models.spec import LayerRun, LayerSpec, ModelSpec
+    from tinyserve_llm_amd.parts.base import PartSpec
+    from tinyserve_llm_amd.weights.random_init import random_params
+    hidden = 32
+    norm = PartSpec("rmsnorm", dict(hidden_size=hidden, eps=1e-5))
+    layer = LayerSpec(PartSpec("attention", dict(hidden_size=hidden, num_heads=2, num_kv_heads=2, head_dim=16, position=None)),
+                      PartSpec("gated_mlp", dict(hidden_size=hidden, intermediate_size=48)), norm, norm)
+    spec = ModelSpec("Toy2", 50, hidden, 64, [layer, layer], [LayerRun(0), LayerRun(1, cache=0, store=False)], norm,
+                     tie_word_embeddings=True)
+    model = DecoderModel(spec)
+    assert len(model.cache_plan()) == 1
+    params = random_params(model, 3, torch.float32, "cpu")
+    model.bind({k: v.to(DEV) for k, v in params.items()}, torch.float32, torch.device(DEV))
+    p = {k: v.double() for k, v in params.items()}
+    storage = KVStorage(model.cache_plan(), model.state_plan(), 8, 4, torch.float32, DEV, 2)
+    manager = KVCacheManager(storage, caching=False)
+    runner = ModelRunner(model, storage, manager)
+    ids = [4, 9, 33, 2, 17, 8, 40]
+    n = len(ids)
+    h = p["embed.weight"][torch.tensor(ids)]
+    x = P.rms_norm(h, p["layers.0.mixer_norm.weight"], 1e-5)
+    qkv0 = x @ p["layers.0.mixer.qkv"].T
+    k0, v0 = qkv0[:, 32:64].reshape(n, 2, 16), qkv0[:, 64:].reshape(n, 2, 16)
+    h = h + P.causal_attention(qkv0[:, :32].reshape(n, 2, 16), k0, v0).reshape(n, 32) @ p["layers.0.mixer.o"].T
+    x = P.rms_norm(h, p["layers.0.ff_norm.weight"], 1e-5)
+    h = h + P.silu_mul(x @ p["layers.0.ff.gate_up"].T) @ p["layers.0.ff.down"].T
+    x = P.rms_norm(h, p["layers.1.mixer_norm.weight"], 1e-5)
+    q1 = (x @ p["layers.1.mixer.qkv"].T)[:, :32].reshape(n, 2, 16)
+    h = h + P.causal_attention(q1, k0, v0).reshape(n, 32) @ p["layers.1.mixer.o"].T
+    x = P.rms_norm(h, p["layers.1.ff_norm.weight"], 1e-5)
+    h = h + P.silu_mul(x @ p["layers.1.ff.gate_up"].T) @ p["layers.1.ff.down"].T
+    want = P.rms_norm(h, p["final_norm.weight"], 1e-5) @ p["embed.weight"].T
+    manager.allocate(0, ids[:5])
+    first = runner.step([StepEntry(0, ids[:5], 0, list(range(5)))])
+    manager.commit(0, 5)
+    manager.append_slots(0, ids[5:])
+    rest = runner.step([StepEntry(0, ids[5:], 5, [0, 1])])
+    torch.testing.assert_close(torch.cat([first, rest]).double().cpu(), want, rtol=1e-4, atol=1e-5)
+
+
+def test_bad_orders_are_refused_when_the_model_is_built():
+    from tinyserve_llm_amd.models.decoder import DecoderModel
+    from tinyserve_llm_amd.models.spec import LayerRun
+    register_toy_parts()
+    spec = toy_spec()
+    spec.order = [LayerRun(0), LayerRun(1, cache=2)]
+    with pytest.raises(ValueError, match="does not run before"):
+        DecoderModel(spec)
+    spec.order = [LayerRun(5)]
+    with pytest.raises(ValueError, match="names layer 5"):
+        DecoderModel(spec)
+    spec.order = [LayerRun(1, store=False)]
+    with pytest.raises(ValueError, match="neither owns"):
+        DecoderModel(spec)
+    spec.layers[1] = spec.layers[1].__class__(spec.layers[1].mixer.__class__("no_such_mixer", {}), spec.layers[1].feed_forward,
+                                              spec.layers[1].mixer_norm, spec.layers[1].ff_norm)
+    with pytest.raises(KeyError, match="no mixer named"):
+        DecoderModel(spec)
