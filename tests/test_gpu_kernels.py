@@ -214,6 +214,71 @@ def test_attention_window_edge(dtype):
         assert is_it == seen
 
 
+def head_major(k, v, table, page, pages, dtype):
+    """The engine's own pool layout: [pages, kv_heads, page_size, head_dim] seen as [pages, page_size, kv_heads, head_dim]."""
+    g = gen(19)
+    kp = torch.randn(pages, k.shape[1], page, k.shape[2], generator=g).to(dtype)
+    vp = torch.randn(pages, k.shape[1], page, k.shape[2], generator=g).to(dtype)
+    for p in range(k.shape[0]):
+        kp[table[p // page], :, p % page] = k[p]
+        vp[table[p // page], :, p % page] = v[p]
+    return kp.to(dev()).permute(0, 2, 1, 3), vp.to(dev()).permute(0, 2, 1, 3)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv,hd,page", [(4, 2, 16, 4), (3, 1, 32, 16), (6, 2, 48, 8), (32, 8, 64, 256),
+                                              (5, 5, 128, 32), (8, 1, 256, 16), (24, 8, 128, 64)])
+@pytest.mark.parametrize("chunk", [64, 128, 256])
+def test_split_key_decode_attention(dtype, heads, kv, hd, page, chunk):
+    """One query per request at different context lengths (1, a chunk's edge, mid-chunk, long), on
+    both cache layouts, against the dense formula."""
+    n = 600
+    g = gen(hd + chunk)
+    q = torch.randn(n, heads, hd, generator=g).to(dtype)
+    k, v = torch.randn(n, kv, hd, generator=g).to(dtype), torch.randn(n, kv, hd, generator=g).to(dtype)
+    pages = -(-n // page)
+    table = list(range(pages - 1, -1, -1))
+    dense = P.causal_attention(q.double(), k.double(), v.double())
+    rows = [0, 1, chunk - 1, chunk, chunk + 1, 255, 256, 257, 400, 599]
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev())
+    for kc, vc in (scattered(k, v, table, page, pages, dtype), head_major(k, v, table, page, pages, dtype)):
+        out = hip().paged_attention_decode(q[rows].to(dev()), kc, vc, i32([table, table]), i32([0, 1] * 5), i32(rows),
+                                           hd ** -0.5, chunk=chunk)
+        torch.testing.assert_close(out.double().cpu(), dense[rows], **tol(dtype))
+    wave = run_attention(q[rows], kc, vc, [table], [0] * len(rows), rows, hd ** -0.5)
+    torch.testing.assert_close(out.float(), wave.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_split_key_decode_window_and_far_key(dtype):
+    n, heads, kv, hd, page, window = 700, 4, 2, 64, 64, 300
+    g = gen(21)
+    q = torch.randn(n, heads, hd, generator=g) * 0.1
+    k, v = torch.randn(n, kv, hd, generator=g) * 0.1, torch.randn(n, kv, hd, generator=g)
+    table = list(range(10, -1, -1))
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev())
+    kc, vc = head_major(k.to(dtype), v.to(dtype), table, page, 11, dtype)
+    rows = [5, 299, 300, 301, 699]
+    want = P.causal_attention(q.to(dtype).double(), k.to(dtype).double(), v.to(dtype).double(), window=window)[rows]
+    out = hip().paged_attention_decode(q[rows].to(dtype).to(dev()), kc, vc, i32([table]), i32([0] * 5), i32(rows),
+                                       hd ** -0.5, window=window, chunk=128)
+    torch.testing.assert_close(out.double().cpu(), want, **tol(dtype))
+    for target in (0, 63, 64, 389, 640):
+        kk = k.clone()
+        kk[target] = 0
+        kk[target, :, 5] = 40.0
+        qq = q[[699]].clone()
+        qq[:, :, 5] = 40.0
+        kc, vc = head_major(kk.to(dtype), v.to(dtype), table, page, 11, dtype)
+        out = hip().paged_attention_decode(qq.to(dtype).to(dev()), kc, vc, i32([table]), i32([0]), i32([699]), hd ** -0.5)
+        for h in range(heads):
+            torch.testing.assert_close(out[0, h].float().cpu(), v[target, h // 2].to(dtype).float(), rtol=1e-3, atol=1e-3)
+        seen = target > 699 - window
+        out = hip().paged_attention_decode(qq.to(dtype).to(dev()), kc, vc, i32([table]), i32([0]), i32([699]), hd ** -0.5,
+                                           window=window)
+        assert torch.allclose(out[0, 0].float().cpu(), v[target, 0].to(dtype).float(), rtol=1e-2, atol=1e-2) == seen
+
+
 def test_attention_refuses_sizes_it_cannot_take():
     kc = torch.zeros(2, 4, 1, 24, device=dev())
     with pytest.raises(hip().KernelError, match="multiple of 16"):
@@ -265,10 +330,10 @@ def test_silu_mul(dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_copy_slots_copies_the_leading_slots_of_every_layer(dtype):
-    pool = torch.randn(5, 3, 8, 2, 16, generator=gen(14)).to(dtype).to(dev())
+    pool = torch.randn(5, 3, 2, 8, 16, generator=gen(14)).to(dtype).to(dev())   # [pages, layers, heads, slots, dim]
     before = pool.clone()
     hip().copy_slots(pool, 3, 1, 5)
-    assert torch.equal(pool[1, :, :5], before[3, :, :5]) and torch.equal(pool[1, :, 5:], before[1, :, 5:])
+    assert torch.equal(pool[1, :, :, :5], before[3, :, :, :5]) and torch.equal(pool[1, :, :, 5:], before[1, :, :, 5:])
     keep = [0, 2, 3, 4]
     assert torch.equal(pool[keep], before[keep])
     with pytest.raises(hip().KernelError):

@@ -3,8 +3,10 @@ slots of fixed-size per-request state (tinyserve_llm/kvcache/storage.py:5-49 has
 for all layers).
 
 Layers are grouped by the rows they cache (kv heads, head size) and by whether they keep every key
-or a window. A group's pools are laid out [pages, layers of the group, page_size, kv_heads,
-head_dim], page first, so one page of every layer of the group is one contiguous region. All
+or a window. A group's pools are laid out [pages, layers of the group, kv_heads, page_size,
+head_dim]: page first, so one page of every layer of the group is one contiguous region, and
+within a layer a head's slots lie together, so the attention kernels stream a head's keys from
+consecutive memory. All
 full-history groups share page space 0: a page id addresses the pools of each of them. Every
 window group has a page space of its own.
 """
@@ -25,7 +27,7 @@ class LayerGroup:
     kv: KVSpec
     space: int
     owners: list[int]                 # run-order indices of the layer runs whose caches live here
-    k_pool: torch.Tensor              # [pages, len(owners), page_size, kv_heads, head_dim]
+    k_pool: torch.Tensor              # [pages, len(owners), kv_heads, page_size, head_dim]
     v_pool: torch.Tensor
 
 
@@ -70,7 +72,7 @@ class KVStorage:
         self._where: dict[int, tuple[int, int]] = {}       # owner run -> (group, layer within group)
         for kv, s in assigned:
             owners = [e.owner for e in cache_plan if e.kv == kv]
-            shape = (pages[s], len(owners), page_size, kv.num_kv_heads, kv.head_dim)
+            shape = (pages[s], len(owners), kv.num_kv_heads, page_size, kv.head_dim)
             group = LayerGroup(kv, s, owners, torch.zeros(shape, dtype=dtype, device=self.device),
                                torch.zeros(shape, dtype=dtype, device=self.device))
             for j, owner in enumerate(owners):
@@ -82,10 +84,10 @@ class KVStorage:
 
     def layer_cache(self, owner: int) -> tuple[torch.Tensor, torch.Tensor, int]:
         """(k view, v view, page space) of the cache that run `owner` of the order owns; the views
-        are [pages, page_size, kv_heads, head_dim], strided over pages."""
+        are addressed [pages, page_size, kv_heads, head_dim] (a permuted view of the pool)."""
         g, j = self._where[owner]
         group = self.groups[g]
-        return group.k_pool[:, j], group.v_pool[:, j], group.space
+        return group.k_pool[:, j].permute(0, 2, 1, 3), group.v_pool[:, j].permute(0, 2, 1, 3), group.space
 
     def state(self, run: int) -> torch.Tensor | None:
         return self.states.get(run)

@@ -37,7 +37,7 @@ paged_attention_wave_kernel(T* __restrict__ out, const T* __restrict__ q, const 
                             const T* __restrict__ v_cache, const int32_t* __restrict__ block_tables,
                             const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ positions,
                             int num_tokens, int nh, int nkv, int hd, int page_size, int64_t page_stride,
-                            int64_t slot_stride, int max_blocks, float scale, int window) {
+                            int64_t slot_stride, int64_t head_stride, int max_blocks, float scale, int window) {
   __shared__ float q_s[ATT_WAVES][ATT_MAX_HD];
   __shared__ float p_s[ATT_WAVES][TS_WAVE];
   __shared__ int64_t row_s[ATT_WAVES][TS_WAVE];
@@ -63,7 +63,7 @@ paged_attention_wave_kernel(T* __restrict__ out, const T* __restrict__ q, const 
     int64_t rowoff = 0;
     if (valid) {
       const int page = table[key / page_size];
-      rowoff = (int64_t)page * page_stride + (int64_t)(key % page_size) * slot_stride + (int64_t)kvh * hd;
+      rowoff = (int64_t)page * page_stride + (int64_t)(key % page_size) * slot_stride + (int64_t)kvh * head_stride;
       const T* kr = k_cache + rowoff;
       float dot = 0.f;
       for (int d = 0; d < hd; d += Vec<T>::N) {
@@ -107,14 +107,14 @@ paged_attention_wave_kernel(T* __restrict__ out, const T* __restrict__ q, const 
 extern "C" int ts_paged_attention_wave(void* out, const void* q, const void* k_cache, const void* v_cache,
                                        const int32_t* block_tables, const int32_t* seq_of_token,
                                        const int32_t* positions, int num_tokens, int nh, int nkv, int hd,
-                                       int page_size, int64_t page_stride, int64_t slot_stride, int max_blocks,
-                                       float scale, int window, int dtype, hipStream_t stream) {
+                                       int page_size, int64_t page_stride, int64_t slot_stride, int64_t head_stride,
+                                       int max_blocks, float scale, int window, int dtype, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
   if (hd % 16 || hd > ATT_MAX_HD || hd <= 0 || nkv <= 0 || nh % nkv || page_size <= 0 || max_blocks <= 0)
     return TS_BAD_SHAPE;
   // 16-byte key loads need 16-byte aligned rows
   const int64_t elem = dtype == 0 ? 4 : 2;
-  if ((page_stride * elem) % 16 || (slot_stride * elem) % 16) return TS_BAD_SHAPE;
+  if ((page_stride * elem) % 16 || (slot_stride * elem) % 16 || (head_stride * elem) % 16) return TS_BAD_SHAPE;
   const int64_t items = (int64_t)num_tokens * nh;
   const int64_t blocks = (items + ATT_WAVES - 1) / ATT_WAVES;
   if (blocks > 0x7fffffff) return TS_BAD_SHAPE;
@@ -122,11 +122,11 @@ extern "C" int ts_paged_attention_wave(void* out, const void* q, const void* k_c
   if (dtype == 0)
     paged_attention_wave_kernel<float><<<grid, block, 0, stream>>>(
         (float*)out, (const float*)q, (const float*)k_cache, (const float*)v_cache, block_tables, seq_of_token,
-        positions, num_tokens, nh, nkv, hd, page_size, page_stride, slot_stride, max_blocks, scale, window);
+        positions, num_tokens, nh, nkv, hd, page_size, page_stride, slot_stride, head_stride, max_blocks, scale, window);
   else if (dtype == 1)
     paged_attention_wave_kernel<bf16_t><<<grid, block, 0, stream>>>(
         (bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, seq_of_token,
-        positions, num_tokens, nh, nkv, hd, page_size, page_stride, slot_stride, max_blocks, scale, window);
+        positions, num_tokens, nh, nkv, hd, page_size, page_stride, slot_stride, head_stride, max_blocks, scale, window);
   else
     return TS_BAD_DTYPE;
   return ts_check_launch();

@@ -96,7 +96,7 @@ extern "C" int ts_rmsnorm(void* out, void* res_out, const void* x, const void* r
 // fused with the scatter of rotated k and of v into their cache slots.
 //   qkv   [T, (nh + 2*nkv) * hd]   one token's q heads, then k heads, then v heads
 //   q_out [T, nh * hd]
-//   cache element address: page * page_stride + offset * slot_stride + head * hd + d,
+//   cache element address: page * page_stride + offset * slot_stride + head * head_stride + d,
 //   page = slot / page_size, offset = slot % page_size; slot -1 writes nothing.
 // k_cache == null: this layer does not own a cache; only q is rotated.
 // ------------------------------------------------------------------------------------------
@@ -105,7 +105,7 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
                                   const T* __restrict__ qkv, const float* __restrict__ cos_sin,
                                   const int32_t* __restrict__ positions, const int64_t* __restrict__ slots,
                                   int nh, int nkv, int hd, int rotate, int page_size, int64_t page_stride,
-                                  int64_t slot_stride) {
+                                  int64_t slot_stride, int64_t head_stride) {
   const int t = blockIdx.x;
   const int half = hd / 2;
   const int row = (nh + 2 * nkv) * hd;
@@ -140,26 +140,29 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
       y1 = x1 * c - x2 * s;
       y2 = x2 * c + x1 * s;
     }
-    Num<T>::st(k_cache + base + h * hd + j, y1);
-    Num<T>::st(k_cache + base + h * hd + j + half, y2);
+    Num<T>::st(k_cache + base + h * head_stride + j, y1);
+    Num<T>::st(k_cache + base + h * head_stride + j + half, y2);
   }
-  for (int i = threadIdx.x; i < nkv * hd; i += blockDim.x) v_cache[base + i] = vs[i];
+  for (int i = threadIdx.x; i < nkv * hd; i += blockDim.x) {
+    const int h = i / hd;
+    v_cache[base + h * head_stride + (i - h * hd)] = vs[i];
+  }
 }
 
 extern "C" int ts_rope_store(void* q_out, void* k_cache, void* v_cache, const void* qkv, const float* cos_sin,
                              const int32_t* positions, const int64_t* slots, int num_tokens, int nh, int nkv,
                              int hd, int rotate, int page_size, int64_t page_stride, int64_t slot_stride,
-                             int dtype, hipStream_t stream) {
+                             int64_t head_stride, int dtype, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
   if (hd % 2 || nh <= 0 || nkv < 0 || page_size <= 0) return TS_BAD_SHAPE;
   if (dtype == 0)
     rope_store_kernel<float><<<num_tokens, 256, 0, stream>>>((float*)q_out, (float*)k_cache, (float*)v_cache,
                                                              (const float*)qkv, cos_sin, positions, slots, nh, nkv,
-                                                             hd, rotate, page_size, page_stride, slot_stride);
+                                                             hd, rotate, page_size, page_stride, slot_stride, head_stride);
   else if (dtype == 1)
     rope_store_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache,
                                                               (const bf16_t*)qkv, cos_sin, positions, slots, nh, nkv,
-                                                              hd, rotate, page_size, page_stride, slot_stride);
+                                                              hd, rotate, page_size, page_stride, slot_stride, head_stride);
   else
     return TS_BAD_DTYPE;
   return ts_check_launch();
@@ -196,8 +199,9 @@ extern "C" int ts_silu_mul(void* out, const void* gu, int num_tokens, int inter,
 }
 
 // ------------------------------------------------------------------------------------------
-// Copy the first `num_slots` slots of page `src` to page `dst`, for every layer of a pool laid out
-// [pages, layers, page_size, row] (row = kv_heads * head_dim elements of `elem_bytes` bytes).
+// Copy the first `num_slots` slots of page `src` to page `dst` in a pool laid out
+// [pages, runs, page_size, row]: `runs` = layers x kv heads of the group, row = one head's
+// head_dim elements in bytes.
 // ------------------------------------------------------------------------------------------
 __global__ void copy_slots_kernel(uint8_t* __restrict__ pool, int64_t page_bytes, int64_t layer_bytes,
                                   int64_t copy_bytes, int src, int dst) {

@@ -44,10 +44,11 @@ def _declare(lib: ctypes.CDLL) -> None:
     sig = {
         "ts_embedding": [p, p, p, i, i, i, p],
         "ts_rmsnorm": [p, p, p, p, p, p, i, i, f, i, i, p],
-        "ts_rope_store": [p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i, p],
+        "ts_rope_store": [p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i, p],
         "ts_silu_mul": [p, p, i, i, i, p],
         "ts_copy_slots": [p, i, i, i64, i, i, i, p],
-        "ts_paged_attention_wave": [p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i, f, i, i, p],
+        "ts_paged_attention_wave": [p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i, f, i, i, p],
+        "ts_paged_attention_decode": [p, p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i, i, i, f, i, i, p],
         "ts_gemm_exact": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_sample": [p, p, p, p, u64, i, i, i64, p],
     }
@@ -144,28 +145,40 @@ def rope_store(qkv: torch.Tensor, cos_sin: torch.Tensor | None, positions: torch
     if cos_sin is not None:
         _need(cos_sin.dtype == torch.float32 and cos_sin.dim() == 2 and cos_sin.shape[1] == head_dim
               and cos_sin.is_contiguous(), "the rotation table must be float32 [positions, head_dim]")
-    page_size, page_stride, slot_stride = 1, 0, 0
+    page_size, page_stride, slot_stride, head_stride = 1, 0, 0, 0
     if k_cache is not None:
         _need(v_cache is not None and slots is not None, "a cache write needs k, v and the slots")
         _need(slots.dtype == torch.int64 and slots.shape == (T,) and slots.is_contiguous(), "slots must be int64 [tokens]")
         _check_cache(k_cache, v_cache, qkv.dtype, num_kv_heads, head_dim)
         page_size, page_stride, slot_stride = k_cache.shape[1], k_cache.stride(0), k_cache.stride(1)
+        head_stride = k_cache.stride(2)
     q = torch.empty((T, num_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
     _run("rope_store", library().ts_rope_store(
         _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(qkv), _ptr(cos_sin), _ptr(positions), _ptr(slots), T, num_heads,
-        num_kv_heads, head_dim, int(cos_sin is not None), page_size, page_stride, slot_stride, _code(qkv.dtype),
-        _stream()))
+        num_kv_heads, head_dim, int(cos_sin is not None), page_size, page_stride, slot_stride, head_stride,
+        _code(qkv.dtype), _stream()))
     return q
 
 
 def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, dtype: torch.dtype, nkv: int, hd: int) -> None:
+    """A layer's cache is addressed as [pages, page_size, kv_heads, head_dim]; pages, slots and heads
+    may be strided in any order (the engine's pools keep a head's slots together), head_dim is dense."""
     _need(k_cache.dim() == 4 and k_cache.shape[2] == nkv and k_cache.shape[3] == hd,
           f"cache view must be [pages, page_size, {nkv}, {hd}], got {tuple(k_cache.shape)}")
     _need(k_cache.dtype == dtype and v_cache.dtype == dtype, "cache and activations differ in storage type")
     _need(k_cache.shape == v_cache.shape and k_cache.stride() == v_cache.stride(), "k and v caches must be laid out alike")
-    _need(k_cache.stride(3) == 1 and k_cache.stride(2) == hd, "a token's heads must be contiguous in the cache")
-    _need(k_cache.stride(1) >= nkv * hd and k_cache.stride(0) >= k_cache.shape[1] * k_cache.stride(1),
-          "cache slots overlap")
+    _need(k_cache.stride(3) == 1, "head_dim must be contiguous in the cache")
+    pages, page_size = k_cache.shape[0], k_cache.shape[1]
+    # no two (page, slot, head) rows may overlap: sort the three strides and check each spans the next
+    dims = sorted(((k_cache.stride(0), pages), (k_cache.stride(1), page_size), (k_cache.stride(2), nkv)))
+    span = hd
+    for stride, size in dims:
+        if size > 1:
+            _need(stride >= span, "cache rows overlap")
+            span = stride * size
+    itemsize = k_cache.element_size()
+    _need(all((k_cache.stride(i) * itemsize) % 16 == 0 for i in range(3)) and k_cache.data_ptr() % 16 == 0
+          and v_cache.data_ptr() % 16 == 0, "cache rows must be 16-byte aligned")
 
 
 def paged_attention_wave(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -187,8 +200,47 @@ def paged_attention_wave(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.
     out = torch.empty_like(q)
     _run("paged_attention_wave", library().ts_paged_attention_wave(
         _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_of_token), _ptr(positions),
-        T, nh, nkv, hd, k_cache.shape[1], k_cache.stride(0), k_cache.stride(1), block_tables.shape[1], float(scale),
-        int(window), _code(q.dtype), _stream()))
+        T, nh, nkv, hd, k_cache.shape[1], k_cache.stride(0), k_cache.stride(1), k_cache.stride(2),
+        block_tables.shape[1], float(scale), int(window), _code(q.dtype), _stream()))
+    return out
+
+
+def decode_chunk(num_tokens: int, nkv: int, capacity: int) -> int:
+    """Keys per workgroup of the split-key kernel: the largest of 256/128/64 that still gives the
+    GPU's 256 compute units a few workgroups each."""
+    for chunk in (256, 128):
+        if num_tokens * nkv * -(-capacity // chunk) >= 1024:
+            return chunk
+    return 64
+
+
+def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                           seq_of_token: torch.Tensor, positions: torch.Tensor, scale: float, window: int = 0,
+                           chunk: int | None = None) -> torch.Tensor:
+    """Split-key attention for tokens that each bring one query. Every position in `positions`
+    must lie inside the pages its row of `block_tables` has (checked by the caller on the host)."""
+    _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions)
+    _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
+    T, nh, hd = q.shape
+    nkv = k_cache.shape[2]
+    _check_cache(k_cache, v_cache, q.dtype, nkv, hd)
+    _need(hd % 16 == 0 and hd <= 256, f"head_dim {hd} is not a multiple of 16 up to 256")
+    _need(nh % nkv == 0 and nh // nkv <= 8, f"{nh} heads over {nkv} key/value heads: groups of up to 8 are served")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
+          "block_tables must be contiguous int32 [requests, pages]")
+    for name, t in (("seq_of_token", seq_of_token), ("positions", positions)):
+        _need(t.dtype == torch.int32 and t.shape == (T,) and t.is_contiguous(), f"{name} must be int32 [tokens]")
+    _need(T <= 65535, "at most 65535 tokens per launch")
+    capacity = block_tables.shape[1] * k_cache.shape[1]
+    chunk = chunk or decode_chunk(T, nkv, capacity)
+    splits = -(-capacity // chunk)
+    part_o = torch.empty((T, nh, splits, hd), dtype=torch.float32, device=q.device)
+    part_ml = torch.empty((T, nh, splits, 2), dtype=torch.float32, device=q.device)
+    out = torch.empty_like(q)
+    _run("paged_attention_decode", library().ts_paged_attention_decode(
+        _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
+        _ptr(seq_of_token), _ptr(positions), T, nh, nkv, hd, k_cache.shape[1], k_cache.stride(0), k_cache.stride(1),
+        k_cache.stride(2), block_tables.shape[1], splits, chunk, float(scale), int(window), _code(q.dtype), _stream()))
     return out
 
 
@@ -219,15 +271,16 @@ def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
 
 
 def copy_slots(pool: torch.Tensor, src: int, dst: int, num_slots: int) -> None:
-    """pool[dst, :, :num_slots] = pool[src, :, :num_slots] for a contiguous pool
-    [pages, layers, page_size, kv_heads, head_dim]."""
+    """pool[dst, ..., :num_slots, :] = pool[src, ..., :num_slots, :] for a contiguous pool
+    [pages, layers, kv_heads, page_size, head_dim]."""
     _gpu(pool)
-    _need(pool.dim() == 5 and pool.is_contiguous(), "pool must be contiguous [pages, layers, page_size, heads, dim]")
-    pages, layers, page_size = pool.shape[:3]
+    _need(pool.dim() == 5 and pool.is_contiguous(), "pool must be contiguous [pages, layers, heads, page_size, dim]")
+    pages, layers, heads, page_size = pool.shape[:4]
     _need(0 <= src < pages and 0 <= dst < pages and src != dst, f"pages {src}->{dst} outside 0..{pages - 1}")
     _need(0 <= num_slots <= page_size, f"{num_slots} slots do not fit a page of {page_size}")
-    row_bytes = pool.shape[3] * pool.shape[4] * pool.element_size()
-    _run("copy_slots", library().ts_copy_slots(_ptr(pool), layers, page_size, row_bytes, src, dst, num_slots, _stream()))
+    row_bytes = pool.shape[4] * pool.element_size()
+    _run("copy_slots", library().ts_copy_slots(_ptr(pool), layers * heads, page_size, row_bytes, src, dst, num_slots,
+                                               _stream()))
 
 
 def sample(logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor, seed: int) -> torch.Tensor:
@@ -249,7 +302,11 @@ def sample(logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor,
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx, space: int,
                     scale: float, window: int = 0) -> torch.Tensor:
-    """Attention of a packed step over the cache; picks the kernel for the storage type and shape."""
+    """Attention of a packed step over the cache; picks the kernel for the storage type and shape.
+    float32 always takes the one-wave-per-row kernel, whose sums do not depend on the batch."""
+    if q.dtype == torch.bfloat16 and ctx.max_query_len == 1 and q.shape[1] // k_cache.shape[2] <= 8:
+        return paged_attention_decode(q, k_cache, v_cache, ctx.block_tables[space], ctx.seq_of_token, ctx.positions,
+                                      scale, window)
     return paged_attention_wave(q, k_cache, v_cache, ctx.block_tables[space], ctx.seq_of_token, ctx.positions,
                                 scale, window)
 
