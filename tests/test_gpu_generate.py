@@ -204,3 +204,28 @@ def test_command_line_writes_one_record(folder_a, tmp_path):
     plain = PlainLlama(folder_a, torch.float64)
     assert [c["token_ids"][0] for c in record["completions"]] == [plain.greedy([5, 17, 3], 5), plain.greedy([77, 2, 9], 5)]
     assert record["output_tokens"] == 10 and "wrote" in r.stdout
+
+
+def test_decode_graphs_replay_what_eager_steps_compute(folder_b):
+    """Decode steps come from HIP graphs (one per batch size, idle rows above eight requests);
+    prompts and mixed steps run eagerly in between. Every replay must give what the eager engine
+    gives: float32 logits are bit-equal, so the tokens are."""
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+    sc = SchedulerConfig(max_model_len=128, max_num_seqs=16, max_num_batched_tokens=80, max_prefill_chunk=32)
+    prompts = [prompt(40 + i, 3 + 7 * i, 384) for i in range(13)]
+    params = [SamplingParams(max_tokens=4 + 3 * (i % 5), temperature=0.8 if i % 2 else 0.0, ignore_eos=True) for i in range(13)]
+    outs = []
+    for graphs in (True, False):
+        llm = LLM(folder_b, sc, CacheConfig(block_size=16), dtype=torch.float32, num_blocks=120, seed=5, decode_graphs=graphs)
+        assert (llm.runner.graphs is not None) == graphs
+        outs.append([r.token_ids for r in llm.generate(prompts, params)])
+        if graphs:
+            sizes = sorted({size for size, width in llm.runner.graphs.graphs})
+            assert len(sizes) >= 3 and 16 in sizes, f"several batch sizes were captured, a padded one among them: {sizes}"
+            again = [r.token_ids for r in llm.generate(prompts, params)]      # replays of graphs captured before
+            # new request ids give new noise keys: only the greedy requests repeat exactly
+            assert [a for a, p in zip(again, params) if not p.temperature] == \
+                [a for a, p in zip(outs[0], params) if not p.temperature]
+    assert outs[0] == outs[1]

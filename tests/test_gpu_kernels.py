@@ -214,24 +214,25 @@ def test_attention_window_edge(dtype):
         assert is_it == seen
 
 
-def head_major(k, v, table, page, pages, dtype):
-    """The engine's own pool layout: [pages, kv_heads, page_size, head_dim] seen as [pages, page_size, kv_heads, head_dim]."""
+def engine_layout(k, v, table, page, pages, dtype):
+    """The engine's own pools: keys [pages, kv_heads, page_size, head_dim], values transposed
+    [pages, kv_heads, head_dim, page_size], both seen as [pages, page_size, kv_heads, head_dim]."""
     g = gen(19)
     kp = torch.randn(pages, k.shape[1], page, k.shape[2], generator=g).to(dtype)
-    vp = torch.randn(pages, k.shape[1], page, k.shape[2], generator=g).to(dtype)
+    vp = torch.randn(pages, k.shape[1], k.shape[2], page, generator=g).to(dtype)
     for p in range(k.shape[0]):
         kp[table[p // page], :, p % page] = k[p]
-        vp[table[p // page], :, p % page] = v[p]
-    return kp.to(dev()).permute(0, 2, 1, 3), vp.to(dev()).permute(0, 2, 1, 3)
+        vp[table[p // page], :, :, p % page] = v[p]
+    return kp.to(dev()).permute(0, 2, 1, 3), vp.to(dev()).permute(0, 3, 1, 2)
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,kv,hd,page", [(4, 2, 16, 4), (3, 1, 32, 16), (6, 2, 48, 8), (32, 8, 64, 256),
-                                              (5, 5, 128, 32), (8, 1, 256, 16), (24, 8, 128, 64)])
-@pytest.mark.parametrize("chunk", [64, 128, 256])
-def test_split_key_decode_attention(dtype, heads, kv, hd, page, chunk):
-    """One query per request at different context lengths (1, a chunk's edge, mid-chunk, long), on
-    both cache layouts, against the dense formula."""
+@pytest.mark.parametrize("heads,kv,hd,page", [(3, 1, 32, 16), (6, 2, 96, 8), (32, 8, 64, 256), (5, 5, 128, 32),
+                                              (16, 1, 128, 64), (24, 8, 128, 64), (14, 2, 64, 24)])
+@pytest.mark.parametrize("chunk", [128, 256])
+def test_split_key_decode_attention(heads, kv, hd, page, chunk):
+    """One query per request at different context lengths (1, a chunk's edge, mid-chunk, long)
+    against the dense formula and against the wave kernel on the same pages."""
+    dtype = torch.bfloat16
     n = 600
     g = gen(hd + chunk)
     q = torch.randn(n, heads, hd, generator=g).to(dtype)
@@ -239,25 +240,91 @@ def test_split_key_decode_attention(dtype, heads, kv, hd, page, chunk):
     pages = -(-n // page)
     table = list(range(pages - 1, -1, -1))
     dense = P.causal_attention(q.double(), k.double(), v.double())
-    rows = [0, 1, chunk - 1, chunk, chunk + 1, 255, 256, 257, 400, 599]
+    rows = [0, 1, 31, 32, chunk - 1, chunk, chunk + 1, 255, 256, 257, 400, 599]
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev())
-    for kc, vc in (scattered(k, v, table, page, pages, dtype), head_major(k, v, table, page, pages, dtype)):
-        out = hip().paged_attention_decode(q[rows].to(dev()), kc, vc, i32([table, table]), i32([0, 1] * 5), i32(rows),
-                                           hd ** -0.5, chunk=chunk)
-        torch.testing.assert_close(out.double().cpu(), dense[rows], **tol(dtype))
+    kc, vc = engine_layout(k, v, table, page, pages, dtype)
+    assert hip().decode_kernel_takes(q[rows].to(dev()), kc, vc)
+    out = hip().paged_attention_decode(q[rows].to(dev()), kc, vc, i32([table, table]), i32([0, 1] * 6), i32(rows),
+                                       hd ** -0.5, chunk=chunk)
+    torch.testing.assert_close(out.double().cpu(), dense[rows], **tol(dtype))
     wave = run_attention(q[rows], kc, vc, [table], [0] * len(rows), rows, hd ** -0.5)
     torch.testing.assert_close(out.float(), wave.float(), **tol(dtype))
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-def test_split_key_decode_window_and_far_key(dtype):
+@pytest.mark.parametrize("heads,kv,hd,page", [(3, 1, 32, 16), (6, 2, 96, 8), (32, 8, 64, 256), (5, 5, 128, 32),
+                                              (16, 1, 128, 64), (14, 2, 64, 24)])
+def test_matrix_core_prefill_attention(heads, kv, hd, page):
+    """A packed step of three requests on shared pools: a whole prompt, a portion over a cached
+    prefix, and single decoded tokens; tiles never cross a request."""
+    dtype = torch.bfloat16
+    g = gen(hd * 3 + page)
+    lens = [150, 77, 300]                       # keys each request has after the step
+    fed = [150, 9, 1]                           # tokens of each in the step
+    q_all, k_all, v_all = [], [], []
+    pages_each = [-(-n // page) for n in lens]
+    total_pages = sum(pages_each) + 1
+    kp = torch.randn(total_pages, kv, page, hd, generator=g).to(dtype)
+    vp = torch.randn(total_pages, kv, hd, page, generator=g).to(dtype)
+    tables, nxt = [], 1
+    for n, pe in zip(lens, pages_each):
+        table = list(range(nxt + pe - 1, nxt - 1, -1))
+        nxt += pe
+        tables.append(table)
+        k, v = torch.randn(n, kv, hd, generator=g).to(dtype), torch.randn(n, kv, hd, generator=g).to(dtype)
+        for p_ in range(n):
+            kp[table[p_ // page], :, p_ % page] = k[p_]
+            vp[table[p_ // page], :, :, p_ % page] = v[p_]
+        q_all.append(torch.randn(n, heads, hd, generator=g).to(dtype))
+        k_all.append(k)
+        v_all.append(v)
+    width = max(pages_each)
+    padded = [t + [0] * (width - len(t)) for t in tables]
+    q_step = torch.cat([q_all[i][lens[i] - fed[i]:] for i in range(3)])
+    seq_of = sum(([i] * fed[i] for i in range(3)), [])
+    positions = sum((list(range(lens[i] - fed[i], lens[i])) for i in range(3)), [])
+    cu = [0, fed[0], fed[0] + fed[1], sum(fed)]
+    per_tile = 16 // (heads // kv)
+    flat = hip().attention_tiles(cu, per_tile)
+    assert all(flat[2 * i + 1] <= per_tile for i in range(len(flat) // 2))
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev())
+    kc, vc = kp.to(dev()).permute(0, 2, 1, 3), vp.to(dev()).permute(0, 3, 1, 2)
+    out = hip().paged_attention_prefill(q_step.to(dev()), kc, vc, i32(padded), i32(seq_of), i32(positions),
+                                        i32(flat).view(-1, 2), hd ** -0.5)
+    want = torch.cat([P.causal_attention(q_all[i].double(), k_all[i].double(), v_all[i].double())[lens[i] - fed[i]:]
+                      for i in range(3)])
+    torch.testing.assert_close(out.double().cpu(), want, **tol(dtype))
+    wave = run_attention(q_step, kc, vc, padded, seq_of, positions, hd ** -0.5)
+    torch.testing.assert_close(out.float(), wave.float(), **tol(dtype))
+    win = hip().paged_attention_prefill(q_step.to(dev()), kc, vc, i32(padded), i32(seq_of), i32(positions),
+                                        i32(flat).view(-1, 2), hd ** -0.5, window=40)
+    want = torch.cat([P.causal_attention(q_all[i].double(), k_all[i].double(), v_all[i].double(), window=40)[lens[i] - fed[i]:]
+                      for i in range(3)])
+    torch.testing.assert_close(win.double().cpu(), want, **tol(dtype))
+
+
+def test_decode_kernel_leaves_other_shapes_to_the_wave_kernel():
+    q = torch.zeros(2, 4, 48, dtype=torch.bfloat16, device=dev())
+    kc = torch.zeros(3, 2, 16, 48, dtype=torch.bfloat16, device=dev()).permute(0, 2, 1, 3)
+    vc = torch.zeros(3, 2, 48, 16, dtype=torch.bfloat16, device=dev()).permute(0, 3, 1, 2)
+    assert not hip().decode_kernel_takes(q, kc, vc), "head_dim 48"
+    q64 = torch.zeros(2, 4, 64, dtype=torch.bfloat16, device=dev())
+    plain = torch.zeros(3, 16, 2, 64, dtype=torch.bfloat16, device=dev())
+    assert not hip().decode_kernel_takes(q64, plain, plain), "values not in transposed pages"
+    assert not hip().decode_kernel_takes(q64.float(), plain.float(), plain.float()), "float32"
+    with pytest.raises(hip().KernelError, match="decode kernel takes"):
+        hip().paged_attention_decode(q, kc, vc, torch.zeros(1, 3, dtype=torch.int32, device=dev()),
+                                     torch.zeros(2, dtype=torch.int32, device=dev()), torch.zeros(2, dtype=torch.int32, device=dev()), 1.0)
+
+
+def test_split_key_decode_window_and_far_key():
+    dtype = torch.bfloat16
     n, heads, kv, hd, page, window = 700, 4, 2, 64, 64, 300
     g = gen(21)
     q = torch.randn(n, heads, hd, generator=g) * 0.1
     k, v = torch.randn(n, kv, hd, generator=g) * 0.1, torch.randn(n, kv, hd, generator=g)
     table = list(range(10, -1, -1))
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev())
-    kc, vc = head_major(k.to(dtype), v.to(dtype), table, page, 11, dtype)
+    kc, vc = engine_layout(k.to(dtype), v.to(dtype), table, page, 11, dtype)
     rows = [5, 299, 300, 301, 699]
     want = P.causal_attention(q.to(dtype).double(), k.to(dtype).double(), v.to(dtype).double(), window=window)[rows]
     out = hip().paged_attention_decode(q[rows].to(dtype).to(dev()), kc, vc, i32([table]), i32([0] * 5), i32(rows),
@@ -269,7 +336,7 @@ def test_split_key_decode_window_and_far_key(dtype):
         kk[target, :, 5] = 40.0
         qq = q[[699]].clone()
         qq[:, :, 5] = 40.0
-        kc, vc = head_major(kk.to(dtype), v.to(dtype), table, page, 11, dtype)
+        kc, vc = engine_layout(kk.to(dtype), v.to(dtype), table, page, 11, dtype)
         out = hip().paged_attention_decode(qq.to(dtype).to(dev()), kc, vc, i32([table]), i32([0]), i32([699]), hd ** -0.5)
         for h in range(heads):
             torch.testing.assert_close(out[0, h].float().cpu(), v[target, h // 2].to(dtype).float(), rtol=1e-3, atol=1e-3)
@@ -277,6 +344,17 @@ def test_split_key_decode_window_and_far_key(dtype):
         out = hip().paged_attention_decode(qq.to(dtype).to(dev()), kc, vc, i32([table]), i32([0]), i32([699]), hd ** -0.5,
                                            window=window)
         assert torch.allclose(out[0, 0].float().cpu(), v[target, 0].to(dtype).float(), rtol=1e-2, atol=1e-2) == seen
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_wave_kernel_reads_the_engine_layout(dtype):
+    n, heads, kv, hd, page = 100, 6, 3, 48, 16
+    g = gen(23)
+    q, k, v = (torch.randn(n, h, hd, generator=g).to(dtype) for h in (heads, kv, kv))
+    table = list(range(6, -1, -1))
+    kc, vc = engine_layout(k, v, table, page, 7, dtype)
+    out = run_attention(q, kc, vc, [table], [0] * n, list(range(n)), hd ** -0.5)
+    torch.testing.assert_close(out.double().cpu(), P.causal_attention(q.double(), k.double(), v.double()), **tol(dtype))
 
 
 def test_attention_refuses_sizes_it_cannot_take():
@@ -330,16 +408,21 @@ def test_silu_mul(dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_copy_slots_copies_the_leading_slots_of_every_layer(dtype):
-    pool = torch.randn(5, 3, 2, 8, 16, generator=gen(14)).to(dtype).to(dev())   # [pages, layers, heads, slots, dim]
+    pool = torch.randn(5, 3, 2, 8, 16, generator=gen(14)).to(dtype).to(dev())   # [pages, x, heads, slots, dim]
     before = pool.clone()
-    hip().copy_slots(pool, 3, 1, 5)
+    hip().copy_slots(pool, 3, 1, 5, slot_dim=3)
     assert torch.equal(pool[1, :, :, :5], before[3, :, :, :5]) and torch.equal(pool[1, :, :, 5:], before[1, :, :, 5:])
     keep = [0, 2, 3, 4]
     assert torch.equal(pool[keep], before[keep])
+    vpool = torch.randn(5, 3, 2, 16, 8, generator=gen(15)).to(dtype).to(dev())  # [pages, layers, heads, dim, slots]
+    vbefore = vpool.clone()
+    hip().copy_slots(vpool, 3, 1, 5, slot_dim=4)
+    assert torch.equal(vpool[1, ..., :5], vbefore[3, ..., :5]) and torch.equal(vpool[1, ..., 5:], vbefore[1, ..., 5:])
+    assert torch.equal(vpool[keep], vbefore[keep])
     with pytest.raises(hip().KernelError):
-        hip().copy_slots(pool, 3, 3, 2)
+        hip().copy_slots(pool, 3, 3, 2, slot_dim=3)
     with pytest.raises(hip().KernelError):
-        hip().copy_slots(pool, 0, 5, 2)
+        hip().copy_slots(pool, 0, 5, 2, slot_dim=3)
 
 
 def exp_noise(seed, key, n):

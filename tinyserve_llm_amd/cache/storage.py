@@ -3,10 +3,13 @@ slots of fixed-size per-request state (tinyserve_llm/kvcache/storage.py:5-49 has
 for all layers).
 
 Layers are grouped by the rows they cache (kv heads, head size) and by whether they keep every key
-or a window. A group's pools are laid out [pages, layers of the group, kv_heads, page_size,
-head_dim]: page first, so one page of every layer of the group is one contiguous region, and
-within a layer a head's slots lie together, so the attention kernels stream a head's keys from
-consecutive memory. All
+or a window. A group's key pool is laid out [layers of the group, pages, kv_heads, page_size,
+head_dim]: layer first, because a step reads one layer's pages at a time and reads them faster
+from one compact region (the reference's pool is page first, to copy a page in one piece); within a
+page a head's slots lie together, so the attention kernels stream a head's keys from consecutive
+memory. The value pool is [layers, pages, kv_heads, head_dim, page_size]: pages hold values
+transposed, because the matrix-core product P·V wants, for one dimension, consecutive keys side by
+side. All
 full-history groups share page space 0: a page id addresses the pools of each of them. Every
 window group has a page space of its own.
 """
@@ -27,8 +30,8 @@ class LayerGroup:
     kv: KVSpec
     space: int
     owners: list[int]                 # run-order indices of the layer runs whose caches live here
-    k_pool: torch.Tensor              # [pages, len(owners), kv_heads, page_size, head_dim]
-    v_pool: torch.Tensor
+    k_pool: torch.Tensor              # [len(owners), pages, kv_heads, page_size, head_dim]
+    v_pool: torch.Tensor              # [len(owners), pages, kv_heads, head_dim, page_size]
 
 
 def plan_spaces(kv_specs: list[KVSpec]) -> tuple[list[tuple[KVSpec, int]], int]:
@@ -72,9 +75,10 @@ class KVStorage:
         self._where: dict[int, tuple[int, int]] = {}       # owner run -> (group, layer within group)
         for kv, s in assigned:
             owners = [e.owner for e in cache_plan if e.kv == kv]
-            shape = (pages[s], len(owners), kv.num_kv_heads, page_size, kv.head_dim)
-            group = LayerGroup(kv, s, owners, torch.zeros(shape, dtype=dtype, device=self.device),
-                               torch.zeros(shape, dtype=dtype, device=self.device))
+            k_shape = (len(owners), pages[s], kv.num_kv_heads, page_size, kv.head_dim)
+            v_shape = (len(owners), pages[s], kv.num_kv_heads, kv.head_dim, page_size)
+            group = LayerGroup(kv, s, owners, torch.zeros(k_shape, dtype=dtype, device=self.device),
+                               torch.zeros(v_shape, dtype=dtype, device=self.device))
             for j, owner in enumerate(owners):
                 self._where[owner] = (len(self.groups), j)
             self.groups.append(group)
@@ -87,7 +91,7 @@ class KVStorage:
         are addressed [pages, page_size, kv_heads, head_dim] (a permuted view of the pool)."""
         g, j = self._where[owner]
         group = self.groups[g]
-        return group.k_pool[:, j].permute(0, 2, 1, 3), group.v_pool[:, j].permute(0, 2, 1, 3), group.space
+        return group.k_pool[j].permute(0, 2, 1, 3), group.v_pool[j].permute(0, 3, 1, 2), group.space
 
     def state(self, run: int) -> torch.Tensor | None:
         return self.states.get(run)
@@ -95,8 +99,9 @@ class KVStorage:
     def copy_slots(self, space: int, src: int, dst: int, num_slots: int) -> None:
         for group in self.groups:
             if group.space == space:
-                hip.copy_slots(group.k_pool, src, dst, num_slots)
-                hip.copy_slots(group.v_pool, src, dst, num_slots)
+                for j in range(len(group.owners)):
+                    hip.copy_slots(group.k_pool[j], src, dst, num_slots, slot_dim=2)
+                    hip.copy_slots(group.v_pool[j], src, dst, num_slots, slot_dim=3)
 
     def copy_state(self, src_slot: int, dst_slot: int) -> None:
         for t in self.states.values():

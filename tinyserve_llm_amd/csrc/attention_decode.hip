@@ -1,268 +1,195 @@
-// Split-key paged attention for tokens that each bring one query (decoding): a workgroup takes one
-// (token, key/value head, chunk of keys) and serves all query heads of that key/value head's group
-// from one pass over the chunk, so the cache is read once. Partial results (unnormalised output,
-// running max and sum per chunk) go to a 32-bit workspace; a second kernel combines the chunks of a
-// token in ascending order. The chunk size is chosen on the host (64, 128 or 256 keys) so that few
-// tokens still fill the GPU; chunk boundaries are multiples of it counted from position 0.
-// Scores, softmax and sums are 32-bit whatever the storage type.
-#include "common.h"
+// Split-key paged attention on the matrix cores for tokens that each bring one query (decoding),
+// bfloat16. A workgroup takes one (token, key/value head, chunk of keys) and serves all query heads
+// of that key/value head's group; its four waves take a quarter of the chunk each and work through
+// it 32 keys at a time:
+//     S^T[key, head] = K[key, :] · Q[head, :]      v_mfma_f32_16x16x16_bf16, keys as rows
+//     online softmax per head (32-bit), P = exp(S - max)
+//     O[head, :]    += P[head, key] · V[key, :]
+// The result layout of the first product is the operand layout of the second, so P never leaves
+// its registers. Keys are read as 16-byte pieces of their rows; values are read from pages that
+// hold them transposed ([head_dim, page_size] per head), so that the four consecutive keys an
+// operand needs lie side by side in memory. The waves' partial results meet in LDS; a chunk's
+// unnormalised output with its running max and sum goes to a 32-bit workspace, and a second
+// kernel combines the chunks of a token in ascending order. Chunk boundaries are multiples of
+// the chunk size counted from position 0.
+#include "attention_mfma.h"
 
 #define DEC_THREADS 256
+#define DEC_WAVES 4
 
-template <typename T> struct Row;   // vector loads of cache rows
-template <> struct Row<float> {
-  static constexpr int K = 4;       // elements per 16-byte key load
-  static __device__ __forceinline__ void ldk(const float* p, float* o) {
-    const float4 v = *(const float4*)p;
-    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
-  }
-  static __device__ __forceinline__ void ldv4(const float* p, float* o) {
-    const float4 v = *(const float4*)p;
-    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
-  }
-};
-template <> struct Row<bf16_t> {
-  static constexpr int K = 8;
-  static __device__ __forceinline__ void ldk(const bf16_t* p, float* o) {
-    const uint4 v = *(const uint4*)p;
-    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      o[2 * i] = __uint_as_float(w[i] << 16);
-      o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
-    }
-  }
-  static __device__ __forceinline__ void ldv4(const bf16_t* p, float* o) {
-    const uint2 v = *(const uint2*)p;
-    o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
-    o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
-  }
-};
-
-// dynamic shared memory layout (floats unless noted):
-//   q_s   [G * hd]
-//   sc    [G * chunk]            scores, then probabilities
-//   ml    [2 * G]
-//   red   [nslices * G * hd]
-//   rowo  [chunk] int64          element offset of each key's row
-template <typename T, int G>
+template <int HD>
 __global__ void __launch_bounds__(DEC_THREADS)
-attn_decode_split_kernel(float* __restrict__ part_o, float* __restrict__ part_ml, const T* __restrict__ q,
-                         const T* __restrict__ k_cache, const T* __restrict__ v_cache,
-                         const int32_t* __restrict__ block_tables, const int32_t* __restrict__ seq_of_token,
-                         const int32_t* __restrict__ positions, int nh, int hd, int page_size, int64_t page_stride,
-                         int64_t slot_stride, int64_t head_stride, int max_blocks, int num_splits, int chunk, int tpk,
-                         float scale, int window) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  const int tid = threadIdx.x;
+attn_decode_mfma_kernel(float* __restrict__ part_o, float* __restrict__ part_ml, const bf16_t* __restrict__ q,
+                        const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+                        const int32_t* __restrict__ block_tables, const int32_t* __restrict__ seq_of_token,
+                        const int32_t* __restrict__ positions, int nh, int G, int page_size, int page_shift,
+                        int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
+                        int num_splits, int chunk, float scale2, int window) {
+  constexpr int NC = HD / 32;    // 32-dimension pieces of a key row (one 16-byte load per lane each)
+  constexpr int NDB = HD / 16;   // 16-dimension blocks of the output
+  extern __shared__ __align__(16) float smem[];
+  float* wm = smem;                       // [waves][16]
+  float* wl = wm + DEC_WAVES * 16;        // [waves][16]
+  float* wo = wl + DEC_WAVES * 16;        // [waves][G][HD]
+
+  const int tid = threadIdx.x, wave = tid / TS_WAVE, lane = tid & (TS_WAVE - 1);
+  const int r = lane & 15, g = lane >> 4;
   const int split = blockIdx.x, kvh = blockIdx.y, t = blockIdx.z;
   const int pos = positions[t];
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int k0 = split * chunk;
-  if (k0 > pos || k0 + chunk <= lo) return;   // the whole workgroup leaves: nothing of this chunk is visible
-  const int tpr = hd / 4;                      // threads per value row (4 elements each)
-  const int nslices = DEC_THREADS / tpr;
-
-  int64_t* rowo = (int64_t*)smem;
-  float* q_s = (float*)(rowo + chunk);
-  float* sc = q_s + G * hd;
-  float* ml = sc + G * chunk;
-  float* red = ml + 2 * G;
-
+  if (k0 > pos || k0 + chunk <= lo) return;     // nothing of this chunk is visible
   const int32_t* table = block_tables + (int64_t)seq_of_token[t] * max_blocks;
-  const T* qrow = q + ((int64_t)t * nh + (int64_t)kvh * G) * hd;
-  for (int i = tid; i < G * hd; i += DEC_THREADS) q_s[i] = Num<T>::ld(qrow + i);
-  __syncthreads();
+  const PageMath pm{page_size, page_shift};
 
-  // ---- scores: `tpk` threads share a key, each takes hd / tpk dimensions
-  {
-    const int kidx = tid / tpk, part = tid - kidx * tpk;
-    const int key = k0 + kidx;
-    const bool valid = kidx < chunk && key <= pos && key >= lo;
-    float dots[G];
+  uint4 qreg[NC];
 #pragma unroll
-    for (int g = 0; g < G; ++g) dots[g] = 0.f;
-    int64_t off = 0;
-    if (valid) {
-      const int page = table[key / page_size];
-      off = (int64_t)page * page_stride + (int64_t)(key % page_size) * slot_stride + (int64_t)kvh * head_stride;
-      const int span = hd / tpk, d0 = part * span;
-      const T* kr = k_cache + off + d0;
-      for (int d = 0; d < span; d += Row<T>::K) {
-        float kv[Row<T>::K];
-        Row<T>::ldk(kr + d, kv);
+  for (int c = 0; c < NC; ++c) qreg[c] = make_uint4(0, 0, 0, 0);
+  if (r < G) {
+    const bf16_t* qrow = q + ((int64_t)t * nh + (int64_t)kvh * G + r) * HD + 8 * g;
 #pragma unroll
-        for (int g = 0; g < G; ++g) {
-          const float* qg = q_s + g * hd + d0 + d;
-#pragma unroll
-          for (int i = 0; i < Row<T>::K; ++i) dots[g] = fmaf(qg[i], kv[i], dots[g]);
-        }
-      }
-    }
-    // the tpk threads of a key are neighbouring lanes of one wave
-    for (int o = 1; o < tpk; o <<= 1) {
-#pragma unroll
-      for (int g = 0; g < G; ++g) dots[g] += __shfl_xor(dots[g], o, TS_WAVE);
-    }
-    if (kidx < chunk && part == 0) {
-      rowo[kidx] = off;
-#pragma unroll
-      for (int g = 0; g < G; ++g) sc[g * chunk + kidx] = valid ? dots[g] * scale : -INFINITY;
-    }
+    for (int c = 0; c < NC; ++c) qreg[c] = *(const uint4*)(qrow + 32 * c);
   }
-  __syncthreads();
+  float m = -INFINITY, l = 0.f;
+  float4_t o[NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db) o[db] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
-  // ---- softmax over the chunk, one wave per query head at a time
-  {
-    const int wave = tid / TS_WAVE, lane = tid & (TS_WAVE - 1);
-    for (int g = wave; g < G; g += DEC_THREADS / TS_WAVE) {
-      float m = -INFINITY;
-      for (int j = lane; j < chunk; j += TS_WAVE) m = fmaxf(m, sc[g * chunk + j]);
-      m = wave_max(m);
-      float l = 0.f;
-      for (int j = lane; j < chunk; j += TS_WAVE) {
-        const float s = sc[g * chunk + j];
-        const float p = s == -INFINITY ? 0.f : expf(s - m);
-        sc[g * chunk + j] = p;
-        l += p;
-      }
-      l = wave_sum(l);
-      if (lane == 0) { ml[2 * g] = m; ml[2 * g + 1] = l; }
+  // this wave's keys, 32 at a time; the next step's loads are issued before this step's products
+  const int kpw = chunk / DEC_WAVES;
+  int kb = k0 + wave * kpw;
+  int kend = kb + kpw;
+  if (kend > pos + 1) kend = pos + 1;
+  if (kb < (lo & ~31)) kb = lo & ~31;
+#define TS_LOAD(T, KB) load_tile<HD>(T, KB, r, g, lo, pos, kvh, table, pm, k_cache, v_cache, kp, ks, kh, vp, vh, vd)
+#define TS_USE(T, KB) use_tile<HD>(T, KB, g, lo, pos, qreg, scale2, m, l, o)
+  if (kb < kend) {
+    KVTile<HD> A, B;
+    TS_LOAD(A, kb);
+    while (true) {
+      const bool more_b = kb + 32 < kend;
+      if (more_b) TS_LOAD(B, kb + 32);
+      TS_USE(A, kb);
+      if (!more_b) break;
+      kb += 32;
+      const bool more_a = kb + 32 < kend;
+      if (more_a) TS_LOAD(A, kb + 32);
+      TS_USE(B, kb);
+      if (!more_a) break;
+      kb += 32;
+    }
+  }
+#undef TS_LOAD
+#undef TS_USE
+  // ---- the four waves meet
+  if (g == 0) { wm[wave * 16 + r] = m; wl[wave * 16 + r] = l; }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int head = 4 * g + j;
+    if (head < G) {
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) wo[((int64_t)wave * G + head) * HD + 16 * db + r] = o[db][j];
     }
   }
   __syncthreads();
-
-  // ---- weighted sum of values: thread = (slice of keys, 4 dimensions)
-  {
-    const int slice = tid / tpr, c = (tid - slice * tpr) * 4;
-    if (slice < nslices) {
-      float acc[G][4];
+  for (int i = tid; i < G * HD; i += DEC_THREADS) {
+    const int head = i / HD, d = i - head * HD;
+    float M = -INFINITY;
 #pragma unroll
-      for (int g = 0; g < G; ++g)
+    for (int w = 0; w < DEC_WAVES; ++w) M = fmaxf(M, wm[w * 16 + head]);
+    float acc = 0.f, L = 0.f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[g][i] = 0.f;
-      const int first = lo > k0 ? lo - k0 : 0;
-      const int last = pos - k0 < chunk - 1 ? pos - k0 : chunk - 1;
-      for (int j = first + slice; j <= last; j += nslices) {
-        float v[4];
-        Row<T>::ldv4(v_cache + rowo[j] + c, v);
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-          const float p = sc[g * chunk + j];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) acc[g][i] = fmaf(p, v[i], acc[g][i]);
-        }
-      }
-#pragma unroll
-      for (int g = 0; g < G; ++g)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) red[((int64_t)slice * G + g) * hd + c + i] = acc[g][i];
+    for (int w = 0; w < DEC_WAVES; ++w) {
+      const float wgt = fast_exp2(wm[w * 16 + head] - M);
+      acc = fmaf(wo[((int64_t)w * G + head) * HD + d], wgt, acc);
+      L = fmaf(wl[w * 16 + head], wgt, L);
     }
-  }
-  __syncthreads();
-  for (int i = tid; i < G * hd; i += DEC_THREADS) {
-    float sum = 0.f;
-    for (int s = 0; s < nslices; ++s) sum += red[(int64_t)s * G * hd + i];
-    const int g = i / hd, d = i - g * hd;
-    part_o[(((int64_t)t * nh + kvh * G + g) * num_splits + split) * hd + d] = sum;
-  }
-  if (tid < 2 * G) {
-    const int g = tid >> 1;
-    part_ml[(((int64_t)t * nh + kvh * G + g) * num_splits + split) * 2 + (tid & 1)] = ml[tid];
+    const int64_t row = ((int64_t)t * nh + (int64_t)kvh * G + head) * num_splits + split;
+    part_o[row * HD + d] = acc;
+    if (d == 0) { part_ml[row * 2] = M; part_ml[row * 2 + 1] = L; }
   }
 }
 
-// out[t, h, :] = sum_s o_s e^{m_s - M} / sum_s l_s e^{m_s - M} over the chunks s that hold visible keys
-template <typename T>
-__global__ void attn_decode_combine_kernel(T* __restrict__ out, const float* __restrict__ part_o,
-                                           const float* __restrict__ part_ml, const int32_t* __restrict__ positions,
-                                           int nh, int hd, int num_splits, int chunk, int window) {
-  const int t = blockIdx.x / nh;
+// out[t, h, :] = sum_s o_s 2^{m_s - M} / sum_s l_s 2^{m_s - M} over the chunks s that hold visible keys
+// (the running maxima are in units of log2).
+// One 64-thread workgroup per (token, head): the lanes fetch the chunks' (m, l) side by side, then
+// every lane sums its output dimensions over the chunks in ascending order.
+#define COMBINE_MAX_SPLITS 1024
+__global__ void __launch_bounds__(TS_WAVE)
+attn_decode_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ part_o,
+                           const float* __restrict__ part_ml, const int32_t* __restrict__ positions, int nh, int hd,
+                           int num_splits, int chunk, int window) {
+  __shared__ float wgt[COMBINE_MAX_SPLITS];
+  const int t = blockIdx.x / nh, lane = threadIdx.x;
   const int64_t th = blockIdx.x;
   const int pos = positions[t];
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int s0 = lo / chunk, s1 = pos / chunk;
   const float* ml = part_ml + th * num_splits * 2;
   float M = -INFINITY;
-  for (int s = s0; s <= s1; ++s) M = fmaxf(M, ml[2 * s]);
+  for (int s = s0 + lane; s <= s1; s += TS_WAVE) M = fmaxf(M, ml[2 * s]);
+  M = wave_max(M);
   float L = 0.f;
-  for (int s = s0; s <= s1; ++s) L += ml[2 * s + 1] * expf(ml[2 * s] - M);
-  const float inv = 1.0f / L;
-  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-    float acc = 0.f;
-    for (int s = s0; s <= s1; ++s) acc += part_o[(th * num_splits + s) * hd + d] * expf(ml[2 * s] - M);
-    Num<T>::st(out + th * hd + d, acc * inv);
+  for (int s = s0 + lane; s <= s1; s += TS_WAVE) {
+    const float w = fast_exp2(ml[2 * s] - M);
+    wgt[s - s0] = w;
+    L += ml[2 * s + 1] * w;
   }
-}
-
-static size_t dec_smem_bytes(int G, int hd, int chunk) {
-  const int tpr = hd / 4, nslices = DEC_THREADS / tpr;
-  return (size_t)chunk * 8 + sizeof(float) * ((size_t)G * hd + (size_t)G * chunk + 2 * G + (size_t)nslices * G * hd);
-}
-
-template <typename T, int G>
-static int launch_split(float* part_o, float* part_ml, const void* q, const void* kc, const void* vc,
-                        const int32_t* tables, const int32_t* seq_of, const int32_t* positions, int num_tokens, int nh,
-                        int nkv, int hd, int page_size, int64_t page_stride, int64_t slot_stride, int64_t head_stride,
-                        int max_blocks, int num_splits, int chunk, int tpk, float scale, int window,
-                        hipStream_t stream) {
-  const size_t smem = dec_smem_bytes(G, hd, chunk);
-  if (smem > 64 * 1024) return TS_BAD_SHAPE;
-  dim3 grid(num_splits, nkv, num_tokens);
-  attn_decode_split_kernel<T, G><<<grid, DEC_THREADS, smem, stream>>>(
-      part_o, part_ml, (const T*)q, (const T*)kc, (const T*)vc, tables, seq_of, positions, nh, hd, page_size,
-      page_stride, slot_stride, head_stride, max_blocks, num_splits, chunk, tpk, scale, window);
-  return ts_check_launch();
+  L = wave_sum(L);
+  wave_sync();
+  const float inv = 1.0f / L;
+  const float* po = part_o + (th * num_splits + s0) * hd;
+  for (int d = lane; d < hd; d += TS_WAVE) {
+    float acc = 0.f;
+#pragma unroll 4
+    for (int s = 0; s <= s1 - s0; ++s) acc = fmaf(po[(int64_t)s * hd + d], wgt[s], acc);
+    out[th * hd + d] = f2bf(acc * inv);
+  }
 }
 
 // part_o [tokens, nh, num_splits, hd] and part_ml [tokens, nh, num_splits, 2] are float workspaces.
-// num_splits * chunk must cover every position that `positions` holds.
+// num_splits * chunk must cover every position that `positions` holds. Keys: rows dense in
+// head_dim, strides kp/ks/kh (page, slot, head). Values: transposed pages, slot stride 1, strides
+// vp/vh/vd (page, head, dimension).
 extern "C" int ts_paged_attention_decode(void* out, float* part_o, float* part_ml, const void* q, const void* k_cache,
                                          const void* v_cache, const int32_t* block_tables,
                                          const int32_t* seq_of_token, const int32_t* positions, int num_tokens, int nh,
-                                         int nkv, int hd, int page_size, int64_t page_stride, int64_t slot_stride,
-                                         int64_t head_stride, int max_blocks, int num_splits, int chunk, float scale,
-                                         int window, int dtype, hipStream_t stream) {
+                                         int nkv, int hd, int page_size, int64_t kp, int64_t ks, int64_t kh,
+                                         int64_t vp, int64_t vh, int64_t vd, int max_blocks, int num_splits, int chunk,
+                                         float scale, int window, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
-  if (hd % 16 || hd > 256 || hd <= 0 || nkv <= 0 || nh % nkv || page_size <= 0 || max_blocks <= 0 || num_splits <= 0)
+  if (nkv <= 0 || nh % nkv || page_size <= 0 || page_size % 8 || max_blocks <= 0 || num_splits <= 0)
     return TS_BAD_SHAPE;
-  if (chunk != 64 && chunk != 128 && chunk != 256) return TS_BAD_SHAPE;
+  if (chunk < 128 || chunk % 128 || num_splits > COMBINE_MAX_SPLITS) return TS_BAD_SHAPE;
   if (num_tokens > 65535 || nkv > 65535) return TS_BAD_SHAPE;
   const int G = nh / nkv;
-  if (G > 8) return TS_BAD_SHAPE;
-  const int64_t elem = dtype == 0 ? 4 : 2;
-  if ((page_stride * elem) % 16 || (slot_stride * elem) % 16 || (head_stride * elem) % 16) return TS_BAD_SHAPE;
-  // threads per key: as many as divide the row into whole 16-byte loads
-  const int per_load = dtype == 0 ? 4 : 8;
-  int tpk = DEC_THREADS / chunk;
-  while (tpk > 1 && (hd % tpk || (hd / tpk) % per_load)) tpk >>= 1;
-  int rc;
-#define TS_DEC_CASE(GG)                                                                                              \
-  case GG:                                                                                                           \
-    rc = dtype == 0 ? launch_split<float, GG>(part_o, part_ml, q, k_cache, v_cache, block_tables, seq_of_token,      \
-                                              positions, num_tokens, nh, nkv, hd, page_size, page_stride,            \
-                                              slot_stride, head_stride, max_blocks, num_splits, chunk, tpk, scale,   \
-                                              window, stream)                                                        \
-                    : launch_split<bf16_t, GG>(part_o, part_ml, q, k_cache, v_cache, block_tables, seq_of_token,     \
-                                               positions, num_tokens, nh, nkv, hd, page_size, page_stride,           \
-                                               slot_stride, head_stride, max_blocks, num_splits, chunk, tpk, scale,  \
-                                               window, stream);                                                      \
-    break;
-  if (dtype != 0 && dtype != 1) return TS_BAD_DTYPE;
-  switch (G) {
-    TS_DEC_CASE(1) TS_DEC_CASE(2) TS_DEC_CASE(3) TS_DEC_CASE(4) TS_DEC_CASE(5) TS_DEC_CASE(6) TS_DEC_CASE(7)
-    TS_DEC_CASE(8)
+  if (G > 16 || G * hd > 2048) return TS_BAD_SHAPE;
+  // 16-byte loads: key rows and the 8-key pieces of value rows must be 16-byte aligned
+  if ((kp % 8) || (ks % 8) || (kh % 8) || (vp % 8) || (vh % 8) || (vd % 8)) return TS_BAD_SHAPE;
+  if ((((uintptr_t)q) | ((uintptr_t)k_cache) | ((uintptr_t)v_cache)) & 15) return TS_BAD_SHAPE;
+  const size_t smem = sizeof(float) * (2 * DEC_WAVES * 16 + (size_t)DEC_WAVES * G * hd);
+  int page_shift = -1;
+  if ((page_size & (page_size - 1)) == 0) {
+    page_shift = 0;
+    while ((1 << page_shift) < page_size) ++page_shift;
+  }
+  dim3 grid(num_splits, nkv, num_tokens);
+#define TS_DEC(HH)                                                                                              \
+  attn_decode_mfma_kernel<HH><<<grid, DEC_THREADS, smem, stream>>>(                                             \
+      part_o, part_ml, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,          \
+      seq_of_token, positions, nh, G, page_size, page_shift, kp, ks, kh, vp, vh, vd, max_blocks, num_splits,    \
+      chunk, scale * 1.44269504088896340736f, window)
+  switch (hd) {
+    case 32: TS_DEC(32); break;
+    case 64: TS_DEC(64); break;
+    case 96: TS_DEC(96); break;
+    case 128: TS_DEC(128); break;
     default: return TS_BAD_SHAPE;
   }
-#undef TS_DEC_CASE
+#undef TS_DEC
+  int rc = ts_check_launch();
   if (rc) return rc;
-  const int threads = hd < 64 ? 64 : (hd > 256 ? 256 : hd);
-  if (dtype == 0)
-    attn_decode_combine_kernel<float><<<num_tokens * nh, threads, 0, stream>>>((float*)out, part_o, part_ml, positions,
-                                                                              nh, hd, num_splits, chunk, window);
-  else
-    attn_decode_combine_kernel<bf16_t><<<num_tokens * nh, threads, 0, stream>>>((bf16_t*)out, part_o, part_ml,
-                                                                               positions, nh, hd, num_splits, chunk,
-                                                                               window);
+  attn_decode_combine_kernel<<<num_tokens * nh, TS_WAVE, 0, stream>>>((bf16_t*)out, part_o, part_ml, positions, nh, hd,
+                                                                      num_splits, chunk, window);
   return ts_check_launch();
 }

@@ -2,7 +2,8 @@
 // storage type, head size (a multiple of 16 up to 256), head grouping and page size, for prompt
 // portions and decoded tokens alike: a token at position p sees the keys of its request at
 // positions max(0, p - window + 1) .. p, all of them read from the cache pages (the step's own keys
-// are written before this runs). Keys are visited in chunks of 64 counted from position 0, so the
+// are written before this runs). Key rows are dense in head_dim; value elements are addressed
+// with four strides (page, slot, head, dimension), so any page layout of the values works. Keys are visited in chunks of 64 counted from position 0, so the
 // order of every sum depends only on the token's position, never on the batch or on the portion.
 // Scores, softmax and the weighted sum are 32-bit.
 #include "common.h"
@@ -37,10 +38,11 @@ paged_attention_wave_kernel(T* __restrict__ out, const T* __restrict__ q, const 
                             const T* __restrict__ v_cache, const int32_t* __restrict__ block_tables,
                             const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ positions,
                             int num_tokens, int nh, int nkv, int hd, int page_size, int64_t page_stride,
-                            int64_t slot_stride, int64_t head_stride, int max_blocks, float scale, int window) {
+                            int64_t slot_stride, int64_t head_stride, int64_t vp, int64_t vs, int64_t vh, int64_t vd,
+                            int max_blocks, float scale, int window) {
   __shared__ float q_s[ATT_WAVES][ATT_MAX_HD];
   __shared__ float p_s[ATT_WAVES][TS_WAVE];
-  __shared__ int64_t row_s[ATT_WAVES][TS_WAVE];
+  __shared__ int64_t row_s[ATT_WAVES][TS_WAVE];   // element offset of each key's value row
   const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
   const int64_t item = (int64_t)blockIdx.x * ATT_WAVES + wave;
   if (item >= (int64_t)num_tokens * nh) return;  // whole wave leaves together; no block barrier below
@@ -63,8 +65,9 @@ paged_attention_wave_kernel(T* __restrict__ out, const T* __restrict__ q, const 
     int64_t rowoff = 0;
     if (valid) {
       const int page = table[key / page_size];
-      rowoff = (int64_t)page * page_stride + (int64_t)(key % page_size) * slot_stride + (int64_t)kvh * head_stride;
-      const T* kr = k_cache + rowoff;
+      const int slot = key % page_size;
+      rowoff = (int64_t)page * vp + (int64_t)slot * vs + (int64_t)kvh * vh;
+      const T* kr = k_cache + (int64_t)page * page_stride + (int64_t)slot * slot_stride + (int64_t)kvh * head_stride;
       float dot = 0.f;
       for (int d = 0; d < hd; d += Vec<T>::N) {
         float kv[Vec<T>::N];
@@ -89,7 +92,7 @@ paged_attention_wave_kernel(T* __restrict__ out, const T* __restrict__ q, const 
       const int d = lane + i * TS_WAVE;
       if (d < hd) {
         float a = acc[i] * alpha;
-        for (int j = first; j <= last; ++j) a = fmaf(p_s[wave][j], Num<T>::ld(v_cache + row_s[wave][j] + d), a);
+        for (int j = first; j <= last; ++j) a = fmaf(p_s[wave][j], Num<T>::ld(v_cache + row_s[wave][j] + (int64_t)d * vd), a);
         acc[i] = a;
       }
     }
@@ -108,7 +111,8 @@ extern "C" int ts_paged_attention_wave(void* out, const void* q, const void* k_c
                                        const int32_t* block_tables, const int32_t* seq_of_token,
                                        const int32_t* positions, int num_tokens, int nh, int nkv, int hd,
                                        int page_size, int64_t page_stride, int64_t slot_stride, int64_t head_stride,
-                                       int max_blocks, float scale, int window, int dtype, hipStream_t stream) {
+                                       int64_t vp, int64_t vs, int64_t vh, int64_t vd, int max_blocks, float scale,
+                                       int window, int dtype, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
   if (hd % 16 || hd > ATT_MAX_HD || hd <= 0 || nkv <= 0 || nh % nkv || page_size <= 0 || max_blocks <= 0)
     return TS_BAD_SHAPE;
@@ -122,11 +126,13 @@ extern "C" int ts_paged_attention_wave(void* out, const void* q, const void* k_c
   if (dtype == 0)
     paged_attention_wave_kernel<float><<<grid, block, 0, stream>>>(
         (float*)out, (const float*)q, (const float*)k_cache, (const float*)v_cache, block_tables, seq_of_token,
-        positions, num_tokens, nh, nkv, hd, page_size, page_stride, slot_stride, head_stride, max_blocks, scale, window);
+        positions, num_tokens, nh, nkv, hd, page_size, page_stride, slot_stride, head_stride, vp, vs, vh, vd, max_blocks,
+        scale, window);
   else if (dtype == 1)
     paged_attention_wave_kernel<bf16_t><<<grid, block, 0, stream>>>(
         (bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, seq_of_token,
-        positions, num_tokens, nh, nkv, hd, page_size, page_stride, slot_stride, head_stride, max_blocks, scale, window);
+        positions, num_tokens, nh, nkv, hd, page_size, page_stride, slot_stride, head_stride, vp, vs, vh, vd, max_blocks,
+        scale, window);
   else
     return TS_BAD_DTYPE;
   return ts_check_launch();

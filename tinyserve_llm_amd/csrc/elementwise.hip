@@ -96,73 +96,93 @@ extern "C" int ts_rmsnorm(void* out, void* res_out, const void* x, const void* r
 // fused with the scatter of rotated k and of v into their cache slots.
 //   qkv   [T, (nh + 2*nkv) * hd]   one token's q heads, then k heads, then v heads
 //   q_out [T, nh * hd]
-//   cache element address: page * page_stride + offset * slot_stride + head * head_stride + d,
+//   key element address:   page * kp + offset * ks + head * kh + d          (d dense)
+//   value element address: page * vp + offset * vs + head * vh + d * vd     (any layout: the engine
+//                          keeps values transposed inside a page, vs = 1 and vd = page_size)
 //   page = slot / page_size, offset = slot % page_size; slot -1 writes nothing.
 // k_cache == null: this layer does not own a cache; only q is rotated.
+// A workgroup takes ROPE_TOK consecutive tokens and one of gridDim.y slices of their elements
+// (few tokens are spread over more workgroups); value elements are assigned token-fastest so that
+// neighbouring threads write neighbouring slots of a transposed page.
 // ------------------------------------------------------------------------------------------
+#define ROPE_TOK 16
+
 template <typename T>
 __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
                                   const T* __restrict__ qkv, const float* __restrict__ cos_sin,
                                   const int32_t* __restrict__ positions, const int64_t* __restrict__ slots,
-                                  int nh, int nkv, int hd, int rotate, int page_size, int64_t page_stride,
-                                  int64_t slot_stride, int64_t head_stride) {
-  const int t = blockIdx.x;
+                                  int num_tokens, int nh, int nkv, int hd, int rotate, int page_size, int64_t kp,
+                                  int64_t ks, int64_t kh, int64_t vp, int64_t vs, int64_t vh, int64_t vd) {
+  const int t0 = blockIdx.x * ROPE_TOK;
+  const int nt = num_tokens - t0 < ROPE_TOK ? num_tokens - t0 : ROPE_TOK;
   const int half = hd / 2;
   const int row = (nh + 2 * nkv) * hd;
-  const T* src = qkv + (int64_t)t * row;
-  const float* cs = cos_sin + (int64_t)positions[t] * hd;
-  // q heads
-  T* qo = q_out + (int64_t)t * nh * hd;
-  for (int i = threadIdx.x; i < nh * half; i += blockDim.x) {
-    const int h = i / half, j = i - h * half;
-    const float x1 = Num<T>::ld(src + h * hd + j), x2 = Num<T>::ld(src + h * hd + j + half);
+  const int qpairs = nh * half, kpairs = nkv * half;
+  // q and k pairs of every token of the group: this workgroup's slice of them
+  const int npairs = nt * (qpairs + kpairs);
+  const int pbeg = (int)((int64_t)npairs * blockIdx.y / gridDim.y), pend = (int)((int64_t)npairs * (blockIdx.y + 1) / gridDim.y);
+  for (int i = pbeg + threadIdx.x; i < pend; i += blockDim.x) {
+    const int tl = i / (qpairs + kpairs), e = i - tl * (qpairs + kpairs);
+    const int t = t0 + tl;
+    const bool is_k = e >= qpairs;
+    const int pe = is_k ? e - qpairs : e;
+    const int h = pe / half, j = pe - h * half;
+    const T* src = qkv + (int64_t)t * row + (is_k ? nh * hd : 0) + h * hd;
+    if (is_k && (!k_cache || slots[t] < 0)) continue;
+    const float x1 = Num<T>::ld(src + j), x2 = Num<T>::ld(src + j + half);
     float y1 = x1, y2 = x2;
     if (rotate) {
-      const float c = cs[j], s = cs[half + j];
-      y1 = x1 * c - x2 * s;
-      y2 = x2 * c + x1 * s;
+      const float* cs = cos_sin + (int64_t)positions[t] * hd;
+      const float c = cs[j], sn = cs[half + j];
+      y1 = x1 * c - x2 * sn;
+      y2 = x2 * c + x1 * sn;
     }
-    Num<T>::st(qo + h * hd + j, y1);
-    Num<T>::st(qo + h * hd + j + half, y2);
+    T* dst;
+    if (is_k) {
+      const int64_t slot = slots[t];
+      dst = k_cache + (slot / page_size) * kp + (slot % page_size) * ks + (int64_t)h * kh;
+    } else {
+      dst = q_out + ((int64_t)t * nh + h) * hd;
+    }
+    Num<T>::st(dst + j, y1);
+    Num<T>::st(dst + j + half, y2);
   }
   if (!k_cache) return;
-  const int64_t slot = slots[t];
-  if (slot < 0) return;
-  const int64_t base = (slot / page_size) * page_stride + (slot % page_size) * slot_stride;
-  const T* ks = src + nh * hd;
-  const T* vs = ks + nkv * hd;
-  for (int i = threadIdx.x; i < nkv * half; i += blockDim.x) {
-    const int h = i / half, j = i - h * half;
-    const float x1 = Num<T>::ld(ks + h * hd + j), x2 = Num<T>::ld(ks + h * hd + j + half);
-    float y1 = x1, y2 = x2;
-    if (rotate) {
-      const float c = cs[j], s = cs[half + j];
-      y1 = x1 * c - x2 * s;
-      y2 = x2 * c + x1 * s;
-    }
-    Num<T>::st(k_cache + base + h * head_stride + j, y1);
-    Num<T>::st(k_cache + base + h * head_stride + j + half, y2);
-  }
-  for (int i = threadIdx.x; i < nkv * hd; i += blockDim.x) {
-    const int h = i / hd;
-    v_cache[base + h * head_stride + (i - h * hd)] = vs[i];
+  // values: thread -> (element, token), token fastest
+  const int vel = nkv * hd;
+  const int vbeg = (int)((int64_t)vel * blockIdx.y / gridDim.y) * ROPE_TOK;
+  const int vend = (int)((int64_t)vel * (blockIdx.y + 1) / gridDim.y) * ROPE_TOK;
+  for (int i = vbeg + threadIdx.x; i < vend; i += blockDim.x) {
+    const int tl = i % ROPE_TOK, e = i / ROPE_TOK;
+    if (tl >= nt) continue;
+    const int t = t0 + tl;
+    const int64_t slot = slots[t];
+    if (slot < 0) continue;
+    const int h = e / hd, d = e - h * hd;
+    v_cache[(slot / page_size) * vp + (slot % page_size) * vs + (int64_t)h * vh + (int64_t)d * vd] =
+        qkv[(int64_t)t * row + (nh + nkv) * hd + e];
   }
 }
 
 extern "C" int ts_rope_store(void* q_out, void* k_cache, void* v_cache, const void* qkv, const float* cos_sin,
                              const int32_t* positions, const int64_t* slots, int num_tokens, int nh, int nkv,
-                             int hd, int rotate, int page_size, int64_t page_stride, int64_t slot_stride,
-                             int64_t head_stride, int dtype, hipStream_t stream) {
+                             int hd, int rotate, int page_size, int64_t kp, int64_t ks, int64_t kh, int64_t vp,
+                             int64_t vs, int64_t vh, int64_t vd, int dtype, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
   if (hd % 2 || nh <= 0 || nkv < 0 || page_size <= 0) return TS_BAD_SHAPE;
+  const int groups = (num_tokens + ROPE_TOK - 1) / ROPE_TOK;
+  int slices = 512 / groups;
+  if (slices < 1) slices = 1;
+  if (slices > 32) slices = 32;
+  const dim3 blocks(groups, slices);
   if (dtype == 0)
-    rope_store_kernel<float><<<num_tokens, 256, 0, stream>>>((float*)q_out, (float*)k_cache, (float*)v_cache,
-                                                             (const float*)qkv, cos_sin, positions, slots, nh, nkv,
-                                                             hd, rotate, page_size, page_stride, slot_stride, head_stride);
+    rope_store_kernel<float><<<blocks, 256, 0, stream>>>((float*)q_out, (float*)k_cache, (float*)v_cache,
+                                                         (const float*)qkv, cos_sin, positions, slots, num_tokens, nh,
+                                                         nkv, hd, rotate, page_size, kp, ks, kh, vp, vs, vh, vd);
   else if (dtype == 1)
-    rope_store_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache,
-                                                              (const bf16_t*)qkv, cos_sin, positions, slots, nh, nkv,
-                                                              hd, rotate, page_size, page_stride, slot_stride, head_stride);
+    rope_store_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache,
+                                                          (const bf16_t*)qkv, cos_sin, positions, slots, num_tokens,
+                                                          nh, nkv, hd, rotate, page_size, kp, ks, kh, vp, vs, vh, vd);
   else
     return TS_BAD_DTYPE;
   return ts_check_launch();
@@ -199,32 +219,31 @@ extern "C" int ts_silu_mul(void* out, const void* gu, int num_tokens, int inter,
 }
 
 // ------------------------------------------------------------------------------------------
-// Copy the first `num_slots` slots of page `src` to page `dst` in a pool laid out
-// [pages, runs, page_size, row]: `runs` = layers x kv heads of the group, row = one head's
-// head_dim elements in bytes.
+// Copy the leading part of every run of page `src` to page `dst`. A page of a pool is `runs` runs of
+// `run_units` 2-byte units; the first `copy_units` of each run are copied. For keys
+// [pages, layers, heads, page_size, head_dim] a run is one head's slots and the leading part is the
+// first n slots; for transposed values [pages, layers, heads, head_dim, page_size] a run is one
+// dimension's slots.
 // ------------------------------------------------------------------------------------------
-__global__ void copy_slots_kernel(uint8_t* __restrict__ pool, int64_t page_bytes, int64_t layer_bytes,
-                                  int64_t copy_bytes, int src, int dst) {
-  const int layer = blockIdx.y;
-  const uint8_t* s = pool + src * page_bytes + layer * layer_bytes;
-  uint8_t* d = pool + dst * page_bytes + layer * layer_bytes;
-  // rows are multiples of 4 bytes (an even head_dim of 2-byte elements at least)
-  const int64_t words = copy_bytes / 4;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < words; i += (int64_t)gridDim.x * blockDim.x)
-    ((uint32_t*)d)[i] = ((const uint32_t*)s)[i];
+__global__ void copy_slots_kernel(uint16_t* __restrict__ pool, int64_t page_units, int64_t run_units,
+                                  int64_t copy_units, int64_t total, int src, int dst) {
+  const uint16_t* s = pool + src * page_units;
+  uint16_t* d = pool + dst * page_units;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t run = i / copy_units, o = i - run * copy_units;
+    d[run * run_units + o] = s[run * run_units + o];
+  }
 }
 
-extern "C" int ts_copy_slots(void* pool, int num_layers, int page_size, int64_t row_bytes, int src, int dst,
-                             int num_slots, hipStream_t stream) {
-  if (num_slots <= 0 || num_layers <= 0) return TS_OK;
-  if (num_slots > page_size || row_bytes % 4 || src == dst) return TS_BAD_SHAPE;
-  const int64_t layer_bytes = (int64_t)page_size * row_bytes;
-  const int64_t page_bytes = layer_bytes * num_layers;
-  const int64_t copy_bytes = (int64_t)num_slots * row_bytes;
-  int64_t bx = (copy_bytes / 4 + 255) / 256;
-  if (bx > 64) bx = 64;
-  if (bx < 1) bx = 1;
-  copy_slots_kernel<<<dim3((int)bx, num_layers), 256, 0, stream>>>((uint8_t*)pool, page_bytes, layer_bytes,
-                                                                    copy_bytes, src, dst);
+extern "C" int ts_copy_slots(void* pool, int64_t runs, int64_t run_bytes, int64_t copy_bytes, int src, int dst,
+                             hipStream_t stream) {
+  if (copy_bytes <= 0 || runs <= 0) return TS_OK;
+  if (copy_bytes > run_bytes || run_bytes % 2 || copy_bytes % 2 || src == dst || src < 0 || dst < 0)
+    return TS_BAD_SHAPE;
+  const int64_t total = runs * (copy_bytes / 2);
+  int64_t blocks = (total + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  copy_slots_kernel<<<(int)blocks, 256, 0, stream>>>((uint16_t*)pool, runs * (run_bytes / 2), run_bytes / 2,
+                                                     copy_bytes / 2, total, src, dst);
   return ts_check_launch();
 }

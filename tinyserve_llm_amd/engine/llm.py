@@ -68,6 +68,7 @@ class LLM:
             load_tokenizer: bool | None = None,      # None: only if the folder holds a tokenizer
             random_weights: tuple[object, int] | None = None,   # (typed configuration, seed) instead of a folder
             model: DecoderModel | None = None,       # an already bound model (shares its weights)
+            decode_graphs: bool = True,              # replay decode steps from HIP graphs
     ) -> None:
         self.device = require_gpu(cache_config.device if cache_config.device != "cuda" else "cuda:0")
         self.dtype = as_dtype(dtype)
@@ -103,6 +104,8 @@ class LLM:
         self.manager = KVCacheManager(self.storage, caching=cache_config.caching)
         self.scheduler = Scheduler(scheduler_config, self.manager)
         self.runner = ModelRunner(self.model, self.storage, self.manager)
+        if decode_graphs:
+            self.runner.enable_decode_graphs(scheduler_config.max_model_len, scheduler_config.max_num_seqs)
         self.steps: list[StepRecord] = []
         logger.info("KV cache: %d blocks of %d tokens", num_blocks, cache_config.block_size)
 

@@ -54,11 +54,13 @@ class ModelRunner:
                 mem.k_cache, mem.v_cache, mem.space = storage.layer_cache(owner)
             self.memory.append(mem)
         self.windows = [s.window for s in storage.spaces]
+        self.graphs: DecodeGraphs | None = None
 
     # ---- packing ----------------------------------------------------------------------------
-    def prepare(self, entries: Sequence[StepEntry]) -> tuple[StepContext, torch.Tensor, int]:
-        """Packs a step into device tensors; returns (context, wanted rows, number of wanted rows).
-        Everything a kernel will index with is checked here first."""
+    def _pack(self, entries: Sequence[StepEntry], table_widths: list[int] | None = None, pad_to: int = 0):
+        """Checks a step on the host and lays it out as flat integer lists. With `table_widths`
+        every block table is padded to that width; with `pad_to` the batch is filled up with idle
+        one-token rows (position 0, no cache write, page 0) to that many requests."""
         if not entries:
             raise StepError("a step needs at least one entry")
         ps = self.storage.page_size
@@ -109,17 +111,35 @@ class ModelRunner:
                 tables[sp].append(table)
                 slot_maps[sp].extend(table[p // ps] * ps + p % ps for p in range(e.start, end))
             cu.append(cu[-1] + n)
-        T, S, R = len(ids), len(entries), len(rows)
-        widths = [max(len(t) for t in tables[sp]) for sp in range(num_spaces)]
+        for s in range(len(entries), pad_to):           # idle rows of a fixed-size batch
+            ids.append(0)
+            positions.append(0)
+            seq_of.append(s)
+            starts.append(0)
+            ctx_lens.append(1)
+            slots.append(0)
+            rows.append(cu[-1])
+            cu.append(cu[-1] + 1)
+            for sp in range(num_spaces):
+                tables[sp].append([0])
+                slot_maps[sp].append(-1)
+        T, S, R = len(ids), len(cu) - 1, len(rows)
+        widths = table_widths or [max(len(t) for t in tables[sp]) for sp in range(num_spaces)]
         flat: list[int] = ids + positions + seq_of + cu + ctx_lens + slots + rows
         offsets = []
         for sp in range(num_spaces):
             offsets.append(len(flat))
             for t in tables[sp]:
+                if len(t) > widths[sp]:
+                    raise StepError(f"a block table of {len(t)} pages exceeds the fixed width {widths[sp]}")
                 flat.extend(0 if p == FREED else p for p in t)
                 flat.extend([0] * (widths[sp] - len(t)))
-        packed = torch.tensor(flat, dtype=torch.int32).to(self.device, non_blocking=True)
-        slot_packed = torch.tensor([x for m in slot_maps for x in m], dtype=torch.int64).to(self.device, non_blocking=True)
+        slot_flat = [x for m in slot_maps for x in m]
+        host = dict(cu=cu, starts=starts, ctx_lens=ctx_lens, slots=slots)
+        return flat, slot_flat, (T, S, R, widths, offsets), host
+
+    def _context(self, packed: torch.Tensor, slot_packed: torch.Tensor, dims, host) -> tuple[StepContext, torch.Tensor]:
+        T, S, R, widths, offsets = dims
         o = 0
 
         def cut(n: int) -> torch.Tensor:
@@ -131,20 +151,116 @@ class ModelRunner:
         ctx = StepContext(
             num_tokens=T, num_seqs=S, token_ids=cut(T), positions=cut(T), seq_of_token=cut(T), cu_seqlens=cut(S + 1),
             context_lens=cut(S), state_slots=cut(S), slot_mapping=[], block_tables=[],
-            host_cu_seqlens=cu, host_starts=starts, host_context_lens=ctx_lens, host_state_slots=slots)
+            host_cu_seqlens=host["cu"], host_starts=host["starts"], host_context_lens=host["ctx_lens"],
+            host_state_slots=host["slots"])
         row_t = cut(R)
-        for sp in range(num_spaces):
+        for sp in range(len(widths)):
             ctx.block_tables.append(packed[offsets[sp]:offsets[sp] + S * widths[sp]].view(S, widths[sp]))
             ctx.slot_mapping.append(slot_packed[sp * T:(sp + 1) * T])
-        return ctx, row_t, R
+        return ctx, row_t
+
+    def prepare(self, entries: Sequence[StepEntry]) -> tuple[StepContext, torch.Tensor, int]:
+        """Packs a step into device tensors; returns (context, wanted rows, number of wanted rows).
+        Everything a kernel will index with is checked here first."""
+        flat, slot_flat, dims, host = self._pack(entries)
+        packed = torch.tensor(flat, dtype=torch.int32).to(self.device, non_blocking=True)
+        slot_packed = torch.tensor(slot_flat, dtype=torch.int64).to(self.device, non_blocking=True)
+        ctx, rows = self._context(packed, slot_packed, dims, host)
+        return ctx, rows, dims[2]
 
     # ---- running ----------------------------------------------------------------------------
     @torch.inference_mode()
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Runs the step; returns float32 logits [wanted, vocab] on the device (an empty tensor
         if nothing is wanted; the tokens' keys and values are written all the same)."""
+        if self.graphs is not None and self.graphs.takes(entries):
+            return self.graphs.run(entries)
         ctx, rows, num_rows = self.prepare(entries)
         hidden, residual = self.model.forward(ctx, self.memory)
         if num_rows == 0:
             return torch.empty((0, self.model.spec.vocab_size), dtype=torch.float32, device=self.device)
         return self.model.logits(hidden, residual, rows)
+
+    def enable_decode_graphs(self, max_context: int, max_batch: int) -> bool:
+        """Decode steps (every entry one token whose logits are wanted) are then replayed from HIP
+        graphs, one per batch size, instead of being launched kernel by kernel. Only for models
+        whose parts all declare `graph_safe`. Returns whether graphs are on."""
+        if not self.model.graph_safe():
+            return False
+        self.graphs = DecodeGraphs(self, max_context, max_batch)
+        return True
+
+
+class DecodeGraphs:
+    """HIP graphs of the decode step. A graph is captured the first time a (batch size, context
+    bucket) pair is met: sizes above 8 round up to a multiple of 8 and idle rows fill the batch;
+    the longest context of the batch rounds up to a multiple of 256 positions and fixes the width
+    of the block tables, and with it the attention kernels' grids. A graph's inputs live in fixed
+    device buffers that every replay overwrites with one copy from pinned host memory."""
+
+    def __init__(self, runner: ModelRunner, max_context: int, max_batch: int) -> None:
+        self.runner = runner
+        self.page_size = runner.storage.page_size
+        self.num_spaces = len(runner.storage.spaces)
+        self.bucket = max(256, self.page_size)
+        self.max_context = max_context
+        self.max_batch = max_batch
+        self.can_pad = not runner.model.state_plan()
+        self.graphs: dict[int, tuple] = {}
+        self.pool = None
+
+    def _size(self, n: int) -> int:
+        return n if n <= 8 or not self.can_pad else -(-n // 8) * 8
+
+    def takes(self, entries: Sequence[StepEntry]) -> bool:
+        if len(entries) > self.max_batch:
+            return False
+        for e in entries:
+            if len(e.tokens) != 1 or list(e.want) != [0] or e.start + 1 > self.max_context:
+                return False
+        return True
+
+    def _capture(self, size: int, flat: list[int], slot_flat: list[int], dims, host):
+        r = self.runner
+        host_i32 = torch.empty(len(flat), dtype=torch.int32, pin_memory=True)
+        host_i64 = torch.empty(len(slot_flat), dtype=torch.int64, pin_memory=True)
+        dev_i32 = torch.zeros(len(flat), dtype=torch.int32, device=r.device)
+        dev_i64 = torch.zeros(len(slot_flat), dtype=torch.int64, device=r.device)
+        host_i32.copy_(torch.tensor(flat, dtype=torch.int32))
+        host_i64.copy_(torch.tensor(slot_flat, dtype=torch.int64))
+        dev_i32.copy_(host_i32, non_blocking=True)
+        dev_i64.copy_(host_i64, non_blocking=True)
+        ctx, rows = r._context(dev_i32, dev_i64, dims, host)
+        # once without capture: libraries set up their workspaces, the kernel library loads
+        side = torch.cuda.Stream(device=r.device)
+        side.wait_stream(torch.cuda.current_stream(r.device))
+        with torch.cuda.stream(side):
+            hidden, residual = r.model.forward(ctx, r.memory)
+            r.model.logits(hidden, residual, rows)
+        torch.cuda.current_stream(r.device).wait_stream(side)
+        torch.cuda.synchronize(r.device)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, pool=self.pool):
+            hidden, residual = r.model.forward(ctx, r.memory)
+            logits = r.model.logits(hidden, residual, rows)
+        if self.pool is None:
+            self.pool = graph.pool()
+        return graph, host_i32, host_i64, dev_i32, dev_i64, logits
+
+    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        size = self._size(len(entries))
+        longest = max(e.start + 1 for e in entries)
+        reach = min(-(-longest // self.bucket) * self.bucket, -(-self.max_context // self.bucket) * self.bucket)
+        width = -(-reach // self.page_size)
+        key = (size, width)
+        flat, slot_flat, dims, host = self.runner._pack(entries, [width] * self.num_spaces, pad_to=size)
+        if key not in self.graphs:
+            self.graphs[key] = self._capture(size, flat, slot_flat, dims, host)
+            # the capture recorded the step without running it: the replay below runs it
+        graph, host_i32, host_i64, dev_i32, dev_i64, logits = self.graphs[key]
+        host_i32.copy_(torch.tensor(flat, dtype=torch.int32))
+        host_i64.copy_(torch.tensor(slot_flat, dtype=torch.int64))
+        dev_i32.copy_(host_i32, non_blocking=True)
+        dev_i64.copy_(host_i64, non_blocking=True)
+        graph.replay()
+        return logits[:len(entries)]

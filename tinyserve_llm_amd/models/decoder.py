@@ -34,7 +34,6 @@ class DecoderModel:
     def __init__(self, spec: ModelSpec) -> None:
         self.spec = spec
         self.layers: list[Layer] = []
-        built: dict[int, Layer] = {}
         for ls in spec.layers:
             # one LayerSpec object listed at several indices still gives one set of weights per index
             self.layers.append(Layer(
@@ -42,7 +41,6 @@ class DecoderModel:
                 mixer_norm=base.make("norm", ls.mixer_norm), ff_norm=base.make("norm", ls.ff_norm), block=ls.block))
             if ls.block not in base.BLOCKS:
                 raise KeyError(f"no block arrangement named {ls.block!r}; registered: {sorted(base.BLOCKS)}")
-        del built
         self.final_norm = base.make("norm", spec.final_norm)
         self.position_encodings = {name: base.make("position_encoding", ps)
                                    for name, ps in spec.position_encodings.items()}
@@ -85,6 +83,12 @@ class DecoderModel:
             if st is not None:
                 plan.append(StatePlanEntry(i, st))
         return plan
+
+    def graph_safe(self) -> bool:
+        """True if every part may be recorded into a HIP graph (see Part.graph_safe)."""
+        parts = [p for layer in self.layers for p in layer.parts().values()]
+        parts += [self.final_norm, *self.position_encodings.values()]
+        return all(getattr(p, "graph_safe", False) for p in parts)
 
     # ---- parameters --------------------------------------------------------------------------
     def param_specs(self) -> dict[str, ParamSpec]:

@@ -44,13 +44,16 @@ def _declare(lib: ctypes.CDLL) -> None:
     sig = {
         "ts_embedding": [p, p, p, i, i, i, p],
         "ts_rmsnorm": [p, p, p, p, p, p, i, i, f, i, i, p],
-        "ts_rope_store": [p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i, p],
+        "ts_rope_store": [p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i64, i, p],
         "ts_silu_mul": [p, p, i, i, i, p],
-        "ts_copy_slots": [p, i, i, i64, i, i, i, p],
-        "ts_paged_attention_wave": [p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i, f, i, i, p],
-        "ts_paged_attention_decode": [p, p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i, i, i, f, i, i, p],
+        "ts_copy_slots": [p, i64, i64, i64, i, i, p],
+        "ts_paged_attention_wave": [p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i64, i, f, i, i, p],
+        "ts_paged_attention_decode": [p, p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, i, i, f, i,
+                                      p],
         "ts_gemm_exact": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_sample": [p, p, p, p, u64, i, i, i64, p],
+        "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, p],
+        "ts_gemm_skinny_bf16": [p, p, p, i, i, i, i64, i64, i64, i, p],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -145,40 +148,38 @@ def rope_store(qkv: torch.Tensor, cos_sin: torch.Tensor | None, positions: torch
     if cos_sin is not None:
         _need(cos_sin.dtype == torch.float32 and cos_sin.dim() == 2 and cos_sin.shape[1] == head_dim
               and cos_sin.is_contiguous(), "the rotation table must be float32 [positions, head_dim]")
-    page_size, page_stride, slot_stride, head_stride = 1, 0, 0, 0
+    page_size, kst, vst = 1, (0, 0, 0), (0, 0, 0, 0)
     if k_cache is not None:
         _need(v_cache is not None and slots is not None, "a cache write needs k, v and the slots")
         _need(slots.dtype == torch.int64 and slots.shape == (T,) and slots.is_contiguous(), "slots must be int64 [tokens]")
         _check_cache(k_cache, v_cache, qkv.dtype, num_kv_heads, head_dim)
-        page_size, page_stride, slot_stride = k_cache.shape[1], k_cache.stride(0), k_cache.stride(1)
-        head_stride = k_cache.stride(2)
+        page_size, kst, vst = k_cache.shape[1], k_cache.stride()[:3], v_cache.stride()
     q = torch.empty((T, num_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
     _run("rope_store", library().ts_rope_store(
         _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(qkv), _ptr(cos_sin), _ptr(positions), _ptr(slots), T, num_heads,
-        num_kv_heads, head_dim, int(cos_sin is not None), page_size, page_stride, slot_stride, head_stride,
-        _code(qkv.dtype), _stream()))
+        num_kv_heads, head_dim, int(cos_sin is not None), page_size, *kst, *vst, _code(qkv.dtype), _stream()))
     return q
 
 
 def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, dtype: torch.dtype, nkv: int, hd: int) -> None:
-    """A layer's cache is addressed as [pages, page_size, kv_heads, head_dim]; pages, slots and heads
-    may be strided in any order (the engine's pools keep a head's slots together), head_dim is dense."""
-    _need(k_cache.dim() == 4 and k_cache.shape[2] == nkv and k_cache.shape[3] == hd,
-          f"cache view must be [pages, page_size, {nkv}, {hd}], got {tuple(k_cache.shape)}")
-    _need(k_cache.dtype == dtype and v_cache.dtype == dtype, "cache and activations differ in storage type")
-    _need(k_cache.shape == v_cache.shape and k_cache.stride() == v_cache.stride(), "k and v caches must be laid out alike")
-    _need(k_cache.stride(3) == 1, "head_dim must be contiguous in the cache")
-    pages, page_size = k_cache.shape[0], k_cache.shape[1]
-    # no two (page, slot, head) rows may overlap: sort the three strides and check each spans the next
-    dims = sorted(((k_cache.stride(0), pages), (k_cache.stride(1), page_size), (k_cache.stride(2), nkv)))
-    span = hd
-    for stride, size in dims:
-        if size > 1:
-            _need(stride >= span, "cache rows overlap")
-            span = stride * size
+    """A layer's caches are addressed as [pages, page_size, kv_heads, head_dim]. Keys: head_dim
+    dense, the other three strided in any order. Values: all four strided in any order (the
+    engine's pools keep a head's slots of one dimension together, i.e. pages transposed)."""
+    for name, c in (("key", k_cache), ("value", v_cache)):
+        _need(c.dim() == 4 and c.shape[2] == nkv and c.shape[3] == hd,
+              f"{name} cache view must be [pages, page_size, {nkv}, {hd}], got {tuple(c.shape)}")
+        _need(c.dtype == dtype, "cache and activations differ in storage type")
+        # no two elements may overlap: sort the strides and check each spans the dimensions below it
+        span = 1
+        for stride, size in sorted(zip(c.stride(), c.shape)):
+            if size > 1:
+                _need(stride >= span, f"{name} cache elements overlap")
+                span = stride * size
+    _need(k_cache.shape == v_cache.shape, "key and value caches differ in shape")
+    _need(k_cache.stride(3) == 1, "head_dim must be contiguous in the key cache")
     itemsize = k_cache.element_size()
-    _need(all((k_cache.stride(i) * itemsize) % 16 == 0 for i in range(3)) and k_cache.data_ptr() % 16 == 0
-          and v_cache.data_ptr() % 16 == 0, "cache rows must be 16-byte aligned")
+    _need(all((k_cache.stride(i) * itemsize) % 16 == 0 for i in range(3)) and k_cache.data_ptr() % 16 == 0,
+          "key rows must be 16-byte aligned")
 
 
 def paged_attention_wave(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -200,47 +201,64 @@ def paged_attention_wave(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.
     out = torch.empty_like(q)
     _run("paged_attention_wave", library().ts_paged_attention_wave(
         _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_of_token), _ptr(positions),
-        T, nh, nkv, hd, k_cache.shape[1], k_cache.stride(0), k_cache.stride(1), k_cache.stride(2),
+        T, nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3], *v_cache.stride(),
         block_tables.shape[1], float(scale), int(window), _code(q.dtype), _stream()))
     return out
 
 
+MAX_DECODE_SPLITS = 1024     # chunks per token that the combining kernel takes
+DECODE_HEAD_DIMS = (32, 64, 96, 128)
+
+
 def decode_chunk(num_tokens: int, nkv: int, capacity: int) -> int:
-    """Keys per workgroup of the split-key kernel: the largest of 256/128/64 that still gives the
-    GPU's 256 compute units a few workgroups each."""
-    for chunk in (256, 128):
-        if num_tokens * nkv * -(-capacity // chunk) >= 1024:
-            return chunk
-    return 64
+    """Keys per workgroup of the split-key kernel: 128, unless so many workgroups come of it that
+    fewer, larger ones save workspace traffic, or more chunks than the combining kernel takes."""
+    chunk = 256 if num_tokens * nkv * -(-capacity // 128) >= 16384 else 128
+    while -(-capacity // chunk) > MAX_DECODE_SPLITS:
+        chunk *= 2
+    return chunk
+
+
+def decode_kernel_takes(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor) -> bool:
+    """Whether the matrix-core decode kernel serves these operands (else the wave kernel does)."""
+    nh, hd = q.shape[1], q.shape[2]
+    nkv, page = k_cache.shape[2], k_cache.shape[1]
+    return (q.dtype == torch.bfloat16 and hd in DECODE_HEAD_DIMS and nh // nkv <= 16 and (nh // nkv) * hd <= 2048
+            and page % 8 == 0 and v_cache.stride(1) == 1 and q.shape[0] <= 65535
+            and all(st % 8 == 0 for st in (*k_cache.stride()[:3], v_cache.stride(0), v_cache.stride(2), v_cache.stride(3)))
+            and v_cache.data_ptr() % 16 == 0)
 
 
 def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                            seq_of_token: torch.Tensor, positions: torch.Tensor, scale: float, window: int = 0,
                            chunk: int | None = None) -> torch.Tensor:
-    """Split-key attention for tokens that each bring one query. Every position in `positions`
-    must lie inside the pages its row of `block_tables` has (checked by the caller on the host)."""
+    """Split-key attention on the matrix cores for tokens that each bring one query (bfloat16,
+    values in transposed pages). Every position in `positions` must lie inside the pages its row
+    of `block_tables` has (checked by the caller on the host)."""
     _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions)
     _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
     T, nh, hd = q.shape
     nkv = k_cache.shape[2]
     _check_cache(k_cache, v_cache, q.dtype, nkv, hd)
-    _need(hd % 16 == 0 and hd <= 256, f"head_dim {hd} is not a multiple of 16 up to 256")
-    _need(nh % nkv == 0 and nh // nkv <= 8, f"{nh} heads over {nkv} key/value heads: groups of up to 8 are served")
+    _need(nh % nkv == 0, f"{nh} heads do not divide into {nkv} key/value heads")
+    _need(decode_kernel_takes(q, k_cache, v_cache),
+          "the decode kernel takes bfloat16, head_dim 32/64/96/128, groups of up to 16 heads, values in transposed pages")
     _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
           "block_tables must be contiguous int32 [requests, pages]")
     for name, t in (("seq_of_token", seq_of_token), ("positions", positions)):
         _need(t.dtype == torch.int32 and t.shape == (T,) and t.is_contiguous(), f"{name} must be int32 [tokens]")
-    _need(T <= 65535, "at most 65535 tokens per launch")
     capacity = block_tables.shape[1] * k_cache.shape[1]
     chunk = chunk or decode_chunk(T, nkv, capacity)
     splits = -(-capacity // chunk)
+    _need(chunk % 128 == 0 and splits <= MAX_DECODE_SPLITS, f"chunk {chunk} over {capacity} positions")
     part_o = torch.empty((T, nh, splits, hd), dtype=torch.float32, device=q.device)
     part_ml = torch.empty((T, nh, splits, 2), dtype=torch.float32, device=q.device)
     out = torch.empty_like(q)
     _run("paged_attention_decode", library().ts_paged_attention_decode(
         _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
-        _ptr(seq_of_token), _ptr(positions), T, nh, nkv, hd, k_cache.shape[1], k_cache.stride(0), k_cache.stride(1),
-        k_cache.stride(2), block_tables.shape[1], splits, chunk, float(scale), int(window), _code(q.dtype), _stream()))
+        _ptr(seq_of_token), _ptr(positions), T, nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3],
+        v_cache.stride(0), v_cache.stride(2), v_cache.stride(3), block_tables.shape[1], splits, chunk, float(scale),
+        int(window), _stream()))
     return out
 
 
@@ -270,16 +288,24 @@ def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def copy_slots(pool: torch.Tensor, src: int, dst: int, num_slots: int) -> None:
-    """pool[dst, ..., :num_slots, :] = pool[src, ..., :num_slots, :] for a contiguous pool
-    [pages, layers, kv_heads, page_size, head_dim]."""
+def copy_slots(pool: torch.Tensor, src: int, dst: int, num_slots: int, slot_dim: int) -> None:
+    """Copies the first `num_slots` slots of page `src` to page `dst` in a contiguous pool whose
+    first dimension is the page and whose dimension `slot_dim` is the slot, e.g. keys
+    [pages, heads, page_size, head_dim] (slot_dim 2) or transposed values
+    [pages, heads, head_dim, page_size] (slot_dim 3)."""
     _gpu(pool)
-    _need(pool.dim() == 5 and pool.is_contiguous(), "pool must be contiguous [pages, layers, heads, page_size, dim]")
-    pages, layers, heads, page_size = pool.shape[:4]
+    _need(pool.is_contiguous() and 1 <= slot_dim < pool.dim(), "pool must be contiguous, pages first")
+    _need(pool.element_size() % 2 == 0, "pool elements must be 2 or 4 bytes")
+    pages, page_size = pool.shape[0], pool.shape[slot_dim]
     _need(0 <= src < pages and 0 <= dst < pages and src != dst, f"pages {src}->{dst} outside 0..{pages - 1}")
     _need(0 <= num_slots <= page_size, f"{num_slots} slots do not fit a page of {page_size}")
-    row_bytes = pool.shape[4] * pool.element_size()
-    _run("copy_slots", library().ts_copy_slots(_ptr(pool), layers * heads, page_size, row_bytes, src, dst, num_slots,
+    runs = 1
+    for n in pool.shape[1:slot_dim]:
+        runs *= n
+    inner = pool.element_size()
+    for n in pool.shape[slot_dim + 1:]:
+        inner *= n
+    _run("copy_slots", library().ts_copy_slots(_ptr(pool), runs, page_size * inner, num_slots * inner, src, dst,
                                                _stream()))
 
 
@@ -300,21 +326,93 @@ def sample(logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor,
 
 # ---- dispatchers ---------------------------------------------------------------------------------
 
+def attention_tiles(cu_seqlens: list[int], tokens_per_tile: int) -> list[int]:
+    """Row tiles of a packed step for the matrix-core prefill kernel: (first token, token count)
+    pairs, flattened; a tile never crosses a request."""
+    flat: list[int] = []
+    for a, b in zip(cu_seqlens, cu_seqlens[1:]):
+        for t in range(a, b, tokens_per_tile):
+            flat += (t, min(tokens_per_tile, b - t))
+    return flat
+
+
+def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                            seq_of_token: torch.Tensor, positions: torch.Tensor, tiles: torch.Tensor, scale: float,
+                            window: int = 0) -> torch.Tensor:
+    """Attention of a packed step on the matrix cores (bfloat16, values in transposed pages).
+    `tiles` int32 [num_tiles, 2] lists (first token, token count <= 16 // group) per row tile,
+    every tile inside one request; the caller has checked positions against the block tables."""
+    _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles)
+    _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
+    T, nh, hd = q.shape
+    nkv = k_cache.shape[2]
+    _check_cache(k_cache, v_cache, q.dtype, nkv, hd)
+    _need(nh % nkv == 0, f"{nh} heads do not divide into {nkv} key/value heads")
+    _need(decode_kernel_takes(q, k_cache, v_cache),
+          "the prefill kernel takes bfloat16, head_dim 32/64/96/128, groups of up to 16 heads, values in transposed pages")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
+          "block_tables must be contiguous int32 [requests, pages]")
+    for name, t in (("seq_of_token", seq_of_token), ("positions", positions)):
+        _need(t.dtype == torch.int32 and t.shape == (T,) and t.is_contiguous(), f"{name} must be int32 [tokens]")
+    _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 2 and tiles.is_contiguous(),
+          "tiles must be contiguous int32 [tiles, 2]")
+    out = torch.empty_like(q)
+    _run("paged_attention_prefill", library().ts_paged_attention_prefill(
+        _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_of_token), _ptr(positions),
+        _ptr(tiles), tiles.shape[0], nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3], v_cache.stride(0),
+        v_cache.stride(2), v_cache.stride(3), block_tables.shape[1], float(scale), int(window), _stream()))
+    return out
+
+
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx, space: int,
                     scale: float, window: int = 0) -> torch.Tensor:
     """Attention of a packed step over the cache; picks the kernel for the storage type and shape.
-    float32 always takes the one-wave-per-row kernel, whose sums do not depend on the batch."""
-    if q.dtype == torch.bfloat16 and ctx.max_query_len == 1 and q.shape[1] // k_cache.shape[2] <= 8:
-        return paged_attention_decode(q, k_cache, v_cache, ctx.block_tables[space], ctx.seq_of_token, ctx.positions,
-                                      scale, window)
-    return paged_attention_wave(q, k_cache, v_cache, ctx.block_tables[space], ctx.seq_of_token, ctx.positions,
-                                scale, window)
+    float32 always takes the one-wave-per-row kernel, whose sums do not depend on the batch;
+    bfloat16 takes the matrix-core kernels where they serve the shape."""
+    tables = ctx.block_tables[space]
+    if decode_kernel_takes(q, k_cache, v_cache):
+        capacity = tables.shape[1] * k_cache.shape[1]
+        if ctx.max_query_len == 1 and -(-capacity // 1024) <= MAX_DECODE_SPLITS:
+            return paged_attention_decode(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, window)
+        per_tile = 16 // (q.shape[1] // k_cache.shape[2])
+        tiles = ctx.scratch.get(("attention_tiles", per_tile))
+        if tiles is None:
+            flat = attention_tiles(ctx.host_cu_seqlens, per_tile)
+            tiles = torch.tensor(flat, dtype=torch.int32).view(-1, 2).to(q.device, non_blocking=True)
+            ctx.scratch[("attention_tiles", per_tile)] = tiles
+        return paged_attention_prefill(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, tiles, scale, window)
+    return paged_attention_wave(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, window)
 
 
-def linear_bf16(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-    """bfloat16 x [M, K] · weight [N, K]^T through the vendor matrix library."""
+SKINNY_MAX_ROWS = 64
+
+
+def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """bfloat16 x [M <= 64, K] · weight [N, K]^T by the weight-streaming MFMA kernel; K a multiple of 128."""
+    _gpu(x, weight)
+    _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "gemm_skinny takes bfloat16")
+    _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
+          f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
+    M, K = x.shape
+    _need(M <= SKINNY_MAX_ROWS and K % 128 == 0, f"gemm_skinny takes up to {SKINNY_MAX_ROWS} rows and K % 128 == 0")
+    _need(x.stride(1) == 1 and weight.stride(1) == 1 and x.stride(0) % 8 == 0 and weight.stride(0) % 8 == 0
+          and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0, "rows must be contiguous and 16-byte aligned")
+    out = torch.empty((M, weight.shape[0]), dtype=out_dtype, device=x.device)
+    _run("gemm_skinny", library().ts_gemm_skinny_bf16(_ptr(out), _ptr(x), _ptr(weight), M, weight.shape[0], K,
+                                                      x.stride(0), weight.stride(0), out.stride(0), _code(out_dtype),
+                                                      _stream()))
+    return out
+
+
+def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """bfloat16 x [M, K] · weight [N, K]^T: few rows go to the weight-streaming kernel, many to
+    the vendor matrix library."""
     _gpu(x, weight)
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "linear_bf16 takes bfloat16")
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
           f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
-    return torch.matmul(x, weight.t())
+    if (x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 128 == 0 and x.is_contiguous() and weight.is_contiguous()
+            and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
+        return gemm_skinny(x, weight, out_dtype)
+    y = torch.matmul(x, weight.t())
+    return y if out_dtype == torch.bfloat16 else y.to(out_dtype)

@@ -17,6 +17,8 @@ from tinyserve_llm_amd.parts.linear import linear
 
 @register("mixer", "attention")
 class Attention(Mixer):
+    graph_safe = True
+
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position: str | None = "rope", scale: float | None = None, window: int = 0) -> None:
         if num_heads % num_kv_heads:

@@ -82,6 +82,7 @@ class StepContext:
     host_context_lens: list[int] = field(default_factory=list)
     host_state_slots: list[int] = field(default_factory=list)
     position_encodings: dict[str, "PositionEncoding"] = field(default_factory=dict)
+    scratch: dict = field(default_factory=dict)     # what parts derive from a step once and share
 
     @property
     def max_query_len(self) -> int:
@@ -93,6 +94,11 @@ class StepContext:
 
 class Part:
     """Base of every part: declares parameters, receives them."""
+
+    # True if forward() only launches work on the current stream from the device tensors of the
+    # step context (no host reads of them, no Python branching on the host lists): such a part
+    # can be recorded into a HIP graph and replayed with new inputs.
+    graph_safe = False
 
     def param_specs(self) -> dict[str, ParamSpec]:
         return {}

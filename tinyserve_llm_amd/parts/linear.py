@@ -19,5 +19,4 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype | None 
         raise hip.KernelError(f"linear: no path for {x.dtype}")
     if not x.is_cuda:
         raise hip.KernelError("linear: GPU tensors only; there is no CPU path")
-    y = hip.linear_bf16(x, weight)
-    return y if out_dtype in (None, torch.bfloat16) else y.to(out_dtype)
+    return hip.linear_bf16(x, weight, out_dtype or torch.bfloat16)

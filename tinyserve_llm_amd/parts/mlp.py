@@ -12,6 +12,8 @@ from tinyserve_llm_amd.parts.linear import linear
 
 @register("feed_forward", "gated_mlp")
 class GatedMLP(FeedForward):
+    graph_safe = True
+
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu") -> None:
         if activation != "silu":
             raise ValueError(f"activation {activation!r}: the gated feed-forward kernel computes silu")

@@ -15,6 +15,8 @@ from tinyserve_llm_amd.parts.base import Norm, ParamSpec, register
 
 @register("norm", "rmsnorm")
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, hidden_size: int, eps: float) -> None:
         self.hidden_size = hidden_size
         self.eps = eps

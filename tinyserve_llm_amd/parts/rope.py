@@ -31,6 +31,8 @@ def inverse_frequencies(head_dim: int, theta: float, scaling: dict | None, max_p
 
 @register("position_encoding", "rope")
 class Rope(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, head_dim: int, max_position: int, theta: float, scaling: dict | None = None) -> None:
         self.head_dim = head_dim
         self.max_position = max_position
