@@ -397,6 +397,57 @@ def test_linear_bfloat16(m, n, k):
     assert f.dtype == torch.float32
 
 
+@pytest.mark.parametrize("m", [1, 3, 8, 16, 17, 32])
+@pytest.mark.parametrize("n,k", [(3072, 2048), (2048, 2048), (16384, 2048), (2048, 8192), (992, 512), (130, 3072), (64, 4096)])
+def test_weight_streaming_gemm_and_its_fused_inputs(m, n, k):
+    """The skinny kernel plain, with residual + RMSNorm on the way in, and with the SiLU gate on
+    the way in, against the same operations done one after the other in float64 with the storage
+    type's roundings in between."""
+    g = gen(m * 7 + n + k)
+    w = (torch.randn(n, k, generator=g) * 0.05).bfloat16()
+    x = torch.randn(m, k, generator=g).bfloat16()
+    assert hip().skinny_takes(m, k)
+    out, none = hip().gemm_skinny(x.to(dev()), w.to(dev()))
+    want = x.double() @ w.double().T
+    assert none is None and out.dtype == torch.bfloat16
+    torch.testing.assert_close(out.double().cpu(), want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
+    f32, _ = hip().gemm_skinny(x.to(dev()), w.to(dev()), torch.float32)
+    torch.testing.assert_close(f32.double().cpu(), want, rtol=1e-4, atol=1e-4 * float(want.abs().max()))
+    one, _ = hip().gemm_skinny(x[m // 2:m // 2 + 1].contiguous().to(dev()), w.to(dev()), torch.float32)
+    assert torch.equal(one, f32[m // 2:m // 2 + 1]), "a row's result does not depend on the other rows"
+    if hip().skinny_fuses(m, k, True, False):
+        res = torch.randn(m, k, generator=g).bfloat16()
+        nw = (1 + 0.1 * torch.randn(k, generator=g)).bfloat16()
+        for r in (res, None):
+            for glu in (False, True):
+                if glu and not (n % 32 == 0 and hip().skinny_fuses(m, k, True, True)):
+                    continue
+                out, res_out = hip().gemm_skinny(x.to(dev()), w.to(dev()), residual=None if r is None else r.to(dev()),
+                                                 norm_weight=nw.to(dev()), eps=1e-5, glu=glu)
+                s = x.float() + (r.float() if r is not None else 0)
+                assert torch.equal(res_out.cpu(), s.bfloat16()), "the new residual is the sum, rounded once"
+                y = (s * torch.rsqrt(s.pow(2).mean(-1, keepdim=True) + 1e-5)).bfloat16() * nw      # llama.py:63-67
+                want = y.double() @ w.double().T
+                if glu:
+                    want = P.silu_mul(want)
+                torch.testing.assert_close(out.double().cpu(), want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
+    if n % 32 == 0 and hip().skinny_fuses(m, k, False, True):
+        out, _ = hip().gemm_skinny(x.to(dev()), w.to(dev()), glu=True)
+        want = P.silu_mul(x.double() @ w.double().T)
+        assert out.shape == (m, n // 2)
+        torch.testing.assert_close(out.double().cpu(), want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
+
+
+def test_weight_streaming_gemm_refuses_what_it_cannot_take():
+    x = torch.zeros(33, 2048, dtype=torch.bfloat16, device=dev())
+    w = torch.zeros(64, 2048, dtype=torch.bfloat16, device=dev())
+    assert not hip().skinny_takes(33, 2048) and not hip().skinny_takes(8, 96) and not hip().skinny_takes(8, 14336)
+    with pytest.raises(hip().KernelError, match="rows"):
+        hip().gemm_skinny(x, w)
+    from tinyserve_llm_amd.parts.linear import linear
+    assert linear(x, w).shape == (33, 64), "the vendor library takes what the skinny kernel does not"
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_silu_mul(dtype):
     gu = torch.randn(9, 2 * 150, generator=gen(13)).to(dtype)

@@ -1,137 +1,276 @@
-// y[M, N] = x[M, K] · W[N, K]^T for bfloat16 with few rows of x (decoding: M up to 64), where time
-// goes to reading W once from HBM. A workgroup of four waves owns 16 or 32 rows of W; the waves
-// split K among them, stream their slice of those rows with 16-byte loads straight into MFMA
-// operands (v_mfma_f32_16x16x16_bf16: W rows are the A matrix, x^T the B matrix), and the four
-// partial tiles are summed in LDS in a fixed order. x is read through the caches (it is tiny and
-// shared by every workgroup). Accumulation is 32-bit; the result is rounded once.
+// y[M, N] = e(f(x)[M, K] · W[N, K]^T) for bfloat16 with few rows of x (decoding: M up to 32), where
+// time goes to reading W once from HBM. A workgroup owns 16 to 64 rows of W over the whole of K;
+// each of its waves takes a slice of K of 256 or 512 and issues every load of its slice of W before
+// it uses the first, so that a cold matrix streams at memory speed; the rows go straight from the
+// 16-byte loads into MFMA operands (v_mfma_f32_16x16x16_bf16: W rows are the A matrix, x^T the B
+// matrix), and the waves' partial tiles are summed in LDS in a fixed order. Accumulation is 32-bit;
+// the result is rounded once.
+//
+// x is read through the caches (it is tiny and shared by every workgroup). What precedes and
+// follows the product in a layer can ride along, so that no separate kernel has to run:
+//   MODE_NORM  f(x) = T(T((x + res) * rsqrt(mean((x + res)^2) + eps)) * nw): residual + RMSNorm on
+//              the way in (up to 16 rows); workgroup 0 also writes T(x + res) as the new residual
+//   EPI_GLU    W = [gate rows | up rows]; a workgroup takes matching rows of both and writes
+//              silu(gate) * up, y being [M, N / 2]
 #include "common.h"
 
 typedef short short4_t __attribute__((ext_vector_type(4)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
-#define SK_WAVES 4
-#define SK_KSTEP 32   // k covered by one pair of MFMAs: lane group g holds k = 8 g .. 8 g + 7
+#define SK_KSTEP 32      // k covered by one pair of MFMAs: lane group g holds k = 8 g .. 8 g + 7
+#define MODE_PLAIN 0
+#define MODE_NORM 1
 
-// RT: 16-row tiles of W per workgroup (1 or 2); CB: 16-row blocks of x (1..4)
-template <int RT, int CB, typename OUT>
-__global__ void __launch_bounds__(SK_WAVES * TS_WAVE)
-gemm_skinny_kernel(OUT* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, int M, int N,
-                   int K, int64_t ldx, int64_t ldw, int64_t ldy) {
-  __shared__ float part[SK_WAVES][RT][CB][16 * 16];
+static __device__ __forceinline__ short4_t sk_lo(const uint4& v) { return __builtin_bit_cast(short4_t, make_uint2(v.x, v.y)); }
+static __device__ __forceinline__ short4_t sk_hi(const uint4& v) { return __builtin_bit_cast(short4_t, make_uint2(v.z, v.w)); }
+
+static __device__ __forceinline__ void sk_unpack(const uint4& v, float* f) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[2 * i] = __uint_as_float(w[i] << 16);
+    f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+// round to nearest even; the values here are finite sums and products of finite activations
+static __device__ __forceinline__ uint32_t sk_round(float f) {
+  const uint32_t u = __float_as_uint(f);
+  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+static __device__ __forceinline__ uint4 sk_pack(const float* f) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = sk_round(f[2 * i]) | (sk_round(f[2 * i + 1]) << 16);
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+static __device__ __forceinline__ float sk_silu(float g) {
+  return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896340736f * g));
+}
+
+struct SkinnyArgs {
+  const bf16_t* x;      // [M, K] (MODE_GATE: [M, 2K])
+  const bf16_t* res;    // MODE_NORM: residual [M, K] or null
+  const bf16_t* nw;     // MODE_NORM: norm weight [K]
+  bf16_t* res_out;      // MODE_NORM with res: new residual [M, K]
+  const bf16_t* w;      // [N, K]
+  void* y;              // [M, N]
+  int M, N, K;
+  int64_t ldx, ldw, ldy;
+  float eps;
+};
+
+// RT: 16-row tiles of W per workgroup; CB: 16-row blocks of x; STEPS: 32-wide k steps per wave;
+// MAXT: most threads a workgroup of this instance is launched with (it bounds the registers)
+template <int RT, int CB, int STEPS, int MODE, int GLU, int MAXT, typename OUT>
+__global__ void __launch_bounds__(MAXT)
+gemm_skinny_kernel(const SkinnyArgs a) {
+  static_assert(MODE == MODE_PLAIN || CB == 1, "the fused norm serves one block of rows");
+  static_assert(!GLU || RT % 2 == 0, "gate and up tiles come in pairs");
+  constexpr int SK_XBATCH = (CB == 2 && MAXT > 512) ? 4 : 8;   // steps of x fetched at a time
+  extern __shared__ __align__(16) float smem[];
+  const int nwaves = blockDim.x / TS_WAVE;
+  float* part = smem;                                   // [nwaves][RT][CB][256]
+  float* ssq = smem + (size_t)nwaves * RT * CB * 256;   // [nwaves][16]
   const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * 16 * RT;
-  const int kslice = K / SK_WAVES;              // a multiple of SK_KSTEP (checked on the host)
-  const int kbeg = wave * kslice;
+  // GLU: tiles 0 .. RT/2-1 are gate rows n0 + 16 t, tiles RT/2 .. RT-1 the up rows N/2 below them
+  constexpr int OT = GLU ? RT / 2 : RT;                 // 16-column tiles of the output per workgroup
+  const int n0 = blockIdx.x * 16 * OT;
+  const int half = a.N / 2;
+  const int kbeg = wave * STEPS * SK_KSTEP + 8 * g;     // this lane's first k
 
-  float4_t acc[RT][CB];
+  // ---- every load of this wave's slice of W, at once
+  uint4 wreg[RT][STEPS];
 #pragma unroll
-  for (int a = 0; a < RT; ++a)
+  for (int t = 0; t < RT; ++t) {
+    int n = GLU ? (t < OT ? n0 + t * 16 + r : half + n0 + (t - OT) * 16 + r) : n0 + t * 16 + r;
+    const int limit = GLU ? (t < OT ? half : a.N) : a.N;
+    if (n >= limit) n = limit - 1;                      // rows past the end are computed and not stored
+    const bf16_t* wrow = a.w + (int64_t)n * a.ldw + kbeg;
 #pragma unroll
-    for (int b = 0; b < CB; ++b) acc[a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
-
-  const bf16_t* wrow[RT];
-#pragma unroll
-  for (int a = 0; a < RT; ++a) {
-    int n = n0 + a * 16 + r;
-    if (n >= N) n = N - 1;                       // rows past the end are computed and not stored
-    wrow[a] = w + (int64_t)n * ldw + kbeg + 8 * g;
+    for (int s = 0; s < STEPS; ++s) wreg[t][s] = *(const uint4*)(wrow + s * SK_KSTEP);
   }
+
   const bf16_t* xrow[CB];
   bool xok[CB];
 #pragma unroll
   for (int b = 0; b < CB; ++b) {
     const int m = b * 16 + r;
-    xok[b] = m < M;
-    xrow[b] = x + (int64_t)(xok[b] ? m : 0) * ldx + kbeg + 8 * g;
+    xok[b] = m < a.M;
+    xrow[b] = a.x + (int64_t)(xok[b] ? m : 0) * a.ldx + kbeg;
   }
 
-#pragma unroll 4
-  for (int k = 0; k < kslice; k += SK_KSTEP) {
-    uint4 wa[RT], xb[CB];
+  float4_t acc[RT][CB];
 #pragma unroll
-    for (int a = 0; a < RT; ++a) wa[a] = *(const uint4*)(wrow[a] + k);
+  for (int t = 0; t < RT; ++t)
 #pragma unroll
-    for (int b = 0; b < CB; ++b) xb[b] = xok[b] ? *(const uint4*)(xrow[b] + k) : make_uint4(0, 0, 0, 0);
+    for (int b = 0; b < CB; ++b) acc[t][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+
+  if (MODE == MODE_NORM) {
+    // ---- x + res of this wave's slice stays in registers: summed squares first (all waves of the
+    // workgroup together), then scaled, rounded and used
+    float xs[STEPS][8];
+    float sq = 0.f;
 #pragma unroll
-    for (int a = 0; a < RT; ++a) {
-      const short4_t a0 = __builtin_bit_cast(short4_t, make_uint2(wa[a].x, wa[a].y));
-      const short4_t a1 = __builtin_bit_cast(short4_t, make_uint2(wa[a].z, wa[a].w));
+    for (int s = 0; s < STEPS; ++s) {
 #pragma unroll
-      for (int b = 0; b < CB; ++b) {
-        const short4_t b0 = __builtin_bit_cast(short4_t, make_uint2(xb[b].x, xb[b].y));
-        const short4_t b1 = __builtin_bit_cast(short4_t, make_uint2(xb[b].z, xb[b].w));
-        acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a0, b0, acc[a][b], 0, 0, 0);
-        acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a1, b1, acc[a][b], 0, 0, 0);
+      for (int i = 0; i < 8; ++i) xs[s][i] = 0.f;
+      if (xok[0]) {
+        sk_unpack(*(const uint4*)(xrow[0] + s * SK_KSTEP), xs[s]);
+        if (a.res) {
+          float rv[8];
+          sk_unpack(*(const uint4*)(a.res + (int64_t)r * a.K + kbeg + s * SK_KSTEP), rv);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) xs[s][i] += rv[i];
+          if (blockIdx.x == 0) *(uint4*)(a.res_out + (int64_t)r * a.K + kbeg + s * SK_KSTEP) = sk_pack(xs[s]);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sq = fmaf(xs[s][i], xs[s][i], sq);
       }
     }
-  }
-  // acc[a][b][j] = sum over this wave's k of W[n0 + 16 a + 4 g + j, k] * x[16 b + r, k]
+    sq += __shfl_xor(sq, 16, TS_WAVE);
+    sq += __shfl_xor(sq, 32, TS_WAVE);
+    if (g == 0) ssq[wave * 16 + r] = sq;
+    __syncthreads();
+    float total = 0.f;
+    for (int wv = 0; wv < nwaves; ++wv) total += ssq[wv * 16 + r];
+    const float inv = 1.0f / sqrtf(total / (float)a.K + a.eps);
 #pragma unroll
-  for (int a = 0; a < RT; ++a)
+    for (int s = 0; s < STEPS; ++s) {
+      float nv[8];
+      sk_unpack(*(const uint4*)(a.nw + kbeg + s * SK_KSTEP), nv);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) xs[s][i] = __uint_as_float(sk_round(xs[s][i] * inv) << 16) * nv[i];
+      const uint4 xb = sk_pack(xs[s]);
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        acc[t][0] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(sk_lo(wreg[t][s]), sk_lo(xb), acc[t][0], 0, 0, 0);
+        acc[t][0] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(sk_hi(wreg[t][s]), sk_hi(xb), acc[t][0], 0, 0, 0);
+      }
+    }
+  } else {
+    // ---- x in batches of steps, then the products
+#pragma unroll
+    for (int s0 = 0; s0 < STEPS; s0 += SK_XBATCH) {
+      uint4 xb[CB][SK_XBATCH];
+#pragma unroll
+      for (int b = 0; b < CB; ++b)
+#pragma unroll
+        for (int s = 0; s < SK_XBATCH; ++s)
+          xb[b][s] = xok[b] ? *(const uint4*)(xrow[b] + (s0 + s) * SK_KSTEP) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int s = 0; s < SK_XBATCH; ++s)
+#pragma unroll
+        for (int t = 0; t < RT; ++t)
+#pragma unroll
+          for (int b = 0; b < CB; ++b) {
+            acc[t][b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(sk_lo(wreg[t][s0 + s]), sk_lo(xb[b][s]), acc[t][b], 0, 0, 0);
+            acc[t][b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(sk_hi(wreg[t][s0 + s]), sk_hi(xb[b][s]), acc[t][b], 0, 0, 0);
+          }
+    }
+  }
+  // acc[t][b][j] = sum over this wave's k of W[row 16 t + 4 g + j of the workgroup, k] * f(x)[16 b + r, k]
+#pragma unroll
+  for (int t = 0; t < RT; ++t)
 #pragma unroll
     for (int b = 0; b < CB; ++b)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) part[wave][a][b][r * 16 + 4 * g + j] = acc[a][b][j];
+      for (int j = 0; j < 4; ++j) part[(((size_t)wave * RT + t) * CB + b) * 256 + r * 16 + 4 * g + j] = acc[t][b][j];
   __syncthreads();
-  // part[.][a][b][m_local * 16 + n_local]: each thread sums 4 consecutive n of one m, all waves in order
-  for (int idx = threadIdx.x; idx < RT * CB * 64; idx += SK_WAVES * TS_WAVE) {
+  // part[.][t][b][m_local * 16 + n_local]: a thread sums 4 consecutive n of one m over the waves in order
+  OUT* y = (OUT*)a.y;
+  const int ncols = GLU ? half : a.N;
+  for (int idx = threadIdx.x; idx < OT * CB * 64; idx += blockDim.x) {
     const int tile = idx >> 6, e = idx & 63;
-    const int a = tile / CB, b = tile - a * CB;
+    const int t = tile / CB, b = tile - t * CB;
     const int ml = e >> 2, nl = (e & 3) * 4;
-    const int m = b * 16 + ml, n = n0 + a * 16 + nl;
-    if (m >= M) continue;
-    float s[4];
+    const int m = b * 16 + ml, n = n0 + t * 16 + nl;
+    if (m >= a.M) continue;
+    float s[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int wv = 0; wv < nwaves; ++wv) {
+      const float* p = part + (((size_t)wv * RT + t) * CB + b) * 256 + ml * 16 + nl;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      float t = 0.f;
+      for (int j = 0; j < 4; ++j) s[j] += p[j];
+      if (GLU) {
+        const float* pu = part + (((size_t)wv * RT + t + OT) * CB + b) * 256 + ml * 16 + nl;
 #pragma unroll
-      for (int wv = 0; wv < SK_WAVES; ++wv) t += part[wv][a][b][ml * 16 + nl + j];
-      s[j] = t;
+        for (int j = 0; j < 4; ++j) u[j] += pu[j];
+      }
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      if (n + j < N) Num<OUT>::st(y + (int64_t)m * ldy + n + j, s[j]);
+      if (n + j < ncols) Num<OUT>::st(y + (int64_t)m * a.ldy + n + j, GLU ? sk_silu(s[j]) * u[j] : s[j]);
   }
 }
 
-template <typename OUT>
-static int launch_skinny(void* y, const void* x, const void* w, int M, int N, int K, int64_t ldx, int64_t ldw,
-                         int64_t ldy, hipStream_t stream) {
-  const int cb = (M + 15) / 16;
-  // two row tiles per workgroup once that still leaves a few workgroups per compute unit
-  const int rt = (N >= 16 * 2 * 1024) ? 2 : 1;
-  dim3 grid((N + 16 * rt - 1) / (16 * rt)), block(SK_WAVES * TS_WAVE);
-#define SK_LAUNCH(RT, CB)                                                                                      \
-  gemm_skinny_kernel<RT, CB, OUT><<<grid, block, 0, stream>>>((OUT*)y, (const bf16_t*)x, (const bf16_t*)w, M, N, \
-                                                              K, ldx, ldw, ldy)
-  if (rt == 1) {
-    switch (cb) {
-      case 1: SK_LAUNCH(1, 1); break;
-      case 2: SK_LAUNCH(1, 2); break;
-      case 3: SK_LAUNCH(1, 3); break;
-      default: SK_LAUNCH(1, 4); break;
-    }
-  } else {
-    switch (cb) {
-      case 1: SK_LAUNCH(2, 1); break;
-      case 2: SK_LAUNCH(2, 2); break;
-      case 3: SK_LAUNCH(2, 3); break;
-      default: SK_LAUNCH(2, 4); break;
-    }
-  }
-#undef SK_LAUNCH
+template <int RT, int CB, int STEPS, int MODE, int GLU, typename OUT>
+static int sk_launch(const SkinnyArgs& a, hipStream_t stream) {
+  const int nwaves = a.K / (STEPS * SK_KSTEP);
+  const size_t smem = sizeof(float) * ((size_t)nwaves * RT * CB * 256 + (size_t)nwaves * 16);
+  constexpr int OT = GLU ? RT / 2 : RT;
+  const int ncols = GLU ? a.N / 2 : a.N;
+  dim3 grid((ncols + 16 * OT - 1) / (16 * OT)), block(nwaves * TS_WAVE);
+  if (nwaves <= 8)
+    gemm_skinny_kernel<RT, CB, STEPS, MODE, GLU, 512, OUT><<<grid, block, smem, stream>>>(a);
+  else
+    gemm_skinny_kernel<RT, CB, STEPS, MODE, GLU, 1024, OUT><<<grid, block, smem, stream>>>(a);
   return ts_check_launch();
 }
 
-// out_dtype: 1 bfloat16, 0 float. Requires M <= 64, K a multiple of 128, 16-byte aligned rows.
-extern "C" int ts_gemm_skinny_bf16(void* y, const void* x, const void* w, int M, int N, int K, int64_t ldx,
-                                   int64_t ldw, int64_t ldy, int out_dtype, hipStream_t stream) {
-  if (M <= 0 || N <= 0) return TS_OK;
-  if (M > 64 || K <= 0 || K % (SK_WAVES * SK_KSTEP) || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ldy < N)
+// Picks the instance: slices of 256 k while that needs at most 16 waves, else slices of 512; more
+// rows of W per workgroup for wide matrices once that still leaves a workgroup per compute unit
+// (fewer workgroups repeat less of the work on x).
+template <int MODE, int GLU, typename OUT>
+static int sk_dispatch(const SkinnyArgs& a, hipStream_t stream) {
+  const int steps = (a.K % 256 == 0 && a.K / 256 <= 16) ? 8 : 16;
+  if (a.K % (steps * SK_KSTEP) || a.K / (steps * SK_KSTEP) > 16) return TS_BAD_SHAPE;
+  const int nwaves = a.K / (steps * SK_KSTEP);
+  const int cb = (a.M + 15) / 16;
+  if ((MODE == MODE_NORM || GLU) && cb != 1) return TS_BAD_SHAPE;
+  const int ncols = GLU ? a.N / 2 : a.N;
+#define SK_GO(RT, CB, ST) return sk_launch<RT, CB, ST, MODE, GLU, OUT>(a, stream)
+  if constexpr (MODE == MODE_NORM || GLU != 0) {
+    // the instances that hold x + res or four row tiles need the registers of a workgroup of 8 waves
+    if (steps != 8) return TS_BAD_SHAPE;
+    if (nwaves <= 8) {
+      if (ncols >= 4096 * (GLU ? 1 : 2)) SK_GO(4, 1, 8);
+      if (GLU || ncols >= 4096) SK_GO(2, 1, 8);
+    }
+    if constexpr (GLU == 0) SK_GO(1, 1, 8);
     return TS_BAD_SHAPE;
-  if (((uintptr_t)x | (uintptr_t)w) & 15) return TS_BAD_SHAPE;
-  if (out_dtype == 1) return launch_skinny<bf16_t>(y, x, w, M, N, K, ldx, ldw, ldy, stream);
-  if (out_dtype == 0) return launch_skinny<float>(y, x, w, M, N, K, ldx, ldw, ldy, stream);
+  } else {
+    const bool two = a.N >= 8192 && nwaves <= 8;
+    if (steps == 8) {
+      if (two) { if (cb == 1) SK_GO(2, 1, 8); else SK_GO(2, 2, 8); }
+      if (cb == 1) SK_GO(1, 1, 8); else SK_GO(1, 2, 8);
+    }
+    if (cb == 1) SK_GO(1, 1, 16); else SK_GO(1, 2, 16);
+  }
+#undef SK_GO
+}
+
+// mode: 0 plain, 1 residual + RMSNorm on the way in (M <= 16, K in steps of 256 up to 4096). glu: W holds
+// gate rows then up rows, y is [M, N / 2] = silu(gate) * up (M <= 16). out_dtype: 1 bfloat16, 0 float
+// (plain only). Requires M <= 32, K a multiple of 256 (up to 4096) or of 512 (up to 8192), contiguous
+// 16-byte aligned rows; mode 1 takes x, res, res_out as dense [M, K].
+extern "C" int ts_gemm_skinny_bf16(void* y, const void* x, const void* w, const void* res, const void* nw,
+                                   void* res_out, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldy,
+                                   float eps, int mode, int glu, int out_dtype, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return TS_OK;
+  if (M > 32 || K <= 0 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ldy < (glu ? N / 2 : N)) return TS_BAD_SHAPE;
+  if (glu && (N % 2 || (N / 2) % 16)) return TS_BAD_SHAPE;
+  if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)res | (uintptr_t)nw | (uintptr_t)res_out) & 15) return TS_BAD_SHAPE;
+  if (mode == MODE_NORM && (!nw || (res && !res_out))) return TS_BAD_SHAPE;
+  SkinnyArgs a;
+  a.x = (const bf16_t*)x; a.res = (const bf16_t*)res; a.nw = (const bf16_t*)nw; a.res_out = (bf16_t*)res_out;
+  a.w = (const bf16_t*)w; a.y = y; a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldw = ldw; a.ldy = ldy; a.eps = eps;
+  if (out_dtype == 1) {
+    if (mode == MODE_PLAIN && !glu) return sk_dispatch<MODE_PLAIN, 0, bf16_t>(a, stream);
+    if (mode == MODE_PLAIN && glu) return sk_dispatch<MODE_PLAIN, 1, bf16_t>(a, stream);
+    if (mode == MODE_NORM && !glu) return sk_dispatch<MODE_NORM, 0, bf16_t>(a, stream);
+    if (mode == MODE_NORM && glu) return sk_dispatch<MODE_NORM, 1, bf16_t>(a, stream);
+    return TS_BAD_SHAPE;
+  }
+  if (out_dtype == 0 && mode == MODE_PLAIN && !glu) return sk_dispatch<MODE_PLAIN, 0, float>(a, stream);
   return TS_BAD_DTYPE;
 }

@@ -53,7 +53,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_gemm_exact": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_sample": [p, p, p, p, u64, i, i, i64, p],
         "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, p],
-        "ts_gemm_skinny_bf16": [p, p, p, i, i, i, i64, i64, i64, i, p],
+        "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, p],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -384,24 +384,61 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     return paged_attention_wave(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, window)
 
 
-SKINNY_MAX_ROWS = 64
+SKINNY_MAX_ROWS = 32
+SKINNY_FUSED_ROWS = 16       # the fused norm and the gated epilogue serve one 16-row block of x
 
 
-def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
-    """bfloat16 x [M <= 64, K] · weight [N, K]^T by the weight-streaming MFMA kernel; K a multiple of 128."""
-    _gpu(x, weight)
+def skinny_takes(rows: int, k: int) -> bool:
+    """Whether the weight-streaming kernel serves `rows` rows of x over a reduction of `k`."""
+    return rows <= SKINNY_MAX_ROWS and ((k % 256 == 0 and k // 256 <= 16) or (k % 512 == 0 and k // 512 <= 16))
+
+
+def skinny_fuses(rows: int, k: int, norm: bool, glu: bool) -> bool:
+    """Whether the kernel can apply the norm on the way in and/or the gate on the way out."""
+    if not (norm or glu):
+        return skinny_takes(rows, k)
+    return rows <= SKINNY_FUSED_ROWS and k % 256 == 0 and k // 256 <= (8 if glu else 16)
+
+
+def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, *,
+                residual: torch.Tensor | None = None, norm_weight: torch.Tensor | None = None, eps: float = 0.0,
+                glu: bool = False) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """bfloat16 e(f(x) [M <= 32, K] · weight [N, K]^T) by the weight-streaming MFMA kernel.
+    With `norm_weight`: f = RMSNorm(x + residual) * norm_weight, and x + residual comes back as the
+    second result. With `glu`: weight holds gate rows then up rows and the result is
+    silu(gate) * up, [M, N / 2]."""
+    _gpu(x, weight, residual, norm_weight)
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "gemm_skinny takes bfloat16")
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
           f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
     M, K = x.shape
-    _need(M <= SKINNY_MAX_ROWS and K % 128 == 0, f"gemm_skinny takes up to {SKINNY_MAX_ROWS} rows and K % 128 == 0")
-    _need(x.stride(1) == 1 and weight.stride(1) == 1 and x.stride(0) % 8 == 0 and weight.stride(0) % 8 == 0
-          and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0, "rows must be contiguous and 16-byte aligned")
-    out = torch.empty((M, weight.shape[0]), dtype=out_dtype, device=x.device)
-    _run("gemm_skinny", library().ts_gemm_skinny_bf16(_ptr(out), _ptr(x), _ptr(weight), M, weight.shape[0], K,
-                                                      x.stride(0), weight.stride(0), out.stride(0), _code(out_dtype),
-                                                      _stream()))
-    return out
+    N = weight.shape[0]
+    norm = norm_weight is not None
+    _need(skinny_fuses(M, K, norm, glu),
+          f"gemm_skinny takes up to {SKINNY_MAX_ROWS} rows ({SKINNY_FUSED_ROWS} when fused) and K in steps of 256 up to "
+          "4096 (2048 with the gate) or of 512 up to 8192")
+    _need(x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0,
+          "rows must be contiguous and 16-byte aligned")
+    _need(not glu or (N % 32 == 0), "gate and up rows come in whole 16-row tiles")
+    res_out = None
+    if norm:
+        _need(norm_weight.dtype == torch.bfloat16 and norm_weight.shape == (K,) and norm_weight.is_contiguous(),
+              "the norm weight must be bfloat16 [K]")
+        if residual is not None:
+            _need(residual.shape == x.shape and residual.dtype == x.dtype and residual.is_contiguous(),
+                  "residual must match the input")
+            res_out = torch.empty_like(x)
+        else:
+            res_out = x
+    else:
+        _need(residual is None, "a residual comes with a norm weight")
+    _need(out_dtype == torch.bfloat16 or not (norm or glu), "float32 output comes with the plain product only")
+    out = torch.empty((M, N // 2 if glu else N), dtype=out_dtype, device=x.device)
+    _run("gemm_skinny", library().ts_gemm_skinny_bf16(
+        _ptr(out), _ptr(x), _ptr(weight), _ptr(residual), _ptr(norm_weight),
+        _ptr(res_out) if residual is not None else None, M, N, K, x.stride(0), weight.stride(0), out.stride(0),
+        float(eps), int(norm), int(glu), _code(out_dtype), _stream()))
+    return out, res_out
 
 
 def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
@@ -411,8 +448,8 @@ def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "linear_bf16 takes bfloat16")
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
           f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
-    if (x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 128 == 0 and x.is_contiguous() and weight.is_contiguous()
+    if (skinny_takes(x.shape[0], x.shape[1]) and x.is_contiguous() and weight.is_contiguous()
             and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
-        return gemm_skinny(x, weight, out_dtype)
+        return gemm_skinny(x, weight, out_dtype)[0]
     y = torch.matmul(x, weight.t())
     return y if out_dtype == torch.bfloat16 else y.to(out_dtype)

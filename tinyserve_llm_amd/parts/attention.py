@@ -18,6 +18,7 @@ from tinyserve_llm_amd.parts.linear import linear
 @register("mixer", "attention")
 class Attention(Mixer):
     graph_safe = True
+    takes_deferred_norm = True
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position: str | None = "rope", scale: float | None = None, window: int = 0) -> None:

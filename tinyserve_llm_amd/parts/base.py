@@ -114,6 +114,12 @@ class Norm(Part):
         """(normalised(x + residual), x + residual); `rows` restricts the output to some rows."""
         raise NotImplementedError
 
+    def defer(self, x: torch.Tensor, residual: torch.Tensor | None = None):
+        """Optionally the norm as an operand for a part that declares `takes_deferred_norm`: an
+        object whose first consumer computes it (possibly fused into its own kernel) and which
+        then holds `residual_out`. None (the default): this norm is always computed by itself."""
+        return None
+
 
 class PositionEncoding(Part):
     def prepare(self, device: torch.device) -> None:
@@ -129,6 +135,10 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    # True if forward() passes x to exactly one `linear()` call and uses it nowhere else, so that a
+    # norm may hand it over deferred (see Norm.defer)
+    takes_deferred_norm = False
+
     def kv_spec(self) -> KVSpec | None:
         return None
 
@@ -140,6 +150,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    takes_deferred_norm = False    # as for Mixer
+
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         raise NotImplementedError
 

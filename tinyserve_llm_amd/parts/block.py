@@ -27,8 +27,18 @@ class Layer:
 @register("block", "pre_norm")
 def pre_norm_block(layer: Layer, hidden: torch.Tensor, residual: torch.Tensor | None, ctx: StepContext,
                    mem: LayerMemory) -> tuple[torch.Tensor, torch.Tensor]:
-    x, residual = layer.mixer_norm(hidden, residual)
-    x = layer.mixer.forward(x, ctx, mem)
-    x, residual = layer.ff_norm(x, residual)
-    x = layer.feed_forward.forward(x, ctx)
+    pending = layer.mixer_norm.defer(hidden, residual) if layer.mixer.takes_deferred_norm else None
+    if pending is None:
+        x, residual = layer.mixer_norm(hidden, residual)
+        x = layer.mixer.forward(x, ctx, mem)
+    else:
+        x = layer.mixer.forward(pending, ctx, mem)
+        residual = pending.residual_out
+    pending = layer.ff_norm.defer(x, residual) if layer.feed_forward.takes_deferred_norm else None
+    if pending is None:
+        x, residual = layer.ff_norm(x, residual)
+        x = layer.feed_forward.forward(x, ctx)
+    else:
+        x = layer.feed_forward.forward(pending, ctx)
+        residual = pending.residual_out
     return x, residual

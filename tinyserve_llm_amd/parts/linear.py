@@ -1,8 +1,14 @@
 """y = x · Wᵀ for bias-free projections stored [out, in] (tinyserve_llm/model/llama.py:179,201,221,293).
 
 float32 runs the engine's own exact kernel (32-bit multiply-adds, ascending k, independent of the
-batch). bfloat16 uses the skinny weight-streaming kernel for few rows and the vendor matrix
-library for many, as the reference uses a vendor library for every projection.
+batch). bfloat16 uses the weight-streaming kernel for few rows and the vendor matrix library for
+many, as the reference uses a vendor library for every projection.
+
+With few rows a step's time goes to launching kernels and to waiting for memory, so what
+precedes or follows a projection can ride along with it: a norm may hand its input over as a
+`DeferredNorm` and the projection applies residual add and normalisation while it reads x; a
+gated feed-forward may ask for silu(gate) * up straight out of the gate|up projection. Where the
+fused kernel does not serve the shape, the same calls run the separate kernels.
 """
 
 from __future__ import annotations
@@ -12,7 +18,40 @@ import torch
 from tinyserve_llm_amd.ops import hip
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+class DeferredNorm:
+    """norm(x + residual) * weight, not yet computed: the first projection that takes it either
+    fuses it or materialises it. Either way `residual_out` then holds x + residual."""
+
+    def __init__(self, x: torch.Tensor, residual: torch.Tensor | None, weight: torch.Tensor, eps: float) -> None:
+        self.x, self.residual, self.weight, self.eps = x, residual, weight, eps
+        self.residual_out: torch.Tensor | None = None
+
+    def materialize(self) -> torch.Tensor:
+        out, self.residual_out = hip.rmsnorm(self.x, self.weight, self.eps, self.residual)
+        return out
+
+
+def _streams(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.is_cuda and x.is_contiguous()
+            and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+
+
+def linear(x: torch.Tensor | DeferredNorm, weight: torch.Tensor, out_dtype: torch.dtype | None = None,
+           glu: bool = False) -> torch.Tensor:
+    """x · Wᵀ; with `glu`, W holds gate rows then up rows and silu(gate) * up comes back."""
+    if isinstance(x, DeferredNorm):
+        d = x
+        if (out_dtype in (None, torch.bfloat16) and _streams(d.x, weight) and d.weight.dtype == torch.bfloat16
+                and (d.residual is None or d.residual.is_contiguous())
+                and hip.skinny_fuses(d.x.shape[0], weight.shape[1], True, glu) and (not glu or weight.shape[0] % 32 == 0)):
+            y, d.residual_out = hip.gemm_skinny(d.x, weight, residual=d.residual, norm_weight=d.weight, eps=d.eps, glu=glu)
+            return y
+        x = d.materialize()
+    if glu:
+        if (out_dtype in (None, torch.bfloat16) and _streams(x, weight) and weight.shape[0] % 32 == 0
+                and hip.skinny_fuses(x.shape[0], weight.shape[1], False, True)):
+            return hip.gemm_skinny(x, weight, glu=True)[0]
+        return hip.silu_mul(linear(x, weight, out_dtype))
     if x.dtype == torch.float32:
         return hip.gemm_exact(x, weight, out_dtype)
     if x.dtype != torch.bfloat16:

@@ -5,7 +5,6 @@ from __future__ import annotations
 
 import torch
 
-from tinyserve_llm_amd.ops import hip
 from tinyserve_llm_amd.parts.base import FeedForward, ParamSpec, StepContext, register
 from tinyserve_llm_amd.parts.linear import linear
 
@@ -13,6 +12,7 @@ from tinyserve_llm_amd.parts.linear import linear
 @register("feed_forward", "gated_mlp")
 class GatedMLP(FeedForward):
     graph_safe = True
+    takes_deferred_norm = True
 
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu") -> None:
         if activation != "silu":
@@ -27,4 +27,4 @@ class GatedMLP(FeedForward):
                 "down": ParamSpec((self.hidden_size, self.intermediate_size))}
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
-        return linear(hip.silu_mul(linear(x, self.gate_up)), self.down)
+        return linear(linear(x, self.gate_up, glu=True), self.down)

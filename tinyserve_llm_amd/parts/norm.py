@@ -11,6 +11,7 @@ import torch
 
 from tinyserve_llm_amd.ops import hip
 from tinyserve_llm_amd.parts.base import Norm, ParamSpec, register
+from tinyserve_llm_amd.parts.linear import DeferredNorm
 
 
 @register("norm", "rmsnorm")
@@ -27,3 +28,7 @@ class RMSNorm(Norm):
 
     def __call__(self, x, residual=None, rows=None):
         return hip.rmsnorm(x, self.weight, self.eps, residual, rows)
+
+    def defer(self, x, residual=None) -> DeferredNorm:
+        """The same norm as an operand that the next projection may fuse."""
+        return DeferredNorm(x, residual, self.weight, self.eps)
