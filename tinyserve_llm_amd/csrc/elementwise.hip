@@ -13,7 +13,12 @@ __global__ void embedding_kernel(T* __restrict__ out, const T* __restrict__ tabl
   const int t = blockIdx.x;
   const T* src = table + (int64_t)ids[t] * hidden;
   T* dst = out + (int64_t)t * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = src[i];
+  constexpr int V = 16 / sizeof(T);
+  if (hidden % V == 0 && (((uintptr_t)table | (uintptr_t)out) & 15) == 0) {
+    for (int i = threadIdx.x; i < hidden / V; i += blockDim.x) ((uint4*)dst)[i] = ((const uint4*)src)[i];
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = src[i];
+  }
 }
 
 extern "C" int ts_embedding(void* out, const void* table, const int32_t* ids, int num_tokens,
@@ -37,7 +42,37 @@ extern "C" int ts_embedding(void* out, const void* table, const int32_t* ids, in
 // does not depend on what else is in the batch.
 // ------------------------------------------------------------------------------------------
 #define NORM_THREADS 256
+#define NORM_MAX_CHUNKS 4     // 16-byte pieces of a row that a thread of the single-pass kernel keeps
 
+template <typename T> struct Pack16;   // a 16-byte piece of a row as floats
+template <> struct Pack16<float> {
+  static constexpr int N = 4;
+  static __device__ __forceinline__ void ld(const float* p, float* f) {
+    const float4 v = *(const float4*)p;
+    f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+  }
+  static __device__ __forceinline__ void st(float* p, const float* f) { *(float4*)p = make_float4(f[0], f[1], f[2], f[3]); }
+};
+template <> struct Pack16<bf16_t> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void ld(const bf16_t* p, float* f) {
+    const uint4 v = *(const uint4*)p;
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __uint_as_float(w[i] << 16);
+      f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ void st(bf16_t* p, const float* f) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = (uint32_t)f2bf(f[2 * i]) | ((uint32_t)f2bf(f[2 * i + 1]) << 16);
+    *(uint4*)p = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+};
+
+// The general form: two passes over the row, any width, any weight storage.
 template <typename T, typename WT>
 __global__ void rmsnorm_kernel(T* __restrict__ out, T* __restrict__ res_out, const T* __restrict__ x,
                                const T* __restrict__ res, const WT* __restrict__ w,
@@ -71,12 +106,80 @@ __global__ void rmsnorm_kernel(T* __restrict__ out, T* __restrict__ res_out, con
   }
 }
 
+// One pass: a thread keeps its 16-byte pieces of the row in registers between the sum of squares
+// and the scaling. For rows of up to 256 * NORM_MAX_CHUNKS pieces whose width is a whole number of
+// pieces. The order of the sums differs from the general form's but is as fixed per row; which of
+// the two runs depends on the width and the storage types only, never on the batch.
+template <typename T>
+__global__ void __launch_bounds__(NORM_THREADS)
+rmsnorm_row_kernel(T* __restrict__ out, T* __restrict__ res_out, const T* __restrict__ x, const T* __restrict__ res,
+                   const T* __restrict__ w, const int32_t* __restrict__ rows, int hidden, float eps) {
+  constexpr int N = Pack16<T>::N;
+  __shared__ float partial[NORM_THREADS / TS_WAVE];
+  const int r = blockIdx.x;
+  const int64_t src = rows ? (int64_t)rows[r] : (int64_t)r;
+  const T* xr = x + src * hidden;
+  const T* rr = res ? res + src * hidden : nullptr;
+  const int pieces = hidden / N;
+  float v[NORM_MAX_CHUNKS][N];
+  float acc = 0.f;
+#pragma unroll
+  for (int c = 0; c < NORM_MAX_CHUNKS; ++c) {
+    const int i = threadIdx.x + c * NORM_THREADS;
+    if (i < pieces) {
+      Pack16<T>::ld(xr + (int64_t)i * N, v[c]);
+      if (rr) {
+        float t[N];
+        Pack16<T>::ld(rr + (int64_t)i * N, t);
+#pragma unroll
+        for (int k = 0; k < N; ++k) v[c][k] += t[k];
+      }
+#pragma unroll
+      for (int k = 0; k < N; ++k) acc = fmaf(v[c][k], v[c][k], acc);
+    }
+  }
+  acc = wave_sum(acc);
+  if ((threadIdx.x & (TS_WAVE - 1)) == 0) partial[threadIdx.x / TS_WAVE] = acc;
+  __syncthreads();
+  float total = 0.f;
+#pragma unroll
+  for (int i = 0; i < NORM_THREADS / TS_WAVE; ++i) total += partial[i];
+  const float inv = 1.0f / sqrtf(total / (float)hidden + eps);
+  T* orow = out + (int64_t)r * hidden;
+  T* rorow = res_out ? res_out + (int64_t)r * hidden : nullptr;
+#pragma unroll
+  for (int c = 0; c < NORM_MAX_CHUNKS; ++c) {
+    const int i = threadIdx.x + c * NORM_THREADS;
+    if (i < pieces) {
+      if (rorow) Pack16<T>::st(rorow + (int64_t)i * N, v[c]);
+      float wv[N];
+      Pack16<T>::ld(w + (int64_t)i * N, wv);
+#pragma unroll
+      for (int k = 0; k < N; ++k) v[c][k] = Num<T>::round(v[c][k] * inv) * wv[k];
+      Pack16<T>::st(orow + (int64_t)i * N, v[c]);
+    }
+  }
+}
+
 // wdtype: storage of the weight vector (0 float, 1 bfloat16); dtype: storage of activations.
 extern "C" int ts_rmsnorm(void* out, void* res_out, const void* x, const void* res, const void* w,
                           const int32_t* rows, int num_rows, int hidden, float eps, int dtype,
                           int wdtype, hipStream_t stream) {
   if (num_rows <= 0) return TS_OK;
   dim3 grid(num_rows), block(NORM_THREADS);
+  const int per16 = dtype == 0 ? 4 : 8;
+  const bool aligned = ((((uintptr_t)out) | ((uintptr_t)res_out) | ((uintptr_t)x) | ((uintptr_t)res) | ((uintptr_t)w)) & 15) == 0;
+  if (dtype == wdtype && aligned && hidden % per16 == 0 && hidden / per16 <= NORM_THREADS * NORM_MAX_CHUNKS) {
+    if (dtype == 0)
+      rmsnorm_row_kernel<float><<<grid, block, 0, stream>>>((float*)out, (float*)res_out, (const float*)x,
+                                                            (const float*)res, (const float*)w, rows, hidden, eps);
+    else if (dtype == 1)
+      rmsnorm_row_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t*)out, (bf16_t*)res_out, (const bf16_t*)x,
+                                                             (const bf16_t*)res, (const bf16_t*)w, rows, hidden, eps);
+    else
+      return TS_BAD_DTYPE;
+    return ts_check_launch();
+  }
   if (dtype == 0 && wdtype == 0)
     rmsnorm_kernel<float, float><<<grid, block, 0, stream>>>((float*)out, (float*)res_out, (const float*)x,
                                                              (const float*)res, (const float*)w, rows, hidden, eps);
@@ -112,7 +215,7 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
                                   const T* __restrict__ qkv, const float* __restrict__ cos_sin,
                                   const int32_t* __restrict__ positions, const int64_t* __restrict__ slots,
                                   int num_tokens, int nh, int nkv, int hd, int rotate, int page_size, int64_t kp,
-                                  int64_t ks, int64_t kh, int64_t vp, int64_t vs, int64_t vh, int64_t vd) {
+                                  int64_t ks, int64_t kh, int64_t vp, int64_t vs, int64_t vh, int64_t vd, int vec) {
   const int t0 = blockIdx.x * ROPE_TOK;
   const int nt = num_tokens - t0 < ROPE_TOK ? num_tokens - t0 : ROPE_TOK;
   const int half = hd / 2;
@@ -120,6 +223,43 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
   const int qpairs = nh * half, kpairs = nkv * half;
   // q and k pairs of every token of the group: this workgroup's slice of them
   const int npairs = nt * (qpairs + kpairs);
+  constexpr int V = 16 / sizeof(T);
+  if (vec) {
+    // 16 bytes of each half of a head at a time
+    const int per_head = half / V;
+    const int npieces = nt * (nh + nkv) * per_head;
+    const int pbeg = (int)((int64_t)npieces * blockIdx.y / gridDim.y), pend = (int)((int64_t)npieces * (blockIdx.y + 1) / gridDim.y);
+    for (int i = pbeg + threadIdx.x; i < pend; i += blockDim.x) {
+      const int tl = i / ((nh + nkv) * per_head), e = i - tl * ((nh + nkv) * per_head);
+      const int t = t0 + tl;
+      const int h = e / per_head, j = (e - h * per_head) * V;
+      const bool is_k = h >= nh;
+      if (is_k && (!k_cache || slots[t] < 0)) continue;
+      const T* src = qkv + (int64_t)t * row + h * hd;      // k heads follow the q heads in a row
+      float x1[V], x2[V];
+      Pack16<T>::ld(src + j, x1);
+      Pack16<T>::ld(src + j + half, x2);
+      if (rotate) {
+        const float* cs = cos_sin + (int64_t)positions[t] * hd;
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+          const float c = cs[j + k], sn = cs[half + j + k];
+          const float y1 = x1[k] * c - x2[k] * sn, y2 = x2[k] * c + x1[k] * sn;
+          x1[k] = y1;
+          x2[k] = y2;
+        }
+      }
+      T* dst;
+      if (is_k) {
+        const int64_t slot = slots[t];
+        dst = k_cache + (slot / page_size) * kp + (slot % page_size) * ks + (int64_t)(h - nh) * kh;
+      } else {
+        dst = q_out + ((int64_t)t * nh + h) * hd;
+      }
+      Pack16<T>::st(dst + j, x1);
+      Pack16<T>::st(dst + j + half, x2);
+    }
+  } else {
   const int pbeg = (int)((int64_t)npairs * blockIdx.y / gridDim.y), pend = (int)((int64_t)npairs * (blockIdx.y + 1) / gridDim.y);
   for (int i = pbeg + threadIdx.x; i < pend; i += blockDim.x) {
     const int tl = i / (qpairs + kpairs), e = i - tl * (qpairs + kpairs);
@@ -146,6 +286,7 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
     }
     Num<T>::st(dst + j, y1);
     Num<T>::st(dst + j + half, y2);
+  }
   }
   if (!k_cache) return;
   // values: thread -> (element, token), token fastest
@@ -175,14 +316,19 @@ extern "C" int ts_rope_store(void* q_out, void* k_cache, void* v_cache, const vo
   if (slices < 1) slices = 1;
   if (slices > 32) slices = 32;
   const dim3 blocks(groups, slices);
+  // 16-byte pieces need halves of whole pieces and aligned rows everywhere
+  const int per16 = dtype == 0 ? 4 : 8;
+  const int row = (nh + 2 * nkv) * hd;
+  const int vec = (hd / 2) % per16 == 0 && row % per16 == 0 && kp % per16 == 0 && ks % per16 == 0 && kh % per16 == 0 &&
+                  ((((uintptr_t)q_out) | ((uintptr_t)k_cache) | ((uintptr_t)qkv)) & 15) == 0;
   if (dtype == 0)
     rope_store_kernel<float><<<blocks, 256, 0, stream>>>((float*)q_out, (float*)k_cache, (float*)v_cache,
                                                          (const float*)qkv, cos_sin, positions, slots, num_tokens, nh,
-                                                         nkv, hd, rotate, page_size, kp, ks, kh, vp, vs, vh, vd);
+                                                         nkv, hd, rotate, page_size, kp, ks, kh, vp, vs, vh, vd, vec);
   else if (dtype == 1)
     rope_store_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache,
                                                           (const bf16_t*)qkv, cos_sin, positions, slots, num_tokens,
-                                                          nh, nkv, hd, rotate, page_size, kp, ks, kh, vp, vs, vh, vd);
+                                                          nh, nkv, hd, rotate, page_size, kp, ks, kh, vp, vs, vh, vd, vec);
   else
     return TS_BAD_DTYPE;
   return ts_check_launch();
@@ -204,17 +350,45 @@ __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, i
   }
 }
 
+// 16 bytes of gate and of up per thread; for widths that are whole numbers of such pieces
+template <typename T>
+__global__ void silu_mul_vec_kernel(T* __restrict__ out, const T* __restrict__ gu, int64_t pieces, int inter) {
+  constexpr int N = Pack16<T>::N;
+  const int per_row = inter / N;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < pieces;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t t = idx / per_row;
+    const int i = (int)(idx - t * per_row) * N;
+    float g[N], u[N];
+    Pack16<T>::ld(gu + t * 2 * inter + i, g);
+    Pack16<T>::ld(gu + t * 2 * inter + inter + i, u);
+#pragma unroll
+    for (int k = 0; k < N; ++k) g[k] = g[k] / (1.0f + expf(-g[k])) * u[k];
+    Pack16<T>::st(out + t * inter + i, g);
+  }
+}
+
 extern "C" int ts_silu_mul(void* out, const void* gu, int num_tokens, int inter, int dtype, hipStream_t stream) {
   const int64_t total = (int64_t)num_tokens * inter;
   if (total <= 0) return TS_OK;
+  if (dtype != 0 && dtype != 1) return TS_BAD_DTYPE;
+  const int per16 = dtype == 0 ? 4 : 8;
+  if (inter % per16 == 0 && ((((uintptr_t)out) | ((uintptr_t)gu)) & 15) == 0) {
+    const int64_t pieces = total / per16;
+    int64_t blocks = (pieces + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    if (dtype == 0)
+      silu_mul_vec_kernel<float><<<(int)blocks, 256, 0, stream>>>((float*)out, (const float*)gu, pieces, inter);
+    else
+      silu_mul_vec_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, pieces, inter);
+    return ts_check_launch();
+  }
   int64_t blocks = (total + 255) / 256;
   if (blocks > 65536) blocks = 65536;
   if (dtype == 0)
     silu_mul_kernel<float><<<(int)blocks, 256, 0, stream>>>((float*)out, (const float*)gu, total, inter);
-  else if (dtype == 1)
-    silu_mul_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, total, inter);
   else
-    return TS_BAD_DTYPE;
+    silu_mul_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, total, inter);
   return ts_check_launch();
 }
 
