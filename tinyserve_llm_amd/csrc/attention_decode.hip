@@ -148,7 +148,9 @@ attn_decode_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ p
 }
 
 // part_o [tokens, nh, num_splits, hd] and part_ml [tokens, nh, num_splits, 2] are float workspaces.
-// num_splits * chunk must cover every position that `positions` holds. Keys: rows dense in
+// num_splits * chunk must cover every position that `positions` holds. (Letting the last workgroup
+// of a token combine its chunks inside the first kernel was tried and is slower: on a GPU of several
+// dies the device-scope fences it needs write back and invalidate each die's L2.) Keys: rows dense in
 // head_dim, strides kp/ks/kh (page, slot, head). Values: transposed pages, slot stride 1, strides
 // vp/vh/vd (page, head, dimension).
 extern "C" int ts_paged_attention_decode(void* out, float* part_o, float* part_ml, const void* q, const void* k_cache,

@@ -1,4 +1,5 @@
-// Token choice from 32-bit logits, one block per row: the highest logit at temperature 0, else a
+// Token choice from 32-bit logits (64 workgroups share a row, a second kernel picks among their
+// bests): the highest logit at temperature 0, else a
 // draw from softmax(logits / temperature) by the exponential race
 //     argmax_i  softmax_i / E_i   =   argmax_i  logit_i / t - log(E_i),   E_i ~ Exp(1), E_i >= 1e-10
 // (tinyserve_llm/engine/sampler.py:13-23). The noise of element i of a row comes from a counter
@@ -6,7 +7,8 @@
 // draw does not depend on the row's place in the batch. Ties go to the lowest index.
 #include "common.h"
 
-#define SAMPLE_THREADS 1024
+#define SAMPLE_THREADS 256
+#define SAMPLE_SLICES 64       // workgroups that share a row
 
 __device__ __forceinline__ uint64_t mix64(uint64_t x) {
   x ^= x >> 30; x *= 0xBF58476D1CE4E5B9ull;
@@ -24,18 +26,22 @@ __device__ __forceinline__ float exp1_noise(uint64_t seed, uint64_t key, uint32_
 
 __device__ __forceinline__ bool better(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
 
+// Stage 1: workgroup (slice, row) finds the best of its slice of the vocabulary.
 __global__ void __launch_bounds__(SAMPLE_THREADS)
-sample_kernel(int32_t* __restrict__ out, const float* __restrict__ logits, const float* __restrict__ temps,
-              const int64_t* __restrict__ keys, uint64_t seed, int vocab, int64_t ld) {
+sample_slice_kernel(float* __restrict__ best_v, int32_t* __restrict__ best_i, const float* __restrict__ logits,
+                    const float* __restrict__ temps, const int64_t* __restrict__ keys, uint64_t seed, int vocab,
+                    int64_t ld) {
   __shared__ float sv[SAMPLE_THREADS / TS_WAVE];
   __shared__ int si[SAMPLE_THREADS / TS_WAVE];
-  const int r = blockIdx.x;
+  const int r = blockIdx.y, slice = blockIdx.x;
   const float* row = logits + (int64_t)r * ld;
   const float t = temps[r];
   const uint64_t key = (uint64_t)keys[r];
+  const int per = (vocab + SAMPLE_SLICES - 1) / SAMPLE_SLICES;
+  const int beg = slice * per, end = beg + per < vocab ? beg + per : vocab;
   float bv = -INFINITY;
   int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
+  for (int i = beg + threadIdx.x; i < end; i += SAMPLE_THREADS) {
     float v = row[i];
     if (t > 0.f) v = v / t - logf(exp1_noise(seed, key, (uint32_t)i));
     if (better(v, i, bv, bi)) { bv = v; bi = i; }
@@ -51,14 +57,36 @@ sample_kernel(int32_t* __restrict__ out, const float* __restrict__ logits, const
   if (threadIdx.x == 0) {
     for (int w = 1; w < SAMPLE_THREADS / TS_WAVE; ++w)
       if (better(sv[w], si[w], bv, bi)) { bv = sv[w]; bi = si[w]; }
-    out[r] = bi == 0x7fffffff ? 0 : bi;
+    best_v[r * SAMPLE_SLICES + slice] = bv;
+    best_i[r * SAMPLE_SLICES + slice] = bi;
   }
 }
 
-extern "C" int ts_sample(int32_t* out, const float* logits, const float* temps, const int64_t* keys,
-                         uint64_t seed, int rows, int vocab, int64_t ld, hipStream_t stream) {
+// Stage 2: one wave per row picks among the slices' bests.
+__global__ void __launch_bounds__(TS_WAVE)
+sample_pick_kernel(int32_t* __restrict__ out, const float* __restrict__ best_v, const int32_t* __restrict__ best_i) {
+  const int r = blockIdx.x, lane = threadIdx.x;
+  float bv = lane < SAMPLE_SLICES ? best_v[r * SAMPLE_SLICES + lane] : -INFINITY;
+  int bi = lane < SAMPLE_SLICES ? best_i[r * SAMPLE_SLICES + lane] : 0x7fffffff;
+#pragma unroll
+  for (int off = TS_WAVE / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, TS_WAVE);
+    const int oi = __shfl_xor(bi, off, TS_WAVE);
+    if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+  }
+  if (lane == 0) out[r] = bi == 0x7fffffff ? 0 : bi;
+}
+
+// work_v, work_i: [rows, SAMPLE_SLICES] float / int32 workspaces
+extern "C" int ts_sample(int32_t* out, float* work_v, int32_t* work_i, const float* logits, const float* temps,
+                         const int64_t* keys, uint64_t seed, int rows, int vocab, int64_t ld, hipStream_t stream) {
   if (rows <= 0) return TS_OK;
-  if (vocab <= 0 || ld < vocab) return TS_BAD_SHAPE;
-  sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(out, logits, temps, keys, seed, vocab, ld);
+  if (vocab <= 0 || ld < vocab || rows > 65535) return TS_BAD_SHAPE;
+  static_assert(SAMPLE_SLICES <= TS_WAVE, "one wave picks among the slices");
+  sample_slice_kernel<<<dim3(SAMPLE_SLICES, rows), SAMPLE_THREADS, 0, stream>>>(work_v, work_i, logits, temps, keys,
+                                                                              seed, vocab, ld);
+  int rc = ts_check_launch();
+  if (rc) return rc;
+  sample_pick_kernel<<<rows, TS_WAVE, 0, stream>>>(out, work_v, work_i);
   return ts_check_launch();
 }

@@ -51,7 +51,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_paged_attention_decode": [p, p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, i, i, f, i,
                                       p],
         "ts_gemm_exact": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
-        "ts_sample": [p, p, p, p, u64, i, i, i64, p],
+        "ts_sample": [p, p, p, p, p, p, u64, i, i, i64, p],
         "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, p],
         "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, p],
     }
@@ -319,8 +319,11 @@ def sample(logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor,
           "temperatures must be float32 [rows]")
     _need(keys.dtype == torch.int64 and keys.shape == (R,) and keys.is_contiguous(), "keys must be int64 [rows]")
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
-    _run("sample", library().ts_sample(_ptr(out), _ptr(logits), _ptr(temperatures), _ptr(keys),
-                                       seed & 0xFFFFFFFFFFFFFFFF, R, logits.shape[1], logits.stride(0), _stream()))
+    work_v = torch.empty((R, 64), dtype=torch.float32, device=logits.device)
+    work_i = torch.empty((R, 64), dtype=torch.int32, device=logits.device)
+    _run("sample", library().ts_sample(_ptr(out), _ptr(work_v), _ptr(work_i), _ptr(logits), _ptr(temperatures),
+                                       _ptr(keys), seed & 0xFFFFFFFFFFFFFFFF, R, logits.shape[1], logits.stride(0),
+                                       _stream()))
     return out
 
 
