@@ -97,7 +97,7 @@ def test_rope_and_cache_write_on_a_strided_layer_view(dtype):
     g = gen(5)
     qkv = torch.randn(T, (nh + 2 * nkv) * hd, generator=g).to(dtype)
     positions = torch.tensor([30, 31, 32, 33, 0, 1, 2, 7], dtype=torch.int32)
-    slots = torch.tensor([12, 13, 14, 15, 4, 5, 6, -1], dtype=torch.int64)
+    slots = torch.tensor([12, 13, 14, 15, 4, 5, 6, -1], dtype=torch.int32)
     cos, sin = P.rope_tables(hd, 10000.0, None, 64, 64, torch.float64)
     table = torch.cat((cos, sin), -1).float()
     k_pool = torch.zeros(6, 3, page, nkv, hd, dtype=dtype, device=dev())
@@ -228,8 +228,8 @@ def engine_layout(k, v, table, page, pages, dtype):
 
 @pytest.mark.parametrize("heads,kv,hd,page", [(3, 1, 32, 16), (6, 2, 96, 8), (32, 8, 64, 256), (5, 5, 128, 32),
                                               (16, 1, 128, 64), (24, 8, 128, 64), (14, 2, 64, 24)])
-@pytest.mark.parametrize("chunk", [128, 256])
-def test_split_key_decode_attention(heads, kv, hd, page, chunk):
+@pytest.mark.parametrize("chunk,waves", [(128, 4), (256, 4), (256, 8), (640, 5), (1024, 8), (1024, 16)])
+def test_split_key_decode_attention(heads, kv, hd, page, chunk, waves):
     """One query per request at different context lengths (1, a chunk's edge, mid-chunk, long)
     against the dense formula and against the wave kernel on the same pages."""
     dtype = torch.bfloat16
@@ -240,12 +240,17 @@ def test_split_key_decode_attention(heads, kv, hd, page, chunk):
     pages = -(-n // page)
     table = list(range(pages - 1, -1, -1))
     dense = P.causal_attention(q.double(), k.double(), v.double())
-    rows = [0, 1, 31, 32, chunk - 1, chunk, chunk + 1, 255, 256, 257, 400, 599]
+    rows = [min(x, n - 1) for x in (0, 1, 31, 32, chunk - 1, chunk, chunk + 1, 255, 256, 257, 400, 599)]
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev())
     kc, vc = engine_layout(k, v, table, page, pages, dtype)
     assert hip().decode_kernel_takes(q[rows].to(dev()), kc, vc)
+    if waves > 8 or 4 * (32 * waves + waves * (heads // kv) * hd) > 65536:
+        with pytest.raises(hip().KernelError, match="waves"):
+            hip().paged_attention_decode(q[rows].to(dev()), kc, vc, i32([table, table]), i32([0, 1] * 6), i32(rows),
+                                         hd ** -0.5, chunk=chunk, waves=waves)
+        return
     out = hip().paged_attention_decode(q[rows].to(dev()), kc, vc, i32([table, table]), i32([0, 1] * 6), i32(rows),
-                                       hd ** -0.5, chunk=chunk)
+                                       hd ** -0.5, chunk=chunk, waves=waves)
     torch.testing.assert_close(out.double().cpu(), dense[rows], **tol(dtype))
     wave = run_attention(q[rows], kc, vc, [table], [0] * len(rows), rows, hd ** -0.5)
     torch.testing.assert_close(out.float(), wave.float(), **tol(dtype))
@@ -253,9 +258,11 @@ def test_split_key_decode_attention(heads, kv, hd, page, chunk):
 
 @pytest.mark.parametrize("heads,kv,hd,page", [(3, 1, 32, 16), (6, 2, 96, 8), (32, 8, 64, 256), (5, 5, 128, 32),
                                               (16, 1, 128, 64), (14, 2, 64, 24)])
-def test_matrix_core_prefill_attention(heads, kv, hd, page):
+@pytest.mark.parametrize("row_tiles", [1, 2, 4])
+def test_matrix_core_prefill_attention(heads, kv, hd, page, row_tiles):
     """A packed step of three requests on shared pools: a whole prompt, a portion over a cached
-    prefix, and single decoded tokens; tiles never cross a request."""
+    prefix, and single decoded tokens; tiles never cross a request. Once for each number of row
+    tiles that a wave of the kernel may hold."""
     dtype = torch.bfloat16
     g = gen(hd * 3 + page)
     lens = [150, 77, 300]                       # keys each request has after the step
@@ -283,20 +290,21 @@ def test_matrix_core_prefill_attention(heads, kv, hd, page):
     seq_of = sum(([i] * fed[i] for i in range(3)), [])
     positions = sum((list(range(lens[i] - fed[i], lens[i])) for i in range(3)), [])
     cu = [0, fed[0], fed[0] + fed[1], sum(fed)]
-    per_tile = 16 // (heads // kv)
-    flat = hip().attention_tiles(cu, per_tile)
+    per_tile = row_tiles * hip().PREFILL_WAVES * (16 // (heads // kv))
+    flat = hip().attention_tiles(cu, [lens[i] - fed[i] for i in range(3)], per_tile)
     assert all(flat[2 * i + 1] <= per_tile for i in range(len(flat) // 2))
+    assert sum(flat[1::2]) == sum(fed) and len(flat) // 2 == sum(-(-f // per_tile) for f in fed)
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev())
     kc, vc = kp.to(dev()).permute(0, 2, 1, 3), vp.to(dev()).permute(0, 3, 1, 2)
     out = hip().paged_attention_prefill(q_step.to(dev()), kc, vc, i32(padded), i32(seq_of), i32(positions),
-                                        i32(flat).view(-1, 2), hd ** -0.5)
+                                        i32(flat).view(-1, 2), hd ** -0.5, tile_tokens=per_tile)
     want = torch.cat([P.causal_attention(q_all[i].double(), k_all[i].double(), v_all[i].double())[lens[i] - fed[i]:]
                       for i in range(3)])
     torch.testing.assert_close(out.double().cpu(), want, **tol(dtype))
     wave = run_attention(q_step, kc, vc, padded, seq_of, positions, hd ** -0.5)
     torch.testing.assert_close(out.float(), wave.float(), **tol(dtype))
     win = hip().paged_attention_prefill(q_step.to(dev()), kc, vc, i32(padded), i32(seq_of), i32(positions),
-                                        i32(flat).view(-1, 2), hd ** -0.5, window=40)
+                                        i32(flat).view(-1, 2), hd ** -0.5, window=40, tile_tokens=per_tile)
     want = torch.cat([P.causal_attention(q_all[i].double(), k_all[i].double(), v_all[i].double(), window=40)[lens[i] - fed[i]:]
                       for i in range(3)])
     torch.testing.assert_close(win.double().cpu(), want, **tol(dtype))

@@ -35,7 +35,7 @@ def context(lengths, starts, page, tables, encodings=None):
     return StepContext(
         num_tokens=len(pos), num_seqs=len(lengths), token_ids=i32([0] * len(pos)), positions=i32(pos),
         seq_of_token=i32(seq_of), cu_seqlens=i32(cu), context_lens=i32([a + b for a, b in zip(lengths, starts)]),
-        state_slots=i32(list(range(len(lengths)))), slot_mapping=[torch.tensor(slots, dtype=torch.int64, device=DEV)],
+        state_slots=i32(list(range(len(lengths)))), slot_mapping=[torch.tensor(slots, dtype=torch.int32, device=DEV)],
         block_tables=[i32([t + [0] * (width - len(t)) for t in tables])], host_cu_seqlens=cu, host_starts=list(starts),
         host_context_lens=[a + b for a, b in zip(lengths, starts)], host_state_slots=list(range(len(lengths))),
         position_encodings=encodings or {})

@@ -1,0 +1,54 @@
+"""Host-side planning of the attention kernels: pure Python, no GPU."""
+
+import random
+
+from tinyserve_llm_amd.ops import hip
+
+
+def test_attention_tiles_cover_each_token_once_and_never_cross_a_request():
+    rng = random.Random(3)
+    for _ in range(50):
+        lens = [rng.randrange(1, 200) for _ in range(rng.randrange(1, 6))]
+        starts = [rng.randrange(0, 500) for _ in lens]
+        cu = [0]
+        for n in lens:
+            cu.append(cu[-1] + n)
+        per = rng.choice([4, 12, 16, 64])
+        first = rng.randrange(0, len(lens))
+        flat = hip.attention_tiles(cu, starts, per, first)
+        tiles = list(zip(flat[::2], flat[1::2]))
+        seen = []
+        for t0, n in tiles:
+            assert 1 <= n <= per
+            seq = max(s for s in range(len(lens)) if cu[s] <= t0)
+            assert t0 + n <= cu[seq + 1], "a tile stays inside its request"
+            seen.extend(range(t0, t0 + n))
+        assert sorted(seen) == list(range(cu[first], cu[-1]))
+        # ascending in the last position of the tile: the longest walks come last
+        ends = []
+        for t0, n in tiles:
+            seq = max(s for s in range(len(lens)) if cu[s] <= t0)
+            ends.append(starts[seq] + t0 - cu[seq] + n)
+        assert ends == sorted(ends)
+
+
+def test_prefill_tile_tokens_keeps_the_chip_busy():
+    assert hip.prefill_tile_tokens(2048, 8, 4) == 16          # one row tile per wave
+    assert hip.prefill_tile_tokens(8192, 8, 4) == 64          # four
+    assert hip.prefill_tile_tokens(10, 1, 16) == 4
+    for tokens, nkv, group in ((100, 2, 3), (5000, 4, 8), (100000, 8, 1)):
+        per_wave = hip.PREFILL_WAVES * (16 // group)
+        assert hip.prefill_tile_tokens(tokens, nkv, group) in (per_wave, 2 * per_wave, 4 * per_wave)
+
+
+def test_decode_plan_divides_the_context_into_32_key_steps_per_wave():
+    for tokens in (1, 8, 64, 512):
+        for nkv, group, hd in ((8, 4, 64), (1, 16, 128), (2, 3, 96), (5, 1, 32)):
+            for capacity in (8, 64, 256, 300, 2304, 4096, 8192, 131072, 1 << 21):
+                chunk, waves = hip.decode_plan(tokens, nkv, group, hd, capacity)
+                assert 1 <= waves <= hip.MAX_DECODE_WAVES and chunk % (32 * waves) == 0
+                assert -(-capacity // chunk) <= hip.MAX_DECODE_SPLITS
+                assert 4 * (32 * waves + waves * group * hd) <= 65536
+    assert hip.decode_plan(8, 8, 4, 64, 2304) == (128, 4)
+    assert hip.decode_plan(64, 8, 4, 64, 2304) == (2304, 8)
+    assert hip.decode_plan(1, 8, 4, 64, 192) == (192, 6)

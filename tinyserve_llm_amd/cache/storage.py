@@ -67,6 +67,8 @@ class KVStorage:
         pages = num_pages if isinstance(num_pages, (list, tuple)) else [num_pages] * num_spaces
         if len(pages) != num_spaces:
             raise ValueError(f"{num_spaces} page spaces but {len(pages)} page counts")
+        if any(n * page_size >= 2 ** 31 for n in pages):
+            raise ValueError("a page space holds fewer than 2^31 slots (slot numbers travel as int32)")
         windows = [0] * num_spaces
         for kv, s in assigned:
             windows[s] = kv.window

@@ -1,25 +1,25 @@
 // Split-key paged attention on the matrix cores for tokens that each bring one query (decoding),
 // bfloat16. A workgroup takes one (token, key/value head, chunk of keys) and serves all query heads
-// of that key/value head's group; its four waves take a quarter of the chunk each and work through
-// it 32 keys at a time:
-//     S^T[key, head] = K[key, :] · Q[head, :]      v_mfma_f32_16x16x16_bf16, keys as rows
+// of that key/value head's group; its waves (up to 8) take an equal share of the chunk each and work
+// through it 32 keys at a time:
+//     S^T[key, head] = K[key, :] · Q[head, :]      v_mfma_f32_16x16x32_bf16, keys as rows
 //     online softmax per head (32-bit), P = exp(S - max)
 //     O[head, :]    += P[head, key] · V[key, :]
 // The result layout of the first product is the operand layout of the second, so P never leaves
 // its registers. Keys are read as 16-byte pieces of their rows; values are read from pages that
 // hold them transposed ([head_dim, page_size] per head), so that the four consecutive keys an
-// operand needs lie side by side in memory. The waves' partial results meet in LDS; a chunk's
-// unnormalised output with its running max and sum goes to a 32-bit workspace, and a second
-// kernel combines the chunks of a token in ascending order. Chunk boundaries are multiples of
-// the chunk size counted from position 0.
+// operand needs lie side by side in memory. The waves' partial results meet in LDS. With one chunk
+// per token (few tokens, contexts short enough for one workgroup to stream) the workgroup
+// normalises and writes the output itself. Otherwise a chunk's unnormalised output with its running
+// max and sum goes to a 32-bit workspace, and a second kernel combines the chunks of a token in
+// ascending order. Chunk boundaries are multiples of the chunk size counted from position 0.
 #include "attention_mfma.h"
 
-#define DEC_THREADS 256
-#define DEC_WAVES 4
+#define DEC_MAX_WAVES 8
 
 template <int HD>
-__global__ void __launch_bounds__(DEC_THREADS)
-attn_decode_mfma_kernel(float* __restrict__ part_o, float* __restrict__ part_ml, const bf16_t* __restrict__ q,
+__global__ void __launch_bounds__(DEC_MAX_WAVES * TS_WAVE)
+attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, const bf16_t* __restrict__ q,
                         const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
                         const int32_t* __restrict__ block_tables, const int32_t* __restrict__ seq_of_token,
                         const int32_t* __restrict__ positions, int nh, int G, int page_size, int page_shift,
@@ -28,11 +28,12 @@ attn_decode_mfma_kernel(float* __restrict__ part_o, float* __restrict__ part_ml,
   constexpr int NC = HD / 32;    // 32-dimension pieces of a key row (one 16-byte load per lane each)
   constexpr int NDB = HD / 16;   // 16-dimension blocks of the output
   extern __shared__ __align__(16) float smem[];
+  const int nw = blockDim.x / TS_WAVE;
   float* wm = smem;                       // [waves][16]
-  float* wl = wm + DEC_WAVES * 16;        // [waves][16]
-  float* wo = wl + DEC_WAVES * 16;        // [waves][G][HD]
+  float* wl = wm + nw * 16;               // [waves][16]
+  float* wo = wl + nw * 16;               // [waves][G][HD]
 
-  const int tid = threadIdx.x, wave = tid / TS_WAVE, lane = tid & (TS_WAVE - 1);
+  const int tid = threadIdx.x, wave = wave_index(), lane = tid & (TS_WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
   const int split = blockIdx.x, kvh = blockIdx.y, t = blockIdx.z;
   const int pos = positions[t];
@@ -56,13 +57,13 @@ attn_decode_mfma_kernel(float* __restrict__ part_o, float* __restrict__ part_ml,
   for (int db = 0; db < NDB; ++db) o[db] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
   // this wave's keys, 32 at a time; the next step's loads are issued before this step's products
-  const int kpw = chunk / DEC_WAVES;
+  const int kpw = chunk / nw;
   int kb = k0 + wave * kpw;
   int kend = kb + kpw;
   if (kend > pos + 1) kend = pos + 1;
   if (kb < (lo & ~31)) kb = lo & ~31;
 #define TS_LOAD(T, KB) load_tile<HD>(T, KB, r, g, lo, pos, kvh, table, pm, k_cache, v_cache, kp, ks, kh, vp, vh, vd)
-#define TS_USE(T, KB) use_tile<HD>(T, KB, g, lo, pos, qreg, scale2, m, l, o)
+#define TS_USE(T, KB) use_tile_auto<HD>(T, KB, r, g, lo, pos, pos, lo, qreg, scale2, m, l, o)
   if (kb < kend) {
     KVTile<HD> A, B;
     TS_LOAD(A, kb);
@@ -81,7 +82,8 @@ attn_decode_mfma_kernel(float* __restrict__ part_o, float* __restrict__ part_ml,
   }
 #undef TS_LOAD
 #undef TS_USE
-  // ---- the four waves meet
+  // ---- the waves meet
+  l = row_sum(l);
   if (g == 0) { wm[wave * 16 + r] = m; wl[wave * 16 + r] = l; }
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -92,21 +94,23 @@ attn_decode_mfma_kernel(float* __restrict__ part_o, float* __restrict__ part_ml,
     }
   }
   __syncthreads();
-  for (int i = tid; i < G * HD; i += DEC_THREADS) {
+  for (int i = tid; i < G * HD; i += blockDim.x) {
     const int head = i / HD, d = i - head * HD;
     float M = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < DEC_WAVES; ++w) M = fmaxf(M, wm[w * 16 + head]);
+    for (int w = 0; w < nw; ++w) M = fmaxf(M, wm[w * 16 + head]);
     float acc = 0.f, L = 0.f;
-#pragma unroll
-    for (int w = 0; w < DEC_WAVES; ++w) {
-      const float wgt = fast_exp2(wm[w * 16 + head] - M);
+    for (int w = 0; w < nw; ++w) {
+      const float wgt = fast_exp2(wm[w * 16 + head] - M);   // a wave without keys: 2^-inf = 0
       acc = fmaf(wo[((int64_t)w * G + head) * HD + d], wgt, acc);
       L = fmaf(wl[w * 16 + head], wgt, L);
     }
-    const int64_t row = ((int64_t)t * nh + (int64_t)kvh * G + head) * num_splits + split;
-    part_o[row * HD + d] = acc;
-    if (d == 0) { part_ml[row * 2] = M; part_ml[row * 2 + 1] = L; }
+    if (num_splits == 1) {                  // the whole context was this workgroup's: position `pos` is always visible
+      out[((int64_t)t * nh + (int64_t)kvh * G + head) * HD + d] = f2bf(acc / L);
+    } else {
+      const int64_t row = ((int64_t)t * nh + (int64_t)kvh * G + head) * num_splits + split;
+      part_o[row * HD + d] = acc;
+      if (d == 0) { part_ml[row * 2] = M; part_ml[row * 2 + 1] = L; }
+    }
   }
 }
 
@@ -147,8 +151,9 @@ attn_decode_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ p
   }
 }
 
-// part_o [tokens, nh, num_splits, hd] and part_ml [tokens, nh, num_splits, 2] are float workspaces.
-// num_splits * chunk must cover every position that `positions` holds. (Letting the last workgroup
+// part_o [tokens, nh, num_splits, hd] and part_ml [tokens, nh, num_splits, 2] are float workspaces
+// (unused and may be null when num_splits is 1). num_splits * chunk must cover every position that
+// `positions` holds; a workgroup has `waves` waves, each with chunk / waves keys, a multiple of 32. (Letting the last workgroup
 // of a token combine its chunks inside the first kernel was tried and is slower: on a GPU of several
 // dies the device-scope fences it needs write back and invalidate each die's L2.) Keys: rows dense in
 // head_dim, strides kp/ks/kh (page, slot, head). Values: transposed pages, slot stride 1, strides
@@ -158,18 +163,21 @@ extern "C" int ts_paged_attention_decode(void* out, float* part_o, float* part_m
                                          const int32_t* seq_of_token, const int32_t* positions, int num_tokens, int nh,
                                          int nkv, int hd, int page_size, int64_t kp, int64_t ks, int64_t kh,
                                          int64_t vp, int64_t vh, int64_t vd, int max_blocks, int num_splits, int chunk,
-                                         float scale, int window, hipStream_t stream) {
+                                         int waves, float scale, int window, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
   if (nkv <= 0 || nh % nkv || page_size <= 0 || page_size % 8 || max_blocks <= 0 || num_splits <= 0)
     return TS_BAD_SHAPE;
-  if (chunk < 128 || chunk % 128 || num_splits > COMBINE_MAX_SPLITS) return TS_BAD_SHAPE;
+  if (waves < 1 || waves > DEC_MAX_WAVES || chunk <= 0 || chunk % (32 * waves) || num_splits > COMBINE_MAX_SPLITS)
+    return TS_BAD_SHAPE;
+  if (num_splits > 1 && (!part_o || !part_ml)) return TS_BAD_SHAPE;
   if (num_tokens > 65535 || nkv > 65535) return TS_BAD_SHAPE;
   const int G = nh / nkv;
   if (G > 16 || G * hd > 2048) return TS_BAD_SHAPE;
   // 16-byte loads: key rows and the 8-key pieces of value rows must be 16-byte aligned
   if ((kp % 8) || (ks % 8) || (kh % 8) || (vp % 8) || (vh % 8) || (vd % 8)) return TS_BAD_SHAPE;
   if ((((uintptr_t)q) | ((uintptr_t)k_cache) | ((uintptr_t)v_cache)) & 15) return TS_BAD_SHAPE;
-  const size_t smem = sizeof(float) * (2 * DEC_WAVES * 16 + (size_t)DEC_WAVES * G * hd);
+  const size_t smem = sizeof(float) * (2 * waves * 16 + (size_t)waves * G * hd);
+  if (smem > 65536) return TS_BAD_SHAPE;
   int page_shift = -1;
   if ((page_size & (page_size - 1)) == 0) {
     page_shift = 0;
@@ -177,10 +185,10 @@ extern "C" int ts_paged_attention_decode(void* out, float* part_o, float* part_m
   }
   dim3 grid(num_splits, nkv, num_tokens);
 #define TS_DEC(HH)                                                                                              \
-  attn_decode_mfma_kernel<HH><<<grid, DEC_THREADS, smem, stream>>>(                                             \
-      part_o, part_ml, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,          \
-      seq_of_token, positions, nh, G, page_size, page_shift, kp, ks, kh, vp, vh, vd, max_blocks, num_splits,    \
-      chunk, scale * 1.44269504088896340736f, window)
+  attn_decode_mfma_kernel<HH><<<grid, waves * TS_WAVE, smem, stream>>>(                                     \
+      (bf16_t*)out, part_o, part_ml, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,          \
+      block_tables, seq_of_token, positions, nh, G, page_size, page_shift, kp, ks, kh, vp, vh, vd, max_blocks,  \
+      num_splits, chunk, scale * 1.44269504088896340736f, window)
   switch (hd) {
     case 32: TS_DEC(32); break;
     case 64: TS_DEC(64); break;
@@ -190,7 +198,7 @@ extern "C" int ts_paged_attention_decode(void* out, float* part_o, float* part_m
   }
 #undef TS_DEC
   int rc = ts_check_launch();
-  if (rc) return rc;
+  if (rc || num_splits == 1) return rc;
   attn_decode_combine_kernel<<<num_tokens * nh, TS_WAVE, 0, stream>>>((bf16_t*)out, part_o, part_ml, positions, nh, hd,
                                                                       num_splits, chunk, window);
   return ts_check_launch();

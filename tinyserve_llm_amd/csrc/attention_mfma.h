@@ -1,8 +1,12 @@
 // Building blocks of the matrix-core attention kernels (bfloat16): 32 keys at a time,
-//     S^T[key, row] = K[key, :] · Q[row, :]        v_mfma_f32_16x16x16_bf16, keys as rows
-//     online softmax per row (32-bit, in units of log2), P = 2^(S - max)
+//     S^T[key, row] = K[key, :] · Q[row, :]        v_mfma_f32_16x16x32_bf16, keys as rows
+//     online softmax per row (32-bit, in units of log2), P = 2^(S - m)
 //     O[row, :]    += P[row, key] · V[key, :]
 // for a tile of 16 rows, a row being one (token, query head) pair of one key/value head's group.
+// m follows the row's running maximum lazily: it is raised (and the sums rescaled) only when a score
+// exceeds it by more than 2^8, so that most steps need no exchange between lanes; P stays below 2^8,
+// the sums are 32-bit, and a row's m depends on that row's scores alone. Each lane sums the P of its
+// own keys; the four lanes of a row add theirs up once, at the end (`row_sum`).
 // The result layout of the first product is the operand layout of the second, so P never leaves
 // its registers. Keys are read as 16-byte pieces of their rows; values are read from pages that
 // hold them transposed ([head_dim, page_size] per head), so that the consecutive keys an operand
@@ -10,25 +14,19 @@
 #pragma once
 #include "common.h"
 
-typedef short short4_t __attribute__((ext_vector_type(4)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
-static __device__ __forceinline__ short4_t lo_half(const uint4& v) {
-  return __builtin_bit_cast(short4_t, make_uint2(v.x, v.y));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+// acc + A · B over 32 k: lane (r, g) gives eight consecutive k (8 g .. 8 g + 7) of row r of A and of
+// column r of B, 16 bytes each (v_mfma_f32_16x16x32_bf16); lane (r, g) gets D[4 g + j][r], j = 0..3
+static __device__ __forceinline__ float4_t mfma32(const uint4& a, const uint4& b, float4_t acc) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
 }
-static __device__ __forceinline__ short4_t hi_half(const uint4& v) {
-  return __builtin_bit_cast(short4_t, make_uint2(v.z, v.w));
-}
-// probabilities are finite and in [0, 1]: round to nearest even without the NaN case
-static __device__ __forceinline__ short4_t pack_bf16(float a, float b, float c, float d) {
-  const float f[4] = {a, b, c, d};
-  short4_t r;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const uint32_t u = __float_as_uint(f[i]);
-    r[i] = (short)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
-  }
-  return r;
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
+// two floats to a pair of bfloat16, round to nearest even (the hardware's packed conversion)
+static __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector((float2_t){a, b}, bf16x2_t));
 }
 
 // 2^x by the hardware's exponential; scores are kept in units of log2 so that one multiply
@@ -39,13 +37,37 @@ struct PageMath {   // key -> (page index in the table, slot inside the page)
   int size, shift;  // shift >= 0: the page size is 2^shift
   __device__ __forceinline__ int page(int key) const { return shift >= 0 ? key >> shift : key / size; }
   __device__ __forceinline__ int slot(int key, int pg) const { return key - pg * size; }
+  // pages of a multiple of 32 keys: a 32-key step (kb a multiple of 32) lies inside one page, and
+  // its table entry is one scalar lookup for the whole wave
+  __device__ __forceinline__ bool whole_steps() const { return (size & 31) == 0; }
 };
+
+// the wave's index in its workgroup, as a scalar the compiler knows to be uniform
+static __device__ __forceinline__ int wave_index() { return __builtin_amdgcn_readfirstlane(threadIdx.x / TS_WAVE); }
 
 template <int HD> struct KVTile {
   uint4 k[2][HD / 32];   // two 16-key tiles as A operands: row i of tile tau is key kb + 8 (i / 4) + 4 tau + i % 4
   uint4 v[HD / 16];      // transposed values: keys kb + 8 g .. + 7 of dimension 16 db + r
 };
 
+// Exchanges between the four lanes (r, g = 0..3) that share a row, by the register swaps of the
+// hardware: after v_permlane16_swap of x with itself one result holds the even rows of 16 lanes
+// twice and the other the odd rows, after v_permlane32_swap the lower and the upper half.
+static __device__ __forceinline__ float row_max(float x) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+static __device__ __forceinline__ float row_sum(float x) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+// Loads the 32-key step at kb (a multiple of 32) of one request's pages into operand registers;
+// keys outside [lo, pos] read as zeros.
 template <int HD>
 static __device__ __forceinline__ void load_tile(KVTile<HD>& T, int kb, int r, int g, int lo, int pos, int kvh,
                                                  const int32_t* __restrict__ table, const PageMath pm,
@@ -53,6 +75,28 @@ static __device__ __forceinline__ void load_tile(KVTile<HD>& T, int kb, int r, i
                                                  int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vh,
                                                  int64_t vd) {
   constexpr int NC = HD / 32, NDB = HD / 16;
+  if (pm.whole_steps()) {
+    // one page for the whole step: its base addresses are scalars, the lanes add fixed offsets
+    const int pg = pm.page(kb);
+    const int64_t page = table[pg];
+    const int slot = pm.slot(kb, pg);
+    const bf16_t* kbase = k_cache + page * kp + (int64_t)slot * ks + (int64_t)kvh * kh;
+    const bf16_t* vbase = v_cache + page * vp + slot + (int64_t)kvh * vh;
+    const bool inner = kb >= lo && kb + 31 <= pos;
+#pragma unroll
+    for (int tau = 0; tau < 2; ++tau) {
+      const int koff = 8 * (r >> 2) + 4 * tau + (r & 3);
+      const bf16_t* kr = kbase + (int64_t)koff * ks + 8 * g;
+      const bool ok = inner || (kb + koff <= pos && kb + koff >= lo);
+#pragma unroll
+      for (int c = 0; c < NC; ++c) T.k[tau][c] = ok ? *(const uint4*)(kr + 32 * c) : make_uint4(0, 0, 0, 0);
+    }
+    const bf16_t* vr = vbase + 8 * g + (int64_t)r * vd;
+    const bool vok = inner || (kb + 8 * g <= pos && kb + 8 * g + 7 >= lo);
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) T.v[db] = vok ? *(const uint4*)(vr + (int64_t)(16 * db) * vd) : make_uint4(0, 0, 0, 0);
+    return;
+  }
 #pragma unroll
   for (int tau = 0; tau < 2; ++tau) {
     const int key = kb + 8 * (r >> 2) + 4 * tau + (r & 3);
@@ -65,7 +109,7 @@ static __device__ __forceinline__ void load_tile(KVTile<HD>& T, int kb, int r, i
       for (int c = 0; c < NC; ++c) T.k[tau][c] = *(const uint4*)(kr + 32 * c);
     }
   }
-  const int vkey = kb + 8 * g;
+  const int vkey = kb + 8 * g;      // page sizes are multiples of 8: the 8 keys share a page
 #pragma unroll
   for (int db = 0; db < NDB; ++db) T.v[db] = make_uint4(0, 0, 0, 0);
   if (vkey <= pos && vkey + 7 >= lo) {
@@ -76,10 +120,15 @@ static __device__ __forceinline__ void load_tile(KVTile<HD>& T, int kb, int r, i
   }
 }
 
+#define TS_LAZY_MAX 8.0f     // a row's reference maximum is raised when a score exceeds it by more than this (log2 units)
+
 // One 32-key step of the online softmax for the 16 rows that `qreg` holds (lane r = row r of the
-// score tile; output row 4 g + j). `m` is the running max in units of log2, `l` the running sum.
-template <int HD>
-static __device__ __forceinline__ void use_tile(const KVTile<HD>& T, int kb, int g, int lo, int pos,
+// score tile; output row 4 g + j). `m` is the row's reference maximum in units of log2 (the same in
+// the row's four lanes), `l` this lane's share of the row's sum. scale2 > 0.
+// MASKED: rows mask the keys beyond their position and before their window; without it every key
+// of the step is visible to every row (the caller has checked).
+template <int HD, bool MASKED>
+static __device__ __forceinline__ void use_tile(const KVTile<HD>& T, int kb, int r, int g, int lo, int pos,
                                                 const uint4 (&qreg)[HD / 32], float scale2, float& m, float& l,
                                                 float4_t (&o)[HD / 16]) {
   constexpr int NC = HD / 32, NDB = HD / 16;
@@ -88,53 +137,60 @@ static __device__ __forceinline__ void use_tile(const KVTile<HD>& T, int kb, int
   for (int tau = 0; tau < 2; ++tau) {
     s[tau] = (float4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int c = 0; c < NC; ++c) {
-      s[tau] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(lo_half(T.k[tau][c]), lo_half(qreg[c]), s[tau], 0, 0, 0);
-      s[tau] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(hi_half(T.k[tau][c]), hi_half(qreg[c]), s[tau], 0, 0, 0);
-    }
+    for (int c = 0; c < NC; ++c) s[tau] = mfma32(T.k[tau][c], qreg[c], s[tau]);
   }
   // this lane: row r, keys kb + 8 g + 4 tau + j
-  float sv[2][4];
   float mloc = -INFINITY;
 #pragma unroll
   for (int tau = 0; tau < 2; ++tau)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int key = kb + 8 * g + 4 * tau + j;
-      sv[tau][j] = (key <= pos && key >= lo) ? s[tau][j] * scale2 : -INFINITY;
-      mloc = fmaxf(mloc, sv[tau][j]);
+      if (MASKED) {
+        const int key = kb + 8 * g + 4 * tau + j;
+        if (!(key <= pos && key >= lo)) s[tau][j] = -INFINITY;
+      }
+      mloc = fmaxf(mloc, s[tau][j]);
     }
-  mloc = fmaxf(mloc, __shfl_xor(mloc, 16, TS_WAVE));
-  mloc = fmaxf(mloc, __shfl_xor(mloc, 32, TS_WAVE));
-  const float m_new = fmaxf(m, mloc);
-  const float m_safe = m_new == -INFINITY ? 0.f : m_new;   // nothing visible yet: every term below is 0
-  const float alpha = fast_exp2(m - m_safe);
+  mloc *= scale2;
+  const uint64_t hit = __builtin_amdgcn_ballot_w64(mloc > m + TS_LAZY_MAX);
+  if (hit) {
+    // some row's scores have outgrown its reference: those rows move it to their maximum so far
+    const float mrow = row_max(mloc);
+    const bool mine = ((hit >> r) & 0x0001000100010001ull) != 0;   // a lane of this lane's row
+    const float m_new = mine ? fmaxf(m, mrow) : m;                 // finite where it changes
+    const float alpha = m_new == m ? 1.0f : fast_exp2(m - m_new);
+    l *= alpha;
+    // output row 4 g + j belongs to score row 4 g + j, whose alpha lane 4 g + j holds
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float aj = __shfl(alpha, 4 * g + j, TS_WAVE);
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) o[db][j] *= aj;
+    }
+    m = m_new;
+  }
+  const float neg_m = (MASKED && m == -INFINITY) ? 0.f : -m;   // nothing visible yet: every term below is 0
   float p[2][4];
-  float lsum = 0.f;
 #pragma unroll
   for (int tau = 0; tau < 2; ++tau)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      p[tau][j] = fast_exp2(sv[tau][j] - m_safe);
-      lsum += p[tau][j];
+      p[tau][j] = fast_exp2(fmaf(s[tau][j], scale2, neg_m));
+      l += p[tau][j];
     }
-  lsum += __shfl_xor(lsum, 16, TS_WAVE);
-  lsum += __shfl_xor(lsum, 32, TS_WAVE);
-  l = l * alpha + lsum;
-  m = m_new;
-  // output row 4 g + j belongs to score row 4 g + j, whose alpha lane 4 g + j holds
+  // this lane's eight keys kb + 8 g .. + 7, in the order the value registers hold them
+  const uint4 pa = make_uint4(pack_bf16(p[0][0], p[0][1]), pack_bf16(p[0][2], p[0][3]), pack_bf16(p[1][0], p[1][1]),
+                              pack_bf16(p[1][2], p[1][3]));
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const float aj = __shfl(alpha, 4 * g + j, TS_WAVE);
-#pragma unroll
-    for (int db = 0; db < NDB; ++db) o[db][j] *= aj;
-  }
-  const short4_t pa0 = pack_bf16(p[0][0], p[0][1], p[0][2], p[0][3]);
-  const short4_t pa1 = pack_bf16(p[1][0], p[1][1], p[1][2], p[1][3]);
-#pragma unroll
-  for (int db = 0; db < NDB; ++db) {
-    o[db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pa0, lo_half(T.v[db]), o[db], 0, 0, 0);
-    o[db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pa1, hi_half(T.v[db]), o[db], 0, 0, 0);
-  }
+  for (int db = 0; db < NDB; ++db) o[db] = mfma32(pa, T.v[db], o[db]);
 }
 
+// The same, choosing the variant: `pmin` and `lomax` are the smallest position and the largest
+// window start among the wave's rows (wave-uniform).
+template <int HD>
+static __device__ __forceinline__ void use_tile_auto(const KVTile<HD>& T, int kb, int r, int g, int lo, int pos,
+                                                     int pmin, int lomax, const uint4 (&qreg)[HD / 32], float scale2,
+                                                     float& m, float& l, float4_t (&o)[HD / 16]) {
+  if (kb + 31 <= pmin && kb >= lomax) use_tile<HD, false>(T, kb, r, g, lo, pos, qreg, scale2, m, l, o);
+  else use_tile<HD, true>(T, kb, r, g, lo, pos, qreg, scale2, m, l, o);
+}

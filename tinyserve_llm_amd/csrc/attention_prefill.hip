@@ -1,18 +1,211 @@
-// Paged attention on the matrix cores for steps that bring portions of prompts (and whatever
-// decoded tokens ride along), bfloat16. The step's (token, query head) pairs of one key/value head
-// are cut into tiles of 16 rows: 16 / G consecutive tokens of one request with the G heads of the
-// group. A wave owns a tile and walks the request's keys from the first position any of its rows
-// may see to the last, 32 keys at a time, with the next step's loads in flight; every row masks
-// the keys beyond its own position (and before its window). Nothing is split and nothing is
-// combined: a row's sums run over the keys in ascending order, whatever the batch.
+// Paged attention on the matrix cores for steps that bring portions of prompts, bfloat16. The
+// step's (token, query head) pairs of one key/value head are cut into tiles of 16 rows: 16 / G
+// consecutive tokens of one request with the G heads of the group. A workgroup of four waves takes
+// up to 4 RT such tiles of consecutive tokens (RT per wave) and walks the request's keys from the
+// first position any of its rows may see to the last, 32 keys at a time. Each step's keys and
+// values are fetched from the pages once per workgroup: every wave loads a quarter of the operand
+// registers, leaves them in LDS in the order the lanes use them, and all four waves read the whole
+// step back from there, two steps ahead of the loads in flight. A row masks the keys beyond its own
+// position (and before its window); steps that lie wholly inside every row's range skip the masks.
+// Nothing is split and nothing is combined: a row's sums run over the keys in ascending order,
+// whatever the batch.
 //
 // The host lists the tiles: tiles[2 i] = index of the tile's first token in the step,
-// tiles[2 i + 1] = number of its tokens (at most 16 / G, all of one request).
+// tiles[2 i + 1] = number of its tokens (at most 4 RT (16 / G), all of one request), in ascending
+// order of the number of keys a tile walks. Workgroup b takes tile n - 1 - b and then tile b, a long
+// one and a short one, so that all workgroups have about the same work.
 #include "attention_mfma.h"
 
 #define PRE_WAVES 4
 
 template <int HD>
+struct PrefillLds {
+  uint4 stage[2][HD / 8][TS_WAVE];   // two steps of operand registers, [register][lane]
+  int range[2][PRE_WAVES];
+};
+
+template <int HD, int RT>
+static __device__ __forceinline__ void
+prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
+             const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+             const int32_t* __restrict__ block_tables, const int32_t* __restrict__ seq_of_token,
+             const int32_t* __restrict__ positions, const int32_t* __restrict__ tiles, int nh, int G, int page_size,
+             int page_shift, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
+             float scale2, int window) {
+  constexpr int NC = HD / 32, NDB = HD / 16;   // operand registers of a 32-key step: 2 NC of K, NDB of V
+  auto& stage = lds.stage;
+  auto& wg_range = lds.range;
+  const int wave = wave_index(), lane = threadIdx.x & (TS_WAVE - 1);
+  const int r = lane & 15, g = lane >> 4;
+  const int t0 = tiles[2 * tile], ntok = tiles[2 * tile + 1];
+  const int32_t* table = block_tables + (int64_t)seq_of_token[t0] * max_blocks;
+  const PageMath pm{page_size, page_shift};
+  const int tpt = 16 / G;                                   // tokens per row tile
+
+  // lane r carries row r of each of its wave's score tiles: token tk[j], head r % G of the group
+  const int hh = r % G;
+  int pos[RT], lo[RT], tk[RT];
+  int pmax = -1, lmin = 0x7fffffff;
+#pragma unroll
+  for (int j = 0; j < RT; ++j) {
+    tk[j] = (wave * RT + j) * tpt + r / G;
+    const bool ok = r / G < tpt && tk[j] < ntok;
+    pos[j] = ok ? positions[t0 + tk[j]] : -1;               // -1: no key is visible, the row stays empty
+    lo[j] = (window > 0 && pos[j] - window + 1 > 0) ? pos[j] - window + 1 : 0;
+    if (!ok) tk[j] = -1;
+    pmax = max(pmax, pos[j]);
+    lmin = min(lmin, ok ? lo[j] : 0x7fffffff);
+  }
+  // per row tile: the smallest position and largest window start of its rows (wave-uniform)
+  int tile_pmin[RT], tile_lomax[RT], tile_pmax[RT], tile_lomin[RT];
+#pragma unroll
+  for (int j = 0; j < RT; ++j) {
+    tile_pmin[j] = pos[j]; tile_lomax[j] = lo[j]; tile_pmax[j] = pos[j];
+    tile_lomin[j] = tk[j] >= 0 ? lo[j] : 0x7fffffff;
+  }
+#pragma unroll
+  for (int off = 1; off < TS_WAVE; off <<= 1) {
+    pmax = max(pmax, __shfl_xor(pmax, off, TS_WAVE));
+    lmin = min(lmin, __shfl_xor(lmin, off, TS_WAVE));
+#pragma unroll
+    for (int j = 0; j < RT; ++j) {
+      tile_pmin[j] = min(tile_pmin[j], __shfl_xor(tile_pmin[j], off, TS_WAVE));
+      tile_pmax[j] = max(tile_pmax[j], __shfl_xor(tile_pmax[j], off, TS_WAVE));
+      tile_lomax[j] = max(tile_lomax[j], __shfl_xor(tile_lomax[j], off, TS_WAVE));
+      tile_lomin[j] = min(tile_lomin[j], __shfl_xor(tile_lomin[j], off, TS_WAVE));
+    }
+  }
+  // the workgroup's key range
+  if (lane == 0) { wg_range[0][wave] = lmin; wg_range[1][wave] = pmax; }
+  __syncthreads();
+  int wlo = wg_range[0][0], whi = wg_range[1][0];
+#pragma unroll
+  for (int w = 1; w < PRE_WAVES; ++w) { wlo = min(wlo, wg_range[0][w]); whi = max(whi, wg_range[1][w]); }
+  // every lane holds the same values: say so, and loop control and page lookups become scalar
+  wlo = __builtin_amdgcn_readfirstlane(wlo);
+  whi = __builtin_amdgcn_readfirstlane(whi);
+#pragma unroll
+  for (int j = 0; j < RT; ++j) {
+    tile_pmin[j] = __builtin_amdgcn_readfirstlane(tile_pmin[j]);
+    tile_pmax[j] = __builtin_amdgcn_readfirstlane(tile_pmax[j]);
+    tile_lomax[j] = __builtin_amdgcn_readfirstlane(tile_lomax[j]);
+    tile_lomin[j] = __builtin_amdgcn_readfirstlane(tile_lomin[j]);
+  }
+
+  uint4 qreg[RT][NC];
+  float m[RT], l[RT];
+  float4_t o[RT][NDB];
+#pragma unroll
+  for (int j = 0; j < RT; ++j) {
+    m[j] = -INFINITY; l[j] = 0.f;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) qreg[j][c] = make_uint4(0, 0, 0, 0);
+    if (tk[j] >= 0) {
+      const bf16_t* qrow = q + ((int64_t)(t0 + tk[j]) * nh + (int64_t)kvh * G + hh) * HD + 8 * g;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) qreg[j][c] = *(const uint4*)(qrow + 32 * c);
+    }
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) o[j][db] = (float4_t){0.f, 0.f, 0.f, 0.f};
+  }
+
+  // This wave's quarter of a step's operand registers: waves 0 and 1 the two 16-key tiles of K
+  // (NC registers each), waves 2 and 3 half of the NDB registers of V each (NDB = 2 NC).
+  uint4 fetched[NC];
+  const bool whole = pm.whole_steps();
+  auto fetch = [&](int kb) {
+    if (whole) {
+      // one page for the whole step: its base addresses are scalars, the lanes add fixed offsets
+      const int pg = pm.page(kb);
+      const int64_t page = table[pg];
+      const int slot = pm.slot(kb, pg);
+      const bool inner = kb >= wlo && kb + 31 <= whi;
+      if (wave < 2) {
+        const int koff = 8 * (r >> 2) + 4 * wave + (r & 3);
+        const bf16_t* kr = k_cache + page * kp + (int64_t)slot * ks + (int64_t)kvh * kh + (int64_t)koff * ks + 8 * g;
+        const bool ok = inner || (kb + koff <= whi && kb + koff >= wlo);
+#pragma unroll
+        for (int c = 0; c < NC; ++c) fetched[c] = ok ? *(const uint4*)(kr + 32 * c) : make_uint4(0, 0, 0, 0);
+      } else {
+        const bf16_t* vr = v_cache + page * vp + slot + (int64_t)kvh * vh + 8 * g +
+                           (int64_t)((wave - 2) * NC * 16 + r) * vd;
+        const bool ok = inner || (kb + 8 * g <= whi && kb + 8 * g + 7 >= wlo);
+#pragma unroll
+        for (int c = 0; c < NC; ++c) fetched[c] = ok ? *(const uint4*)(vr + (int64_t)(16 * c) * vd) : make_uint4(0, 0, 0, 0);
+      }
+      return;
+    }
+#pragma unroll
+    for (int c = 0; c < NC; ++c) fetched[c] = make_uint4(0, 0, 0, 0);
+    if (wave < 2) {
+      const int key = kb + 8 * (r >> 2) + 4 * wave + (r & 3);
+      if (key <= whi && key >= wlo) {
+        const int pg = pm.page(key);
+        const bf16_t* kr = k_cache + (int64_t)table[pg] * kp + (int64_t)pm.slot(key, pg) * ks + (int64_t)kvh * kh + 8 * g;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) fetched[c] = *(const uint4*)(kr + 32 * c);
+      }
+    } else {
+      const int vkey = kb + 8 * g;
+      if (vkey <= whi && vkey + 7 >= wlo) {
+        const int pg = pm.page(vkey);
+        const bf16_t* vr = v_cache + (int64_t)table[pg] * vp + pm.slot(vkey, pg) + (int64_t)kvh * vh +
+                           (int64_t)((wave - 2) * NC * 16 + r) * vd;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) fetched[c] = *(const uint4*)(vr + (int64_t)(16 * c) * vd);
+      }
+    }
+  };
+  auto put = [&](int buf) {
+#pragma unroll
+    for (int c = 0; c < NC; ++c) stage[buf][wave * NC + c][lane] = fetched[c];
+  };
+
+  const int kbeg = wlo & ~31;
+  const int kend = whi + 1;
+  if (kbeg < kend) {                         // uniform over the workgroup
+    fetch(kbeg);
+    put(0);
+    if (kbeg + 32 < kend) fetch(kbeg + 32);
+    __syncthreads();
+    int buf = 0;
+    for (int kb = kbeg; kb < kend; kb += 32, buf ^= 1) {
+      KVTile<HD> T;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) { T.k[0][c] = stage[buf][c][lane]; T.k[1][c] = stage[buf][NC + c][lane]; }
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) T.v[db] = stage[buf][2 * NC + db][lane];
+      if (kb + 32 < kend) put(buf ^ 1);      // the other buffer was last read before the previous barrier
+      if (kb + 64 < kend) fetch(kb + 64);
+#pragma unroll
+      for (int j = 0; j < RT; ++j)
+        // a step wholly beyond the tile's last position, or wholly before all its windows, has nothing for it
+        if (kb <= tile_pmax[j] && kb + 31 >= tile_lomin[j])
+          use_tile_auto<HD>(T, kb, r, g, lo[j], pos[j], tile_pmin[j], tile_lomax[j], qreg[j], scale2, m[j], l[j], o[j]);
+      __syncthreads();
+    }
+  }
+  // output row 4 g + i of row tile j: its token and head; its sum sits in lane 4 g + i
+  float lsum[RT];
+#pragma unroll
+  for (int j = 0; j < RT; ++j) lsum[j] = row_sum(l[j]);
+#pragma unroll
+  for (int j = 0; j < RT; ++j)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 4 * g + i;
+      const float lj = __shfl(lsum[j], row, TS_WAVE);
+      const int rtk = (wave * RT + j) * tpt + row / G, rhh = row % G;
+      if (row / G < tpt && rtk < ntok && lj > 0.f) {
+        const float inv = 1.0f / lj;
+        bf16_t* orow = out + ((int64_t)(t0 + rtk) * nh + (int64_t)kvh * G + rhh) * HD;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) orow[16 * db + r] = f2bf(o[j][db][i] * inv);
+      }
+    }
+}
+
+template <int HD, int RT>
 __global__ void __launch_bounds__(PRE_WAVES * TS_WAVE)
 attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
                          const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables,
@@ -20,92 +213,36 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
                          const int32_t* __restrict__ tiles, int num_tiles, int nh, int G, int page_size,
                          int page_shift, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd,
                          int max_blocks, float scale2, int window) {
-  constexpr int NC = HD / 32, NDB = HD / 16;
-  const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
-  const int r = lane & 15, g = lane >> 4;
-  // the longest tiles (the last tokens of long prompts) are listed last: hand them out first
-  const int tile = num_tiles - 1 - (blockIdx.x * PRE_WAVES + wave);
-  const int kvh = blockIdx.y;
-  if (tile < 0) return;                      // whole wave; no workgroup barrier below
-  const int t0 = tiles[2 * tile], ntok = tiles[2 * tile + 1];
-  const int32_t* table = block_tables + (int64_t)seq_of_token[t0] * max_blocks;
-  const PageMath pm{page_size, page_shift};
-
-  // lane r carries row r of the score tile: token t0 + r / G, head r % G of the group
-  const int tk = r / G, hh = r - tk * G;
-  const bool row_ok = tk < ntok;
-  const int pos = row_ok ? positions[t0 + tk] : -1;          // -1: no key is visible, the row stays empty
-  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  // the tile's key range
-  int pmax = pos, lmin = row_ok ? lo : 0x7fffffff;
-#pragma unroll
-  for (int off = 1; off < TS_WAVE; off <<= 1) {
-    pmax = max(pmax, __shfl_xor(pmax, off, TS_WAVE));
-    lmin = min(lmin, __shfl_xor(lmin, off, TS_WAVE));
+  __shared__ PrefillLds<HD> lds;
+  const int b = blockIdx.x, kvh = blockIdx.y;
+  const int far = num_tiles - 1 - b;             // b <= far by the size of the grid
+#define TS_TILE(I)                                                                                              \
+  prefill_tile<HD, RT>(lds, I, kvh, out, q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, nh, \
+                       G, page_size, page_shift, kp, ks, kh, vp, vh, vd, max_blocks, scale2, window)
+  TS_TILE(far);
+  if (b < far) {
+    __syncthreads();                             // the first tile's last reads of LDS are done
+    TS_TILE(b);
   }
-
-  uint4 qreg[NC];
-#pragma unroll
-  for (int c = 0; c < NC; ++c) qreg[c] = make_uint4(0, 0, 0, 0);
-  if (row_ok) {
-    const bf16_t* qrow = q + ((int64_t)(t0 + tk) * nh + (int64_t)kvh * G + hh) * HD + 8 * g;
-#pragma unroll
-    for (int c = 0; c < NC; ++c) qreg[c] = *(const uint4*)(qrow + 32 * c);
-  }
-  float m = -INFINITY, l = 0.f;
-  float4_t o[NDB];
-#pragma unroll
-  for (int db = 0; db < NDB; ++db) o[db] = (float4_t){0.f, 0.f, 0.f, 0.f};
-
-  int kb = lmin & ~31;
-  const int kend = pmax + 1;
-#define TS_LOAD(T, KB) load_tile<HD>(T, KB, r, g, lmin, pmax, kvh, table, pm, k_cache, v_cache, kp, ks, kh, vp, vh, vd)
-#define TS_USE(T, KB) use_tile<HD>(T, KB, g, lo, pos, qreg, scale2, m, l, o)
-  if (kb < kend) {
-    KVTile<HD> A, B;
-    TS_LOAD(A, kb);
-    while (true) {
-      const bool more_b = kb + 32 < kend;
-      if (more_b) TS_LOAD(B, kb + 32);
-      TS_USE(A, kb);
-      if (!more_b) break;
-      kb += 32;
-      const bool more_a = kb + 32 < kend;
-      if (more_a) TS_LOAD(A, kb + 32);
-      TS_USE(B, kb);
-      if (!more_a) break;
-      kb += 32;
-    }
-  }
-#undef TS_LOAD
-#undef TS_USE
-  // output row 4 g + j: token t0 + (4 g + j) / G, head (4 g + j) % G; its sum sits in lane 4 g + j
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int row = 4 * g + j;
-    const float lj = __shfl(l, row, TS_WAVE);
-    const int rtk = row / G, rhh = row - rtk * G;
-    if (rtk < ntok && lj > 0.f) {
-      const float inv = 1.0f / lj;
-      bf16_t* orow = out + ((int64_t)(t0 + rtk) * nh + (int64_t)kvh * G + rhh) * HD;
-#pragma unroll
-      for (int db = 0; db < NDB; ++db) orow[16 * db + r] = f2bf(o[db][j] * inv);
-    }
-  }
+#undef TS_TILE
 }
 
 // Keys: rows dense in head_dim, strides kp/ks/kh (page, slot, head). Values: transposed pages,
-// slot stride 1, strides vp/vh/vd (page, head, dimension).
+// slot stride 1, strides vp/vh/vd (page, head, dimension). tile_tokens: the most tokens a listed
+// tile holds, 4 RT (16 / G) for RT of 1, 2 or 4.
 extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* k_cache, const void* v_cache,
                                           const int32_t* block_tables, const int32_t* seq_of_token,
-                                          const int32_t* positions, const int32_t* tiles, int num_tiles, int nh,
-                                          int nkv, int hd, int page_size, int64_t kp, int64_t ks, int64_t kh,
-                                          int64_t vp, int64_t vh, int64_t vd, int max_blocks, float scale, int window,
-                                          hipStream_t stream) {
+                                          const int32_t* positions, const int32_t* tiles, int num_tiles,
+                                          int tile_tokens, int nh, int nkv, int hd, int page_size, int64_t kp,
+                                          int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
+                                          float scale, int window, hipStream_t stream) {
   if (num_tiles <= 0) return TS_OK;
   if (nkv <= 0 || nh % nkv || page_size <= 0 || page_size % 8 || max_blocks <= 0) return TS_BAD_SHAPE;
   const int G = nh / nkv;
   if (G > 16 || nkv > 65535) return TS_BAD_SHAPE;
+  const int per_wave = PRE_WAVES * (16 / G);
+  if (tile_tokens != per_wave && tile_tokens != 2 * per_wave && tile_tokens != 4 * per_wave) return TS_BAD_SHAPE;
+  const int rt = tile_tokens / per_wave;
   if ((kp % 8) || (ks % 8) || (kh % 8) || (vp % 8) || (vh % 8) || (vd % 8)) return TS_BAD_SHAPE;
   if ((((uintptr_t)q) | ((uintptr_t)k_cache) | ((uintptr_t)v_cache)) & 15) return TS_BAD_SHAPE;
   int page_shift = -1;
@@ -113,19 +250,22 @@ extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* 
     page_shift = 0;
     while ((1 << page_shift) < page_size) ++page_shift;
   }
-  dim3 grid((num_tiles + PRE_WAVES - 1) / PRE_WAVES, nkv);
-#define TS_PRE(HH)                                                                                              \
-  attn_prefill_mfma_kernel<HH><<<grid, PRE_WAVES * TS_WAVE, 0, stream>>>(                                       \
+  dim3 grid((num_tiles + 1) / 2, nkv);
+#define TS_PRE(HH, RR)                                                                                          \
+  attn_prefill_mfma_kernel<HH, RR><<<grid, PRE_WAVES * TS_WAVE, 0, stream>>>(                                   \
       (bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,             \
       seq_of_token, positions, tiles, num_tiles, nh, G, page_size, page_shift, kp, ks, kh, vp, vh, vd,          \
       max_blocks, scale * 1.44269504088896340736f, window)
+#define TS_PRE_RT(HH)                                                                                           \
+  if (rt == 1) TS_PRE(HH, 1); else if (rt == 2) TS_PRE(HH, 2); else TS_PRE(HH, 4)
   switch (hd) {
-    case 32: TS_PRE(32); break;
-    case 64: TS_PRE(64); break;
-    case 96: TS_PRE(96); break;
-    case 128: TS_PRE(128); break;
+    case 32: TS_PRE_RT(32); break;
+    case 64: TS_PRE_RT(64); break;
+    case 96: TS_PRE_RT(96); break;
+    case 128: TS_PRE_RT(128); break;
     default: return TS_BAD_SHAPE;
   }
+#undef TS_PRE_RT
 #undef TS_PRE
   return ts_check_launch();
 }

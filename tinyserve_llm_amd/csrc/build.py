@@ -25,6 +25,9 @@ FLAGS = [
     "-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17",
     # packed 32-bit float instructions are switched off for all device code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # matrix-core results stay in ordinary vector registers: the softmax and the epilogues work on
+    # them with vector instructions, and copies to and from the accumulation registers cost more
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-Wno-unused-command-line-argument", "-Wno-unknown-attributes",
 ]
 

@@ -213,7 +213,7 @@ extern "C" int ts_rmsnorm(void* out, void* res_out, const void* x, const void* r
 template <typename T>
 __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
                                   const T* __restrict__ qkv, const float* __restrict__ cos_sin,
-                                  const int32_t* __restrict__ positions, const int64_t* __restrict__ slots,
+                                  const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
                                   int num_tokens, int nh, int nkv, int hd, int rotate, int page_size, int64_t kp,
                                   int64_t ks, int64_t kh, int64_t vp, int64_t vs, int64_t vh, int64_t vd, int vec) {
   const int t0 = blockIdx.x * ROPE_TOK;
@@ -306,7 +306,7 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
 }
 
 extern "C" int ts_rope_store(void* q_out, void* k_cache, void* v_cache, const void* qkv, const float* cos_sin,
-                             const int32_t* positions, const int64_t* slots, int num_tokens, int nh, int nkv,
+                             const int32_t* positions, const int32_t* slots, int num_tokens, int nh, int nkv,
                              int hd, int rotate, int page_size, int64_t kp, int64_t ks, int64_t kh, int64_t vp,
                              int64_t vs, int64_t vh, int64_t vd, int dtype, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;

@@ -2,7 +2,7 @@
 // time goes to reading W once from HBM. A workgroup owns 16 to 64 rows of W over the whole of K;
 // each of its waves takes a slice of K of 256 or 512 and issues every load of its slice of W before
 // it uses the first, so that a cold matrix streams at memory speed; the rows go straight from the
-// 16-byte loads into MFMA operands (v_mfma_f32_16x16x16_bf16: W rows are the A matrix, x^T the B
+// 16-byte loads into MFMA operands (v_mfma_f32_16x16x32_bf16: W rows are the A matrix, x^T the B
 // matrix), and the waves' partial tiles are summed in LDS in a fixed order. Accumulation is 32-bit;
 // the result is rounded once.
 //
@@ -14,15 +14,17 @@
 //              silu(gate) * up, y being [M, N / 2]
 #include "common.h"
 
-typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
-#define SK_KSTEP 32      // k covered by one pair of MFMAs: lane group g holds k = 8 g .. 8 g + 7
+#define SK_KSTEP 32      // k covered by one MFMA: lane group g holds k = 8 g .. 8 g + 7
 #define MODE_PLAIN 0
 #define MODE_NORM 1
 
-static __device__ __forceinline__ short4_t sk_lo(const uint4& v) { return __builtin_bit_cast(short4_t, make_uint2(v.x, v.y)); }
-static __device__ __forceinline__ short4_t sk_hi(const uint4& v) { return __builtin_bit_cast(short4_t, make_uint2(v.z, v.w)); }
+// acc + A · B over 32 k: lane (r, g) gives k = 8 g .. 8 g + 7 of row r of A and of column r of B
+static __device__ __forceinline__ float4_t sk_mfma(const uint4& a, const uint4& b, float4_t acc) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
+}
 
 static __device__ __forceinline__ void sk_unpack(const uint4& v, float* f) {
   const uint32_t w[4] = {v.x, v.y, v.z, v.w};
@@ -144,8 +146,7 @@ gemm_skinny_kernel(const SkinnyArgs a) {
       const uint4 xb = sk_pack(xs[s]);
 #pragma unroll
       for (int t = 0; t < RT; ++t) {
-        acc[t][0] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(sk_lo(wreg[t][s]), sk_lo(xb), acc[t][0], 0, 0, 0);
-        acc[t][0] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(sk_hi(wreg[t][s]), sk_hi(xb), acc[t][0], 0, 0, 0);
+        acc[t][0] = sk_mfma(wreg[t][s], xb, acc[t][0]);
       }
     }
   } else {
@@ -163,10 +164,7 @@ gemm_skinny_kernel(const SkinnyArgs a) {
 #pragma unroll
         for (int t = 0; t < RT; ++t)
 #pragma unroll
-          for (int b = 0; b < CB; ++b) {
-            acc[t][b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(sk_lo(wreg[t][s0 + s]), sk_lo(xb[b][s]), acc[t][b], 0, 0, 0);
-            acc[t][b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(sk_hi(wreg[t][s0 + s]), sk_hi(xb[b][s]), acc[t][b], 0, 0, 0);
-          }
+          for (int b = 0; b < CB; ++b) acc[t][b] = sk_mfma(wreg[t][s0 + s], xb[b][s], acc[t][b]);
     }
   }
   // acc[t][b][j] = sum over this wave's k of W[row 16 t + 4 g + j of the workgroup, k] * f(x)[16 b + r, k]

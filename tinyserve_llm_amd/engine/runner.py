@@ -134,12 +134,14 @@ class ModelRunner:
                     raise StepError(f"a block table of {len(t)} pages exceeds the fixed width {widths[sp]}")
                 flat.extend(0 if p == FREED else p for p in t)
                 flat.extend([0] * (widths[sp] - len(t)))
-        slot_flat = [x for m in slot_maps for x in m]
+        slot_offset = len(flat)
+        for m in slot_maps:
+            flat.extend(m)
         host = dict(cu=cu, starts=starts, ctx_lens=ctx_lens, slots=slots)
-        return flat, slot_flat, (T, S, R, widths, offsets), host
+        return flat, (T, S, R, widths, offsets, slot_offset), host
 
-    def _context(self, packed: torch.Tensor, slot_packed: torch.Tensor, dims, host) -> tuple[StepContext, torch.Tensor]:
-        T, S, R, widths, offsets = dims
+    def _context(self, packed: torch.Tensor, dims, host) -> tuple[StepContext, torch.Tensor]:
+        T, S, R, widths, offsets, slot_offset = dims
         o = 0
 
         def cut(n: int) -> torch.Tensor:
@@ -156,16 +158,15 @@ class ModelRunner:
         row_t = cut(R)
         for sp in range(len(widths)):
             ctx.block_tables.append(packed[offsets[sp]:offsets[sp] + S * widths[sp]].view(S, widths[sp]))
-            ctx.slot_mapping.append(slot_packed[sp * T:(sp + 1) * T])
+            ctx.slot_mapping.append(packed[slot_offset + sp * T:slot_offset + (sp + 1) * T])
         return ctx, row_t
 
     def prepare(self, entries: Sequence[StepEntry]) -> tuple[StepContext, torch.Tensor, int]:
         """Packs a step into device tensors; returns (context, wanted rows, number of wanted rows).
         Everything a kernel will index with is checked here first."""
-        flat, slot_flat, dims, host = self._pack(entries)
+        flat, dims, host = self._pack(entries)
         packed = torch.tensor(flat, dtype=torch.int32).to(self.device, non_blocking=True)
-        slot_packed = torch.tensor(slot_flat, dtype=torch.int64).to(self.device, non_blocking=True)
-        ctx, rows = self._context(packed, slot_packed, dims, host)
+        ctx, rows = self._context(packed, dims, host)
         return ctx, rows, dims[2]
 
     # ---- running ----------------------------------------------------------------------------
@@ -220,17 +221,13 @@ class DecodeGraphs:
                 return False
         return True
 
-    def _capture(self, size: int, flat: list[int], slot_flat: list[int], dims, host):
+    def _capture(self, size: int, flat: list[int], dims, host):
         r = self.runner
         host_i32 = torch.empty(len(flat), dtype=torch.int32, pin_memory=True)
-        host_i64 = torch.empty(len(slot_flat), dtype=torch.int64, pin_memory=True)
         dev_i32 = torch.zeros(len(flat), dtype=torch.int32, device=r.device)
-        dev_i64 = torch.zeros(len(slot_flat), dtype=torch.int64, device=r.device)
         host_i32.copy_(torch.tensor(flat, dtype=torch.int32))
-        host_i64.copy_(torch.tensor(slot_flat, dtype=torch.int64))
         dev_i32.copy_(host_i32, non_blocking=True)
-        dev_i64.copy_(host_i64, non_blocking=True)
-        ctx, rows = r._context(dev_i32, dev_i64, dims, host)
+        ctx, rows = r._context(dev_i32, dims, host)
         # once without capture: libraries set up their workspaces, the kernel library loads
         side = torch.cuda.Stream(device=r.device)
         side.wait_stream(torch.cuda.current_stream(r.device))
@@ -245,7 +242,7 @@ class DecodeGraphs:
             logits = r.model.logits(hidden, residual, rows)
         if self.pool is None:
             self.pool = graph.pool()
-        return graph, host_i32, host_i64, dev_i32, dev_i64, logits
+        return graph, host_i32, dev_i32, logits
 
     def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         size = self._size(len(entries))
@@ -253,14 +250,12 @@ class DecodeGraphs:
         reach = min(-(-longest // self.bucket) * self.bucket, -(-self.max_context // self.bucket) * self.bucket)
         width = -(-reach // self.page_size)
         key = (size, width)
-        flat, slot_flat, dims, host = self.runner._pack(entries, [width] * self.num_spaces, pad_to=size)
+        flat, dims, host = self.runner._pack(entries, [width] * self.num_spaces, pad_to=size)
         if key not in self.graphs:
-            self.graphs[key] = self._capture(size, flat, slot_flat, dims, host)
+            self.graphs[key] = self._capture(size, flat, dims, host)
             # the capture recorded the step without running it: the replay below runs it
-        graph, host_i32, host_i64, dev_i32, dev_i64, logits = self.graphs[key]
+        graph, host_i32, dev_i32, logits = self.graphs[key]
         host_i32.copy_(torch.tensor(flat, dtype=torch.int32))
-        host_i64.copy_(torch.tensor(slot_flat, dtype=torch.int64))
         dev_i32.copy_(host_i32, non_blocking=True)
-        dev_i64.copy_(host_i64, non_blocking=True)
         graph.replay()
         return logits[:len(entries)]

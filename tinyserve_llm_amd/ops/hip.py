@@ -48,11 +48,11 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_silu_mul": [p, p, i, i, i, p],
         "ts_copy_slots": [p, i64, i64, i64, i, i, p],
         "ts_paged_attention_wave": [p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i64, i, f, i, i, p],
-        "ts_paged_attention_decode": [p, p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, i, i, f, i,
-                                      p],
+        "ts_paged_attention_decode": [p, p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, i, i, i, f,
+                                      i, p],
         "ts_gemm_exact": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_sample": [p, p, p, p, p, p, u64, i, i, i64, p],
-        "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, p],
+        "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, p],
         "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, p],
     }
     for name, args in sig.items():
@@ -151,7 +151,7 @@ def rope_store(qkv: torch.Tensor, cos_sin: torch.Tensor | None, positions: torch
     page_size, kst, vst = 1, (0, 0, 0), (0, 0, 0, 0)
     if k_cache is not None:
         _need(v_cache is not None and slots is not None, "a cache write needs k, v and the slots")
-        _need(slots.dtype == torch.int64 and slots.shape == (T,) and slots.is_contiguous(), "slots must be int64 [tokens]")
+        _need(slots.dtype == torch.int32 and slots.shape == (T,) and slots.is_contiguous(), "slots must be int32 [tokens]")
         _check_cache(k_cache, v_cache, qkv.dtype, num_kv_heads, head_dim)
         page_size, kst, vst = k_cache.shape[1], k_cache.stride()[:3], v_cache.stride()
     q = torch.empty((T, num_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
@@ -207,16 +207,33 @@ def paged_attention_wave(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.
 
 
 MAX_DECODE_SPLITS = 1024     # chunks per token that the combining kernel takes
+MAX_DECODE_TOKENS = 65535    # tokens are a grid dimension of the decode kernel
 DECODE_HEAD_DIMS = (32, 64, 96, 128)
 
 
-def decode_chunk(num_tokens: int, nkv: int, capacity: int) -> int:
-    """Keys per workgroup of the split-key kernel: 128, unless so many workgroups come of it that
-    fewer, larger ones save workspace traffic, or more chunks than the combining kernel takes."""
+MAX_DECODE_WAVES = 8
+
+
+def decode_plan(num_tokens: int, nkv: int, group: int, hd: int, capacity: int) -> tuple[int, int]:
+    """(keys per workgroup, waves per workgroup) of the split-key kernel for a step of `num_tokens`
+    one-query tokens over block tables that reach `capacity` positions. One workgroup per (token,
+    key/value head) takes the whole context, and nothing is combined, where a wave has one 32-key
+    step of it, or where the step has a workgroup for every compute unit anyway and the context is
+    moderate. Otherwise four waves share chunks of 128 keys, or of 256 when so many workgroups come
+    of it that fewer, larger ones save workspace traffic, or of more when the combining kernel would
+    not take the number of chunks."""
+    most = MAX_DECODE_WAVES
+    while most > 1 and 4 * (32 * most + most * group * hd) > 65536:
+        most //= 2
+    if capacity <= 32 * most:
+        waves = -(-capacity // 32)
+        return 32 * waves, waves
+    if num_tokens * nkv >= 256 and capacity <= 4096:
+        return -(-capacity // (32 * most)) * 32 * most, most
     chunk = 256 if num_tokens * nkv * -(-capacity // 128) >= 16384 else 128
     while -(-capacity // chunk) > MAX_DECODE_SPLITS:
         chunk *= 2
-    return chunk
+    return chunk, 4
 
 
 def decode_kernel_takes(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor) -> bool:
@@ -224,17 +241,18 @@ def decode_kernel_takes(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
     nh, hd = q.shape[1], q.shape[2]
     nkv, page = k_cache.shape[2], k_cache.shape[1]
     return (q.dtype == torch.bfloat16 and hd in DECODE_HEAD_DIMS and nh // nkv <= 16 and (nh // nkv) * hd <= 2048
-            and page % 8 == 0 and v_cache.stride(1) == 1 and q.shape[0] <= 65535
+            and page % 8 == 0 and v_cache.stride(1) == 1
             and all(st % 8 == 0 for st in (*k_cache.stride()[:3], v_cache.stride(0), v_cache.stride(2), v_cache.stride(3)))
             and v_cache.data_ptr() % 16 == 0)
 
 
 def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                            seq_of_token: torch.Tensor, positions: torch.Tensor, scale: float, window: int = 0,
-                           chunk: int | None = None) -> torch.Tensor:
+                           chunk: int | None = None, waves: int | None = None,
+                           out: torch.Tensor | None = None) -> torch.Tensor:
     """Split-key attention on the matrix cores for tokens that each bring one query (bfloat16,
     values in transposed pages). Every position in `positions` must lie inside the pages its row
-    of `block_tables` has (checked by the caller on the host)."""
+    of `block_tables` has (checked by the caller on the host). `out`, if given, receives the result."""
     _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions)
     _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
     T, nh, hd = q.shape
@@ -247,18 +265,25 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
           "block_tables must be contiguous int32 [requests, pages]")
     for name, t in (("seq_of_token", seq_of_token), ("positions", positions)):
         _need(t.dtype == torch.int32 and t.shape == (T,) and t.is_contiguous(), f"{name} must be int32 [tokens]")
+    _need(T <= MAX_DECODE_TOKENS, f"the decode kernel takes up to {MAX_DECODE_TOKENS} tokens a launch")
     capacity = block_tables.shape[1] * k_cache.shape[1]
-    chunk = chunk or decode_chunk(T, nkv, capacity)
+    if chunk is None:
+        chunk, waves = decode_plan(T, nkv, nh // nkv, hd, capacity)
+    waves = waves or 4
     splits = -(-capacity // chunk)
-    _need(chunk % 128 == 0 and splits <= MAX_DECODE_SPLITS, f"chunk {chunk} over {capacity} positions")
-    part_o = torch.empty((T, nh, splits, hd), dtype=torch.float32, device=q.device)
-    part_ml = torch.empty((T, nh, splits, 2), dtype=torch.float32, device=q.device)
-    out = torch.empty_like(q)
+    _need(1 <= waves <= MAX_DECODE_WAVES and chunk % (32 * waves) == 0 and splits <= MAX_DECODE_SPLITS,
+          f"chunk {chunk} in {waves} waves over {capacity} positions")
+    _need(4 * (32 * waves + waves * (nh // nkv) * hd) <= 65536, f"{waves} waves of {nh // nkv} heads exceed the LDS of a workgroup")
+    part_o = part_ml = None
+    if splits > 1:
+        part_o = torch.empty((T, nh, splits, hd), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((T, nh, splits, 2), dtype=torch.float32, device=q.device)
+    out = _out_like(q, out)
     _run("paged_attention_decode", library().ts_paged_attention_decode(
         _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
         _ptr(seq_of_token), _ptr(positions), T, nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3],
-        v_cache.stride(0), v_cache.stride(2), v_cache.stride(3), block_tables.shape[1], splits, chunk, float(scale),
-        int(window), _stream()))
+        v_cache.stride(0), v_cache.stride(2), v_cache.stride(3), block_tables.shape[1], splits, chunk, waves,
+        float(scale), int(window), _stream()))
     return out
 
 
@@ -329,22 +354,55 @@ def sample(logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor,
 
 # ---- dispatchers ---------------------------------------------------------------------------------
 
-def attention_tiles(cu_seqlens: list[int], tokens_per_tile: int) -> list[int]:
-    """Row tiles of a packed step for the matrix-core prefill kernel: (first token, token count)
-    pairs, flattened; a tile never crosses a request."""
-    flat: list[int] = []
-    for a, b in zip(cu_seqlens, cu_seqlens[1:]):
+def _out_like(q: torch.Tensor, out: torch.Tensor | None) -> torch.Tensor:
+    if out is None:
+        return torch.empty_like(q)
+    _gpu(out)
+    _need(out.shape == q.shape and out.dtype == q.dtype and out.is_contiguous(), "out must match q")
+    return out
+
+
+PREFILL_WAVES = 4            # waves of a workgroup of the prefill kernel; each holds 1, 2 or 4 row tiles
+PREFILL_MIN_WORKGROUPS = 512 # larger tiles only while this many workgroups remain
+
+
+def prefill_tile_tokens(num_tokens: int, nkv: int, group: int) -> int:
+    """Tokens per tile of the prefill kernel: as many row tiles per wave (4, 2 or 1) as still leave
+    the chip two workgroups per compute unit (a workgroup takes two tiles)."""
+    per_wave = PREFILL_WAVES * (16 // group)
+    for rt in (4, 2):
+        if -(-num_tokens // (2 * rt * per_wave)) * nkv >= PREFILL_MIN_WORKGROUPS:
+            return rt * per_wave
+    return per_wave
+
+
+def attention_tiles(cu_seqlens: list[int], starts: list[int], tokens_per_tile: int, first_seq: int = 0) -> list[int]:
+    """Tiles of a packed step for the matrix-core prefill kernel: (first token, token count) pairs,
+    flattened, for the requests from `first_seq` on. A tile never crosses a request; `starts[s]` is
+    the position of request s's first token in the step, and the tiles come in ascending order of
+    their last position, which is the number of keys the kernel walks for them."""
+    found: list[tuple[int, int, int]] = []
+    for s in range(first_seq, len(cu_seqlens) - 1):
+        a, b = cu_seqlens[s], cu_seqlens[s + 1]
         for t in range(a, b, tokens_per_tile):
-            flat += (t, min(tokens_per_tile, b - t))
+            n = min(tokens_per_tile, b - t)
+            found.append((starts[s] + t - a + n, t, n))
+    found.sort()
+    flat: list[int] = []
+    for _, t, n in found:
+        flat += (t, n)
     return flat
 
 
 def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                             seq_of_token: torch.Tensor, positions: torch.Tensor, tiles: torch.Tensor, scale: float,
-                            window: int = 0) -> torch.Tensor:
+                            window: int = 0, tile_tokens: int | None = None, out: torch.Tensor | None = None
+                            ) -> torch.Tensor:
     """Attention of a packed step on the matrix cores (bfloat16, values in transposed pages).
-    `tiles` int32 [num_tiles, 2] lists (first token, token count <= 16 // group) per row tile,
-    every tile inside one request; the caller has checked positions against the block tables."""
+    `tiles` int32 [num_tiles, 2] lists (first token, token count <= tile_tokens) per workgroup,
+    every tile inside one request and inside the step (the caller built the list from the step's
+    own lengths and has checked positions against the block tables), long tiles last; `tile_tokens`
+    is 4, 8 or 16 times 16 // group (default 4 times). Tokens that no tile lists keep what `out` held."""
     _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles)
     _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
     T, nh, hd = q.shape
@@ -359,10 +417,13 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         _need(t.dtype == torch.int32 and t.shape == (T,) and t.is_contiguous(), f"{name} must be int32 [tokens]")
     _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 2 and tiles.is_contiguous(),
           "tiles must be contiguous int32 [tiles, 2]")
-    out = torch.empty_like(q)
+    per_wave = PREFILL_WAVES * (16 // (nh // nkv))
+    tile_tokens = tile_tokens or per_wave
+    _need(tile_tokens in (per_wave, 2 * per_wave, 4 * per_wave), f"tiles of {tile_tokens} tokens; {per_wave}, twice or four times that")
+    out = _out_like(q, out)
     _run("paged_attention_prefill", library().ts_paged_attention_prefill(
         _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_of_token), _ptr(positions),
-        _ptr(tiles), tiles.shape[0], nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3], v_cache.stride(0),
+        _ptr(tiles), tiles.shape[0], tile_tokens, nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3], v_cache.stride(0),
         v_cache.stride(2), v_cache.stride(3), block_tables.shape[1], float(scale), int(window), _stream()))
     return out
 
@@ -375,15 +436,27 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     tables = ctx.block_tables[space]
     if decode_kernel_takes(q, k_cache, v_cache):
         capacity = tables.shape[1] * k_cache.shape[1]
-        if ctx.max_query_len == 1 and -(-capacity // 1024) <= MAX_DECODE_SPLITS:
+        decode_ok = -(-capacity // 1024) <= MAX_DECODE_SPLITS and q.shape[0] <= MAX_DECODE_TOKENS
+        if ctx.max_query_len == 1 and decode_ok:
             return paged_attention_decode(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, window)
-        per_tile = 16 // (q.shape[1] // k_cache.shape[2])
-        tiles = ctx.scratch.get(("attention_tiles", per_tile))
+        # the one-token requests that lead the step go to the split-key kernel, the rest to the tiles
+        cu = ctx.host_cu_seqlens
+        lead = 0
+        while decode_ok and lead + 1 < len(cu) and cu[lead + 1] - cu[lead] == 1:
+            lead += 1
+        nkv = k_cache.shape[2]
+        tile_tokens = prefill_tile_tokens(q.shape[0] - lead, nkv, q.shape[1] // nkv)
+        tiles = ctx.scratch.get(("attention_tiles", tile_tokens, lead))
         if tiles is None:
-            flat = attention_tiles(ctx.host_cu_seqlens, per_tile)
+            flat = attention_tiles(cu, ctx.host_starts, tile_tokens, lead)
             tiles = torch.tensor(flat, dtype=torch.int32).view(-1, 2).to(q.device, non_blocking=True)
-            ctx.scratch[("attention_tiles", per_tile)] = tiles
-        return paged_attention_prefill(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, tiles, scale, window)
+            ctx.scratch[("attention_tiles", tile_tokens, lead)] = tiles
+        out = torch.empty_like(q)
+        if lead:
+            paged_attention_decode(q[:lead], k_cache, v_cache, tables, ctx.seq_of_token[:lead], ctx.positions[:lead],
+                                   scale, window, out=out[:lead])
+        return paged_attention_prefill(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, tiles, scale,
+                                       window, tile_tokens=tile_tokens, out=out)
     return paged_attention_wave(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, window)
 
 
@@ -451,7 +524,8 @@ def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "linear_bf16 takes bfloat16")
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
           f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
-    if (skinny_takes(x.shape[0], x.shape[1]) and x.is_contiguous() and weight.is_contiguous()
+    # reductions longer than 4096 leave the kernel too few workgroups; the library streams those faster
+    if (skinny_takes(x.shape[0], x.shape[1]) and x.shape[1] <= 4096 and x.is_contiguous() and weight.is_contiguous()
             and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
         return gemm_skinny(x, weight, out_dtype)[0]
     y = torch.matmul(x, weight.t())

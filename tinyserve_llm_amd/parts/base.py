@@ -75,7 +75,7 @@ class StepContext:
     cu_seqlens: torch.Tensor              # [S+1] int32
     context_lens: torch.Tensor            # [S] int32, keys of each request after this step's writes
     state_slots: torch.Tensor             # [S] int32
-    slot_mapping: list[torch.Tensor]      # per space: [T] int64, page * page_size + offset
+    slot_mapping: list[torch.Tensor]      # per space: [T] int32, page * page_size + offset
     block_tables: list[torch.Tensor]      # per space: [S, max_pages] int32
     host_cu_seqlens: list[int] = field(default_factory=list)
     host_starts: list[int] = field(default_factory=list)      # first position fed, per request

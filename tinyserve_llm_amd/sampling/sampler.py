@@ -24,7 +24,8 @@ def row_key(request_id: int, sample_index: int, position: int) -> int:
 
 def sample(logits: torch.Tensor, temperatures: list[float], keys: list[int], seed: int) -> torch.Tensor:
     """One token id per row of float32 logits [rows, vocab] -> int32 [rows] on the device."""
-    device = logits.device
-    t = torch.tensor(temperatures, dtype=torch.float32).to(device, non_blocking=True)
-    k = torch.tensor(keys, dtype=torch.int64).to(device, non_blocking=True)
-    return hip.sample(logits, t, k, seed)
+    n = len(keys)
+    # keys and temperatures travel to the device in one copy
+    packed = torch.cat([torch.tensor(keys, dtype=torch.int64).view(torch.int32),
+                        torch.tensor(temperatures, dtype=torch.float32).view(torch.int32)]).to(logits.device, non_blocking=True)
+    return hip.sample(logits, packed[2 * n:].view(torch.float32), packed[:2 * n].view(torch.int64), seed)
