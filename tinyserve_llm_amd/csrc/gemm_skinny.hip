@@ -81,6 +81,34 @@ gemm_skinny_kernel(const SkinnyArgs a) {
   const int half = a.N / 2;
   const int kbeg = wave * STEPS * SK_KSTEP + 8 * g;     // this lane's first k
 
+  const bf16_t* xrow[CB];
+  bool xok[CB];
+#pragma unroll
+  for (int b = 0; b < CB; ++b) {
+    const int m = b * 16 + r;
+    xok[b] = m < a.M;
+    xrow[b] = a.x + (int64_t)(xok[b] ? m : 0) * a.ldx + kbeg;
+  }
+  // ---- MODE_NORM: this wave's slice of x, the residual and the norm weight are asked for before W.
+  // Loads come back in the order they were issued, and these are short and hit the cache: the norm
+  // is computed while W is still streaming in.
+  // (Workgroups of more than 8 waves have no registers to hold the norm weight meanwhile: they
+  // fetch it when they need it.)
+  constexpr bool EARLY_NW = MODE == MODE_NORM && MAXT <= 512;
+  uint4 xraw[MODE == MODE_NORM ? STEPS : 1], rraw[MODE == MODE_NORM ? STEPS : 1], nraw[EARLY_NW ? STEPS : 1];
+  if (MODE == MODE_NORM) {
+    // unconditional loads from addresses that always exist (rows past M read row 0, a missing
+    // residual reads x again): what does not count is dropped after it has arrived
+    const bf16_t* rrow = a.res ? a.res + (int64_t)(xok[0] ? r : 0) * a.K + kbeg : xrow[0];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      xraw[s] = *(const uint4*)(xrow[0] + s * SK_KSTEP);
+      rraw[s] = *(const uint4*)(rrow + s * SK_KSTEP);
+      if (EARLY_NW) nraw[s] = *(const uint4*)(a.nw + kbeg + s * SK_KSTEP);
+    }
+    __builtin_amdgcn_sched_barrier(0);                  // the compiler keeps these loads ahead of W's
+  }
+
   // ---- every load of this wave's slice of W, at once
   uint4 wreg[RT][STEPS];
 #pragma unroll
@@ -92,15 +120,9 @@ gemm_skinny_kernel(const SkinnyArgs a) {
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) wreg[t][s] = *(const uint4*)(wrow + s * SK_KSTEP);
   }
-
-  const bf16_t* xrow[CB];
-  bool xok[CB];
-#pragma unroll
-  for (int b = 0; b < CB; ++b) {
-    const int m = b * 16 + r;
-    xok[b] = m < a.M;
-    xrow[b] = a.x + (int64_t)(xok[b] ? m : 0) * a.ldx + kbeg;
-  }
+  // all of W's loads are in flight before anything waits: left to itself the compiler interleaves
+  // them with the products to save registers, and the matrix no longer streams at memory speed
+  __builtin_amdgcn_sched_barrier(0);
 
   float4_t acc[RT][CB];
 #pragma unroll
@@ -113,22 +135,21 @@ gemm_skinny_kernel(const SkinnyArgs a) {
     // workgroup together), then scaled, rounded and used
     float xs[STEPS][8];
     float sq = 0.f;
+    const bool has_res = a.res != nullptr;
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
+      // (both loads are used whatever the case, so that neither moves behind the loads of W)
+      float rv[8];
+      sk_unpack(xraw[s], xs[s]);
+      sk_unpack(rraw[s], rv);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) xs[s][i] = 0.f;
-      if (xok[0]) {
-        sk_unpack(*(const uint4*)(xrow[0] + s * SK_KSTEP), xs[s]);
-        if (a.res) {
-          float rv[8];
-          sk_unpack(*(const uint4*)(a.res + (int64_t)r * a.K + kbeg + s * SK_KSTEP), rv);
-#pragma unroll
-          for (int i = 0; i < 8; ++i) xs[s][i] += rv[i];
-          if (blockIdx.x == 0) *(uint4*)(a.res_out + (int64_t)r * a.K + kbeg + s * SK_KSTEP) = sk_pack(xs[s]);
-        }
-#pragma unroll
-        for (int i = 0; i < 8; ++i) sq = fmaf(xs[s][i], xs[s][i], sq);
+      for (int i = 0; i < 8; ++i) {
+        const float sum = xs[s][i] + (has_res ? rv[i] : 0.f);
+        xs[s][i] = xok[0] ? sum : 0.f;                   // rows past M count as zeros
       }
+      if (has_res && blockIdx.x == 0 && xok[0]) *(uint4*)(a.res_out + (int64_t)r * a.K + kbeg + s * SK_KSTEP) = sk_pack(xs[s]);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) sq = fmaf(xs[s][i], xs[s][i], sq);
     }
     sq += __shfl_xor(sq, 16, TS_WAVE);
     sq += __shfl_xor(sq, 32, TS_WAVE);
@@ -137,18 +158,21 @@ gemm_skinny_kernel(const SkinnyArgs a) {
     float total = 0.f;
     for (int wv = 0; wv < nwaves; ++wv) total += ssq[wv * 16 + r];
     const float inv = 1.0f / sqrtf(total / (float)a.K + a.eps);
+    // the normalised operand of every step is ready before the first product waits for W
+    uint4 xb[STEPS];
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
       float nv[8];
-      sk_unpack(*(const uint4*)(a.nw + kbeg + s * SK_KSTEP), nv);
+      sk_unpack(EARLY_NW ? nraw[s] : *(const uint4*)(a.nw + kbeg + s * SK_KSTEP), nv);
 #pragma unroll
       for (int i = 0; i < 8; ++i) xs[s][i] = __uint_as_float(sk_round(xs[s][i] * inv) << 16) * nv[i];
-      const uint4 xb = sk_pack(xs[s]);
-#pragma unroll
-      for (int t = 0; t < RT; ++t) {
-        acc[t][0] = sk_mfma(wreg[t][s], xb, acc[t][0]);
-      }
+      xb[s] = sk_pack(xs[s]);
     }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+      for (int t = 0; t < RT; ++t) acc[t][0] = sk_mfma(wreg[t][s], xb[s], acc[t][0]);
   } else {
     // ---- x in batches of steps, then the products
 #pragma unroll
@@ -158,7 +182,8 @@ gemm_skinny_kernel(const SkinnyArgs a) {
       for (int b = 0; b < CB; ++b)
 #pragma unroll
         for (int s = 0; s < SK_XBATCH; ++s)
-          xb[b][s] = xok[b] ? *(const uint4*)(xrow[b] + (s0 + s) * SK_KSTEP) : make_uint4(0, 0, 0, 0);
+          xb[b][s] = *(const uint4*)(xrow[b] + (s0 + s) * SK_KSTEP);   // rows past M repeat row 0 and are not stored
+      __builtin_amdgcn_sched_barrier(0);                // the batch is asked for at once
 #pragma unroll
       for (int s = 0; s < SK_XBATCH; ++s)
 #pragma unroll
@@ -208,10 +233,13 @@ static int sk_launch(const SkinnyArgs& a, hipStream_t stream) {
   constexpr int OT = GLU ? RT / 2 : RT;
   const int ncols = GLU ? a.N / 2 : a.N;
   dim3 grid((ncols + 16 * OT - 1) / (16 * OT)), block(nwaves * TS_WAVE);
-  if (nwaves <= 8)
+  if (nwaves <= 8) {
     gemm_skinny_kernel<RT, CB, STEPS, MODE, GLU, 512, OUT><<<grid, block, smem, stream>>>(a);
-  else
-    gemm_skinny_kernel<RT, CB, STEPS, MODE, GLU, 1024, OUT><<<grid, block, smem, stream>>>(a);
+  } else {
+    // only single row tiles leave a workgroup of 16 waves the registers it needs
+    if constexpr (RT == 1) gemm_skinny_kernel<RT, CB, STEPS, MODE, GLU, 1024, OUT><<<grid, block, smem, stream>>>(a);
+    else return TS_BAD_SHAPE;
+  }
   return ts_check_launch();
 }
 
