@@ -41,6 +41,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--points", default="1,64", help="further decode batch sizes (comma-separated; '' for none)")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--only", default="all", choices=["all", "prefill"],
+                    help="'prefill': time the 2,048-token prefill alone and print its record (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -109,6 +111,17 @@ def main() -> int:
             assert not llm.scheduler.has_unfinished()
         return min(times)
 
+    def prefill_record() -> dict:
+        t = prefill()
+        T = PROMPT_LEN
+        linear_flops = 2 * T * args.layers * layer_weights + 2 * c.vocab_size * c.hidden_size
+        attn_flops = args.layers * 4 * c.q_size * T * (T + 1) / 2
+        return {"value": T / t, "tokens": T, "ms": 1e3 * t, "frac": (linear_flops + attn_flops) / t / PEAK_FLOPS[args.dtype]}
+
+    if args.only == "prefill":
+        print(json.dumps({"prefill": prefill_record()}))
+        return 0
+
     seconds, mean_ctx = decode(args.batch, args.steps, args.warmup)
     value = args.batch * args.steps / seconds
     step_bytes = weight_bytes + args.batch * mean_ctx * kv_bytes_per_token
@@ -127,12 +140,7 @@ def main() -> int:
                      "frac": achieved / HBM_BYTES_PER_S},
     }
     if not args.no_prefill:
-        t = prefill()
-        T = PROMPT_LEN
-        linear_flops = 2 * T * args.layers * layer_weights + 2 * c.vocab_size * c.hidden_size
-        attn_flops = args.layers * 4 * c.q_size * T * (T + 1) / 2
-        record["prefill"] = {"value": T / t, "tokens": T, "ms": 1e3 * t,
-                             "frac": (linear_flops + attn_flops) / t / PEAK_FLOPS[args.dtype]}
+        record["prefill"] = prefill_record()
     points = {}
     for b in [int(x) for x in args.points.split(",") if x.strip()]:
         k = max(16, min(args.steps, 64))

@@ -274,16 +274,21 @@ class KVCacheManager:
         return need
 
     def can_append(self, seq_id: int, num_tokens: int) -> bool:
+        seq = self.seqs[seq_id]
+        if num_tokens and (seq.reserved % self.block_size) + num_tokens <= self.block_size and seq.reserved % self.block_size:
+            # the tokens stay inside the last page: pages are needed only to copy a shared tail
+            return all(sp.refs[t[-1]] <= 1 or sp.available() >= 1 for sp, t in zip(self.spaces, seq.tables))
         return all(self.blocks_needed_for_append(seq_id, num_tokens, i) <= sp.available()
                    for i, sp in enumerate(self.spaces))
 
-    def append_slots(self, seq_id: int, token_ids: Sequence[int]) -> None:
+    def append_slots(self, seq_id: int, token_ids: Sequence[int], checked: bool = False) -> None:
         """Reserves slots for the tokens a step feeds to an admitted request: a decoded token or the
-        next portion of its prompt. Closed by commit()."""
+        next portion of its prompt. Closed by commit(). `checked`: the caller has just asked
+        can_append for this very request and count."""
         assert token_ids, "a step feeds at least one token"
         seq = self.seqs[seq_id]
         assert seq.reserved == seq.committed, "the previous step was not committed"
-        assert self.can_append(seq_id, len(token_ids)), "not enough free pages; preempt first"
+        assert checked or self.can_append(seq_id, len(token_ids)), "not enough free pages; preempt first"
         self._reserve(seq, token_ids)
 
     def commit(self, seq_id: int, num_accepted: int) -> None:

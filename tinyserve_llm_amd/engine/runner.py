@@ -105,11 +105,15 @@ class ModelRunner:
                 if len(table) * ps < end:
                     raise StepError(f"request {e.seq_id}: {len(table)} pages reserved, positions up to {end - 1} fed")
                 first_read = max(0, e.start - self.windows[sp] + 1) if self.windows[sp] else 0
-                for j in range(first_read // ps, (end - 1) // ps + 1):
-                    if not 0 <= table[j] < self.storage.spaces[sp].num_pages:
-                        raise StepError(f"request {e.seq_id}: page {j} of space {sp} is {table[j]}")
+                read = table[first_read // ps:(end - 1) // ps + 1]
+                if min(read) < 0 or max(read) >= self.storage.spaces[sp].num_pages:
+                    raise StepError(f"request {e.seq_id}: its pages {first_read // ps}..{(end - 1) // ps} of space {sp} "
+                                    f"hold {min(read)}..{max(read)}")
                 tables[sp].append(table)
-                slot_maps[sp].extend(table[p // ps] * ps + p % ps for p in range(e.start, end))
+                if n == 1:
+                    slot_maps[sp].append(table[e.start // ps] * ps + e.start % ps)
+                else:
+                    slot_maps[sp].extend(table[p // ps] * ps + p % ps for p in range(e.start, end))
             cu.append(cu[-1] + n)
         for s in range(len(entries), pad_to):           # idle rows of a fixed-size batch
             ids.append(0)
@@ -132,7 +136,10 @@ class ModelRunner:
             for t in tables[sp]:
                 if len(t) > widths[sp]:
                     raise StepError(f"a block table of {len(t)} pages exceeds the fixed width {widths[sp]}")
-                flat.extend(0 if p == FREED else p for p in t)
+                if self.windows[sp]:
+                    flat.extend(0 if p == FREED else p for p in t)     # pages a window has passed
+                else:
+                    flat.extend(t)
                 flat.extend([0] * (widths[sp] - len(t)))
         slot_offset = len(flat)
         for m in slot_maps:

@@ -157,7 +157,8 @@ class Scheduler:
                 if budget <= 0:
                     continue
                 tokens = [seq.pending_token]
-            while not self.kv.can_append(seq.seq_id, len(tokens)):
+            fits = self.kv.can_append(seq.seq_id, len(tokens))
+            while not fits:
                 victim = self._lowest_unscheduled(now, exclude=seq, gone=gone)
                 if victim is None:
                     break
@@ -165,11 +166,12 @@ class Scheduler:
                 gone.add(victim.seq_id)
                 if victim in mine:
                     mine.remove(victim)
-            if not self.kv.can_append(seq.seq_id, len(tokens)):
+                fits = self.kv.can_append(seq.seq_id, len(tokens))
+            if not fits:
                 self._preempt(seq)
                 gone.add(seq.seq_id)
                 break
-            self.kv.append_slots(seq.seq_id, tokens)
+            self.kv.append_slots(seq.seq_id, tokens, checked=True)
             final = seq.num_computed + len(tokens) >= seq.prefill_target
             samples = 1
             if want_prefill:
