@@ -540,3 +540,60 @@ def test_sampler_draw_is_the_exponential_race_and_ignores_the_row_order():
     perm = torch.randperm(rows, generator=gen(16)).tolist()
     shuffled = sample(logits[perm].contiguous().to(dev()), [temps[i] for i in perm], [keys[i] for i in perm], seed=42).tolist()
     assert shuffled == [got[i] for i in perm]
+
+
+@pytest.mark.parametrize("nh,nkv,hd,K,M,page", [(32, 8, 64, 2048, 8, 64), (6, 2, 96, 768, 5, 16), (4, 4, 128, 256, 16, 8),
+                                                 (3, 1, 32, 1280, 1, 32)])
+@pytest.mark.parametrize("norm", [False, True])
+@pytest.mark.parametrize("rotate", [True, False])
+def test_fused_projection_rotation_and_cache_write(nh, nkv, hd, K, M, page, norm, rotate):
+    """The one-kernel path against projection, then rope_store: q, every written slot of k and v, and
+    slots it must not touch (slot -1, and pages of other requests)."""
+    g = gen(nh * 7 + K)
+    dtype = torch.bfloat16
+    x = (torch.randn(M, K, generator=g) * 0.5).to(dtype).to(dev())
+    w = (torch.randn((nh + 2 * nkv) * hd, K, generator=g) * K ** -0.5).to(dtype).to(dev())
+    res = (torch.randn(M, K, generator=g) * 0.5).to(dtype).to(dev())
+    nw = (1 + 0.1 * torch.randn(K, generator=g)).to(dtype).to(dev())
+    table = torch.randn(64, hd, generator=g).to(dev()) if rotate else None
+    positions = torch.randint(0, 64, (M,), generator=g, dtype=torch.int32).to(dev())
+    pages = 6
+    perm = torch.randperm(pages * page, generator=g)[:M].to(torch.int32)
+    if M > 2:
+        perm[1] = -1
+    slots = perm.to(dev())
+    def pools():
+        kp = torch.full((pages, nkv, page, hd), 7.0, dtype=dtype, device=dev())
+        vp = torch.full((pages, nkv, hd, page), 7.0, dtype=dtype, device=dev())
+        return kp, vp
+    kp1, vp1 = pools()
+    kp2, vp2 = pools()
+    if norm:
+        xn, res_want = hip().rmsnorm(x, nw, 1e-5, res)
+    else:
+        xn, res_want = x, None
+    qkv = hip().gemm_skinny(xn, w)[0]
+    q_want = hip().rope_store(qkv, table, positions, slots, kp1.permute(0, 2, 1, 3), vp1.permute(0, 3, 1, 2), nh, nkv, hd)
+    assert hip().qkv_rope_fuses(x, w, hd, kp2.permute(0, 2, 1, 3))
+    q, res_out = hip().qkv_rope_store(x, w, table, positions, slots, kp2.permute(0, 2, 1, 3), vp2.permute(0, 3, 1, 2),
+                                      nh, nkv, hd, **(dict(residual=res, norm_weight=nw, eps=1e-5) if norm else {}))
+    torch.testing.assert_close(q.float(), q_want.float(), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(kp2.float(), kp1.float(), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(vp2.float(), vp1.float(), rtol=2e-2, atol=2e-2)
+    assert int((kp2 != 7.0).any(dim=(1, 3)).sum()) == int((slots >= 0).sum()), "only the named slots are written"
+    if norm:
+        assert torch.equal(res_out, res_want)
+    # without a cache of its own a layer only gets q
+    q_only, _ = hip().qkv_rope_store(x, w, table, positions, None, None, None, nh, nkv, hd,
+                                     **(dict(residual=res, norm_weight=nw, eps=1e-5) if norm else {}))
+    assert torch.equal(q_only, q)
+
+
+def test_fused_projection_refuses_what_it_cannot_serve():
+    x = torch.zeros(17, 256, dtype=torch.bfloat16, device=dev())
+    w = torch.zeros(3 * 64, 256, dtype=torch.bfloat16, device=dev())
+    assert not hip().qkv_rope_fuses(x, w, 64, None), "17 rows"
+    assert not hip().qkv_rope_fuses(x[:4], w, 48, None), "head_dim 48"
+    assert not hip().qkv_rope_fuses(torch.zeros(4, 2304, dtype=torch.bfloat16, device=dev()), w, 64, None), "K beyond 2048"
+    with pytest.raises(hip().KernelError, match="qkv_rope_store takes"):
+        hip().qkv_rope_store(x, w, None, torch.zeros(17, dtype=torch.int32, device=dev()), None, None, None, 1, 1, 64)

@@ -12,6 +12,10 @@
 //              the way in (up to 16 rows); workgroup 0 also writes T(x + res) as the new residual
 //   EPI_GLU    W = [gate rows | up rows]; a workgroup takes matching rows of both and writes
 //              silu(gate) * up, y being [M, N / 2]
+//   EPI_ROPE   W = [q heads | k heads | v heads] of head_dim columns each; a workgroup takes 16
+//              columns of the first half of a head and the 16 that rotate with them, rounds the
+//              products as y would hold them, rotates q and k by the token's position, and writes q
+//              to its own tensor and k and v into their cache slots: y itself is never stored
 #include "common.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -20,6 +24,9 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 #define SK_KSTEP 32      // k covered by one MFMA: lane group g holds k = 8 g .. 8 g + 7
 #define MODE_PLAIN 0
 #define MODE_NORM 1
+#define EPI_NONE 0
+#define EPI_GLU 1
+#define EPI_ROPE 2
 
 // acc + A · B over 32 k: lane (r, g) gives k = 8 g .. 8 g + 7 of row r of A and of column r of B
 static __device__ __forceinline__ float4_t sk_mfma(const uint4& a, const uint4& b, float4_t acc) {
@@ -59,15 +66,26 @@ struct SkinnyArgs {
   int M, N, K;
   int64_t ldx, ldw, ldy;
   float eps;
+  // EPI_ROPE: N = (nh + 2 nkv) * hd; cos_sin [max_pos, hd] 32-bit, [cos | sin] halves; slot -1 stores nothing.
+  // key element: page * kp + offset * ks + head * kh + d; value element: page * vp + offset * vs + head * vh + d * vd
+  const float* cos_sin;
+  const int32_t* positions;
+  const int32_t* slots;
+  bf16_t* q_out;        // [M, nh * hd]
+  bf16_t* k_cache;      // null: this layer owns no cache, only q is produced
+  bf16_t* v_cache;
+  int nh, nkv, hd, rotate, page_size;
+  int64_t kp, ks, kh, vp, vs, vh, vd;
 };
 
 // RT: 16-row tiles of W per workgroup; CB: 16-row blocks of x; STEPS: 32-wide k steps per wave;
 // MAXT: most threads a workgroup of this instance is launched with (it bounds the registers)
-template <int RT, int CB, int STEPS, int MODE, int GLU, int MAXT, typename OUT>
+template <int RT, int CB, int STEPS, int MODE, int EPI, int MAXT, typename OUT>
 __global__ void __launch_bounds__(MAXT)
 gemm_skinny_kernel(const SkinnyArgs a) {
+  constexpr bool GLU = EPI == EPI_GLU, ROPE = EPI == EPI_ROPE, PAIRS = EPI != EPI_NONE;
   static_assert(MODE == MODE_PLAIN || CB == 1, "the fused norm serves one block of rows");
-  static_assert(!GLU || RT % 2 == 0, "gate and up tiles come in pairs");
+  static_assert(!PAIRS || RT % 2 == 0, "gate and up tiles, and the halves of a head, come in pairs");
   constexpr int SK_XBATCH = (CB == 2 && MAXT > 512) ? 4 : 8;   // steps of x fetched at a time
   extern __shared__ __align__(16) float smem[];
   const int nwaves = blockDim.x / TS_WAVE;
@@ -75,8 +93,10 @@ gemm_skinny_kernel(const SkinnyArgs a) {
   float* ssq = smem + (size_t)nwaves * RT * CB * 256;   // [nwaves][16]
   const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
-  // GLU: tiles 0 .. RT/2-1 are gate rows n0 + 16 t, tiles RT/2 .. RT-1 the up rows N/2 below them
-  constexpr int OT = GLU ? RT / 2 : RT;                 // 16-column tiles of the output per workgroup
+  // GLU: tiles 0 .. RT/2-1 are gate rows n0 + 16 t, tiles RT/2 .. RT-1 the up rows N/2 below them.
+  // ROPE: tiles 0 .. RT/2-1 are 16-row blocks of first halves of heads (block j of the matrix: head
+  // j / (hd / 32), rows 16 (j % (hd / 32)) of it), tiles RT/2 .. RT-1 the rows hd / 2 below them.
+  constexpr int OT = PAIRS ? RT / 2 : RT;               // 16-column tiles of the output per workgroup
   const int n0 = blockIdx.x * 16 * OT;
   const int half = a.N / 2;
   const int kbeg = wave * STEPS * SK_KSTEP + 8 * g;     // this lane's first k
@@ -114,7 +134,12 @@ gemm_skinny_kernel(const SkinnyArgs a) {
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
     int n = GLU ? (t < OT ? n0 + t * 16 + r : half + n0 + (t - OT) * 16 + r) : n0 + t * 16 + r;
-    const int limit = GLU ? (t < OT ? half : a.N) : a.N;
+    int limit = GLU ? (t < OT ? half : a.N) : a.N;
+    if (ROPE) {
+      const int per_head = a.hd / 32, j = blockIdx.x * OT + (t < OT ? t : t - OT);
+      n = (j / per_head) * a.hd + 16 * (j % per_head) + (t < OT ? 0 : a.hd / 2) + r;
+      limit = a.N;
+    }
     if (n >= limit) n = limit - 1;                      // rows past the end are computed and not stored
     const bf16_t* wrow = a.w + (int64_t)n * a.ldw + kbeg;
 #pragma unroll
@@ -214,11 +239,57 @@ gemm_skinny_kernel(const SkinnyArgs a) {
       const float* p = part + (((size_t)wv * RT + t) * CB + b) * 256 + ml * 16 + nl;
 #pragma unroll
       for (int j = 0; j < 4; ++j) s[j] += p[j];
-      if (GLU) {
+      if (PAIRS) {
         const float* pu = part + (((size_t)wv * RT + t + OT) * CB + b) * 256 + ml * 16 + nl;
 #pragma unroll
         for (int j = 0; j < 4; ++j) u[j] += pu[j];
       }
+    }
+    if (ROPE) {
+      const int per_head = a.hd / 32, jb = blockIdx.x * OT + t, hdh = a.hd / 2;
+      const int head = jb / per_head, d0 = 16 * (jb % per_head) + nl;   // d0 .. d0 + 3 of the head's first half
+      if (head >= a.nh + 2 * a.nkv) continue;
+      float y1[4], y2[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {                       // as the product would be stored
+        y1[j] = __uint_as_float(sk_round(s[j]) << 16);
+        y2[j] = __uint_as_float(sk_round(u[j]) << 16);
+      }
+      if (a.rotate && head < a.nh + a.nkv) {
+        const float* cs = a.cos_sin + (int64_t)a.positions[m] * a.hd + d0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float c = cs[j], sn = cs[hdh + j];
+          const float r1 = y1[j] * c - y2[j] * sn, r2 = y2[j] * c + y1[j] * sn;
+          y1[j] = r1;
+          y2[j] = r2;
+        }
+      }
+      const uint2 o1 = make_uint2(sk_round(y1[0]) | (sk_round(y1[1]) << 16), sk_round(y1[2]) | (sk_round(y1[3]) << 16));
+      const uint2 o2 = make_uint2(sk_round(y2[0]) | (sk_round(y2[1]) << 16), sk_round(y2[2]) | (sk_round(y2[3]) << 16));
+      if (head < a.nh) {
+        bf16_t* dst = a.q_out + ((int64_t)m * a.nh + head) * a.hd + d0;
+        *(uint2*)dst = o1;
+        *(uint2*)(dst + hdh) = o2;
+        continue;
+      }
+      const int64_t slot = a.slots ? a.slots[m] : -1;
+      if (!a.k_cache || slot < 0) continue;
+      const int64_t page = slot / a.page_size, off = slot - page * a.page_size;
+      if (head < a.nh + a.nkv) {
+        bf16_t* dst = a.k_cache + page * a.kp + off * a.ks + (int64_t)(head - a.nh) * a.kh + d0;
+        *(uint2*)dst = o1;
+        *(uint2*)(dst + hdh) = o2;
+      } else {
+        bf16_t* dst = a.v_cache + page * a.vp + off * a.vs + (int64_t)(head - a.nh - a.nkv) * a.vh + (int64_t)d0 * a.vd;
+        const uint32_t w1[2] = {o1.x, o1.y}, w2[2] = {o2.x, o2.y};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          dst[(int64_t)j * a.vd] = (bf16_t)(w1[j >> 1] >> (16 * (j & 1)));
+          dst[(int64_t)(hdh + j) * a.vd] = (bf16_t)(w2[j >> 1] >> (16 * (j & 1)));
+        }
+      }
+      continue;
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j)
@@ -230,8 +301,8 @@ template <int RT, int CB, int STEPS, int MODE, int GLU, typename OUT>
 static int sk_launch(const SkinnyArgs& a, hipStream_t stream) {
   const int nwaves = a.K / (STEPS * SK_KSTEP);
   const size_t smem = sizeof(float) * ((size_t)nwaves * RT * CB * 256 + (size_t)nwaves * 16);
-  constexpr int OT = GLU ? RT / 2 : RT;
-  const int ncols = GLU ? a.N / 2 : a.N;
+  constexpr int OT = GLU != EPI_NONE ? RT / 2 : RT;
+  const int ncols = GLU != EPI_NONE ? a.N / 2 : a.N;    // EPI_ROPE: the first halves of all heads
   dim3 grid((ncols + 16 * OT - 1) / (16 * OT)), block(nwaves * TS_WAVE);
   if (nwaves <= 8) {
     gemm_skinny_kernel<RT, CB, STEPS, MODE, GLU, 512, OUT><<<grid, block, smem, stream>>>(a);
@@ -287,7 +358,7 @@ extern "C" int ts_gemm_skinny_bf16(void* y, const void* x, const void* w, const 
   if (glu && (N % 2 || (N / 2) % 16)) return TS_BAD_SHAPE;
   if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)res | (uintptr_t)nw | (uintptr_t)res_out) & 15) return TS_BAD_SHAPE;
   if (mode == MODE_NORM && (!nw || (res && !res_out))) return TS_BAD_SHAPE;
-  SkinnyArgs a;
+  SkinnyArgs a = {};
   a.x = (const bf16_t*)x; a.res = (const bf16_t*)res; a.nw = (const bf16_t*)nw; a.res_out = (bf16_t*)res_out;
   a.w = (const bf16_t*)w; a.y = y; a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldw = ldw; a.ldy = ldy; a.eps = eps;
   if (out_dtype == 1) {
@@ -299,4 +370,34 @@ extern "C" int ts_gemm_skinny_bf16(void* y, const void* x, const void* w, const 
   }
   if (out_dtype == 0 && mode == MODE_PLAIN && !glu) return sk_dispatch<MODE_PLAIN, 0, float>(a, stream);
   return TS_BAD_DTYPE;
+}
+
+// The qkv projection of an attention layer with the rotation and the cache write on the way out:
+// q_out [M, nh * hd] gets the rotated queries, the rotated keys and the values go to the slots
+// `slots[m]` of the pages (see SkinnyArgs); w is [(nh + 2 nkv) * hd, K]. mode as above. Requires
+// M <= 16, hd a multiple of 32, K a multiple of 256 up to 2048, 8-byte aligned cache strides.
+extern "C" int ts_gemm_skinny_rope_bf16(void* q_out, const void* x, const void* w, const void* res, const void* nw,
+                                        void* res_out, int M, int K, int64_t ldx, int64_t ldw, float eps, int mode,
+                                        const float* cos_sin, const int32_t* positions, const int32_t* slots,
+                                        void* k_cache, void* v_cache, int nh, int nkv, int hd, int rotate,
+                                        int page_size, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vs,
+                                        int64_t vh, int64_t vd, hipStream_t stream) {
+  if (M <= 0) return TS_OK;
+  if (M > 16 || K <= 0 || K % 256 || K / 256 > 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K) return TS_BAD_SHAPE;
+  if (nh <= 0 || nkv < 0 || hd <= 0 || hd % 32 || page_size <= 0) return TS_BAD_SHAPE;
+  if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)res | (uintptr_t)nw | (uintptr_t)res_out | (uintptr_t)q_out) & 15)
+    return TS_BAD_SHAPE;
+  if (mode == MODE_NORM && (!nw || (res && !res_out))) return TS_BAD_SHAPE;
+  if (rotate && (!cos_sin || !positions)) return TS_BAD_SHAPE;
+  if (k_cache && (!v_cache || !slots || (kp % 4) || (ks % 4) || (kh % 4) || (((uintptr_t)k_cache) & 7))) return TS_BAD_SHAPE;
+  SkinnyArgs a;
+  a.x = (const bf16_t*)x; a.res = (const bf16_t*)res; a.nw = (const bf16_t*)nw; a.res_out = (bf16_t*)res_out;
+  a.w = (const bf16_t*)w; a.y = nullptr; a.M = M; a.N = (nh + 2 * nkv) * hd; a.K = K; a.ldx = ldx; a.ldw = ldw;
+  a.ldy = 0; a.eps = eps;
+  a.cos_sin = cos_sin; a.positions = positions; a.slots = slots; a.q_out = (bf16_t*)q_out;
+  a.k_cache = (bf16_t*)k_cache; a.v_cache = (bf16_t*)v_cache; a.nh = nh; a.nkv = nkv; a.hd = hd; a.rotate = rotate;
+  a.page_size = page_size; a.kp = kp; a.ks = ks; a.kh = kh; a.vp = vp; a.vs = vs; a.vh = vh; a.vd = vd;
+  if (mode == MODE_PLAIN) return sk_launch<2, 1, 8, MODE_PLAIN, EPI_ROPE, bf16_t>(a, stream);
+  if (mode == MODE_NORM) return sk_launch<2, 1, 8, MODE_NORM, EPI_ROPE, bf16_t>(a, stream);
+  return TS_BAD_SHAPE;
 }

@@ -54,6 +54,8 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_sample": [p, p, p, p, p, p, u64, i, i, i64, p],
         "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, p],
         "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, p],
+        "ts_gemm_skinny_rope_bf16": [p, p, p, p, p, p, i, i, i64, i64, f, i, p, p, p, p, p, i, i, i, i, i, i64, i64, i64,
+                                     i64, i64, i64, i64, p],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -515,6 +517,62 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
         _ptr(res_out) if residual is not None else None, M, N, K, x.stride(0), weight.stride(0), out.stride(0),
         float(eps), int(norm), int(glu), _code(out_dtype), _stream()))
     return out, res_out
+
+
+def qkv_rope_fuses(x: torch.Tensor, weight: torch.Tensor, head_dim: int, k_cache: torch.Tensor | None) -> bool:
+    """Whether `qkv_rope_store` serves these operands: few bfloat16 rows, a reduction of up to 2048 in
+    steps of 256, heads of a multiple of 32 dimensions, keys whose strides allow 8-byte stores."""
+    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.dim() == 2 and x.shape[0] <= SKINNY_FUSED_ROWS
+            and x.shape[1] % 256 == 0 and x.shape[1] // 256 <= 8 and head_dim % 32 == 0
+            and x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0
+            and (k_cache is None or (all(st % 4 == 0 for st in k_cache.stride()[:3]) and k_cache.data_ptr() % 8 == 0)))
+
+
+def qkv_rope_store(x: torch.Tensor, weight: torch.Tensor, cos_sin: torch.Tensor | None, positions: torch.Tensor,
+                   slots: torch.Tensor | None, k_cache: torch.Tensor | None, v_cache: torch.Tensor | None,
+                   num_heads: int, num_kv_heads: int, head_dim: int, *, residual: torch.Tensor | None = None,
+                   norm_weight: torch.Tensor | None = None, eps: float = 0.0
+                   ) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """`rope_store(f(x) · weight^T, ...)` in one kernel for few rows of x: the projection is never
+    stored, q [tokens, nh, hd] comes back rotated, rotated k and v go to their cache slots. With
+    `norm_weight`, f = RMSNorm(x + residual) * norm_weight and x + residual is the second result."""
+    _gpu(x, weight, cos_sin, positions, slots, k_cache, v_cache, residual, norm_weight)
+    _need(qkv_rope_fuses(x, weight, head_dim, k_cache), "qkv_rope_store takes up to 16 bfloat16 rows, K in steps of 256 "
+          "up to 2048, head_dim in steps of 32")
+    M, K = x.shape
+    _need(weight.shape == ((num_heads + 2 * num_kv_heads) * head_dim, K), f"weight {tuple(weight.shape)} for "
+          f"{num_heads}+2x{num_kv_heads} heads of {head_dim} over {K}")
+    _need(positions.dtype == torch.int32 and positions.shape == (M,) and positions.is_contiguous(),
+          "positions must be int32 [tokens]")
+    if cos_sin is not None:
+        _need(cos_sin.dtype == torch.float32 and cos_sin.dim() == 2 and cos_sin.shape[1] == head_dim
+              and cos_sin.is_contiguous(), "the rotation table must be float32 [positions, head_dim]")
+    page_size, kst, vst = 1, (0, 0, 0), (0, 0, 0, 0)
+    if k_cache is not None:
+        _need(v_cache is not None and slots is not None, "a cache write needs k, v and the slots")
+        _need(slots.dtype == torch.int32 and slots.shape == (M,) and slots.is_contiguous(), "slots must be int32 [tokens]")
+        _check_cache(k_cache, v_cache, x.dtype, num_kv_heads, head_dim)
+        page_size, kst, vst = k_cache.shape[1], k_cache.stride()[:3], v_cache.stride()
+    norm = norm_weight is not None
+    res_out = None
+    if norm:
+        _need(norm_weight.dtype == torch.bfloat16 and norm_weight.shape == (K,) and norm_weight.is_contiguous(),
+              "the norm weight must be bfloat16 [K]")
+        if residual is not None:
+            _need(residual.shape == x.shape and residual.dtype == x.dtype and residual.is_contiguous(),
+                  "residual must match the input")
+            res_out = torch.empty_like(x)
+        else:
+            res_out = x
+    else:
+        _need(residual is None, "a residual comes with a norm weight")
+    q = torch.empty((M, num_heads, head_dim), dtype=x.dtype, device=x.device)
+    _run("qkv_rope_store", library().ts_gemm_skinny_rope_bf16(
+        _ptr(q), _ptr(x), _ptr(weight), _ptr(residual), _ptr(norm_weight),
+        _ptr(res_out) if residual is not None else None, M, K, x.stride(0), weight.stride(0), float(eps), int(norm),
+        _ptr(cos_sin), _ptr(positions), _ptr(slots), _ptr(k_cache), _ptr(v_cache), num_heads, num_kv_heads, head_dim,
+        int(cos_sin is not None), page_size, *kst, *vst, _stream()))
+    return q, res_out
 
 
 def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:

@@ -12,7 +12,7 @@ import torch
 
 from tinyserve_llm_amd.ops import hip
 from tinyserve_llm_amd.parts.base import KVSpec, LayerMemory, Mixer, ParamSpec, StepContext, register
-from tinyserve_llm_amd.parts.linear import linear
+from tinyserve_llm_amd.parts.linear import DeferredNorm, linear
 
 
 @register("mixer", "attention")
@@ -44,6 +44,23 @@ class Attention(Mixer):
     def kv_size(self) -> int:
         return self.num_kv_heads * self.head_dim
 
+    def _project_fused(self, x, table, positions, slots, k_store, v_store) -> torch.Tensor | None:
+        """Projection, rotation and cache write in one kernel where a step is small enough for the
+        weight-streaming kernel; None where it is not."""
+        d = x if isinstance(x, DeferredNorm) else None
+        rows = d.x if d is not None else x
+        if not (rows.is_cuda and hip.qkv_rope_fuses(rows, self.qkv, self.head_dim, k_store)):
+            return None
+        if d is None:
+            return hip.qkv_rope_store(rows, self.qkv, table, positions, slots, k_store, v_store, self.num_heads,
+                                      self.num_kv_heads, self.head_dim)[0]
+        if d.weight.dtype != torch.bfloat16 or (d.residual is not None and not d.residual.is_contiguous()):
+            return None
+        q, d.residual_out = hip.qkv_rope_store(rows, self.qkv, table, positions, slots, k_store, v_store, self.num_heads,
+                                               self.num_kv_heads, self.head_dim, residual=d.residual,
+                                               norm_weight=d.weight, eps=d.eps)
+        return q
+
     def param_specs(self) -> dict[str, ParamSpec]:
         return {"qkv": ParamSpec((self.q_size + 2 * self.kv_size, self.hidden_size)),
                 "o": ParamSpec((self.hidden_size, self.q_size))}
@@ -52,10 +69,13 @@ class Attention(Mixer):
         return KVSpec(self.num_kv_heads, self.head_dim, self.window)
 
     def forward(self, x: torch.Tensor, ctx: StepContext, mem: LayerMemory) -> torch.Tensor:
-        qkv = linear(x, self.qkv)
         table = ctx.position_encodings[self.position].rotary_table() if self.position else None
-        q = hip.rope_store(qkv, table, ctx.positions, ctx.slot_mapping[mem.space] if mem.store else None,
-                           mem.k_cache if mem.store else None, mem.v_cache if mem.store else None,
-                           self.num_heads, self.num_kv_heads, self.head_dim)
+        slots = ctx.slot_mapping[mem.space] if mem.store else None
+        k_store, v_store = (mem.k_cache, mem.v_cache) if mem.store else (None, None)
+        q = self._project_fused(x, table, ctx.positions, slots, k_store, v_store)
+        if q is None:
+            qkv = linear(x, self.qkv)
+            q = hip.rope_store(qkv, table, ctx.positions, slots, k_store, v_store, self.num_heads, self.num_kv_heads,
+                               self.head_dim)
         o = hip.paged_attention(q, mem.k_cache, mem.v_cache, ctx, mem.space, self.scale, self.window)
         return linear(o.view(ctx.num_tokens, self.q_size), self.o)
