@@ -1,0 +1,91 @@
+"""The layer sizes that bench.py measures (Llama-3.2-1B: width 2048, 32 query and 8 key/value heads
+of 64, feed-forward 8192, vocabulary 128256, llama3 rope scaling), with two layers and random
+weights, against the plain implementation: a prompt fed whole and in portions, then tokens decoded
+one by one (the steps bench.py times), for two requests side by side. The tiny configurations of
+the other tests never reach the kernels' instances for these sizes."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+from tests.helpers import prompt
+from tests.plain.llama import PlainLlama
+from tinyserve_llm_amd.config import LlamaConfig, RopeScaling
+from tinyserve_llm_amd.weights.random_init import write_random_model
+
+pytestmark = pytest.mark.gpu
+
+CONFIG = LlamaConfig(
+    vocab_size=128256, hidden_size=2048, intermediate_size=8192, num_hidden_layers=2, num_attention_heads=32,
+    num_key_value_heads=8, head_dim=64, max_position_embeddings=131072, rms_norm_eps=1e-5, rope_theta=500000.0,
+    rope_scaling=RopeScaling(factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                             original_max_position_embeddings=8192),
+    tie_word_embeddings=True, eos_token_id=128001)
+# float32: a sum of K terms in ascending order carries a rounding error of about sqrt(K) * 2^-24 of
+# its partial sums; K is 2048 and 8192 here (64 to 128 in the tiny configurations), logits are of
+# order 1, and a logit lies behind a dozen such sums: a few 1e-6 each, 5e-5 bounds them together.
+# A wrong kernel instance shows at 1e-3 and above.
+# bfloat16: rounding an activation to 8 bits of mantissa moves a logit by about 1e-3 of the logits'
+# spread, and a logit lies behind a few dozen roundings: the error is a fraction of a percent of the
+# spread in the mean and a few percent at worst among the 1.8 million logits compared. The spread is
+# 0.9 here (0.16 for the tiny configurations, whose bound of 1.5e-2 is the same tenth of it), so
+# the bounds are stated in units of it: root mean square 1.5 %, worst 10 %.
+TOL = {"float32": dict(atol=5e-5, rtol=1e-5)}
+BF16_RMS, BF16_WORST = 0.015, 0.10
+LENGTHS = [300, 77]
+DECODED = 6
+
+
+@pytest.fixture(scope="module")
+def case(tmp_path_factory):
+    folder = str(tmp_path_factory.mktemp("bench_shape"))
+    write_random_model(folder, CONFIG, 3, torch.bfloat16)
+    prompts = [prompt(50 + i, n, CONFIG.vocab_size) for i, n in enumerate(LENGTHS)]
+    plain = PlainLlama(folder, torch.float64)        # stored in bfloat16: both engines see the same weights
+    rows = {}
+    for r, p in enumerate(prompts):
+        logits = plain.logits(p)
+        for pos in range(len(p) - DECODED - 1, len(p)):
+            rows[(r, pos)] = logits[pos].clone()
+        del logits
+    del plain
+    return folder, prompts, rows
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prompt_portions_then_decoding_side_by_side(case, dtype):
+    from tinyserve_llm_amd.engine.replay import Replay
+    folder, prompts, rows = case
+    rep = Replay(folder, dtype, 512)
+    got = {}
+    # request 0 in two portions (200 tokens, then the rest of its prompt beside all of request 1's)
+    heads = [len(p) - DECODED for p in prompts]
+    rep.step([{"id": "r0", "tokens": prompts[0][:200], "want": []}], [])
+    logits = rep.step([{"id": "r0", "tokens": prompts[0][200:heads[0]], "want": [heads[0] - 200 - 1]},
+                       {"id": "r1", "tokens": prompts[1][:heads[1]], "want": [heads[1] - 1]}], [])
+    got[(0, heads[0] - 1)], got[(1, heads[1] - 1)] = logits[0], logits[1]
+    # then both decode, one token each per step
+    for k in range(DECODED):
+        last = k == DECODED - 1
+        logits = rep.step([{"id": f"r{r}", "tokens": [prompts[r][heads[r] + k]], "want": [0]} for r in range(2)],
+                          ["r0", "r1"] if last else [])
+        for r in range(2):
+            got[(r, heads[r] + k)] = logits[r]
+    spread = float(torch.stack(list(rows.values())).std())
+    assert spread > 0.05, "the comparison would be empty on logits that are all alike"
+    worst, squares, count = 0.0, 0.0, 0
+    for key, row in got.items():
+        want = rows[key]
+        err = row.double().cpu() - want
+        if dtype == "float32":
+            torch.testing.assert_close(row.double().cpu(), want, **TOL[dtype], msg=lambda m: f"request/position {key}: {m}")
+        else:
+            rms = float(err.pow(2).mean().sqrt())
+            assert rms <= BF16_RMS * spread, f"request/position {key}: root mean square error {rms:.3e}, spread {spread:.3f}"
+            assert float(err.abs().max()) <= BF16_WORST * spread, f"request/position {key}: worst error {float(err.abs().max()):.3e}"
+        worst = max(worst, float(err.abs().max()))
+        squares += float(err.pow(2).sum())
+        count += err.numel()
+    print(f"[{dtype}] worst absolute logit error {worst:.3e}, root mean square {(squares / count) ** 0.5:.3e} over "
+          f"{len(got)} rows; logits have standard deviation {spread:.3f}")

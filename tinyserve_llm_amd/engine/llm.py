@@ -105,7 +105,7 @@ class LLM:
         self.scheduler = Scheduler(scheduler_config, self.manager)
         self.runner = ModelRunner(self.model, self.storage, self.manager)
         if decode_graphs:
-            self.runner.enable_decode_graphs(scheduler_config.max_model_len, scheduler_config.max_num_seqs)
+            self.runner.enable_decode_graphs(scheduler_config.max_model_len, scheduler_config.max_num_seqs, self.seed)
         self.steps: list[StepRecord] = []
         logger.info("KV cache: %d blocks of %d tokens", num_blocks, cache_config.block_size)
 
@@ -149,6 +149,12 @@ class LLM:
         entries, temps, keys, owners = [], [], [], []
         for seq, tokens, num_samples, start in batch:
             entries.append(StepEntry(seq.seq_id, tokens, start, [len(tokens) - 1] if num_samples else []))
+        if all(b.num_samples == 1 for b in batch):
+            # one draw per entry: the step function draws too (decode steps replay one graph for both)
+            for seq, tokens, num_samples, start in batch:
+                temps.append(seq.params.temperature)
+                keys.append(row_key(seq.request_id, seq.sample_index, len(seq.output_token_ids)))
+            return [[t] for t in self.runner.step_sample(entries, temps, keys, self.seed).tolist()]
         logits = self.runner.step(entries)
         row = 0
         rows: list[int] = []

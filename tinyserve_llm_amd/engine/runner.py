@@ -189,13 +189,25 @@ class ModelRunner:
             return torch.empty((0, self.model.spec.vocab_size), dtype=torch.float32, device=self.device)
         return self.model.logits(hidden, residual, rows)
 
-    def enable_decode_graphs(self, max_context: int, max_batch: int) -> bool:
+    @torch.inference_mode()
+    def step_sample(self, entries: Sequence[StepEntry], temperatures: Sequence[float], keys: Sequence[int],
+                    seed: int) -> torch.Tensor:
+        """Runs a step in which every entry wants the logits of exactly one place and draws one token
+        from each: int32 [entries] on the device. `keys[i]` names the draw of entry i (see
+        `sampling.sampler`). Decode steps replay a graph that holds the draw as well."""
+        if self.graphs is not None and self.graphs.seed == seed and self.graphs.takes(entries):
+            return self.graphs.run(entries, (temperatures, keys))
+        from tinyserve_llm_amd.sampling.sampler import sample
+        return sample(self.step(entries), list(temperatures), list(keys), seed)
+
+    def enable_decode_graphs(self, max_context: int, max_batch: int, seed: int = 0) -> bool:
         """Decode steps (every entry one token whose logits are wanted) are then replayed from HIP
         graphs, one per batch size, instead of being launched kernel by kernel. Only for models
-        whose parts all declare `graph_safe`. Returns whether graphs are on."""
+        whose parts all declare `graph_safe`. `seed` is the one the graphs' draws use. Returns
+        whether graphs are on."""
         if not self.model.graph_safe():
             return False
-        self.graphs = DecodeGraphs(self, max_context, max_batch)
+        self.graphs = DecodeGraphs(self, max_context, max_batch, seed)
         return True
 
 
@@ -203,10 +215,12 @@ class DecodeGraphs:
     """HIP graphs of the decode step. A graph is captured the first time a (batch size, context
     bucket) pair is met: sizes above 8 round up to a multiple of 8 and idle rows fill the batch;
     the longest context of the batch rounds up to a multiple of 256 positions and fixes the width
-    of the block tables, and with it the attention kernels' grids. A graph's inputs live in fixed
-    device buffers that every replay overwrites with one copy from pinned host memory."""
+    of the block tables, and with it the attention kernels' grids. A graph's inputs live in one
+    fixed device buffer that every replay overwrites with one copy from pinned host memory: the
+    step's integers, then the draws' keys and temperatures. A graph ends with the logits and with
+    the tokens drawn from them; a caller that only wants logits ignores the tokens."""
 
-    def __init__(self, runner: ModelRunner, max_context: int, max_batch: int) -> None:
+    def __init__(self, runner: ModelRunner, max_context: int, max_batch: int, seed: int = 0) -> None:
         self.runner = runner
         self.page_size = runner.storage.page_size
         self.num_spaces = len(runner.storage.spaces)
@@ -216,6 +230,7 @@ class DecodeGraphs:
         self.can_pad = not runner.model.state_plan()
         self.graphs: dict[int, tuple] = {}
         self.pool = None
+        self.seed = seed                  # of the draws the graphs hold
 
     def _size(self, n: int) -> int:
         return n if n <= 8 or not self.can_pad else -(-n // 8) * 8
@@ -228,41 +243,62 @@ class DecodeGraphs:
                 return False
         return True
 
-    def _capture(self, size: int, flat: list[int], dims, host):
+    @staticmethod
+    def _with_draws(flat: list[int], size: int, draws) -> tuple[torch.Tensor, int]:
+        """The upload: `flat`, padded to an even length, then `size` keys (int64) and `size`
+        temperatures (float32) as raw words; rows without a draw get key 0 and temperature 0."""
+        start = len(flat) + (len(flat) & 1)
+        words = torch.zeros(start + 3 * size, dtype=torch.int32)
+        words[:len(flat)] = torch.tensor(flat, dtype=torch.int32)
+        if draws is not None:
+            temperatures, keys = draws
+            n = len(keys)
+            words[start:start + 2 * n] = torch.tensor(keys, dtype=torch.int64).view(torch.int32)
+            words[start + 2 * size:start + 2 * size + n] = torch.tensor(temperatures, dtype=torch.float32).view(torch.int32)
+        return words, start
+
+    def _capture(self, size: int, words: torch.Tensor, start: int, dims, host):
+        from tinyserve_llm_amd.ops import hip
         r = self.runner
-        host_i32 = torch.empty(len(flat), dtype=torch.int32, pin_memory=True)
-        dev_i32 = torch.zeros(len(flat), dtype=torch.int32, device=r.device)
-        host_i32.copy_(torch.tensor(flat, dtype=torch.int32))
+        host_i32 = torch.empty(len(words), dtype=torch.int32, pin_memory=True)
+        dev_i32 = torch.zeros(len(words), dtype=torch.int32, device=r.device)
+        host_i32.copy_(words)
         dev_i32.copy_(host_i32, non_blocking=True)
         ctx, rows = r._context(dev_i32, dims, host)
+        draw_keys = dev_i32[start:start + 2 * size].view(torch.int64)
+        draw_temps = dev_i32[start + 2 * size:start + 3 * size].view(torch.float32)
         # once without capture: libraries set up their workspaces, the kernel library loads
         side = torch.cuda.Stream(device=r.device)
         side.wait_stream(torch.cuda.current_stream(r.device))
         with torch.cuda.stream(side):
             hidden, residual = r.model.forward(ctx, r.memory)
-            r.model.logits(hidden, residual, rows)
+            hip.sample(r.model.logits(hidden, residual, rows), draw_temps, draw_keys, self.seed)
         torch.cuda.current_stream(r.device).wait_stream(side)
         torch.cuda.synchronize(r.device)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, pool=self.pool):
             hidden, residual = r.model.forward(ctx, r.memory)
             logits = r.model.logits(hidden, residual, rows)
+            tokens = hip.sample(logits, draw_temps, draw_keys, self.seed)
         if self.pool is None:
             self.pool = graph.pool()
-        return graph, host_i32, dev_i32, logits
+        return graph, host_i32, dev_i32, logits, tokens
 
-    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def run(self, entries: Sequence[StepEntry], draws=None) -> torch.Tensor:
+        """Replays the step's graph. Without `draws` the logits [entries, vocab] come back; with
+        `draws` = (temperatures, keys) the tokens drawn from them, int32 [entries]."""
         size = self._size(len(entries))
         longest = max(e.start + 1 for e in entries)
         reach = min(-(-longest // self.bucket) * self.bucket, -(-self.max_context // self.bucket) * self.bucket)
         width = -(-reach // self.page_size)
         key = (size, width)
         flat, dims, host = self.runner._pack(entries, [width] * self.num_spaces, pad_to=size)
+        words, start = self._with_draws(flat, size, draws)
         if key not in self.graphs:
-            self.graphs[key] = self._capture(size, flat, dims, host)
+            self.graphs[key] = self._capture(size, words, start, dims, host)
             # the capture recorded the step without running it: the replay below runs it
-        graph, host_i32, dev_i32, logits = self.graphs[key]
-        host_i32.copy_(torch.tensor(flat, dtype=torch.int32))
+        graph, host_i32, dev_i32, logits, tokens = self.graphs[key]
+        host_i32.copy_(words)
         dev_i32.copy_(host_i32, non_blocking=True)
         graph.replay()
-        return logits[:len(entries)]
+        return (logits if draws is None else tokens)[:len(entries)]
