@@ -1,6 +1,6 @@
 // Split-key paged attention on the matrix cores for tokens that each bring one query (decoding),
 // bfloat16. A workgroup takes one (token, key/value head, chunk of keys) and serves all query heads
-// of that key/value head's group; its waves (up to 8) take an equal share of the chunk each and work
+// of that key/value head's group; its waves (up to 8, or 4 for heads wider than 64) take an equal share of the chunk each and work
 // through it 32 keys at a time:
 //     S^T[key, head] = K[key, :] · Q[head, :]      v_mfma_f32_16x16x32_bf16, keys as rows
 //     online softmax per head (32-bit), P = exp(S - max)
@@ -16,9 +16,13 @@
 #include "attention_mfma.h"
 
 #define DEC_MAX_WAVES 8
+// heads wider than 64 keep two steps of wide rows in registers: their workgroups have up to 4 waves
+#define DEC_WAVES_FOR(HD) ((HD) > 64 ? 4 : DEC_MAX_WAVES)
 
-template <int HD>
-__global__ void __launch_bounds__(DEC_MAX_WAVES * TS_WAVE)
+// ONE: a wave has a single 32-key step (chunk = 32 waves); without the second buffer of the
+// general loop the kernel needs fewer registers and more workgroups share a compute unit
+template <int HD, bool ONE>
+__global__ void __launch_bounds__(DEC_WAVES_FOR(HD) * TS_WAVE)
 attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, const bf16_t* __restrict__ q,
                         const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
                         const int32_t* __restrict__ block_tables, const int32_t* __restrict__ seq_of_token,
@@ -64,7 +68,13 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, fl
   if (kb < (lo & ~31)) kb = lo & ~31;
 #define TS_LOAD(T, KB) load_tile<HD>(T, KB, r, g, lo, pos, kvh, table, pm, k_cache, v_cache, kp, ks, kh, vp, vh, vd)
 #define TS_USE(T, KB) use_tile_auto<HD>(T, KB, r, g, lo, pos, pos, lo, qreg, scale2, m, l, o)
-  if (kb < kend) {
+  if (ONE) {
+    if (kb < kend) {
+      KVTile<HD> A;
+      TS_LOAD(A, kb);
+      TS_USE(A, kb);
+    }
+  } else if (kb < kend) {
     KVTile<HD> A, B;
     TS_LOAD(A, kb);
     while (true) {
@@ -167,7 +177,7 @@ extern "C" int ts_paged_attention_decode(void* out, float* part_o, float* part_m
   if (num_tokens <= 0) return TS_OK;
   if (nkv <= 0 || nh % nkv || page_size <= 0 || page_size % 8 || max_blocks <= 0 || num_splits <= 0)
     return TS_BAD_SHAPE;
-  if (waves < 1 || waves > DEC_MAX_WAVES || chunk <= 0 || chunk % (32 * waves) || num_splits > COMBINE_MAX_SPLITS)
+  if (waves < 1 || waves > DEC_WAVES_FOR(hd) || chunk <= 0 || chunk % (32 * waves) || num_splits > COMBINE_MAX_SPLITS)
     return TS_BAD_SHAPE;
   if (num_splits > 1 && (!part_o || !part_ml)) return TS_BAD_SHAPE;
   if (num_tokens > 65535 || nkv > 65535) return TS_BAD_SHAPE;
@@ -184,11 +194,12 @@ extern "C" int ts_paged_attention_decode(void* out, float* part_o, float* part_m
     while ((1 << page_shift) < page_size) ++page_shift;
   }
   dim3 grid(num_splits, nkv, num_tokens);
-#define TS_DEC(HH)                                                                                              \
-  attn_decode_mfma_kernel<HH><<<grid, waves * TS_WAVE, smem, stream>>>(                                     \
+#define TS_DEC1(HH, ON)                                                                                         \
+  attn_decode_mfma_kernel<HH, ON><<<grid, waves * TS_WAVE, smem, stream>>>(                                 \
       (bf16_t*)out, part_o, part_ml, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,          \
       block_tables, seq_of_token, positions, nh, G, page_size, page_shift, kp, ks, kh, vp, vh, vd, max_blocks,  \
       num_splits, chunk, scale * 1.44269504088896340736f, window)
+#define TS_DEC(HH) if (chunk == 32 * waves) TS_DEC1(HH, true); else TS_DEC1(HH, false)
   switch (hd) {
     case 32: TS_DEC(32); break;
     case 64: TS_DEC(64); break;
@@ -197,6 +208,7 @@ extern "C" int ts_paged_attention_decode(void* out, float* part_o, float* part_m
     default: return TS_BAD_SHAPE;
   }
 #undef TS_DEC
+#undef TS_DEC1
   int rc = ts_check_launch();
   if (rc || num_splits == 1) return rc;
   attn_decode_combine_kernel<<<num_tokens * nh, TS_WAVE, 0, stream>>>((bf16_t*)out, part_o, part_ml, positions, nh, hd,

@@ -216,26 +216,31 @@ DECODE_HEAD_DIMS = (32, 64, 96, 128)
 MAX_DECODE_WAVES = 8
 
 
+def decode_waves(hd: int) -> int:
+    """Most waves of a workgroup of the decode kernel: heads wider than 64 leave registers for 4."""
+    return 4 if hd > 64 else MAX_DECODE_WAVES
+
+
 def decode_plan(num_tokens: int, nkv: int, group: int, hd: int, capacity: int) -> tuple[int, int]:
     """(keys per workgroup, waves per workgroup) of the split-key kernel for a step of `num_tokens`
-    one-query tokens over block tables that reach `capacity` positions. One workgroup per (token,
-    key/value head) takes the whole context, and nothing is combined, where a wave has one 32-key
-    step of it, or where the step has a workgroup for every compute unit anyway and the context is
-    moderate. Otherwise four waves share chunks of 128 keys, or of 256 when so many workgroups come
-    of it that fewer, larger ones save workspace traffic, or of more when the combining kernel would
-    not take the number of chunks."""
-    most = MAX_DECODE_WAVES
+    one-query tokens over block tables that reach `capacity` positions; measured choices. One
+    workgroup per (token, key/value head) takes the whole context, and nothing is combined, where a
+    wave has one 32-key step of it, or where the step has a workgroup for every compute unit anyway
+    and the context is moderate. Otherwise a workgroup's waves take one 32-key step each (the
+    instance without a second buffer: more workgroups share a compute unit), four steps each for
+    very long contexts, or more when the combining kernel would not take the number of chunks."""
+    most = decode_waves(hd)
     while most > 1 and 4 * (32 * most + most * group * hd) > 65536:
         most //= 2
     if capacity <= 32 * most:
         waves = -(-capacity // 32)
         return 32 * waves, waves
-    if num_tokens * nkv >= 256 and capacity <= 4096:
+    if num_tokens * nkv >= 256 and capacity <= 16384:
         return -(-capacity // (32 * most)) * 32 * most, most
-    chunk = 256 if num_tokens * nkv * -(-capacity // 128) >= 16384 else 128
+    chunk = 32 * most if capacity <= 16384 else 128 * most
     while -(-capacity // chunk) > MAX_DECODE_SPLITS:
         chunk *= 2
-    return chunk, 4
+    return chunk, most
 
 
 def decode_kernel_takes(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor) -> bool:
@@ -273,7 +278,7 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
         chunk, waves = decode_plan(T, nkv, nh // nkv, hd, capacity)
     waves = waves or 4
     splits = -(-capacity // chunk)
-    _need(1 <= waves <= MAX_DECODE_WAVES and chunk % (32 * waves) == 0 and splits <= MAX_DECODE_SPLITS,
+    _need(1 <= waves <= decode_waves(hd) and chunk % (32 * waves) == 0 and splits <= MAX_DECODE_SPLITS,
           f"chunk {chunk} in {waves} waves over {capacity} positions")
     _need(4 * (32 * waves + waves * (nh // nkv) * hd) <= 65536, f"{waves} waves of {nh // nkv} heads exceed the LDS of a workgroup")
     part_o = part_ml = None
