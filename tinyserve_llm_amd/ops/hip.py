@@ -469,6 +469,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 
 SKINNY_MAX_ROWS = 32
 SKINNY_FUSED_ROWS = 16       # the fused norm and the gated epilogue serve one 16-row block of x
+SKINNY_WIDE_ELEMENTS = 8 << 20   # largest matrix that `linear_bf16` gives the kernel with 17 to 32 rows
 
 
 def skinny_takes(rows: int, k: int) -> bool:
@@ -587,9 +588,12 @@ def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "linear_bf16 takes bfloat16")
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
           f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
-    # reductions longer than 4096 leave the kernel too few workgroups; the library streams those faster
-    if (skinny_takes(x.shape[0], x.shape[1]) and x.shape[1] <= 4096 and x.is_contiguous() and weight.is_contiguous()
-            and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
+    # Measured: reductions longer than 4096 leave the kernel too few workgroups, and with more than 16
+    # rows it only wins on small matrices (8M elements: a layer's qkv and o, not its gate_up or the
+    # head); the library streams the rest faster.
+    if (skinny_takes(x.shape[0], x.shape[1]) and x.shape[1] <= 4096
+            and (x.shape[0] <= SKINNY_FUSED_ROWS or weight.numel() <= SKINNY_WIDE_ELEMENTS)
+            and x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
         return gemm_skinny(x, weight, out_dtype)[0]
     y = torch.matmul(x, weight.t())
     return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
