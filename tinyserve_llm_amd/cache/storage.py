@@ -22,7 +22,7 @@ import torch
 
 from tinyserve_llm_amd.cache.manager import SpaceSpec
 from tinyserve_llm_amd.ops import hip
-from tinyserve_llm_amd.parts.base import KVSpec, StateSpec
+from tinyserve_llm_amd.parts.base import KVSpec
 
 
 @dataclass

@@ -10,6 +10,7 @@ logits [wanted, vocab] in the order of the entries and of their `want` lists.
 
 from __future__ import annotations
 
+import struct
 from dataclasses import dataclass, field
 from typing import Protocol, Sequence
 
@@ -147,6 +148,52 @@ class ModelRunner:
         host = dict(cu=cu, starts=starts, ctx_lens=ctx_lens, slots=slots)
         return flat, (T, S, R, widths, offsets, slot_offset), host
 
+    def _pack_decode(self, entries: Sequence[StepEntry], table_widths: list[int], pad_to: int):
+        """`_pack` for steps whose entries all feed one token and want its logits: the same checks
+        and the same layout, without the per-token loops."""
+        ps = self.storage.page_size
+        vocab, max_pos = self.model.spec.vocab_size, self.model.spec.max_position
+        num_spaces = len(self.storage.spaces)
+        S, n = max(pad_to, len(entries)), len(entries)
+        ids = [e.tokens[0] for e in entries]
+        starts = [e.start for e in entries]
+        if len({e.seq_id for e in entries}) != n:
+            raise StepError("a request appears twice in one step")
+        if min(ids) < 0 or max(ids) >= vocab:
+            raise StepError(f"a token id outside the vocabulary of {vocab}")
+        if min(starts) < 0 or max(starts) >= max_pos:
+            raise StepError(f"a position outside the model's {max_pos}")
+        pad = S - n
+        slots = [self.view.state_slot(e.seq_id) for e in entries]
+        flat = (ids + [0] * pad + starts + [0] * pad + list(range(S)) + list(range(S + 1))
+                + [p + 1 for p in starts] + [1] * pad + slots + [0] * pad + list(range(S)))
+        offsets, slot_flat = [], []
+        for sp in range(num_spaces):
+            offsets.append(len(flat))
+            width, window, pages = table_widths[sp], self.windows[sp], self.storage.spaces[sp].num_pages
+            for e in entries:
+                table = self.view.block_table(e.seq_id, sp)
+                last = e.start // ps
+                if len(table) <= last or len(table) > width:
+                    raise StepError(f"request {e.seq_id}: {len(table)} pages reserved for position {e.start} "
+                                    f"(fixed width {width})")
+                read = table[max(0, e.start - window + 1) // ps if window else 0:last + 1]
+                if min(read) < 0 or max(read) >= pages:
+                    raise StepError(f"request {e.seq_id}: its pages of space {sp} hold {min(read)}..{max(read)}")
+                if window:
+                    flat.extend(0 if p == FREED else p for p in table)
+                else:
+                    flat.extend(table)
+                flat.extend([0] * (width - len(table)))
+                slot_flat.append(table[last] * ps + e.start % ps)
+            flat.extend([0] * (pad * width))
+            slot_flat.extend([-1] * pad)
+        slot_offset = len(flat)
+        flat.extend(slot_flat)
+        host = dict(cu=list(range(S + 1)), starts=starts + [0] * pad, ctx_lens=[p + 1 for p in starts] + [1] * pad,
+                    slots=slots + [0] * pad)
+        return flat, (S, S, S, table_widths, offsets, slot_offset), host
+
     def _context(self, packed: torch.Tensor, dims, host) -> tuple[StepContext, torch.Tensor]:
         T, S, R, widths, offsets, slot_offset = dims
         o = 0
@@ -245,17 +292,24 @@ class DecodeGraphs:
 
     @staticmethod
     def _with_draws(flat: list[int], size: int, draws) -> tuple[torch.Tensor, int]:
-        """The upload: `flat`, padded to an even length, then `size` keys (int64) and `size`
-        temperatures (float32) as raw words; rows without a draw get key 0 and temperature 0."""
+        """The upload: `flat`, padded to an even length, then `size` keys (int64, low word first)
+        and `size` temperatures (float32) as raw 32-bit words; rows without a draw get key 0 and
+        temperature 0."""
         start = len(flat) + (len(flat) & 1)
-        words = torch.zeros(start + 3 * size, dtype=torch.int32)
-        words[:len(flat)] = torch.tensor(flat, dtype=torch.int32)
-        if draws is not None:
+        words = flat + [0] * (start - len(flat))
+        if draws is None:
+            words += [0] * (3 * size)
+        else:
             temperatures, keys = draws
             n = len(keys)
-            words[start:start + 2 * n] = torch.tensor(keys, dtype=torch.int64).view(torch.int32)
-            words[start + 2 * size:start + 2 * size + n] = torch.tensor(temperatures, dtype=torch.float32).view(torch.int32)
-        return words, start
+            for k in keys:                                   # two's complement halves, as int32
+                lo, hi = k & 0xFFFFFFFF, (k >> 32) & 0xFFFFFFFF
+                words.append(lo - (1 << 32) if lo >= 1 << 31 else lo)
+                words.append(hi - (1 << 32) if hi >= 1 << 31 else hi)
+            words += [0] * (2 * (size - n))
+            words += struct.unpack(f"{n}i", struct.pack(f"{n}f", *temperatures))
+            words += [0] * (size - n)
+        return torch.tensor(words, dtype=torch.int32), start
 
     def _capture(self, size: int, words: torch.Tensor, start: int, dims, host):
         from tinyserve_llm_amd.ops import hip
@@ -292,7 +346,7 @@ class DecodeGraphs:
         reach = min(-(-longest // self.bucket) * self.bucket, -(-self.max_context // self.bucket) * self.bucket)
         width = -(-reach // self.page_size)
         key = (size, width)
-        flat, dims, host = self.runner._pack(entries, [width] * self.num_spaces, pad_to=size)
+        flat, dims, host = self.runner._pack_decode(entries, [width] * self.num_spaces, pad_to=size)
         words, start = self._with_draws(flat, size, draws)
         if key not in self.graphs:
             self.graphs[key] = self._capture(size, words, start, dims, host)
