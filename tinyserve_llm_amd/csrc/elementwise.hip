@@ -209,26 +209,42 @@ extern "C" int ts_rmsnorm(void* out, void* res_out, const void* x, const void* r
 // neighbouring threads write neighbouring slots of a transposed page.
 // ------------------------------------------------------------------------------------------
 #define ROPE_TOK 16
+#define ROPE_VTILE 256     // value elements of a token that pass through LDS at a time
 
 template <typename T>
 __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
                                   const T* __restrict__ qkv, const float* __restrict__ cos_sin,
                                   const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
                                   int num_tokens, int nh, int nkv, int hd, int rotate, int page_size, int64_t kp,
-                                  int64_t ks, int64_t kh, int64_t vp, int64_t vs, int64_t vh, int64_t vd, int vec) {
+                                  int64_t ks, int64_t kh, int64_t vp, int64_t vs, int64_t vh, int64_t vd, int vec, int vtile,
+                                  int v_slices) {
   const int t0 = blockIdx.x * ROPE_TOK;
   const int nt = num_tokens - t0 < ROPE_TOK ? num_tokens - t0 : ROPE_TOK;
   const int half = hd / 2;
+  // v_slices > 0: the last v_slices of the gridDim.y slices write the values, the others rotate q
+  // and k (the two are independent chains of loads and stores: side by side they take half the
+  // time); v_slices == 0: every workgroup does its slice of both
+  int by = blockIdx.y, ny = gridDim.y;
+  bool do_qk = true, do_v = true;
+  if (v_slices > 0) {
+    const int qk_slices = gridDim.y - v_slices;
+    if (by < qk_slices) { do_v = false; ny = qk_slices; }
+    else { do_qk = false; by -= qk_slices; ny = v_slices; }
+  }
+  // slot -> (page, offset) in 32-bit arithmetic; a shift where the page size is a power of two
+  const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
+  auto page_of = [&](int slot) { return page_shift >= 0 ? slot >> page_shift : slot / page_size; };
   const int row = (nh + 2 * nkv) * hd;
   const int qpairs = nh * half, kpairs = nkv * half;
   // q and k pairs of every token of the group: this workgroup's slice of them
   const int npairs = nt * (qpairs + kpairs);
   constexpr int V = 16 / sizeof(T);
-  if (vec) {
+  if (!do_qk) {
+  } else if (vec) {
     // 16 bytes of each half of a head at a time
     const int per_head = half / V;
     const int npieces = nt * (nh + nkv) * per_head;
-    const int pbeg = (int)((int64_t)npieces * blockIdx.y / gridDim.y), pend = (int)((int64_t)npieces * (blockIdx.y + 1) / gridDim.y);
+    const int pbeg = (int)((int64_t)npieces * by / ny), pend = (int)((int64_t)npieces * (by + 1) / ny);
     for (int i = pbeg + threadIdx.x; i < pend; i += blockDim.x) {
       const int tl = i / ((nh + nkv) * per_head), e = i - tl * ((nh + nkv) * per_head);
       const int t = t0 + tl;
@@ -251,8 +267,8 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
       }
       T* dst;
       if (is_k) {
-        const int64_t slot = slots[t];
-        dst = k_cache + (slot / page_size) * kp + (slot % page_size) * ks + (int64_t)(h - nh) * kh;
+        const int slot = slots[t], pg = page_of(slot);
+        dst = k_cache + (int64_t)pg * kp + (int64_t)(slot - pg * page_size) * ks + (int64_t)(h - nh) * kh;
       } else {
         dst = q_out + ((int64_t)t * nh + h) * hd;
       }
@@ -260,7 +276,7 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
       Pack16<T>::st(dst + j + half, x2);
     }
   } else {
-  const int pbeg = (int)((int64_t)npairs * blockIdx.y / gridDim.y), pend = (int)((int64_t)npairs * (blockIdx.y + 1) / gridDim.y);
+  const int pbeg = (int)((int64_t)npairs * by / ny), pend = (int)((int64_t)npairs * (by + 1) / ny);
   for (int i = pbeg + threadIdx.x; i < pend; i += blockDim.x) {
     const int tl = i / (qpairs + kpairs), e = i - tl * (qpairs + kpairs);
     const int t = t0 + tl;
@@ -279,8 +295,8 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
     }
     T* dst;
     if (is_k) {
-      const int64_t slot = slots[t];
-      dst = k_cache + (slot / page_size) * kp + (slot % page_size) * ks + (int64_t)h * kh;
+      const int slot = slots[t], pg = page_of(slot);
+      dst = k_cache + (int64_t)pg * kp + (int64_t)(slot - pg * page_size) * ks + (int64_t)h * kh;
     } else {
       dst = q_out + ((int64_t)t * nh + h) * hd;
     }
@@ -288,19 +304,81 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
     Num<T>::st(dst + j + half, y2);
   }
   }
-  if (!k_cache) return;
-  // values: thread -> (element, token), token fastest
+  if (!k_cache || !do_v) return;
   const int vel = nkv * hd;
-  const int vbeg = (int)((int64_t)vel * blockIdx.y / gridDim.y) * ROPE_TOK;
-  const int vend = (int)((int64_t)vel * (blockIdx.y + 1) / gridDim.y) * ROPE_TOK;
+  if (vtile) {
+    // values through LDS: rows of the step are read 16 bytes at a time, then every thread takes one
+    // (head, dimension) and writes its 8 consecutive tokens as one 16-byte piece of a transposed
+    // page where their slots are consecutive, aligned and inside one page
+    __shared__ T tile[ROPE_TOK][ROPE_VTILE];
+    __shared__ int base_slot[ROPE_TOK / 8];          // first slot of each run of 8 tokens, or -1: no fast path
+    constexpr int VP = 16 / sizeof(T);                // elements of a 16-byte piece
+    static_assert(VP == 8 || sizeof(T) == 4, "runs of 8 tokens are pieces of bfloat16");
+    if (threadIdx.x < ROPE_TOK / 8) {
+      const int first = t0 + 8 * threadIdx.x;
+      int s0 = -1;
+      if (8 * threadIdx.x + 7 < nt) {
+        int sl[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) sl[k] = slots[first + k];
+        s0 = sl[0];
+        bool ok = s0 >= 0 && s0 % 8 == 0 && s0 % page_size + 7 < page_size;
+#pragma unroll
+        for (int k = 1; k < 8; ++k) ok = ok & (sl[k] == s0 + k);
+        if (!ok) s0 = -1;
+      }
+      base_slot[threadIdx.x] = s0;
+    }
+    const int ebeg = (int)((int64_t)(vel / VP) * by / ny) * VP;
+    const int eend = (int)((int64_t)(vel / VP) * (by + 1) / ny) * VP;
+    for (int eb = ebeg; eb < eend; eb += ROPE_VTILE) {
+      __syncthreads();                                // the previous tile has been read (and base_slot written)
+      for (int p = threadIdx.x; p < ROPE_TOK * (ROPE_VTILE / VP); p += blockDim.x) {
+        const int tl = p / (ROPE_VTILE / VP), e = eb + (p % (ROPE_VTILE / VP)) * VP;
+        if (tl < nt && e < eend)
+          *(uint4*)&tile[tl][e - eb] = *(const uint4*)(qkv + (int64_t)(t0 + tl) * row + (nh + nkv) * hd + e);
+      }
+      __syncthreads();
+      for (int el = threadIdx.x; el < ROPE_VTILE && eb + el < eend; el += blockDim.x) {
+        const int e = eb + el, h = e / hd, d = e - h * hd;
+#pragma unroll
+        for (int run = 0; run < ROPE_TOK / 8; ++run) {
+          const int s0 = base_slot[run];
+          if (s0 >= 0 && sizeof(T) == 2) {
+            uint32_t w[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+              w[k] = (uint32_t)(*(const uint16_t*)&tile[8 * run + 2 * k][el]) |
+                     ((uint32_t)(*(const uint16_t*)&tile[8 * run + 2 * k + 1][el]) << 16);
+            const int pg = page_of(s0);
+            *(uint4*)(v_cache + (int64_t)pg * vp + (s0 - pg * page_size) + (int64_t)h * vh + (int64_t)d * vd) =
+                make_uint4(w[0], w[1], w[2], w[3]);
+          } else {
+            for (int k = 0; k < 8; ++k) {
+              const int tl = 8 * run + k;
+              if (tl >= nt) break;
+              const int slot = slots[t0 + tl];
+              if (slot < 0) continue;
+              const int pg = page_of(slot);
+              v_cache[(int64_t)pg * vp + (int64_t)(slot - pg * page_size) * vs + (int64_t)h * vh + (int64_t)d * vd] = tile[tl][el];
+            }
+          }
+        }
+      }
+    }
+    return;
+  }
+  // values: thread -> (element, token), token fastest
+  const int vbeg = (int)((int64_t)vel * by / ny) * ROPE_TOK;
+  const int vend = (int)((int64_t)vel * (by + 1) / ny) * ROPE_TOK;
   for (int i = vbeg + threadIdx.x; i < vend; i += blockDim.x) {
     const int tl = i % ROPE_TOK, e = i / ROPE_TOK;
     if (tl >= nt) continue;
     const int t = t0 + tl;
-    const int64_t slot = slots[t];
+    const int slot = slots[t];
     if (slot < 0) continue;
-    const int h = e / hd, d = e - h * hd;
-    v_cache[(slot / page_size) * vp + (slot % page_size) * vs + (int64_t)h * vh + (int64_t)d * vd] =
+    const int h = e / hd, d = e - h * hd, pg = page_of(slot);
+    v_cache[(int64_t)pg * vp + (int64_t)(slot - pg * page_size) * vs + (int64_t)h * vh + (int64_t)d * vd] =
         qkv[(int64_t)t * row + (nh + nkv) * hd + e];
   }
 }
@@ -312,23 +390,33 @@ extern "C" int ts_rope_store(void* q_out, void* k_cache, void* v_cache, const vo
   if (num_tokens <= 0) return TS_OK;
   if (hd % 2 || nh <= 0 || nkv < 0 || page_size <= 0) return TS_BAD_SHAPE;
   const int groups = (num_tokens + ROPE_TOK - 1) / ROPE_TOK;
-  int slices = 512 / groups;
+  int slices = 2048 / groups;                       // enough workgroups to hide the loads' latency
   if (slices < 1) slices = 1;
   if (slices > 32) slices = 32;
-  const dim3 blocks(groups, slices);
+  dim3 blocks(groups, slices);
   // 16-byte pieces need halves of whole pieces and aligned rows everywhere
   const int per16 = dtype == 0 ? 4 : 8;
   const int row = (nh + 2 * nkv) * hd;
   const int vec = (hd / 2) % per16 == 0 && row % per16 == 0 && kp % per16 == 0 && ks % per16 == 0 && kh % per16 == 0 &&
                   ((((uintptr_t)q_out) | ((uintptr_t)k_cache) | ((uintptr_t)qkv)) & 15) == 0;
+  // values through LDS: bfloat16 steps of several tokens into transposed pages (slot stride 1) whose
+  // 8-slot pieces are 16-byte aligned
+  const int vtile = dtype == 1 && num_tokens >= 8 && v_cache && vs == 1 && row % 8 == 0 && ((nh + nkv) * hd) % 8 == 0 &&
+                    (nkv * hd) % 8 == 0 && page_size % 8 == 0 && vp % 8 == 0 && vh % 8 == 0 && vd % 8 == 0 &&
+                    ((((uintptr_t)v_cache) | ((uintptr_t)qkv)) & 15) == 0;
+  int v_slices = 0;
+  if (vtile) {                                        // values are a sixth or so of the work
+    v_slices = slices / 4 > 0 ? slices / 4 : 1;
+    blocks.y = slices + v_slices;
+  }
   if (dtype == 0)
     rope_store_kernel<float><<<blocks, 256, 0, stream>>>((float*)q_out, (float*)k_cache, (float*)v_cache,
                                                          (const float*)qkv, cos_sin, positions, slots, num_tokens, nh,
-                                                         nkv, hd, rotate, page_size, kp, ks, kh, vp, vs, vh, vd, vec);
+                                                         nkv, hd, rotate, page_size, kp, ks, kh, vp, vs, vh, vd, vec, 0, 0);
   else if (dtype == 1)
     rope_store_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache,
                                                           (const bf16_t*)qkv, cos_sin, positions, slots, num_tokens,
-                                                          nh, nkv, hd, rotate, page_size, kp, ks, kh, vp, vs, vh, vd, vec);
+                                                          nh, nkv, hd, rotate, page_size, kp, ks, kh, vp, vs, vh, vd, vec, vtile, v_slices);
   else
     return TS_BAD_DTYPE;
   return ts_check_launch();
