@@ -1,13 +1,13 @@
 // Split-key paged attention on the matrix cores for tokens that each bring one query (decoding),
 // bfloat16. A workgroup takes one (token, key/value head, chunk of keys) and serves all query heads
-// of that key/value head's group; its waves (up to 8, or 4 for heads wider than 64) take an equal share of the chunk each and work
-// through it 32 keys at a time:
+// of that key/value head's group; its waves (up to 8, or 4 for heads wider than 64) take an equal
+// share of the chunk each and work through it 32 keys at a time:
 //     S^T[key, head] = K[key, :] · Q[head, :]      v_mfma_f32_16x16x32_bf16, keys as rows
-//     online softmax per head (32-bit), P = exp(S - max)
+//     online softmax per head (32-bit), P = 2^(S - m)
 //     O[head, :]    += P[head, key] · V[key, :]
 // The result layout of the first product is the operand layout of the second, so P never leaves
 // its registers. Keys are read as 16-byte pieces of their rows; values are read from pages that
-// hold them transposed ([head_dim, page_size] per head), so that the four consecutive keys an
+// hold them transposed ([head_dim, page_size] per head), so that the eight consecutive keys an
 // operand needs lie side by side in memory. The waves' partial results meet in LDS. With one chunk
 // per token (few tokens, contexts short enough for one workgroup to stream) the workgroup
 // normalises and writes the output itself. Otherwise a chunk's unnormalised output with its running
@@ -23,8 +23,8 @@
 // general loop the kernel needs fewer registers and more workgroups share a compute unit
 template <int HD, bool ONE>
 __global__ void __launch_bounds__(DEC_WAVES_FOR(HD) * TS_WAVE)
-attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, const bf16_t* __restrict__ q,
-                        const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
+                        const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
                         const int32_t* __restrict__ block_tables, const int32_t* __restrict__ seq_of_token,
                         const int32_t* __restrict__ positions, int nh, int G, int page_size, int page_shift,
                         int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
