@@ -229,3 +229,35 @@ def test_decode_graphs_replay_what_eager_steps_compute(folder_b):
             assert [a for a, p in zip(again, params) if not p.temperature] == \
                 [a for a, p in zip(outs[0], params) if not p.temperature]
     assert outs[0] == outs[1]
+
+
+@pytest.mark.parametrize("num_blocks", [120, 18])
+def test_steps_closed_in_two_halves_generate_the_same(folder_b, num_blocks):
+    """With `run_ahead` a decode step is scheduled and packed while the one before it still runs,
+    from a placeholder for the token under way. Tokens must equal those of the engine that closes
+    every step before it schedules the next: with sampling (keys name request, sample and position),
+    with sequences that end by themselves, and with so few pages that sequences are preempted."""
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+    base = dict(max_model_len=128, max_num_seqs=8, max_num_batched_tokens=80, max_prefill_chunk=32, watermark=0.0)
+    prompts = [prompt(70 + i, 3 + 5 * i, 384) for i in range(11)]
+    params = [SamplingParams(max_tokens=3 + 4 * (i % 6), temperature=1.5 if i % 3 else 0.0, n=2 if i == 4 else 1,
+                             ignore_eos=i % 2 == 0) for i in range(11)]
+    # an end token that some request draws in the middle of its output: found with a token nobody draws
+    free = LLM(folder_b, SchedulerConfig(eos_token_id=10 ** 6, **base), CacheConfig(block_size=16), dtype=torch.float32,
+               num_blocks=120, seed=11, run_ahead=False)
+    drawn = [r.token_ids[0] for r, p in zip(free.generate(prompts, params), params) if not p.ignore_eos]
+    eos = next(out[len(out) // 2] for out in drawn if len(out) >= 5)
+    sc = SchedulerConfig(eos_token_id=eos, **base)
+    outs, stats = [], []
+    for ahead in (True, False):
+        llm = LLM(folder_b, sc, CacheConfig(block_size=16), dtype=torch.float32, num_blocks=num_blocks, seed=11,
+                  run_ahead=ahead)
+        outs.append([(r.token_ids, r.finish_reasons) for r in llm.generate(prompts, params)])
+        stats.append(llm.scheduler.stats())
+        assert llm.manager.stats().blocks_in_use == 0 and llm._ahead is None
+    assert outs[0] == outs[1]
+    assert any("eos" in reasons for _, reasons in outs[0]) and any("length" in reasons for _, reasons in outs[0])
+    if num_blocks == 18:
+        assert stats[0].preemptions > 0 and stats[1].preemptions > 0

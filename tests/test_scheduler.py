@@ -69,6 +69,54 @@ def run_step(s, now, token_for=model):
     return batch, outputs
 
 
+class AheadLoop:
+    """The engine's other order of a step: a step of decodes only is closed in two halves, with the
+    schedule of the next step in between (the device would still be running then)."""
+
+    def __init__(self, s, token_for=model):
+        self.s, self.token_for, self.ahead = s, token_for, None
+        self.used_ahead = 0
+
+    def launch(self, batch):
+        m = self.s.kv
+        sampled = []
+        for seq, fed, num_samples, start in batch:
+            st = m.seqs[seq.seq_id]
+            assert st.committed == start and st.token_ids[start:] == list(fed), "positions start where the cache ends"
+            assert list(fed) == seq.all_token_ids[start:start + len(fed)] and -1 not in fed
+            forward(m, seq.seq_id)
+            history = [m.storage.slots[0][st.block_table[p // B]][p % B] for p in range(st.reserved)]
+            sampled.append([self.token_for(history, k) for k in range(num_samples)])
+        return sampled
+
+    def step(self, now):
+        s = self.s
+        batch, self.ahead = (self.ahead, None) if self.ahead else (s.schedule(now), None)
+        assert sum(len(b.token_ids) for b in batch) <= s.config.max_num_batched_tokens
+        sampled = self.launch(batch)
+        if s.decodes_only(batch):
+            s.commit_decodes(batch)
+            nxt = s.schedule(now + 0.05) if s.has_unfinished() else []
+            outputs, nxt = s.deliver_tokens(batch, sampled, now, nxt)
+            self.ahead = nxt or None
+            self.used_ahead += 1
+            held = {b.seq.seq_id for b in nxt}
+            if not nxt:
+                check_invariants(s.kv)                # it expects no open reservation
+            assert set(s.kv.seqs) == {q.seq_id for q in s.running}, "exactly the running sequences hold pages"
+            for q in s.running:                       # the same state as after a whole postprocess and a schedule
+                st = s.kv.seqs[q.seq_id]
+                assert q.in_step == (q.seq_id in held) and st.committed == q.num_computed
+                assert -1 not in st.token_ids and -1 not in q.output_token_ids, "no placeholder outlives the delivery"
+                assert st.token_ids == q.all_token_ids[:st.reserved]
+            for b in nxt:
+                assert -1 not in b.token_ids and list(b.token_ids) == b.seq.all_token_ids[b.start:b.start + len(b.token_ids)]
+        else:
+            outputs = s.postprocess(batch, sampled, now)
+            check_scheduler(s)
+        return batch, outputs
+
+
 def unbatched(prompt, params, sample):
     out = [model(prompt, sample)]
     while not ((out[-1] == EOS and not params.ignore_eos) or len(out) == params.max_tokens):
@@ -305,6 +353,61 @@ def test_stats_snapshot_is_a_copy():
 
 
 # ---- random workloads (tests/test_scheduler.py:382-429) -------------------------------------------------
+
+def eos_model(history, sample):
+    """Like `model`, but one draw in six is the end token."""
+    h = hash((tuple(history), sample))
+    return EOS if h % 6 == 0 else h % VOCAB + 2
+
+
+def unbatched_with(token_for, prompt, params, sample):
+    out = [token_for(prompt, sample)]
+    while not ((out[-1] == EOS and not params.ignore_eos) or len(out) == params.max_tokens):
+        out.append(token_for(prompt + out, 0))
+    return out
+
+
+@pytest.mark.parametrize("seed", range(20))
+@pytest.mark.parametrize("caching", [True, False])
+def test_random_workload_with_steps_closed_in_two_halves(seed, caching):
+    """The same workloads with decode steps closed in two halves around the next schedule, and a
+    model that also ends sequences by itself: what was scheduled ahead for a sequence that turns
+    out finished goes back, preempted sequences get their token while they wait."""
+    rng = random.Random(1000 + seed)
+    over = dict(max_num_seqs=rng.choice([2, 4, 8]), max_skip_wait=rng.choice([0.3, 5.0]),
+                max_prefill_chunk=rng.choice([0, 3, 8]), step_mode=rng.choice(["mixed", "mixed", "prefill_first"]))
+    over["max_num_batched_tokens"] = rng.choice([over["max_num_seqs"] + 1, 16, 72])
+    s = make(pages=rng.choice([18, 24, 40]), caching=caching, **over)
+    loop = AheadLoop(s, eos_model)
+    stems = [[2 + rng.randrange(6) for _ in range(rng.randrange(1, 25))] for _ in range(3)]
+    expected, done, now = {}, {}, 0.0
+    arrivals = 14
+    for step_no in range(4000):
+        if arrivals and (rng.random() < 0.3 or not s.has_unfinished()):
+            prompt = rng.choice(stems)[:rng.randrange(1, 25)] + [2 + rng.randrange(6) for _ in range(rng.randrange(0, 6))]
+            params = SamplingParams(max_tokens=rng.randrange(1, 12), n=rng.choice([1, 1, 2, 3]),
+                                    ignore_eos=rng.random() < 0.5)
+            if params.n <= over["max_num_seqs"]:
+                try:
+                    rid = s.add_request(prompt, params, now)
+                    expected[rid] = [unbatched_with(eos_model, prompt, params, k) for k in range(params.n)]
+                except ValueError:
+                    pass
+            arrivals -= 1
+        if not s.has_unfinished():
+            if not arrivals:
+                break
+            continue
+        now += 0.1
+        for o in loop.step(now)[1]:
+            assert o.request_id not in done
+            done[o.request_id] = [q.output_token_ids for q in o.sequences]
+    assert not s.has_unfinished() and loop.ahead is None, "the scheduler stopped making progress"
+    assert done == expected
+    assert loop.used_ahead > 0
+    assert s.kv.stats().blocks_in_use == 0 and not s.kv.seqs
+    assert len(s.kv.free_state_slots) == s.kv.storage.num_state_slots
+
 
 @pytest.mark.parametrize("seed", range(20))
 @pytest.mark.parametrize("caching", [True, False])

@@ -291,6 +291,13 @@ class KVCacheManager:
         assert checked or self.can_append(seq_id, len(token_ids)), "not enough free pages; preempt first"
         self._reserve(seq, token_ids)
 
+    def set_token(self, seq_id: int, position: int, token: int) -> None:
+        """Names the token of a reserved, not yet committed slot whose token was not known when the
+        slot was reserved (pages are published by their tokens, at commit)."""
+        seq = self.seqs[seq_id]
+        assert seq.committed <= position < seq.reserved, "only a reserved slot can still be named"
+        seq.token_ids[position] = token
+
     def commit(self, seq_id: int, num_accepted: int) -> None:
         """Closes a step: keeps the first `num_accepted` slots reserved since the last commit,
         drops the rest, publishes pages that became full, frees pages a window has passed."""

@@ -17,7 +17,8 @@ from tinyserve_llm_amd.cache.storage import KVStorage, bytes_per_page
 from tinyserve_llm_amd.models.decoder import DecoderModel
 from tinyserve_llm_amd.engine.loading import as_dtype, load_model, random_model, require_gpu
 from tinyserve_llm_amd.engine.runner import ModelRunner, StepEntry
-from tinyserve_llm_amd.engine.scheduler import RequestOutput, ScheduledSeq, Scheduler, SchedulerConfig, SchedulerStats
+from tinyserve_llm_amd.engine.scheduler import (PENDING, RequestOutput, ScheduledSeq, Scheduler, SchedulerConfig,
+                                                SchedulerStats)
 from tinyserve_llm_amd.engine.sequence import SamplingParams
 from tinyserve_llm_amd.sampling.sampler import row_key, sample
 
@@ -69,6 +70,7 @@ class LLM:
             random_weights: tuple[object, int] | None = None,   # (typed configuration, seed) instead of a folder
             model: DecoderModel | None = None,       # an already bound model (shares its weights)
             decode_graphs: bool = True,              # replay decode steps from HIP graphs
+            run_ahead: bool = True,                  # schedule and pack the next decode step while this one runs
     ) -> None:
         self.device = require_gpu(cache_config.device if cache_config.device != "cuda" else "cuda:0")
         self.dtype = as_dtype(dtype)
@@ -106,6 +108,8 @@ class LLM:
         self.runner = ModelRunner(self.model, self.storage, self.manager)
         if decode_graphs:
             self.runner.enable_decode_graphs(scheduler_config.max_model_len, scheduler_config.max_num_seqs, self.seed)
+        self.run_ahead = run_ahead
+        self._ahead: tuple | None = None             # (the step scheduled ahead, its packing or None)
         self.steps: list[StepRecord] = []
         logger.info("KV cache: %d blocks of %d tokens", num_blocks, cache_config.block_size)
 
@@ -144,20 +148,27 @@ class LLM:
             raise ValueError(f"prompt holds token ids outside the vocabulary of {vocab}")
         return self.scheduler.add_request(token_ids, params, time.perf_counter() if arrival_time is None else arrival_time)
 
-    def _run(self, batch: list[ScheduledSeq]) -> list[list[int]]:
-        """One forward pass and the draws; one host sync (model_runner.py:120-133)."""
-        entries, temps, keys, owners = [], [], [], []
-        for seq, tokens, num_samples, start in batch:
-            entries.append(StepEntry(seq.seq_id, tokens, start, [len(tokens) - 1] if num_samples else []))
+    def _draws(self, batch: list[ScheduledSeq]) -> tuple[list[float], list[int]]:
+        """Temperature and key of the one draw of every entry (a key names request, sample and
+        output position; a placeholder output already counts as the token it stands for)."""
+        temps = [b.seq.params.temperature for b in batch]
+        keys = [row_key(b.seq.request_id, b.seq.sample_index, len(b.seq.output_token_ids)) for b in batch]
+        return temps, keys
+
+    def _launch(self, batch: list[ScheduledSeq], prepared=None) -> tuple:
+        """Starts one forward pass and the draws on the device (model_runner.py:120-133); `_finish`
+        waits for them."""
+        if prepared is not None:
+            return self.runner.launch_decode(prepared, [b.token_ids[0] for b in batch]), None
+        entries = [StepEntry(seq.seq_id, tokens, start, [len(tokens) - 1] if num_samples else [])
+                   for seq, tokens, num_samples, start in batch]
         if all(b.num_samples == 1 for b in batch):
             # one draw per entry: the step function draws too (decode steps replay one graph for both)
-            for seq, tokens, num_samples, start in batch:
-                temps.append(seq.params.temperature)
-                keys.append(row_key(seq.request_id, seq.sample_index, len(seq.output_token_ids)))
-            return [[t] for t in self.runner.step_sample(entries, temps, keys, self.seed).tolist()]
+            temps, keys = self._draws(batch)
+            return self.runner.step_sample(entries, temps, keys, self.seed), None
         logits = self.runner.step(entries)
+        temps, keys, owners, rows = [], [], [], []
         row = 0
-        rows: list[int] = []
         for seq, tokens, num_samples, start in batch:
             for k in range(num_samples):
                 # the k-th sample of a group's first token; later tokens belong to seq.sample_index
@@ -169,24 +180,59 @@ class LLM:
                 row += 1
             owners.append(num_samples)
         if not rows:
-            torch.cuda.current_stream().synchronize()
-            return [[] for _ in batch]
+            return None, owners
         picked = logits if rows == list(range(logits.shape[0])) else logits[torch.tensor(rows, device=logits.device)]
-        tokens = sample(picked, temps, keys, self.seed).tolist()
+        return sample(picked, temps, keys, self.seed), owners
+
+    def _finish(self, launched: tuple) -> list[list[int]]:
+        """Waits for a launched step; the one host sync of a step. Tokens per entry."""
+        drawn, owners = launched
+        if drawn is None:
+            torch.cuda.current_stream().synchronize()
+            return [[] for _ in owners]
+        tokens = drawn.tolist()
+        if owners is None:
+            return [[t] for t in tokens]
         out, i = [], 0
         for n in owners:
             out.append(tokens[i:i + n])
             i += n
         return out
 
+    def _prepare_ahead(self, ahead: list[ScheduledSeq]):
+        """Packs the next step while the device runs this one, if it is one of decodes only."""
+        if not ahead or not self.scheduler.decodes_only(ahead):
+            return None
+        entries = [StepEntry(b.seq.seq_id, [0 if t == PENDING else t for t in b.token_ids], b.start, [0]) for b in ahead]
+        temps, keys = self._draws(ahead)
+        return self.runner.prepare_decode(entries, temps, keys, self.seed)
+
     def step(self) -> list[RequestOutput]:
+        """One step of the engine. A step of decodes only is closed in two halves around the
+        scheduling and packing of the next step, which so happen while the device is still busy;
+        any other step is scheduled, run and closed in turn."""
         start = time.perf_counter()
-        batch = self.scheduler.schedule(start)
+        batch, prepared = self._ahead if self._ahead is not None else (None, None)
+        self._ahead = None
+        if batch is None:
+            batch = self.scheduler.schedule(start)
         if not batch:
             raise RuntimeError("the scheduler produced an empty step")
-        sampled = self._run(batch)
+        launched = self._launch(batch, prepared)
+        halves = self.run_ahead and self.scheduler.decodes_only(batch)
+        if halves:
+            self.scheduler.commit_decodes(batch)
+            ahead = self.scheduler.schedule(time.perf_counter()) if self.scheduler.has_unfinished() else []
+            prepared = self._prepare_ahead(ahead)
+        sampled = self._finish(launched)
         end = time.perf_counter()
-        outputs = self.scheduler.postprocess(batch, sampled, end)
+        if halves:
+            outputs, left = self.scheduler.deliver_tokens(batch, sampled, end, ahead)
+            if left:
+                # whoever turned out finished has left the step: it is packed again when it runs
+                self._ahead = (left, prepared if len(left) == len(ahead) else None)
+        else:
+            outputs = self.scheduler.postprocess(batch, sampled, end)
         self.steps.append(StepRecord(start, end, len(batch), sum(len(b.token_ids) for b in batch),
                                      self.scheduler.stats(), self.manager.stats()))
         return outputs

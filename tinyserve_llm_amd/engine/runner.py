@@ -247,6 +247,21 @@ class ModelRunner:
         from tinyserve_llm_amd.sampling.sampler import sample
         return sample(self.step(entries), list(temperatures), list(keys), seed)
 
+    def prepare_decode(self, entries: Sequence[StepEntry], temperatures: Sequence[float], keys: Sequence[int],
+                       seed: int):
+        """Checks and packs a decode step with its draws ahead of time, on the host alone, while the
+        device is busy; the entries' token ids may be stand-ins (`launch_decode` takes the real ones).
+        None if the step is not one the decode graphs take."""
+        if self.graphs is not None and self.graphs.seed == seed and self.graphs.takes(entries):
+            return self.graphs.prepare(entries, (temperatures, keys))
+        return None
+
+    @torch.inference_mode()
+    def launch_decode(self, prepared, token_ids: Sequence[int]) -> torch.Tensor:
+        """Starts a step that `prepare_decode` packed, with the entries' token ids now known:
+        the drawn tokens, int32 [entries] on the device."""
+        return self.graphs.launch(prepared, token_ids)
+
     def enable_decode_graphs(self, max_context: int, max_batch: int, seed: int = 0) -> bool:
         """Decode steps (every entry one token whose logits are wanted) are then replayed from HIP
         graphs, one per batch size, instead of being launched kernel by kernel. Only for models
@@ -338,21 +353,37 @@ class DecodeGraphs:
             self.pool = graph.pool()
         return graph, host_i32, dev_i32, logits, tokens
 
-    def run(self, entries: Sequence[StepEntry], draws=None) -> torch.Tensor:
-        """Replays the step's graph. Without `draws` the logits [entries, vocab] come back; with
-        `draws` = (temperatures, keys) the tokens drawn from them, int32 [entries]."""
+    def prepare(self, entries: Sequence[StepEntry], draws=None) -> tuple:
+        """The host half of `run`: checks and packs the step. The entries' token ids may still be
+        placeholders (any id inside the vocabulary); `launch` takes the real ones."""
         size = self._size(len(entries))
         longest = max(e.start + 1 for e in entries)
         reach = min(-(-longest // self.bucket) * self.bucket, -(-self.max_context // self.bucket) * self.bucket)
         width = -(-reach // self.page_size)
-        key = (size, width)
         flat, dims, host = self.runner._pack_decode(entries, [width] * self.num_spaces, pad_to=size)
         words, start = self._with_draws(flat, size, draws)
+        return (size, width), words, start, dims, host, len(entries), draws is not None
+
+    def launch(self, prepared: tuple, token_ids: Sequence[int] | None = None) -> torch.Tensor:
+        """The device half: uploads the packed step (with `token_ids` in the entries' places, if
+        given) and replays its graph. Logits [entries, vocab], or the tokens drawn if the step was
+        prepared with draws."""
+        key, words, start, dims, host, n, drawn = prepared
+        if token_ids is not None:
+            vocab = self.runner.model.spec.vocab_size
+            if len(token_ids) != n or min(token_ids) < 0 or max(token_ids) >= vocab:
+                raise StepError(f"{len(token_ids)} token ids for {n} entries, or one outside the vocabulary of {vocab}")
+            words[:n] = torch.tensor(token_ids, dtype=torch.int32)
         if key not in self.graphs:
-            self.graphs[key] = self._capture(size, words, start, dims, host)
+            self.graphs[key] = self._capture(key[0], words, start, dims, host)
             # the capture recorded the step without running it: the replay below runs it
         graph, host_i32, dev_i32, logits, tokens = self.graphs[key]
         host_i32.copy_(words)
         dev_i32.copy_(host_i32, non_blocking=True)
         graph.replay()
-        return (logits if draws is None else tokens)[:len(entries)]
+        return (tokens if drawn else logits)[:n]
+
+    def run(self, entries: Sequence[StepEntry], draws=None) -> torch.Tensor:
+        """Replays the step's graph. Without `draws` the logits [entries, vocab] come back; with
+        `draws` = (temperatures, keys) the tokens drawn from them, int32 [entries]."""
+        return self.launch(self.prepare(entries, draws))

@@ -7,6 +7,13 @@ uncached tokens (as much as the step's budget and `max_prefill_chunk` allow); a 
 still inside its prompt feeds the next portion each step, after the decodes and before new
 admissions; only the final portion yields a token.
 
+A decode step can be closed in two halves, `commit_decodes` (all that does not depend on the drawn
+tokens) and `deliver_tokens` (all that does), with a `schedule` for the next step in between: the
+engine schedules and packs step n+1 while the device still runs step n. Between the halves a
+sequence's newest output is the placeholder `PENDING`; the next step feeds the placeholder, and
+delivery puts the token in its place (in the sequence, in the scheduled entry and in the cache
+manager's record of the slot).
+
 When pages run out: a running sequence that cannot get the page it needs makes the lowest-ranked
 sequences not yet scheduled in this step give up theirs (preemption: pages released, which keeps
 them in the prefix cache while nobody else needs them; the sequence returns to the waiting queue
@@ -55,6 +62,9 @@ class SchedulerStats:
     decode_tokens: int = 0
     num_waiting: int = 0
     num_running: int = 0
+
+
+PENDING = -1      # stands in for a token that the device has drawn and the host has not read yet
 
 
 class ScheduledSeq(NamedTuple):
@@ -115,6 +125,8 @@ class Scheduler:
     def _ranked_waiting(self, now: float) -> list[tuple[Sequence, float]]:
         ranked = []
         for seq in self.waiting:
+            if seq.output_token_ids and seq.output_token_ids[-1] == PENDING:
+                continue                           # preempted with a token under way: it waits for the token
             tokens = seq.all_token_ids
             hit = self._hit(len(tokens), self.kv.calculate_admission_cost(tokens))
             ranked.append((self._score(hit, seq, now), seq))
@@ -156,6 +168,8 @@ class Scheduler:
             else:
                 if budget <= 0:
                     continue
+                if seq.output_token_ids[-1] == PENDING and len(seq.output_token_ids) >= seq.params.max_tokens:
+                    continue                       # the token under way is its last one
                 tokens = [seq.pending_token]
             fits = self.kv.can_append(seq.seq_id, len(tokens))
             while not fits:
@@ -310,6 +324,65 @@ class Scheduler:
             if all(s.status is SequenceStatus.FINISHED for s in group):
                 outputs.append(RequestOutput(request_id, self.groups.pop(request_id)))
         return outputs
+
+    # ---- the same for decode steps, in two halves -------------------------------------------------
+    @staticmethod
+    def decodes_only(scheduled: list[ScheduledSeq]) -> bool:
+        """Whether every entry of the step feeds one decoded token and draws one."""
+        return all(len(b.token_ids) == 1 and b.num_samples == 1 and b.seq.output_token_ids for b in scheduled)
+
+    def commit_decodes(self, scheduled: list[ScheduledSeq]) -> None:
+        """First half of `postprocess` for a step of decodes only: what does not depend on the
+        tokens drawn. Each sequence's newest output is `PENDING` until `deliver_tokens`."""
+        for seq, token_ids, num_samples, _ in scheduled:
+            assert len(token_ids) == 1 and num_samples == 1 and seq.output_token_ids
+            seq.in_step = False
+            self.kv.commit(seq.seq_id, 1)
+            seq.num_computed += 1
+            seq.prefill_target = seq.num_computed
+            seq.output_token_ids.append(PENDING)
+
+    def deliver_tokens(self, scheduled: list[ScheduledSeq], sampled: list[list[int]], now: float,
+                       ahead: list[ScheduledSeq] | None = None) -> tuple[list[RequestOutput], list[ScheduledSeq]]:
+        """Second half: the drawn tokens take the placeholders' place, what finished is released.
+        `ahead` is the step scheduled in between: its entries that feed a placeholder get the token,
+        entries of sequences that turn out finished are dropped. Returns the finished requests and
+        what is left of `ahead`."""
+        finished: list[Sequence] = []
+        fed_ahead = {b.seq.seq_id: b for b in ahead or ()}
+        for (seq, _, _, _), tokens in zip(scheduled, sampled, strict=True):
+            assert len(tokens) == 1 and seq.output_token_ids[-1] == PENDING
+            token = tokens[0]
+            seq.output_token_ids[-1] = token
+            entry = fed_ahead.get(seq.seq_id)
+            reason = self._finish_reason(seq, token)
+            if reason is None:
+                if entry is not None:
+                    assert entry.token_ids == [PENDING] and entry.start == seq.num_computed
+                    entry.token_ids[0] = token
+                    self.kv.set_token(seq.seq_id, entry.start, token)
+                continue
+            if seq.status is SequenceStatus.RUNNING:
+                if entry is not None:              # scheduled again before anyone knew: the slot goes back
+                    self.kv.commit(seq.seq_id, 0)
+                    seq.in_step = False
+                    del fed_ahead[seq.seq_id]
+                self.kv.release(seq.seq_id)
+            else:                                  # preempted in between: its pages went back then
+                self.waiting = [s for s in self.waiting if s.seq_id != seq.seq_id]
+            seq.status = SequenceStatus.FINISHED
+            seq.finish_reason = reason
+            seq.finish_time = now
+            finished.append(seq)
+        if finished:
+            done = {s.seq_id for s in finished}
+            self.running = [s for s in self.running if s.seq_id not in done]
+        outputs = []
+        for request_id in dict.fromkeys(s.request_id for s in finished):
+            group = self.groups[request_id]
+            if all(s.status is SequenceStatus.FINISHED for s in group):
+                outputs.append(RequestOutput(request_id, self.groups.pop(request_id)))
+        return outputs, [b for b in ahead or () if b.seq.seq_id in fed_ahead]
 
     def stats(self) -> SchedulerStats:
         return replace(self.counters, num_waiting=len(self.waiting), num_running=len(self.running))
