@@ -597,3 +597,56 @@ def test_fused_projection_refuses_what_it_cannot_serve():
     assert not hip().qkv_rope_fuses(torch.zeros(4, 2304, dtype=torch.bfloat16, device=dev()), w, 64, None), "K beyond 2048"
     with pytest.raises(hip().KernelError, match="qkv_rope_store takes"):
         hip().qkv_rope_store(x, w, None, torch.zeros(17, dtype=torch.int32, device=dev()), None, None, None, 1, 1, 64)
+
+
+@pytest.mark.parametrize("heads,kv,hd,page", [(32, 8, 64, 256), (8, 2, 128, 64), (3, 1, 32, 24)])
+def test_split_key_decode_attention_over_a_long_context(heads, kv, hd, page):
+    """Several thousand keys: many chunks per token, several 32-key steps per wave, the plans
+    that `decode_plan` picks for long contexts, and one key far back made to dominate."""
+    dtype = torch.bfloat16
+    n = 5000
+    g = gen(hd + page)
+    q = (torch.randn(4, heads, hd, generator=g) * 0.5).to(dtype)
+    k, v = (torch.randn(n, kv, hd, generator=g) * 0.5).to(dtype), torch.randn(n, kv, hd, generator=g).to(dtype)
+    k[37] = 0
+    k[37, :, 3] = 30.0
+    q[3] = 0
+    q[3, :, 3] = 30.0                                # its score with key 37 stands out by far
+    pages = -(-n // page)
+    table = torch.randperm(pages, generator=g).tolist()
+    kc, vc = engine_layout(k, v, table, page, pages, dtype)
+    rows = [4999, 2047, 1024, 4100]                  # positions of the four queries
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev())
+    want = torch.stack([P.causal_attention(torch.cat([torch.zeros(p, heads, hd, dtype=torch.float64), q[i:i + 1].double()]),
+                                           k[:p + 1].double(), v[:p + 1].double())[-1] for i, p in enumerate(rows)])
+    waves = hip().decode_waves(hd)
+    plans = [(32 * waves, waves), (128 * waves, waves), (1024, 4), hip().decode_plan(4, kv, heads // kv, hd, pages * page)]
+    for chunk, w in plans:
+        out = hip().paged_attention_decode(q.to(dev()), kc, vc, i32([table]), i32([0] * 4), i32(rows), hd ** -0.5,
+                                           chunk=chunk, waves=w)
+        torch.testing.assert_close(out.double().cpu(), want, **tol(dtype), msg=lambda m: f"chunk {chunk}, {w} waves: {m}")
+    for h in range(heads):
+        torch.testing.assert_close(out[3, h].float().cpu(), v[37, h // (heads // kv)].float(), rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("heads,kv,hd,page,row_tiles", [(8, 2, 64, 64, 4), (4, 1, 128, 256, 2), (6, 6, 32, 16, 1)])
+def test_matrix_core_prefill_attention_over_a_long_prompt(heads, kv, hd, page, row_tiles):
+    """A portion of 1,200 tokens over a cached prefix of 333: dozens of 32-key steps per tile, most
+    of them inside every row's range (no mask), long tiles paired with short ones, and a window."""
+    dtype = torch.bfloat16
+    g = gen(hd + 11 * row_tiles)
+    n, fed = 1533, 1200
+    q = (torch.randn(n, heads, hd, generator=g) * 0.5).to(dtype)
+    k, v = (torch.randn(n, kv, hd, generator=g) * 0.5).to(dtype), torch.randn(n, kv, hd, generator=g).to(dtype)
+    pages = -(-n // page)
+    table = torch.randperm(pages, generator=g).tolist()
+    kc, vc = engine_layout(k, v, table, page, pages, dtype)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev())
+    per_tile = row_tiles * hip().PREFILL_WAVES * (16 // (heads // kv))
+    flat = hip().attention_tiles([0, fed], [n - fed], per_tile)
+    positions = list(range(n - fed, n))
+    for window in (0, 200):
+        out = hip().paged_attention_prefill(q[n - fed:].to(dev()), kc, vc, i32([table]), i32([0] * fed), i32(positions),
+                                            i32(flat).view(-1, 2), hd ** -0.5, window=window, tile_tokens=per_tile)
+        want = P.causal_attention(q.double(), k.double(), v.double(), window=window)[n - fed:]
+        torch.testing.assert_close(out.double().cpu(), want, **tol(dtype), msg=lambda m: f"window {window}: {m}")
