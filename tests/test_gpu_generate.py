@@ -261,3 +261,33 @@ def test_steps_closed_in_two_halves_generate_the_same(folder_b, num_blocks):
     assert any("eos" in reasons for _, reasons in outs[0]) and any("length" in reasons for _, reasons in outs[0])
     if num_blocks == 18:
         assert stats[0].preemptions > 0 and stats[1].preemptions > 0
+
+
+def test_streaming_copies_of_the_weights_change_nothing(tmp_path):
+    """Layers may keep their weights once more in the decode kernels' reading order; decode steps
+    read the copies, steps with many rows the weights themselves. Same tokens either way. (A width of
+    256 is the least the weight-streaming kernel takes; the tiny configurations never reach it.)"""
+    from tinyserve_llm_amd.config import LlamaConfig
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+    from tinyserve_llm_amd.weights.random_init import write_random_model
+    config = LlamaConfig(vocab_size=300, hidden_size=256, intermediate_size=512, num_hidden_layers=2,
+                         num_attention_heads=4, num_key_value_heads=2, head_dim=64, max_position_embeddings=256,
+                         rms_norm_eps=1e-5, rope_theta=10000.0, rope_scaling=None, tie_word_embeddings=True, eos_token_id=299)
+    write_random_model(str(tmp_path), config, 4, torch.bfloat16)
+    sc = SchedulerConfig(max_model_len=128, max_num_seqs=8, max_num_batched_tokens=80)
+    prompts = [prompt(90 + i, 4 + 9 * i, 300) for i in range(5)]
+    outs = []
+    for keep in (True, False):
+        llm = LLM(str(tmp_path), sc, CacheConfig(block_size=16), dtype=torch.bfloat16, num_blocks=60, seed=2,
+                  keep_streaming_copies=keep)
+        mixer, ff = llm.model.layers[0].mixer, llm.model.layers[0].feed_forward
+        assert (mixer.qkv_packed is not None) == keep and (mixer.o_packed is not None) == keep
+        assert (ff.gate_up_packed is not None) == keep and (ff.down_packed is not None) == keep
+        outs.append([r.token_ids for r in llm.generate(prompts, SamplingParams(max_tokens=10, temperature=0.7, ignore_eos=True))])
+    assert outs[0] == outs[1]
+    plain = PlainLlama(str(tmp_path), torch.float64)
+    got = LLM(str(tmp_path), sc, CacheConfig(block_size=16), dtype=torch.float32, num_blocks=60).generate(
+        prompts[:2], SamplingParams(max_tokens=6, temperature=0.0, ignore_eos=True))
+    assert [r.token_ids[0] for r in got] == [plain.greedy(p, 6) for p in prompts[:2]]

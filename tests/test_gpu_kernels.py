@@ -650,3 +650,48 @@ def test_matrix_core_prefill_attention_over_a_long_prompt(heads, kv, hd, page, r
                                             i32(flat).view(-1, 2), hd ** -0.5, window=window, tile_tokens=per_tile)
         want = P.causal_attention(q.double(), k.double(), v.double(), window=window)[n - fed:]
         torch.testing.assert_close(out.double().cpu(), want, **tol(dtype), msg=lambda m: f"window {window}: {m}")
+
+
+@pytest.mark.parametrize("m", [1, 8, 16, 23])
+@pytest.mark.parametrize("n,k", [(3072, 2048), (16384, 2048), (992, 512), (130, 3072), (64, 4096), (2048, 8192)])
+def test_weight_streaming_gemm_reads_the_packed_copy_to_the_same_result(m, n, k):
+    """`pack_weight` lays the matrix out in the kernel's reading order; every form of the kernel must
+    give bit for bit what it gives from the matrix itself (a width that is no multiple of 16 ends in
+    a tile padded with zeros)."""
+    g = gen(m + n + k)
+    w = (torch.randn(n, k, generator=g) * 0.05).bfloat16().to(dev())
+    x = torch.randn(m, k, generator=g).bfloat16().to(dev())
+    p = hip().pack_weight(w)
+    assert p.shape == (-(-n // 16), k // 32, 64, 8)
+    assert torch.equal(p[1, 2, 5 + 16 * 3], w[16 + 5, 64 + 24:64 + 32]), "lane r + 16 g: row 16 tile + r, k = 32 step + 8 g .."
+    assert torch.equal(hip().gemm_skinny(x, w, packed=p)[0], hip().gemm_skinny(x, w)[0])
+    assert torch.equal(hip().gemm_skinny(x, w, torch.float32, packed=p)[0], hip().gemm_skinny(x, w, torch.float32)[0])
+    res = torch.randn(m, k, generator=g).bfloat16().to(dev())
+    nw = (1 + 0.1 * torch.randn(k, generator=g)).bfloat16().to(dev())
+    for norm in (False, True):
+        for glu in (False, True):
+            if not (norm or glu) or (glu and n % 32) or not hip().skinny_fuses(m, k, norm, glu):
+                continue
+            kw = dict(residual=res, norm_weight=nw, eps=1e-5) if norm else {}
+            a, b = hip().gemm_skinny(x, w, glu=glu, packed=p, **kw), hip().gemm_skinny(x, w, glu=glu, **kw)
+            assert torch.equal(a[0], b[0]) and (not norm or torch.equal(a[1], b[1]))
+    with pytest.raises(hip().KernelError, match="packed copy"):
+        hip().gemm_skinny(x, w, packed=p[1:])
+
+
+def test_fused_projection_reads_the_packed_copy_to_the_same_result():
+    g = gen(77)
+    nh, nkv, hd, K, M, page = 6, 2, 64, 1024, 7, 16
+    x = torch.randn(M, K, generator=g).bfloat16().to(dev())
+    w = (torch.randn((nh + 2 * nkv) * hd, K, generator=g) * K ** -0.5).bfloat16().to(dev())
+    table = torch.randn(64, hd, generator=g).to(dev())
+    positions = torch.randint(0, 64, (M,), generator=g, dtype=torch.int32).to(dev())
+    slots = torch.randperm(4 * page, generator=g)[:M].to(torch.int32).to(dev())
+    outs = []
+    for packed in (None, hip().pack_weight(w)):
+        kp = torch.zeros(4, nkv, page, hd, dtype=torch.bfloat16, device=dev())
+        vp = torch.zeros(4, nkv, hd, page, dtype=torch.bfloat16, device=dev())
+        q, _ = hip().qkv_rope_store(x, w, table, positions, slots, kp.permute(0, 2, 1, 3), vp.permute(0, 3, 1, 2),
+                                    nh, nkv, hd, packed=packed)
+        outs.append((q, kp, vp))
+    assert all(torch.equal(a, b) for a, b in zip(*outs))

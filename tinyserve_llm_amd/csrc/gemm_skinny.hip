@@ -63,7 +63,7 @@ struct SkinnyArgs {
   bf16_t* res_out;      // MODE_NORM with res: new residual [M, K]
   const bf16_t* w;      // [N, K]
   void* y;              // [M, N]
-  int M, N, K;
+  int M, N, K, packed;
   int64_t ldx, ldw, ldy;
   float eps;
   // EPI_ROPE: N = (nh + 2 nkv) * hd; cos_sin [max_pos, hd] 32-bit, [cos | sin] halves; slot -1 stores nothing.
@@ -140,10 +140,22 @@ gemm_skinny_kernel(const SkinnyArgs a) {
       n = (j / per_head) * a.hd + 16 * (j % per_head) + (t < OT ? 0 : a.hd / 2) + r;
       limit = a.N;
     }
-    if (n >= limit) n = limit - 1;                      // rows past the end are computed and not stored
-    const bf16_t* wrow = a.w + (int64_t)n * a.ldw + kbeg;
+    if (a.packed) {
+      // W in 1 KB blocks [16-row tile][32-wide k step][lane][8 k]: one load of a wave is one
+      // contiguous kilobyte and a wave's slice of a tile a contiguous run of them (rows past N are
+      // zeros in the last tile; tiles past the last are computed from it and not stored)
+      int tile_n = (n - r) / 16;
+      const int last = (a.N - 1) / 16;
+      if (tile_n > last) tile_n = last;
+      const bf16_t* wblk = a.w + (((int64_t)tile_n * (a.K / SK_KSTEP) + (int64_t)wave * STEPS) * 64 + lane) * 8;
 #pragma unroll
-    for (int s = 0; s < STEPS; ++s) wreg[t][s] = *(const uint4*)(wrow + s * SK_KSTEP);
+      for (int s = 0; s < STEPS; ++s) wreg[t][s] = *(const uint4*)(wblk + (int64_t)s * 512);
+    } else {
+      if (n >= limit) n = limit - 1;                    // rows past the end are computed and not stored
+      const bf16_t* wrow = a.w + (int64_t)n * a.ldw + kbeg;
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) wreg[t][s] = *(const uint4*)(wrow + s * SK_KSTEP);
+    }
   }
   // all of W's loads are in flight before anything waits: left to itself the compiler interleaves
   // them with the products to save registers, and the matrix no longer streams at memory speed
@@ -348,11 +360,11 @@ static int sk_dispatch(const SkinnyArgs& a, hipStream_t stream) {
 
 // mode: 0 plain, 1 residual + RMSNorm on the way in (M <= 16, K in steps of 256 up to 4096). glu: W holds
 // gate rows then up rows, y is [M, N / 2] = silu(gate) * up (M <= 16). out_dtype: 1 bfloat16, 0 float
-// (plain only). Requires M <= 32, K a multiple of 256 (up to 4096) or of 512 (up to 8192), contiguous
+// (plain only). packed: w holds the matrix in the kernel's own order (see the loads of W), ldw is unused. Requires M <= 32, K a multiple of 256 (up to 4096) or of 512 (up to 8192), contiguous
 // 16-byte aligned rows; mode 1 takes x, res, res_out as dense [M, K].
 extern "C" int ts_gemm_skinny_bf16(void* y, const void* x, const void* w, const void* res, const void* nw,
                                    void* res_out, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldy,
-                                   float eps, int mode, int glu, int out_dtype, hipStream_t stream) {
+                                   float eps, int mode, int glu, int out_dtype, int packed, hipStream_t stream) {
   if (M <= 0 || N <= 0) return TS_OK;
   if (M > 32 || K <= 0 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ldy < (glu ? N / 2 : N)) return TS_BAD_SHAPE;
   if (glu && (N % 2 || (N / 2) % 16)) return TS_BAD_SHAPE;
@@ -360,7 +372,7 @@ extern "C" int ts_gemm_skinny_bf16(void* y, const void* x, const void* w, const 
   if (mode == MODE_NORM && (!nw || (res && !res_out))) return TS_BAD_SHAPE;
   SkinnyArgs a = {};
   a.x = (const bf16_t*)x; a.res = (const bf16_t*)res; a.nw = (const bf16_t*)nw; a.res_out = (bf16_t*)res_out;
-  a.w = (const bf16_t*)w; a.y = y; a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldw = ldw; a.ldy = ldy; a.eps = eps;
+  a.w = (const bf16_t*)w; a.y = y; a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldw = ldw; a.ldy = ldy; a.eps = eps; a.packed = packed;
   if (out_dtype == 1) {
     if (mode == MODE_PLAIN && !glu) return sk_dispatch<MODE_PLAIN, 0, bf16_t>(a, stream);
     if (mode == MODE_PLAIN && glu) return sk_dispatch<MODE_PLAIN, 1, bf16_t>(a, stream);
@@ -378,7 +390,7 @@ extern "C" int ts_gemm_skinny_bf16(void* y, const void* x, const void* w, const 
 // M <= 16, hd a multiple of 32, K a multiple of 256 up to 2048, 8-byte aligned cache strides.
 extern "C" int ts_gemm_skinny_rope_bf16(void* q_out, const void* x, const void* w, const void* res, const void* nw,
                                         void* res_out, int M, int K, int64_t ldx, int64_t ldw, float eps, int mode,
-                                        const float* cos_sin, const int32_t* positions, const int32_t* slots,
+                                        int packed, const float* cos_sin, const int32_t* positions, const int32_t* slots,
                                         void* k_cache, void* v_cache, int nh, int nkv, int hd, int rotate,
                                         int page_size, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vs,
                                         int64_t vh, int64_t vd, hipStream_t stream) {
@@ -390,10 +402,10 @@ extern "C" int ts_gemm_skinny_rope_bf16(void* q_out, const void* x, const void* 
   if (mode == MODE_NORM && (!nw || (res && !res_out))) return TS_BAD_SHAPE;
   if (rotate && (!cos_sin || !positions)) return TS_BAD_SHAPE;
   if (k_cache && (!v_cache || !slots || (kp % 4) || (ks % 4) || (kh % 4) || (((uintptr_t)k_cache) & 7))) return TS_BAD_SHAPE;
-  SkinnyArgs a;
+  SkinnyArgs a = {};
   a.x = (const bf16_t*)x; a.res = (const bf16_t*)res; a.nw = (const bf16_t*)nw; a.res_out = (bf16_t*)res_out;
   a.w = (const bf16_t*)w; a.y = nullptr; a.M = M; a.N = (nh + 2 * nkv) * hd; a.K = K; a.ldx = ldx; a.ldw = ldw;
-  a.ldy = 0; a.eps = eps;
+  a.ldy = 0; a.eps = eps; a.packed = packed;
   a.cos_sin = cos_sin; a.positions = positions; a.slots = slots; a.q_out = (bf16_t*)q_out;
   a.k_cache = (bf16_t*)k_cache; a.v_cache = (bf16_t*)v_cache; a.nh = nh; a.nkv = nkv; a.hd = hd; a.rotate = rotate;
   a.page_size = page_size; a.kp = kp; a.ks = ks; a.kh = kh; a.vp = vp; a.vs = vs; a.vh = vh; a.vd = vd;

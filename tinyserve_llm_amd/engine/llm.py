@@ -71,6 +71,7 @@ class LLM:
             model: DecoderModel | None = None,       # an already bound model (shares its weights)
             decode_graphs: bool = True,              # replay decode steps from HIP graphs
             run_ahead: bool = True,                  # schedule and pack the next decode step while this one runs
+            keep_streaming_copies: bool | None = None,   # layer weights once more in the decode kernels' order; None: if memory is ample
     ) -> None:
         self.device = require_gpu(cache_config.device if cache_config.device != "cuda" else "cuda:0")
         self.dtype = as_dtype(dtype)
@@ -79,11 +80,11 @@ class LLM:
             self.dtype = model.dtype
         elif random_weights is not None:
             self.config, weight_seed = random_weights
-            self.model = random_model(self.config, weight_seed, self.dtype, self.device)
+            self.model = random_model(self.config, weight_seed, self.dtype, self.device, keep_streaming_copies)
         else:
             if model_path is None:
                 raise ValueError("give a model folder or random_weights=(config, seed)")
-            self.model, self.config = load_model(model_path, self.dtype, self.device)
+            self.model, self.config = load_model(model_path, self.dtype, self.device, keep_streaming_copies)
         spec = self.model.spec
         if scheduler_config.max_model_len > spec.max_position:
             raise ValueError(f"max_model_len {scheduler_config.max_model_len} exceeds the model's "

@@ -124,6 +124,11 @@ class DecoderModel:
             enc.prepare(device)
         self.final_norm.bind(grouped.get("final_norm", {}))
 
+    def keep_streaming_copies(self) -> int:
+        """Lets every part of every layer keep its weights once more in a decode kernel's reading
+        order; returns the bytes that takes."""
+        return sum(part.keep_streaming_copies() for layer in self.layers for part in layer.parts().values())
+
     # ---- one step ----------------------------------------------------------------------------
     def forward(self, ctx: StepContext, memory: list[LayerMemory]) -> tuple[torch.Tensor, torch.Tensor | None]:
         """Runs the step's tokens through every entry of the order; returns the last feed-forward

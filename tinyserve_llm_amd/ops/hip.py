@@ -53,8 +53,8 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_gemm_exact": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_sample": [p, p, p, p, p, p, u64, i, i, i64, p],
         "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, p],
-        "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, p],
-        "ts_gemm_skinny_rope_bf16": [p, p, p, p, p, p, i, i, i64, i64, f, i, p, p, p, p, p, i, i, i, i, i, i64, i64, i64,
+        "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p],
+        "ts_gemm_skinny_rope_bf16": [p, p, p, p, p, p, i, i, i64, i64, f, i, i, p, p, p, p, p, i, i, i, i, i, i64, i64, i64,
                                      i64, i64, i64, i64, p],
     }
     for name, args in sig.items():
@@ -477,6 +477,28 @@ def skinny_takes(rows: int, k: int) -> bool:
     return rows <= SKINNY_MAX_ROWS and ((k % 256 == 0 and k // 256 <= 16) or (k % 512 == 0 and k // 512 <= 16))
 
 
+def pack_weight(weight: torch.Tensor) -> torch.Tensor:
+    """A copy of bfloat16 `weight` [N, K] (K a multiple of 32) in the order the weight-streaming
+    kernel reads it: [N / 16 tiles, K / 32 steps, 64 lanes, 8], lane r + 16 g holding row 16 tile + r,
+    k = 32 step + 8 g .. + 7; rows past N are zeros. Every load of a wave is then one contiguous
+    kilobyte, which streams about a sixth faster than sixteen 64-byte pieces of sixteen rows."""
+    _gpu(weight)
+    _need(weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.shape[1] % 32 == 0,
+          "pack_weight takes bfloat16 [N, K] with K a multiple of 32")
+    n, k = weight.shape
+    tiles = -(-n // 16)
+    padded = weight if n == 16 * tiles else torch.cat([weight, weight.new_zeros(16 * tiles - n, k)])
+    return padded.view(tiles, 16, k // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(tiles, k // 32, 64, 8)
+
+
+def _check_packed(packed: torch.Tensor | None, weight: torch.Tensor) -> None:
+    if packed is not None:
+        n, k = weight.shape
+        _gpu(packed)
+        _need(packed.dtype == torch.bfloat16 and packed.shape == (-(-n // 16), k // 32, 64, 8) and packed.is_contiguous()
+              and packed.data_ptr() % 16 == 0, f"the packed copy does not belong to a weight of {n} x {k}")
+
+
 def skinny_fuses(rows: int, k: int, norm: bool, glu: bool) -> bool:
     """Whether the kernel can apply the norm on the way in and/or the gate on the way out."""
     if not (norm or glu):
@@ -486,11 +508,11 @@ def skinny_fuses(rows: int, k: int, norm: bool, glu: bool) -> bool:
 
 def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, *,
                 residual: torch.Tensor | None = None, norm_weight: torch.Tensor | None = None, eps: float = 0.0,
-                glu: bool = False) -> tuple[torch.Tensor, torch.Tensor | None]:
+                glu: bool = False, packed: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor | None]:
     """bfloat16 e(f(x) [M <= 32, K] · weight [N, K]^T) by the weight-streaming MFMA kernel.
     With `norm_weight`: f = RMSNorm(x + residual) * norm_weight, and x + residual comes back as the
     second result. With `glu`: weight holds gate rows then up rows and the result is
-    silu(gate) * up, [M, N / 2]."""
+    silu(gate) * up, [M, N / 2]. With `packed` (= pack_weight(weight)) the kernel reads that copy."""
     _gpu(x, weight, residual, norm_weight)
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "gemm_skinny takes bfloat16")
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
@@ -504,6 +526,7 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     _need(x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0,
           "rows must be contiguous and 16-byte aligned")
     _need(not glu or (N % 32 == 0), "gate and up rows come in whole 16-row tiles")
+    _check_packed(packed, weight)
     res_out = None
     if norm:
         _need(norm_weight.dtype == torch.bfloat16 and norm_weight.shape == (K,) and norm_weight.is_contiguous(),
@@ -519,9 +542,9 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     _need(out_dtype == torch.bfloat16 or not (norm or glu), "float32 output comes with the plain product only")
     out = torch.empty((M, N // 2 if glu else N), dtype=out_dtype, device=x.device)
     _run("gemm_skinny", library().ts_gemm_skinny_bf16(
-        _ptr(out), _ptr(x), _ptr(weight), _ptr(residual), _ptr(norm_weight),
+        _ptr(out), _ptr(x), _ptr(weight if packed is None else packed), _ptr(residual), _ptr(norm_weight),
         _ptr(res_out) if residual is not None else None, M, N, K, x.stride(0), weight.stride(0), out.stride(0),
-        float(eps), int(norm), int(glu), _code(out_dtype), _stream()))
+        float(eps), int(norm), int(glu), _code(out_dtype), int(packed is not None), _stream()))
     return out, res_out
 
 
@@ -537,17 +560,19 @@ def qkv_rope_fuses(x: torch.Tensor, weight: torch.Tensor, head_dim: int, k_cache
 def qkv_rope_store(x: torch.Tensor, weight: torch.Tensor, cos_sin: torch.Tensor | None, positions: torch.Tensor,
                    slots: torch.Tensor | None, k_cache: torch.Tensor | None, v_cache: torch.Tensor | None,
                    num_heads: int, num_kv_heads: int, head_dim: int, *, residual: torch.Tensor | None = None,
-                   norm_weight: torch.Tensor | None = None, eps: float = 0.0
+                   norm_weight: torch.Tensor | None = None, eps: float = 0.0, packed: torch.Tensor | None = None
                    ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """`rope_store(f(x) · weight^T, ...)` in one kernel for few rows of x: the projection is never
     stored, q [tokens, nh, hd] comes back rotated, rotated k and v go to their cache slots. With
-    `norm_weight`, f = RMSNorm(x + residual) * norm_weight and x + residual is the second result."""
+    `norm_weight`, f = RMSNorm(x + residual) * norm_weight and x + residual is the second result.
+    With `packed` (= pack_weight(weight)) the kernel reads that copy."""
     _gpu(x, weight, cos_sin, positions, slots, k_cache, v_cache, residual, norm_weight)
     _need(qkv_rope_fuses(x, weight, head_dim, k_cache), "qkv_rope_store takes up to 16 bfloat16 rows, K in steps of 256 "
           "up to 2048, head_dim in steps of 32")
     M, K = x.shape
     _need(weight.shape == ((num_heads + 2 * num_kv_heads) * head_dim, K), f"weight {tuple(weight.shape)} for "
           f"{num_heads}+2x{num_kv_heads} heads of {head_dim} over {K}")
+    _check_packed(packed, weight)
     _need(positions.dtype == torch.int32 and positions.shape == (M,) and positions.is_contiguous(),
           "positions must be int32 [tokens]")
     if cos_sin is not None:
@@ -574,16 +599,17 @@ def qkv_rope_store(x: torch.Tensor, weight: torch.Tensor, cos_sin: torch.Tensor 
         _need(residual is None, "a residual comes with a norm weight")
     q = torch.empty((M, num_heads, head_dim), dtype=x.dtype, device=x.device)
     _run("qkv_rope_store", library().ts_gemm_skinny_rope_bf16(
-        _ptr(q), _ptr(x), _ptr(weight), _ptr(residual), _ptr(norm_weight),
+        _ptr(q), _ptr(x), _ptr(weight if packed is None else packed), _ptr(residual), _ptr(norm_weight),
         _ptr(res_out) if residual is not None else None, M, K, x.stride(0), weight.stride(0), float(eps), int(norm),
-        _ptr(cos_sin), _ptr(positions), _ptr(slots), _ptr(k_cache), _ptr(v_cache), num_heads, num_kv_heads, head_dim,
+        int(packed is not None), _ptr(cos_sin), _ptr(positions), _ptr(slots), _ptr(k_cache), _ptr(v_cache), num_heads, num_kv_heads, head_dim,
         int(cos_sin is not None), page_size, *kst, *vst, _stream()))
     return q, res_out
 
 
-def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
-    """bfloat16 x [M, K] · weight [N, K]^T: few rows go to the weight-streaming kernel, many to
-    the vendor matrix library."""
+def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
+                packed: torch.Tensor | None = None) -> torch.Tensor:
+    """bfloat16 x [M, K] · weight [N, K]^T: few rows go to the weight-streaming kernel (which reads
+    `packed`, the weight in its own order, if there is one), many to the vendor matrix library."""
     _gpu(x, weight)
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "linear_bf16 takes bfloat16")
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
@@ -594,6 +620,6 @@ def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     if (skinny_takes(x.shape[0], x.shape[1]) and x.shape[1] <= 4096
             and (x.shape[0] <= SKINNY_FUSED_ROWS or weight.numel() <= SKINNY_WIDE_ELEMENTS)
             and x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
-        return gemm_skinny(x, weight, out_dtype)[0]
+        return gemm_skinny(x, weight, out_dtype, packed=packed)[0]
     y = torch.matmul(x, weight.t())
     return y if out_dtype == torch.bfloat16 else y.to(out_dtype)

@@ -12,7 +12,7 @@ import torch
 
 from tinyserve_llm_amd.ops import hip
 from tinyserve_llm_amd.parts.base import KVSpec, LayerMemory, Mixer, ParamSpec, StepContext, register
-from tinyserve_llm_amd.parts.linear import DeferredNorm, linear
+from tinyserve_llm_amd.parts.linear import DeferredNorm, linear, streaming_copy
 
 
 @register("mixer", "attention")
@@ -35,6 +35,8 @@ class Attention(Mixer):
         self.window = window
         self.qkv: torch.Tensor | None = None
         self.o: torch.Tensor | None = None
+        self.qkv_packed: torch.Tensor | None = None
+        self.o_packed: torch.Tensor | None = None
 
     @property
     def q_size(self) -> int:
@@ -43,6 +45,10 @@ class Attention(Mixer):
     @property
     def kv_size(self) -> int:
         return self.num_kv_heads * self.head_dim
+
+    def keep_streaming_copies(self) -> int:
+        self.qkv_packed, self.o_packed = streaming_copy(self.qkv), streaming_copy(self.o)
+        return sum(t.numel() * t.element_size() for t in (self.qkv_packed, self.o_packed) if t is not None)
 
     def _project_fused(self, x, table, positions, slots, k_store, v_store) -> torch.Tensor | None:
         """Projection, rotation and cache write in one kernel where a step is small enough for the
@@ -53,12 +59,12 @@ class Attention(Mixer):
             return None
         if d is None:
             return hip.qkv_rope_store(rows, self.qkv, table, positions, slots, k_store, v_store, self.num_heads,
-                                      self.num_kv_heads, self.head_dim)[0]
+                                      self.num_kv_heads, self.head_dim, packed=self.qkv_packed)[0]
         if d.weight.dtype != torch.bfloat16 or (d.residual is not None and not d.residual.is_contiguous()):
             return None
         q, d.residual_out = hip.qkv_rope_store(rows, self.qkv, table, positions, slots, k_store, v_store, self.num_heads,
                                                self.num_kv_heads, self.head_dim, residual=d.residual,
-                                               norm_weight=d.weight, eps=d.eps)
+                                               norm_weight=d.weight, eps=d.eps, packed=self.qkv_packed)
         return q
 
     def param_specs(self) -> dict[str, ParamSpec]:
@@ -74,8 +80,8 @@ class Attention(Mixer):
         k_store, v_store = (mem.k_cache, mem.v_cache) if mem.store else (None, None)
         q = self._project_fused(x, table, ctx.positions, slots, k_store, v_store)
         if q is None:
-            qkv = linear(x, self.qkv)
+            qkv = linear(x, self.qkv, packed=self.qkv_packed)
             q = hip.rope_store(qkv, table, ctx.positions, slots, k_store, v_store, self.num_heads, self.num_kv_heads,
                                self.head_dim)
         o = hip.paged_attention(q, mem.k_cache, mem.v_cache, ctx, mem.space, self.scale, self.window)
-        return linear(o.view(ctx.num_tokens, self.q_size), self.o)
+        return linear(o.view(ctx.num_tokens, self.q_size), self.o, packed=self.o_packed)

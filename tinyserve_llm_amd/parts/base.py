@@ -107,6 +107,12 @@ class Part:
         for name, tensor in params.items():
             setattr(self, name, tensor)
 
+    def keep_streaming_copies(self) -> int:
+        """Optionally keeps second copies of weights in the order a decode kernel reads them
+        (`parts.linear.streaming_copy`), to hand to `linear(..., packed=)`; returns the bytes they
+        take. Called after `bind` when memory allows. The default keeps none."""
+        return 0
+
 
 class Norm(Part):
     def __call__(self, x: torch.Tensor, residual: torch.Tensor | None = None,

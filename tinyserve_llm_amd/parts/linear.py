@@ -36,26 +36,38 @@ def _streams(x: torch.Tensor, weight: torch.Tensor) -> bool:
             and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
 
 
+def streaming_copy(weight: torch.Tensor) -> torch.Tensor | None:
+    """The weight once more in the order the weight-streaming kernel reads it, for a part to keep
+    beside the weight and hand to `linear` (decode steps read it, steps with many rows read the
+    weight itself through the library); None where that kernel would never take the weight."""
+    if (weight.is_cuda and weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous()
+            and hip.skinny_takes(1, weight.shape[1]) and weight.shape[1] <= 4096):
+        return hip.pack_weight(weight)
+    return None
+
+
 def linear(x: torch.Tensor | DeferredNorm, weight: torch.Tensor, out_dtype: torch.dtype | None = None,
-           glu: bool = False) -> torch.Tensor:
-    """x · Wᵀ; with `glu`, W holds gate rows then up rows and silu(gate) * up comes back."""
+           glu: bool = False, packed: torch.Tensor | None = None) -> torch.Tensor:
+    """x · Wᵀ; with `glu`, W holds gate rows then up rows and silu(gate) * up comes back.
+    `packed` is `streaming_copy(weight)` if the part keeps one."""
     if isinstance(x, DeferredNorm):
         d = x
         if (out_dtype in (None, torch.bfloat16) and _streams(d.x, weight) and d.weight.dtype == torch.bfloat16
                 and (d.residual is None or d.residual.is_contiguous())
                 and hip.skinny_fuses(d.x.shape[0], weight.shape[1], True, glu) and (not glu or weight.shape[0] % 32 == 0)):
-            y, d.residual_out = hip.gemm_skinny(d.x, weight, residual=d.residual, norm_weight=d.weight, eps=d.eps, glu=glu)
+            y, d.residual_out = hip.gemm_skinny(d.x, weight, residual=d.residual, norm_weight=d.weight, eps=d.eps, glu=glu,
+                                                packed=packed)
             return y
         x = d.materialize()
     if glu:
         if (out_dtype in (None, torch.bfloat16) and _streams(x, weight) and weight.shape[0] % 32 == 0
                 and hip.skinny_fuses(x.shape[0], weight.shape[1], False, True)):
-            return hip.gemm_skinny(x, weight, glu=True)[0]
-        return hip.silu_mul(linear(x, weight, out_dtype))
+            return hip.gemm_skinny(x, weight, glu=True, packed=packed)[0]
+        return hip.silu_mul(linear(x, weight, out_dtype, packed=packed))
     if x.dtype == torch.float32:
         return hip.gemm_exact(x, weight, out_dtype)
     if x.dtype != torch.bfloat16:
         raise hip.KernelError(f"linear: no path for {x.dtype}")
     if not x.is_cuda:
         raise hip.KernelError("linear: GPU tensors only; there is no CPU path")
-    return hip.linear_bf16(x, weight, out_dtype or torch.bfloat16)
+    return hip.linear_bf16(x, weight, out_dtype or torch.bfloat16, packed)

@@ -6,7 +6,7 @@ from __future__ import annotations
 import torch
 
 from tinyserve_llm_amd.parts.base import FeedForward, ParamSpec, StepContext, register
-from tinyserve_llm_amd.parts.linear import linear
+from tinyserve_llm_amd.parts.linear import linear, streaming_copy
 
 
 @register("feed_forward", "gated_mlp")
@@ -21,10 +21,16 @@ class GatedMLP(FeedForward):
         self.intermediate_size = intermediate_size
         self.gate_up: torch.Tensor | None = None
         self.down: torch.Tensor | None = None
+        self.gate_up_packed: torch.Tensor | None = None
+        self.down_packed: torch.Tensor | None = None
 
     def param_specs(self) -> dict[str, ParamSpec]:
         return {"gate_up": ParamSpec((2 * self.intermediate_size, self.hidden_size)),
                 "down": ParamSpec((self.hidden_size, self.intermediate_size))}
 
+    def keep_streaming_copies(self) -> int:
+        self.gate_up_packed, self.down_packed = streaming_copy(self.gate_up), streaming_copy(self.down)
+        return sum(t.numel() * t.element_size() for t in (self.gate_up_packed, self.down_packed) if t is not None)
+
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
-        return linear(linear(x, self.gate_up, glu=True), self.down)
+        return linear(linear(x, self.gate_up, glu=True, packed=self.gate_up_packed), self.down, packed=self.down_packed)
