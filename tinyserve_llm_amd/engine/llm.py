@@ -1,6 +1,7 @@
 """The engine loop and the Python entry point: LLM(path).generate(prompts, SamplingParams(...))
 (tinyserve_llm/engine/llm_engine.py:26-185). schedule -> run the step -> sample -> postprocess,
-until nothing is waiting or running."""
+until nothing is waiting or running. Decode steps overlap with the host: while the device runs
+one, the next is already scheduled and packed (see `LLM.step`)."""
 
 from __future__ import annotations
 

@@ -4,6 +4,8 @@ tinyserve_llm/engine/model_runner.py:100-108, tinyserve_llm/attention/torch_page
 One fused projection gives q | k | v; q and k are rotated by the named position encoding; k and v
 of the step's tokens are written to their cache slots; then every token attends, causally, over
 the cache pages of its request (its own key included), and the output projection follows.
+For steps of up to 16 tokens projection, rotation and cache write are one kernel
+(`hip.qkv_rope_store`), which also takes a deferred norm; larger steps run them one after the other.
 """
 
 from __future__ import annotations
