@@ -5,6 +5,13 @@
 A "step" is one decode step of the whole engine (scheduler, step function, kernels, sampling) at
 batch 8 with 2,048-token contexts that grow while decoding. Prints ONE JSON line. The same line
 carries the 2,048-token prefill, the decode step's HBM roofline, and decode at batch 1 and 64.
+
+    python bench.py --scenario requests-3b | chunked-8b [--layers L]
+
+runs a whole workload through `LLM.generate` instead and prints one JSON line of its own: many
+requests that arrive together, at the layer sizes of Llama 3.2 3B (prompts of 512 to 4,096 tokens, a
+quarter of them behind a common 1,024-token prefix, prefix cache on) or of Llama 3.1 8B (8,192-token
+contexts whose prompts are fed in portions of 2,048 tokens beside the decoding requests).
 """
 
 from __future__ import annotations
@@ -30,6 +37,91 @@ SHAPE = dict(vocab_size=128256, hidden_size=2048, intermediate_size=8192, num_at
 ROPE = dict(factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=8192)
 PROMPT_LEN, MAX_MODEL_LEN, PAGE = 2048, 4096, 256
 
+# whole workloads: layer sizes, requests, and how the scheduler is set for them
+SCENARIOS = {
+    "requests-3b": dict(
+        model="llama-3.2-3b-shape", layers_full=28, rope_factor=32.0,
+        shape=dict(vocab_size=128256, hidden_size=3072, intermediate_size=8192, num_attention_heads=24,
+                   num_key_value_heads=8, head_dim=128, max_position_embeddings=131072, rms_norm_eps=1e-5,
+                   rope_theta=500000.0, tie_word_embeddings=True),
+        requests=64, prompt=(512, 4096), shared=(0.25, 1024), decode=256, budget=8192, chunk=0, caching=True),
+    "chunked-8b": dict(
+        model="llama-3.1-8b-shape", layers_full=32, rope_factor=8.0,
+        shape=dict(vocab_size=128256, hidden_size=4096, intermediate_size=14336, num_attention_heads=32,
+                   num_key_value_heads=8, head_dim=128, max_position_embeddings=131072, rms_norm_eps=1e-5,
+                   rope_theta=500000.0, tie_word_embeddings=False),
+        requests=32, prompt=(7936, 7936), shared=(0.0, 0), decode=256, budget=2048 + 32, chunk=2048, caching=False),
+}
+
+
+def scenario(name: str, layers: int | None, dtype_name: str) -> int:
+    """One workload from first request to last token through `LLM.generate`; one JSON line."""
+    import torch
+
+    from tinyserve_llm_amd.config import LlamaConfig, RopeScaling
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.loading import random_model
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+
+    w = SCENARIOS[name]
+    layers = layers or w["layers_full"]
+    config = LlamaConfig(num_hidden_layers=layers, rope_scaling=RopeScaling(**{**ROPE, "factor": w["rope_factor"]}),
+                         **w["shape"])
+    dtype = torch.bfloat16 if dtype_name == "bf16" else torch.float32
+    model = random_model(config, 0, dtype, "cuda:0")
+    rng = random.Random(0)
+    lo, hi = w["prompt"]
+    share, prefix_len = w["shared"]
+    prefix = [rng.randrange(config.vocab_size) for _ in range(prefix_len)]
+    prompts = []
+    for i in range(w["requests"]):
+        n = rng.randint(lo, hi)
+        head = prefix if i < share * w["requests"] and n > prefix_len else []
+        prompts.append(head + [rng.randrange(config.vocab_size) for _ in range(n - len(head))])
+    rng.shuffle(prompts)
+    max_len = hi + w["decode"]
+    pages = sum(-(-(len(p) + w["decode"]) // PAGE) for p in prompts) + 8
+    sc = SchedulerConfig(max_model_len=max_len, max_num_seqs=w["requests"], max_num_batched_tokens=w["budget"],
+                         max_prefill_chunk=w["chunk"])
+    sp = SamplingParams(max_tokens=w["decode"], temperature=0.0, ignore_eos=True)
+
+    def run(subset) -> tuple[float, LLM]:
+        llm = LLM(None, sc, CacheConfig(block_size=PAGE, caching=w["caching"]), dtype=dtype, num_blocks=pages,
+                  seed=0, model=model)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        llm.generate(subset, sp)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0, llm
+
+    run(prompts[:2])                                   # libraries pick their kernels, graphs are captured
+    seconds, llm = run(prompts)
+    st, cs = llm.scheduler.stats(), llm.manager.stats()
+    portions = [r for r in llm.steps if r.num_tokens > r.num_seqs]
+    decodes = [r for r in llm.steps if r.num_tokens == r.num_seqs]
+    prompt_tokens = sum(len(p) for p in prompts)
+    record = {
+        "metric": f"tokens/s of a whole workload ({name})", "value": (prompt_tokens + st.decode_tokens) / seconds,
+        "unit": "tokens/s", "n_gpus": 1, "seconds": seconds, "steps": len(llm.steps), "higher_is_better": True,
+        "dtype": dtype_name, "data": "synthetic uniform token ids, random weights N(0,0.02)",
+        "output_tokens_per_s": st.decode_tokens / seconds, "prompt_tokens": prompt_tokens,
+        "prefilled_tokens": st.prefill_tokens, "cached_tokens": st.cached_tokens, "output_tokens": st.decode_tokens,
+        "preemptions": st.preemptions, "evictions": cs.evictions,
+        "steps_with_prompt_portions": {"steps": len(portions), "seconds": sum(r.end - r.start for r in portions),
+                                       "tokens": sum(r.num_tokens for r in portions)},
+        "steps_of_decodes_only": {"steps": len(decodes), "seconds": sum(r.end - r.start for r in decodes),
+                                  "tokens": sum(r.num_tokens for r in decodes)},
+        "config": {"model": w["model"], "layers": layers, "layers_full": w["layers_full"],
+                   "hidden": config.hidden_size, "heads": config.num_attention_heads,
+                   "kv_heads": config.num_key_value_heads, "head_dim": config.head_dim,
+                   "intermediate": config.intermediate_size, "vocab": config.vocab_size, "requests": w["requests"],
+                   "prompt_min": lo, "prompt_max": hi, "shared_prefix": prefix_len, "decode_tokens": w["decode"],
+                   "token_budget": w["budget"], "prefill_chunk": w["chunk"], "page_size": PAGE, "pages": pages},
+    }
+    print(json.dumps(record))
+    return 0
+
 
 def main() -> int:
     ap = argparse.ArgumentParser()
@@ -37,16 +129,21 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS)
+    ap.add_argument("--layers", type=int, default=None)
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--points", default="1,64", help="further decode batch sizes (comma-separated; '' for none)")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--only", default="all", choices=["all", "prefill"],
                     help="'prefill': time the 2,048-token prefill alone and print its record (for profiling)")
+    ap.add_argument("--scenario", default=None, choices=sorted(SCENARIOS),
+                    help="run a whole workload through LLM.generate instead of the decode step")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
         return 2
+    if args.scenario:
+        return scenario(args.scenario, args.layers, args.dtype)
+    args.layers = args.layers or FULL_LAYERS
 
     import torch
 

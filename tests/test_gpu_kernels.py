@@ -257,7 +257,8 @@ def test_split_key_decode_attention(heads, kv, hd, page, chunk, waves):
 
 
 @pytest.mark.parametrize("heads,kv,hd,page", [(3, 1, 32, 16), (6, 2, 96, 8), (32, 8, 64, 256), (5, 5, 128, 32),
-                                              (16, 1, 128, 64), (14, 2, 64, 24)])
+                                              (16, 1, 128, 64), (14, 2, 64, 24), (12, 6, 32, 16), (32, 16, 64, 64),
+                                              (8, 4, 96, 32), (24, 12, 32, 8)])
 @pytest.mark.parametrize("row_tiles", [1, 2, 4])
 def test_matrix_core_prefill_attention(heads, kv, hd, page, row_tiles):
     """A packed step of three requests on shared pools: a whole prompt, a portion over a cached

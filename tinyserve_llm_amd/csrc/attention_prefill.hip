@@ -12,8 +12,11 @@
 //
 // The host lists the tiles: tiles[2 i] = index of the tile's first token in the step,
 // tiles[2 i + 1] = number of its tokens (at most 4 RT (16 / G), all of one request), in ascending
-// order of the number of keys a tile walks. Workgroup b takes tile n - 1 - b and then tile b, a long
-// one and a short one, so that all workgroups have about the same work.
+// order of the number of keys a tile walks. There is one workgroup per (key/value head, tile), and
+// the long tiles start first. The chip hands consecutive workgroups to its eight dies in turn, and
+// each die has a cache of its own, so the kernel maps workgroups to work such that those which walk
+// one head's keys sit on as few dies as possible: with eight heads (or a multiple) each die works
+// on heads of its own and reads their keys from memory once.
 #include "attention_mfma.h"
 
 #define PRE_WAVES 4
@@ -210,21 +213,19 @@ __global__ void __launch_bounds__(PRE_WAVES * TS_WAVE)
 attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
                          const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables,
                          const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ positions,
-                         const int32_t* __restrict__ tiles, int num_tiles, int nh, int G, int page_size,
-                         int page_shift, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd,
-                         int max_blocks, float scale2, int window) {
+                         const int32_t* __restrict__ tiles, int num_tiles, int nh, int G, int dies_per_group,
+                         int heads_per_group, int page_size, int page_shift, int64_t kp, int64_t ks, int64_t kh,
+                         int64_t vp, int64_t vh, int64_t vd, int max_blocks, float scale2, int window) {
   __shared__ PrefillLds<HD> lds;
-  const int b = blockIdx.x, kvh = blockIdx.y;
-  const int far = num_tiles - 1 - b;             // b <= far by the size of the grid
-#define TS_TILE(I)                                                                                              \
-  prefill_tile<HD, RT>(lds, I, kvh, out, q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, nh, \
-                       G, page_size, page_shift, kp, ks, kh, vp, vh, vd, max_blocks, scale2, window)
-  TS_TILE(far);
-  if (b < far) {
-    __syncthreads();                             // the first tile's last reads of LDS are done
-    TS_TILE(b);
-  }
-#undef TS_TILE
+  // die = workgroup index mod 8. The dies form `groups` groups of `dies_per_group`, the heads as
+  // many groups of `heads_per_group`; a group's (tile, head) pairs go round its dies, long tiles first.
+  const int die = blockIdx.x % 8, turn = blockIdx.x / 8;
+  const int item = turn * dies_per_group + die % dies_per_group;
+  if (item >= num_tiles * heads_per_group) return;
+  const int tile = num_tiles - 1 - item / heads_per_group;
+  const int kvh = (die / dies_per_group) * heads_per_group + item % heads_per_group;
+  prefill_tile<HD, RT>(lds, tile, kvh, out, q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, nh,
+                       G, page_size, page_shift, kp, ks, kh, vp, vh, vd, max_blocks, scale2, window);
 }
 
 // Keys: rows dense in head_dim, strides kp/ks/kh (page, slot, head). Values: transposed pages,
@@ -239,7 +240,7 @@ extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* 
   if (num_tiles <= 0) return TS_OK;
   if (nkv <= 0 || nh % nkv || page_size <= 0 || page_size % 8 || max_blocks <= 0) return TS_BAD_SHAPE;
   const int G = nh / nkv;
-  if (G > 16 || nkv > 65535) return TS_BAD_SHAPE;
+  if (G > 16) return TS_BAD_SHAPE;
   const int per_wave = PRE_WAVES * (16 / G);
   if (tile_tokens != per_wave && tile_tokens != 2 * per_wave && tile_tokens != 4 * per_wave) return TS_BAD_SHAPE;
   const int rt = tile_tokens / per_wave;
@@ -250,12 +251,17 @@ extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* 
     page_shift = 0;
     while ((1 << page_shift) < page_size) ++page_shift;
   }
-  dim3 grid((num_tiles + 1) / 2, nkv);
+  int groups = 8;                                   // gcd(nkv, 8)
+  while (nkv % groups) groups /= 2;
+  const int dies_per_group = 8 / groups, heads_per_group = nkv / groups;
+  const int64_t turns = ((int64_t)num_tiles * heads_per_group + dies_per_group - 1) / dies_per_group;
+  if (turns * 8 > 0x7fffffff) return TS_BAD_SHAPE;
+  dim3 grid((unsigned)(8 * turns));
 #define TS_PRE(HH, RR)                                                                                          \
   attn_prefill_mfma_kernel<HH, RR><<<grid, PRE_WAVES * TS_WAVE, 0, stream>>>(                                   \
       (bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,             \
-      seq_of_token, positions, tiles, num_tiles, nh, G, page_size, page_shift, kp, ks, kh, vp, vh, vd,          \
-      max_blocks, scale * 1.44269504088896340736f, window)
+      seq_of_token, positions, tiles, num_tiles, nh, G, dies_per_group, heads_per_group, page_size, page_shift, kp,  \
+      ks, kh, vp, vh, vd, max_blocks, scale * 1.44269504088896340736f, window)
 #define TS_PRE_RT(HH)                                                                                           \
   if (rt == 1) TS_PRE(HH, 1); else if (rt == 2) TS_PRE(HH, 2); else TS_PRE(HH, 4)
   switch (hd) {

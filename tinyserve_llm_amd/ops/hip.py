@@ -370,16 +370,18 @@ def _out_like(q: torch.Tensor, out: torch.Tensor | None) -> torch.Tensor:
 
 
 PREFILL_WAVES = 4            # waves of a workgroup of the prefill kernel; each holds 1, 2 or 4 row tiles
-PREFILL_MIN_WORKGROUPS = 512 # larger tiles only while this many workgroups remain
+PREFILL_MIN_WORKGROUPS = 1024     # four row tiles per wave only while four workgroups per compute unit remain
+PREFILL_WIDE_HEAD_DIM = 64        # and only up to this head size
 
 
-def prefill_tile_tokens(num_tokens: int, nkv: int, group: int) -> int:
-    """Tokens per tile of the prefill kernel: as many row tiles per wave (4, 2 or 1) as still leave
-    the chip two workgroups per compute unit (a workgroup takes two tiles)."""
+def prefill_tile_tokens(num_tokens: int, nkv: int, group: int, head_dim: int) -> int:
+    """Tokens per tile of the prefill kernel. One row tile per wave, so that a step becomes many
+    workgroups, except for large steps with small heads: there four row tiles per wave, which read
+    the keys a quarter as often, measured faster (8,192 tokens at head size 64: 506 µs against 537;
+    at head size 128 the small tiles win at every size)."""
     per_wave = PREFILL_WAVES * (16 // group)
-    for rt in (4, 2):
-        if -(-num_tokens // (2 * rt * per_wave)) * nkv >= PREFILL_MIN_WORKGROUPS:
-            return rt * per_wave
+    if head_dim <= PREFILL_WIDE_HEAD_DIM and -(-num_tokens // (4 * per_wave)) * nkv >= PREFILL_MIN_WORKGROUPS:
+        return 4 * per_wave
     return per_wave
 
 
@@ -452,7 +454,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         while decode_ok and lead + 1 < len(cu) and cu[lead + 1] - cu[lead] == 1:
             lead += 1
         nkv = k_cache.shape[2]
-        tile_tokens = prefill_tile_tokens(q.shape[0] - lead, nkv, q.shape[1] // nkv)
+        tile_tokens = prefill_tile_tokens(q.shape[0] - lead, nkv, q.shape[1] // nkv, q.shape[2])
         tiles = ctx.scratch.get(("attention_tiles", tile_tokens, lead))
         if tiles is None:
             flat = attention_tiles(cu, ctx.host_starts, tile_tokens, lead)
