@@ -17,6 +17,7 @@
 // each die has a cache of its own, so the kernel maps workgroups to work such that those which walk
 // one head's keys sit on as few dies as possible: with eight heads (or a multiple) each die works
 // on heads of its own and reads their keys from memory once.
+#include <type_traits>
 #include "attention_mfma.h"
 
 #define PRE_WAVES 4
@@ -24,7 +25,7 @@
 template <int HD>
 struct PrefillLds {
   uint4 stage[2][HD / 8][TS_WAVE];   // two steps of operand registers, [register][lane]
-  int range[2][PRE_WAVES];
+  int range[4][PRE_WAVES];
 };
 
 template <int HD, int RT>
@@ -60,11 +61,13 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
     lmin = min(lmin, ok ? lo[j] : 0x7fffffff);
   }
   // per row tile: the smallest position and largest window start of its rows (wave-uniform)
-  int tile_pmin[RT], tile_lomax[RT], tile_pmax[RT], tile_lomin[RT];
+  // (tile_vpmin: the smallest position among the rows that exist; rows that do not are never stored)
+  int tile_lomax[RT], tile_pmax[RT], tile_lomin[RT], tile_vpmin[RT];
 #pragma unroll
   for (int j = 0; j < RT; ++j) {
-    tile_pmin[j] = pos[j]; tile_lomax[j] = lo[j]; tile_pmax[j] = pos[j];
+    tile_lomax[j] = lo[j]; tile_pmax[j] = pos[j];
     tile_lomin[j] = tk[j] >= 0 ? lo[j] : 0x7fffffff;
+    tile_vpmin[j] = tk[j] >= 0 ? pos[j] : 0x7fffffff;
   }
 #pragma unroll
   for (int off = 1; off < TS_WAVE; off <<= 1) {
@@ -72,24 +75,33 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
     lmin = min(lmin, __shfl_xor(lmin, off, TS_WAVE));
 #pragma unroll
     for (int j = 0; j < RT; ++j) {
-      tile_pmin[j] = min(tile_pmin[j], __shfl_xor(tile_pmin[j], off, TS_WAVE));
+      tile_vpmin[j] = min(tile_vpmin[j], __shfl_xor(tile_vpmin[j], off, TS_WAVE));
       tile_pmax[j] = max(tile_pmax[j], __shfl_xor(tile_pmax[j], off, TS_WAVE));
       tile_lomax[j] = max(tile_lomax[j], __shfl_xor(tile_lomax[j], off, TS_WAVE));
       tile_lomin[j] = min(tile_lomin[j], __shfl_xor(tile_lomin[j], off, TS_WAVE));
     }
   }
-  // the workgroup's key range
-  if (lane == 0) { wg_range[0][wave] = lmin; wg_range[1][wave] = pmax; }
-  __syncthreads();
-  int wlo = wg_range[0][0], whi = wg_range[1][0];
+  // the workgroup's key range [wlo, whi], and the range every one of its rows sees whole: [wfull_lo, wfull_hi]
+  if (lane == 0) {
+    int pmin = 0x7fffffff, lomax = 0;
 #pragma unroll
-  for (int w = 1; w < PRE_WAVES; ++w) { wlo = min(wlo, wg_range[0][w]); whi = max(whi, wg_range[1][w]); }
+    for (int j = 0; j < RT; ++j) { pmin = min(pmin, tile_vpmin[j]); lomax = max(lomax, tile_lomax[j]); }
+    wg_range[0][wave] = lmin; wg_range[1][wave] = pmax; wg_range[2][wave] = pmin; wg_range[3][wave] = lomax;
+  }
+  __syncthreads();
+  int wlo = wg_range[0][0], whi = wg_range[1][0], wfull_hi = wg_range[2][0], wfull_lo = wg_range[3][0];
+#pragma unroll
+  for (int w = 1; w < PRE_WAVES; ++w) {
+    wlo = min(wlo, wg_range[0][w]); whi = max(whi, wg_range[1][w]);
+    wfull_hi = min(wfull_hi, wg_range[2][w]); wfull_lo = max(wfull_lo, wg_range[3][w]);
+  }
   // every lane holds the same values: say so, and loop control and page lookups become scalar
   wlo = __builtin_amdgcn_readfirstlane(wlo);
   whi = __builtin_amdgcn_readfirstlane(whi);
+  wfull_lo = __builtin_amdgcn_readfirstlane(wfull_lo);
+  wfull_hi = __builtin_amdgcn_readfirstlane(wfull_hi);
 #pragma unroll
   for (int j = 0; j < RT; ++j) {
-    tile_pmin[j] = __builtin_amdgcn_readfirstlane(tile_pmin[j]);
     tile_pmax[j] = __builtin_amdgcn_readfirstlane(tile_pmax[j]);
     tile_lomax[j] = __builtin_amdgcn_readfirstlane(tile_lomax[j]);
     tile_lomin[j] = __builtin_amdgcn_readfirstlane(tile_lomin[j]);
@@ -166,13 +178,16 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
 
   const int kbeg = wlo & ~31;
   const int kend = whi + 1;
-  if (kbeg < kend) {                         // uniform over the workgroup
-    fetch(kbeg);
-    put(0);
-    if (kbeg + 32 < kend) fetch(kbeg + 32);
-    __syncthreads();
-    int buf = 0;
-    for (int kb = kbeg; kb < kend; kb += 32, buf ^= 1) {
+  // The walk has three stretches: steps that some row sees in part (before the last window start),
+  // steps that every row of the workgroup sees whole, and the steps around the rows' own positions.
+  // The middle one, nearly all of a long walk, runs without masks and without the test whether a
+  // tile has anything to do; each stretch is a loop of its own so that the accumulators stay in
+  // their registers from one step to the next.
+  const int full_lo = min(max((wfull_lo + 31) & ~31, kbeg), kend);
+  const int full_hi = min(max(wfull_hi == 0x7fffffff ? 0 : ((wfull_hi + 1) & ~31), full_lo), kend);
+  int buf = 0;
+  auto walk = [&](int from, int to, auto masked) {
+    for (int kb = from; kb < to; kb += 32, buf ^= 1) {
       KVTile<HD> T;
 #pragma unroll
       for (int c = 0; c < NC; ++c) { T.k[0][c] = stage[buf][c][lane]; T.k[1][c] = stage[buf][NC + c][lane]; }
@@ -181,12 +196,26 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
       if (kb + 32 < kend) put(buf ^ 1);      // the other buffer was last read before the previous barrier
       if (kb + 64 < kend) fetch(kb + 64);
 #pragma unroll
-      for (int j = 0; j < RT; ++j)
-        // a step wholly beyond the tile's last position, or wholly before all its windows, has nothing for it
-        if (kb <= tile_pmax[j] && kb + 31 >= tile_lomin[j])
-          use_tile_auto<HD>(T, kb, r, g, lo[j], pos[j], tile_pmin[j], tile_lomax[j], qreg[j], scale2, m[j], l[j], o[j]);
+      for (int j = 0; j < RT; ++j) {
+        if constexpr (decltype(masked)::value) {
+          // a step wholly beyond the tile's last position, or wholly before all its windows, has nothing for it
+          if (kb <= tile_pmax[j] && kb + 31 >= tile_lomin[j])
+            use_tile<HD, true>(T, kb, r, g, lo[j], pos[j], qreg[j], scale2, m[j], l[j], o[j]);
+        } else {
+          use_tile<HD, false>(T, kb, r, g, lo[j], pos[j], qreg[j], scale2, m[j], l[j], o[j]);
+        }
+      }
       __syncthreads();
     }
+  };
+  if (kbeg < kend) {                         // uniform over the workgroup
+    fetch(kbeg);
+    put(0);
+    if (kbeg + 32 < kend) fetch(kbeg + 32);
+    __syncthreads();
+    walk(kbeg, full_lo, std::true_type{});
+    walk(full_lo, full_hi, std::false_type{});
+    walk(full_hi, kend, std::true_type{});
   }
   // output row 4 g + i of row tile j: its token and head; its sum sits in lane 4 g + i
   float lsum[RT];

@@ -370,18 +370,26 @@ def _out_like(q: torch.Tensor, out: torch.Tensor | None) -> torch.Tensor:
 
 
 PREFILL_WAVES = 4            # waves of a workgroup of the prefill kernel; each holds 1, 2 or 4 row tiles
-PREFILL_MIN_WORKGROUPS = 1024     # four row tiles per wave only while four workgroups per compute unit remain
-PREFILL_WIDE_HEAD_DIM = 64        # and only up to this head size
+PREFILL_TWO_TILES_WORKGROUPS = 512      # two row tiles per wave while this many workgroups remain (two per compute unit)
+PREFILL_FOUR_TILES_WORKGROUPS = 2048    # four while this many remain,
+PREFILL_FOUR_TILES_HEAD_DIM = 64        # and only up to this head size (beyond it the accumulators crowd the registers)
 
 
 def prefill_tile_tokens(num_tokens: int, nkv: int, group: int, head_dim: int) -> int:
-    """Tokens per tile of the prefill kernel. One row tile per wave, so that a step becomes many
-    workgroups, except for large steps with small heads: there four row tiles per wave, which read
-    the keys a quarter as often, measured faster (8,192 tokens at head size 64: 506 µs against 537;
-    at head size 128 the small tiles win at every size)."""
+    """Tokens per tile of the prefill kernel. A wave that holds two or four row tiles works on them
+    side by side and reads each key once for all of them, which is faster as long as the step still
+    makes enough workgroups to fill the chip (measured: 2,048 tokens over 6,144 cached ones at head
+    size 128 take 534 / 295 / 375 µs with 1 / 2 / 4 row tiles per wave; 512 tokens over 1,536 at
+    head size 64 take 36 / 46 / 66 µs; 16,384 tokens at head size 64 take 1.89 / 1.33 / 1.23 ms)."""
     per_wave = PREFILL_WAVES * (16 // group)
-    if head_dim <= PREFILL_WIDE_HEAD_DIM and -(-num_tokens // (4 * per_wave)) * nkv >= PREFILL_MIN_WORKGROUPS:
+
+    def workgroups(rt: int) -> int:
+        return -(-num_tokens // (rt * per_wave)) * nkv
+
+    if head_dim <= PREFILL_FOUR_TILES_HEAD_DIM and workgroups(4) >= PREFILL_FOUR_TILES_WORKGROUPS:
         return 4 * per_wave
+    if workgroups(2) >= PREFILL_TWO_TILES_WORKGROUPS:
+        return 2 * per_wave
     return per_wave
 
 
