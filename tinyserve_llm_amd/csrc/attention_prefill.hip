@@ -135,18 +135,25 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
       const int64_t page = table[pg];
       const int slot = pm.slot(kb, pg);
       const bool inner = kb >= wlo && kb + 31 <= whi;
+      const bf16_t* src;              // this lane's first piece; the others follow at a fixed stride
+      int64_t stride;
+      bool ok;
       if (wave < 2) {
         const int koff = 8 * (r >> 2) + 4 * wave + (r & 3);
-        const bf16_t* kr = k_cache + page * kp + (int64_t)slot * ks + (int64_t)kvh * kh + (int64_t)koff * ks + 8 * g;
-        const bool ok = inner || (kb + koff <= whi && kb + koff >= wlo);
-#pragma unroll
-        for (int c = 0; c < NC; ++c) fetched[c] = ok ? *(const uint4*)(kr + 32 * c) : make_uint4(0, 0, 0, 0);
+        src = k_cache + page * kp + (int64_t)slot * ks + (int64_t)kvh * kh + (int64_t)koff * ks + 8 * g;
+        stride = 32;
+        ok = kb + koff <= whi && kb + koff >= wlo;
       } else {
-        const bf16_t* vr = v_cache + page * vp + slot + (int64_t)kvh * vh + 8 * g +
-                           (int64_t)((wave - 2) * NC * 16 + r) * vd;
-        const bool ok = inner || (kb + 8 * g <= whi && kb + 8 * g + 7 >= wlo);
+        src = v_cache + page * vp + slot + (int64_t)kvh * vh + 8 * g + (int64_t)((wave - 2) * NC * 16 + r) * vd;
+        stride = 16 * vd;
+        ok = kb + 8 * g <= whi && kb + 8 * g + 7 >= wlo;
+      }
+      if (inner) {                    // nearly every step: nothing to leave out, nothing to clear
 #pragma unroll
-        for (int c = 0; c < NC; ++c) fetched[c] = ok ? *(const uint4*)(vr + (int64_t)(16 * c) * vd) : make_uint4(0, 0, 0, 0);
+        for (int c = 0; c < NC; ++c) fetched[c] = *(const uint4*)(src + c * stride);
+      } else {
+#pragma unroll
+        for (int c = 0; c < NC; ++c) fetched[c] = ok ? *(const uint4*)(src + c * stride) : make_uint4(0, 0, 0, 0);
       }
       return;
     }
