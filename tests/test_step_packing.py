@@ -55,6 +55,32 @@ def test_decode_packing_equals_general_packing(windows):
         assert a[0] == b[0] and a[1] == b[1] and a[2] == b[2]
 
 
+def test_general_packing_lays_out_portions_of_prompts():
+    """Tokens, positions, request of each token, lengths, wanted rows, padded block tables and the
+    cache slot of every token (page * page size + place in the page), for portions that start
+    inside a page, cross pages and end at a page's edge, beside a single decoded token."""
+    ps = 8
+    tables = [{1: [5, 2, 9], 2: [7, 0, 3, 6], 3: [4]}]
+    r = runner(ps, [16], (0,), tables, {1: 2, 2: 0, 3: 1})
+    entries = [StepEntry(1, list(range(20, 31)), 6, [10]),        # positions 6..16: three pages
+               StepEntry(2, [50], 25, [0]),                       # one decoded token, fourth page
+               StepEntry(3, list(range(60, 68)), 0, [0, 7])]      # a whole page, to its edge
+    flat, (T, S, R, widths, offsets, slot_offset), host = r._pack(entries)
+    assert (T, S, R, widths) == (20, 3, 4, [4])
+    ids = list(range(20, 31)) + [50] + list(range(60, 68))
+    positions = list(range(6, 17)) + [25] + list(range(8))
+    seq_of = [0] * 11 + [1] + [2] * 8
+    assert flat[:T] == ids and flat[T:2 * T] == positions and flat[2 * T:3 * T] == seq_of
+    assert flat[3 * T:3 * T + 4] == [0, 11, 12, 20] == host["cu"]
+    assert flat[3 * T + 4:3 * T + 7] == [17, 26, 8] == host["ctx_lens"]
+    assert flat[3 * T + 7:3 * T + 10] == [2, 0, 1]
+    assert flat[3 * T + 10:3 * T + 14] == [10, 11, 12, 19]
+    assert flat[offsets[0]:offsets[0] + 12] == [5, 2, 9, 0, 7, 0, 3, 6, 4, 0, 0, 0]
+    table_of = {0: tables[0][1], 1: tables[0][2], 2: tables[0][3]}
+    want = [table_of[s][p // ps] * ps + p % ps for s, p in zip(seq_of, positions)]
+    assert flat[slot_offset:slot_offset + T] == want and len(flat) == slot_offset + T
+
+
 def test_decode_packing_refuses_what_the_general_packing_refuses():
     r = runner(16, [8], (0,), [{1: [3, 9]}], {1: 0})
     for bad in ([StepEntry(1, [100], 5, [0])], [StepEntry(1, [5], 40, [0])], [StepEntry(1, [5], 20, [0])],

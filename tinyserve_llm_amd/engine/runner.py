@@ -11,6 +11,7 @@ logits [wanted, vocab] in the order of the entries and of their `want` lists.
 from __future__ import annotations
 
 import struct
+from array import array
 from dataclasses import dataclass, field
 from typing import Protocol, Sequence
 
@@ -114,7 +115,12 @@ class ModelRunner:
                 if n == 1:
                     slot_maps[sp].append(table[e.start // ps] * ps + e.start % ps)
                 else:
-                    slot_maps[sp].extend(table[p // ps] * ps + p % ps for p in range(e.start, end))
+                    p = e.start
+                    while p < end:                       # page by page: consecutive positions, consecutive slots
+                        page, stop = p // ps, min(end, (p // ps + 1) * ps)
+                        base = table[page] * ps - page * ps
+                        slot_maps[sp].extend(range(base + p, base + stop))
+                        p = stop
             cu.append(cu[-1] + n)
         for s in range(len(entries), pad_to):           # idle rows of a fixed-size batch
             ids.append(0)
@@ -219,7 +225,8 @@ class ModelRunner:
         """Packs a step into device tensors; returns (context, wanted rows, number of wanted rows).
         Everything a kernel will index with is checked here first."""
         flat, dims, host = self._pack(entries)
-        packed = torch.tensor(flat, dtype=torch.int32).to(self.device, non_blocking=True)
+        # (a list goes into an int32 tensor fastest through the array module)
+        packed = torch.frombuffer(array("i", flat), dtype=torch.int32).to(self.device, non_blocking=True)
         ctx, rows = self._context(packed, dims, host)
         return ctx, rows, dims[2]
 
