@@ -291,3 +291,32 @@ def test_streaming_copies_of_the_weights_change_nothing(tmp_path):
     got = LLM(str(tmp_path), sc, CacheConfig(block_size=16), dtype=torch.float32, num_blocks=60).generate(
         prompts[:2], SamplingParams(max_tokens=6, temperature=0.0, ignore_eos=True))
     assert [r.token_ids[0] for r in got] == [plain.greedy(p, 6) for p in prompts[:2]]
+
+
+def test_recorded_steps_with_library_products_replay_what_eager_steps_compute(tmp_path):
+    """Above 32 requests a decode step's projections go to the vendor's matrix library, inside the
+    recorded graph as well. In bfloat16 the graph's replays (several, with prompts run eagerly in
+    between, and again in a second round of requests) must give the tokens of the engine that runs
+    every step eagerly: the same kernels on the same numbers."""
+    from tinyserve_llm_amd.config import LlamaConfig
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+    from tinyserve_llm_amd.weights.random_init import write_random_model
+    config = LlamaConfig(vocab_size=300, hidden_size=256, intermediate_size=512, num_hidden_layers=2,
+                         num_attention_heads=4, num_key_value_heads=2, head_dim=64, max_position_embeddings=256,
+                         rms_norm_eps=1e-5, rope_theta=10000.0, rope_scaling=None, tie_word_embeddings=True, eos_token_id=299)
+    write_random_model(str(tmp_path), config, 6, torch.bfloat16)
+    sc = SchedulerConfig(max_model_len=96, max_num_seqs=48, max_num_batched_tokens=256)
+    prompts = [prompt(300 + i, 3 + i % 11, 300) for i in range(44)]
+    params = [SamplingParams(max_tokens=5 + i % 7, temperature=0.0, ignore_eos=True) for i in range(44)]
+    outs = []
+    for graphs in (True, False):
+        llm = LLM(str(tmp_path), sc, CacheConfig(block_size=16), dtype=torch.bfloat16, num_blocks=300, seed=1,
+                  decode_graphs=graphs)
+        outs.append([r.token_ids for r in llm.generate(prompts, params)])
+        if graphs:
+            sizes = sorted({size for size, width in llm.runner.graphs.graphs})
+            assert max(sizes) > 32, f"a batch above 32 requests was recorded: {sizes}"
+            assert [r.token_ids for r in llm.generate(prompts, params)] == outs[0]
+    assert outs[0] == outs[1]

@@ -406,6 +406,25 @@ def test_linear_bfloat16(m, n, k):
     assert f.dtype == torch.float32
 
 
+@pytest.mark.parametrize("m,n,k", [(33, 384, 96), (2056, 16384, 2048), (100, 1000, 160), (257, 130, 3072), (64, 128256, 512)])
+def test_library_product_called_directly(m, n, k):
+    """x · W^T through the vendor's library with the algorithm kept per shape: against 64-bit, twice
+    (the second call takes the kept plan), and with rows of x that lie apart in memory."""
+    g = gen(m + n + k)
+    a, w = torch.randn(m, 2 * k, generator=g).bfloat16(), (torch.randn(n, k, generator=g) * 0.05).bfloat16()
+    want = a[:, :k].double() @ w.double().T
+    tolerance = dict(rtol=2e-2, atol=2e-2 * float(want.abs().max()))
+    ad, wd = a.to(dev()), w.to(dev())
+    dense = ad[:, :k].contiguous()
+    for _ in range(2):
+        out = hip().gemm_library(dense, wd)
+        assert out.dtype == torch.bfloat16 and out.shape == (m, n)
+        torch.testing.assert_close(out.double().cpu(), want, **tolerance)
+    torch.testing.assert_close(hip().gemm_library(ad[:, :k], wd).float(), out.float(), rtol=0, atol=0)
+    with pytest.raises(hip().KernelError):
+        hip().gemm_library(ad.t()[:k].t()[:, ::2], wd[:, ::2])      # elements of a row must be adjacent
+
+
 @pytest.mark.parametrize("m", [1, 3, 8, 16, 17, 32])
 @pytest.mark.parametrize("n,k", [(3072, 2048), (2048, 2048), (16384, 2048), (2048, 8192), (992, 512), (130, 3072), (64, 4096)])
 def test_weight_streaming_gemm_and_its_fused_inputs(m, n, k):

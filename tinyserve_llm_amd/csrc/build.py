@@ -32,13 +32,17 @@ FLAGS = [
 ]
 
 
+# the vendor's matrix library, which gemm_library.hip calls for products with many rows
+LINK = ["-lhipblaslt"]
+
+
 def sources() -> list[str]:
     return sorted(f for f in os.listdir(HERE) if f.endswith(".hip"))
 
 
 def source_hash() -> str:
     h = hashlib.sha256()
-    h.update(" ".join(FLAGS).encode())
+    h.update(" ".join(FLAGS + LINK).encode())
     for name in sorted(f for f in os.listdir(HERE) if f.endswith((".hip", ".h"))):
         h.update(name.encode())
         with open(os.path.join(HERE, name), "rb") as f:
@@ -128,7 +132,7 @@ def build(verbose: bool = True, force: bool = True) -> str:
         raise RuntimeError("hipcc failed:\n" + "\n".join(errors))
     lib = os.path.join(out_dir, LIB_NAME)
     tmp = lib + f".tmp{os.getpid()}"
-    cmd = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", *objs, "-o", tmp]
+    cmd = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", *objs, *LINK, "-o", tmp]
     r = subprocess.run(cmd, capture_output=True, text=True, env=env)
     if r.returncode:
         raise RuntimeError(f"link failed: {' '.join(cmd)}\n{r.stdout}{r.stderr}")

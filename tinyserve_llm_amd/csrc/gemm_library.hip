@@ -1,0 +1,132 @@
+// y[M, N] = x[M, K] · W[N, K]^T in bfloat16 with 32-bit accumulation for many rows of x, through the
+// vendor's matrix library (hipBLASLt), called directly: the descriptors and the algorithm the
+// library's heuristic picks for a shape are made once and kept, so that a call costs little more
+// than the launch (a framework's general matmul asks the heuristic again at every call, which is
+// most of its 20 µs on the host, and that is what bounds steps of a few hundred tokens).
+// Row-major y = x · W^T is, in the library's column-major terms, y^T = W^T-as-stored transposed
+// times x^T-as-stored: A = W with op T (K x N, leading dimension ldw), B = x with op N (K x M,
+// leading dimension ldx), D = y (N x M, leading dimension ldy).
+#include <hipblaslt/hipblaslt.h>
+
+#include <map>
+#include <mutex>
+#include <tuple>
+
+#include "common.h"
+
+namespace {
+
+constexpr size_t LT_WORKSPACE_BYTES = 128u << 20;  // what the library may use per device, allocated once
+constexpr int LT_MAX_DEVICES = 16;
+constexpr size_t LT_MAX_PLANS = 8192;              // per device; a serving process meets many row counts
+
+struct LtPlan {
+  hipblasLtMatmulDesc_t desc = nullptr;
+  hipblasLtMatrixLayout_t a = nullptr, b = nullptr, d = nullptr;
+  hipblasLtMatmulAlgo_t algo;
+  size_t workspace = 0;
+};
+
+struct LtDevice {
+  hipblasLtHandle_t handle = nullptr;
+  void* workspace = nullptr;
+  std::map<std::tuple<int, int, int, int64_t, int64_t, int64_t>, LtPlan> plans;
+};
+
+std::mutex lt_mutex;
+LtDevice lt_devices[LT_MAX_DEVICES];
+
+// The plan for a shape on the current device; made (and the library asked for its best algorithm)
+// the first time the shape is met. Returns null if the library has nothing for it.
+const LtPlan* lt_plan(LtDevice& dev, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldy) {
+  const auto key = std::make_tuple(M, N, K, ldx, ldw, ldy);
+  auto it = dev.plans.find(key);
+  if (it != dev.plans.end()) return it->second.desc ? &it->second : nullptr;
+  if (dev.plans.size() >= LT_MAX_PLANS) {   // start over rather than grow without bound
+    for (auto& kv : dev.plans) {
+      if (!kv.second.desc) continue;
+      hipblasLtMatrixLayoutDestroy(kv.second.a);
+      hipblasLtMatrixLayoutDestroy(kv.second.b);
+      hipblasLtMatrixLayoutDestroy(kv.second.d);
+      hipblasLtMatmulDescDestroy(kv.second.desc);
+    }
+    dev.plans.clear();
+  }
+  LtPlan plan;
+  bool ok = hipblasLtMatmulDescCreate(&plan.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) == HIPBLAS_STATUS_SUCCESS;
+  const hipblasOperation_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
+  ok = ok && hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta)) == HIPBLAS_STATUS_SUCCESS;
+  ok = ok && hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &tb, sizeof(tb)) == HIPBLAS_STATUS_SUCCESS;
+  ok = ok && hipblasLtMatrixLayoutCreate(&plan.a, HIP_R_16BF, K, N, ldw) == HIPBLAS_STATUS_SUCCESS;
+  ok = ok && hipblasLtMatrixLayoutCreate(&plan.b, HIP_R_16BF, K, M, ldx) == HIPBLAS_STATUS_SUCCESS;
+  ok = ok && hipblasLtMatrixLayoutCreate(&plan.d, HIP_R_16BF, N, M, ldy) == HIPBLAS_STATUS_SUCCESS;
+  hipblasLtMatmulPreference_t pref = nullptr;
+  ok = ok && hipblasLtMatmulPreferenceCreate(&pref) == HIPBLAS_STATUS_SUCCESS;
+  const uint64_t limit = LT_WORKSPACE_BYTES;
+  ok = ok && hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &limit, sizeof(limit)) == HIPBLAS_STATUS_SUCCESS;
+  // the library's candidates come best first, whatever workspace they want: the first that fits is taken
+  constexpr int LT_CANDIDATES = 16;
+  hipblasLtMatmulHeuristicResult_t found[LT_CANDIDATES];
+  int count = 0, pick = -1;
+  ok = ok && hipblasLtMatmulAlgoGetHeuristic(dev.handle, plan.desc, plan.a, plan.b, plan.d, plan.d, pref, LT_CANDIDATES, found, &count) == HIPBLAS_STATUS_SUCCESS;
+  for (int i = 0; ok && i < count && pick < 0; ++i)
+    if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize <= LT_WORKSPACE_BYTES) pick = i;
+  ok = ok && pick >= 0;
+  if (pref) hipblasLtMatmulPreferenceDestroy(pref);
+  if (ok) {
+    plan.algo = found[pick].algo;
+    plan.workspace = found[pick].workspaceSize;
+  } else {
+    if (plan.a) hipblasLtMatrixLayoutDestroy(plan.a);
+    if (plan.b) hipblasLtMatrixLayoutDestroy(plan.b);
+    if (plan.d) hipblasLtMatrixLayoutDestroy(plan.d);
+    if (plan.desc) hipblasLtMatmulDescDestroy(plan.desc);
+    plan = LtPlan();                        // remembered as "nothing for this shape"
+  }
+  auto& kept = dev.plans[key];
+  kept = plan;
+  return kept.desc ? &kept : nullptr;
+}
+
+}  // namespace
+
+// The current device's handle and workspace; made at the first call on the device.
+static LtDevice* lt_device() {
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= LT_MAX_DEVICES) return nullptr;
+  LtDevice& dev = lt_devices[device];
+  if (!dev.handle) {
+    if (hipblasLtCreate(&dev.handle) != HIPBLAS_STATUS_SUCCESS) { dev.handle = nullptr; return nullptr; }
+    if (hipMalloc(&dev.workspace, LT_WORKSPACE_BYTES) != hipSuccess) {
+      hipblasLtDestroy(dev.handle);
+      dev.handle = nullptr;
+      return nullptr;
+    }
+  }
+  return &dev;
+}
+
+// Makes the current device's library handle and workspace (128 MB, kept until the process ends).
+// The products below do it themselves at their first call; a caller that will record them into a
+// graph calls this beforehand, since memory cannot be allocated while a stream is captured.
+extern "C" int ts_gemm_library_init() {
+  std::lock_guard<std::mutex> guard(lt_mutex);
+  return lt_device() ? TS_OK : TS_LAUNCH_FAILED;
+}
+
+// y, x, w bfloat16; rows of x, w and y are ldx, ldw, ldy elements apart (each at least the row's
+// length). The stream may be one that is being captured into a graph (after ts_gemm_library_init).
+extern "C" int ts_gemm_library_bf16(void* y, const void* x, const void* w, int M, int N, int K, int64_t ldx,
+                                    int64_t ldw, int64_t ldy, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return TS_OK;
+  if (K <= 0 || ldx < K || ldw < K || ldy < N || !y || !x || !w) return TS_BAD_SHAPE;
+  std::lock_guard<std::mutex> guard(lt_mutex);
+  LtDevice* dev = lt_device();
+  if (!dev) return TS_LAUNCH_FAILED;
+  const LtPlan* plan = lt_plan(*dev, M, N, K, ldx, ldw, ldy);
+  if (!plan) return TS_BAD_SHAPE;
+  const float one = 1.0f, zero = 0.0f;
+  const hipblasStatus_t st = hipblasLtMatmul(dev->handle, plan->desc, &one, w, plan->a, x, plan->b, &zero, y, plan->d, y,
+                                             plan->d, &plan->algo, dev->workspace, LT_WORKSPACE_BYTES, stream);
+  return st == HIPBLAS_STATUS_SUCCESS ? TS_OK : TS_LAUNCH_FAILED;
+}

@@ -300,6 +300,8 @@ class DecodeGraphs:
         self.graphs: dict[int, tuple] = {}
         self.pool = None
         self.seed = seed                  # of the draws the graphs hold
+        from tinyserve_llm_amd.ops import hip
+        hip.gemm_library_init()           # its workspace cannot be allocated while a graph is recorded
 
     def _size(self, n: int) -> int:
         return n if n <= 8 or not self.can_pad else -(-n // 8) * 8

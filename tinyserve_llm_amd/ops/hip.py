@@ -52,6 +52,8 @@ def _declare(lib: ctypes.CDLL) -> None:
                                       i, p],
         "ts_gemm_exact": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_sample": [p, p, p, p, p, p, u64, i, i, i64, p],
+        "ts_gemm_library_bf16": [p, p, p, i, i, i, i64, i64, i64, p],
+        "ts_gemm_library_init": [],
         "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, p],
         "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p],
         "ts_gemm_skinny_rope_bf16": [p, p, p, p, p, p, i, i, i64, i64, f, i, i, p, p, p, p, p, i, i, i, i, i, i64, i64, i64,
@@ -63,7 +65,13 @@ def _declare(lib: ctypes.CDLL) -> None:
         fn.restype = ctypes.c_int
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    """The current stream's handle (the short way where torch has it: a launch asks for it every time)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -631,5 +639,24 @@ def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
             and (x.shape[0] <= SKINNY_FUSED_ROWS or weight.numel() <= SKINNY_WIDE_ELEMENTS)
             and x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
         return gemm_skinny(x, weight, out_dtype, packed=packed)[0]
-    y = torch.matmul(x, weight.t())
+    y = gemm_library(x, weight)
     return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
+
+
+def gemm_library_init() -> None:
+    """Makes the matrix library's handle and workspace on the current device. Steps that are recorded
+    into graphs need it done beforehand (the runner does it when it is made)."""
+    _run("gemm_library_init", library().ts_gemm_library_init())
+
+
+def gemm_library(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """bfloat16 x [M, K] · weight [N, K]^T by the vendor's matrix library, called directly with the
+    algorithm it picked for the shape the first time (see gemm_library.hip). Rows may be strided."""
+    _need(x.stride(1) == 1 and weight.stride(1) == 1, "rows of x and of the weight must be dense")
+    M, K = x.shape
+    N = weight.shape[0]
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    if M and N:
+        _run("gemm_library", library().ts_gemm_library_bf16(_ptr(y), _ptr(x), _ptr(weight), M, N, K, x.stride(0),
+                                                            weight.stride(0), N, _stream()))
+    return y
