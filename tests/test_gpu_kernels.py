@@ -652,7 +652,8 @@ def test_split_key_decode_attention_over_a_long_context(heads, kv, hd, page):
 @pytest.mark.parametrize("heads,kv,hd,page,row_tiles", [(8, 2, 64, 64, 4), (4, 1, 128, 256, 2), (6, 6, 32, 16, 1)])
 def test_matrix_core_prefill_attention_over_a_long_prompt(heads, kv, hd, page, row_tiles):
     """A portion of 1,200 tokens over a cached prefix of 333: dozens of 32-key steps per tile, most
-    of them inside every row's range (no mask), long tiles paired with short ones, and a window."""
+    of them inside every row's range (the loop without masks), the steps before a window's start and
+    around the rows' own positions in the masked loops, long tiles first."""
     dtype = torch.bfloat16
     g = gen(hd + 11 * row_tiles)
     n, fed = 1533, 1200
