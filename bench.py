@@ -224,7 +224,7 @@ def main() -> int:
     step_bytes = weight_bytes + args.batch * mean_ctx * kv_bytes_per_token
     achieved = step_bytes / (seconds / args.steps)
     record = {
-        "metric": "decode tok/s at batch 8 (Llama-3.2-1B shape, 2,048-token contexts)",
+        "metric": f"decode tok/s at batch {args.batch} (Llama-3.2-1B shape, 2,048-token contexts)",
         "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": 1e3 * seconds / args.steps, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": args.dtype, "data": "synthetic uniform token ids, random weights N(0,0.02)",

@@ -3,6 +3,12 @@
 // library's heuristic picks for a shape are made once and kept, so that a call costs little more
 // than the launch (a framework's general matmul asks the heuristic again at every call, which is
 // most of its 20 µs on the host, and that is what bounds steps of a few hundred tokens).
+// For products with few rows (decode steps of 33 to 256 requests) the heuristic's first candidate is
+// often not the fastest (measured at 64 rows with weights read from memory, the layer sizes of a 1B
+// Llama: qkv 12.0 µs against 8.9 for the best candidate, o 11.8 against 8.8, down 23.2 against
+// 15.5), so a caller may ask for such a shape to be tuned: every candidate is timed on the call's
+// own operands, with the caches swept in between as they are when a step reads each weight once,
+// and the fastest is kept.
 // Row-major y = x · W^T is, in the library's column-major terms, y^T = W^T-as-stored transposed
 // times x^T-as-stored: A = W with op T (K x N, leading dimension ldw), B = x with op N (K x M,
 // leading dimension ldx), D = y (N x M, leading dimension ldy).
@@ -19,12 +25,17 @@ namespace {
 constexpr size_t LT_WORKSPACE_BYTES = 128u << 20;  // what the library may use per device, allocated once
 constexpr int LT_MAX_DEVICES = 16;
 constexpr size_t LT_MAX_PLANS = 8192;              // per device; a serving process meets many row counts
+constexpr int LT_CANDIDATES = 16;                  // asked of the heuristic for a plan,
+constexpr int LT_TUNE_CANDIDATES = 48;             // and when a shape is tuned
+constexpr int LT_TUNE_MAX_ROWS = 256;              // shapes with more rows keep the heuristic's choice
+constexpr int LT_TUNE_RUNS = 3;                    // timed runs per candidate; the fastest counts
 
 struct LtPlan {
   hipblasLtMatmulDesc_t desc = nullptr;
   hipblasLtMatrixLayout_t a = nullptr, b = nullptr, d = nullptr;
   hipblasLtMatmulAlgo_t algo;
   size_t workspace = 0;
+  bool tuned = false;
 };
 
 struct LtDevice {
@@ -38,7 +49,7 @@ LtDevice lt_devices[LT_MAX_DEVICES];
 
 // The plan for a shape on the current device; made (and the library asked for its best algorithm)
 // the first time the shape is met. Returns null if the library has nothing for it.
-const LtPlan* lt_plan(LtDevice& dev, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldy) {
+LtPlan* lt_plan(LtDevice& dev, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldy) {
   const auto key = std::make_tuple(M, N, K, ldx, ldw, ldy);
   auto it = dev.plans.find(key);
   if (it != dev.plans.end()) return it->second.desc ? &it->second : nullptr;
@@ -65,7 +76,6 @@ const LtPlan* lt_plan(LtDevice& dev, int M, int N, int K, int64_t ldx, int64_t l
   const uint64_t limit = LT_WORKSPACE_BYTES;
   ok = ok && hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &limit, sizeof(limit)) == HIPBLAS_STATUS_SUCCESS;
   // the library's candidates come best first, whatever workspace they want: the first that fits is taken
-  constexpr int LT_CANDIDATES = 16;
   hipblasLtMatmulHeuristicResult_t found[LT_CANDIDATES];
   int count = 0, pick = -1;
   ok = ok && hipblasLtMatmulAlgoGetHeuristic(dev.handle, plan.desc, plan.a, plan.b, plan.d, plan.d, pref, LT_CANDIDATES, found, &count) == HIPBLAS_STATUS_SUCCESS;
@@ -86,6 +96,51 @@ const LtPlan* lt_plan(LtDevice& dev, int M, int N, int K, int64_t ldx, int64_t l
   auto& kept = dev.plans[key];
   kept = plan;
   return kept.desc ? &kept : nullptr;
+}
+
+// Times the library's candidates for the plan's shape on the operands of this call and keeps the
+// fastest. Before every timed run `flush_bytes` at `flush` are overwritten, which empties the caches
+// of the weights. Synchronizes with the stream; never called while it is being captured.
+void lt_tune(LtDevice& dev, LtPlan& plan, void* y, const void* x, const void* w, void* flush, size_t flush_bytes,
+             hipStream_t stream) {
+  plan.tuned = true;
+  hipblasLtMatmulPreference_t pref = nullptr;
+  if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return;
+  const uint64_t limit = LT_WORKSPACE_BYTES;
+  hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &limit, sizeof(limit));
+  hipblasLtMatmulHeuristicResult_t found[LT_TUNE_CANDIDATES];
+  int count = 0;
+  const bool listed = hipblasLtMatmulAlgoGetHeuristic(dev.handle, plan.desc, plan.a, plan.b, plan.d, plan.d, pref,
+                                                      LT_TUNE_CANDIDATES, found, &count) == HIPBLAS_STATUS_SUCCESS;
+  hipblasLtMatmulPreferenceDestroy(pref);
+  hipEvent_t begin = nullptr, end = nullptr;
+  if (!listed || hipEventCreate(&begin) != hipSuccess || hipEventCreate(&end) != hipSuccess) {
+    if (begin) hipEventDestroy(begin);
+    return;
+  }
+  const float one = 1.0f, zero = 0.0f;
+  float best = -1.0f;
+  for (int i = 0; i < count; ++i) {
+    if (found[i].state != HIPBLAS_STATUS_SUCCESS || found[i].workspaceSize > LT_WORKSPACE_BYTES) continue;
+    float fastest = -1.0f;
+    for (int run = 0; run <= LT_TUNE_RUNS; ++run) {         // the first run is not timed
+      if (flush && flush_bytes && hipMemsetAsync(flush, run, flush_bytes, stream) != hipSuccess) break;
+      hipEventRecord(begin, stream);
+      if (hipblasLtMatmul(dev.handle, plan.desc, &one, w, plan.a, x, plan.b, &zero, y, plan.d, y, plan.d, &found[i].algo,
+                          dev.workspace, LT_WORKSPACE_BYTES, stream) != HIPBLAS_STATUS_SUCCESS) { fastest = -1.0f; break; }
+      hipEventRecord(end, stream);
+      if (hipEventSynchronize(end) != hipSuccess) { fastest = -1.0f; break; }
+      float ms = 0.0f;
+      if (run && hipEventElapsedTime(&ms, begin, end) == hipSuccess && (fastest < 0.0f || ms < fastest)) fastest = ms;
+    }
+    if (fastest >= 0.0f && (best < 0.0f || fastest < best)) {
+      best = fastest;
+      plan.algo = found[i].algo;
+      plan.workspace = found[i].workspaceSize;
+    }
+  }
+  hipEventDestroy(begin);
+  hipEventDestroy(end);
 }
 
 }  // namespace
@@ -116,15 +171,24 @@ extern "C" int ts_gemm_library_init() {
 
 // y, x, w bfloat16; rows of x, w and y are ldx, ldw, ldy elements apart (each at least the row's
 // length). The stream may be one that is being captured into a graph (after ts_gemm_library_init).
+// tune != 0: a shape of at most 256 rows that has not been tuned yet is tuned first (see above),
+// unless the stream is being captured; `flush` is device memory of `flush_bytes` that may be
+// overwritten (more than the caches hold, 512 MB say), or null to time with warm caches.
 extern "C" int ts_gemm_library_bf16(void* y, const void* x, const void* w, int M, int N, int K, int64_t ldx,
-                                    int64_t ldw, int64_t ldy, hipStream_t stream) {
+                                    int64_t ldw, int64_t ldy, int tune, void* flush, size_t flush_bytes,
+                                    hipStream_t stream) {
   if (M <= 0 || N <= 0) return TS_OK;
   if (K <= 0 || ldx < K || ldw < K || ldy < N || !y || !x || !w) return TS_BAD_SHAPE;
   std::lock_guard<std::mutex> guard(lt_mutex);
   LtDevice* dev = lt_device();
   if (!dev) return TS_LAUNCH_FAILED;
-  const LtPlan* plan = lt_plan(*dev, M, N, K, ldx, ldw, ldy);
+  LtPlan* plan = lt_plan(*dev, M, N, K, ldx, ldw, ldy);
   if (!plan) return TS_BAD_SHAPE;
+  if (tune && !plan->tuned && M <= LT_TUNE_MAX_ROWS) {
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone)
+      lt_tune(*dev, *plan, y, x, w, flush, flush_bytes, stream);
+  }
   const float one = 1.0f, zero = 0.0f;
   const hipblasStatus_t st = hipblasLtMatmul(dev->handle, plan->desc, &one, w, plan->a, x, plan->b, &zero, y, plan->d, y,
                                              plan->d, &plan->algo, dev->workspace, LT_WORKSPACE_BYTES, stream);

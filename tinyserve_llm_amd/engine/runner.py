@@ -345,10 +345,11 @@ class DecodeGraphs:
         ctx, rows = r._context(dev_i32, dims, host)
         draw_keys = dev_i32[start:start + 2 * size].view(torch.int64)
         draw_temps = dev_i32[start + 2 * size:start + 3 * size].view(torch.float32)
-        # once without capture: libraries set up their workspaces, the kernel library loads
+        # once without capture: libraries set up their workspaces, the kernel library loads, and
+        # the matrix library's candidates for this batch size are timed and the fastest kept
         side = torch.cuda.Stream(device=r.device)
         side.wait_stream(torch.cuda.current_stream(r.device))
-        with torch.cuda.stream(side):
+        with torch.cuda.stream(side), hip.library_tuning():
             hidden, residual = r.model.forward(ctx, r.memory)
             hip.sample(r.model.logits(hidden, residual, rows), draw_temps, draw_keys, self.seed)
         torch.cuda.current_stream(r.device).wait_stream(side)

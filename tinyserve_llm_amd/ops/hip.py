@@ -8,6 +8,7 @@ bounds takes the GPU down with it.
 
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import threading
 
@@ -52,7 +53,7 @@ def _declare(lib: ctypes.CDLL) -> None:
                                       i, p],
         "ts_gemm_exact": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_sample": [p, p, p, p, p, p, u64, i, i, i64, p],
-        "ts_gemm_library_bf16": [p, p, p, i, i, i, i64, i64, i64, p],
+        "ts_gemm_library_bf16": [p, p, p, i, i, i, i64, i64, i64, i, p, ctypes.c_size_t, p],
         "ts_gemm_library_init": [],
         "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, p],
         "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p],
@@ -649,14 +650,34 @@ def gemm_library_init() -> None:
     _run("gemm_library_init", library().ts_gemm_library_init())
 
 
+LIBRARY_TUNING_SWEEP_BYTES = 512 << 20    # overwritten between timed runs: more than the caches hold
+_library_tuning: torch.Tensor | None = None
+
+
+@contextlib.contextmanager
+def library_tuning():
+    """While this is open, library products of at most 256 rows whose shape has not been tuned yet
+    are tuned at their call: the library's candidates are timed on the call's operands with the
+    caches swept in between, and the fastest serves the shape from then on (in this process, for
+    every caller). Open it around the eager run that precedes the recording of a decode step."""
+    global _library_tuning
+    _library_tuning = torch.empty(LIBRARY_TUNING_SWEEP_BYTES, dtype=torch.uint8, device="cuda")
+    try:
+        yield
+    finally:
+        _library_tuning = None
+
+
 def gemm_library(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """bfloat16 x [M, K] · weight [N, K]^T by the vendor's matrix library, called directly with the
-    algorithm it picked for the shape the first time (see gemm_library.hip). Rows may be strided."""
+    algorithm kept for the shape (see gemm_library.hip). Rows may be strided."""
     _need(x.stride(1) == 1 and weight.stride(1) == 1, "rows of x and of the weight must be dense")
     M, K = x.shape
     N = weight.shape[0]
     y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
     if M and N:
-        _run("gemm_library", library().ts_gemm_library_bf16(_ptr(y), _ptr(x), _ptr(weight), M, N, K, x.stride(0),
-                                                            weight.stride(0), N, _stream()))
+        sweep = _library_tuning
+        _run("gemm_library", library().ts_gemm_library_bf16(
+            _ptr(y), _ptr(x), _ptr(weight), M, N, K, x.stride(0), weight.stride(0), N, int(sweep is not None),
+            _ptr(sweep), 0 if sweep is None else sweep.numel(), _stream()))
     return y
