@@ -27,8 +27,9 @@ constexpr int LT_MAX_DEVICES = 16;
 constexpr size_t LT_MAX_PLANS = 8192;              // per device; a serving process meets many row counts
 constexpr int LT_CANDIDATES = 16;                  // asked of the heuristic for a plan,
 constexpr int LT_TUNE_CANDIDATES = 48;             // and when a shape is tuned
-constexpr int LT_TUNE_MAX_ROWS = 256;              // shapes with more rows keep the heuristic's choice
-constexpr int LT_TUNE_RUNS = 3;                    // timed runs per candidate; the fastest counts
+constexpr int LT_TUNE_MIN_ROWS = 9;                // shapes with fewer rows keep the heuristic's choice (little to gain),
+constexpr int LT_TUNE_MAX_ROWS = 256;              // and so do shapes with more (the first candidate was the fastest)
+constexpr int LT_TUNE_RUNS = 2;                    // timed runs per candidate; the faster counts
 
 struct LtPlan {
   hipblasLtMatmulDesc_t desc = nullptr;
@@ -171,9 +172,9 @@ extern "C" int ts_gemm_library_init() {
 
 // y, x, w bfloat16; rows of x, w and y are ldx, ldw, ldy elements apart (each at least the row's
 // length). The stream may be one that is being captured into a graph (after ts_gemm_library_init).
-// tune != 0: a shape of at most 256 rows that has not been tuned yet is tuned first (see above),
+// tune != 0: a shape of 9 to 256 rows that has not been tuned yet is tuned first (see above),
 // unless the stream is being captured; `flush` is device memory of `flush_bytes` that may be
-// overwritten (more than the caches hold, 512 MB say), or null to time with warm caches.
+// overwritten (more than the caches hold), or null to time with warm caches.
 extern "C" int ts_gemm_library_bf16(void* y, const void* x, const void* w, int M, int N, int K, int64_t ldx,
                                     int64_t ldw, int64_t ldy, int tune, void* flush, size_t flush_bytes,
                                     hipStream_t stream) {
@@ -184,7 +185,7 @@ extern "C" int ts_gemm_library_bf16(void* y, const void* x, const void* w, int M
   if (!dev) return TS_LAUNCH_FAILED;
   LtPlan* plan = lt_plan(*dev, M, N, K, ldx, ldw, ldy);
   if (!plan) return TS_BAD_SHAPE;
-  if (tune && !plan->tuned && M <= LT_TUNE_MAX_ROWS) {
+  if (tune && !plan->tuned && M >= LT_TUNE_MIN_ROWS && M <= LT_TUNE_MAX_ROWS) {
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone)
       lt_tune(*dev, *plan, y, x, w, flush, flush_bytes, stream);

@@ -650,13 +650,13 @@ def gemm_library_init() -> None:
     _run("gemm_library_init", library().ts_gemm_library_init())
 
 
-LIBRARY_TUNING_SWEEP_BYTES = 512 << 20    # overwritten between timed runs: more than the caches hold
+LIBRARY_TUNING_SWEEP_BYTES = 320 << 20    # overwritten between timed runs: more than the caches hold (256 MB)
 _library_tuning: torch.Tensor | None = None
 
 
 @contextlib.contextmanager
 def library_tuning():
-    """While this is open, library products of at most 256 rows whose shape has not been tuned yet
+    """While this is open, library products of 9 to 256 rows whose shape has not been tuned yet
     are tuned at their call: the library's candidates are timed on the call's operands with the
     caches swept in between, and the fastest serves the shape from then on (in this process, for
     every caller). Open it around the eager run that precedes the recording of a decode step."""
