@@ -320,3 +320,34 @@ def test_recorded_steps_with_library_products_replay_what_eager_steps_compute(tm
             assert max(sizes) > 32, f"a batch above 32 requests was recorded: {sizes}"
             assert [r.token_ids for r in llm.generate(prompts, params)] == outs[0]
     assert outs[0] == outs[1]
+
+
+@pytest.mark.parametrize("hidden,inter,vocab,heads,kv,hd", [(100, 150, 333, 5, 5, 16), (104, 152, 1001, 6, 2, 48),
+                                                             (36, 20, 77, 3, 1, 16)])
+def test_awkward_sizes_run_in_both_precisions(tmp_path, hidden, inter, vocab, heads, kv, hd):
+    """Widths whose rows are not 16-byte aligned, odd vocabularies, head counts that divide nothing:
+    the kernels' general forms serve them (or the vector forms, where a size happens to allow),
+    never a wrong result. A prompt in two portions against the plain model, float32 and bfloat16."""
+    from tinyserve_llm_amd.config import LlamaConfig
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.runner import StepEntry
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    from tinyserve_llm_amd.weights.random_init import write_random_model
+    config = LlamaConfig(vocab_size=vocab, hidden_size=hidden, intermediate_size=inter, num_hidden_layers=2,
+                         num_attention_heads=heads, num_key_value_heads=kv, head_dim=hd, max_position_embeddings=128,
+                         rms_norm_eps=1e-5, rope_theta=10000.0, rope_scaling=None, tie_word_embeddings=True,
+                         eos_token_id=vocab - 1)
+    write_random_model(str(tmp_path), config, 3, torch.float32)
+    ids = prompt(7, 70, vocab)
+    sc = SchedulerConfig(max_model_len=128, max_num_seqs=4, max_num_batched_tokens=256)
+    for dtype, tolerance in ((torch.float32, 2e-5), (torch.bfloat16, 3e-2)):
+        want = PlainLlama(str(tmp_path), torch.float64, weights_as=None if dtype == torch.float32 else dtype).logits(ids)
+        llm = LLM(str(tmp_path), sc, CacheConfig(block_size=16), dtype=dtype, num_blocks=20)
+        llm.manager.allocate(0, ids[:40])
+        first = llm.runner.step([StepEntry(0, ids[:40], 0, list(range(40)))])
+        llm.manager.commit(0, 40)
+        llm.manager.append_slots(0, ids[40:])
+        rest = llm.runner.step([StepEntry(0, ids[40:], 40, list(range(30)))])
+        got = torch.cat([first, rest]).double().cpu()
+        spread = float(want.max() - want.min())
+        assert float((got - want).abs().max()) <= tolerance * spread, f"{dtype}: {float((got - want).abs().max())} of {spread}"
