@@ -30,27 +30,31 @@ sys.path.insert(0, ROOT)
 HBM_BYTES_PER_S = 8.0e12
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
-FULL_LAYERS = 16
-SHAPE = dict(vocab_size=128256, hidden_size=2048, intermediate_size=8192, num_attention_heads=32,
-             num_key_value_heads=8, head_dim=64, max_position_embeddings=131072, rms_norm_eps=1e-5,
-             rope_theta=500000.0, tie_word_embeddings=True)
+# layer sizes (--shape); the default, "1b", is the one the headline numbers are quoted on
+SHAPES = {
+    "1b": dict(model="llama-3.2-1b-shape", layers_full=16, rope_factor=32.0,
+               shape=dict(vocab_size=128256, hidden_size=2048, intermediate_size=8192, num_attention_heads=32,
+                          num_key_value_heads=8, head_dim=64, max_position_embeddings=131072, rms_norm_eps=1e-5,
+                          rope_theta=500000.0, tie_word_embeddings=True)),
+    "3b": dict(model="llama-3.2-3b-shape", layers_full=28, rope_factor=32.0,
+               shape=dict(vocab_size=128256, hidden_size=3072, intermediate_size=8192, num_attention_heads=24,
+                          num_key_value_heads=8, head_dim=128, max_position_embeddings=131072, rms_norm_eps=1e-5,
+                          rope_theta=500000.0, tie_word_embeddings=True)),
+    "8b": dict(model="llama-3.1-8b-shape", layers_full=32, rope_factor=8.0,
+               shape=dict(vocab_size=128256, hidden_size=4096, intermediate_size=14336, num_attention_heads=32,
+                          num_key_value_heads=8, head_dim=128, max_position_embeddings=131072, rms_norm_eps=1e-5,
+                          rope_theta=500000.0, tie_word_embeddings=False)),
+}
 ROPE = dict(factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=8192)
 PROMPT_LEN, MAX_MODEL_LEN, PAGE = 2048, 4096, 256
+SHAPE = SHAPES["1b"]["shape"]
 
 # whole workloads: layer sizes, requests, and how the scheduler is set for them
 SCENARIOS = {
-    "requests-3b": dict(
-        model="llama-3.2-3b-shape", layers_full=28, rope_factor=32.0,
-        shape=dict(vocab_size=128256, hidden_size=3072, intermediate_size=8192, num_attention_heads=24,
-                   num_key_value_heads=8, head_dim=128, max_position_embeddings=131072, rms_norm_eps=1e-5,
-                   rope_theta=500000.0, tie_word_embeddings=True),
-        requests=64, prompt=(512, 4096), shared=(0.25, 1024), decode=256, budget=8192, chunk=0, caching=True),
-    "chunked-8b": dict(
-        model="llama-3.1-8b-shape", layers_full=32, rope_factor=8.0,
-        shape=dict(vocab_size=128256, hidden_size=4096, intermediate_size=14336, num_attention_heads=32,
-                   num_key_value_heads=8, head_dim=128, max_position_embeddings=131072, rms_norm_eps=1e-5,
-                   rope_theta=500000.0, tie_word_embeddings=False),
-        requests=32, prompt=(7936, 7936), shared=(0.0, 0), decode=256, budget=2048 + 32, chunk=2048, caching=False),
+    "requests-3b": dict(**SHAPES["3b"], requests=64, prompt=(512, 4096), shared=(0.25, 1024), decode=256, budget=8192,
+                        chunk=0, caching=True),
+    "chunked-8b": dict(**SHAPES["8b"], requests=32, prompt=(7936, 7936), shared=(0.0, 0), decode=256,
+                       budget=2048 + 32, chunk=2048, caching=False),
 }
 
 
@@ -132,6 +136,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=None)
+    ap.add_argument("--shape", default="1b", choices=sorted(SHAPES), help="layer sizes of the decode and prefill steps")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--points", default="1,64", help="further decode batch sizes (comma-separated; '' for none)")
     ap.add_argument("--no-prefill", action="store_true")
@@ -145,7 +150,9 @@ def main() -> int:
         return 2
     if args.scenario:
         return scenario(args.scenario, args.layers, args.dtype)
-    args.layers = args.layers or FULL_LAYERS
+    sizes = SHAPES[args.shape]
+    full_layers = sizes["layers_full"]
+    args.layers = args.layers or full_layers
 
     import torch
 
@@ -155,7 +162,8 @@ def main() -> int:
     from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
     from tinyserve_llm_amd.engine.sequence import SamplingParams
 
-    config = LlamaConfig(num_hidden_layers=args.layers, rope_scaling=RopeScaling(**ROPE), **SHAPE)
+    config = LlamaConfig(num_hidden_layers=args.layers, rope_scaling=RopeScaling(**{**ROPE, "factor": sizes["rope_factor"]}),
+                         **sizes["shape"])
     dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
     itemsize = 2 if args.dtype == "bf16" else 4
     model = random_model(config, 0, dtype, "cuda:0")
@@ -164,7 +172,7 @@ def main() -> int:
     c = config
     layer_weights = (c.q_size + 2 * c.kv_size) * c.hidden_size + c.hidden_size * c.q_size \
         + 3 * c.intermediate_size * c.hidden_size
-    weight_bytes = (args.layers * layer_weights + c.vocab_size * c.hidden_size) * itemsize
+    weight_bytes = (args.layers * layer_weights + c.vocab_size * c.hidden_size) * itemsize   # the head; the embedding reads rows
     kv_bytes_per_token = 2 * args.layers * c.kv_size * itemsize
 
     def engine(batch: int, steps: int) -> LLM:
@@ -226,11 +234,11 @@ def main() -> int:
     step_bytes = weight_bytes + args.batch * mean_ctx * kv_bytes_per_token
     achieved = step_bytes / (seconds / args.steps)
     record = {
-        "metric": f"decode tok/s at batch {args.batch} (Llama-3.2-1B shape, 2,048-token contexts)",
+        "metric": f"decode tok/s at batch {args.batch} ({sizes['model']}, 2,048-token contexts)",
         "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": 1e3 * seconds / args.steps, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": args.dtype, "data": "synthetic uniform token ids, random weights N(0,0.02)",
-        "config": {"model": "llama-3.2-1b-shape", "layers": args.layers, "layers_full": FULL_LAYERS,
+        "config": {"model": sizes["model"], "layers": args.layers, "layers_full": full_layers,
                    "hidden": c.hidden_size, "heads": c.num_attention_heads, "kv_heads": c.num_key_value_heads,
                    "head_dim": c.head_dim, "intermediate": c.intermediate_size, "vocab": c.vocab_size,
                    "global_batch": args.batch, "prompt_len": PROMPT_LEN, "seq_len": MAX_MODEL_LEN,

@@ -426,7 +426,8 @@ def test_library_product_called_directly(m, n, k):
 
 
 @pytest.mark.parametrize("m", [1, 3, 8, 16, 17, 32])
-@pytest.mark.parametrize("n,k", [(3072, 2048), (2048, 2048), (16384, 2048), (2048, 8192), (992, 512), (130, 3072), (64, 4096)])
+@pytest.mark.parametrize("n,k", [(3072, 2048), (2048, 2048), (16384, 2048), (2048, 8192), (992, 512), (130, 3072), (64, 4096),
+                                 (8192, 3072), (8256, 4096)])
 def test_weight_streaming_gemm_and_its_fused_inputs(m, n, k):
     """The skinny kernel plain, with residual + RMSNorm on the way in, and with the SiLU gate on
     the way in, against the same operations done one after the other in float64 with the storage
@@ -563,7 +564,7 @@ def test_sampler_draw_is_the_exponential_race_and_ignores_the_row_order():
 
 
 @pytest.mark.parametrize("nh,nkv,hd,K,M,page", [(32, 8, 64, 2048, 8, 64), (6, 2, 96, 768, 5, 16), (4, 4, 128, 256, 16, 8),
-                                                 (3, 1, 32, 1280, 1, 32)])
+                                                 (3, 1, 32, 1280, 1, 32), (24, 8, 128, 3072, 8, 64), (8, 2, 128, 4096, 3, 32)])
 @pytest.mark.parametrize("norm", [False, True])
 @pytest.mark.parametrize("rotate", [True, False])
 def test_fused_projection_rotation_and_cache_write(nh, nkv, hd, K, M, page, norm, rotate):
@@ -595,6 +596,12 @@ def test_fused_projection_rotation_and_cache_write(nh, nkv, hd, K, M, page, norm
     qkv = hip().gemm_skinny(xn, w)[0]
     q_want = hip().rope_store(qkv, table, positions, slots, kp1.permute(0, 2, 1, 3), vp1.permute(0, 3, 1, 2), nh, nkv, hd)
     assert hip().qkv_rope_fuses(x, w, hd, kp2.permute(0, 2, 1, 3))
+    if norm and K > 2048:            # the norm rides along only up to 2048; a part runs it by itself beyond
+        assert not hip().qkv_rope_fuses(x, w, hd, kp2.permute(0, 2, 1, 3), norm=True)
+        with pytest.raises(hip().KernelError, match="qkv_rope_store takes"):
+            hip().qkv_rope_store(x, w, table, positions, slots, kp2.permute(0, 2, 1, 3), vp2.permute(0, 3, 1, 2),
+                                 nh, nkv, hd, residual=res, norm_weight=nw, eps=1e-5)
+        return
     q, res_out = hip().qkv_rope_store(x, w, table, positions, slots, kp2.permute(0, 2, 1, 3), vp2.permute(0, 3, 1, 2),
                                       nh, nkv, hd, **(dict(residual=res, norm_weight=nw, eps=1e-5) if norm else {}))
     torch.testing.assert_close(q.float(), q_want.float(), rtol=2e-2, atol=2e-2)
@@ -614,7 +621,9 @@ def test_fused_projection_refuses_what_it_cannot_serve():
     w = torch.zeros(3 * 64, 256, dtype=torch.bfloat16, device=dev())
     assert not hip().qkv_rope_fuses(x, w, 64, None), "17 rows"
     assert not hip().qkv_rope_fuses(x[:4], w, 48, None), "head_dim 48"
-    assert not hip().qkv_rope_fuses(torch.zeros(4, 2304, dtype=torch.bfloat16, device=dev()), w, 64, None), "K beyond 2048"
+    assert not hip().qkv_rope_fuses(torch.zeros(4, 4352, dtype=torch.bfloat16, device=dev()), w, 64, None), "K beyond 4096"
+    assert not hip().qkv_rope_fuses(torch.zeros(4, 2304, dtype=torch.bfloat16, device=dev()), w, 64, None, norm=True), \
+        "K beyond 2048 with the norm"
     with pytest.raises(hip().KernelError, match="qkv_rope_store takes"):
         hip().qkv_rope_store(x, w, None, torch.zeros(17, dtype=torch.int32, device=dev()), None, None, None, 1, 1, 64)
 

@@ -319,8 +319,9 @@ static int sk_launch(const SkinnyArgs& a, hipStream_t stream) {
   if (nwaves <= 8) {
     gemm_skinny_kernel<RT, CB, STEPS, MODE, GLU, 512, OUT><<<grid, block, smem, stream>>>(a);
   } else {
-    // only single row tiles leave a workgroup of 16 waves the registers it needs
-    if constexpr (RT == 1) gemm_skinny_kernel<RT, CB, STEPS, MODE, GLU, 1024, OUT><<<grid, block, smem, stream>>>(a);
+    // a workgroup of 16 waves has 128 registers a lane: single row tiles, or two without the norm's copy of x
+    if constexpr (RT == 1 || (RT == 2 && CB == 1 && MODE == MODE_PLAIN))
+      gemm_skinny_kernel<RT, CB, STEPS, MODE, GLU, 1024, OUT><<<grid, block, smem, stream>>>(a);
     else return TS_BAD_SHAPE;
   }
   return ts_check_launch();
@@ -346,9 +347,10 @@ static int sk_dispatch(const SkinnyArgs& a, hipStream_t stream) {
       if (GLU || ncols >= 4096) SK_GO(2, 1, 8);
     }
     if constexpr (GLU == 0) SK_GO(1, 1, 8);
+    if constexpr (MODE == MODE_PLAIN) SK_GO(2, 1, 8);   // the gate alone, in a workgroup of up to 16 waves
     return TS_BAD_SHAPE;
   } else {
-    const bool two = a.N >= 8192 && nwaves <= 8;
+    const bool two = a.N >= 8192 && (nwaves <= 8 || cb == 1);
     if (steps == 8) {
       if (two) { if (cb == 1) SK_GO(2, 1, 8); else SK_GO(2, 2, 8); }
       if (cb == 1) SK_GO(1, 1, 8); else SK_GO(1, 2, 8);
@@ -359,7 +361,7 @@ static int sk_dispatch(const SkinnyArgs& a, hipStream_t stream) {
 }
 
 // mode: 0 plain, 1 residual + RMSNorm on the way in (M <= 16, K in steps of 256 up to 4096). glu: W holds
-// gate rows then up rows, y is [M, N / 2] = silu(gate) * up (M <= 16). out_dtype: 1 bfloat16, 0 float
+// gate rows then up rows, y is [M, N / 2] = silu(gate) * up (M <= 16, K up to 4096, 2048 with the norm). out_dtype: 1 bfloat16, 0 float
 // (plain only). packed: w holds the matrix in the kernel's own order (see the loads of W), ldw is unused. Requires M <= 32, K a multiple of 256 (up to 4096) or of 512 (up to 8192), contiguous
 // 16-byte aligned rows; mode 1 takes x, res, res_out as dense [M, K].
 extern "C" int ts_gemm_skinny_bf16(void* y, const void* x, const void* w, const void* res, const void* nw,
@@ -387,7 +389,8 @@ extern "C" int ts_gemm_skinny_bf16(void* y, const void* x, const void* w, const 
 // The qkv projection of an attention layer with the rotation and the cache write on the way out:
 // q_out [M, nh * hd] gets the rotated queries, the rotated keys and the values go to the slots
 // `slots[m]` of the pages (see SkinnyArgs); w is [(nh + 2 nkv) * hd, K]. mode as above. Requires
-// M <= 16, hd a multiple of 32, K a multiple of 256 up to 2048, 8-byte aligned cache strides.
+// M <= 16, hd a multiple of 32, K a multiple of 256 up to 4096 (2048 with the norm), 8-byte aligned
+// cache strides.
 extern "C" int ts_gemm_skinny_rope_bf16(void* q_out, const void* x, const void* w, const void* res, const void* nw,
                                         void* res_out, int M, int K, int64_t ldx, int64_t ldw, float eps, int mode,
                                         int packed, const float* cos_sin, const int32_t* positions, const int32_t* slots,
@@ -395,7 +398,7 @@ extern "C" int ts_gemm_skinny_rope_bf16(void* q_out, const void* x, const void* 
                                         int page_size, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vs,
                                         int64_t vh, int64_t vd, hipStream_t stream) {
   if (M <= 0) return TS_OK;
-  if (M > 16 || K <= 0 || K % 256 || K / 256 > 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K) return TS_BAD_SHAPE;
+  if (M > 16 || K <= 0 || K % 256 || K / 256 > (mode == MODE_NORM ? 8 : 16) || ldx % 8 || ldw % 8 || ldx < K || ldw < K) return TS_BAD_SHAPE;
   if (nh <= 0 || nkv < 0 || hd <= 0 || hd % 32 || page_size <= 0) return TS_BAD_SHAPE;
   if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)res | (uintptr_t)nw | (uintptr_t)res_out | (uintptr_t)q_out) & 15)
     return TS_BAD_SHAPE;

@@ -59,11 +59,13 @@ class Attention(Mixer):
         rows = d.x if d is not None else x
         if not (rows.is_cuda and hip.qkv_rope_fuses(rows, self.qkv, self.head_dim, k_store)):
             return None
+        if d is not None and not (hip.qkv_rope_fuses(rows, self.qkv, self.head_dim, k_store, norm=True)
+                                  and d.weight.dtype == torch.bfloat16
+                                  and (d.residual is None or d.residual.is_contiguous())):
+            rows, d = d.materialize(), None      # the norm by its own kernel, the rest in one
         if d is None:
             return hip.qkv_rope_store(rows, self.qkv, table, positions, slots, k_store, v_store, self.num_heads,
                                       self.num_kv_heads, self.head_dim, packed=self.qkv_packed)[0]
-        if d.weight.dtype != torch.bfloat16 or (d.residual is not None and not d.residual.is_contiguous()):
-            return None
         q, d.residual_out = hip.qkv_rope_store(rows, self.qkv, table, positions, slots, k_store, v_store, self.num_heads,
                                                self.num_kv_heads, self.head_dim, residual=d.residual,
                                                norm_weight=d.weight, eps=d.eps, packed=self.qkv_packed)
