@@ -229,8 +229,9 @@ class Scheduler:
         `max_skip_wait`: then admission stops so that what frees up goes to it
         (scheduler.py:160-204)."""
         admitted: list[ScheduledSeq] = []
-        if budget <= 0:
-            return admitted
+        owed = self._owed_forks()                # kept up to date as groups are admitted below
+        if budget <= 0 or not self.waiting or len(self.running) + owed + 1 > self.config.max_num_seqs:
+            return admitted                      # no one can be admitted: nothing to rank
         for seq, _ in self._ranked_waiting(now):
             if budget <= 0:
                 break
@@ -240,7 +241,6 @@ class Scheduler:
             cost = self.kv.calculate_admission_cost(tokens, feed)
             hit = self._hit(len(tokens), whole)
             forks = seq.params.n - 1 if self._first_of_group(seq) else 0
-            owed = self._owed_forks()
             fits = (feed >= 1
                     and len(self.running) + owed + 1 + forks <= self.config.max_num_seqs
                     and self.kv.fits(cost.per_space, owed + forks + self.watermark_blocks))
@@ -265,6 +265,7 @@ class Scheduler:
             final = cached + len(fed) >= len(tokens)
             samples = 0 if not final else (seq.params.n if forks else 1)
             self.running.append(seq)
+            owed += forks
             seq.in_step = True
             admitted.append(ScheduledSeq(seq, fed, samples, cached))
         if admitted:
