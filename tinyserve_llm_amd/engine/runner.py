@@ -310,7 +310,7 @@ class DecodeGraphs:
         if len(entries) > self.max_batch:
             return False
         for e in entries:
-            if len(e.tokens) != 1 or list(e.want) != [0] or e.start + 1 > self.max_context:
+            if len(e.tokens) != 1 or len(e.want) != 1 or e.want[0] != 0 or e.start + 1 > self.max_context:
                 return False
         return True
 
