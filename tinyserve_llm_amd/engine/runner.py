@@ -349,7 +349,7 @@ class DecodeGraphs:
         # the matrix library's candidates for this batch size are timed and the fastest kept
         side = torch.cuda.Stream(device=r.device)
         side.wait_stream(torch.cuda.current_stream(r.device))
-        with torch.cuda.stream(side), hip.library_tuning():
+        with hip.library_tuning(), torch.cuda.stream(side):      # (the sweep buffer belongs to the current stream)
             hidden, residual = r.model.forward(ctx, r.memory)
             hip.sample(r.model.logits(hidden, residual, rows), draw_temps, draw_keys, self.seed)
         torch.cuda.current_stream(r.device).wait_stream(side)
