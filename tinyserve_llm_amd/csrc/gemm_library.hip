@@ -30,6 +30,7 @@ constexpr int LT_TUNE_CANDIDATES = 48;             // and when a shape is tuned
 constexpr int LT_TUNE_MIN_ROWS = 9;                // shapes with fewer rows keep the heuristic's choice (little to gain),
 constexpr int LT_TUNE_MAX_ROWS = 256;              // and so do shapes with more (the first candidate was the fastest)
 constexpr int LT_TUNE_RUNS = 2;                    // timed runs per candidate; the faster counts
+constexpr int LT_GRAPH_MAX_ROWS = 1024;            // the most rows of a step that may be recorded into a graph
 
 struct LtPlan {
   hipblasLtMatmulDesc_t desc = nullptr;
@@ -80,6 +81,10 @@ LtPlan* lt_plan(LtDevice& dev, int M, int N, int K, int64_t ldx, int64_t ldw, in
   hipblasLtMatmulHeuristicResult_t found[LT_CANDIDATES];
   int count = 0, pick = -1;
   ok = ok && hipblasLtMatmulAlgoGetHeuristic(dev.handle, plan.desc, plan.a, plan.b, plan.d, plan.d, pref, LT_CANDIDATES, found, &count) == HIPBLAS_STATUS_SUCCESS;
+  // (shapes that a recorded decode step may hold take a candidate without workspace if there is one:
+  // an algorithm that clears its workspace would put a memory-set node into the graph)
+  for (int i = 0; ok && M <= LT_GRAPH_MAX_ROWS && i < count && pick < 0; ++i)
+    if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize == 0) pick = i;
   for (int i = 0; ok && i < count && pick < 0; ++i)
     if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize <= LT_WORKSPACE_BYTES) pick = i;
   ok = ok && pick >= 0;
@@ -122,7 +127,7 @@ void lt_tune(LtDevice& dev, LtPlan& plan, void* y, const void* x, const void* w,
   const float one = 1.0f, zero = 0.0f;
   float best = -1.0f;
   for (int i = 0; i < count; ++i) {
-    if (found[i].state != HIPBLAS_STATUS_SUCCESS || found[i].workspaceSize > LT_WORKSPACE_BYTES) continue;
+    if (found[i].state != HIPBLAS_STATUS_SUCCESS || found[i].workspaceSize != 0) continue;   // see lt_plan
     float fastest = -1.0f;
     for (int run = 0; run <= LT_TUNE_RUNS; ++run) {         // the first run is not timed
       if (flush && flush_bytes && hipMemsetAsync(flush, run, flush_bytes, stream) != hipSuccess) break;
