@@ -111,3 +111,30 @@ def test_prompt_portions_then_decoding_side_by_side(case, dtype):
         count += err.numel()
     print(f"[{dtype}] worst absolute logit error {worst:.3e}, root mean square {(squares / count) ** 0.5:.3e} over "
           f"{len(got)} rows; logits have standard deviation {spread:.3f}")
+
+
+def test_a_recorded_batch_of_forty_at_the_1b_sizes(tmp_path):
+    """Forty requests decode together through recorded steps at the 1B layer sizes: above 32 rows the
+    projections are the matrix library's, with the candidate that was fastest when the step was
+    recorded. The replays (a dozen, with the host's own work in between) must give the tokens of
+    eager steps, and every token must lie within the logit gap of the plain implementation's choice."""
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+    folder = str(tmp_path)
+    write_random_model(folder, CONFIG, 9, torch.bfloat16)
+    prompts = [prompt(700 + i, 24, CONFIG.vocab_size) for i in range(40)]
+    sp = SamplingParams(max_tokens=12, temperature=0.0, ignore_eos=True)
+    sc = SchedulerConfig(max_model_len=64, max_num_seqs=40, max_num_batched_tokens=1024)
+    outs = []
+    for graphs in (True, False):
+        llm = LLM(folder, sc, CacheConfig(block_size=16), dtype=torch.bfloat16, num_blocks=200, seed=0, decode_graphs=graphs)
+        outs.append([c.token_ids[0] for c in llm.generate(prompts, sp)])
+        if graphs:
+            assert 40 in {size for size, width in llm.runner.graphs.graphs}
+    assert outs[0] == outs[1]
+    plain = PlainLlama(folder, torch.float64)
+    for p, tokens in list(zip(prompts, outs[0]))[:3]:
+        logits = plain.logits(p + tokens[:-1])[len(p) - 1:]
+        gaps = logits.max(-1).values - logits[torch.arange(len(tokens)), torch.tensor(tokens)]
+        assert float(gaps.max()) <= 0.05 * float(logits.std()), f"a token far from the best: gaps {gaps.tolist()}"
