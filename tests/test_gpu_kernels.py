@@ -604,10 +604,31 @@ def test_fused_projection_rotation_and_cache_write(nh, nkv, hd, K, M, page, norm
         return
     q, res_out = hip().qkv_rope_store(x, w, table, positions, slots, kp2.permute(0, 2, 1, 3), vp2.permute(0, 3, 1, 2),
                                       nh, nkv, hd, **(dict(residual=res, norm_weight=nw, eps=1e-5) if norm else {}))
-    torch.testing.assert_close(q.float(), q_want.float(), rtol=2e-2, atol=2e-2)
-    torch.testing.assert_close(kp2.float(), kp1.float(), rtol=2e-2, atol=2e-2)
-    torch.testing.assert_close(vp2.float(), vp1.float(), rtol=2e-2, atol=2e-2)
+    # Both paths round to the storage type on the way (the one kernel applies the norm's row scale
+    # to the finished sums, the separate norm kernel to the operands), so neither is the measure of
+    # the other: the measure is the same chain in float64 without any rounding, and the one kernel
+    # must be as close to it as the kernels one after the other are.
+    s64 = x.double().cpu() + (res.double().cpu() if norm else 0)
+    y64 = s64 * torch.rsqrt(s64.pow(2).mean(-1, keepdim=True) + 1e-5) * nw.double().cpu() if norm else s64
+    t64 = (y64 @ w.double().cpu().T).view(M, nh + 2 * nkv, hd)
+    if rotate:
+        cs = table.double().cpu()[positions.cpu().long()]
+        c, sn = cs[:, None, :hd // 2], cs[:, None, hd // 2:]
+        a, b = t64[:, :nh + nkv, :hd // 2].clone(), t64[:, :nh + nkv, hd // 2:].clone()
+        t64[:, :nh + nkv, :hd // 2], t64[:, :nh + nkv, hd // 2:] = a * c - b * sn, b * c + a * sn
+    live = (slots >= 0).cpu()
+    pg, off = (slots.cpu().long() // page)[live], (slots.cpu().long() % page)[live]
+    def written(kp, vp):
+        return kp.double().cpu()[pg, :, off, :], vp.double().cpu()[pg, :, :, off]
+    (k_one, v_one), (k_seq, v_seq) = written(kp2, vp2), written(kp1, vp1)
+    for name, one, seq, truth in (("q", q.double().cpu(), q_want.double().cpu(), t64[:, :nh]),
+                                  ("k", k_one, k_seq, t64[live][:, nh:nh + nkv]), ("v", v_one, v_seq, t64[live][:, nh + nkv:])):
+        e_one, e_seq = (one - truth).abs(), (seq - truth).abs()
+        assert float(e_seq.max()) <= 3e-2 * max(1.0, float(truth.abs().max())), f"{name}: the separate kernels are off"
+        assert float(e_one.max()) <= 1.25 * float(e_seq.max()) + 1e-3, f"{name}: worst error {float(e_one.max())} vs {float(e_seq.max())}"
+        assert float(e_one.pow(2).mean().sqrt()) <= 1.1 * float(e_seq.pow(2).mean().sqrt()) + 1e-4, f"{name}: mean error"
     assert int((kp2 != 7.0).any(dim=(1, 3)).sum()) == int((slots >= 0).sum()), "only the named slots are written"
+    assert torch.equal(kp2 == 7.0, kp1 == 7.0) and torch.equal(vp2 == 7.0, vp1 == 7.0), "the same places are written"
     if norm:
         assert torch.equal(res_out, res_want)
     # without a cache of its own a layer only gets q

@@ -8,8 +8,11 @@
 //
 // x is read through the caches (it is tiny and shared by every workgroup). What precedes and
 // follows the product in a layer can ride along, so that no separate kernel has to run:
-//   MODE_NORM  f(x) = T(T((x + res) * rsqrt(mean((x + res)^2) + eps)) * nw): residual + RMSNorm on
-//              the way in (up to 16 rows); workgroup 0 also writes T(x + res) as the new residual
+//   MODE_NORM  residual + RMSNorm on the way in (up to 16 rows): the operand is T((x + res) * nw) and
+//              the row's scale rsqrt(mean((x + res)^2) + eps), 32-bit, multiplies the finished sums
+//              (the separate norm kernel rounds (x + res) * scale first and the product with nw
+//              again: the same value up to the rounding of the storage type); workgroup 0 also writes
+//              T(x + res) as the new residual
 //   EPI_GLU    W = [gate rows | up rows]; a workgroup takes matching rows of both and writes
 //              silu(gate) * up, y being [M, N / 2]
 //   EPI_ROPE   W = [q heads | k heads | v heads] of head_dim columns each; a workgroup takes 16
@@ -167,7 +170,45 @@ gemm_skinny_kernel(const SkinnyArgs a) {
 #pragma unroll
     for (int b = 0; b < CB; ++b) acc[t][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
-  if (MODE == MODE_NORM) {
+  // DEFER: the norm's row scale multiplies the finished sums instead of the operands
+  constexpr bool DEFER = MODE == MODE_NORM && MAXT <= 512;
+  float sq = 0.f;                                       // DEFER: this lane's share of its row's sum of squares
+  if (DEFER) {
+    // ---- (x + res) * nw of this wave's slice, rounded, is the operand. The row's scale
+    // rsqrt(mean((x + res)^2) + eps) is a number per row: it multiplies the finished sums on the way
+    // out instead of every operand on the way in, so no wave waits for the others' squares first.
+    const bool has_res = a.res != nullptr;
+    uint4 xb[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      // (both loads are used whatever the case, so that neither moves behind the loads of W)
+      float xs[8], rv[8], nv[8];
+      sk_unpack(xraw[s], xs);
+      sk_unpack(rraw[s], rv);
+      sk_unpack(EARLY_NW ? nraw[s] : *(const uint4*)(a.nw + kbeg + s * SK_KSTEP), nv);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float sum = xs[i] + (has_res ? rv[i] : 0.f);
+        xs[i] = xok[0] ? sum : 0.f;                      // rows past M count as zeros
+      }
+      if (has_res && blockIdx.x == 0 && xok[0]) *(uint4*)(a.res_out + (int64_t)r * a.K + kbeg + s * SK_KSTEP) = sk_pack(xs);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        sq = fmaf(xs[i], xs[i], sq);
+        xs[i] *= nv[i];
+      }
+      xb[s] = sk_pack(xs);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+      for (int t = 0; t < RT; ++t) acc[t][0] = sk_mfma(wreg[t][s], xb[s], acc[t][0]);
+    sq += __shfl_xor(sq, 16, TS_WAVE);
+    sq += __shfl_xor(sq, 32, TS_WAVE);
+    if (g == 0) ssq[wave * 16 + r] = sq;
+  } else if (MODE == MODE_NORM) {
+    // (a workgroup of 16 waves has no registers for the form above: it scales on the way in)
     // ---- x + res of this wave's slice stays in registers: summed squares first (all waves of the
     // workgroup together), then scaled, rounded and used
     float xs[STEPS][8];
@@ -256,6 +297,13 @@ gemm_skinny_kernel(const SkinnyArgs a) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) u[j] += pu[j];
       }
+    }
+    if (DEFER) {                                          // the row's scale, from every wave's squares
+      float total = 0.f;
+      for (int wv = 0; wv < nwaves; ++wv) total += ssq[wv * 16 + ml];
+      const float inv = 1.0f / sqrtf(total / (float)a.K + a.eps);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) { s[j] *= inv; u[j] *= inv; }
     }
     if (ROPE) {
       const int per_head = a.hd / 32, jb = blockIdx.x * OT + t, hdh = a.hd / 2;
