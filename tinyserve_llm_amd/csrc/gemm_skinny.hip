@@ -49,10 +49,14 @@ static __device__ __forceinline__ uint32_t sk_round(float f) {
   const uint32_t u = __float_as_uint(f);
   return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
 }
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
+// eight floats to eight bfloat16, round to nearest even, by the hardware's packed conversion
 static __device__ __forceinline__ uint4 sk_pack(const float* f) {
   uint32_t w[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) w[i] = sk_round(f[2 * i]) | (sk_round(f[2 * i + 1]) << 16);
+  for (int i = 0; i < 4; ++i)
+    w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector((float2_t){f[2 * i], f[2 * i + 1]}, bf16x2_t));
   return make_uint4(w[0], w[1], w[2], w[3]);
 }
 static __device__ __forceinline__ float sk_silu(float g) {
