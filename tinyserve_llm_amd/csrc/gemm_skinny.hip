@@ -119,10 +119,10 @@ gemm_skinny_kernel(const SkinnyArgs a) {
   // ---- MODE_NORM: this wave's slice of x, the residual and the norm weight are asked for before W.
   // Loads come back in the order they were issued, and these are short and hit the cache: the norm
   // is computed while W is still streaming in.
-  // (Workgroups of more than 8 waves have no registers to hold the norm weight meanwhile: they
-  // fetch it when they need it.)
-  constexpr bool EARLY_NW = MODE == MODE_NORM && MAXT <= 512;
-  uint4 xraw[MODE == MODE_NORM ? STEPS : 1], rraw[MODE == MODE_NORM ? STEPS : 1], nraw[EARLY_NW ? STEPS : 1];
+  // (Up to 8 waves a workgroup: 16 waves have no registers for it, and their callers run the norm
+  // as a kernel of its own.)
+  static_assert(MODE != MODE_NORM || MAXT <= 512, "the fused norm needs the registers of a workgroup of 8 waves");
+  uint4 xraw[MODE == MODE_NORM ? STEPS : 1], rraw[MODE == MODE_NORM ? STEPS : 1], nraw[MODE == MODE_NORM ? STEPS : 1];
   if (MODE == MODE_NORM) {
     // unconditional loads from addresses that always exist (rows past M read row 0, a missing
     // residual reads x again): what does not count is dropped after it has arrived
@@ -131,7 +131,7 @@ gemm_skinny_kernel(const SkinnyArgs a) {
     for (int s = 0; s < STEPS; ++s) {
       xraw[s] = *(const uint4*)(xrow[0] + s * SK_KSTEP);
       rraw[s] = *(const uint4*)(rrow + s * SK_KSTEP);
-      if (EARLY_NW) nraw[s] = *(const uint4*)(a.nw + kbeg + s * SK_KSTEP);
+      nraw[s] = *(const uint4*)(a.nw + kbeg + s * SK_KSTEP);
     }
     __builtin_amdgcn_sched_barrier(0);                  // the compiler keeps these loads ahead of W's
   }
@@ -174,10 +174,8 @@ gemm_skinny_kernel(const SkinnyArgs a) {
 #pragma unroll
     for (int b = 0; b < CB; ++b) acc[t][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
-  // DEFER: the norm's row scale multiplies the finished sums instead of the operands
-  constexpr bool DEFER = MODE == MODE_NORM && MAXT <= 512;
-  float sq = 0.f;                                       // DEFER: this lane's share of its row's sum of squares
-  if (DEFER) {
+  float sq = 0.f;                                       // MODE_NORM: this lane's share of its row's sum of squares
+  if (MODE == MODE_NORM) {
     // ---- (x + res) * nw of this wave's slice, rounded, is the operand. The row's scale
     // rsqrt(mean((x + res)^2) + eps) is a number per row: it multiplies the finished sums on the way
     // out instead of every operand on the way in, so no wave waits for the others' squares first.
@@ -189,7 +187,7 @@ gemm_skinny_kernel(const SkinnyArgs a) {
       float xs[8], rv[8], nv[8];
       sk_unpack(xraw[s], xs);
       sk_unpack(rraw[s], rv);
-      sk_unpack(EARLY_NW ? nraw[s] : *(const uint4*)(a.nw + kbeg + s * SK_KSTEP), nv);
+      sk_unpack(nraw[s], nv);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const float sum = xs[i] + (has_res ? rv[i] : 0.f);
@@ -211,50 +209,6 @@ gemm_skinny_kernel(const SkinnyArgs a) {
     sq += __shfl_xor(sq, 16, TS_WAVE);
     sq += __shfl_xor(sq, 32, TS_WAVE);
     if (g == 0) ssq[wave * 16 + r] = sq;
-  } else if (MODE == MODE_NORM) {
-    // (a workgroup of 16 waves has no registers for the form above: it scales on the way in)
-    // ---- x + res of this wave's slice stays in registers: summed squares first (all waves of the
-    // workgroup together), then scaled, rounded and used
-    float xs[STEPS][8];
-    float sq = 0.f;
-    const bool has_res = a.res != nullptr;
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      // (both loads are used whatever the case, so that neither moves behind the loads of W)
-      float rv[8];
-      sk_unpack(xraw[s], xs[s]);
-      sk_unpack(rraw[s], rv);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float sum = xs[s][i] + (has_res ? rv[i] : 0.f);
-        xs[s][i] = xok[0] ? sum : 0.f;                   // rows past M count as zeros
-      }
-      if (has_res && blockIdx.x == 0 && xok[0]) *(uint4*)(a.res_out + (int64_t)r * a.K + kbeg + s * SK_KSTEP) = sk_pack(xs[s]);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) sq = fmaf(xs[s][i], xs[s][i], sq);
-    }
-    sq += __shfl_xor(sq, 16, TS_WAVE);
-    sq += __shfl_xor(sq, 32, TS_WAVE);
-    if (g == 0) ssq[wave * 16 + r] = sq;
-    __syncthreads();
-    float total = 0.f;
-    for (int wv = 0; wv < nwaves; ++wv) total += ssq[wv * 16 + r];
-    const float inv = 1.0f / sqrtf(total / (float)a.K + a.eps);
-    // the normalised operand of every step is ready before the first product waits for W
-    uint4 xb[STEPS];
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      float nv[8];
-      sk_unpack(EARLY_NW ? nraw[s] : *(const uint4*)(a.nw + kbeg + s * SK_KSTEP), nv);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) xs[s][i] = __uint_as_float(sk_round(xs[s][i] * inv) << 16) * nv[i];
-      xb[s] = sk_pack(xs[s]);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s)
-#pragma unroll
-      for (int t = 0; t < RT; ++t) acc[t][0] = sk_mfma(wreg[t][s], xb[s], acc[t][0]);
   } else {
     // ---- x in batches of steps, then the products
 #pragma unroll
@@ -302,7 +256,7 @@ gemm_skinny_kernel(const SkinnyArgs a) {
         for (int j = 0; j < 4; ++j) u[j] += pu[j];
       }
     }
-    if (DEFER) {                                          // the row's scale, from every wave's squares
+    if (MODE == MODE_NORM) {                              // the row's scale, from every wave's squares
       float total = 0.f;
       for (int wv = 0; wv < nwaves; ++wv) total += ssq[wv * 16 + ml];
       const float inv = 1.0f / sqrtf(total / (float)a.K + a.eps);
@@ -371,8 +325,8 @@ static int sk_launch(const SkinnyArgs& a, hipStream_t stream) {
   if (nwaves <= 8) {
     gemm_skinny_kernel<RT, CB, STEPS, MODE, GLU, 512, OUT><<<grid, block, smem, stream>>>(a);
   } else {
-    // a workgroup of 16 waves has 128 registers a lane: single row tiles, or two without the norm's copy of x
-    if constexpr (RT == 1 || (RT == 2 && CB == 1 && MODE == MODE_PLAIN))
+    // a workgroup of 16 waves has 128 registers a lane: one or two row tiles, and no fused norm
+    if constexpr (MODE == MODE_PLAIN && (RT == 1 || (RT == 2 && CB == 1)))
       gemm_skinny_kernel<RT, CB, STEPS, MODE, GLU, 1024, OUT><<<grid, block, smem, stream>>>(a);
     else return TS_BAD_SHAPE;
   }
@@ -412,7 +366,7 @@ static int sk_dispatch(const SkinnyArgs& a, hipStream_t stream) {
 #undef SK_GO
 }
 
-// mode: 0 plain, 1 residual + RMSNorm on the way in (M <= 16, K in steps of 256 up to 4096). glu: W holds
+// mode: 0 plain, 1 residual + RMSNorm on the way in (M <= 16, K in steps of 256 up to 2048). glu: W holds
 // gate rows then up rows, y is [M, N / 2] = silu(gate) * up (M <= 16, K up to 4096, 2048 with the norm). out_dtype: 1 bfloat16, 0 float
 // (plain only). packed: w holds the matrix in the kernel's own order (see the loads of W), ldw is unused. Requires M <= 32, K a multiple of 256 (up to 4096) or of 512 (up to 8192), contiguous
 // 16-byte aligned rows; mode 1 takes x, res, res_out as dense [M, K].

@@ -522,7 +522,7 @@ def skinny_fuses(rows: int, k: int, norm: bool, glu: bool) -> bool:
     """Whether the kernel can apply the norm on the way in and/or the gate on the way out."""
     if not (norm or glu):
         return skinny_takes(rows, k)
-    return rows <= SKINNY_FUSED_ROWS and k % 256 == 0 and k // 256 <= (8 if glu and norm else 16)
+    return rows <= SKINNY_FUSED_ROWS and k % 256 == 0 and k // 256 <= (8 if norm else 16)
 
 
 def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, *,
@@ -541,7 +541,7 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     norm = norm_weight is not None
     _need(skinny_fuses(M, K, norm, glu),
           f"gemm_skinny takes up to {SKINNY_MAX_ROWS} rows ({SKINNY_FUSED_ROWS} when fused) and K in steps of 256 up to "
-          "4096 (2048 with norm and gate together) or of 512 up to 8192")
+          "4096 (2048 with the norm) or of 512 up to 8192")
     _need(x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0,
           "rows must be contiguous and 16-byte aligned")
     _need(not glu or (N % 32 == 0), "gate and up rows come in whole 16-row tiles")
