@@ -291,6 +291,23 @@ class KVCacheManager:
         assert checked or self.can_append(seq_id, len(token_ids)), "not enough free pages; preempt first"
         self._reserve(seq, token_ids)
 
+    def try_append_one(self, seq_id: int, token: int) -> bool:
+        """`can_append` and `append_slots` for the one token of a decoding request, in one pass
+        (a step of hundreds of requests asks this for every one of them): reserves the slot and
+        returns True, or changes nothing and returns False where pages are missing."""
+        seq = self.seqs[seq_id]
+        reserved = len(seq.token_ids)
+        assert reserved == seq.committed, "the previous step was not committed"
+        used_in_last = reserved % self.block_size
+        for space, table in zip(self.spaces, seq.tables):       # first pass: is there room everywhere
+            if used_in_last:
+                if space.refs[table[-1]] > 1 and space.available() < 1:
+                    return False
+            elif self._pages_for(reserved + 1) > len(table) and space.available() < 1:
+                return False
+        self._reserve(seq, (token,))
+        return True
+
     def set_token(self, seq_id: int, position: int, token: int) -> None:
         """Names the token of a reserved, not yet committed slot whose token was not known when the
         slot was reserved (pages are published by their tokens, at commit)."""

@@ -171,7 +171,8 @@ class Scheduler:
                 if seq.output_token_ids[-1] == PENDING and len(seq.output_token_ids) >= seq.params.max_tokens:
                     continue                       # the token under way is its last one
                 tokens = [seq.pending_token]
-            fits = self.kv.can_append(seq.seq_id, len(tokens))
+            one = not want_prefill       # a decoded token: asked for and reserved in one call
+            fits = self.kv.try_append_one(seq.seq_id, tokens[0]) if one else self.kv.can_append(seq.seq_id, len(tokens))
             while not fits:
                 victim = self._lowest_unscheduled(now, exclude=seq, gone=gone)
                 if victim is None:
@@ -180,12 +181,13 @@ class Scheduler:
                 gone.add(victim.seq_id)
                 if victim in mine:
                     mine.remove(victim)
-                fits = self.kv.can_append(seq.seq_id, len(tokens))
+                fits = self.kv.try_append_one(seq.seq_id, tokens[0]) if one else self.kv.can_append(seq.seq_id, len(tokens))
             if not fits:
                 self._preempt(seq)
                 gone.add(seq.seq_id)
                 break
-            self.kv.append_slots(seq.seq_id, tokens, checked=True)
+            if not one:
+                self.kv.append_slots(seq.seq_id, tokens, checked=True)
             final = seq.num_computed + len(tokens) >= seq.prefill_target
             samples = 1
             if want_prefill:
