@@ -54,5 +54,9 @@ def test_decode_plan_divides_the_context_into_32_key_steps_per_wave():
     assert hip.decode_plan(8, 8, 4, 64, 2304) == (256, 8)          # one step per wave
     assert hip.decode_plan(8, 8, 4, 128, 2304) == (128, 4)         # wide heads: four waves
     assert hip.decode_plan(64, 8, 4, 64, 2304) == (2304, 8)        # a workgroup per compute unit: nothing to combine
+    assert hip.decode_plan(64, 8, 4, 64, 32768) == (4096, 8)       # ... but not over a very long context
     assert hip.decode_plan(1, 8, 4, 64, 192) == (192, 6)           # short context: one workgroup
-    assert hip.decode_plan(1, 8, 4, 64, 32768) == (1024, 8)        # very long: four steps per wave
+    assert hip.decode_plan(1, 8, 4, 64, 32768) == (1024, 8)        # long: 32 chunks of a token's 8 heads fill the chip
+    assert hip.decode_plan(8, 8, 4, 128, 8192) == (2048, 4)        # 4 chunks for 64 (token, head) pairs
+    assert hip.decode_plan(8, 8, 4, 128, 32768) == (4096, 4)       # chunks stay within 4,096 keys
+    assert hip.decode_plan(4, 8, 4, 64, 8192) == (1024, 8)

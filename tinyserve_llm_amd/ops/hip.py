@@ -230,23 +230,36 @@ def decode_waves(hd: int) -> int:
     return 4 if hd > 64 else MAX_DECODE_WAVES
 
 
+DECODE_ONE_STEP_SPLITS = 18      # up to this many chunks per token a wave takes one 32-key step (the leanest instance)
+DECODE_TARGET_WORKGROUPS = 256   # beyond: as many chunks as give every compute unit a workgroup,
+DECODE_MAX_CHUNK = 4096          # of at most this many keys
+
+
 def decode_plan(num_tokens: int, nkv: int, group: int, hd: int, capacity: int) -> tuple[int, int]:
     """(keys per workgroup, waves per workgroup) of the split-key kernel for a step of `num_tokens`
-    one-query tokens over block tables that reach `capacity` positions; measured choices. One
-    workgroup per (token, key/value head) takes the whole context, and nothing is combined, where a
-    wave has one 32-key step of it, or where the step has a workgroup for every compute unit anyway
-    and the context is moderate. Otherwise a workgroup's waves take one 32-key step each (the
-    instance without a second buffer: more workgroups share a compute unit), four steps each for
-    very long contexts, or more when the combining kernel would not take the number of chunks."""
+    one-query tokens over block tables that reach `capacity` positions. Measured over batches of 1
+    to 64 and contexts of 2K to 32K at head sizes 64 and 128: where the step has a workgroup per
+    (token, key/value head) for every compute unit anyway, a workgroup takes the whole context and
+    nothing is combined (chunks of 4,096 keys beyond 16K); short contexts are cut so that a wave
+    has a single 32-key step (the instance without a second buffer); longer ones into as many
+    chunks as give the chip about one workgroup per compute unit, since the time of the combining
+    kernel grows with the number of chunks (head size 128, 8 tokens over 16K keys: 151 µs in
+    128-key chunks, 109 µs in 4,096-key chunks)."""
     most = decode_waves(hd)
     while most > 1 and 4 * (32 * most + most * group * hd) > 65536:
         most //= 2
-    if capacity <= 32 * most:
+    one = 32 * most
+    if capacity <= one:
         waves = -(-capacity // 32)
         return 32 * waves, waves
-    if num_tokens * nkv >= 256 and capacity <= 16384:
-        return -(-capacity // (32 * most)) * 32 * most, most
-    chunk = 32 * most if capacity <= 16384 else 128 * most
+    rows = num_tokens * nkv
+    if rows >= DECODE_TARGET_WORKGROUPS:
+        chunk = -(-capacity // one) * one if capacity <= 16384 else DECODE_MAX_CHUNK
+    elif -(-capacity // one) <= DECODE_ONE_STEP_SPLITS:
+        chunk = one
+    else:
+        splits = max(1, DECODE_TARGET_WORKGROUPS // rows)
+        chunk = min(max(-(-capacity // (splits * one)) * one, one), DECODE_MAX_CHUNK)
     while -(-capacity // chunk) > MAX_DECODE_SPLITS:
         chunk *= 2
     return chunk, most
