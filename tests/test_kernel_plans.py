@@ -35,12 +35,14 @@ def test_attention_tiles_cover_each_token_once_and_never_cross_a_request():
 def test_prefill_tile_tokens_keeps_the_chip_busy():
     assert hip.prefill_tile_tokens(512, 8, 4, 64) == 16           # one row tile per wave: 256 workgroups
     assert hip.prefill_tile_tokens(2048, 8, 4, 64) == 32          # two: 64 tiles for each of 8 heads
-    assert hip.prefill_tile_tokens(16384, 8, 4, 64) == 64         # four: 256 tiles for each of 8 heads
-    assert hip.prefill_tile_tokens(16384, 8, 4, 128) == 32        # large heads stop at two
+    assert hip.prefill_tile_tokens(2048, 8, 3, 128) == 40         # groups of three: 52 tiles of 40 tokens
+    assert hip.prefill_tile_tokens(4096, 8, 4, 64, mean_keys=2048) == 32
+    assert hip.prefill_tile_tokens(4096, 8, 4, 64, mean_keys=4096) == 64      # four: small heads, a long walk
+    assert hip.prefill_tile_tokens(16384, 8, 4, 128, mean_keys=8192) == 32    # large heads stop at two
     assert hip.prefill_tile_tokens(10, 1, 16, 32) == 4
     for tokens, nkv, group in ((100, 2, 3), (5000, 4, 8), (100000, 8, 1)):
         per_wave = hip.PREFILL_WAVES * (16 // group)
-        assert hip.prefill_tile_tokens(tokens, nkv, group, 64) in (per_wave, 2 * per_wave, 4 * per_wave)
+        assert hip.prefill_tile_tokens(tokens, nkv, group, 64, 5000.0) in (per_wave, 2 * per_wave, 4 * per_wave)
 
 
 def test_decode_plan_divides_the_context_into_32_key_steps_per_wave():

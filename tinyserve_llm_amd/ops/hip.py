@@ -392,23 +392,28 @@ def _out_like(q: torch.Tensor, out: torch.Tensor | None) -> torch.Tensor:
 
 
 PREFILL_WAVES = 4            # waves of a workgroup of the prefill kernel; each holds 1, 2 or 4 row tiles
-PREFILL_TWO_TILES_WORKGROUPS = 512      # two row tiles per wave while this many workgroups remain (two per compute unit)
-PREFILL_FOUR_TILES_WORKGROUPS = 2048    # four while this many remain,
-PREFILL_FOUR_TILES_HEAD_DIM = 64        # and only up to this head size (beyond it the accumulators crowd the registers)
+PREFILL_TWO_TILES_WORKGROUPS = 384      # two row tiles per wave while this many workgroups remain (1.5 per compute unit)
+PREFILL_FOUR_TILES_WORKGROUPS = 512     # four while this many remain,
+PREFILL_FOUR_TILES_HEAD_DIM = 64        # only up to this head size (beyond it the accumulators crowd the registers)
+PREFILL_FOUR_TILES_MEAN_KEYS = 4096     # and only where a row walks this many keys on average
 
 
-def prefill_tile_tokens(num_tokens: int, nkv: int, group: int, head_dim: int) -> int:
+def prefill_tile_tokens(num_tokens: int, nkv: int, group: int, head_dim: int, mean_keys: float = 0.0) -> int:
     """Tokens per tile of the prefill kernel. A wave that holds two or four row tiles works on them
     side by side and reads each key once for all of them, which is faster as long as the step still
-    makes enough workgroups to fill the chip (measured: 2,048 tokens over 6,144 cached ones at head
-    size 128 take 534 / 295 / 375 µs with 1 / 2 / 4 row tiles per wave; 512 tokens over 1,536 at
-    head size 64 take 36 / 46 / 66 µs; 16,384 tokens at head size 64 take 1.89 / 1.33 / 1.23 ms)."""
+    makes enough workgroups to fill the chip; four pay only for small heads over long contexts
+    (`mean_keys`: the keys a row of the step walks on average). Thresholds from a sweep over steps of
+    128 to 8,192 tokens, 0 to 6,144 cached tokens before them, head sizes 64 and 128 and groups of
+    3, 4 and 8 heads: e.g. 2,048 tokens over 6,144 cached ones at head size 128 take 484 / 272 / 333 µs
+    with 1 / 2 / 4 row tiles per wave, 512 tokens 161 / 181 / 267 µs; 4,096 tokens over 2,048 at
+    head size 64 take 246 / 220 / 190 µs."""
     per_wave = PREFILL_WAVES * (16 // group)
 
     def workgroups(rt: int) -> int:
         return -(-num_tokens // (rt * per_wave)) * nkv
 
-    if head_dim <= PREFILL_FOUR_TILES_HEAD_DIM and workgroups(4) >= PREFILL_FOUR_TILES_WORKGROUPS:
+    if (head_dim <= PREFILL_FOUR_TILES_HEAD_DIM and workgroups(4) >= PREFILL_FOUR_TILES_WORKGROUPS
+            and mean_keys >= PREFILL_FOUR_TILES_MEAN_KEYS):
         return 4 * per_wave
     if workgroups(2) >= PREFILL_TWO_TILES_WORKGROUPS:
         return 2 * per_wave
@@ -484,7 +489,9 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         while decode_ok and lead + 1 < len(cu) and cu[lead + 1] - cu[lead] == 1:
             lead += 1
         nkv = k_cache.shape[2]
-        tile_tokens = prefill_tile_tokens(q.shape[0] - lead, nkv, q.shape[1] // nkv, q.shape[2])
+        walked = sum((cu[i + 1] - cu[i]) * (ctx.host_starts[i] + (cu[i + 1] - cu[i] + 1) / 2) for i in range(lead, len(cu) - 1))
+        tile_tokens = prefill_tile_tokens(q.shape[0] - lead, nkv, q.shape[1] // nkv, q.shape[2],
+                                          walked / max(1, q.shape[0] - lead))
         tiles = ctx.scratch.get(("attention_tiles", tile_tokens, lead))
         if tiles is None:
             flat = attention_tiles(cu, ctx.host_starts, tile_tokens, lead)
