@@ -351,3 +351,43 @@ def test_awkward_sizes_run_in_both_precisions(tmp_path, hidden, inter, vocab, he
         got = torch.cat([first, rest]).double().cpu()
         spread = float(want.max() - want.min())
         assert float((got - want).abs().max()) <= tolerance * spread, f"{dtype}: {float((got - want).abs().max())} of {spread}"
+
+
+def test_small_portions_over_a_long_context_walk_the_keys_in_chunks(tmp_path):
+    """Behind 2,500 cached tokens the next portions are small: too few tiles to fill the chip, so
+    the bfloat16 attention kernel cuts each tile's keys into chunks and combines them. A portion of
+    60 alone, then one of 40 behind another request's decoded token (which goes to the decode
+    kernel in the same step), against the plain model over the whole prompt."""
+    from tinyserve_llm_amd.config import LlamaConfig
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.runner import StepEntry
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    from tinyserve_llm_amd.ops import hip
+    from tinyserve_llm_amd.weights.random_init import write_random_model
+    config = LlamaConfig(vocab_size=300, hidden_size=128, intermediate_size=192, num_hidden_layers=2,
+                         num_attention_heads=4, num_key_value_heads=2, head_dim=64, max_position_embeddings=4096,
+                         rms_norm_eps=1e-5, rope_theta=10000.0, rope_scaling=None, tie_word_embeddings=True,
+                         eos_token_id=299)
+    write_random_model(str(tmp_path), config, 5, torch.float32)
+    ids, other = prompt(11, 2600, 300), prompt(12, 31, 300)
+    assert hip.prefill_splits(2 * 2, 2560)[0] > 1, "the step below is one the plan cuts"
+    sc = SchedulerConfig(max_model_len=4096, max_num_seqs=4, max_num_batched_tokens=4096)
+    for dtype, tolerance in ((torch.float32, 2e-5), (torch.bfloat16, 3e-2)):
+        plain = PlainLlama(str(tmp_path), torch.float64, weights_as=None if dtype == torch.float32 else dtype)
+        want, want_other = plain.logits(ids), plain.logits(other)
+        llm = LLM(str(tmp_path), sc, CacheConfig(block_size=64), dtype=dtype, num_blocks=48)
+        llm.manager.allocate(0, ids[:2500])
+        llm.manager.allocate(1, other[:30])
+        llm.runner.step([StepEntry(0, ids[:2500], 0, []), StepEntry(1, other[:30], 0, [])])
+        llm.manager.commit(0, 2500)
+        llm.manager.commit(1, 30)
+        llm.manager.append_slots(0, ids[2500:2560])
+        alone = llm.runner.step([StepEntry(0, ids[2500:2560], 2500, list(range(60)))])
+        llm.manager.commit(0, 60)
+        llm.manager.append_slots(0, ids[2560:])
+        llm.manager.append_slots(1, other[30:])
+        mixed = llm.runner.step([StepEntry(1, other[30:], 30, [0]), StepEntry(0, ids[2560:], 2560, list(range(40)))])
+        got = torch.cat([alone, mixed[1:]]).double().cpu()
+        spread = float(want.max() - want.min())
+        assert float((got - want[2500:]).abs().max()) <= tolerance * spread, f"{dtype}: {float((got - want[2500:]).abs().max())} of {spread}"
+        assert float((mixed[0].double().cpu() - want_other[30]).abs().max()) <= tolerance * spread

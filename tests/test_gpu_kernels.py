@@ -703,6 +703,56 @@ def test_matrix_core_prefill_attention_over_a_long_prompt(heads, kv, hd, page, r
         torch.testing.assert_close(out.double().cpu(), want, **tol(dtype), msg=lambda m: f"window {window}: {m}")
 
 
+@pytest.mark.parametrize("heads,kv,hd,page,row_tiles", [(8, 2, 64, 64, 1), (4, 1, 128, 256, 2), (6, 6, 32, 16, 4),
+                                                       (14, 2, 96, 24, 1)])
+@pytest.mark.parametrize("splits,chunk", [(2, 1024), (5, 288), (7, 224), (3, 96), (64, 32)])
+def test_matrix_core_prefill_attention_with_the_keys_cut_into_chunks(heads, kv, hd, page, row_tiles, splits, chunk):
+    """Two one-token requests that are left alone, then a portion of 90 tokens over a cached prefix
+    of 1,357 and one of 41 tokens over 610, their keys walked in chunks: chunks that end inside the
+    cached prefix, inside the portion (where the causal masks are), chunks that lie wholly before a
+    window's start, chunks that a request does not reach, and chunks that together fall short of the
+    context (the last one takes the rest). One key far back carries most of one row's weight, so a
+    chunk that is dropped or weighted wrongly shows."""
+    dtype = torch.bfloat16
+    g = gen(hd + 7 * splits)
+    lens, fed = [50, 20, 1447, 651], [1, 1, 90, 41]
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev())
+    pages_each = [-(-n // page) for n in lens]
+    order = torch.randperm(sum(pages_each), generator=g).tolist()
+    kp = torch.randn(len(order), kv, page, hd, generator=g).to(dtype)
+    vp = torch.randn(len(order), kv, hd, page, generator=g).to(dtype)
+    qs, ks, vs, tables = [], [], [], []
+    for n, pe in zip(lens, pages_each):
+        table, order = order[:pe], order[pe:]
+        q = (torch.randn(n, heads, hd, generator=g) * 0.5).to(dtype)
+        k, v = (torch.randn(n, kv, hd, generator=g) * 0.5).to(dtype), torch.randn(n, kv, hd, generator=g).to(dtype)
+        if n > 1000:
+            k[3], q[n - 5] = k[3] * 6, q[n - 5].abs() * k[3].sign().repeat_interleave(heads // kv, 0)  # row n - 5 looks at key 3
+        for p_ in range(n):
+            kp[table[p_ // page], :, p_ % page] = k[p_]
+            vp[table[p_ // page], :, :, p_ % page] = v[p_]
+        qs.append(q), ks.append(k), vs.append(v), tables.append(table + [0] * (max(pages_each) - pe))
+    kc, vc = kp.to(dev()).permute(0, 2, 1, 3), vp.to(dev()).permute(0, 3, 1, 2)
+    q_step = torch.cat([qs[i][lens[i] - fed[i]:] for i in range(4)]).to(dev())
+    seq_of = sum(([i] * fed[i] for i in range(4)), [])
+    positions = sum((list(range(lens[i] - fed[i], lens[i])) for i in range(4)), [])
+    cu = [0, 1, 2, 92, 133]
+    per_tile = row_tiles * hip().PREFILL_WAVES * (16 // (heads // kv))
+    flat = hip().attention_tiles(cu, [lens[i] - fed[i] for i in range(4)], per_tile, 2)
+    for window in (0, 333):
+        out = torch.full_like(q_step, 7.0)
+        hip().paged_attention_prefill(q_step, kc, vc, i32(tables), i32(seq_of), i32(positions), i32(flat).view(-1, 2),
+                                      hd ** -0.5, window=window, tile_tokens=per_tile, out=out, num_splits=splits,
+                                      chunk=chunk, first_token=2)
+        assert out[:2].eq(7.0).all(), "the tokens before first_token belong to another kernel"
+        want = torch.cat([P.causal_attention(qs[i].double(), ks[i].double(), vs[i].double(), window=window)[lens[i] - fed[i]:]
+                          for i in (2, 3)])
+        torch.testing.assert_close(out[2:].double().cpu(), want, **tol(dtype), msg=lambda m: f"window {window}: {m}")
+    with pytest.raises(hip().KernelError, match="multiple of 32"):
+        hip().paged_attention_prefill(q_step, kc, vc, i32(tables), i32(seq_of), i32(positions), i32(flat).view(-1, 2),
+                                      hd ** -0.5, tile_tokens=per_tile, num_splits=2, chunk=100, first_token=2)
+
+
 @pytest.mark.parametrize("m", [1, 8, 16, 23])
 @pytest.mark.parametrize("n,k", [(3072, 2048), (16384, 2048), (992, 512), (130, 3072), (64, 4096), (2048, 8192)])
 def test_weight_streaming_gemm_reads_the_packed_copy_to_the_same_result(m, n, k):

@@ -45,6 +45,17 @@ def test_prefill_tile_tokens_keeps_the_chip_busy():
         assert hip.prefill_tile_tokens(tokens, nkv, group, 64, 5000.0) in (per_wave, 2 * per_wave, 4 * per_wave)
 
 
+def test_prefill_splits_cut_long_walks_of_few_tiles():
+    assert hip.prefill_splits(64, 6272) == (8, 800)            # 8 tiles for each of 8 heads over 6K keys
+    assert hip.prefill_splits(512, 6272) == (1, 0)             # enough tiles: uncut
+    assert hip.prefill_splits(64, 1500) == (1, 0)              # a short context: uncut
+    assert hip.prefill_splits(8, 2304) == (4, 576)             # chunks of at least 512 keys
+    for workgroups, longest in ((1, 100000), (300, 2048), (17, 5000), (2, 1 << 20), (1, 2049)):
+        splits, chunk = hip.prefill_splits(workgroups, longest)
+        assert splits == 1 or (chunk % 32 == 0 and splits * chunk >= longest and (splits - 1) * chunk < longest
+                               and splits <= hip.MAX_DECODE_SPLITS)
+
+
 def test_decode_plan_divides_the_context_into_32_key_steps_per_wave():
     for tokens in (1, 8, 64, 512):
         for nkv, group, hd in ((8, 4, 64), (1, 16, 128), (2, 3, 96), (5, 1, 32)):

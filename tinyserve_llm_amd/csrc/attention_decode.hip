@@ -138,7 +138,7 @@ attn_decode_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ p
   const int64_t th = blockIdx.x;
   const int pos = positions[t];
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int s0 = lo / chunk, s1 = pos / chunk;
+  const int s0 = min(lo / chunk, num_splits - 1), s1 = min(pos / chunk, num_splits - 1);  // the last chunk is open-ended
   const float* ml = part_ml + th * num_splits * 2;
   float M = -INFINITY;
   for (int s = s0 + lane; s <= s1; s += TS_WAVE) M = fmaxf(M, ml[2 * s]);
@@ -159,6 +159,16 @@ attn_decode_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ p
     for (int s = 0; s <= s1 - s0; ++s) acc = fmaf(po[(int64_t)s * hd + d], wgt[s], acc);
     out[th * hd + d] = f2bf(acc * inv);
   }
+}
+
+// The combining kernel alone, for the prefill kernel's split walks (declared in attention_mfma.h).
+int ts_launch_attention_combine(void* out, const float* part_o, const float* part_ml, const int32_t* positions,
+                                int num_tokens, int nh, int hd, int num_splits, int chunk, int window,
+                                hipStream_t stream) {
+  if (num_splits > COMBINE_MAX_SPLITS) return TS_BAD_SHAPE;
+  attn_decode_combine_kernel<<<num_tokens * nh, TS_WAVE, 0, stream>>>((bf16_t*)out, part_o, part_ml, positions, nh, hd,
+                                                                      num_splits, chunk, window);
+  return ts_check_launch();
 }
 
 // part_o [tokens, nh, num_splits, hd] and part_ml [tokens, nh, num_splits, 2] are float workspaces

@@ -194,3 +194,10 @@ static __device__ __forceinline__ void use_tile_auto(const KVTile<HD>& T, int kb
   if (kb + 31 <= pmin && kb >= lomax) use_tile<HD, false>(T, kb, r, g, lo, pos, qreg, scale2, m, l, o);
   else use_tile<HD, true>(T, kb, r, g, lo, pos, qreg, scale2, m, l, o);
 }
+
+// out[t, h, :] from the chunks' partial results part_o [tokens, nh, num_splits, hd] and part_ml
+// [tokens, nh, num_splits, 2] (reference maximum in units of log2, sum), over the chunks that hold
+// keys visible from positions[t] (defined in attention_decode.hip).
+int ts_launch_attention_combine(void* out, const float* part_o, const float* part_ml, const int32_t* positions,
+                                int num_tokens, int nh, int hd, int num_splits, int chunk, int window,
+                                hipStream_t stream);

@@ -7,8 +7,11 @@
 // registers, leaves them in LDS in the order the lanes use them, and all four waves read the whole
 // step back from there, two steps ahead of the loads in flight. A row masks the keys beyond its own
 // position (and before its window); steps that lie wholly inside every row's range skip the masks.
-// Nothing is split and nothing is combined: a row's sums run over the keys in ascending order,
-// whatever the batch.
+// Normally nothing is split and nothing is combined: a row's sums run over the keys in ascending
+// order, whatever the batch. A step of few tokens over a long context has too few tiles to fill the
+// chip: then the keys are cut into chunks (num_splits > 1), a workgroup walks one chunk for its
+// tile and leaves the rows' partial results (part_o, part_ml, as the decode kernel does), and the
+// decode kernel's combining kernel sums the chunks in ascending order.
 //
 // The host lists the tiles: tiles[2 i] = index of the tile's first token in the step,
 // tiles[2 i + 1] = number of its tokens (at most 4 RT (16 / G), all of one request), in ascending
@@ -35,7 +38,8 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
              const int32_t* __restrict__ block_tables, const int32_t* __restrict__ seq_of_token,
              const int32_t* __restrict__ positions, const int32_t* __restrict__ tiles, int nh, int G, int page_size,
              int page_shift, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
-             float scale2, int window) {
+             float scale2, int window, float* __restrict__ part_o, float* __restrict__ part_ml, int num_splits,
+             int chunk, int split) {
   constexpr int NC = HD / 32, NDB = HD / 16;   // operand registers of a 32-key step: 2 NC of K, NDB of V
   auto& stage = lds.stage;
   auto& wg_range = lds.range;
@@ -94,6 +98,17 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
   for (int w = 1; w < PRE_WAVES; ++w) {
     wlo = min(wlo, wg_range[0][w]); whi = max(whi, wg_range[1][w]);
     wfull_hi = min(wfull_hi, wg_range[2][w]); wfull_lo = max(wfull_lo, wg_range[3][w]);
+  }
+  if (num_splits > 1) {
+    // this workgroup walks one chunk of the keys only (chunks are multiples of 32 keys, so no step
+    // straddles two); what the rows see of it is combined with the other chunks afterwards
+    // (the last chunk has no upper end, so every position is in some chunk whatever the caller chose)
+    wlo = max(wlo, split * chunk);
+    wfull_lo = max(wfull_lo, split * chunk);
+    if (split + 1 < num_splits) {
+      whi = min(whi, split * chunk + chunk - 1);
+      if (wfull_hi != 0x7fffffff) wfull_hi = min(wfull_hi, split * chunk + chunk - 1);
+    }
   }
   // every lane holds the same values: say so, and loop control and page lookups become scalar
   wlo = __builtin_amdgcn_readfirstlane(wlo);
@@ -235,6 +250,17 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
       const int row = 4 * g + i;
       const float lj = __shfl(lsum[j], row, TS_WAVE);
       const int rtk = (wave * RT + j) * tpt + row / G, rhh = row % G;
+      if (num_splits > 1) {
+        // the chunk's share of the row, not normalised: sums, and the reference maximum they are relative to
+        const float mj = __shfl(m[j], row, TS_WAVE);
+        if (row / G < tpt && rtk < ntok) {
+          const int64_t at = (((int64_t)(t0 + rtk) * nh + (int64_t)kvh * G + rhh) * num_splits + split);
+#pragma unroll
+          for (int db = 0; db < NDB; ++db) part_o[at * HD + 16 * db + r] = o[j][db][i];
+          if (r == 0) { part_ml[at * 2] = mj; part_ml[at * 2 + 1] = lj; }
+        }
+        continue;
+      }
       if (row / G < tpt && rtk < ntok && lj > 0.f) {
         const float inv = 1.0f / lj;
         bf16_t* orow = out + ((int64_t)(t0 + rtk) * nh + (int64_t)kvh * G + rhh) * HD;
@@ -251,7 +277,8 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
                          const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ positions,
                          const int32_t* __restrict__ tiles, int num_tiles, int nh, int G, int dies_per_group,
                          int heads_per_group, int page_size, int page_shift, int64_t kp, int64_t ks, int64_t kh,
-                         int64_t vp, int64_t vh, int64_t vd, int max_blocks, float scale2, int window) {
+                         int64_t vp, int64_t vh, int64_t vd, int max_blocks, float scale2, int window,
+                         float* __restrict__ part_o, float* __restrict__ part_ml, int num_splits, int chunk) {
   __shared__ PrefillLds<HD> lds;
   // die = workgroup index mod 8. The dies form `groups` groups of `dies_per_group`, the heads as
   // many groups of `heads_per_group`; a group's (tile, head) pairs go round its dies, long tiles first.
@@ -261,19 +288,27 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
   const int tile = num_tiles - 1 - item / heads_per_group;
   const int kvh = (die / dies_per_group) * heads_per_group + item % heads_per_group;
   prefill_tile<HD, RT>(lds, tile, kvh, out, q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, nh,
-                       G, page_size, page_shift, kp, ks, kh, vp, vh, vd, max_blocks, scale2, window);
+                       G, page_size, page_shift, kp, ks, kh, vp, vh, vd, max_blocks, scale2, window, part_o, part_ml,
+                       num_splits, chunk, blockIdx.y);
 }
 
 // Keys: rows dense in head_dim, strides kp/ks/kh (page, slot, head). Values: transposed pages,
 // slot stride 1, strides vp/vh/vd (page, head, dimension). tile_tokens: the most tokens a listed
-// tile holds, 4 RT (16 / G) for RT of 1, 2 or 4.
+// tile holds, 4 RT (16 / G) for RT of 1, 2 or 4. num_splits > 1: chunk (a multiple of 32; the last chunk
+// takes every key from its start on) and the float workspaces part_o [num_tokens, nh, num_splits, hd] and
+// part_ml [num_tokens, nh, num_splits, 2]; every token from first_token on must then be in a tile (the ones
+// before it keep what `out` held).
 extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* k_cache, const void* v_cache,
                                           const int32_t* block_tables, const int32_t* seq_of_token,
                                           const int32_t* positions, const int32_t* tiles, int num_tiles,
                                           int tile_tokens, int nh, int nkv, int hd, int page_size, int64_t kp,
                                           int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
-                                          float scale, int window, hipStream_t stream) {
+                                          float scale, int window, int first_token, int num_tokens, int num_splits,
+                                          int chunk, float* part_o, float* part_ml, hipStream_t stream) {
   if (num_tiles <= 0) return TS_OK;
+  if (num_splits < 1 || num_splits > 65535) return TS_BAD_SHAPE;
+  if (num_splits > 1 && (chunk <= 0 || chunk % 32 || !part_o || !part_ml || first_token < 0 || num_tokens <= first_token))
+    return TS_BAD_SHAPE;
   if (nkv <= 0 || nh % nkv || page_size <= 0 || page_size % 8 || max_blocks <= 0) return TS_BAD_SHAPE;
   const int G = nh / nkv;
   if (G > 16) return TS_BAD_SHAPE;
@@ -292,12 +327,12 @@ extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* 
   const int dies_per_group = 8 / groups, heads_per_group = nkv / groups;
   const int64_t turns = ((int64_t)num_tiles * heads_per_group + dies_per_group - 1) / dies_per_group;
   if (turns * 8 > 0x7fffffff) return TS_BAD_SHAPE;
-  dim3 grid((unsigned)(8 * turns));
+  dim3 grid((unsigned)(8 * turns), num_splits);
 #define TS_PRE(HH, RR)                                                                                          \
   attn_prefill_mfma_kernel<HH, RR><<<grid, PRE_WAVES * TS_WAVE, 0, stream>>>(                                   \
       (bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,             \
       seq_of_token, positions, tiles, num_tiles, nh, G, dies_per_group, heads_per_group, page_size, page_shift, kp,  \
-      ks, kh, vp, vh, vd, max_blocks, scale * 1.44269504088896340736f, window)
+      ks, kh, vp, vh, vd, max_blocks, scale * 1.44269504088896340736f, window, part_o, part_ml, num_splits, chunk)
 #define TS_PRE_RT(HH)                                                                                           \
   if (rt == 1) TS_PRE(HH, 1); else if (rt == 2) TS_PRE(HH, 2); else TS_PRE(HH, 4)
   switch (hd) {
@@ -309,5 +344,10 @@ extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* 
   }
 #undef TS_PRE_RT
 #undef TS_PRE
-  return ts_check_launch();
+  const int rc = ts_check_launch();
+  if (rc || num_splits == 1) return rc;
+  const int64_t skip = (int64_t)first_token * nh;     // rows of the tokens before the first listed one
+  return ts_launch_attention_combine((bf16_t*)out + skip * hd, part_o + skip * num_splits * hd,
+                                     part_ml + skip * num_splits * 2, positions + first_token,
+                                     num_tokens - first_token, nh, hd, num_splits, chunk, window, stream);
 }

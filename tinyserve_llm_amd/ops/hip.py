@@ -55,7 +55,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_sample": [p, p, p, p, p, p, u64, i, i, i64, p],
         "ts_gemm_library_bf16": [p, p, p, i, i, i, i64, i64, i64, i, p, ctypes.c_size_t, p],
         "ts_gemm_library_init": [],
-        "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, p],
+        "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, i, i, i, i, p, p, p],
         "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p],
         "ts_gemm_skinny_rope_bf16": [p, p, p, p, p, p, i, i, i64, i64, f, i, i, p, p, p, p, p, i, i, i, i, i, i64, i64, i64,
                                      i64, i64, i64, i64, p],
@@ -420,6 +420,29 @@ def prefill_tile_tokens(num_tokens: int, nkv: int, group: int, head_dim: int, me
     return per_wave
 
 
+PREFILL_SPLIT_BELOW_WORKGROUPS = 384    # a step whose tiles make fewer workgroups than this may cut its keys into chunks
+PREFILL_SPLIT_TARGET_WORKGROUPS = 512   # so that about this many workgroups walk them,
+PREFILL_SPLIT_MIN_CHUNK = 512           # each at least this many keys
+PREFILL_SPLIT_MIN_CONTEXT = 2048        # if the longest context reaches this
+
+
+def prefill_splits(workgroups: int, longest: int) -> tuple[int, int]:
+    """(number of chunks, keys per chunk) for the prefill kernel's key walk; (1, 0) where it is not
+    cut. Few tokens over a long context (a short new turn behind a cached conversation, a small
+    portion of a long prompt) make too few tiles to fill the chip and each walks thousands of keys:
+    128 tokens over 6,144 cached ones take 153 µs uncut and 42 µs in 8 chunks (heads of 128), 256
+    tokens of a single key/value head over 8,000 take 193 µs and 36 µs in 16. `workgroups` is
+    tiles times key/value heads, `longest` the longest context of the step's portions (the last chunk
+    takes whatever lies beyond the others, so an estimate that is too low costs balance only)."""
+    if workgroups >= PREFILL_SPLIT_BELOW_WORKGROUPS or longest < PREFILL_SPLIT_MIN_CONTEXT:
+        return 1, 0
+    splits = min(-(-PREFILL_SPLIT_TARGET_WORKGROUPS // max(1, workgroups)), longest // PREFILL_SPLIT_MIN_CHUNK, MAX_DECODE_SPLITS)
+    if splits < 2:
+        return 1, 0
+    chunk = -(-longest // (splits * 32)) * 32
+    return -(-longest // chunk), chunk
+
+
 def attention_tiles(cu_seqlens: list[int], starts: list[int], tokens_per_tile: int, first_seq: int = 0) -> list[int]:
     """Tiles of a packed step for the matrix-core prefill kernel: (first token, token count) pairs,
     flattened, for the requests from `first_seq` on. A tile never crosses a request; `starts[s]` is
@@ -440,13 +463,17 @@ def attention_tiles(cu_seqlens: list[int], starts: list[int], tokens_per_tile: i
 
 def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                             seq_of_token: torch.Tensor, positions: torch.Tensor, tiles: torch.Tensor, scale: float,
-                            window: int = 0, tile_tokens: int | None = None, out: torch.Tensor | None = None
-                            ) -> torch.Tensor:
+                            window: int = 0, tile_tokens: int | None = None, out: torch.Tensor | None = None,
+                            num_splits: int = 1, chunk: int = 0, first_token: int = 0) -> torch.Tensor:
     """Attention of a packed step on the matrix cores (bfloat16, values in transposed pages).
     `tiles` int32 [num_tiles, 2] lists (first token, token count <= tile_tokens) per workgroup,
     every tile inside one request and inside the step (the caller built the list from the step's
     own lengths and has checked positions against the block tables), long tiles last; `tile_tokens`
-    is 4, 8 or 16 times 16 // group (default 4 times). Tokens that no tile lists keep what `out` held."""
+    is 4, 8 or 16 times 16 // group (default 4 times). Tokens that no tile lists keep what `out` held.
+    With `num_splits` > 1 every tile's keys are walked in that many chunks of `chunk` keys (a
+    multiple of 32; the last takes every key from its start on) by workgroups of their own, and the
+    chunks are combined afterwards: for steps of few tokens over long contexts, which have too few
+    tiles to fill the chip. The tiles must then list every token from `first_token` on."""
     _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles)
     _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
     T, nh, hd = q.shape
@@ -465,10 +492,17 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     tile_tokens = tile_tokens or per_wave
     _need(tile_tokens in (per_wave, 2 * per_wave, 4 * per_wave), f"tiles of {tile_tokens} tokens; {per_wave}, twice or four times that")
     out = _out_like(q, out)
+    part_o = part_ml = None
+    if num_splits > 1:
+        _need(chunk > 0 and chunk % 32 == 0 and 0 <= first_token < T, "chunks of a multiple of 32 keys, from a token of the step on")
+        _need(num_splits <= MAX_DECODE_SPLITS, f"at most {MAX_DECODE_SPLITS} chunks")
+        part_o = torch.empty((T, nh, num_splits, hd), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((T, nh, num_splits, 2), dtype=torch.float32, device=q.device)
     _run("paged_attention_prefill", library().ts_paged_attention_prefill(
         _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_of_token), _ptr(positions),
         _ptr(tiles), tiles.shape[0], tile_tokens, nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3], v_cache.stride(0),
-        v_cache.stride(2), v_cache.stride(3), block_tables.shape[1], float(scale), int(window), _stream()))
+        v_cache.stride(2), v_cache.stride(3), block_tables.shape[1], float(scale), int(window), first_token, T,
+        num_splits, chunk, _ptr(part_o), _ptr(part_ml), _stream()))
     return out
 
 
@@ -501,8 +535,10 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         if lead:
             paged_attention_decode(q[:lead], k_cache, v_cache, tables, ctx.seq_of_token[:lead], ctx.positions[:lead],
                                    scale, window, out=out[:lead])
+        splits, chunk = prefill_splits(tiles.shape[0] * nkv, max(ctx.host_context_lens[lead:]))
         return paged_attention_prefill(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, tiles, scale,
-                                       window, tile_tokens=tile_tokens, out=out)
+                                       window, tile_tokens=tile_tokens, out=out, num_splits=splits, chunk=chunk,
+                                       first_token=cu[lead])
     return paged_attention_wave(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, window)
 
 
