@@ -38,6 +38,78 @@ def test_trie_insert_of_a_longer_run_extends_the_old_path():
     assert not trie.root.next
 
 
+class PerTokenTrie:
+    """One node per token, as the reference keeps it (tinyserve_llm/kvcache/trie.py:9-68): the
+    meaning that the trie's edges of several tokens must keep."""
+
+    def __init__(self):
+        self.root = ({}, set())
+
+    def insert(self, page, tokens):
+        at = self.root
+        for tok in tokens:
+            at = at[0].setdefault(tok, ({}, set()))
+            at[1].add(page)
+
+    def remove(self, page, tokens):
+        at = self.root
+        for tok in tokens:
+            nxt = at[0][tok]
+            nxt[1].remove(page)
+            if not nxt[1]:
+                del at[0][tok]
+                return
+            at = nxt
+
+    def longest_match(self, tokens):
+        at, depth = self.root, 0
+        for tok in tokens:
+            if tok not in at[0]:
+                break
+            at, depth = at[0][tok], depth + 1
+        return depth, at[1]
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_trie_with_edges_of_several_tokens_answers_as_one_node_per_token_does(seed):
+    """Random inserts, extensions, removals and lookups over a small alphabet, so that runs share
+    prefixes, end inside each other and split each other's edges."""
+    import random
+    rng = random.Random(seed)
+    trie, plain, runs = TokenTrie(), PerTokenTrie(), {}
+    for step in range(600):
+        what = rng.random()
+        if what < 0.4 or not runs:
+            page, run = object(), [rng.randrange(3) for _ in range(rng.randint(1, 9))]
+            runs[page] = run
+            trie.insert(page, run), plain.insert(page, run)
+        elif what < 0.55:
+            page = rng.choice(list(runs))
+            runs[page] = runs[page] + [rng.randrange(3) for _ in range(rng.randint(1, 4))]
+            trie.insert(page, runs[page]), plain.insert(page, runs[page])
+        elif what < 0.8:
+            page = rng.choice(list(runs))
+            run = runs.pop(page)
+            trie.remove(page, run), plain.remove(page, run)
+        probe = tuple(rng.randrange(3) for _ in range(rng.randint(0, 12)))
+        assert trie.longest_match(probe) == plain.longest_match(probe), f"step {step}: {probe}"
+        for page, run in runs.items():
+            depth, pages = trie.longest_match(run)
+            assert depth == len(run) and page in pages
+    for page, run in list(runs.items()):
+        trie.remove(page, run)
+    assert not trie.root.next and not trie.root.pages
+
+
+def test_a_page_that_shares_nothing_is_one_edge():
+    trie, p, q = TokenTrie(), object(), object()
+    trie.insert(p, list(range(256)))
+    assert len(trie.root.next) == 1 and not trie.root.next[0].next
+    trie.insert(q, list(range(100)) + [7])
+    upper = trie.root.next[0]
+    assert len(upper.label) == 100 and upper.pages == {p, q} and set(upper.next) == {100, 7}
+
+
 def test_publish_returns_the_twin_on_a_duplicate():
     t = PageTree(B)
     a = t.publish(t.root, 1, FULL)

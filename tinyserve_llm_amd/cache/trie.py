@@ -1,6 +1,12 @@
 """A trie over the token runs of one page's child pages, for token-granular prefix lookup
-(tinyserve_llm/kvcache/trie.py:9-68). A trie node remembers every child page whose tokens pass
-through it, so the deepest node reached names all pages that share the matched run."""
+(tinyserve_llm/kvcache/trie.py:9-68). A position in the trie remembers every child page whose
+tokens pass through it, so the deepest position reached names all pages that share the matched run.
+
+Runs of tokens that no other page leaves are kept as one edge (a page of 256 tokens that shares
+nothing with its siblings is one node, not 256): an edge carries its tokens as a tuple and the set
+of pages that pass through it, and every page that enters an edge reaches its end, because a run
+that ends inside an edge splits the edge there. All positions inside an edge therefore see the same
+pages, the set of the node at the edge's end."""
 
 from __future__ import annotations
 
@@ -8,11 +14,23 @@ from typing import Hashable, Iterable, Sequence
 
 
 class _Node:
-    __slots__ = ("next", "pages")
+    __slots__ = ("label", "next", "pages")
 
-    def __init__(self) -> None:
-        self.next: dict[int, _Node] = {}
-        self.pages: set = set()
+    def __init__(self, label: tuple[int, ...] = (), pages: set | None = None) -> None:
+        self.label = label                       # the tokens from the parent to here; empty for the root only
+        self.next: dict[int, _Node] = {}         # first token of an edge -> the node at its end
+        self.pages: set = set() if pages is None else pages
+
+
+def _shared(label: tuple[int, ...], tokens: tuple[int, ...], at: int) -> int:
+    """How many leading tokens of `label` equal tokens[at:]."""
+    n = min(len(label), len(tokens) - at)
+    if tokens[at:at + n] == label[:n]:
+        return n
+    m = 0
+    while label[m] == tokens[at + m]:
+        m += 1
+    return m
 
 
 class TokenTrie:
@@ -21,37 +39,56 @@ class TokenTrie:
     def __init__(self) -> None:
         self.root = _Node()
 
+    @staticmethod
+    def _split(parent: _Node, node: _Node, m: int) -> _Node:
+        """Cuts the edge into `node` after m of its tokens; returns the new node at the cut."""
+        upper = _Node(node.label[:m], set(node.pages))
+        node.label = node.label[m:]
+        upper.next[node.label[0]] = node
+        parent.next[upper.label[0]] = upper
+        return upper
+
     def insert(self, page: Hashable, tokens: Sequence[int]) -> None:
         """Records `page` along the path of `tokens`. Inserting a longer run of a page already
         present walks its old path again (adding nothing there) and extends it."""
         if not tokens:
             raise AssertionError("a page in the trie holds at least one token")
-        at = self.root
-        for tok in tokens:
-            nxt = at.next.get(tok)
+        run = tuple(tokens)
+        at, i = self.root, 0
+        while i < len(run):
+            nxt = at.next.get(run[i])
             if nxt is None:
-                nxt = at.next[tok] = _Node()
+                at.next[run[i]] = _Node(run[i:], {page})
+                return
+            m = _shared(nxt.label, run, i)
+            if m < len(nxt.label):           # the run leaves the edge, or ends inside it
+                nxt = self._split(at, nxt, m)
             nxt.pages.add(page)
-            at = nxt
+            at, i = nxt, i + m
 
     def remove(self, page: Hashable, tokens: Sequence[int]) -> None:
-        """Takes `page` off its path and prunes the part of the path nobody else uses."""
-        at = self.root
-        for tok in tokens:
-            nxt = at.next[tok]
+        """Takes `page` off its path (`tokens` is the run it was last inserted with) and prunes
+        the part of the path nobody else uses."""
+        at, i = self.root, 0
+        while i < len(tokens):
+            nxt = at.next[tokens[i]]
             nxt.pages.remove(page)
             if not nxt.pages:
-                del at.next[tok]   # everything below belonged to this page alone
+                del at.next[tokens[i]]   # everything below belonged to this page alone
                 return
-            at = nxt
+            at, i = nxt, i + len(nxt.label)
 
     def longest_match(self, tokens: Iterable[int]) -> tuple[int, set]:
-        """(number of leading tokens found, the pages at the deepest node). The set is the trie's
-        own: read it, do not change it."""
+        """(number of leading tokens found, the pages at the deepest position). The set is the
+        trie's own: read it, do not change it."""
+        run = tokens if isinstance(tokens, tuple) else tuple(tokens)
         at, depth = self.root, 0
-        for tok in tokens:
-            nxt = at.next.get(tok)
+        while depth < len(run):
+            nxt = at.next.get(run[depth])
             if nxt is None:
                 break
-            at, depth = nxt, depth + 1
+            m = _shared(nxt.label, run, depth)
+            if m < len(nxt.label):
+                return depth + m, nxt.pages
+            at, depth = nxt, depth + m
         return depth, at.pages
