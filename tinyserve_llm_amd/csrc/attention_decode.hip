@@ -1,7 +1,7 @@
 // Split-key paged attention on the matrix cores for tokens that each bring one query (decoding),
 // bfloat16. A workgroup takes one (token, key/value head, chunk of keys) and serves all query heads
-// of that key/value head's group; its waves (up to 8, or 4 for heads wider than 64) take an equal
-// share of the chunk each and work through it 32 keys at a time:
+// of that key/value head's group; its waves (up to 8, or 4 for heads wider than 64) take the chunk's
+// 32-key steps in turn:
 //     S^T[key, head] = K[key, :] · Q[head, :]      v_mfma_f32_16x16x32_bf16, keys as rows
 //     online softmax per head (32-bit), P = 2^(S - m)
 //     O[head, :]    += P[head, key] · V[key, :]
@@ -60,12 +60,13 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, fl
 #pragma unroll
   for (int db = 0; db < NDB; ++db) o[db] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
-  // this wave's keys, 32 at a time; the next step's loads are issued before this step's products
-  const int kpw = chunk / nw;
-  int kb = k0 + wave * kpw;
-  int kend = kb + kpw;
+  // the chunk's visible keys, 32 at a time, dealt to the waves in turn (however few keys a request
+  // has in the chunk, every wave gets its share of them, and the workgroup reads the chunk front to
+  // back); the next step's loads are issued before this step's products
+  const int stride = 32 * nw;
+  int kend = k0 + chunk;
   if (kend > pos + 1) kend = pos + 1;
-  if (kb < (lo & ~31)) kb = lo & ~31;
+  int kb = (k0 > (lo & ~31) ? k0 : (lo & ~31)) + 32 * wave;
 #define TS_LOAD(T, KB) load_tile<HD>(T, KB, r, g, lo, pos, kvh, table, pm, k_cache, v_cache, kp, ks, kh, vp, vh, vd)
 #define TS_USE(T, KB) use_tile_auto<HD>(T, KB, r, g, lo, pos, pos, lo, qreg, scale2, m, l, o)
   if (ONE) {
@@ -78,16 +79,16 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, fl
     KVTile<HD> A, B;
     TS_LOAD(A, kb);
     while (true) {
-      const bool more_b = kb + 32 < kend;
-      if (more_b) TS_LOAD(B, kb + 32);
+      const bool more_b = kb + stride < kend;
+      if (more_b) TS_LOAD(B, kb + stride);
       TS_USE(A, kb);
       if (!more_b) break;
-      kb += 32;
-      const bool more_a = kb + 32 < kend;
-      if (more_a) TS_LOAD(A, kb + 32);
+      kb += stride;
+      const bool more_a = kb + stride < kend;
+      if (more_a) TS_LOAD(A, kb + stride);
       TS_USE(B, kb);
       if (!more_a) break;
-      kb += 32;
+      kb += stride;
     }
   }
 #undef TS_LOAD
@@ -173,7 +174,7 @@ int ts_launch_attention_combine(void* out, const float* part_o, const float* par
 
 // part_o [tokens, nh, num_splits, hd] and part_ml [tokens, nh, num_splits, 2] are float workspaces
 // (unused and may be null when num_splits is 1). num_splits * chunk must cover every position that
-// `positions` holds; a workgroup has `waves` waves, each with chunk / waves keys, a multiple of 32. (Letting the last workgroup
+// `positions` holds; a workgroup has `waves` waves that take the chunk's 32-key steps in turn (chunk is a multiple of 32 waves). (Letting the last workgroup
 // of a token combine its chunks inside the first kernel was tried and is slower: on a GPU of several
 // dies the device-scope fences it needs write back and invalidate each die's L2.) Keys: rows dense in
 // head_dim, strides kp/ks/kh (page, slot, head). Values: transposed pages, slot stride 1, strides
