@@ -183,6 +183,20 @@ def test_decodes_go_first_and_portions_share_what_is_left():
     assert [(len(b.token_ids), b.num_samples) for b in batch] == [(1, 1), (6, 0), (5, 1)]
 
 
+def test_a_steps_decodes_come_longest_context_first():
+    """Who decodes in a step is a matter of rank; inside the step the decoding requests are laid
+    out by the length of their contexts, which is the order the attention kernel starts them in."""
+    s = make(pages=64, max_num_batched_tokens=72, max_num_seqs=8)
+    for n, at in ((5, 0.0), (23, 0.1), (2, 0.2), (14, 0.3)):
+        s.add_request(list(range(2, 2 + n)), SamplingParams(max_tokens=6, ignore_eos=True), at)
+    run_step(s, 0.4)
+    for now in (0.5, 0.6):
+        batch, _ = run_step(s, now)
+        assert all(len(b.token_ids) == 1 for b in batch) and len(batch) == 4
+        assert [b.start for b in batch] == sorted((b.start for b in batch), reverse=True)
+        assert [len(b.seq.prompt_token_ids) for b in batch] == [23, 14, 5, 2]
+
+
 def test_portions_and_whole_prompts_generate_the_same():
     prompts = [[2 + (i * 7 + j) % 6 for j in range(n)] for i, n in enumerate((30, 3, 17, 45, 9))]
     params = SamplingParams(max_tokens=6, ignore_eos=True)
