@@ -406,7 +406,8 @@ def test_linear_bfloat16(m, n, k):
     assert f.dtype == torch.float32
 
 
-@pytest.mark.parametrize("m,n,k", [(33, 384, 96), (2056, 16384, 2048), (100, 1000, 160), (257, 130, 3072), (64, 128256, 512)])
+@pytest.mark.parametrize("m,n,k", [(33, 384, 96), (2056, 16384, 2048), (100, 1000, 160), (257, 130, 3072), (64, 128256, 512),
+                                   (777, 2048, 8192), (2063, 4096, 1024)])
 def test_library_product_called_directly(m, n, k):
     """x · W^T through the vendor's library with the algorithm kept per shape: against 64-bit, twice
     (the second call takes the kept plan), and with rows of x that lie apart in memory."""
@@ -420,7 +421,8 @@ def test_library_product_called_directly(m, n, k):
         out = hip().gemm_library(dense, wd)
         assert out.dtype == torch.bfloat16 and out.shape == (m, n)
         torch.testing.assert_close(out.double().cpu(), want, **tolerance)
-    torch.testing.assert_close(hip().gemm_library(ad[:, :k], wd).float(), out.float(), rtol=0, atol=0)
+    # rows that lie apart are a shape of their own, which may keep another algorithm (another order of sums)
+    torch.testing.assert_close(hip().gemm_library(ad[:, :k], wd).double().cpu(), want, **tolerance)
     with pytest.raises(hip().KernelError):
         hip().gemm_library(ad.t()[:k].t()[:, ::2], wd[:, ::2])      # elements of a row must be adjacent
 

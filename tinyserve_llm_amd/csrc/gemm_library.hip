@@ -9,10 +9,18 @@
 // 15.5), so a caller may ask for such a shape to be tuned: every candidate is timed on the call's
 // own operands, with the caches swept in between as they are when a step reads each weight once,
 // and the fastest is kept.
+// For products with many rows the heuristic's choice depends on the row count in a way the work does
+// not: at the layer sizes of an 8B Llama, 2,048 rows take 761 µs for a layer's four products and
+// 2,063 rows (a prompt portion beside fifteen decoding requests) 865 µs, the down projection alone
+// 209 and 357; 4,096 rows 1,167 µs and 4,127 rows 1,711. So a shape of more than 256 rows that is
+// no multiple of 256 also tries the algorithms the heuristic picks for the multiples of 256 below
+// and above it, where the library supports them for the shape, and keeps the fastest of the three
+// (timed once, at the shape's first call outside a capture, on that call's operands).
 // Row-major y = x · W^T is, in the library's column-major terms, y^T = W^T-as-stored transposed
 // times x^T-as-stored: A = W with op T (K x N, leading dimension ldw), B = x with op N (K x M,
 // leading dimension ldx), D = y (N x M, leading dimension ldy).
 #include <hipblaslt/hipblaslt.h>
+#include <hipblaslt/hipblaslt-ext.hpp>
 
 #include <map>
 #include <mutex>
@@ -31,6 +39,7 @@ constexpr int LT_TUNE_MIN_ROWS = 9;                // shapes with fewer rows kee
 constexpr int LT_TUNE_MAX_ROWS = 256;              // and so do shapes with more (the first candidate was the fastest)
 constexpr int LT_TUNE_RUNS = 2;                    // timed runs per candidate; the faster counts
 constexpr int LT_GRAPH_MAX_ROWS = 1024;            // the most rows of a step that may be recorded into a graph
+constexpr int LT_BORROW_ROWS = 256;                // shapes beyond the tuned ones borrow from the multiples of this many rows
 
 struct LtPlan {
   hipblasLtMatmulDesc_t desc = nullptr;
@@ -38,6 +47,11 @@ struct LtPlan {
   hipblasLtMatmulAlgo_t algo;
   size_t workspace = 0;
   bool tuned = false;
+  // algorithms picked for neighbouring row counts that also serve this shape, until one of them
+  // or `algo` has been chosen by timing
+  int borrowed = 0;
+  hipblasLtMatmulAlgo_t other[2];
+  size_t other_workspace[2] = {0, 0};
 };
 
 struct LtDevice {
@@ -48,6 +62,51 @@ struct LtDevice {
 
 std::mutex lt_mutex;
 LtDevice lt_devices[LT_MAX_DEVICES];
+
+// The first of the library's candidates for these layouts that fits the workspace (they come best
+// first, whatever workspace they want). Shapes that a recorded decode step may hold take a candidate
+// without workspace if there is one: an algorithm that clears its workspace would put a memory-set
+// node into the graph.
+bool lt_first(LtDevice& dev, hipblasLtMatmulDesc_t desc, hipblasLtMatrixLayout_t a, hipblasLtMatrixLayout_t b,
+              hipblasLtMatrixLayout_t d, int M, hipblasLtMatmulAlgo_t* algo, size_t* workspace) {
+  hipblasLtMatmulPreference_t pref = nullptr;
+  if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return false;
+  const uint64_t limit = LT_WORKSPACE_BYTES;
+  bool ok = hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &limit, sizeof(limit)) == HIPBLAS_STATUS_SUCCESS;
+  hipblasLtMatmulHeuristicResult_t found[LT_CANDIDATES];
+  int count = 0, pick = -1;
+  ok = ok && hipblasLtMatmulAlgoGetHeuristic(dev.handle, desc, a, b, d, d, pref, LT_CANDIDATES, found, &count) == HIPBLAS_STATUS_SUCCESS;
+  for (int i = 0; ok && M <= LT_GRAPH_MAX_ROWS && i < count && pick < 0; ++i)
+    if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize == 0) pick = i;
+  for (int i = 0; ok && i < count && pick < 0; ++i)
+    if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize <= LT_WORKSPACE_BYTES) pick = i;
+  hipblasLtMatmulPreferenceDestroy(pref);
+  if (!ok || pick < 0) return false;
+  *algo = found[pick].algo;
+  *workspace = found[pick].workspaceSize;
+  return true;
+}
+
+// What the heuristic picks for `rows` rows of the plan's shape, if the library supports it for the
+// plan's own row count too (within the workspace, and without one where the shape may be recorded).
+void lt_borrow(LtDevice& dev, LtPlan& plan, int M, int N, int K, int64_t ldx, int64_t ldy, int rows) {
+  hipblasLtMatrixLayout_t b = nullptr, d = nullptr;
+  hipblasLtMatmulAlgo_t algo;
+  size_t workspace = 0;
+  const float one = 1.0f, zero = 0.0f;
+  if (hipblasLtMatrixLayoutCreate(&b, HIP_R_16BF, K, rows, ldx) == HIPBLAS_STATUS_SUCCESS &&
+      hipblasLtMatrixLayoutCreate(&d, HIP_R_16BF, N, rows, ldy) == HIPBLAS_STATUS_SUCCESS &&
+      lt_first(dev, plan.desc, plan.a, b, d, M, &algo, &workspace) &&
+      hipblaslt_ext::matmulIsAlgoSupported(dev.handle, plan.desc, &one, plan.a, plan.b, &zero, plan.d, plan.d, algo,
+                                           workspace) == HIPBLAS_STATUS_SUCCESS &&
+      workspace <= LT_WORKSPACE_BYTES && (M > LT_GRAPH_MAX_ROWS || workspace == 0)) {
+    plan.other[plan.borrowed] = algo;
+    plan.other_workspace[plan.borrowed] = workspace;
+    ++plan.borrowed;
+  }
+  if (b) hipblasLtMatrixLayoutDestroy(b);
+  if (d) hipblasLtMatrixLayoutDestroy(d);
+}
 
 // The plan for a shape on the current device; made (and the library asked for its best algorithm)
 // the first time the shape is met. Returns null if the library has nothing for it.
@@ -73,25 +132,12 @@ LtPlan* lt_plan(LtDevice& dev, int M, int N, int K, int64_t ldx, int64_t ldw, in
   ok = ok && hipblasLtMatrixLayoutCreate(&plan.a, HIP_R_16BF, K, N, ldw) == HIPBLAS_STATUS_SUCCESS;
   ok = ok && hipblasLtMatrixLayoutCreate(&plan.b, HIP_R_16BF, K, M, ldx) == HIPBLAS_STATUS_SUCCESS;
   ok = ok && hipblasLtMatrixLayoutCreate(&plan.d, HIP_R_16BF, N, M, ldy) == HIPBLAS_STATUS_SUCCESS;
-  hipblasLtMatmulPreference_t pref = nullptr;
-  ok = ok && hipblasLtMatmulPreferenceCreate(&pref) == HIPBLAS_STATUS_SUCCESS;
-  const uint64_t limit = LT_WORKSPACE_BYTES;
-  ok = ok && hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &limit, sizeof(limit)) == HIPBLAS_STATUS_SUCCESS;
-  // the library's candidates come best first, whatever workspace they want: the first that fits is taken
-  hipblasLtMatmulHeuristicResult_t found[LT_CANDIDATES];
-  int count = 0, pick = -1;
-  ok = ok && hipblasLtMatmulAlgoGetHeuristic(dev.handle, plan.desc, plan.a, plan.b, plan.d, plan.d, pref, LT_CANDIDATES, found, &count) == HIPBLAS_STATUS_SUCCESS;
-  // (shapes that a recorded decode step may hold take a candidate without workspace if there is one:
-  // an algorithm that clears its workspace would put a memory-set node into the graph)
-  for (int i = 0; ok && M <= LT_GRAPH_MAX_ROWS && i < count && pick < 0; ++i)
-    if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize == 0) pick = i;
-  for (int i = 0; ok && i < count && pick < 0; ++i)
-    if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize <= LT_WORKSPACE_BYTES) pick = i;
-  ok = ok && pick >= 0;
-  if (pref) hipblasLtMatmulPreferenceDestroy(pref);
+  ok = ok && lt_first(dev, plan.desc, plan.a, plan.b, plan.d, M, &plan.algo, &plan.workspace);
   if (ok) {
-    plan.algo = found[pick].algo;
-    plan.workspace = found[pick].workspaceSize;
+    if (M > LT_TUNE_MAX_ROWS && M % LT_BORROW_ROWS) {
+      lt_borrow(dev, plan, M, N, K, ldx, ldy, M / LT_BORROW_ROWS * LT_BORROW_ROWS);
+      lt_borrow(dev, plan, M, N, K, ldx, ldy, (M / LT_BORROW_ROWS + 1) * LT_BORROW_ROWS);
+    }
   } else {
     if (plan.a) hipblasLtMatrixLayoutDestroy(plan.a);
     if (plan.b) hipblasLtMatrixLayoutDestroy(plan.b);
@@ -149,6 +195,45 @@ void lt_tune(LtDevice& dev, LtPlan& plan, void* y, const void* x, const void* w,
   hipEventDestroy(end);
 }
 
+// Times the plan's own algorithm and the borrowed ones on the operands of this call (caches as
+// they are: products of this many rows are bound by arithmetic) and keeps the fastest.
+// Synchronizes with the stream; never called while it is being captured.
+void lt_choose(LtDevice& dev, LtPlan& plan, void* y, const void* x, const void* w, hipStream_t stream) {
+  const int candidates = plan.borrowed + 1;
+  plan.borrowed = 0;
+  hipEvent_t begin = nullptr, end = nullptr;
+  if (hipEventCreate(&begin) != hipSuccess || hipEventCreate(&end) != hipSuccess) {
+    if (begin) hipEventDestroy(begin);
+    return;
+  }
+  const float one = 1.0f, zero = 0.0f;
+  float best = -1.0f;
+  int pick = 0;
+  for (int i = 0; i < candidates; ++i) {
+    hipblasLtMatmulAlgo_t* algo = i ? &plan.other[i - 1] : &plan.algo;
+    float fastest = -1.0f;
+    for (int run = 0; run <= LT_TUNE_RUNS; ++run) {         // the first run is not timed
+      hipEventRecord(begin, stream);
+      if (hipblasLtMatmul(dev.handle, plan.desc, &one, w, plan.a, x, plan.b, &zero, y, plan.d, y, plan.d, algo,
+                          dev.workspace, LT_WORKSPACE_BYTES, stream) != HIPBLAS_STATUS_SUCCESS) { fastest = -1.0f; break; }
+      hipEventRecord(end, stream);
+      if (hipEventSynchronize(end) != hipSuccess) { fastest = -1.0f; break; }
+      float ms = 0.0f;
+      if (run && hipEventElapsedTime(&ms, begin, end) == hipSuccess && (fastest < 0.0f || ms < fastest)) fastest = ms;
+    }
+    if (fastest >= 0.0f && (best < 0.0f || fastest < best)) {
+      best = fastest;
+      pick = i;
+    }
+  }
+  if (pick) {
+    plan.algo = plan.other[pick - 1];
+    plan.workspace = plan.other_workspace[pick - 1];
+  }
+  hipEventDestroy(begin);
+  hipEventDestroy(end);
+}
+
 }  // namespace
 
 // The current device's handle and workspace; made at the first call on the device.
@@ -194,6 +279,11 @@ extern "C" int ts_gemm_library_bf16(void* y, const void* x, const void* w, int M
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone)
       lt_tune(*dev, *plan, y, x, w, flush, flush_bytes, stream);
+  }
+  if (plan->borrowed) {
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone)
+      lt_choose(*dev, *plan, y, x, w, stream);
   }
   const float one = 1.0f, zero = 0.0f;
   const hipblasStatus_t st = hipblasLtMatmul(dev->handle, plan->desc, &one, w, plan->a, x, plan->b, &zero, y, plan->d, y,
