@@ -144,7 +144,12 @@ def main() -> int:
                     help="'prefill': time the 2,048-token prefill alone and print its record (for profiling)")
     ap.add_argument("--scenario", default=None, choices=sorted(SCENARIOS),
                     help="run a whole workload through LLM.generate instead of the decode step")
+    ap.add_argument("--many-rows-products", default="library", choices=["library", "tiled"],
+                    help="bfloat16 products of many rows: the vendor's library, or the engine's own tiled kernel")
     args = ap.parse_args()
+    if args.many_rows_products != "library":
+        from tinyserve_llm_amd.ops import hip
+        hip.many_rows_products(args.many_rows_products)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
         return 2

@@ -391,3 +391,52 @@ def test_small_portions_over_a_long_context_walk_the_keys_in_chunks(tmp_path):
         spread = float(want.max() - want.min())
         assert float((got - want[2500:]).abs().max()) <= tolerance * spread, f"{dtype}: {float((got - want[2500:]).abs().max())} of {spread}"
         assert float((mixed[0].double().cpu() - want_other[30]).abs().max()) <= tolerance * spread
+
+
+def test_the_engines_own_tiled_products_serve_steps_of_many_rows(tmp_path):
+    """With `many_rows_products("tiled")` a prompt's projections, its gated feed-forward and its
+    head run on the engine's own tiled kernel instead of the vendor library: the logits of a prompt
+    in two portions against the plain model, and the same tokens generated as with the library."""
+    from tinyserve_llm_amd.config import LlamaConfig
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.runner import StepEntry
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    from tinyserve_llm_amd.ops import hip
+    from tinyserve_llm_amd.weights.random_init import write_random_model
+    config = LlamaConfig(vocab_size=300, hidden_size=128, intermediate_size=192, num_hidden_layers=2,
+                         num_attention_heads=4, num_key_value_heads=2, head_dim=32, max_position_embeddings=256,
+                         rms_norm_eps=1e-5, rope_theta=10000.0, rope_scaling=None, tie_word_embeddings=False,
+                         eos_token_id=299)
+    write_random_model(str(tmp_path), config, 9, torch.bfloat16)
+    ids = prompt(21, 150, 300)
+    want = PlainLlama(str(tmp_path), torch.float64, weights_as=torch.bfloat16).logits(ids)
+    sc = SchedulerConfig(max_model_len=256, max_num_seqs=4, max_num_batched_tokens=256)
+    calls = []
+    tiled = hip.gemm_tiled
+    try:
+        hip.many_rows_products("tiled")
+        hip.gemm_tiled = lambda *a, **k: (calls.append(k.get("glu", False)), tiled(*a, **k))[1]
+        llm = LLM(str(tmp_path), sc, CacheConfig(block_size=16), dtype=torch.bfloat16, num_blocks=20)
+        llm.manager.allocate(0, ids[:90])
+        first = llm.runner.step([StepEntry(0, ids[:90], 0, list(range(90)))])
+        llm.manager.commit(0, 90)
+        llm.manager.append_slots(0, ids[90:])
+        rest = llm.runner.step([StepEntry(0, ids[90:], 90, list(range(60)))])
+        llm.manager.commit(0, 60)
+        llm.manager.release(0)
+        assert calls.count(True) == 4 and calls.count(False) == 2 * (2 * 3 + 1), "gate_up twice per layer; qkv, o, down and the head"
+        got = torch.cat([first, rest]).double().cpu()
+        spread = float(want.max() - want.min())
+        assert float((got - want).abs().max()) <= 3e-2 * spread
+        own = [c.token_ids for c in llm.generate([ids[:50], ids[50:120]], greedy(8))]
+    finally:
+        hip.gemm_tiled = tiled
+        hip.many_rows_products("library")
+    llm = LLM(str(tmp_path), sc, CacheConfig(block_size=16), dtype=torch.bfloat16, num_blocks=20)
+    lib = [c.token_ids for c in llm.generate([ids[:50], ids[50:120]], greedy(8))]
+    plain = PlainLlama(str(tmp_path), torch.float64, weights_as=torch.bfloat16)
+    for p_, a_, b_ in zip((ids[:50], ids[50:120]), own, lib):
+        if a_ != b_:      # a draw between two close logits may fall either way in bfloat16: then both must be close calls
+            at = next(i for i, (x_, y_) in enumerate(zip(a_, b_)) if x_ != y_)
+            row = plain.logits(p_ + a_[:at])[-1]
+            assert float(row.max() - row[[a_[at], b_[at]]].min()) <= 3e-2 * float(row.max() - row.min())

@@ -427,6 +427,33 @@ def test_library_product_called_directly(m, n, k):
         hip().gemm_library(ad.t()[:k].t()[:, ::2], wd[:, ::2])      # elements of a row must be adjacent
 
 
+@pytest.mark.parametrize("m,n,k", [(300, 384, 64), (2056, 16384, 2048), (100, 1000, 192), (257, 132, 3072), (515, 128256, 128),
+                                   (2048, 2048, 8192), (33, 8, 320), (1, 4, 64)])
+def test_tiled_product(m, n, k):
+    """The engine's own product for many rows against 64-bit: tiles that hang over the last rows
+    and columns, one, two, three and many k-steps (odd and even counts end differently), rows of x
+    that lie apart, and the gated form against the separate steps with their roundings."""
+    g = gen(m + n + k)
+    a, w = torch.randn(m, 2 * k, generator=g).bfloat16(), (torch.randn(n, k, generator=g) * 0.05).bfloat16()
+    want = a[:, :k].double() @ w.double().T
+    tolerance = dict(rtol=2e-2, atol=2e-2 * float(want.abs().max()))
+    ad, wd = a.to(dev()), w.to(dev())
+    out = hip().gemm_tiled(ad[:, :k].contiguous(), wd)
+    assert out.dtype == torch.bfloat16 and out.shape == (m, n)
+    torch.testing.assert_close(out.double().cpu(), want, **tolerance)
+    assert torch.equal(hip().gemm_tiled(ad[:, :k], wd), out), "the order of the sums does not depend on the strides"
+    if n % 8 == 0:
+        gated = hip().gemm_tiled(ad[:, :k], wd, glu=True)
+        y = want.bfloat16().double()
+        ref = (torch.nn.functional.silu(y[:, :n // 2]) * y[:, n // 2:])
+        assert gated.shape == (m, n // 2)
+        torch.testing.assert_close(gated.double().cpu(), ref, rtol=3e-2, atol=3e-2 * float(ref.abs().max()))
+    with pytest.raises(hip().KernelError, match="tiled kernel takes"):
+        hip().gemm_tiled(ad[:, :k - 8], wd[:, :k - 8])
+    with pytest.raises(hip().KernelError, match="tiled kernel takes"):
+        hip().gemm_tiled(ad[:, :k], wd[:n - 1])
+
+
 @pytest.mark.parametrize("m", [1, 3, 8, 16, 17, 32])
 @pytest.mark.parametrize("n,k", [(3072, 2048), (2048, 2048), (16384, 2048), (2048, 8192), (992, 512), (130, 3072), (64, 4096),
                                  (8192, 3072), (8256, 4096)])

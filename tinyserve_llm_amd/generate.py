@@ -46,6 +46,8 @@ def parse_args(argv=None) -> argparse.Namespace:
     p.add_argument("--max-num-batched-tokens", type=int, default=16384)
     p.add_argument("--max-prefill-chunk", type=int, default=0)
     p.add_argument("--device", default="cuda")
+    p.add_argument("--many-rows-products", choices=["library", "tiled"], default="library",
+                   help="bfloat16 products of many rows: the vendor's matrix library, or the engine's own tiled kernel (slower)")
     p.add_argument("--out", help="write the JSON record here as well as printing a summary")
     return p.parse_args(argv)
 
@@ -68,6 +70,9 @@ def main(argv=None) -> int:
     sc = SchedulerConfig(max_model_len=args.max_model_len, max_num_seqs=args.max_num_seqs,
                          max_num_batched_tokens=args.max_num_batched_tokens, max_prefill_chunk=args.max_prefill_chunk)
     cc = CacheConfig(block_size=args.block_size, caching=args.caching == "on", device=args.device)
+    if args.many_rows_products != "library":
+        from tinyserve_llm_amd.ops import hip
+        hip.many_rows_products(args.many_rows_products)
     llm = LLM(args.model, sc, cc, dtype=args.dtype, num_blocks=args.num_blocks,
               gpu_memory_utilization=args.gpu_memory_utilization, seed=args.seed, random_weights=random_weights)
     vocab = llm.model.spec.vocab_size

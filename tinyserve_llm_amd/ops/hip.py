@@ -54,6 +54,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_gemm_exact": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_sample": [p, p, p, p, p, p, u64, i, i, i64, p],
         "ts_gemm_library_bf16": [p, p, p, i, i, i, i64, i64, i64, i, p, ctypes.c_size_t, p],
+        "ts_gemm_tiled_bf16": [p, p, p, i, i, i, i64, i64, i64, i, p],
         "ts_gemm_library_init": [],
         "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, i, i, i, i, p, p, p],
         "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p],
@@ -683,6 +684,46 @@ def qkv_rope_store(x: torch.Tensor, weight: torch.Tensor, cos_sin: torch.Tensor 
     return q, res_out
 
 
+MANY_ROWS_PRODUCTS = ("library", "tiled")
+_many_rows = "library"
+
+
+def many_rows_products(which: str | None = None) -> str:
+    """Which kernel serves bfloat16 products of many rows: "library" (the vendor's, the faster one
+    and the default) or "tiled" (this repository's LDS-tiled matrix-core kernel, for the shapes it
+    takes). Sets it if `which` is given; returns the setting. It holds for the process."""
+    global _many_rows
+    if which is not None:
+        _need(which in MANY_ROWS_PRODUCTS, f"products of many rows are one of {MANY_ROWS_PRODUCTS}, not {which!r}")
+        _many_rows = which
+    return _many_rows
+
+
+def tiled_takes(x: torch.Tensor, weight: torch.Tensor, glu: bool = False) -> bool:
+    """Whether the tiled kernel serves these operands (see gemm_tiled.hip for the conditions)."""
+    n, k = weight.shape
+    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and k % 64 == 0 and n % (8 if glu else 4) == 0
+            and x.stride(1) == 1 and weight.stride(1) == 1 and x.stride(0) % 8 == 0 and weight.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+
+
+def gemm_tiled(x: torch.Tensor, weight: torch.Tensor, glu: bool = False) -> torch.Tensor:
+    """bfloat16 x [M, K] · weight [N, K]^T by the LDS-tiled matrix-core kernel; with `glu` the weight
+    holds N / 2 gate rows, then N / 2 up rows, and silu(gate) · up [M, N / 2] comes back."""
+    _gpu(x, weight)
+    _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
+          f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
+    _need(tiled_takes(x, weight, glu), "the tiled kernel takes bfloat16 operands with dense, 16-byte aligned rows, a "
+          "reduction that is a multiple of 64 and a width that is a multiple of 4 (8 with the gate)")
+    M, K = x.shape
+    N = weight.shape[0]
+    y = torch.empty((M, N // 2 if glu else N), dtype=torch.bfloat16, device=x.device)
+    if M and N:
+        _run("gemm_tiled", library().ts_gemm_tiled_bf16(_ptr(y), _ptr(x), _ptr(weight), M, N, K, x.stride(0),
+                                                        weight.stride(0), y.stride(0), int(glu), _stream()))
+    return y
+
+
 def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
                 packed: torch.Tensor | None = None) -> torch.Tensor:
     """bfloat16 x [M, K] · weight [N, K]^T: few rows go to the weight-streaming kernel (which reads
@@ -698,7 +739,7 @@ def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
             and (x.shape[0] <= SKINNY_FUSED_ROWS or weight.numel() <= SKINNY_WIDE_ELEMENTS)
             and x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
         return gemm_skinny(x, weight, out_dtype, packed=packed)[0]
-    y = gemm_library(x, weight)
+    y = gemm_tiled(x, weight) if _many_rows == "tiled" and tiled_takes(x, weight) else gemm_library(x, weight)
     return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
 
 

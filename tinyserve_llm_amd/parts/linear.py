@@ -2,7 +2,8 @@
 
 float32 runs the engine's own exact kernel (32-bit multiply-adds, ascending k, independent of the
 batch). bfloat16 uses the weight-streaming kernel for few rows and the vendor matrix library for
-many, as the reference uses a vendor library for every projection.
+many, as the reference uses a vendor library for every projection (or, if
+`hip.many_rows_products("tiled")` says so, the engine's own tiled kernel, which is slower).
 
 With few rows a step's time goes to launching kernels and to waiting for memory, so what
 precedes or follows a projection can ride along with it: a norm may hand its input over as a
@@ -63,6 +64,9 @@ def linear(x: torch.Tensor | DeferredNorm, weight: torch.Tensor, out_dtype: torc
         if (out_dtype in (None, torch.bfloat16) and _streams(x, weight) and weight.shape[0] % 32 == 0
                 and hip.skinny_fuses(x.shape[0], weight.shape[1], False, True)):
             return hip.gemm_skinny(x, weight, glu=True, packed=packed)[0]
+        if (out_dtype in (None, torch.bfloat16) and hip.many_rows_products() == "tiled" and x.is_cuda
+                and hip.tiled_takes(x, weight, glu=True)):
+            return hip.gemm_tiled(x, weight, glu=True)
         return hip.silu_mul(linear(x, weight, out_dtype, packed=packed))
     if x.dtype == torch.float32:
         return hip.gemm_exact(x, weight, out_dtype)
