@@ -536,7 +536,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         if lead:
             paged_attention_decode(q[:lead], k_cache, v_cache, tables, ctx.seq_of_token[:lead], ctx.positions[:lead],
                                    scale, window, out=out[:lead])
-        splits, chunk = prefill_splits(tiles.shape[0] * nkv, max(ctx.host_context_lens[lead:]))
+        splits, chunk = prefill_splits(tiles.shape[0] * nkv, max(ctx.host_context_lens[lead:], default=0))
         return paged_attention_prefill(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, tiles, scale,
                                        window, tile_tokens=tile_tokens, out=out, num_splits=splits, chunk=chunk,
                                        first_token=cu[lead])
