@@ -111,7 +111,7 @@ class LLM:
         if decode_graphs:
             self.runner.enable_decode_graphs(scheduler_config.max_model_len, scheduler_config.max_num_seqs, self.seed)
         self.run_ahead = run_ahead
-        self._ahead: tuple | None = None             # (the step scheduled ahead, its packing or None)
+        self._ahead: tuple | None = None             # (the step scheduled ahead, its packing or None, its launch or None)
         self.steps: list[StepRecord] = []
         logger.info("KV cache: %d blocks of %d tokens", num_blocks, cache_config.block_size)
 
@@ -212,15 +212,18 @@ class LLM:
     def step(self) -> list[RequestOutput]:
         """One step of the engine. A step of decodes only is closed in two halves around the
         scheduling and packing of the next step, which so happen while the device is still busy;
-        any other step is scheduled, run and closed in turn."""
+        once its tokens are read and none of them ends a sequence, the packed step is started
+        before the tokens are entered into the books, so that the device waits for the host only
+        as long as the read and the launch take. Any other step is scheduled, run and closed in turn."""
         start = time.perf_counter()
-        batch, prepared = self._ahead if self._ahead is not None else (None, None)
+        batch, prepared, launched = self._ahead if self._ahead is not None else (None, None, None)
         self._ahead = None
         if batch is None:
             batch = self.scheduler.schedule(start)
         if not batch:
             raise RuntimeError("the scheduler produced an empty step")
-        launched = self._launch(batch, prepared)
+        if launched is None:
+            launched = self._launch(batch, prepared)
         halves = self.run_ahead and self.scheduler.decodes_only(batch)
         if halves:
             self.scheduler.commit_decodes(batch)
@@ -229,10 +232,17 @@ class LLM:
         sampled = self._finish(launched)
         end = time.perf_counter()
         if halves:
+            early = None
+            if prepared is not None and self.scheduler.all_go_on(batch, sampled):
+                # nobody leaves: the packed step starts now, and the books below are kept beside it
+                drawn = {b.seq.seq_id: tokens[0] for b, tokens in zip(batch, sampled)}
+                fed = [drawn[b.seq.seq_id] if b.token_ids[0] == PENDING else b.token_ids[0] for b in ahead]
+                early = (self.runner.launch_decode(prepared, fed), None)
             outputs, left = self.scheduler.deliver_tokens(batch, sampled, end, ahead)
+            assert early is None or len(left) == len(ahead), "a step was started with a sequence that had ended"
             if left:
                 # whoever turned out finished has left the step: it is packed again when it runs
-                self._ahead = (left, prepared if len(left) == len(ahead) else None)
+                self._ahead = (left, prepared if len(left) == len(ahead) else None, early)
         else:
             outputs = self.scheduler.postprocess(batch, sampled, end)
         self.steps.append(StepRecord(start, end, len(batch), sum(len(b.token_ids) for b in batch),
