@@ -233,8 +233,9 @@ def test_decode_graphs_replay_what_eager_steps_compute(folder_b):
 
 @pytest.mark.parametrize("num_blocks", [120, 18])
 def test_steps_closed_in_two_halves_generate_the_same(folder_b, num_blocks):
-    """With `run_ahead` a decode step is scheduled and packed while the one before it still runs,
-    from a placeholder for the token under way. Tokens must equal those of the engine that closes
+    """With `run_ahead` a decode step is scheduled, packed and started while the one before it
+    still runs, from a placeholder for the token under way, which it takes on the device; a
+    sequence that ends has a row in the step already started, which is dropped. Tokens must equal those of the engine that closes
     every step before it schedules the next: with sampling (keys name request, sample and position),
     with sequences that end by themselves, and with so few pages that sequences are preempted."""
     from tinyserve_llm_amd.engine.llm import LLM, CacheConfig

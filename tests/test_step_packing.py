@@ -94,8 +94,11 @@ def test_decode_packing_refuses_what_the_general_packing_refuses():
 def test_draw_words_round_trip():
     import torch
     words, start = DecodeGraphs._with_draws([1, 2, 3], 4, ([0.5, 0.0, 1.25], [5, (1 << 63) - 1, 0x123456789ABCDEF]))
-    assert start == 4 and words.dtype == torch.int32 and len(words) == 4 + 3 * 4
+    assert start == 4 and words.dtype == torch.int32 and len(words) == 4 + 4 * 4
     assert words[start:start + 8].view(torch.int64).tolist() == [5, (1 << 63) - 1, 0x123456789ABCDEF, 0]
-    assert words[start + 8:].view(torch.float32).tolist() == [0.5, 0.0, 1.25, 0.0]
+    assert words[start + 8:start + 12].view(torch.float32).tolist() == [0.5, 0.0, 1.25, 0.0]
+    assert words[start + 12:].tolist() == [-1] * 4, "no entry takes its token from the step before"
+    fed, _ = DecodeGraphs._with_draws([1, 2, 3], 4, ([0.5, 0.0, 1.25], [5, 6, 7]), feed=[2, -1, 0])
+    assert fed[start + 12:].tolist() == [2, -1, 0, -1], "the rows of the step before, then the idle rows"
     none, _ = DecodeGraphs._with_draws([1, 2], 2, None)
-    assert none.tolist() == [1, 2, 0, 0, 0, 0, 0, 0]
+    assert none.tolist() == [1, 2, 0, 0, 0, 0, 0, 0, -1, -1]

@@ -90,3 +90,22 @@ extern "C" int ts_sample(int32_t* out, float* work_v, int32_t* work_i, const flo
   sample_pick_kernel<<<rows, TS_WAVE, 0, stream>>>(out, work_v, work_i);
   return ts_check_launch();
 }
+
+// ids[i] = prev[src[i]] where src[i] >= 0: the tokens a step drew become the next step's input
+// without passing through the host (src names, per entry of the next step, the row of the step
+// before whose token it feeds; -1 keeps the id the host packed).
+__global__ void feed_tokens_kernel(int32_t* __restrict__ ids, const int32_t* __restrict__ prev,
+                                   const int32_t* __restrict__ src, int n, int prev_n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int s = src[i];
+  if (s >= 0 && s < prev_n) ids[i] = prev[s];
+}
+
+extern "C" int ts_feed_tokens(int32_t* ids, const int32_t* prev, const int32_t* src, int n, int prev_n,
+                              hipStream_t stream) {
+  if (n <= 0) return TS_OK;
+  if (!ids || !prev || !src || prev_n <= 0) return TS_BAD_SHAPE;
+  feed_tokens_kernel<<<(n + 255) / 256, 256, 0, stream>>>(ids, prev, src, n, prev_n);
+  return ts_check_launch();
+}

@@ -111,7 +111,7 @@ class LLM:
         if decode_graphs:
             self.runner.enable_decode_graphs(scheduler_config.max_model_len, scheduler_config.max_num_seqs, self.seed)
         self.run_ahead = run_ahead
-        self._ahead: tuple | None = None             # (the step scheduled ahead, its packing or None, its launch or None)
+        self._ahead: tuple | None = None             # (what is left of the step scheduled ahead, its launch or None, its rows)
         self.steps: list[StepRecord] = []
         logger.info("KV cache: %d blocks of %d tokens", num_blocks, cache_config.block_size)
 
@@ -157,11 +157,9 @@ class LLM:
         keys = [row_key(b.seq.request_id, b.seq.sample_index, len(b.seq.output_token_ids)) for b in batch]
         return temps, keys
 
-    def _launch(self, batch: list[ScheduledSeq], prepared=None) -> tuple:
+    def _launch(self, batch: list[ScheduledSeq]) -> tuple:
         """Starts one forward pass and the draws on the device (model_runner.py:120-133); `_finish`
         waits for them."""
-        if prepared is not None:
-            return self.runner.launch_decode(prepared, [b.token_ids[0] for b in batch]), None
         entries = [StepEntry(seq.seq_id, tokens, start, [len(tokens) - 1] if num_samples else [])
                    for seq, tokens, num_samples, start in batch]
         if all(b.num_samples == 1 for b in batch):
@@ -201,48 +199,55 @@ class LLM:
             i += n
         return out
 
-    def _prepare_ahead(self, ahead: list[ScheduledSeq]):
-        """Packs the next step while the device runs this one, if it is one of decodes only."""
-        if not ahead or not self.scheduler.decodes_only(ahead):
+    def _launch_ahead(self, ahead: list[ScheduledSeq], launched: tuple, order: list[int]) -> tuple | None:
+        """Packs and starts the next step while the device runs this one, if it is one of decodes
+        only that the decode graphs take. Its entries whose token is still a placeholder take it on
+        the device from what the running step draws (`order`: the sequence of each of its rows), so
+        neither step waits for the host. None if the step has to be started the plain way."""
+        drawn, owners = launched
+        if not ahead or drawn is None or owners is not None or not self.scheduler.decodes_only(ahead):
             return None
+        row = {seq_id: k for k, seq_id in enumerate(order)}
         entries = [StepEntry(b.seq.seq_id, [0 if t == PENDING else t for t in b.token_ids], b.start, [0]) for b in ahead]
+        feed = [row[b.seq.seq_id] if b.token_ids[0] == PENDING else -1 for b in ahead]
         temps, keys = self._draws(ahead)
-        return self.runner.prepare_decode(entries, temps, keys, self.seed)
+        prepared = self.runner.prepare_decode(entries, temps, keys, self.seed, feed)
+        if prepared is None:
+            return None
+        return self.runner.launch_decode(prepared, drawn), None
 
     def step(self) -> list[RequestOutput]:
-        """One step of the engine. A step of decodes only is closed in two halves around the
-        scheduling and packing of the next step, which so happen while the device is still busy;
-        once its tokens are read and none of them ends a sequence, the packed step is started
-        before the tokens are entered into the books, so that the device waits for the host only
-        as long as the read and the launch take. Any other step is scheduled, run and closed in turn."""
+        """One step of the engine. A step of decodes only is closed in two halves: the slots are
+        committed, the next step is scheduled, packed and started behind this one on the device
+        (taking the tokens this one draws where they are, on the device), and only then are this
+        step's tokens read and entered into the books. A sequence that turns out to have ended has
+        a row in the step already started; that row is dropped when the step is read. Any other
+        step is scheduled, run and closed in turn."""
         start = time.perf_counter()
-        batch, prepared, launched = self._ahead if self._ahead is not None else (None, None, None)
+        # (what is left of the step scheduled ahead, its launch, the sequence of each launched row)
+        batch, launched, order = self._ahead if self._ahead is not None else (None, None, None)
         self._ahead = None
         if batch is None:
             batch = self.scheduler.schedule(start)
         if not batch:
             raise RuntimeError("the scheduler produced an empty step")
         if launched is None:
-            launched = self._launch(batch, prepared)
+            launched, order = self._launch(batch), [b.seq.seq_id for b in batch]
         halves = self.run_ahead and self.scheduler.decodes_only(batch)
+        early = None
         if halves:
             self.scheduler.commit_decodes(batch)
             ahead = self.scheduler.schedule(time.perf_counter()) if self.scheduler.has_unfinished() else []
-            prepared = self._prepare_ahead(ahead)
+            early = self._launch_ahead(ahead, launched, order)
         sampled = self._finish(launched)
+        if len(order) != len(batch):            # rows of sequences that ended after the step was started
+            row = {seq_id: k for k, seq_id in enumerate(order)}
+            sampled = [sampled[row[b.seq.seq_id]] for b in batch]
         end = time.perf_counter()
         if halves:
-            early = None
-            if prepared is not None and self.scheduler.all_go_on(batch, sampled):
-                # nobody leaves: the packed step starts now, and the books below are kept beside it
-                drawn = {b.seq.seq_id: tokens[0] for b, tokens in zip(batch, sampled)}
-                fed = [drawn[b.seq.seq_id] if b.token_ids[0] == PENDING else b.token_ids[0] for b in ahead]
-                early = (self.runner.launch_decode(prepared, fed), None)
             outputs, left = self.scheduler.deliver_tokens(batch, sampled, end, ahead)
-            assert early is None or len(left) == len(ahead), "a step was started with a sequence that had ended"
             if left:
-                # whoever turned out finished has left the step: it is packed again when it runs
-                self._ahead = (left, prepared if len(left) == len(ahead) else None, early)
+                self._ahead = (left, early, [b.seq.seq_id for b in ahead] if early is not None else None)
         else:
             outputs = self.scheduler.postprocess(batch, sampled, end)
         self.steps.append(StepRecord(start, end, len(batch), sum(len(b.token_ids) for b in batch),

@@ -247,7 +247,8 @@ class ModelRunner:
     def step_sample(self, entries: Sequence[StepEntry], temperatures: Sequence[float], keys: Sequence[int],
                     seed: int) -> torch.Tensor:
         """Runs a step in which every entry wants the logits of exactly one place and draws one token
-        from each: int32 [entries] on the device. `keys[i]` names the draw of entry i (see
+        from each: int32 [entries], as a device tensor or, from a replayed graph, as `DrawnTokens`
+        (`tolist()` gives them either way). `keys[i]` names the draw of entry i (see
         `sampling.sampler`). Decode steps replay a graph that holds the draw as well."""
         if self.graphs is not None and self.graphs.seed == seed and self.graphs.takes(entries):
             return self.graphs.run(entries, (temperatures, keys))
@@ -255,19 +256,21 @@ class ModelRunner:
         return sample(self.step(entries), list(temperatures), list(keys), seed)
 
     def prepare_decode(self, entries: Sequence[StepEntry], temperatures: Sequence[float], keys: Sequence[int],
-                       seed: int):
+                       seed: int, feed: Sequence[int] | None = None):
         """Checks and packs a decode step with its draws ahead of time, on the host alone, while the
-        device is busy; the entries' token ids may be stand-ins (`launch_decode` takes the real ones).
+        device is busy. The token id of an entry may be a stand-in: `feed[i]` >= 0 then names the row
+        of the step before whose drawn token entry i takes (-1: the id given is the real one).
         None if the step is not one the decode graphs take."""
         if self.graphs is not None and self.graphs.seed == seed and self.graphs.takes(entries):
-            return self.graphs.prepare(entries, (temperatures, keys))
+            return self.graphs.prepare(entries, (temperatures, keys), feed)
         return None
 
     @torch.inference_mode()
-    def launch_decode(self, prepared, token_ids: Sequence[int]) -> torch.Tensor:
-        """Starts a step that `prepare_decode` packed, with the entries' token ids now known:
-        the drawn tokens, int32 [entries] on the device."""
-        return self.graphs.launch(prepared, token_ids)
+    def launch_decode(self, prepared, drawn_before: "DrawnTokens | torch.Tensor | None" = None) -> "DrawnTokens":
+        """Starts a step that `prepare_decode` packed; `drawn_before` is what the step before drew
+        (`DrawnTokens` or a device tensor, possibly still being computed), from which the entries that
+        `feed` named take their ids. Returns the drawn tokens as `DrawnTokens`."""
+        return self.graphs.launch(prepared, drawn_before=drawn_before)
 
     def enable_decode_graphs(self, max_context: int, max_batch: int, seed: int = 0) -> bool:
         """Decode steps (every entry one token whose logits are wanted) are then replayed from HIP
@@ -278,6 +281,19 @@ class ModelRunner:
             return False
         self.graphs = DecodeGraphs(self, max_context, max_batch, seed)
         return True
+
+
+class DrawnTokens:
+    """The tokens a replayed step drew: a copy on the device (for the step after it to take its
+    ids from) and one on its way to pinned host memory. `tolist()` waits for that copy alone, not
+    for what was started on the device after it."""
+
+    def __init__(self, on_device: torch.Tensor, host: torch.Tensor, landed: torch.cuda.Event, n: int) -> None:
+        self.on_device, self.host, self.landed, self.n = on_device, host, landed, n
+
+    def tolist(self) -> list[int]:
+        self.landed.synchronize()
+        return self.host[:self.n].tolist()
 
 
 class DecodeGraphs:
@@ -315,10 +331,10 @@ class DecodeGraphs:
         return True
 
     @staticmethod
-    def _with_draws(flat: list[int], size: int, draws) -> tuple[torch.Tensor, int]:
+    def _with_draws(flat: list[int], size: int, draws, feed: Sequence[int] | None = None) -> tuple[torch.Tensor, int]:
         """The upload: `flat`, padded to an even length, then `size` keys (int64, low word first)
         and `size` temperatures (float32) as raw 32-bit words; rows without a draw get key 0 and
-        temperature 0."""
+        temperature 0. Then `size` rows of the step before that feed the entries (-1: none)."""
         start = len(flat) + (len(flat) & 1)
         words = flat + [0] * (start - len(flat))
         if draws is None:
@@ -333,6 +349,7 @@ class DecodeGraphs:
             words += [0] * (2 * (size - n))
             words += struct.unpack(f"{n}i", struct.pack(f"{n}f", *temperatures))
             words += [0] * (size - n)
+        words += [-1] * size if feed is None else list(feed) + [-1] * (size - len(feed))
         return torch.tensor(words, dtype=torch.int32), start
 
     def _capture(self, size: int, words: torch.Tensor, start: int, dims, host):
@@ -361,37 +378,56 @@ class DecodeGraphs:
             tokens = hip.sample(logits, draw_temps, draw_keys, self.seed)
         if self.pool is None:
             self.pool = graph.pool()
-        return graph, host_i32, dev_i32, logits, tokens
+        # the drawn tokens travel to the host through two pinned buffers in turn: a step may be
+        # started before the tokens of the step before it have been read
+        landing = [(torch.empty(size, dtype=torch.int32, pin_memory=True), torch.cuda.Event()) for _ in range(2)]
+        return [graph, host_i32, dev_i32, logits, tokens, torch.cuda.Event(), landing, 0]
 
-    def prepare(self, entries: Sequence[StepEntry], draws=None) -> tuple:
-        """The host half of `run`: checks and packs the step. The entries' token ids may still be
-        placeholders (any id inside the vocabulary); `launch` takes the real ones."""
+    def prepare(self, entries: Sequence[StepEntry], draws=None, feed: Sequence[int] | None = None) -> tuple:
+        """The host half of `run`: checks and packs the step. Token ids of entries that `feed`
+        names a source row for may be placeholders (any id inside the vocabulary)."""
+        if feed is not None and (len(feed) != len(entries) or min(feed) < -1):
+            raise StepError("one source row (or -1) per entry")
         size = self._size(len(entries))
         longest = max(e.start + 1 for e in entries)
         reach = min(-(-longest // self.bucket) * self.bucket, -(-self.max_context // self.bucket) * self.bucket)
         width = -(-reach // self.page_size)
         flat, dims, host = self.runner._pack_decode(entries, [width] * self.num_spaces, pad_to=size)
-        words, start = self._with_draws(flat, size, draws)
-        return (size, width), words, start, dims, host, len(entries), draws is not None
+        words, start = self._with_draws(flat, size, draws, feed)
+        return (size, width), words, start, dims, host, len(entries), draws is not None, feed is not None and max(feed) >= 0
 
-    def launch(self, prepared: tuple, token_ids: Sequence[int] | None = None) -> torch.Tensor:
-        """The device half: uploads the packed step (with `token_ids` in the entries' places, if
-        given) and replays its graph. Logits [entries, vocab], or the tokens drawn if the step was
-        prepared with draws."""
-        key, words, start, dims, host, n, drawn = prepared
-        if token_ids is not None:
-            vocab = self.runner.model.spec.vocab_size
-            if len(token_ids) != n or min(token_ids) < 0 or max(token_ids) >= vocab:
-                raise StepError(f"{len(token_ids)} token ids for {n} entries, or one outside the vocabulary of {vocab}")
-            words[:n] = torch.tensor(token_ids, dtype=torch.int32)
+    def launch(self, prepared: tuple, drawn_before: torch.Tensor | None = None) -> torch.Tensor:
+        """The device half: uploads the packed step, lets the entries that name a source row take
+        their ids from `drawn_before` (the tokens of the step before, on the device) and replays the
+        step's graph. Logits [entries, vocab], or the tokens drawn (`DrawnTokens`: copies, since
+        the next replay writes the graph's own tokens anew and may be started before anyone has
+        read these) if the step was prepared with draws."""
+        from tinyserve_llm_amd.ops import hip
+        key, words, start, dims, host, n, drawn, fed = prepared
+        if fed and drawn_before is None:
+            raise StepError("the step takes ids from the step before, whose tokens were not given")
         if key not in self.graphs:
             self.graphs[key] = self._capture(key[0], words, start, dims, host)
             # the capture recorded the step without running it: the replay below runs it
-        graph, host_i32, dev_i32, logits, tokens = self.graphs[key]
+        kept = self.graphs[key]
+        graph, host_i32, dev_i32, logits, tokens, uploaded, landing, turn = kept
+        uploaded.synchronize()                  # the last upload from the pinned words has long been made
         host_i32.copy_(words)
         dev_i32.copy_(host_i32, non_blocking=True)
+        uploaded.record()
+        if fed:
+            size = key[0]
+            before = drawn_before.on_device if isinstance(drawn_before, DrawnTokens) else drawn_before
+            hip.feed_tokens(dev_i32[:n], before.contiguous(), dev_i32[start + 3 * size:start + 3 * size + n])
         graph.replay()
-        return (tokens if drawn else logits)[:n]
+        if not drawn:
+            return logits[:n]
+        host_tokens, landed = landing[turn]
+        kept[7] = 1 - turn
+        on_device = tokens[:n].clone()
+        host_tokens[:n].copy_(on_device, non_blocking=True)
+        landed.record()
+        return DrawnTokens(on_device, host_tokens, landed, n)
 
     def run(self, entries: Sequence[StepEntry], draws=None) -> torch.Tensor:
         """Replays the step's graph. Without `draws` the logits [entries, vocab] come back; with

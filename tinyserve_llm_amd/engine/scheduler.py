@@ -358,12 +358,6 @@ class Scheduler:
             seq.prefill_target = seq.num_computed
             seq.output_token_ids.append(PENDING)
 
-    def all_go_on(self, scheduled: list[ScheduledSeq], sampled: list[list[int]]) -> bool:
-        """Whether none of a decode step's sequences ends with the token drawn for it (asked between
-        `commit_decodes` and `deliver_tokens`, while the placeholders stand): then the step
-        scheduled in between is run exactly as it was packed."""
-        return all(self._finish_reason(seq, tokens[0]) is None for (seq, _, _, _), tokens in zip(scheduled, sampled))
-
     def deliver_tokens(self, scheduled: list[ScheduledSeq], sampled: list[list[int]], now: float,
                        ahead: list[ScheduledSeq] | None = None) -> tuple[list[RequestOutput], list[ScheduledSeq]]:
         """Second half: the drawn tokens take the placeholders' place, what finished is released.

@@ -53,6 +53,7 @@ def _declare(lib: ctypes.CDLL) -> None:
                                       i, p],
         "ts_gemm_exact": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_sample": [p, p, p, p, p, p, u64, i, i, i64, p],
+        "ts_feed_tokens": [p, p, p, i, i, p],
         "ts_gemm_library_bf16": [p, p, p, i, i, i, i64, i64, i64, i, p, ctypes.c_size_t, p],
         "ts_gemm_tiled_bf16": [p, p, p, i, i, i, i64, i64, i64, i, p],
         "ts_gemm_library_init": [],
@@ -362,6 +363,15 @@ def copy_slots(pool: torch.Tensor, src: int, dst: int, num_slots: int, slot_dim:
         inner *= n
     _run("copy_slots", library().ts_copy_slots(_ptr(pool), runs, page_size * inner, num_slots * inner, src, dst,
                                                _stream()))
+
+
+def feed_tokens(ids: torch.Tensor, prev: torch.Tensor, src: torch.Tensor) -> None:
+    """ids[i] = prev[src[i]] where src[i] >= 0 (all int32, on the device): what one step drew becomes
+    the next step's input without a trip to the host."""
+    _gpu(ids, prev, src)
+    _need(all(t.dtype == torch.int32 and t.dim() == 1 and t.is_contiguous() for t in (ids, prev, src))
+          and src.shape[0] == ids.shape[0] and prev.shape[0] > 0, "feed_tokens takes int32 vectors, one source per id")
+    _run("feed_tokens", library().ts_feed_tokens(_ptr(ids), _ptr(prev), _ptr(src), ids.shape[0], prev.shape[0], _stream()))
 
 
 def sample(logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor, seed: int) -> torch.Tensor:
