@@ -244,7 +244,7 @@ def test_split_key_decode_attention(heads, kv, hd, page, chunk, waves):
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev())
     kc, vc = engine_layout(k, v, table, page, pages, dtype)
     assert hip().decode_kernel_takes(q[rows].to(dev()), kc, vc)
-    if waves > hip().decode_waves(hd) or 4 * (32 * waves + waves * (heads // kv) * hd) > 65536:
+    if waves > hip().decode_waves(hd, chunk == 32 * waves) or 4 * (32 * waves + waves * (heads // kv) * hd) > 65536:
         with pytest.raises(hip().KernelError, match="waves"):
             hip().paged_attention_decode(q[rows].to(dev()), kc, vc, i32([table, table]), i32([0, 1] * 6), i32(rows),
                                          hd ** -0.5, chunk=chunk, waves=waves)

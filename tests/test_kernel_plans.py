@@ -61,15 +61,15 @@ def test_decode_plan_divides_the_context_into_32_key_steps_per_wave():
         for nkv, group, hd in ((8, 4, 64), (1, 16, 128), (2, 3, 96), (5, 1, 32)):
             for capacity in (8, 64, 256, 300, 2304, 4096, 8192, 131072, 1 << 21):
                 chunk, waves = hip.decode_plan(tokens, nkv, group, hd, capacity)
-                assert 1 <= waves <= hip.decode_waves(hd) and chunk % (32 * waves) == 0
+                assert 1 <= waves <= hip.decode_waves(hd, chunk == 32 * waves) and chunk % (32 * waves) == 0
                 assert -(-capacity // chunk) <= hip.MAX_DECODE_SPLITS
                 assert 4 * (32 * waves + waves * group * hd) <= 65536
     assert hip.decode_plan(8, 8, 4, 64, 2304) == (256, 8)          # one step per wave
-    assert hip.decode_plan(8, 8, 4, 128, 2304) == (128, 4)         # wide heads: four waves
+    assert hip.decode_plan(8, 8, 4, 128, 2304) == (256, 8)         # wide heads too, where a wave has one step;
     assert hip.decode_plan(64, 8, 4, 64, 2304) == (2304, 8)        # a workgroup per compute unit: nothing to combine
     assert hip.decode_plan(64, 8, 4, 64, 32768) == (4096, 8)       # ... but not over a very long context
     assert hip.decode_plan(1, 8, 4, 64, 192) == (192, 6)           # short context: one workgroup
     assert hip.decode_plan(1, 8, 4, 64, 32768) == (1024, 8)        # long: 32 chunks of a token's 8 heads fill the chip
-    assert hip.decode_plan(8, 8, 4, 128, 8192) == (2048, 4)        # 4 chunks for 64 (token, head) pairs
+    assert hip.decode_plan(8, 8, 4, 128, 8192) == (2048, 4)        # four waves in the loop over several steps: 4 chunks for 64 (token, head) pairs
     assert hip.decode_plan(8, 8, 4, 128, 32768) == (4096, 4)       # chunks stay within 4,096 keys
     assert hip.decode_plan(4, 8, 4, 64, 8192) == (1024, 8)

@@ -1,6 +1,6 @@
 // Split-key paged attention on the matrix cores for tokens that each bring one query (decoding),
 // bfloat16. A workgroup takes one (token, key/value head, chunk of keys) and serves all query heads
-// of that key/value head's group; its waves (up to 8, or 4 for heads wider than 64) take the chunk's
+// of that key/value head's group; its waves (up to 8; 4 for heads wider than 64 where a wave has more than one step) take the chunk's
 // 32-key steps in turn:
 //     S^T[key, head] = K[key, :] · Q[head, :]      v_mfma_f32_16x16x32_bf16, keys as rows
 //     online softmax per head (32-bit), P = 2^(S - m)
@@ -16,13 +16,15 @@
 #include "attention_mfma.h"
 
 #define DEC_MAX_WAVES 8
-// heads wider than 64 keep two steps of wide rows in registers: their workgroups have up to 4 waves
-#define DEC_WAVES_FOR(HD) ((HD) > 64 ? 4 : DEC_MAX_WAVES)
+// heads wider than 64 keep two steps of wide rows in registers in the general loop: its workgroups
+// have up to 4 waves then (with 8, a lane's 256 registers are overrun by 22, and 64 tokens over
+// 2,560 keys take 137 µs instead of 122); the instance with a single step per wave has room for 8
+#define DEC_WAVES_FOR(HD, ONE) ((HD) > 64 && !(ONE) ? 4 : DEC_MAX_WAVES)
 
 // ONE: a wave has a single 32-key step (chunk = 32 waves); without the second buffer of the
 // general loop the kernel needs fewer registers and more workgroups share a compute unit
 template <int HD, bool ONE>
-__global__ void __launch_bounds__(DEC_WAVES_FOR(HD) * TS_WAVE)
+__global__ void __launch_bounds__(DEC_WAVES_FOR(HD, ONE) * TS_WAVE)
 attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
                         const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
                         const int32_t* __restrict__ block_tables, const int32_t* __restrict__ seq_of_token,
@@ -188,7 +190,7 @@ extern "C" int ts_paged_attention_decode(void* out, float* part_o, float* part_m
   if (num_tokens <= 0) return TS_OK;
   if (nkv <= 0 || nh % nkv || page_size <= 0 || page_size % 8 || max_blocks <= 0 || num_splits <= 0)
     return TS_BAD_SHAPE;
-  if (waves < 1 || waves > DEC_WAVES_FOR(hd) || chunk <= 0 || chunk % (32 * waves) || num_splits > COMBINE_MAX_SPLITS)
+  if (waves < 1 || waves > DEC_WAVES_FOR(hd, chunk == 32 * waves) || chunk <= 0 || chunk % (32 * waves) || num_splits > COMBINE_MAX_SPLITS)
     return TS_BAD_SHAPE;
   if (num_splits > 1 && (!part_o || !part_ml)) return TS_BAD_SHAPE;
   if (num_tokens > 65535 || nkv > 65535) return TS_BAD_SHAPE;

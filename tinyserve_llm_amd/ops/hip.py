@@ -227,9 +227,10 @@ DECODE_HEAD_DIMS = (32, 64, 96, 128)
 MAX_DECODE_WAVES = 8
 
 
-def decode_waves(hd: int) -> int:
-    """Most waves of a workgroup of the decode kernel: heads wider than 64 leave registers for 4."""
-    return 4 if hd > 64 else MAX_DECODE_WAVES
+def decode_waves(hd: int, one_step: bool = False) -> int:
+    """Most waves of a workgroup of the decode kernel: heads wider than 64 leave the loop over
+    several steps registers for 4; the instance with one step per wave has room for 8."""
+    return 4 if hd > 64 and not one_step else MAX_DECODE_WAVES
 
 
 DECODE_ONE_STEP_SPLITS = 18      # up to this many chunks per token a wave takes one 32-key step (the leanest instance)
@@ -247,21 +248,25 @@ def decode_plan(num_tokens: int, nkv: int, group: int, hd: int, capacity: int) -
     chunks as give the chip about one workgroup per compute unit, since the time of the combining
     kernel grows with the number of chunks (head size 128, 8 tokens over 16K keys: 151 µs in
     128-key chunks, 109 µs in 4,096-key chunks)."""
-    most = decode_waves(hd)
-    while most > 1 and 4 * (32 * most + most * group * hd) > 65536:
-        most //= 2
-    one = 32 * most
+    def fitting(waves: int) -> int:          # the waves' partial results meet in 64 KB of LDS
+        while waves > 1 and 4 * (32 * waves + waves * group * hd) > 65536:
+            waves //= 2
+        return waves
+    most, wide = fitting(decode_waves(hd)), fitting(decode_waves(hd, one_step=True))
+    one = 32 * wide
     if capacity <= one:
         waves = -(-capacity // 32)
         return 32 * waves, waves
     rows = num_tokens * nkv
     if rows >= DECODE_TARGET_WORKGROUPS:
-        chunk = -(-capacity // one) * one if capacity <= 16384 else DECODE_MAX_CHUNK
+        step = 32 * most
+        chunk = -(-capacity // step) * step if capacity <= 16384 else DECODE_MAX_CHUNK
     elif -(-capacity // one) <= DECODE_ONE_STEP_SPLITS:
-        chunk = one
+        return one, wide
     else:
+        step = 32 * most
         splits = max(1, DECODE_TARGET_WORKGROUPS // rows)
-        chunk = min(max(-(-capacity // (splits * one)) * one, one), DECODE_MAX_CHUNK)
+        chunk = min(max(-(-capacity // (splits * step)) * step, step), DECODE_MAX_CHUNK)
     while -(-capacity // chunk) > MAX_DECODE_SPLITS:
         chunk *= 2
     return chunk, most
@@ -302,7 +307,7 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
         chunk, waves = decode_plan(T, nkv, nh // nkv, hd, capacity)
     waves = waves or 4
     splits = -(-capacity // chunk)
-    _need(1 <= waves <= decode_waves(hd) and chunk % (32 * waves) == 0 and splits <= MAX_DECODE_SPLITS,
+    _need(1 <= waves <= decode_waves(hd, chunk == 32 * waves) and chunk % (32 * waves) == 0 and splits <= MAX_DECODE_SPLITS,
           f"chunk {chunk} in {waves} waves over {capacity} positions")
     _need(4 * (32 * waves + waves * (nh // nkv) * hd) <= 65536, f"{waves} waves of {nh // nkv} heads exceed the LDS of a workgroup")
     part_o = part_ml = None
