@@ -12,8 +12,7 @@ from __future__ import annotations
 
 import struct
 from array import array
-from dataclasses import dataclass, field
-from typing import Protocol, Sequence
+from typing import NamedTuple, Protocol, Sequence
 
 import torch
 
@@ -23,12 +22,11 @@ from tinyserve_llm_amd.models.decoder import DecoderModel
 from tinyserve_llm_amd.parts.base import LayerMemory, StepContext
 
 
-@dataclass
-class StepEntry:
+class StepEntry(NamedTuple):          # (a tuple: a step of hundreds of requests makes one for each of them)
     seq_id: int
     tokens: Sequence[int]
-    start: int                                        # position of tokens[0] in its request
-    want: Sequence[int] = field(default_factory=list)  # indices into `tokens` whose logits are wanted
+    start: int                        # position of tokens[0] in its request
+    want: Sequence[int] = ()          # indices into `tokens` whose logits are wanted
 
 
 class TableView(Protocol):

@@ -168,7 +168,10 @@ class Scheduler:
         first. Victims of a page shortage are the lowest-ranked sequences of either kind that
         this step has not scheduled."""
         mine = [s for s in self.running if s.in_prefill == want_prefill and not s.in_step]
-        mine.sort(key=lambda s: self._score(s.admission_hit, s, now))       # lowest first
+        if want_prefill or budget < len(mine) or not self.kv.fits([len(mine)] * len(self.kv.spaces)):
+            mine.sort(key=lambda s: self._score(s.admission_hit, s, now))       # lowest first
+        # (decoding sequences that all fit, in tokens and in pages, a page each at most, need no ranking:
+        # all of them run, and the step lays them out by context length anyway)
         scheduled: list[ScheduledSeq] = []
         gone: set[int] = set()
         while mine:
