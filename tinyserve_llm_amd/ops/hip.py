@@ -236,6 +236,7 @@ def decode_waves(hd: int, one_step: bool = False) -> int:
 DECODE_ONE_STEP_SPLITS = 18      # up to this many chunks per token a wave takes one 32-key step (the leanest instance)
 DECODE_TARGET_WORKGROUPS = 256   # beyond: as many chunks as give every compute unit a workgroup,
 DECODE_MAX_CHUNK = 4096          # of at most this many keys
+DECODE_FILL = 0.8                # a last round of workgroups should fill this share of the compute units
 
 
 def decode_plan(num_tokens: int, nkv: int, group: int, hd: int, capacity: int) -> tuple[int, int]:
@@ -247,7 +248,9 @@ def decode_plan(num_tokens: int, nkv: int, group: int, hd: int, capacity: int) -
     has a single 32-key step (the instance without a second buffer); longer ones into as many
     chunks as give the chip about one workgroup per compute unit, since the time of the combining
     kernel grows with the number of chunks (head size 128, 8 tokens over 16K keys: 151 µs in
-    128-key chunks, 109 µs in 4,096-key chunks)."""
+    128-key chunks, 109 µs in 4,096-key chunks). Among the chunk lengths the one is taken whose
+    workgroups come in full rounds of one per compute unit (48 tokens of 8 heads over 8,192 keys:
+    384 workgroups that each take the whole context 332 µs, 768 that take half of it 289 µs)."""
     def fitting(waves: int) -> int:          # the waves' partial results meet in 64 KB of LDS
         while waves > 1 and 4 * (32 * waves + waves * group * hd) > 65536:
             waves //= 2
@@ -258,15 +261,26 @@ def decode_plan(num_tokens: int, nkv: int, group: int, hd: int, capacity: int) -
         waves = -(-capacity // 32)
         return 32 * waves, waves
     rows = num_tokens * nkv
-    if rows >= DECODE_TARGET_WORKGROUPS:
-        step = 32 * most
-        chunk = -(-capacity // step) * step if capacity <= 16384 else DECODE_MAX_CHUNK
+    step = 32 * most
+    whole = -(-capacity // step) * step if capacity <= 16384 else DECODE_MAX_CHUNK
+
+    def fills(workgroups: int) -> bool:
+        """Whether so many workgroups come in rounds of about one per compute unit: 256, 512 or 768
+        of them keep the chip busy to the end, 192 or 384 leave a quarter of it idle."""
+        rounds = -(-workgroups // DECODE_TARGET_WORKGROUPS)
+        return workgroups >= DECODE_FILL * rounds * DECODE_TARGET_WORKGROUPS
+
+    cut = [c for c in (4096, 2048, 1024, 512) if c % step == 0 and c < capacity]
+    if rows >= DECODE_FILL * DECODE_TARGET_WORKGROUPS:
+        chunk = whole
+        if not fills(rows * -(-capacity // whole)) and rows < 4 * DECODE_TARGET_WORKGROUPS:
+            chunk = next((c for c in cut if fills(rows * -(-capacity // c))), whole)
     elif -(-capacity // one) <= DECODE_ONE_STEP_SPLITS:
         return one, wide
     else:
-        step = 32 * most
         splits = max(1, DECODE_TARGET_WORKGROUPS // rows)
-        chunk = min(max(-(-capacity // (splits * step)) * step, step), DECODE_MAX_CHUNK)
+        chunk = next((c for c in cut if fills(rows * -(-capacity // c))),
+                     min(max(-(-capacity // (splits * step)) * step, step), DECODE_MAX_CHUNK))
     while -(-capacity // chunk) > MAX_DECODE_SPLITS:
         chunk *= 2
     return chunk, most
