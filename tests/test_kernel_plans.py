@@ -75,8 +75,9 @@ def test_decode_plan_divides_the_context_into_32_key_steps_per_wave():
     assert hip.decode_plan(4, 8, 4, 64, 8192) == (1024, 8)
     # workgroups in full rounds of one per compute unit: 384 that take everything leave a quarter of the chip idle
     assert hip.decode_plan(48, 8, 4, 128, 8192) == (4096, 4)       # 768 workgroups instead of 384
-    assert hip.decode_plan(48, 8, 4, 128, 4096) == (2048, 4)
-    assert hip.decode_plan(24, 8, 4, 128, 8192) == (2048, 4)       # 768 instead of 384 in chunks of 4,096
-    assert hip.decode_plan(12, 8, 4, 64, 16384) == (2048, 8)
+    assert hip.decode_plan(48, 8, 4, 128, 4096) == (256, 8)        # a short context: the one-step form instead
+    assert hip.decode_plan(20, 8, 4, 128, 16384) == (2816, 4)      # 6 chunks of equal length: 960 workgroups, four rounds
+    assert hip.decode_plan(12, 8, 4, 128, 8192) == (1664, 4)       # 5 chunks of equal length: 480 workgroups
     assert hip.decode_plan(31, 8, 4, 128, 8192) == (8192, 4)       # 248 workgroups are as good as 256
-    assert hip.decode_plan(80, 8, 4, 64, 2304) == (2304, 8)        # 640 of 768: full enough
+    assert hip.decode_plan(24, 8, 4, 64, 2304) == (2304, 8)        # and so are 192
+    assert hip.decode_plan(80, 8, 4, 64, 2304) == (256, 8)         # 640 of 768 are not
