@@ -10,6 +10,7 @@ logits [wanted, vocab] in the order of the entries and of their `want` lists.
 
 from __future__ import annotations
 
+import gc
 import struct
 from array import array
 from typing import NamedTuple, Protocol, Sequence
@@ -370,10 +371,20 @@ class DecodeGraphs:
         torch.cuda.current_stream(r.device).wait_stream(side)
         torch.cuda.synchronize(r.device)
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, pool=self.pool):
-            hidden, residual = r.model.forward(ctx, r.memory)
-            logits = r.model.logits(hidden, residual, rows)
-            tokens = hip.sample(logits, draw_temps, draw_keys, self.seed)
+        # No garbage collection while the stream is being captured: an engine that the process has
+        # dropped earlier may still be waiting to be collected, and destroying its graphs is an
+        # operation the capture forbids (the process then aborts in the graph's destructor). The
+        # capture collects what is pending when it is entered.
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph, pool=self.pool):
+                hidden, residual = r.model.forward(ctx, r.memory)
+                logits = r.model.logits(hidden, residual, rows)
+                tokens = hip.sample(logits, draw_temps, draw_keys, self.seed)
+        finally:
+            if collecting:
+                gc.enable()
         if self.pool is None:
             self.pool = graph.pool()
         # the drawn tokens travel to the host through two pinned buffers in turn: a step may be
