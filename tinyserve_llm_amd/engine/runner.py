@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import gc
 import struct
+import weakref
 from array import array
 from typing import NamedTuple, Protocol, Sequence
 
@@ -305,7 +306,7 @@ class DecodeGraphs:
     the tokens drawn from them; a caller that only wants logits ignores the tokens."""
 
     def __init__(self, runner: ModelRunner, max_context: int, max_batch: int, seed: int = 0) -> None:
-        self.runner = runner
+        self.runner = weakref.proxy(runner)     # (the runner owns the graphs: no cycle, so a dropped engine's memory is freed at once)
         self.page_size = runner.storage.page_size
         self.num_spaces = len(runner.storage.spaces)
         self.bucket = max(256, self.page_size)
