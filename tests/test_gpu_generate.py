@@ -441,3 +441,37 @@ def test_the_engines_own_tiled_products_serve_steps_of_many_rows(tmp_path):
             at = next(i for i, (x_, y_) in enumerate(zip(a_, b_)) if x_ != y_)
             row = plain.logits(p_ + a_[:at])[-1]
             assert float(row.max() - row[[a_[at], b_[at]]].min()) <= 3e-2 * float(row.max() - row.min())
+
+
+@pytest.mark.parametrize("case", range(10))
+def test_random_workloads_generate_the_same_under_every_engine_setting(case, folder_a, folder_b):
+    """Random requests (shared prefixes, forks, sampling, end tokens, lengths), page sizes, pools
+    so small that sequences are preempted, token budgets, portions: recorded or eager decode steps,
+    steps closed in two halves or in one, prefix cache on or off must all generate the same tokens
+    in float32."""
+    import random
+
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+    rng = random.Random(1000 + case)
+    folder, vocab = (folder_a, 256) if rng.random() < 0.5 else (folder_b, 384)
+    shared = prompt(2000 + case, rng.randint(0, 40), vocab - 1)
+    prompts, params = [], []
+    for i in range(rng.randint(3, 24)):
+        prompts.append((shared if rng.random() < 0.4 else []) + prompt(case * 100 + i, rng.randint(1, 60), vocab - 1))
+        params.append(SamplingParams(max_tokens=rng.randint(1, 20), temperature=rng.choice([0.0, 0.0, 0.8]),
+                                     n=rng.choice([1, 1, 1, 2, 3]), ignore_eos=rng.random() < 0.5))
+    page = rng.choice([4, 8, 16])
+    need = max(-(-(len(p) + sp.max_tokens) // page) * sp.n for p, sp in zip(prompts, params))
+    blocks = rng.choice([need + 2, need * 2, need * 6, 400])
+    seqs = rng.choice([4, 8, 40])
+    sc = SchedulerConfig(max_model_len=128, max_num_seqs=seqs, max_num_batched_tokens=max(rng.choice([64, 128, 512]), seqs + 1),
+                         max_prefill_chunk=rng.choice([0, 0, 7, 32]), watermark=0.0)
+    outs = []
+    for graphs, ahead, caching in ((False, False, False), (True, True, True), (True, False, False), (False, True, True)):
+        llm = LLM(folder, sc, CacheConfig(block_size=page, caching=caching), dtype=torch.float32, num_blocks=blocks, seed=case,
+                  decode_graphs=graphs, run_ahead=ahead)
+        outs.append([(c.token_ids, c.finish_reasons) for c in llm.generate(prompts, params)])
+        assert caching or llm.manager.num_available_blocks() == llm.manager.num_blocks, "pages leaked"
+    assert outs[1] == outs[0] and outs[2] == outs[0] and outs[3] == outs[0]
