@@ -52,6 +52,7 @@ __device__ __forceinline__ void wave_sync() {
 #define TS_BAD_DTYPE 1
 #define TS_BAD_SHAPE 2
 #define TS_LAUNCH_FAILED 3
+#define TS_TOO_LARGE 4
 
 static inline int ts_check_launch() {
   return hipGetLastError() == hipSuccess ? TS_OK : TS_LAUNCH_FAILED;

@@ -109,3 +109,46 @@ extern "C" int ts_feed_tokens(int32_t* ids, const int32_t* prev, const int32_t* 
   feed_tokens_kernel<<<(n + 255) / 256, 256, 0, stream>>>(ids, prev, src, n, prev_n);
   return ts_check_launch();
 }
+
+// ---- the draw without any allocation ---------------------------------------------------------------
+// `ts_sample_static` is `ts_sample` with the two workspaces taken from a fixed array in device
+// memory instead of from the caller (declared in sample_static.h, which says whom it is for).
+// The array's name is only a handle on the host: the address that kernels and copies may use is
+// asked for once per device, with that device current, and kept.
+#include <mutex>
+#include "sample_static.h"
+
+#define SAMPLE_STATIC_BYTES ((size_t)TS_SAMPLE_STATIC_MAX_ROWS * SAMPLE_SLICES * (sizeof(float) + sizeof(int32_t)))
+#define SAMPLE_STATIC_MAX_DEVICES 64
+
+static __device__ __align__(256) unsigned char sample_scratch[SAMPLE_STATIC_BYTES];
+
+static std::mutex sample_scratch_lock;
+static void* sample_scratch_ptr[SAMPLE_STATIC_MAX_DEVICES];   // per device: where its copy of the array lies
+
+// The current device's copy of the array, or nullptr if the runtime will not name it.
+static void* sample_scratch_here() {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= SAMPLE_STATIC_MAX_DEVICES) return nullptr;
+  std::lock_guard<std::mutex> hold(sample_scratch_lock);
+  if (sample_scratch_ptr[device] == nullptr) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(sample_scratch)) != hipSuccess) return nullptr;
+    sample_scratch_ptr[device] = ptr;
+  }
+  return sample_scratch_ptr[device];
+}
+
+extern "C" int ts_sample_static(int32_t* out, const float* logits, const float* temps, const int64_t* keys,
+                                uint64_t seed, int rows, int vocab, int64_t ld, hipStream_t stream) {
+  if (rows <= 0) return TS_OK;
+  if (rows > TS_SAMPLE_STATIC_MAX_ROWS) return TS_TOO_LARGE;
+  if (!out || !logits || !temps || !keys) return TS_BAD_SHAPE;
+  unsigned char* base = (unsigned char*)sample_scratch_here();
+  if (base == nullptr) return TS_LAUNCH_FAILED;
+  // every (row, slice) place that the second kernel reads is written by the first kernel of the same
+  // call, so nothing of the last call's contents has to be cleared
+  float* work_v = (float*)base;
+  int32_t* work_i = (int32_t*)(base + (size_t)TS_SAMPLE_STATIC_MAX_ROWS * SAMPLE_SLICES * sizeof(float));
+  return ts_sample(out, work_v, work_i, logits, temps, keys, seed, rows, vocab, ld, stream);
+}

@@ -20,7 +20,8 @@ _lib = None
 _lock = threading.Lock()
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
-_ERRORS = {1: "unsupported storage type", 2: "unsupported shape or stride", 3: "the kernel launch failed"}
+_ERRORS = {1: "unsupported storage type", 2: "unsupported shape or stride", 3: "the kernel launch failed",
+           4: "more than the entry point's fixed workspace holds"}
 
 
 class KernelError(RuntimeError):
@@ -53,6 +54,7 @@ def _declare(lib: ctypes.CDLL) -> None:
                                       i, p],
         "ts_gemm_exact": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_sample": [p, p, p, p, p, p, u64, i, i, i64, p],
+        "ts_sample_static": [p, p, p, p, u64, i, i, i64, p],
         "ts_feed_tokens": [p, p, p, i, i, p],
         "ts_gemm_library_bf16": [p, p, p, i, i, i, i64, i64, i64, i, p, ctypes.c_size_t, p],
         "ts_gemm_tiled_bf16": [p, p, p, i, i, i, i64, i64, i64, i, p],
