@@ -17,11 +17,12 @@ B = 4
 class FakeStorage:
     """Each slot of each space holds the token id whose keys/values it stores (None = never written)."""
 
-    def __init__(self, pages=12, windows=(0,), state_slots=64):
+    def __init__(self, pages=12, windows=(0,), state_slots=64, keeps_state=False):
         pages = pages if isinstance(pages, (list, tuple)) else [pages] * len(windows)
         self.page_size = B
         self.spaces = [SpaceSpec(n, w) for n, w in zip(pages, windows)]
         self.num_state_slots = state_slots
+        self.keeps_state = keeps_state
         self.slots = [[[None] * B for _ in range(n)] for n in pages]
         self.copies: list[tuple[int, int, int]] = []      # of space 0
         self.state = [None] * state_slots
@@ -38,8 +39,8 @@ class FakeStorage:
         self.state[slot] = 0
 
 
-def make(pages=12, caching=True, windows=(0,)):
-    return KVCacheManager(FakeStorage(pages, windows), caching=caching)
+def make(pages=12, caching=True, windows=(0,), keeps_state=False):
+    return KVCacheManager(FakeStorage(pages, windows, keeps_state=keeps_state), caching=caching)
 
 
 def forward(m, seq_id):
@@ -113,9 +114,10 @@ def check_invariants(m):
     used = [s.state_slot for s in m.seqs.values()]
     assert len(set(used)) == len(used) and not set(used) & set(m.free_state_slots)
     assert sorted(used + m.free_state_slots) == list(range(m.storage.num_state_slots)), "a state slot is lost"
-    for s in m.seqs.values():
-        assert m.storage.state[s.state_slot] == sum(s.token_ids[:s.committed]) or m.caching, \
-            "the state slot does not hold this request's state"
+    if m.storage.keeps_state:
+        for s in m.seqs.values():
+            assert m.storage.state[s.state_slot] == sum(s.token_ids[:s.committed]), \
+                "the state slot does not hold this request's state"
 
 
 # ---- admission (tests/test_kvcache_manager.py:89-199) ---------------------------------------------
@@ -334,8 +336,22 @@ def test_forks_copy_the_shared_tail_one_by_one():
     check_invariants(m)
 
 
+def test_a_model_with_state_reuses_no_prefix():
+    """A state slot starts empty at admission and is built only by the tokens that are fed: with
+    prefix reuse the skipped tokens would be missing from it, so the manager turns reuse off by
+    itself, also for a request that comes back after it gave up its pages."""
+    m = make(keeps_state=True)
+    assert not m.caching
+    prefill(m, 1, list(range(10)))
+    m.release(1)
+    assert m.calculate_admission_cost(list(range(10))).prefill_tokens == 10
+    prefill(m, 2, list(range(10)))
+    assert m.num_cached_tokens(2) == 10 and m.storage.state[m.seqs[2].state_slot] == 45
+    check_invariants(m)
+
+
 def test_fork_copies_the_state_slot():
-    m = make(caching=False)
+    m = make(keeps_state=True)
     prefill(m, 1, [1, 2, 3])
     m.fork(1, 2)
     assert m.seqs[2].state_slot != m.seqs[1].state_slot
@@ -455,15 +471,17 @@ def test_window_space_limits_admission():
 # ---- random orders of requests -----------------------------------------------------------------------
 
 @pytest.mark.parametrize("seed", range(12))
-@pytest.mark.parametrize("setup", ["cached", "uncached", "windowed"])
+@pytest.mark.parametrize("setup", ["cached", "uncached", "windowed", "stateful"])
 def test_random_workload_keeps_every_invariant(seed, setup):
     """Admissions in portions, decodes, multi-token appends with partial acceptance, forks,
     releases, in random order (after tests/test_kvcache_manager.py:577-618)."""
     rng = random.Random(seed)
     if setup == "windowed":
-        m = make(pages=[16, 7], windows=(0, 5))
+        m = make(pages=[16, 7], windows=(0, 5), keeps_state=True)
     else:
-        m = make(pages=16, caching=setup == "cached")
+        # ("stateful" asks for prefix reuse as the engine does by default; the manager declines)
+        m = make(pages=16, caching=setup != "uncached", keeps_state=setup != "cached")
+    assert m.caching == (setup == "cached")
     families = [[rng.randrange(6) for _ in range(rng.randrange(2, 14))] for _ in range(4)]
     next_id, pending = 0, {}
     for _ in range(250):

@@ -150,9 +150,29 @@ def register_toy_parts():
                 state[-1] = counts[-1]
             return out
 
+    @register("mixer", "toy_running_mean_on_device")
+    class RunningMeanOnDevice(RunningMean):
+        """The same mixer from the step's device tensors alone (no host lists, no branches on
+        them), so that decode steps with it can be recorded into graphs and replayed."""
+
+        graph_safe = True
+
+        def forward(self, x, ctx, mem):
+            seq, slots, cu = ctx.seq_of_token.long(), ctx.state_slots.long(), ctx.cu_seqlens.long()
+            carried = mem.state[slots] * (ctx.positions.long()[cu[:-1]] != 0).unsqueeze(1)   # a request's first token starts it
+            run = torch.cumsum(x.float(), 0)
+            before = torch.cat([run.new_zeros(1, run.shape[1]), run])[cu[:-1]]                # the sum up to each request's rows
+            sums = carried[seq, :-1] + (run - before[seq])
+            counts = (ctx.positions + 1).float()
+            last = cu[1:] - 1
+            mem.state[slots] = torch.cat([sums[last], counts[last, None]], 1)
+            return (sums / counts[:, None]).to(x.dtype) @ self.w.T
+
     @register("feed_forward", "toy_routed")
     class Routed(FeedForward):
         """Top-1 of E small experts, chosen by a 32-bit router."""
+
+        graph_safe = True
 
         def __init__(self, hidden_size, experts):
             self.hidden_size, self.experts = hidden_size, experts
@@ -170,6 +190,8 @@ def register_toy_parts():
     class Learned(PositionEncoding):
         """A learned vector per position, added to the embedded tokens."""
 
+        graph_safe = True
+
         def __init__(self, hidden_size, max_position):
             self.hidden_size, self.max_position = hidden_size, max_position
 
@@ -180,13 +202,13 @@ def register_toy_parts():
             return hidden + self.table[ctx.positions.long()]
 
 
-def toy_spec(hidden=48, vocab=97):
+def toy_spec(hidden=48, vocab=97, mean_mixer="toy_running_mean"):
     from tinyserve_llm_amd.models.spec import LayerRun, LayerSpec, ModelSpec
     from tinyserve_llm_amd.parts.base import PartSpec
     norm = PartSpec("rmsnorm", dict(hidden_size=hidden, eps=1e-5))
     mlp = PartSpec("gated_mlp", dict(hidden_size=hidden, intermediate_size=64))
     attn = PartSpec("attention", dict(hidden_size=hidden, num_heads=3, num_kv_heads=1, head_dim=16, position=None))
-    layers = [LayerSpec(PartSpec("toy_running_mean", dict(hidden_size=hidden)), mlp, norm, norm),
+    layers = [LayerSpec(PartSpec(mean_mixer, dict(hidden_size=hidden)), mlp, norm, norm),
               LayerSpec(attn, PartSpec("toy_routed", dict(hidden_size=hidden, experts=3)), norm, norm)]
     return ModelSpec(architecture="Toy", vocab_size=vocab, hidden_size=hidden, max_position=128, layers=layers,
                      order=[LayerRun(0), LayerRun(1), LayerRun(0)], final_norm=norm,
@@ -205,7 +227,8 @@ def toy_engine(dtype, seed=0, pages=24, page=8):
     params = random_params(model, seed, dtype, "cpu")
     model.bind({k: v.to(DEV) for k, v in params.items()}, dtype, torch.device(DEV))
     storage = KVStorage(model.cache_plan(), model.state_plan(), pages, page, dtype, DEV, num_state_slots=4)
-    manager = KVCacheManager(storage, caching=False)
+    manager = KVCacheManager(storage)
+    assert not manager.caching, "a model with state slots reuses no prefix"
     return model, {k: v.double() for k, v in params.items()}, storage, manager, ModelRunner(model, storage, manager)
 
 
@@ -268,6 +291,46 @@ def test_toy_parts_register_build_and_step_without_touching_the_framework():
         torch.testing.assert_close(row.double().cpu(), want, rtol=1e-4, atol=1e-5, msg=lambda m: f"{name}{pos}: {m}")
     manager.release(0)
     assert manager.num_available_blocks() == manager.num_blocks and len(manager.free_state_slots) == 4
+
+
+def test_a_model_with_state_generates_through_the_entry_point_with_every_default():
+    """The toy model whose mixer keeps state, through `LLM.generate` as any model goes: prefix reuse
+    asked for (the default), prompts that share prefixes and repeat, portions, a pool so small that
+    requests give up their pages and come back, decode steps replayed from graphs. A reused prefix
+    or a step counted twice would leave tokens out of, or twice in, the running mean."""
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+    from tinyserve_llm_amd.models.decoder import DecoderModel
+    from tinyserve_llm_amd.weights.random_init import random_params
+    register_toy_parts()
+    model = DecoderModel(toy_spec(mean_mixer="toy_running_mean_on_device"))
+    params = random_params(model, 5, torch.float32, "cpu")
+    model.bind({k: v.to(DEV) for k, v in params.items()}, torch.float32, torch.device(DEV))
+    p = {k: v.double() for k, v in params.items()}
+
+    def plain_greedy(ids, n):
+        ids, out = list(ids), []
+        for _ in range(n):
+            out.append(int(toy_plain(p, ids)[-1].argmax()))
+            ids.append(out[-1])
+        return out
+
+    shared = [3, 50, 7, 7, 96, 1, 0, 22, 41]
+    prompts = [shared + [5], shared + [88, 13], shared[:6], [9, 8, 7, 6, 5], shared + [5], shared[:8] + [60]]
+    want = [plain_greedy(q, 10) for q in prompts]
+    sc = SchedulerConfig(max_model_len=64, max_num_seqs=4, max_num_batched_tokens=24, max_prefill_chunk=7)
+    llm = LLM(None, sc, CacheConfig(block_size=4), model=model, num_blocks=16)
+    assert llm.runner.graphs is not None, "every toy part is recordable"
+    assert not llm.manager.caching, "the manager has seen the state slots"
+    sp = SamplingParams(max_tokens=10, temperature=0.0, ignore_eos=True)
+    for _ in range(2):           # the second round finds the first round's pages free, and must not reuse them
+        got = llm.generate(prompts, sp)
+        assert [r.token_ids[0] for r in got] == want
+    st = llm.scheduler.stats()
+    assert st.preemptions > 0 and st.cached_tokens == 0
+    assert len(llm.runner.graphs.graphs) > 0, "decode steps were replayed from graphs"
+    assert llm.manager.stats().blocks_in_use == 0 and len(llm.manager.free_state_slots) == 4
 
 
 def test_a_layer_can_read_another_layers_cache():

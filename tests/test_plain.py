@@ -1,9 +1,12 @@
 """What fixes the plain implementation beside the reference's text: special cases that reduce to
 a library routine, invariants, and the numbers the reference's tests state. Each is chosen so
 that a plausible mistake (a wrong sign or pairing in the rotation, a norm in the wrong place, a
-head served by the wrong key/value head) fails it. Parity with the library's llama3 frequency
-initialiser, which the reference pins bit-for-bit (tests/test_llama.py:99-109), is unpinned here:
-that library's model code is not a source; band membership and limits stand in for it."""
+head served by the wrong key/value head) fails it. The reference pins its llama3 frequencies
+bit-for-bit to an installed library's initialiser at run time (tests/test_llama.py:99-109,141-142)
+and holds no numbers of its own; that library's model code is not a source here, so bit parity
+with it is unpinned. In its place every frequency is checked against the published formula
+evaluated band by band in float64 by separate code, and the blended ones against numbers worked
+out by hand, at the reference test's configuration, at configuration B and at Llama 3.2 1B's values."""
 
 import math
 
@@ -72,6 +75,53 @@ def test_llama3_scaling_bands_and_limits():
     # a missing original_max_position_embeddings means the table length (llama.py:155)
     short = P.rope_inv_freq(32, 500000.0, dict(factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0), 64)
     torch.testing.assert_close(short, scaled)
+
+
+def llama3_by_bands(head_dim, theta, factor, low, high, old_len):
+    """The llama3 rule one frequency at a time, in float64 (arXiv 2407.21783 section 3.4.1 as
+    restated by tinyserve_llm/model/llama.py:107-128): wavelengths shorter than old_len / high are
+    kept, longer than old_len / low are divided by the factor, and those between are a blend
+    whose weight on the unchanged frequency grows from 0 at the long end to 1 at the short end."""
+    out = []
+    for i in range(0, head_dim, 2):
+        f = theta ** (-i / head_dim)
+        wavelength = 2 * math.pi / f
+        if wavelength < old_len / high:
+            out.append(f)
+        elif wavelength > old_len / low:
+            out.append(f / factor)
+        else:
+            keep = (old_len / wavelength - low) / (high - low)
+            out.append(keep * f + (1 - keep) * f / factor)
+    return out
+
+
+# (head_dim, theta, factor, low, high, original length) -> the blended frequencies, worked out by hand
+LLAMA3_CASES = {
+    "reference test (tests/test_llama.py:23-30)": ((16, 10000.0, 4.0, 1.0, 4.0, 32), {1: 0.127323954}),
+    "configuration B": ((32, 500000.0, 8.0, 1.0, 4.0, 64), {2: 0.0794030092}),
+    "Llama 3.2 1B": ((64, 500000.0, 32.0, 1.0, 4.0, 8192), {15: 0.00129054793, 16: 0.000429556797, 17: 9.7082878e-05}),
+}
+
+
+@pytest.mark.parametrize("name", LLAMA3_CASES)
+def test_llama3_frequencies_equal_the_formula_band_by_band(name):
+    """A blend with its weights swapped gives 0.139 instead of 0.0794 at configuration B; a band
+    edge taken on the wrong side moves a frequency by the whole factor."""
+    from tinyserve_llm_amd.parts.rope import inverse_frequencies
+    (head_dim, theta, factor, low, high, old_len), blended = LLAMA3_CASES[name]
+    scaling = dict(factor=factor, low_freq_factor=low, high_freq_factor=high, original_max_position_embeddings=old_len)
+    want = torch.tensor(llama3_by_bands(head_dim, theta, factor, low, high, old_len), dtype=D)
+    plain = P.rope_inv_freq(head_dim, theta, scaling, 4 * old_len)
+    product = inverse_frequencies(head_dim, theta, scaling, 4 * old_len)
+    assert plain.dtype == product.dtype == torch.float32
+    torch.testing.assert_close(plain.double(), want, rtol=2e-6, atol=0)         # float32 arithmetic against float64
+    torch.testing.assert_close(product, plain, rtol=0, atol=0)                  # the engine's table, bit for bit
+    for i, value in blended.items():
+        assert abs(float(plain[i]) / value - 1) < 2e-6, (i, float(plain[i]), value)
+    base = 1.0 / theta ** (torch.arange(0, head_dim, 2, dtype=D) / head_dim)
+    moved = ~torch.isclose(plain.double(), base, rtol=1e-5)
+    assert moved.any() and not moved.all()                                      # the case touches some bands and spares others
 
 
 def test_attention_reduces_to_the_library_routine_and_to_its_limits():

@@ -11,7 +11,8 @@ What is added:
     pools of all of them); layers that only ever read a window of W positions get a space of
     their own, with their own page ids and block tables, and give a page back as soon as the
     window has passed it. Prefix reuse needs every layer's pages to be restorable, so it is only
-    on when all layers are in space 0.
+    on when all layers are in space 0 and none keeps per-request state (a state slot is rebuilt only
+    by feeding the tokens again).
   * portions. `allocate(..., feed=n)` reserves slots for the first n uncached tokens only; the
     rest of a prompt follows through `append_slots`, like decoded tokens.
   * a slot of fixed-size per-request state, taken at allocate, copied at fork, returned at
@@ -40,6 +41,7 @@ class Storage(Protocol):
     page_size: int
     spaces: Sequence[SpaceSpec]
     num_state_slots: int
+    keeps_state: bool     # some layer folds every token it is fed into its request's state slot
 
     def copy_slots(self, space: int, src: int, dst: int, num_slots: int) -> None: ...
     def copy_state(self, src_slot: int, dst_slot: int) -> None: ...
@@ -140,8 +142,12 @@ class KVCacheManager:
         self.block_size = storage.page_size
         self.spaces = [PageSpace(s, self.block_size) for s in storage.spaces]
         assert self.spaces, "a model without any cache still gets one (empty) space"
-        # a prefix can only be reused if every layer's pages for it still exist
-        self.caching = caching and len(self.spaces) == 1 and self.spaces[0].window == 0
+        # A reused prefix is never fed to the model again, so every layer must find what it keeps of
+        # those tokens still in place: pages of a space without a window qualify; pages that a window
+        # has given back do not, and neither does a state slot, which starts empty at admission and
+        # is only ever built by feeding the tokens. A model with either runs every prompt in full.
+        self.caching = (caching and len(self.spaces) == 1 and self.spaces[0].window == 0
+                        and not storage.keeps_state)
         self.seqs: dict[int, SeqState] = {}
         self.free_state_slots = list(range(storage.num_state_slots - 1, -1, -1))
         self.counters = CacheStats()

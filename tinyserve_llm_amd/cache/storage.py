@@ -88,6 +88,12 @@ class KVStorage:
             e.run: torch.zeros((num_state_slots, *e.state.shape), dtype=e.state.dtype, device=self.device)
             for e in state_plan}
 
+    @property
+    def keeps_state(self) -> bool:
+        """Whether some run of the model keeps per-request state (the cache manager then reuses no
+        prefix: a skipped token would be missing from the state)."""
+        return bool(self.states)
+
     def layer_cache(self, owner: int) -> tuple[torch.Tensor, torch.Tensor, int]:
         """(k view, v view, page space) of the cache that run `owner` of the order owns; the views
         are addressed [pages, page_size, kv_heads, head_dim] (a permuted view of the pool)."""
@@ -97,6 +103,10 @@ class KVStorage:
 
     def state(self, run: int) -> torch.Tensor | None:
         return self.states.get(run)
+
+    def state_tensors(self) -> list[torch.Tensor]:
+        """Every state tensor, [slots, ...] each (to save and restore around a step that must not count)."""
+        return list(self.states.values())
 
     def copy_slots(self, space: int, src: int, dst: int, num_slots: int) -> None:
         for group in self.groups:

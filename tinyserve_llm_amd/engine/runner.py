@@ -366,10 +366,17 @@ class DecodeGraphs:
         # the matrix library's candidates for this batch size are timed and the fastest kept
         side = torch.cuda.Stream(device=r.device)
         side.wait_stream(torch.cuda.current_stream(r.device))
+        # (this run and the first replay feed the same tokens: keys and values land in the same slots
+        # twice, which changes nothing, but a mixer's state would take the step twice, so the state
+        # slots are put back as they were)
+        states = r.storage.state_tensors()
+        before = [t.clone() for t in states]
         with hip.library_tuning(), torch.cuda.stream(side):      # (the sweep buffer belongs to the current stream)
             hidden, residual = r.model.forward(ctx, r.memory)
             hip.sample(r.model.logits(hidden, residual, rows), draw_temps, draw_keys, self.seed)
         torch.cuda.current_stream(r.device).wait_stream(side)
+        for t, kept in zip(states, before):
+            t.copy_(kept)
         torch.cuda.synchronize(r.device)
         graph = torch.cuda.CUDAGraph()
         # No garbage collection while the stream is being captured: an engine that the process has
