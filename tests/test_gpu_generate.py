@@ -104,6 +104,76 @@ def test_sampling_is_seeded_and_does_not_depend_on_the_batch(folder_b):
     assert d == a
 
 
+def race_scores(plain_row, temperature, seed, request, sample, position):
+    """What the sampler maximises, from the plain model's logits and the kernel's noise written out
+    on the host: logit / t - log E(seed, key of (request, sample, output position))."""
+    from tests.test_gpu_kernels import exp_noise
+    from tinyserve_llm_amd.sampling.sampler import row_key
+    noise = exp_noise(seed, row_key(request, sample, position), plain_row.shape[0])
+    return plain_row / temperature - noise.log()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shared", [64, 75])
+def test_drawn_tokens_of_a_workload_with_prefix_hits_forks_and_portions_against_the_plain_model(folder_b, dtype, shared):
+    """Configuration B's workload as the baseline states it: prompts of 1, 40, 70 and 129 tokens, the
+    last two behind a common prefix (64 tokens: two whole pages of 32; 75: it ends inside the third page,
+    whose leading slots are copied), the second drawn twice (n = 2: the samples share the prompt's pages
+    and copy its last one when they write), prompts fed in portions of 32 beside decoding requests,
+    12 tokens each at temperature 0.7, prefix reuse on. The fourth arrives when the third has ended
+    (only then is a page that is not full published), while the first two still decode. Every drawn
+    token is checked against the plain model run whole on the same history: in float32 it is the one
+    that wins the race under the kernel's noise; in bfloat16 it lies within a small gap of the winner."""
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+    vocab, seed, t = 384, 9, 0.7
+    common = prompt(50, shared, vocab)
+    tails = prompt(53, max(2, 70 - shared), vocab), prompt(54, 129 - shared, vocab)
+    assert tails[0][0] != tails[1][0], "the prompts part right after the common prefix"
+    prompts = [prompt(51, 1, vocab), prompt(52, 40, vocab), common + tails[0], common + tails[1]]
+    lengths = [12, 12, 3, 12]
+    plain = PlainLlama(folder_b, torch.float64, weights_as=torch.bfloat16)     # (the folder stores bfloat16 already)
+    llm = engine(folder_b, dtype=dtype, block_size=32, num_blocks=24, seed=seed, max_model_len=160, max_num_seqs=8,
+                 max_num_batched_tokens=48, max_prefill_chunk=32)
+
+    def add(i):
+        return llm.add_request(prompts[i], SamplingParams(max_tokens=lengths[i], temperature=t, n=2 if i == 1 else 1,
+                                                          ignore_eos=True), arrival_time=float(i))
+
+    ids = [add(0), add(1), add(2)]
+    done = {}
+    while llm.scheduler.has_unfinished():
+        for out in llm.step():
+            done[out.request_id] = out
+        if ids[2] in done and len(ids) == 3:
+            assert ids[0] not in done and ids[1] not in done, "the first two still decode when the fourth arrives"
+            ids.append(add(3))
+    st, cache = llm.scheduler.stats(), llm.manager.stats()
+    assert st.cached_tokens == shared, "the fourth prompt found the third one's pages"
+    assert cache.cow_copies >= 1, "the two samples copied the prompt's last page"
+    assert cache.partial_copies == (1 if shared % 32 else 0)
+    assert max(s.num_tokens for s in llm.steps) <= 48
+    assert sum(s.num_seqs >= 4 and s.num_tokens >= 20 for s in llm.steps) >= 2, "portions ran beside decoding requests"
+    checked = 0
+    for rid, q, n in zip(ids, prompts, lengths):
+        for seq in done[rid].sequences:
+            history = list(q)
+            assert len(seq.output_token_ids) == n
+            for i, tok in enumerate(seq.output_token_ids):
+                scores = race_scores(plain.logits(history)[-1], t, seed, rid, seq.sample_index, i)
+                where = f"request {rid} sample {seq.sample_index} token {i}"
+                if dtype == torch.float32:
+                    top = torch.topk(scores, 2).values
+                    assert tok == int(scores.argmax()) or float(top[0] - top[1]) < 1e-4, \
+                        f"{where}: drew {tok}, the race's winner is {int(scores.argmax())}"
+                else:
+                    assert float(scores.max() - scores[tok]) <= 0.06, where
+                history.append(tok)
+                checked += 1
+    assert checked == 12 + 2 * 12 + 3 + 12
+    two = done[ids[1]].sequences
+    assert two[0].output_token_ids != two[1].output_token_ids
+
+
 def test_the_end_token_stops_generation(folder_a):
     plain = PlainLlama(folder_a, torch.float64)
     full = plain.greedy(PROMPTS[0], 12)

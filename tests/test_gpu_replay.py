@@ -107,26 +107,30 @@ def test_portions_of_changing_size(case, dtype):
     check(got, oracles[dtype], dtype)
 
 
-def mixed_schedule(prompts):
-    """Steps that keep up to four requests live: while one decodes token by token, others feed
-    portions. Returns a list of (entries, end) with entries (request, start, count, want)."""
+MIXED_LENGTHS = {"A": [100, 33, 17, 5, 70, 120, 64, 9], "B": [129, 70, 40, 1, 65, 100, 128, 30, 200]}
+
+
+def mixed_schedule(prompts, pool_pages, page=64, most_live=4):
+    """Steps that keep up to four requests live on `pool_pages` pages: requests start in the order
+    given as soon as the pages for their whole length are free, feed portions of changing size
+    (often a single token) and end at different times, so that a request that starts later gets the
+    pages of one that has ended while others are still in the middle of theirs. Returns a list of
+    (entries, end) with entries (request, start, count, want)."""
     cursors = [0] * len(prompts)
-    order = sorted(range(len(prompts)), key=lambda r: -len(prompts[r]))
+    pages = [-(-len(p) // page) for p in prompts]
     chunk = [13, 2, 1, 7, 1, 1, 30, 1, 3, 1]
-    steps, tick = [], 0
-    while any(cursors[r] < len(prompts[r]) for r in order):
+    waiting, live, steps, tick = list(range(len(prompts))), [], [], 0
+    while waiting or live:
+        while waiting and len(live) < most_live and sum(pages[r] for r in live) + pages[waiting[0]] <= pool_pages:
+            live.append(waiting.pop(0))
         entries, end = [], []
-        for k, r in enumerate(order):
-            left = len(prompts[r]) - cursors[r]
-            if left == 0:
-                continue
-            if tick < 2 * k:            # staggered starts
-                continue
-            n = min(left, chunk[(tick + 3 * k) % len(chunk)])
+        for k, r in enumerate(live):
+            n = min(len(prompts[r]) - cursors[r], chunk[(tick + 3 * r) % len(chunk)])
             entries.append((r, cursors[r], n, [n - 1] if n > 1 else [0]))
             cursors[r] += n
             if cursors[r] == len(prompts[r]):
                 end.append(r)
+        live = [r for r in live if r not in end]
         steps.append((entries, end))
         tick += 1
     return steps
@@ -134,25 +138,37 @@ def mixed_schedule(prompts):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_mixed_requests_on_few_pages(case, dtype):
-    """The pool holds exactly what the four requests need at once (each rounded up to pages of
-    64); a second round of the same requests then has to run on pages that were used before."""
-    name, folder, config, prompts, oracles = case
-    need = sum(-(-len(p) // 64) * 64 for p in prompts)
-    rep = replayer(folder, dtype, need)
-    assert rep.manager.num_blocks == need // 64
-    for round_ in range(2):
-        got = {}
-        for entries, end in mixed_schedule(prompts):
-            batch = [{"id": f"q{round_}_{r}", "tokens": prompts[r][s:s + n], "want": w} for r, s, n, w in entries]
-            logits = rep.step(batch, [f"q{round_}_{r}" for r in end])
-            row = 0
-            for r, s, n, w in entries:
-                for j in w:
-                    got[(r, s + j)] = logits[row]
-                    row += 1
-            assert row == logits.shape[0]
-        check(got, oracles[dtype], dtype)
-        assert rep.manager.num_available_blocks() == rep.manager.num_blocks
+    """Eight or nine different requests on a pool that holds the first four (each rounded up to pages of
+    64): the later ones run on pages that earlier ones have written and given back, while other
+    requests are in the middle of theirs. A stale page holds another request's keys, so a write
+    that was skipped, or a page number that went to the wrong request, shows in the logits."""
+    name, folder, config, _, _ = case
+    prompts = [prompt(300 + i, n, config.vocab_size) for i, n in enumerate(MIXED_LENGTHS[name])]
+    plain = PlainLlama(folder, torch.float64, weights_as=torch.bfloat16 if dtype == "bfloat16" else None)
+    oracle = [plain.logits(p) for p in prompts]
+    pool = sum(-(-len(p) // 64) for p in prompts[:4])
+    rep = replayer(folder, dtype, 64 * pool)
+    assert rep.manager.num_blocks == pool
+    got, given_back, taken_again_beside = {}, set(), 0
+    for entries, end in mixed_schedule(prompts, pool):
+        batch = [{"id": f"q{r}", "tokens": prompts[r][s:s + n], "want": w} for r, s, n, w in entries]
+        held = {r: set(rep.manager.block_table(rep.ids[f"q{r}"])) for r, s, _, _ in entries if s}
+        logits = rep.step(batch, [])
+        for r, s, n, w in entries:
+            if s == 0 and set(rep.manager.block_table(rep.ids[f"q{r}"])) & given_back and len(held) >= 2:
+                taken_again_beside += 1
+        row = 0
+        for r, s, n, w in entries:
+            for j in w:
+                got[(r, s + j)] = logits[row]
+                row += 1
+        assert row == logits.shape[0]
+        for r in end:
+            given_back |= set(rep.manager.block_table(rep.ids[f"q{r}"]))
+        rep.step([], [f"q{r}" for r in end])
+    assert taken_again_beside >= 2, "requests started on used pages while two others were live"
+    check(got, oracle, dtype)
+    assert rep.manager.num_available_blocks() == rep.manager.num_blocks
 
 
 def test_float32_logits_do_not_depend_on_the_cut(case):
