@@ -138,3 +138,45 @@ def test_a_recorded_batch_of_forty_at_the_1b_sizes(tmp_path):
         logits = plain.logits(p + tokens[:-1])[len(p) - 1:]
         gaps = logits.max(-1).values - logits[torch.arange(len(tokens)), torch.tensor(tokens)]
         assert float(gaps.max()) <= 0.05 * float(logits.std()), f"a token far from the best: gaps {gaps.tolist()}"
+
+
+@pytest.fixture(scope="module")
+def folder_1b(tmp_path_factory):
+    folder = str(tmp_path_factory.mktemp("regime_1B"))
+    write_random_model(folder, CONFIG, 9, torch.bfloat16)
+    return folder
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_benchmarks_own_regime_against_the_plain_model(folder_1b, dtype):
+    """What bench.py times, checked: eight requests of 2,048 tokens (eight full pages of 256 each)
+    decode sixteen tokens through `LLM.generate`, set up as bench.py sets its engine up: decode steps
+    replayed from a graph whose block tables are nine pages wide (the bucket above 2,048 positions),
+    the host one step ahead, the split-key attention kernel over 2,049 to 2,064 keys that cross into
+    a ninth page. Every token against the plain model run whole over the same history: in float32
+    it is the plain model's choice; in bfloat16 it lies within a small gap of it."""
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+    batch, length, decoded, page = 8, 2048, 16, 256
+    prompts = [prompt(900 + i, length, CONFIG.vocab_size) for i in range(batch)]
+    sc = SchedulerConfig(max_model_len=4096, max_num_seqs=batch, max_num_batched_tokens=length + batch, watermark=0.0)
+    llm = LLM(folder_1b, sc, CacheConfig(block_size=page, caching=False), dtype=torch.float32 if dtype == "float32" else torch.bfloat16,
+              num_blocks=batch * (4096 // page) + 2, seed=0)
+    outs = [c.token_ids[0] for c in llm.generate(prompts, SamplingParams(max_tokens=decoded, temperature=0.0, ignore_eos=True))]
+    assert (batch, 9) in llm.runner.graphs.graphs, "the decode steps ran as the graph of eight requests over nine pages"
+    # (a prompt a step is admitted under the token budget; once the last one is in, all eight decode together)
+    assert sum(s.num_tokens == s.num_seqs == batch for s in llm.steps) >= 5
+    plain = PlainLlama(folder_1b, torch.float64)
+    head = plain.w["model.embed_tokens.weight"]
+    for p, tokens in list(zip(prompts, outs))[:batch if dtype == "float32" else 4]:
+        logits = plain.hidden_states(p + tokens[:-1])[length - 1:] @ head.T
+        best = logits.max(-1)
+        if dtype == "float32":
+            close = torch.topk(logits, 2).values
+            for i, tok in enumerate(tokens):
+                assert tok == int(best.indices[i]) or float(close[i, 0] - close[i, 1]) < 2e-4, \
+                    f"token {i}: {tok}, the plain model chooses {int(best.indices[i])}"
+        else:
+            gaps = best.values - logits[torch.arange(decoded), torch.tensor(tokens)]
+            assert float(gaps.max()) <= 0.05 * float(logits.std()), f"a token far from the best: gaps {gaps.tolist()}"

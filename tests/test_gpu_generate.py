@@ -174,6 +174,30 @@ def test_drawn_tokens_of_a_workload_with_prefix_hits_forks_and_portions_against_
     assert two[0].output_token_ids != two[1].output_token_ids
 
 
+def test_recording_a_step_while_a_dropped_engine_awaits_collection(folder_a):
+    """An engine that holds recorded steps is dropped inside a reference cycle, so that only the
+    collector can free it; a second engine then records its own steps with the collector set to run
+    at every opportunity. The recording keeps the collector off (a graph destroyed inside a recording
+    aborted the process once), and the second engine's tokens are the first one's."""
+    import gc
+    first = engine(folder_a)
+    expected = [r.token_ids for r in first.generate(PROMPTS[:3], greedy(5))]
+    assert first.runner.graphs.graphs, "the first engine holds recorded steps"
+    first.myself = first
+    gc.disable()                        # (the cycle stays pending while the second engine is built)
+    old = gc.get_threshold()
+    try:
+        del first
+        second = engine(folder_a)
+        gc.set_threshold(1, 1, 1)
+        gc.enable()
+        got = [r.token_ids for r in second.generate(PROMPTS[:3], greedy(5))]
+    finally:
+        gc.set_threshold(*old)
+        gc.enable()
+    assert got == expected and second.runner.graphs.graphs
+
+
 def test_the_end_token_stops_generation(folder_a):
     plain = PlainLlama(folder_a, torch.float64)
     full = plain.greedy(PROMPTS[0], 12)

@@ -427,6 +427,29 @@ def test_library_product_called_directly(m, n, k):
         hip().gemm_library(ad.t()[:k].t()[:, ::2], wd[:, ::2])      # elements of a row must be adjacent
 
 
+@pytest.mark.parametrize("n,k", [(128256, 2048), (1000, 160), (32000, 4096)])
+def test_float32_logits_are_the_32_bit_sums_whatever_the_number_of_rows(n, k):
+    """The head's product for one row, for 16 (the weight-streaming kernel), and for 17, 40 and 300
+    (the library, which is asked for its 32-bit sums instead of a bfloat16 result widened afterwards):
+    a row's logits agree to 32-bit rounding whichever kernel its step takes, so the choice between two
+    close tokens does not depend on how many requests share the step. A result that had passed through
+    bfloat16 would be off by up to 2^-9 of its size."""
+    from tinyserve_llm_amd.parts.linear import linear
+    g = gen(n + k)
+    a, w = torch.randn(300, k, generator=g).bfloat16(), (torch.randn(n, k, generator=g) * 0.05).bfloat16()
+    want = (a[:1].double() @ w.double().T)[0]
+    ad, wd = a.to(dev()), w.to(dev())
+    scale = float(want.abs().max())
+    for rows in (1, 16, 17, 40, 300):
+        out = linear(ad[:rows].contiguous(), wd, out_dtype=torch.float32)
+        assert out.dtype == torch.float32 and out.shape == (rows, n)
+        err = float((out[0].double().cpu() - want).abs().max())
+        assert err <= 2e-5 * scale, f"{rows} rows: error {err:.3e} of {scale:.3f}"
+    if hip().tiled_takes(ad, wd):
+        out = hip().gemm_tiled(ad[:40].contiguous(), wd, out_dtype=torch.float32)     # the engine's own product for many rows
+        assert out.dtype == torch.float32 and float((out[0].double().cpu() - want).abs().max()) <= 2e-5 * scale
+
+
 @pytest.mark.parametrize("m,n,k", [(300, 384, 64), (2056, 16384, 2048), (100, 1000, 192), (257, 132, 3072), (515, 128256, 128),
                                    (2048, 2048, 8192), (33, 8, 320), (1, 4, 64)])
 def test_tiled_product(m, n, k):

@@ -3,7 +3,7 @@
 No torch headers and no ninja are involved: every kernel has an `extern "C"` launcher that takes
 raw device pointers and a stream, and Python calls them through ctypes. The library is written next
 to the sources; if that folder is read-only, to a per-user folder under the system's temporary
-directory. A sidecar file records a hash of the sources and flags so that a stale library is
+directory (made with mode 0700, and used only if it is this user's own and closed to everyone else). A sidecar file records a hash of the sources and flags so that a stale library is
 rebuilt and a current one is loaded as it is.
 """
 
@@ -58,9 +58,32 @@ def _hipcc() -> str:
                        "the HIP kernels cannot be built and there is no other path")
 
 
-def _writable(folder: str) -> bool:
+def _private(folder: str) -> bool:
+    """Whether a folder outside the package is this user's alone: a real directory (no link) that
+    the user owns and nobody else may write to. The temporary directory is shared, its per-user
+    folder has a name anyone can guess, and a library found there is loaded into the process: a
+    folder that someone else made, or may write into, is not used."""
     try:
-        os.makedirs(folder, exist_ok=True)
+        st = os.lstat(folder)
+    except OSError:
+        return False
+    import stat
+    return stat.S_ISDIR(st.st_mode) and st.st_uid == os.getuid() and not st.st_mode & 0o022
+
+
+def _usable(folder: str, create: bool) -> bool:
+    """Whether the library may be read from (and, with `create`, written to) `folder`."""
+    if folder != HERE:
+        if create and not os.path.lexists(folder):
+            try:
+                os.mkdir(folder, 0o700)
+            except OSError:
+                return False
+        if not _private(folder):
+            return False
+    if not create:
+        return os.path.isdir(folder)
+    try:
         probe = os.path.join(folder, f".probe_{os.getpid()}")
         with open(probe, "w"):
             pass
@@ -78,6 +101,8 @@ def find_current() -> str | None:
     """Path of a built library whose recorded hash matches the sources, or None."""
     want = source_hash()
     for folder in candidate_dirs():
+        if not _usable(folder, create=False):
+            continue
         lib, stamp = os.path.join(folder, LIB_NAME), os.path.join(folder, LIB_NAME + ".hash")
         try:
             with open(stamp) as f:
@@ -95,9 +120,10 @@ def build(verbose: bool = True, force: bool = True) -> str:
         if lib:
             return lib
     hipcc = _hipcc()
-    out_dir = next((d for d in candidate_dirs() if _writable(d)), None)
+    out_dir = next((d for d in candidate_dirs() if _usable(d, create=True)), None)
     if out_dir is None:
-        raise RuntimeError(f"no writable folder for the kernel library among {candidate_dirs()}")
+        raise RuntimeError(f"no folder for the kernel library among {candidate_dirs()}: each is read-only, or is not "
+                           "this user's own (owned by someone else, or writable by others)")
     obj_dir = os.path.join(out_dir, "_build")
     os.makedirs(obj_dir, exist_ok=True)
     env = dict(os.environ)

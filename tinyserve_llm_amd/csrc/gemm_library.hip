@@ -1,4 +1,5 @@
-// y[M, N] = x[M, K] · W[N, K]^T in bfloat16 with 32-bit accumulation for many rows of x, through the
+// y[M, N] = x[M, K] · W[N, K]^T in bfloat16 with 32-bit accumulation (y bfloat16, or the 32-bit sums
+// themselves) for many rows of x, through the
 // vendor's matrix library (hipBLASLt), called directly: the descriptors and the algorithm the
 // library's heuristic picks for a shape are made once and kept, so that a call costs little more
 // than the launch (a framework's general matmul asks the heuristic again at every call, which is
@@ -57,7 +58,7 @@ struct LtPlan {
 struct LtDevice {
   hipblasLtHandle_t handle = nullptr;
   void* workspace = nullptr;
-  std::map<std::tuple<int, int, int, int64_t, int64_t, int64_t>, LtPlan> plans;
+  std::map<std::tuple<int, int, int, int64_t, int64_t, int64_t, int>, LtPlan> plans;   // (..., 32-bit output or not)
 };
 
 std::mutex lt_mutex;
@@ -89,13 +90,13 @@ bool lt_first(LtDevice& dev, hipblasLtMatmulDesc_t desc, hipblasLtMatrixLayout_t
 
 // What the heuristic picks for `rows` rows of the plan's shape, if the library supports it for the
 // plan's own row count too (within the workspace, and without one where the shape may be recorded).
-void lt_borrow(LtDevice& dev, LtPlan& plan, int M, int N, int K, int64_t ldx, int64_t ldy, int rows) {
+void lt_borrow(LtDevice& dev, LtPlan& plan, int M, int N, int K, int64_t ldx, int64_t ldy, int rows, hipDataType out) {
   hipblasLtMatrixLayout_t b = nullptr, d = nullptr;
   hipblasLtMatmulAlgo_t algo;
   size_t workspace = 0;
   const float one = 1.0f, zero = 0.0f;
   if (hipblasLtMatrixLayoutCreate(&b, HIP_R_16BF, K, rows, ldx) == HIPBLAS_STATUS_SUCCESS &&
-      hipblasLtMatrixLayoutCreate(&d, HIP_R_16BF, N, rows, ldy) == HIPBLAS_STATUS_SUCCESS &&
+      hipblasLtMatrixLayoutCreate(&d, out, N, rows, ldy) == HIPBLAS_STATUS_SUCCESS &&
       lt_first(dev, plan.desc, plan.a, b, d, M, &algo, &workspace) &&
       hipblaslt_ext::matmulIsAlgoSupported(dev.handle, plan.desc, &one, plan.a, plan.b, &zero, plan.d, plan.d, algo,
                                            workspace) == HIPBLAS_STATUS_SUCCESS &&
@@ -110,8 +111,9 @@ void lt_borrow(LtDevice& dev, LtPlan& plan, int M, int N, int K, int64_t ldx, in
 
 // The plan for a shape on the current device; made (and the library asked for its best algorithm)
 // the first time the shape is met. Returns null if the library has nothing for it.
-LtPlan* lt_plan(LtDevice& dev, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldy) {
-  const auto key = std::make_tuple(M, N, K, ldx, ldw, ldy);
+LtPlan* lt_plan(LtDevice& dev, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldy, int out_f32) {
+  const auto key = std::make_tuple(M, N, K, ldx, ldw, ldy, out_f32);
+  const hipDataType out = out_f32 ? HIP_R_32F : HIP_R_16BF;
   auto it = dev.plans.find(key);
   if (it != dev.plans.end()) return it->second.desc ? &it->second : nullptr;
   if (dev.plans.size() >= LT_MAX_PLANS) {   // start over rather than grow without bound
@@ -131,12 +133,12 @@ LtPlan* lt_plan(LtDevice& dev, int M, int N, int K, int64_t ldx, int64_t ldw, in
   ok = ok && hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &tb, sizeof(tb)) == HIPBLAS_STATUS_SUCCESS;
   ok = ok && hipblasLtMatrixLayoutCreate(&plan.a, HIP_R_16BF, K, N, ldw) == HIPBLAS_STATUS_SUCCESS;
   ok = ok && hipblasLtMatrixLayoutCreate(&plan.b, HIP_R_16BF, K, M, ldx) == HIPBLAS_STATUS_SUCCESS;
-  ok = ok && hipblasLtMatrixLayoutCreate(&plan.d, HIP_R_16BF, N, M, ldy) == HIPBLAS_STATUS_SUCCESS;
+  ok = ok && hipblasLtMatrixLayoutCreate(&plan.d, out, N, M, ldy) == HIPBLAS_STATUS_SUCCESS;
   ok = ok && lt_first(dev, plan.desc, plan.a, plan.b, plan.d, M, &plan.algo, &plan.workspace);
   if (ok) {
     if (M > LT_TUNE_MAX_ROWS && M % LT_BORROW_ROWS) {
-      lt_borrow(dev, plan, M, N, K, ldx, ldy, M / LT_BORROW_ROWS * LT_BORROW_ROWS);
-      lt_borrow(dev, plan, M, N, K, ldx, ldy, (M / LT_BORROW_ROWS + 1) * LT_BORROW_ROWS);
+      lt_borrow(dev, plan, M, N, K, ldx, ldy, M / LT_BORROW_ROWS * LT_BORROW_ROWS, out);
+      lt_borrow(dev, plan, M, N, K, ldx, ldy, (M / LT_BORROW_ROWS + 1) * LT_BORROW_ROWS, out);
     }
   } else {
     if (plan.a) hipblasLtMatrixLayoutDestroy(plan.a);
@@ -260,20 +262,21 @@ extern "C" int ts_gemm_library_init() {
   return lt_device() ? TS_OK : TS_LAUNCH_FAILED;
 }
 
-// y, x, w bfloat16; rows of x, w and y are ldx, ldw, ldy elements apart (each at least the row's
+// x, w bfloat16; y bfloat16, or float32 if out_f32 (the 32-bit sums as they are, not rounded to
+// bfloat16 on the way); rows of x, w and y are ldx, ldw, ldy elements apart (each at least the row's
 // length). The stream may be one that is being captured into a graph (after ts_gemm_library_init).
 // tune != 0: a shape of 9 to 256 rows that has not been tuned yet is tuned first (see above),
 // unless the stream is being captured; `flush` is device memory of `flush_bytes` that may be
 // overwritten (more than the caches hold), or null to time with warm caches.
 extern "C" int ts_gemm_library_bf16(void* y, const void* x, const void* w, int M, int N, int K, int64_t ldx,
-                                    int64_t ldw, int64_t ldy, int tune, void* flush, size_t flush_bytes,
+                                    int64_t ldw, int64_t ldy, int out_f32, int tune, void* flush, size_t flush_bytes,
                                     hipStream_t stream) {
   if (M <= 0 || N <= 0) return TS_OK;
   if (K <= 0 || ldx < K || ldw < K || ldy < N || !y || !x || !w) return TS_BAD_SHAPE;
   std::lock_guard<std::mutex> guard(lt_mutex);
   LtDevice* dev = lt_device();
   if (!dev) return TS_LAUNCH_FAILED;
-  LtPlan* plan = lt_plan(*dev, M, N, K, ldx, ldw, ldy);
+  LtPlan* plan = lt_plan(*dev, M, N, K, ldx, ldw, ldy, out_f32 != 0);
   if (!plan) return TS_BAD_SHAPE;
   if (tune && !plan->tuned && M >= LT_TUNE_MIN_ROWS && M <= LT_TUNE_MAX_ROWS) {
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;

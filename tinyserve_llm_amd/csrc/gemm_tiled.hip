@@ -27,9 +27,9 @@ static __device__ __forceinline__ float4_t mfma32v(u32x4_t a, u32x4_t b, float4_
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
 }
 
-template <int BM, int BN, int WM, int WN, bool GLU>
+template <int BM, int BN, int WM, int WN, bool GLU, bool OUT32>
 __global__ __launch_bounds__(WM * WN * TS_WAVE) void gemm_tiled_kernel(
-    bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, int M, int N, int K,
+    void* __restrict__ yv, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, int M, int N, int K,
     int64_t ldx, int64_t ldw, int64_t ldy, int row_tiles, int col_tiles, int per_die) {
   constexpr int THREADS = WM * WN * TS_WAVE;
   constexpr int FX = BM / 16 * 2, FW = BN / 16 * 2;       // fragments (a kilobyte each) of a k-step of 64
@@ -37,6 +37,8 @@ __global__ __launch_bounds__(WM * WN * TS_WAVE) void gemm_tiled_kernel(
   constexpr int LX = FX * 64 / THREADS, LW = FW * 64 / THREADS;
   static_assert(FX * 64 % THREADS == 0 && FW * 64 % THREADS == 0, "every thread fetches the same number of pieces");
   static_assert(!GLU || WN == 1, "a gate value and its up value must meet in one wave");
+  static_assert(!(GLU && OUT32), "the gated result is bfloat16");
+  bf16_t* __restrict__ y = (bf16_t*)yv;
   __shared__ u32x4_t lds[2][(FX + FW) * 64];
   // consecutive workgroups go to different dies: a die takes a contiguous run of tiles, column tile
   // by column tile, so that the tiles sharing a slice of W run on the die whose L2 holds it
@@ -154,36 +156,42 @@ __global__ __launch_bounds__(WM * WN * TS_WAVE) void gemm_tiled_kernel(
         const int n = n0 + (wn * TN + j) * 16 + 4 * g;
         if (n >= N) continue;
         const float4_t a = acc[j][i];
-        *(uint2*)(y + (int64_t)m * ldy + n) = make_uint2(pack_bf16(a[0], a[1]), pack_bf16(a[2], a[3]));
+        if constexpr (OUT32) *(float4_t*)((float*)yv + (int64_t)m * ldy + n) = a;      // the 32-bit sums as they are
+        else *(uint2*)(y + (int64_t)m * ldy + n) = make_uint2(pack_bf16(a[0], a[1]), pack_bf16(a[2], a[3]));
       }
     }
   }
 }
 
-template <int BM, int BN, int WM, int WN, bool GLU>
+template <int BM, int BN, int WM, int WN, bool GLU, bool OUT32 = false>
 static int launch_tiled(void* y, const void* x, const void* w, int M, int N, int K, int64_t ldx, int64_t ldw,
                         int64_t ldy, hipStream_t stream) {
   const int row_tiles = (M + BM - 1) / BM, col_tiles = (N + BN - 1) / BN;
   const int per_die = (row_tiles * col_tiles + 7) / 8;
-  gemm_tiled_kernel<BM, BN, WM, WN, GLU><<<8 * per_die, WM * WN * TS_WAVE, 0, stream>>>(
-      (bf16_t*)y, (const bf16_t*)x, (const bf16_t*)w, M, N, K, ldx, ldw, ldy, row_tiles, col_tiles, per_die);
+  gemm_tiled_kernel<BM, BN, WM, WN, GLU, OUT32><<<8 * per_die, WM * WN * TS_WAVE, 0, stream>>>(
+      y, (const bf16_t*)x, (const bf16_t*)w, M, N, K, ldx, ldw, ldy, row_tiles, col_tiles, per_die);
   return ts_check_launch();
 }
 
-// y, x, w bfloat16, 16-byte aligned, rows ldx, ldw, ldy elements apart (multiples of 8; ldy of 4).
-// K a multiple of 64. glu == 0: y [M, N], N a multiple of 4. glu != 0: w holds N / 2 gate rows,
-// then N / 2 up rows, y [M, N / 2] = silu(gate) · up, N a multiple of 8.
+// x, w bfloat16, 16-byte aligned, rows ldx, ldw, ldy elements apart (multiples of 8; ldy of 4).
+// K a multiple of 64. glu == 0: y [M, N], N a multiple of 4, bfloat16, or with out_f32 the 32-bit
+// sums themselves (y float32, 16-byte aligned). glu != 0: w holds N / 2 gate rows, then N / 2 up
+// rows, y [M, N / 2] = silu(gate) · up in bfloat16, N a multiple of 8.
 extern "C" int ts_gemm_tiled_bf16(void* y, const void* x, const void* w, int M, int N, int K, int64_t ldx,
-                                  int64_t ldw, int64_t ldy, int glu, hipStream_t stream) {
+                                  int64_t ldw, int64_t ldy, int glu, int out_f32, hipStream_t stream) {
   if (M <= 0 || N <= 0) return TS_OK;
   if (K <= 0 || K % 64 || N % (glu ? 8 : 4) || ldx < K || ldw < K || ldy < (glu ? N / 2 : N)) return TS_BAD_SHAPE;
   if (ldx % 8 || ldw % 8 || ldy % 4 || !y || !x || !w) return TS_BAD_SHAPE;
-  if ((((uintptr_t)x) | ((uintptr_t)w)) & 15 || ((uintptr_t)y) & 7) return TS_BAD_SHAPE;
+  if ((((uintptr_t)x) | ((uintptr_t)w)) & 15 || ((uintptr_t)y) & (out_f32 ? 15 : 7) || (glu && out_f32)) return TS_BAD_SHAPE;
   // large tiles where they still give every compute unit two workgroups
   const int64_t big = (int64_t)((M + 255) / 256) * ((N + 127) / 128);
   if (glu) {
     if (big >= 512) return launch_tiled<256, 128, 4, 1, true>(y, x, w, M, N, K, ldx, ldw, ldy, stream);
     return launch_tiled<128, 128, 4, 1, true>(y, x, w, M, N, K, ldx, ldw, ldy, stream);
+  }
+  if (out_f32) {
+    if (big >= 512) return launch_tiled<256, 128, 4, 2, false, true>(y, x, w, M, N, K, ldx, ldw, ldy, stream);
+    return launch_tiled<128, 128, 2, 2, false, true>(y, x, w, M, N, K, ldx, ldw, ldy, stream);
   }
   if (big >= 512) return launch_tiled<256, 128, 4, 2, false>(y, x, w, M, N, K, ldx, ldw, ldy, stream);
   return launch_tiled<128, 128, 2, 2, false>(y, x, w, M, N, K, ldx, ldw, ldy, stream);

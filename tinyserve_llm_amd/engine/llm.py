@@ -13,10 +13,9 @@ from typing import Literal
 
 import torch
 
-from tinyserve_llm_amd.cache.manager import CacheStats, KVCacheManager
-from tinyserve_llm_amd.cache.storage import KVStorage, bytes_per_page
-from tinyserve_llm_amd.models.decoder import DecoderModel
+from tinyserve_llm_amd.engine.interface import CacheConfig, CacheStats, build_cache, bytes_per_page
 from tinyserve_llm_amd.engine.loading import as_dtype, load_model, random_model, require_gpu
+from tinyserve_llm_amd.models.decoder import DecoderModel
 from tinyserve_llm_amd.engine.runner import ModelRunner, StepEntry
 from tinyserve_llm_amd.engine.scheduler import (PENDING, RequestOutput, ScheduledSeq, Scheduler, SchedulerConfig,
                                                 SchedulerStats)
@@ -24,13 +23,6 @@ from tinyserve_llm_amd.engine.sequence import SamplingParams
 from tinyserve_llm_amd.sampling.sampler import row_key, sample
 
 logger = logging.getLogger(__name__)
-
-
-@dataclass(frozen=True)
-class CacheConfig:
-    block_size: int = 256
-    caching: bool = True        # False: no prefix reuse; forks still share pages
-    device: str = "cuda"
 
 
 @dataclass
@@ -100,12 +92,11 @@ class LLM:
         if scheduler_config.eos_token_id == -1:
             scheduler_config = replace(scheduler_config, eos_token_id=self._eos_token_id())
         self.seed = 0 if seed is None else seed
-        cache_plan, state_plan = self.model.cache_plan(), self.model.state_plan()
         if num_blocks is None:
             num_blocks = self._size_from_free_memory(scheduler_config, cache_config, gpu_memory_utilization)
-        self.storage = KVStorage(cache_plan, state_plan, num_blocks, cache_config.block_size, self.dtype, self.device,
-                                 num_state_slots=scheduler_config.max_num_seqs)
-        self.manager = KVCacheManager(self.storage, caching=cache_config.caching)
+        self.storage, self.manager = build_cache(self.model, num_blocks, cache_config.block_size, self.dtype, self.device,
+                                                 num_state_slots=scheduler_config.max_num_seqs,
+                                                 caching=cache_config.caching)
         self.scheduler = Scheduler(scheduler_config, self.manager)
         self.runner = ModelRunner(self.model, self.storage, self.manager)
         if decode_graphs:
@@ -129,7 +120,7 @@ class LLM:
                                                         if n.startswith("layers.") and len(p.shape) == 2])
         act = sc.max_num_batched_tokens * widest * 4 * 6 + sc.max_num_seqs * self.model.spec.vocab_size * 4 * 2
         budget = total * utilisation - (total - free) - act
-        per_page = max(1, bytes_per_page(self.model.cache_plan(), cc.block_size, self.dtype))
+        per_page = max(1, bytes_per_page(self.model, cc.block_size, self.dtype))
         pages = int(budget // per_page)
         most_useful = sc.max_num_seqs * (-(-sc.max_model_len // cc.block_size) + 1) + 8
         pages = min(pages, most_useful)

@@ -19,8 +19,7 @@ import sys
 import numpy as np
 import torch
 
-from tinyserve_llm_amd.cache.manager import KVCacheManager
-from tinyserve_llm_amd.cache.storage import KVStorage
+from tinyserve_llm_amd.engine.interface import build_cache
 from tinyserve_llm_amd.engine.loading import as_dtype, load_model
 from tinyserve_llm_amd.engine.runner import ModelRunner, StepEntry
 
@@ -33,10 +32,9 @@ class Replay:
                  page_size: int = REPLAY_PAGE_SIZE) -> None:
         self.model, self.config = load_model(model_dir, dtype, device)
         num_pages = max(1, -(-max_tokens // page_size))
-        self.storage = KVStorage(self.model.cache_plan(), self.model.state_plan(), num_pages, page_size,
-                                 as_dtype(dtype), device, num_state_slots=MAX_LIVE)
         # replay runs exactly the tokens it is given, so nothing is ever taken from a prefix cache
-        self.manager = KVCacheManager(self.storage, caching=False)
+        self.storage, self.manager = build_cache(self.model, num_pages, page_size, as_dtype(dtype), device,
+                                                 num_state_slots=MAX_LIVE, caching=False)
         self.runner = ModelRunner(self.model, self.storage, self.manager)
         self.ids: dict[str, int] = {}
         self.lengths: dict[int, int] = {}

@@ -14,12 +14,11 @@ import gc
 import struct
 import weakref
 from array import array
-from typing import NamedTuple, Protocol, Sequence
+from typing import NamedTuple, Sequence
 
 import torch
 
-from tinyserve_llm_amd.cache.manager import FREED
-from tinyserve_llm_amd.cache.storage import KVStorage
+from tinyserve_llm_amd.engine.interface import StepMemory, TableView
 from tinyserve_llm_amd.models.decoder import DecoderModel
 from tinyserve_llm_amd.parts.base import LayerMemory, StepContext
 
@@ -31,19 +30,12 @@ class StepEntry(NamedTuple):          # (a tuple: a step of hundreds of requests
     want: Sequence[int] = ()          # indices into `tokens` whose logits are wanted
 
 
-class TableView(Protocol):
-    """Read access to the cache manager, valid between reserving a step's slots and committing."""
-
-    def block_table(self, seq_id: int, space: int = 0) -> Sequence[int]: ...
-    def state_slot(self, seq_id: int) -> int: ...
-
-
 class StepError(ValueError):
     pass
 
 
 class ModelRunner:
-    def __init__(self, model: DecoderModel, storage: KVStorage, view: TableView) -> None:
+    def __init__(self, model: DecoderModel, storage: StepMemory, view: TableView) -> None:
         self.model = model
         self.storage = storage
         self.view = view
@@ -144,7 +136,7 @@ class ModelRunner:
                 if len(t) > widths[sp]:
                     raise StepError(f"a block table of {len(t)} pages exceeds the fixed width {widths[sp]}")
                 if self.windows[sp]:
-                    flat.extend(0 if p == FREED else p for p in t)     # pages a window has passed
+                    flat.extend(p if p >= 0 else 0 for p in t)     # (below 0: pages a window has passed)
                 else:
                     flat.extend(t)
                 flat.extend([0] * (widths[sp] - len(t)))
@@ -187,7 +179,7 @@ class ModelRunner:
                 if min(read) < 0 or max(read) >= pages:
                     raise StepError(f"request {e.seq_id}: its pages of space {sp} hold {min(read)}..{max(read)}")
                 if window:
-                    flat.extend(0 if p == FREED else p for p in table)
+                    flat.extend(p if p >= 0 else 0 for p in table)
                 else:
                     flat.extend(table)
                 flat.extend([0] * (width - len(table)))
@@ -379,26 +371,34 @@ class DecodeGraphs:
             t.copy_(kept)
         torch.cuda.synchronize(r.device)
         graph = torch.cuda.CUDAGraph()
-        # No garbage collection while the stream is being captured: an engine that the process has
-        # dropped earlier may still be waiting to be collected, and destroying its graphs is an
-        # operation the capture forbids (the process then aborts in the graph's destructor). The
-        # capture collects what is pending when it is entered.
-        collecting = gc.isenabled()
-        gc.disable()
-        try:
-            with torch.cuda.graph(graph, pool=self.pool):
-                hidden, residual = r.model.forward(ctx, r.memory)
-                logits = r.model.logits(hidden, residual, rows)
-                tokens = hip.sample(logits, draw_temps, draw_keys, self.seed)
-        finally:
-            if collecting:
-                gc.enable()
+
+        def body():
+            hidden, residual = r.model.forward(ctx, r.memory)
+            logits = r.model.logits(hidden, residual, rows)
+            return logits, hip.sample(logits, draw_temps, draw_keys, self.seed)
+
+        logits, tokens = self._record(graph, self.pool, body)
         if self.pool is None:
             self.pool = graph.pool()
         # the drawn tokens travel to the host through two pinned buffers in turn: a step may be
         # started before the tokens of the step before it have been read
         landing = [(torch.empty(size, dtype=torch.int32, pin_memory=True), torch.cuda.Event()) for _ in range(2)]
         return [graph, host_i32, dev_i32, logits, tokens, torch.cuda.Event(), landing, 0]
+
+    @staticmethod
+    def _record(graph, pool, body):
+        """Runs `body` while the current stream is recorded into `graph`, with garbage collection
+        off: an engine that the process has dropped earlier may still be waiting to be collected,
+        and destroying its graphs is an operation that a recording forbids (the process then aborts
+        in the graph's destructor). What is pending is collected after the recording."""
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph, pool=pool):
+                return body()
+        finally:
+            if collecting:
+                gc.enable()
 
     def prepare(self, entries: Sequence[StepEntry], draws=None, feed: Sequence[int] | None = None) -> tuple:
         """The host half of `run`: checks and packs the step. Token ids of entries that `feed`

@@ -56,8 +56,8 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_sample": [p, p, p, p, p, p, u64, i, i, i64, p],
         "ts_sample_static": [p, p, p, p, u64, i, i, i64, p],
         "ts_feed_tokens": [p, p, p, i, i, p],
-        "ts_gemm_library_bf16": [p, p, p, i, i, i, i64, i64, i64, i, p, ctypes.c_size_t, p],
-        "ts_gemm_tiled_bf16": [p, p, p, i, i, i, i64, i64, i64, i, p],
+        "ts_gemm_library_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p, ctypes.c_size_t, p],
+        "ts_gemm_tiled_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_gemm_library_init": [],
         "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, i, i, i, i, p, p, p],
         "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p],
@@ -755,20 +755,25 @@ def tiled_takes(x: torch.Tensor, weight: torch.Tensor, glu: bool = False) -> boo
             and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
 
 
-def gemm_tiled(x: torch.Tensor, weight: torch.Tensor, glu: bool = False) -> torch.Tensor:
+def gemm_tiled(x: torch.Tensor, weight: torch.Tensor, glu: bool = False,
+               out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """bfloat16 x [M, K] · weight [N, K]^T by the LDS-tiled matrix-core kernel; with `glu` the weight
-    holds N / 2 gate rows, then N / 2 up rows, and silu(gate) · up [M, N / 2] comes back."""
+    holds N / 2 gate rows, then N / 2 up rows, and silu(gate) · up [M, N / 2] comes back. The result
+    is bfloat16, or (without `glu`) the 32-bit sums themselves with `out_dtype` float32."""
     _gpu(x, weight)
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
           f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
     _need(tiled_takes(x, weight, glu), "the tiled kernel takes bfloat16 operands with dense, 16-byte aligned rows, a "
           "reduction that is a multiple of 64 and a width that is a multiple of 4 (8 with the gate)")
+    _need(out_dtype == torch.bfloat16 or (out_dtype == torch.float32 and not glu),
+          "the tiled product comes out as bfloat16, or without the gate as float32")
     M, K = x.shape
     N = weight.shape[0]
-    y = torch.empty((M, N // 2 if glu else N), dtype=torch.bfloat16, device=x.device)
+    y = torch.empty((M, N // 2 if glu else N), dtype=out_dtype, device=x.device)
     if M and N:
         _run("gemm_tiled", library().ts_gemm_tiled_bf16(_ptr(y), _ptr(x), _ptr(weight), M, N, K, x.stride(0),
-                                                        weight.stride(0), y.stride(0), int(glu), _stream()))
+                                                        weight.stride(0), y.stride(0), int(glu),
+                                                        int(out_dtype == torch.float32), _stream()))
     return y
 
 
@@ -787,8 +792,12 @@ def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
             and (x.shape[0] <= SKINNY_FUSED_ROWS or weight.numel() <= SKINNY_WIDE_ELEMENTS)
             and x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
         return gemm_skinny(x, weight, out_dtype, packed=packed)[0]
-    y = gemm_tiled(x, weight) if _many_rows == "tiled" and tiled_takes(x, weight) else gemm_library(x, weight)
-    return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
+    # (float32: the 32-bit sums themselves, as the weight-streaming kernel gives them for few rows, so
+    # that a row's logits are rounded the same way whatever the number of rows beside it)
+    _need(out_dtype in (torch.bfloat16, torch.float32), f"bfloat16 products come out as bfloat16 or float32, not {out_dtype}")
+    if _many_rows == "tiled" and tiled_takes(x, weight):
+        return gemm_tiled(x, weight, out_dtype=out_dtype)
+    return gemm_library(x, weight, out_dtype)
 
 
 def gemm_library_init() -> None:
@@ -815,16 +824,19 @@ def library_tuning():
         _library_tuning = None
 
 
-def gemm_library(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+def gemm_library(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """bfloat16 x [M, K] · weight [N, K]^T by the vendor's matrix library, called directly with the
-    algorithm kept for the shape (see gemm_library.hip). Rows may be strided."""
+    algorithm kept for the shape (see gemm_library.hip). Rows may be strided. The result is bfloat16,
+    or the 32-bit sums themselves with `out_dtype` float32."""
     _need(x.stride(1) == 1 and weight.stride(1) == 1, "rows of x and of the weight must be dense")
+    _need(out_dtype in (torch.bfloat16, torch.float32), "the library product comes out as bfloat16 or float32")
     M, K = x.shape
     N = weight.shape[0]
-    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
     if M and N:
         sweep = _library_tuning
         _run("gemm_library", library().ts_gemm_library_bf16(
-            _ptr(y), _ptr(x), _ptr(weight), M, N, K, x.stride(0), weight.stride(0), N, int(sweep is not None),
+            _ptr(y), _ptr(x), _ptr(weight), M, N, K, x.stride(0), weight.stride(0), N, int(out_dtype == torch.float32),
+            int(sweep is not None),
             _ptr(sweep), 0 if sweep is None else sweep.numel(), _stream()))
     return y
