@@ -10,6 +10,7 @@ import random
 import pytest
 
 from tinyserve_llm_amd.cache.manager import FREED, KVCacheManager, SpaceSpec
+from tinyserve_llm_amd.cache.prefix_index import TOP
 
 B = 4
 
@@ -87,30 +88,42 @@ def check_invariants(m):
             for page in table:
                 if page != FREED:
                     holders[page] += 1
-        assert holders == space.refs, "reference counts differ from the holders"
-        tree = space.tree
-        free = {b for b in range(space.num_pages) if space.refs[b] == 0}
-        assert sorted(space.free) == sorted(b for b in free if b not in tree.nodes), "a page is lost or free twice"
-        assert len(set(space.free)) == len(space.free)
-        assert space.free_cached == sum(1 for b in free if b in tree.nodes)
+        assert holders == space.holders, "the counts of holders differ from the tables"
+        index = space.index
+        unheld = {b for b in range(space.num_pages) if space.holders[b] == 0}
+        assert sorted(space.idle) == sorted(b for b in unheld if b not in index), "a page is lost or idle twice"
+        assert len(set(space.idle)) == len(space.idle)
+        assert space.kept == sum(1 for b in unheld if b in index) and set(space.released_at) == {b for b in unheld if b in index}
+        # every kept page that nothing follows stands in the queue under the moment of its release
+        queued = set(space._queue)
+        for b in space.released_at:
+            if index.is_leaf(b):
+                assert (space.released_at[b], b) in queued, "a kept page could never be evicted"
         if not m.caching or sp:
-            assert not tree.nodes
-        for b, node in tree.nodes.items():
-            assert node.block_id == b
-            assert m.storage.slots[sp][b][:len(node.tokens)] == list(node.tokens)
-            assert node.parent.children[node.tokens] is node
-            if len(node.tokens) < B:
-                assert not node.children
-            if space.refs[b] and node.parent is not tree.root:
-                assert space.refs[node.parent.block_id], "a held page's parent is held"
-            depth, pages = node.parent.trie.longest_match(node.tokens)
-            assert depth == len(node.tokens) and node in pages
+            assert len(index) == 0
+        for b in index:
+            tokens, before = index.tokens(b), index.parent(b)
+            assert m.storage.slots[sp][b][:len(tokens)] == list(tokens)
+            if len(tokens) < B:
+                assert index.is_leaf(b)
+            if before != TOP:
+                assert before in index and len(index.tokens(before)) == B and not index.is_leaf(before)
+                if space.holders[b]:
+                    assert space.holders[before], "the page before a held page is held"
+            # found again by its own tokens, after the pages before it
+            path, at = [], b
+            while at != TOP:
+                path.append(at)
+                at = index.parent(at)
+            run = [t for page in reversed(path) for t in index.tokens(page)]
+            assert index.lookup(run + [0]).pages == list(reversed(path))
+        assert sum(index.is_leaf(b) for b in index) <= len(index)
     if m.caching:
         for s in m.seqs.values():
             for i in range(s.committed // B):
-                node = m.tree.nodes[s.block_table[i]]
-                assert node.tokens == tuple(s.token_ids[i * B:(i + 1) * B])
-                assert node.parent is (m.tree.nodes[s.block_table[i - 1]] if i else m.tree.root)
+                page = s.block_table[i]
+                assert m.index.tokens(page) == tuple(s.token_ids[i * B:(i + 1) * B])
+                assert m.index.parent(page) == (s.block_table[i - 1] if i else TOP)
     used = [s.state_slot for s in m.seqs.values()]
     assert len(set(used)) == len(used) and not set(used) & set(m.free_state_slots)
     assert sorted(used + m.free_state_slots) == list(range(m.storage.num_state_slots)), "a state slot is lost"
@@ -184,7 +197,7 @@ def test_free_copy_source_may_be_evicted_once_the_copy_is_made():
     cost = m.calculate_admission_cost(prompt)
     assert (cost.blocks_needed, cost.prefill_tokens) == (2, 4)
     assert list(m.allocate(2, prompt)) == [1, 0]
-    assert m.storage.copies[-1] == (0, 1, 2) and 0 not in m.tree.nodes
+    assert m.storage.copies[-1] == (0, 1, 2) and 0 not in m.index
 
 
 def test_copy_source_cannot_be_its_own_destination():
@@ -204,8 +217,8 @@ def test_refused_admission_changes_nothing():
     sp = m.spaces[0]
 
     def snapshot():
-        return (list(sp.refs), list(sp.free), sp.free_cached, sp.clock, list(m.free_state_slots),
-                {b: (n.tokens, n.last_used) for b, n in m.tree.nodes.items()}, set(m.seqs))
+        return (list(sp.holders), list(sp.idle), sp.kept, dict(sp.released_at), sorted(sp._queue), list(m.free_state_slots),
+                {b: (m.index.tokens(b), m.index.parent(b)) for b in m.index}, set(m.seqs))
 
     before = snapshot()
     assert m.allocate(9, list(range(11))) is None
@@ -219,7 +232,7 @@ def test_matched_pages_are_held_before_a_page_is_taken():
     prefill(m, 2, [7, 7])
     m.release(2)
     table = list(m.allocate(3, [1, 2, 3, 4, 6, 6, 6]))
-    assert table[0] == 0 and 0 in m.tree.nodes
+    assert table[0] == 0 and 0 in m.index
     forward(m, 3)
     m.commit(3, 3)
     check_invariants(m)
@@ -248,16 +261,18 @@ def test_unpublished_pages_first_then_the_least_recently_freed_leaf():
     m = make(4)
     sp = m.spaces[0]
     b0, b1, b2, b3 = (sp.take() for _ in range(4))
-    p0 = m.tree.publish(m.tree.root, b0, [1, 2, 3, 4])
-    p1 = m.tree.publish(p0, b1, [5, 6])
-    p2 = m.tree.publish(m.tree.root, b2, [9, 9, 9, 9])
+    m.index.add(TOP, b0, [1, 2, 3, 4])
+    m.index.add(b0, b1, [5, 6])
+    m.index.add(TOP, b2, [9, 9, 9, 9])
     for b in (b3, b2, b0, b1):
         sp.drop(b)
-    assert sp.free == [3] and sp.free_cached == 3
-    assert (p2.last_used, p0.last_used, p1.last_used) == (1, 2, 3)
+    assert sp.idle == [3] and sp.kept == 3
+    assert (sp.released_at[b2], sp.released_at[b0], sp.released_at[b1]) == (1, 2, 3)
     assert sp.take() == 3
-    assert sp.take() == 2          # p0 is older but has a child
-    assert 2 not in m.tree.nodes and sp.free_cached == 2
+    assert sp.take() == 2          # page 0 was released before page 1, but page 1 follows it
+    assert 2 not in m.index and sp.kept == 2
+    assert sp.take() == 1 and sp.take() == 0, "once nothing follows it, a page's turn comes by its own age"
+    assert sp.available() == 0 and len(m.index) == 0
 
 
 def test_free_pages_are_not_held_or_dropped_behind_the_pool():
@@ -317,7 +332,7 @@ def test_prompt_in_portions_equals_prompt_at_once():
     for a, b in ((5, 6), (6, 15), (15, 23)):
         step(cut, 1, prompt[a:b])
     assert cut.seqs[1].block_table == whole.seqs[1].block_table and cut.seqs[1].token_ids == prompt
-    assert set(cut.tree.nodes) == set(whole.tree.nodes)
+    assert set(cut.index) == set(whole.index)
     check_invariants(cut)
 
 
@@ -369,10 +384,10 @@ def test_fork_copies_the_state_slot():
 def test_commit_publishes_full_pages_only():
     m = make()
     prefill(m, 1, list(range(10)))
-    assert set(m.tree.nodes) == {0, 1}
+    assert set(m.index) == {0, 1}
     step(m, 1, [10])
     step(m, 1, [11])
-    assert m.tree.nodes[2].parent is m.tree.nodes[1]
+    assert m.index.parent(2) == 1
     check_invariants(m)
 
 
@@ -425,7 +440,7 @@ def test_release_stamps_deeper_pages_as_older():
     m = make()
     prefill(m, 1, list(range(10)))
     m.release(1)
-    stamps = [m.tree.nodes[b].last_used for b in (0, 1, 2)]
+    stamps = [m.spaces[0].released_at[b] for b in (0, 1, 2)]
     assert stamps == sorted(stamps, reverse=True)
     check_invariants(m)
 
@@ -434,7 +449,7 @@ def test_caching_off_publishes_nothing_but_forks_still_share():
     m = make(caching=False)
     prefill(m, 1, list(range(10)))
     m.fork(1, 2)
-    assert m.ref_counts[:3] == [2, 2, 2] and not m.tree.nodes
+    assert m.ref_counts[:3] == [2, 2, 2] and len(m.index) == 0
     m.release(1)
     m.release(2)
     assert m.num_available_blocks() == 12 and m.calculate_admission_cost(list(range(10))).prefill_tokens == 10

@@ -615,6 +615,19 @@ def test_sampler_draw_is_the_exponential_race_and_ignores_the_row_order():
     assert shuffled == [got[i] for i in perm]
 
 
+def test_several_draws_may_read_one_row_of_logits():
+    """The n samples of a prompt are drawn from the one row its last position gave: the draws name
+    their rows, and the result is what separate copies of the rows would give."""
+    from tinyserve_llm_amd.sampling.sampler import sample
+    logits = (torch.randn(4, 700, generator=gen(31)) * 0.5).to(dev())        # flat enough for two draws of a row to differ
+    rows, temps, keys = [2, 2, 2, 0, 3, 3], [0.8, 0.8, 0.0, 1.1, 0.6, 0.6], [11, 12, 13, 14, 15, 15]
+    got = sample(logits, temps, keys, seed=5, rows=rows).tolist()
+    want = sample(logits[torch.tensor(rows)].contiguous(), temps, keys, seed=5).tolist()
+    assert got == want and got[2] == int(logits[2].argmax()) and got[4] == got[5] and got[0] != got[1]
+    with pytest.raises(ValueError, match="rows"):
+        sample(logits, temps, keys, seed=5, rows=[0, 1, 2, 3, 4, 0])
+
+
 @pytest.mark.parametrize("nh,nkv,hd,K,M,page", [(32, 8, 64, 2048, 8, 64), (6, 2, 96, 768, 5, 16), (4, 4, 128, 256, 16, 8),
                                                  (3, 1, 32, 1280, 1, 32), (24, 8, 128, 3072, 8, 64), (8, 2, 128, 4096, 3, 32)])
 @pytest.mark.parametrize("norm", [False, True])

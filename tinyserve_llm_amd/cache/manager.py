@@ -3,7 +3,7 @@ pages still hold reusable prefixes. Host-side bookkeeping only; the one device o
 issues is a copy of a page's leading slots (tinyserve_llm/kvcache/manager.py:45-328).
 
 What is kept from the reference: reference counts, block tables per request, token-granular
-prefix reuse through the page tree, copy-on-write of a shared tail page, publish/grow/dedupe at
+prefix reuse through the prefix index, copy-on-write of a shared tail page, publish/grow/dedupe at
 commit, LRU eviction of free leaf pages, forks that share every page.
 
 What is added:
@@ -21,10 +21,11 @@ What is added:
 
 from __future__ import annotations
 
+import heapq
 from dataclasses import dataclass, field, replace
 from typing import Protocol, Sequence
 
-from tinyserve_llm_amd.cache.page_tree import Match, PageNode, PageTree
+from tinyserve_llm_amd.cache.prefix_index import TOP, Hit, PrefixIndex
 
 FREED = -1   # block-table entry of a page that a window has passed and that was given back
 
@@ -85,55 +86,78 @@ class CacheStats:
 
 
 class PageSpace:
-    """Reference counts, the free list and (for space 0) the prefix tree of one set of page ids."""
+    """The page ids of one space and who has them. At any moment a page is in exactly one state:
+
+      idle   nobody holds it and the prefix index does not know it: it lies on the `idle` stack
+      kept   nobody holds it, but the index knows the tokens it holds: a later prompt may take it
+             over, and once no indexed page follows it, it stands in the queue for eviction,
+             oldest release first
+      held   `holders[page]` requests have it in their tables (indexed or not)
+
+    `take` hands out an idle page while there is one and evicts from the queue otherwise, so
+    `available()` = idle + kept is what admission may count on. The queue is a heap of (moment of
+    release, page) for kept pages that nothing follows; entries are not removed when a page is
+    taken over or gets a follower, they are recognised as stale when they come up (the reference
+    finds its victim by a scan over all cached pages, tinyserve_llm/kvcache/manager.py:85-100)."""
 
     def __init__(self, spec: SpaceSpec, page_size: int) -> None:
         self.num_pages = spec.num_pages
         self.window = spec.window
-        self.refs = [0] * spec.num_pages
-        self.free = list(range(spec.num_pages - 1, -1, -1))   # pop() hands out page 0 first
-        self.tree = PageTree(page_size)                        # stays empty unless pages are published
-        self.free_cached = 0                                   # published pages nobody holds
-        self.clock = 0
+        self.holders = [0] * spec.num_pages
+        self.idle = list(range(spec.num_pages - 1, -1, -1))    # pop() hands out page 0 first
+        self.index = PrefixIndex(page_size)                    # stays empty unless pages are published
+        self.kept = 0
+        self.released_at: dict[int, int] = {}                  # kept page -> the moment its last holder let go
+        self._queue: list[tuple[int, int]] = []
+        self._moment = 0
         self.evictions = 0
 
     def available(self) -> int:
-        return len(self.free) + self.free_cached
+        return len(self.idle) + self.kept
 
     def take(self) -> int:
-        """A page with one holder: a never-published free one if there is one, else the least
-        recently released free leaf of the tree."""
-        page = self.free.pop() if self.free else self._evict()
-        assert self.refs[page] == 0
-        self.refs[page] = 1
+        """An unheld page for one holder; the caller has checked `available()`."""
+        page = self.idle.pop() if self.idle else self._evict()
+        assert self.holders[page] == 0
+        self.holders[page] = 1
         return page
 
     def _evict(self) -> int:
-        victim = min((n for n in self.tree.nodes.values() if self.refs[n.block_id] == 0 and not n.children),
-                     key=lambda n: n.last_used, default=None)
-        assert victim is not None, "no free page: the caller must check available() first"
-        self.free_cached -= 1
-        self.evictions += 1
-        return self.tree.evict(victim)
+        while self._queue:
+            moment, page = heapq.heappop(self._queue)
+            if self.released_at.get(page) == moment and self.index.is_leaf(page):     # else: stale
+                before = self.index.parent(page)
+                self.index.discard(page)
+                del self.released_at[page]
+                self.kept -= 1
+                self.evictions += 1
+                if before != TOP and before in self.released_at and self.index.is_leaf(before):
+                    heapq.heappush(self._queue, (self.released_at[before], before))   # its turn comes by its own age
+                return page
+        raise AssertionError("no page to hand out: the caller must check available() first")
 
     def hold(self, page: int) -> None:
-        if self.refs[page] == 0:
-            assert page in self.tree.nodes, "a free unpublished page is handed out by take()"
-            self.free_cached -= 1
-        self.refs[page] += 1
+        """One more request has the page in its table (a kept page is taken over)."""
+        if self.holders[page] == 0:
+            assert page in self.released_at, "an idle page is handed out by take()"
+            del self.released_at[page]
+            self.kept -= 1
+        self.holders[page] += 1
 
     def drop(self, page: int) -> None:
-        assert self.refs[page] > 0, f"page {page} is freed twice"
-        self.refs[page] -= 1
-        if self.refs[page]:
+        """One request less has it; the last one's leaving makes it kept (if indexed) or idle."""
+        assert self.holders[page] > 0, f"page {page} is freed twice"
+        self.holders[page] -= 1
+        if self.holders[page]:
             return
-        node = self.tree.nodes.get(page)
-        if node is None:
-            self.free.append(page)
-        else:
-            self.clock += 1
-            node.last_used = self.clock
-            self.free_cached += 1
+        if page not in self.index:
+            self.idle.append(page)
+            return
+        self._moment += 1
+        self.released_at[page] = self._moment
+        self.kept += 1
+        if self.index.is_leaf(page):
+            heapq.heappush(self._queue, (self._moment, page))
 
 
 class KVCacheManager:
@@ -154,8 +178,8 @@ class KVCacheManager:
 
     # ---- views ------------------------------------------------------------------------------
     @property
-    def tree(self) -> PageTree:
-        return self.spaces[0].tree
+    def index(self) -> PrefixIndex:
+        return self.spaces[0].index
 
     @property
     def num_blocks(self) -> int:
@@ -163,7 +187,7 @@ class KVCacheManager:
 
     @property
     def ref_counts(self) -> list[int]:
-        return self.spaces[0].refs
+        return self.spaces[0].holders
 
     def num_available_blocks(self, space: int = 0) -> int:
         return self.spaces[space].available()
@@ -185,38 +209,37 @@ class KVCacheManager:
     def _pages_for(self, tokens: int) -> int:
         return -(-tokens // self.block_size)
 
-    def _match(self, token_ids: Sequence[int]) -> Match:
-        return self.tree.match(token_ids) if self.caching else Match([])
+    def _lookup(self, token_ids: Sequence[int]) -> Hit:
+        return self.index.lookup(token_ids) if self.caching else Hit()
 
-    def _partial_source(self, match: Match) -> PageNode | None:
-        """The page to copy a partial match from; one that is in use is preferred, because it
-        cannot be evicted while the destination is taken."""
-        if not match.partial_len:
+    def _copy_source(self, hit: Hit) -> int | None:
+        """The page whose leading slots a hit's tail is copied from: a held one if there is one
+        (a kept one could be evicted to make room for the copy), the lowest id among equals."""
+        if not hit.tail:
             return None
-        refs = self.spaces[0].refs
-        return min(match.partial_candidates, key=lambda p: refs[p.block_id] == 0)
+        holders = self.spaces[0].holders
+        return min(hit.tail_holders, key=lambda page: (holders[page] == 0, page))
 
-    def _cost(self, match: Match, source: PageNode | None, num_tokens: int, feed: int | None) -> AdmissionCost:
-        uncached = num_tokens - match.num_tokens
-        now = uncached if feed is None else min(feed, uncached)
-        cover = match.num_tokens + now
-        refs, pages = self.spaces[0].refs, match.pages
-        take = self._pages_for(cover) - len(pages)
-        # the last attached page is partial and somebody holds it: writing past it copies it first
-        if pages and len(pages[-1].tokens) < self.block_size and refs[pages[-1].block_id] > 0:
-            take += 1
-        # copying out of a free page: source and destination must exist side by side
-        if source is not None and refs[source.block_id] == 0:
-            take = max(take, 2)
-        # attached pages that were free leave the free pool too
-        take += sum(1 for p in pages if refs[p.block_id] == 0)
-        rest = tuple(self._pages_for(cover) for _ in self.spaces[1:])
-        return AdmissionCost(take, uncached, (take, *rest))
+    def _cost(self, hit: Hit, source: int | None, num_tokens: int, feed: int | None) -> AdmissionCost:
+        """Pages that leave `available()` of each space if the prompt is admitted on this hit."""
+        main = self.spaces[0]
+        uncached = num_tokens - hit.num_tokens
+        fed = uncached if feed is None else min(feed, uncached)
+        in_all = self._pages_for(hit.num_tokens + fed)
+        fresh = in_all - len(hit.pages)                      # pages to take beyond the ones taken over
+        last = hit.pages[-1] if hit.pages else None
+        if last is not None and len(main.index.tokens(last)) < self.block_size and main.holders[last]:
+            fresh += 1                                       # a shared page that is not full is copied before the first write
+        if source is not None and not main.holders[source]:
+            fresh = max(fresh, 2)                            # a kept source must survive until its copy exists
+        kept_taken_over = sum(1 for page in hit.pages if not main.holders[page])
+        first = fresh + kept_taken_over
+        return AdmissionCost(first, uncached, (first, *(in_all for _ in self.spaces[1:])))
 
     def calculate_admission_cost(self, token_ids: Sequence[int], feed: int | None = None) -> AdmissionCost:
         """What admitting this prompt (its first `feed` uncached tokens) would take. Changes nothing."""
-        match = self._match(token_ids)
-        return self._cost(match, self._partial_source(match), len(token_ids), feed)
+        hit = self._lookup(token_ids)
+        return self._cost(hit, self._copy_source(hit), len(token_ids), feed)
 
     def allocate(self, seq_id: int, token_ids: Sequence[int], feed: int | None = None) -> list[int] | None:
         """Admits a request: attaches its cached prefix, copies a partial match, reserves slots
@@ -224,9 +247,9 @@ class KVCacheManager:
         space 0, or None, with nothing changed, if pages or state slots do not suffice."""
         assert token_ids, "a prompt has at least one token"
         assert seq_id not in self.seqs, "request is already admitted"
-        match = self._match(token_ids)
-        source = self._partial_source(match)
-        cost = self._cost(match, source, len(token_ids), feed)
+        hit = self._lookup(token_ids)
+        source = self._copy_source(hit)
+        cost = self._cost(hit, source, len(token_ids), feed)
         if not self.fits(cost.per_space) or not self.free_state_slots:
             return None
         main = self.spaces[0]
@@ -234,17 +257,17 @@ class KVCacheManager:
         seq.state_slot = self.free_state_slots.pop()
         self.storage.reset_state(seq.state_slot)
         table = seq.tables[0]
-        for page in match.pages:          # hold what matched before anything is taken or evicted
-            main.hold(page.block_id)
-            table.append(page.block_id)
+        for page in hit.pages:            # taken over first: nothing taken below may evict them
+            main.hold(page)
+            table.append(page)
         if source is not None:
-            main.hold(source.block_id)
-            dest = main.take()
-            self.storage.copy_slots(0, source.block_id, dest, match.partial_len)
+            main.hold(source)             # (held for the moment of the copy only)
+            copy = main.take()
+            self.storage.copy_slots(0, source, copy, hit.tail)
             self.counters.partial_copies += 1
-            main.drop(source.block_id)
-            table.append(dest)
-        seq.committed = match.num_tokens
+            main.drop(source)
+            table.append(copy)
+        seq.committed = hit.num_tokens
         seq.token_ids = list(token_ids[:seq.committed])
         uncached = token_ids[seq.committed:]
         self._reserve(seq, uncached if feed is None else uncached[:feed])
@@ -258,15 +281,15 @@ class KVCacheManager:
         for index, (space, table) in enumerate(zip(self.spaces, seq.tables)):
             if used_in_last and token_ids:
                 last = table[-1]
-                if space.refs[last] > 1:       # shared tail: copy before the first write
+                if space.holders[last] > 1:    # shared tail: copy before the first write
                     fresh = space.take()
                     self.storage.copy_slots(index, last, fresh, used_in_last)
                     self.counters.cow_copies += 1
                     space.drop(last)
                     table[-1] = fresh
                 else:
-                    node = space.tree.nodes.get(last)
-                    assert node is None or used_in_last >= len(node.tokens), "a published slot would be overwritten"
+                    assert last not in space.index or used_in_last >= len(space.index.tokens(last)), \
+                        "a published slot would be overwritten"
             while len(table) < want_pages:
                 table.append(space.take())
         seq.token_ids.extend(token_ids)
@@ -275,7 +298,7 @@ class KVCacheManager:
         seq = self.seqs[seq_id]
         table = seq.tables[space]
         need = self._pages_for(seq.reserved + num_tokens) - len(table)
-        if num_tokens and seq.reserved % self.block_size and self.spaces[space].refs[table[-1]] > 1:
+        if num_tokens and seq.reserved % self.block_size and self.spaces[space].holders[table[-1]] > 1:
             need += 1      # the shared tail page is copied first
         return need
 
@@ -283,7 +306,7 @@ class KVCacheManager:
         seq = self.seqs[seq_id]
         if num_tokens and (seq.reserved % self.block_size) + num_tokens <= self.block_size and seq.reserved % self.block_size:
             # the tokens stay inside the last page: pages are needed only to copy a shared tail
-            return all(sp.refs[t[-1]] <= 1 or sp.available() >= 1 for sp, t in zip(self.spaces, seq.tables))
+            return all(sp.holders[t[-1]] <= 1 or sp.available() >= 1 for sp, t in zip(self.spaces, seq.tables))
         return all(self.blocks_needed_for_append(seq_id, num_tokens, i) <= sp.available()
                    for i, sp in enumerate(self.spaces))
 
@@ -307,7 +330,7 @@ class KVCacheManager:
         used_in_last = reserved % self.block_size
         for space, table in zip(self.spaces, seq.tables):       # first pass: is there room everywhere
             if used_in_last:
-                if space.refs[table[-1]] > 1 and space.available() < 1:
+                if space.holders[table[-1]] > 1 and space.available() < 1:
                     return False
             elif self._pages_for(reserved + 1) > len(table) and space.available() < 1:
                 return False
@@ -354,26 +377,23 @@ class KVCacheManager:
             self.counters.window_frees += 1
 
     def _publish(self, seq: SeqState, i: int) -> None:
-        """Records page i of the request in the tree under the page before it; swaps to an
-        identical page if the tree already has one."""
+        """Makes page i of the request findable by the tokens committed into it. If the index has
+        a page with these very tokens after the same page already, the request moves over to that
+        one and lets its own go."""
         main, table = self.spaces[0], seq.tables[0]
-        page = table[i]
-        parent = main.tree.nodes[table[i - 1]] if i else main.tree.root
+        page, index = table[i], main.index
         tokens = seq.token_ids[i * self.block_size:min((i + 1) * self.block_size, seq.committed)]
-        node = main.tree.nodes.get(page)
-        if node is None:
-            kept = main.tree.publish(parent, page, tokens)
-            if kept.block_id == page:
-                self.counters.publishes += 1
-        elif len(node.tokens) < len(tokens):
-            assert node.parent is parent
-            kept = main.tree.grow(node, tokens)      # an attached partial page we wrote further into
+        if page not in index:
+            stands = index.add(table[i - 1] if i else TOP, page, tokens)
+            self.counters.publishes += stands == page
+        elif len(index.tokens(page)) < len(tokens):
+            stands = index.extend(page, tokens)       # a page taken over while it was not full, written further into
         else:
             return
-        if kept.block_id != page:
+        if stands != page:
             self.counters.dedupes += 1
-            main.hold(kept.block_id)
-            table[i] = kept.block_id
+            main.hold(stands)
+            table[i] = stands
             main.drop(page)
 
     # ---- leaving, forking -------------------------------------------------------------------
@@ -413,4 +433,4 @@ class KVCacheManager:
     def stats(self) -> CacheStats:
         main = self.spaces[0]
         return replace(self.counters, evictions=sum(s.evictions for s in self.spaces),
-                       blocks_in_use=main.num_pages - main.available(), cached_pages=len(main.tree.nodes))
+                       blocks_in_use=main.num_pages - main.available(), cached_pages=len(main.index))

@@ -6,7 +6,9 @@ Runs of tokens that no other page leaves are kept as one edge (a page of 256 tok
 nothing with its siblings is one node, not 256): an edge carries its tokens as a tuple and the set
 of pages that pass through it, and every page that enters an edge reaches its end, because a run
 that ends inside an edge splits the edge there. All positions inside an edge therefore see the same
-pages, the set of the node at the edge's end."""
+pages, the set of the node at the edge's end. The node where a page's run ends is marked with that
+page, so the page that holds exactly a given run is found by the same walk (two pages never hold
+the same run: the index above swaps to the first)."""
 
 from __future__ import annotations
 
@@ -14,12 +16,13 @@ from typing import Hashable, Iterable, Sequence
 
 
 class _Node:
-    __slots__ = ("label", "next", "pages")
+    __slots__ = ("label", "next", "pages", "ends")
 
     def __init__(self, label: tuple[int, ...] = (), pages: set | None = None) -> None:
         self.label = label                       # the tokens from the parent to here; empty for the root only
         self.next: dict[int, _Node] = {}         # first token of an edge -> the node at its end
         self.pages: set = set() if pages is None else pages
+        self.ends: Hashable | None = None        # the page whose run ends exactly here
 
 
 def _shared(label: tuple[int, ...], tokens: tuple[int, ...], at: int) -> int:
@@ -58,13 +61,17 @@ class TokenTrie:
         while i < len(run):
             nxt = at.next.get(run[i])
             if nxt is None:
-                at.next[run[i]] = _Node(run[i:], {page})
+                nxt = at.next[run[i]] = _Node(run[i:], {page})
+                nxt.ends = page
                 return
             m = _shared(nxt.label, run, i)
             if m < len(nxt.label):           # the run leaves the edge, or ends inside it
                 nxt = self._split(at, nxt, m)
             nxt.pages.add(page)
+            if nxt.ends == page:
+                nxt.ends = None              # its shorter run ended here; the longer one goes on
             at, i = nxt, i + m
+        at.ends = page
 
     def remove(self, page: Hashable, tokens: Sequence[int]) -> None:
         """Takes `page` off its path (`tokens` is the run it was last inserted with) and prunes
@@ -73,14 +80,16 @@ class TokenTrie:
         while i < len(tokens):
             nxt = at.next[tokens[i]]
             nxt.pages.remove(page)
+            if nxt.ends == page:
+                nxt.ends = None
             if not nxt.pages:
                 del at.next[tokens[i]]   # everything below belonged to this page alone
                 return
             at, i = nxt, i + len(nxt.label)
 
-    def longest_match(self, tokens: Iterable[int]) -> tuple[int, set]:
-        """(number of leading tokens found, the pages at the deepest position). The set is the
-        trie's own: read it, do not change it."""
+    def find(self, tokens: Iterable[int]) -> tuple[int, set, Hashable | None]:
+        """(number of leading tokens found, the pages at the deepest position, the page whose run is
+        exactly those tokens or None). The set is the trie's own: read it, do not change it."""
         run = tokens if isinstance(tokens, tuple) else tuple(tokens)
         at, depth = self.root, 0
         while depth < len(run):
@@ -89,6 +98,16 @@ class TokenTrie:
                 break
             m = _shared(nxt.label, run, depth)
             if m < len(nxt.label):
-                return depth + m, nxt.pages
+                return depth + m, nxt.pages, None          # inside an edge no run ends
             at, depth = nxt, depth + m
-        return depth, at.pages
+        return depth, at.pages, at.ends
+
+    def longest_match(self, tokens: Iterable[int]) -> tuple[int, set]:
+        """(number of leading tokens found, the pages at the deepest position)."""
+        return self.find(tokens)[:2]
+
+    def exact(self, tokens: Iterable[int]) -> Hashable | None:
+        """The page whose run is exactly `tokens`, or None."""
+        run = tokens if isinstance(tokens, tuple) else tuple(tokens)
+        depth, _, page = self.find(run)
+        return page if depth == len(run) else None

@@ -29,12 +29,12 @@ __device__ __forceinline__ bool better(float v, int i, float bv, int bi) { retur
 // Stage 1: workgroup (slice, row) finds the best of its slice of the vocabulary.
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_slice_kernel(float* __restrict__ best_v, int32_t* __restrict__ best_i, const float* __restrict__ logits,
-                    const float* __restrict__ temps, const int64_t* __restrict__ keys, uint64_t seed, int vocab,
-                    int64_t ld) {
+                    const int32_t* __restrict__ row_of, const float* __restrict__ temps, const int64_t* __restrict__ keys,
+                    uint64_t seed, int vocab, int64_t ld) {
   __shared__ float sv[SAMPLE_THREADS / TS_WAVE];
   __shared__ int si[SAMPLE_THREADS / TS_WAVE];
   const int r = blockIdx.y, slice = blockIdx.x;
-  const float* row = logits + (int64_t)r * ld;
+  const float* row = logits + (int64_t)(row_of ? row_of[r] : r) * ld;   // several draws may read one row
   const float t = temps[r];
   const uint64_t key = (uint64_t)keys[r];
   const int per = (vocab + SAMPLE_SLICES - 1) / SAMPLE_SLICES;
@@ -77,18 +77,34 @@ sample_pick_kernel(int32_t* __restrict__ out, const float* __restrict__ best_v, 
   if (lane == 0) out[r] = bi == 0x7fffffff ? 0 : bi;
 }
 
-// work_v, work_i: [rows, SAMPLE_SLICES] float / int32 workspaces
-extern "C" int ts_sample(int32_t* out, float* work_v, int32_t* work_i, const float* logits, const float* temps,
-                         const int64_t* keys, uint64_t seed, int rows, int vocab, int64_t ld, hipStream_t stream) {
+// work_v, work_i: [rows, SAMPLE_SLICES] float / int32 workspaces. row_of: null, or for each of the `rows`
+// draws the row of `logits` it reads (checked by the caller against the rows that `logits` has).
+static int sample_launch(int32_t* out, float* work_v, int32_t* work_i, const float* logits, const int32_t* row_of,
+                         const float* temps, const int64_t* keys, uint64_t seed, int rows, int vocab, int64_t ld,
+                         hipStream_t stream) {
   if (rows <= 0) return TS_OK;
   if (vocab <= 0 || ld < vocab || rows > 65535) return TS_BAD_SHAPE;
   static_assert(SAMPLE_SLICES <= TS_WAVE, "one wave picks among the slices");
-  sample_slice_kernel<<<dim3(SAMPLE_SLICES, rows), SAMPLE_THREADS, 0, stream>>>(work_v, work_i, logits, temps, keys,
-                                                                              seed, vocab, ld);
+  sample_slice_kernel<<<dim3(SAMPLE_SLICES, rows), SAMPLE_THREADS, 0, stream>>>(work_v, work_i, logits, row_of, temps,
+                                                                              keys, seed, vocab, ld);
   int rc = ts_check_launch();
   if (rc) return rc;
   sample_pick_kernel<<<rows, TS_WAVE, 0, stream>>>(out, work_v, work_i);
   return ts_check_launch();
+}
+
+extern "C" int ts_sample(int32_t* out, float* work_v, int32_t* work_i, const float* logits, const float* temps,
+                         const int64_t* keys, uint64_t seed, int rows, int vocab, int64_t ld, hipStream_t stream) {
+  return sample_launch(out, work_v, work_i, logits, nullptr, temps, keys, seed, rows, vocab, ld, stream);
+}
+
+// The same for `rows` draws of which draw r reads row row_of[r] of `logits` (n samples of one prompt
+// read the one row that its last position gave).
+extern "C" int ts_sample_rows(int32_t* out, float* work_v, int32_t* work_i, const float* logits, const int32_t* row_of,
+                              const float* temps, const int64_t* keys, uint64_t seed, int rows, int vocab, int64_t ld,
+                              hipStream_t stream) {
+  if (!row_of) return TS_BAD_SHAPE;
+  return sample_launch(out, work_v, work_i, logits, row_of, temps, keys, seed, rows, vocab, ld, stream);
 }
 
 // ids[i] = prev[src[i]] where src[i] >= 0: the tokens a step drew become the next step's input

@@ -172,8 +172,7 @@ class LLM:
             owners.append(num_samples)
         if not rows:
             return None, owners
-        picked = logits if rows == list(range(logits.shape[0])) else logits[torch.tensor(rows, device=logits.device)]
-        return sample(picked, temps, keys, self.seed), owners
+        return sample(logits, temps, keys, self.seed, None if rows == list(range(logits.shape[0])) else rows), owners
 
     def _finish(self, launched: tuple) -> list[list[int]]:
         """Waits for a launched step; the one host sync of a step. Tokens per entry."""

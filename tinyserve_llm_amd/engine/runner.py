@@ -276,9 +276,10 @@ class ModelRunner:
 
 
 class DrawnTokens:
-    """The tokens a replayed step drew: a copy on the device (for the step after it to take its
-    ids from) and one on its way to pinned host memory. `tolist()` waits for that copy alone, not
-    for what was started on the device after it."""
+    """The tokens a replayed step drew: on the device, where the graph wrote them (for the step
+    started right after it to take its ids from; the graph's next replay overwrites them), and a
+    copy on its way to pinned host memory. `tolist()` waits for that copy alone, not for what was
+    started on the device after it."""
 
     def __init__(self, on_device: torch.Tensor, host: torch.Tensor, landed: torch.cuda.Event, n: int) -> None:
         self.on_device, self.host, self.landed, self.n = on_device, host, landed, n
@@ -416,9 +417,8 @@ class DecodeGraphs:
     def launch(self, prepared: tuple, drawn_before: torch.Tensor | None = None) -> torch.Tensor:
         """The device half: uploads the packed step, lets the entries that name a source row take
         their ids from `drawn_before` (the tokens of the step before, on the device) and replays the
-        step's graph. Logits [entries, vocab], or the tokens drawn (`DrawnTokens`: copies, since
-        the next replay writes the graph's own tokens anew and may be started before anyone has
-        read these) if the step was prepared with draws."""
+        step's graph. Logits [entries, vocab], or the tokens drawn (`DrawnTokens`) if the step was
+        prepared with draws."""
         from tinyserve_llm_amd.ops import hip
         key, words, start, dims, host, n, drawn, fed = prepared
         if fed and drawn_before is None:
@@ -441,10 +441,13 @@ class DecodeGraphs:
             return logits[:n]
         host_tokens, landed = landing[turn]
         kept[7] = 1 - turn
-        on_device = tokens[:n].clone()
-        host_tokens[:n].copy_(on_device, non_blocking=True)
+        # The tokens stay where the graph wrote them. The copy to the host is queued behind this replay
+        # and ahead of the next one, and the step after this one takes its ids from here before its own
+        # replay is queued (`feed_tokens` above), so the next replay of this graph, which writes the
+        # tokens anew, comes after both on the stream.
+        host_tokens[:n].copy_(tokens[:n], non_blocking=True)
         landed.record()
-        return DrawnTokens(on_device, host_tokens, landed, n)
+        return DrawnTokens(tokens[:n], host_tokens, landed, n)
 
     def run(self, entries: Sequence[StepEntry], draws=None) -> torch.Tensor:
         """Replays the step's graph. Without `draws` the logits [entries, vocab] come back; with

@@ -207,7 +207,7 @@ class Scheduler:
             final = seq.num_computed + len(tokens) >= seq.prefill_target
             samples = 1
             if want_prefill:
-                samples = 0 if not final else (seq.params.n if self._first_of_group(seq) else 1)
+                samples = 0 if not final else (seq.params.n if seq.awaits_first_token() else 1)
                 self.counters.prefill_tokens += len(tokens)
             else:
                 self.counters.decode_tokens += 1
@@ -233,13 +233,9 @@ class Scheduler:
         self.running.remove(seq)
         self.waiting.append(seq)
 
-    @staticmethod
-    def _first_of_group(seq: Sequence) -> bool:
-        return seq.params.n > 1 and not seq.output_token_ids
-
     def _owed_forks(self) -> int:
-        """Samples that running groups will still fork off when their prompts end."""
-        return sum(s.params.n - 1 for s in self.running if self._first_of_group(s))
+        """Sequences that running requests will still split off when their prompts end."""
+        return sum(s.params.n - 1 for s in self.running if s.awaits_first_token())
 
     def _admit(self, now: float, budget: int) -> list[ScheduledSeq]:
         """Admits waiting sequences, best score first, within the token budget, the sequence cap
@@ -258,7 +254,7 @@ class Scheduler:
             feed = self._chunk(whole.prefill_tokens, budget)
             cost = self.kv.calculate_admission_cost(tokens, feed)
             hit = self._hit(len(tokens), whole)
-            forks = seq.params.n - 1 if self._first_of_group(seq) else 0
+            forks = seq.params.n - 1 if seq.awaits_first_token() else 0
             fits = (feed >= 1
                     and len(self.running) + owed + 1 + forks <= self.config.max_num_seqs
                     and self.kv.fits(cost.per_space, owed + forks + self.watermark_blocks))
@@ -287,62 +283,59 @@ class Scheduler:
             seq.in_step = True
             admitted.append(ScheduledSeq(seq, fed, samples, cached))
         if admitted:
-            chosen = {s.seq.seq_id for s in admitted}
-            self.waiting = [s for s in self.waiting if s.seq_id not in chosen]
+            self.waiting = [s for s in self.waiting if s.status is SequenceStatus.WAITING]
         return admitted
 
     # ---- after the model ran ----------------------------------------------------------------
-    def _fork(self, parent: Sequence, index: int) -> Sequence:
-        assert not parent.output_token_ids
-        child = Sequence(next(self._seq_ids), parent.request_id, parent.prompt_token_ids, parent.params,
-                         parent.arrival_time, status=SequenceStatus.RUNNING, sample_index=index,
-                         admission_hit=parent.admission_hit, prefill_target=parent.prefill_target,
-                         num_computed=parent.num_computed)
-        self.kv.fork(parent.seq_id, child.seq_id)
-        self.running.append(child)
-        self.groups[parent.request_id].append(child)
-        return child
+    def _split_off(self, first: Sequence, how_many: int) -> list[Sequence]:
+        """The sequences that take the `how_many` tokens drawn from a prompt's last position: the
+        one that was fed, and for n > 1 its new siblings, which share all its pages."""
+        family = [first]
+        for index in range(1, how_many):
+            sibling = first.continuation(next(self._seq_ids), index)
+            self.kv.fork(first.seq_id, sibling.seq_id)
+            self.running.append(sibling)
+            self.groups[first.request_id].append(sibling)
+            family.append(sibling)
+        return family
 
-    def _finish_reason(self, seq: Sequence, token: int) -> Literal["eos", "length"] | None:
-        if token == self.config.eos_token_id and not seq.params.ignore_eos:
-            return "eos"
-        if len(seq.output_token_ids) >= seq.params.max_tokens:
-            return "length"
-        return None
+    def _retire(self, ended: list[Sequence]) -> list[RequestOutput]:
+        """Takes ended sequences off the running list; a request whose sequences have all ended is
+        handed out, in the order in which the requests' last sequences ended."""
+        if not ended:
+            return []
+        gone = {s.seq_id for s in ended}
+        self.running = [s for s in self.running if s.seq_id not in gone]
+        complete = []
+        for seq in ended:
+            family = self.groups.get(seq.request_id)
+            if family is not None and all(s.status is SequenceStatus.FINISHED for s in family):
+                complete.append(RequestOutput(seq.request_id, self.groups.pop(seq.request_id)))
+        return complete
 
     def postprocess(self, scheduled: list[ScheduledSeq], sampled: list[list[int]], now: float) -> list[RequestOutput]:
-        """Commits each sequence's slots, forks a group after its prompt, records new tokens,
-        releases what finished (scheduler.py:236-263)."""
-        finished: list[Sequence] = []
+        """Closes a step in one piece: every entry's slots are committed; where tokens were drawn, the
+        sequence (for n > 1: it and the siblings split off it now) takes them, and what ends with
+        its token gives its pages back (the reference's counterpart is scheduler.py:236-263)."""
+        ended: list[Sequence] = []
         for (seq, token_ids, num_samples, _), tokens in zip(scheduled, sampled, strict=True):
             assert len(tokens) == num_samples
             seq.in_step = False
             self.kv.commit(seq.seq_id, len(token_ids))
             seq.num_computed += len(token_ids)
-            if num_samples == 0:
-                continue
-            samples = [seq] + [self._fork(seq, k) for k in range(1, num_samples)]
-            for sample, token in zip(samples, tokens):
-                sample.output_token_ids.append(token)
-                sample.prefill_target = sample.num_computed      # from here on it decodes
-                if sample.first_token_time is None:
-                    sample.first_token_time = now
-                reason = self._finish_reason(sample, token)
+            if not tokens:
+                continue                                   # a portion that does not end its prompt
+            for taker, token in zip(self._split_off(seq, num_samples), tokens):
+                taker.output_token_ids.append(token)
+                taker.prefill_target = taker.num_computed  # from here on it decodes
+                if taker.first_token_time is None:
+                    taker.first_token_time = now
+                reason = taker.why_it_ends(self.config.eos_token_id)
                 if reason is not None:
-                    self.kv.release(sample.seq_id)
-                    sample.status = SequenceStatus.FINISHED
-                    sample.finish_reason = reason
-                    sample.finish_time = now
-                    finished.append(sample)
-        if finished:
-            done = {s.seq_id for s in finished}
-            self.running = [s for s in self.running if s.seq_id not in done]
-        outputs = []
-        for request_id in dict.fromkeys(s.request_id for s in finished):
-            group = self.groups[request_id]
-            if all(s.status is SequenceStatus.FINISHED for s in group):
-                outputs.append(RequestOutput(request_id, self.groups.pop(request_id)))
-        return outputs
+                    self.kv.release(taker.seq_id)
+                    taker.finish(reason, now)
+                    ended.append(taker)
+        return self._retire(ended)
 
     # ---- the same for decode steps, in two halves -------------------------------------------------
     @staticmethod
@@ -367,14 +360,14 @@ class Scheduler:
         `ahead` is the step scheduled in between: its entries that feed a placeholder get the token,
         entries of sequences that turn out finished are dropped. Returns the finished requests and
         what is left of `ahead`."""
-        finished: list[Sequence] = []
+        ended: list[Sequence] = []
         fed_ahead = {b.seq.seq_id: b for b in ahead or ()}
         for (seq, _, _, _), tokens in zip(scheduled, sampled, strict=True):
             assert len(tokens) == 1 and seq.output_token_ids[-1] == PENDING
             token = tokens[0]
             seq.output_token_ids[-1] = token
             entry = fed_ahead.get(seq.seq_id)
-            reason = self._finish_reason(seq, token)
+            reason = seq.why_it_ends(self.config.eos_token_id)
             if reason is None:
                 if entry is not None:
                     assert entry.token_ids == [PENDING] and entry.start == seq.num_computed
@@ -389,19 +382,9 @@ class Scheduler:
                 self.kv.release(seq.seq_id)
             else:                                  # preempted in between: its pages went back then
                 self.waiting = [s for s in self.waiting if s.seq_id != seq.seq_id]
-            seq.status = SequenceStatus.FINISHED
-            seq.finish_reason = reason
-            seq.finish_time = now
-            finished.append(seq)
-        if finished:
-            done = {s.seq_id for s in finished}
-            self.running = [s for s in self.running if s.seq_id not in done]
-        outputs = []
-        for request_id in dict.fromkeys(s.request_id for s in finished):
-            group = self.groups[request_id]
-            if all(s.status is SequenceStatus.FINISHED for s in group):
-                outputs.append(RequestOutput(request_id, self.groups.pop(request_id)))
-        return outputs, [b for b in ahead or () if b.seq.seq_id in fed_ahead]
+            seq.finish(reason, now)
+            ended.append(seq)
+        return self._retire(ended), [b for b in ahead or () if b.seq.seq_id in fed_ahead]
 
     def stats(self) -> SchedulerStats:
         return replace(self.counters, num_waiting=len(self.waiting), num_running=len(self.running))

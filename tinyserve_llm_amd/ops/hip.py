@@ -55,6 +55,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_gemm_exact": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_sample": [p, p, p, p, p, p, u64, i, i, i64, p],
         "ts_sample_static": [p, p, p, p, u64, i, i, i64, p],
+        "ts_sample_rows": [p, p, p, p, p, p, p, u64, i, i, i64, p],
         "ts_feed_tokens": [p, p, p, i, i, p],
         "ts_gemm_library_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p, ctypes.c_size_t, p],
         "ts_gemm_tiled_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
@@ -412,21 +413,32 @@ def feed_tokens(ids: torch.Tensor, prev: torch.Tensor, src: torch.Tensor) -> Non
     _run("feed_tokens", library().ts_feed_tokens(_ptr(ids), _ptr(prev), _ptr(src), ids.shape[0], prev.shape[0], _stream()))
 
 
-def sample(logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor, seed: int) -> torch.Tensor:
-    """One token per row of float32 `logits`: argmax where the temperature is 0, else a draw whose
-    noise is a function of (seed, keys[row], vocabulary index) alone."""
-    _gpu(logits, temperatures, keys)
+def sample(logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor, seed: int,
+           row_of: torch.Tensor | None = None, num_logit_rows_checked: bool = False) -> torch.Tensor:
+    """One token per draw from float32 `logits`: argmax where the temperature is 0, else a draw whose
+    noise is a function of (seed, keys[draw], vocabulary index) alone. Draw r reads row r, or with
+    `row_of` (int32, values the caller has checked to lie inside `logits`) row row_of[r]: the n
+    samples of one prompt all read the row of its last position."""
+    _gpu(logits, temperatures, keys, row_of)
     _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.stride(1) == 1, "logits must be float32 [rows, vocab]")
     R = logits.shape[0]
+    if row_of is not None:
+        _need(num_logit_rows_checked, "the caller checks the rows that the draws read on the host")
+        _need(row_of.dtype == torch.int32 and row_of.dim() == 1 and row_of.is_contiguous() and R > 0, "row_of must be int32 [draws]")
+        R = row_of.shape[0]
     _need(temperatures.dtype == torch.float32 and temperatures.shape == (R,) and temperatures.is_contiguous(),
-          "temperatures must be float32 [rows]")
-    _need(keys.dtype == torch.int64 and keys.shape == (R,) and keys.is_contiguous(), "keys must be int64 [rows]")
+          "temperatures must be float32 [draws]")
+    _need(keys.dtype == torch.int64 and keys.shape == (R,) and keys.is_contiguous(), "keys must be int64 [draws]")
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
     work_v = torch.empty((R, 64), dtype=torch.float32, device=logits.device)
     work_i = torch.empty((R, 64), dtype=torch.int32, device=logits.device)
-    _run("sample", library().ts_sample(_ptr(out), _ptr(work_v), _ptr(work_i), _ptr(logits), _ptr(temperatures),
-                                       _ptr(keys), seed & 0xFFFFFFFFFFFFFFFF, R, logits.shape[1], logits.stride(0),
-                                       _stream()))
+    if row_of is None:
+        rc = library().ts_sample(_ptr(out), _ptr(work_v), _ptr(work_i), _ptr(logits), _ptr(temperatures), _ptr(keys),
+                                 seed & 0xFFFFFFFFFFFFFFFF, R, logits.shape[1], logits.stride(0), _stream())
+    else:
+        rc = library().ts_sample_rows(_ptr(out), _ptr(work_v), _ptr(work_i), _ptr(logits), _ptr(row_of), _ptr(temperatures),
+                                      _ptr(keys), seed & 0xFFFFFFFFFFFFFFFF, R, logits.shape[1], logits.stride(0), _stream())
+    _run("sample", rc)
     return out
 
 

@@ -22,10 +22,17 @@ def row_key(request_id: int, sample_index: int, position: int) -> int:
     return x & _MASK
 
 
-def sample(logits: torch.Tensor, temperatures: list[float], keys: list[int], seed: int) -> torch.Tensor:
-    """One token id per row of float32 logits [rows, vocab] -> int32 [rows] on the device."""
+def sample(logits: torch.Tensor, temperatures: list[float], keys: list[int], seed: int,
+           rows: list[int] | None = None) -> torch.Tensor:
+    """One token id per draw from float32 logits [rows, vocab] -> int32 [draws] on the device. Draw i
+    reads row i, or row rows[i] if `rows` is given (several draws may read one row)."""
     n = len(keys)
-    # keys and temperatures travel to the device in one copy
-    packed = torch.cat([torch.tensor(keys, dtype=torch.int64).view(torch.int32),
-                        torch.tensor(temperatures, dtype=torch.float32).view(torch.int32)]).to(logits.device, non_blocking=True)
-    return hip.sample(logits, packed[2 * n:].view(torch.float32), packed[:2 * n].view(torch.int64), seed)
+    if rows is not None and (len(rows) != n or min(rows, default=0) < 0 or max(rows, default=0) >= logits.shape[0]):
+        raise ValueError(f"{n} draws name rows outside the {logits.shape[0]} rows of logits")
+    # keys, temperatures and rows travel to the device in one copy
+    words = [torch.tensor(keys, dtype=torch.int64).view(torch.int32), torch.tensor(temperatures, dtype=torch.float32).view(torch.int32)]
+    if rows is not None:
+        words.append(torch.tensor(rows, dtype=torch.int32))
+    packed = torch.cat(words).to(logits.device, non_blocking=True)
+    return hip.sample(logits, packed[2 * n:3 * n].view(torch.float32), packed[:2 * n].view(torch.int64), seed,
+                      packed[3 * n:] if rows is not None else None, num_logit_rows_checked=True)
