@@ -845,6 +845,45 @@ def test_weight_streaming_gemm_reads_the_packed_copy_to_the_same_result(m, n, k)
         hip().gemm_skinny(x, w, packed=p[1:])
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 2048, 2048), (8, 2048, 8192), (5, 3072, 3072), (8, 4096, 14336), (3, 44, 256),
+                                   (8, 2048, 1024), (7, 8, 512), (2, 1000, 4096), (8, 24, 16384)])
+def test_eight_row_form_of_the_weight_streaming_gemm(m, n, k):
+    """The form for at most 8 rows of x (a matrix instruction multiplies 8 rows of W by 8 of x over two
+    halves of 64 k; only the diagonal blocks of its result count): against 64-bit, in both output
+    types, from the matrix and from its packed copy bit for bit, a single row as the same row among
+    eight, and a width that is no multiple of 8. The matrix has one large entry per row in the upper
+    half of a wave's k, which a block taken from off the diagonal would miss or count twice."""
+    g = gen(m * 3 + n + k)
+    w = (torch.randn(n, k, generator=g) * 0.05)
+    steps = hip().skinny8_steps(k)
+    assert steps and hip().skinny8_takes(m, n, k)
+    for row in range(n):
+        w[row, (row * 37) % (32 * steps) + 32 * steps] = 3.0 + row % 5           # in the second half of wave 0's k
+    w = w.bfloat16().to(dev())
+    x = torch.randn(8, k, generator=g).bfloat16().to(dev())
+    want = x[:m].double().cpu() @ w.double().cpu().T
+    out = hip().gemm_skinny8(x[:m].contiguous(), w)
+    assert out.dtype == torch.bfloat16 and out.shape == (m, n)
+    torch.testing.assert_close(out.double().cpu(), want, rtol=1e-2, atol=1e-2 * float(want.abs().max()))
+    f32 = hip().gemm_skinny8(x[:m].contiguous(), w, torch.float32)
+    torch.testing.assert_close(f32.double().cpu(), want, rtol=1e-4, atol=1e-4 * float(want.abs().max()))
+    alone = hip().gemm_skinny8(x[m - 1:m].contiguous(), w, torch.float32)
+    assert torch.equal(alone[0], f32[m - 1]), "a row's sums do not depend on the rows beside it"
+    if n % 8 == 0:
+        p = hip().pack_weight8(w)
+        assert p.shape == (n // 8, k // (64 * steps), steps, 64, 8)
+        assert torch.equal(p[0, 0, 1, 3 + 8 + 16 * 2], w[3, 32 * steps + 32 + 16:32 * steps + 32 + 24]), \
+            "lane r + 16 g: row r % 8, k = 32 steps (r // 8) + 32 step + 8 g .."
+        assert torch.equal(hip().gemm_skinny8(x[:m].contiguous(), w, packed8=p), out)
+        assert torch.equal(hip().gemm_skinny8(x[:m].contiguous(), w, torch.float32, packed8=p), f32)
+        with pytest.raises(hip().KernelError, match="packed copy"):
+            hip().gemm_skinny8(x[:m].contiguous(), w, packed8=p[..., :4])
+    from tinyserve_llm_amd.parts.linear import linear, streaming_copy
+    assert torch.equal(linear(x[:m].contiguous(), w, packed=streaming_copy(w)), out) or n > hip().SKINNY8_MAX_WIDTH
+    with pytest.raises(hip().KernelError):
+        hip().gemm_skinny8(torch.cat([x, x])[:9].contiguous(), w)
+
+
 def test_fused_projection_reads_the_packed_copy_to_the_same_result():
     g = gen(77)
     nh, nkv, hd, K, M, page = 6, 2, 64, 1024, 7, 16

@@ -366,6 +366,108 @@ static int sk_dispatch(const SkinnyArgs& a, hipStream_t stream) {
 #undef SK_GO
 }
 
+// ---- up to 8 rows of x, narrow matrices ------------------------------------------------------------
+// With at most 8 rows of x, half of a 16 x 16 x 32 matrix instruction would multiply rows that do not
+// exist. Here it multiplies 8 rows of W by 8 rows of x over 64 k instead: lanes r < 8 of the A operand
+// hold rows n0 .. n0 + 7 of W at k, lanes r >= 8 the same rows at k + 32 STEPS; the B operand holds
+// the rows of x at k in its columns 0 .. 7 and at k + 32 STEPS in its columns 8 .. 15. Of the 16 x 16
+// result the two 8 x 8 blocks on the diagonal are the two halves of the sum; the other two blocks mix
+// the halves and are dropped. A workgroup then owns 8 rows of W, not 16: a matrix of 2,048 rows
+// gives 256 workgroups, one per compute unit, and a reduction of 8,192 fits the 8 waves of one
+// workgroup (a wave covers 64 STEPS of k), where the 16-row form needs 16 waves on half the chip.
+// packed: W in the order of these loads, [N / 8 tiles][waves][STEPS][lane][8] (see hip.pack_weight8).
+template <int STEPS, int MAXT, typename OUT>
+__global__ void __launch_bounds__(MAXT)
+gemm_skinny8_kernel(const SkinnyArgs a) {
+  extern __shared__ __align__(16) float smem[];         // [nwaves][256]
+  const int nwaves = blockDim.x / TS_WAVE;
+  const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
+  const int r = lane & 15, g = lane >> 4, row = r & 7, half = r >> 3;
+  const int n0 = blockIdx.x * 8;
+  const int kbeg = wave * (2 * STEPS * SK_KSTEP) + half * (STEPS * SK_KSTEP) + 8 * g;   // this lane's first k
+  uint4 wreg[STEPS];
+  if (a.packed) {
+    const bf16_t* blk = a.w + ((((int64_t)blockIdx.x * nwaves + wave) * STEPS) * 64 + lane) * 8;
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) wreg[s] = *(const uint4*)(blk + (int64_t)s * 512);
+  } else {
+    const int n = n0 + row < a.N ? n0 + row : a.N - 1;    // rows past the end are computed and not stored
+    const bf16_t* wrow = a.w + (int64_t)n * a.ldw + kbeg;
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) wreg[s] = *(const uint4*)(wrow + s * SK_KSTEP);
+  }
+  __builtin_amdgcn_sched_barrier(0);                    // all of W's loads are in flight before anything waits
+  const bf16_t* xrow = a.x + (int64_t)(row < a.M ? row : 0) * a.ldx + kbeg;   // rows past M repeat row 0 and are not stored
+  float4_t acc = {0.f, 0.f, 0.f, 0.f};
+  constexpr int XB = STEPS < 8 ? STEPS : 8;
+#pragma unroll
+  for (int s0 = 0; s0 < STEPS; s0 += XB) {
+    uint4 xb[XB];
+#pragma unroll
+    for (int s = 0; s < XB; ++s) xb[s] = *(const uint4*)(xrow + (s0 + s) * SK_KSTEP);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int s = 0; s < XB; ++s) acc = sk_mfma(wreg[s0 + s], xb[s], acc);
+  }
+  // acc[j] = D[4 g + j][r]: W row (4 g + j) & 7 of half (4 g + j) >> 3 times x row r & 7 of half r >> 3
+#pragma unroll
+  for (int j = 0; j < 4; ++j) smem[wave * 256 + r * 16 + 4 * g + j] = acc[j];
+  __syncthreads();
+  if (threadIdx.x >= 64) return;
+  const int m = threadIdx.x >> 3, nl = threadIdx.x & 7;  // x row, W row of the tile
+  float sum = 0.f;
+  for (int wv = 0; wv < nwaves; ++wv)                    // waves in order, within a wave the lower half of k first
+    sum += smem[wv * 256 + m * 16 + nl] + smem[wv * 256 + (m + 8) * 16 + nl + 8];
+  const int n = n0 + nl;
+  if constexpr (sizeof(OUT) == 4) {
+    if (m < a.M && n < a.N) ((float*)a.y)[(int64_t)m * a.ldy + n] = sum;
+  } else {
+    const uint32_t mine = sk_round(sum), next = __shfl_down(mine, 1, TS_WAVE);
+    if (m < a.M && !(nl & 1)) {
+      bf16_t* dst = (bf16_t*)a.y + (int64_t)m * a.ldy + n;
+      if (n + 1 < a.N && !(((uintptr_t)dst) & 3)) *(uint32_t*)dst = mine | (next << 16);
+      else {
+        if (n < a.N) dst[0] = (bf16_t)mine;
+        if (n + 1 < a.N) dst[1] = (bf16_t)next;
+      }
+    }
+  }
+}
+
+template <typename OUT>
+static int sk8_dispatch(const SkinnyArgs& a, hipStream_t stream) {
+  // a wave covers 64 STEPS of k; 8 waves where the reduction allows it, never more than 16
+  int steps = 0;
+  for (int cand : {4, 8, 16})
+    if (!steps && a.K % (64 * cand) == 0 && a.K / (64 * cand) <= 8) steps = cand;
+  if (!steps && a.K % 1024 == 0 && a.K / 1024 <= 16) steps = 16;
+  if (!steps) return TS_BAD_SHAPE;
+  const int nwaves = a.K / (64 * steps);
+  dim3 grid((a.N + 7) / 8), block(nwaves * TS_WAVE);
+  const size_t smem = sizeof(float) * 256 * nwaves;
+  if (steps == 4) gemm_skinny8_kernel<4, 512, OUT><<<grid, block, smem, stream>>>(a);
+  else if (steps == 8) gemm_skinny8_kernel<8, 512, OUT><<<grid, block, smem, stream>>>(a);
+  else if (nwaves <= 8) gemm_skinny8_kernel<16, 512, OUT><<<grid, block, smem, stream>>>(a);
+  else gemm_skinny8_kernel<16, 1024, OUT><<<grid, block, smem, stream>>>(a);
+  return ts_check_launch();
+}
+
+// y [M <= 8, N] = x · W^T by the 8-row form above: K a multiple of 256 up to 8,192 or of 1,024 up to
+// 16,384; contiguous 16-byte aligned rows. out_dtype: 1 bfloat16, 0 float. packed: w is
+// hip.pack_weight8(W) for this K, ldw unused, N a multiple of 8.
+extern "C" int ts_gemm_skinny8_bf16(void* y, const void* x, const void* w, int M, int N, int K, int64_t ldx, int64_t ldw,
+                                    int64_t ldy, int out_dtype, int packed, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return TS_OK;
+  if (M > 8 || K <= 0 || ldx % 8 || ldx < K || ldy < N || (!packed && (ldw % 8 || ldw < K)) || (packed && N % 8)) return TS_BAD_SHAPE;
+  if (((uintptr_t)x | (uintptr_t)w) & 15 || !y) return TS_BAD_SHAPE;
+  SkinnyArgs a = {};
+  a.x = (const bf16_t*)x; a.w = (const bf16_t*)w; a.y = y; a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldw = ldw; a.ldy = ldy;
+  a.packed = packed;
+  if (out_dtype == 1) return sk8_dispatch<bf16_t>(a, stream);
+  if (out_dtype == 0) return sk8_dispatch<float>(a, stream);
+  return TS_BAD_DTYPE;
+}
+
 // mode: 0 plain, 1 residual + RMSNorm on the way in (M <= 16, K in steps of 256 up to 2048). glu: W holds
 // gate rows then up rows, y is [M, N / 2] = silu(gate) * up (M <= 16, K up to 4096, 2048 with the norm). out_dtype: 1 bfloat16, 0 float
 // (plain only). packed: w holds the matrix in the kernel's own order (see the loads of W), ldw is unused. Requires M <= 32, K a multiple of 256 (up to 4096) or of 512 (up to 8192), contiguous

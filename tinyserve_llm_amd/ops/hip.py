@@ -62,6 +62,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_gemm_library_init": [],
         "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, i, i, i, i, p, p, p],
         "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p],
+        "ts_gemm_skinny8_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_gemm_skinny_rope_bf16": [p, p, p, p, p, p, i, i, i64, i64, f, i, i, p, p, p, p, p, i, i, i, i, i, i64, i64, i64,
                                      i64, i64, i64, i64, p],
     }
@@ -635,6 +636,70 @@ def _check_packed(packed: torch.Tensor | None, weight: torch.Tensor) -> None:
               and packed.data_ptr() % 16 == 0, f"the packed copy does not belong to a weight of {n} x {k}")
 
 
+SKINNY8_MAX_ROWS = 8          # rows of x that the 8-row form of the weight-streaming kernel takes
+SKINNY8_MAX_WIDTH = 4096      # widest matrix it is chosen for where the 16-row form would serve as well
+
+
+def skinny8_steps(k: int) -> int:
+    """32-wide k steps per wave of the 8-row form for a reduction of `k` (a wave covers 64 of them per
+    step): the fewest steps that fit 8 waves, else 16 steps in up to 16 waves; 0 if it does not serve k."""
+    for steps in (4, 8, 16):
+        if k % (64 * steps) == 0 and k // (64 * steps) <= 8:
+            return steps
+    return 16 if k % 1024 == 0 and k // 1024 <= 16 else 0
+
+
+def skinny8_takes(rows: int, n: int, k: int) -> bool:
+    """Whether `linear_bf16` gives the product to the 8-row form: at most 8 rows of x, and a matrix
+    narrow enough that 16-row tiles would leave compute units idle, or a reduction too long for them."""
+    return (rows <= SKINNY8_MAX_ROWS and skinny8_steps(k) > 0
+            and (n <= SKINNY8_MAX_WIDTH or not (skinny_takes(rows, k) and k <= 4096)))
+
+
+def pack_weight8(weight: torch.Tensor) -> torch.Tensor:
+    """A copy of bfloat16 `weight` [N, K] in the order the 8-row form reads it:
+    [N / 8 tiles, waves, steps, 64 lanes, 8], lane r + 16 g holding row 8 tile + r % 8 at
+    k = 64 steps wave + 32 steps (r // 8) + 32 step + 8 g .. + 7; rows past N are zeros."""
+    _gpu(weight)
+    _need(weight.dtype == torch.bfloat16 and weight.dim() == 2 and skinny8_steps(weight.shape[1]) > 0,
+          "pack_weight8 takes bfloat16 [N, K] with a K that the 8-row form serves")
+    n, k = weight.shape
+    steps = skinny8_steps(k)
+    waves, tiles = k // (64 * steps), -(-n // 8)
+    padded = weight if n == 8 * tiles else torch.cat([weight, weight.new_zeros(8 * tiles - n, k)])
+    # [tile, row, wave, half, step, g, 8] -> [tile, wave, step, g, half, row, 8]
+    return (padded.view(tiles, 8, waves, 2, steps, 4, 8).permute(0, 2, 4, 5, 3, 1, 6).contiguous()
+            .view(tiles, waves, steps, 64, 8))
+
+
+def gemm_skinny8(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
+                 packed8: torch.Tensor | None = None) -> torch.Tensor:
+    """bfloat16 x [M <= 8, K] · weight [N, K]^T by the weight-streaming kernel's 8-row form (a matrix
+    instruction multiplies 8 rows of W by 8 rows of x over 64 k; a workgroup owns 8 rows of W).
+    With `packed8` (= pack_weight8(weight)) the kernel reads that copy."""
+    _gpu(x, weight, packed8)
+    _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "gemm_skinny8 takes bfloat16")
+    _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
+          f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
+    M, K = x.shape
+    N = weight.shape[0]
+    steps = skinny8_steps(K)
+    _need(M <= SKINNY8_MAX_ROWS and steps > 0, f"gemm_skinny8 takes up to {SKINNY8_MAX_ROWS} rows and K in steps of 256 up to "
+          "8192 or of 1024 up to 16384")
+    _need(x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0,
+          "rows must be contiguous and 16-byte aligned")
+    _need(out_dtype in (torch.bfloat16, torch.float32), "the result is bfloat16 or float32")
+    if packed8 is not None:
+        _need(packed8.dtype == torch.bfloat16 and packed8.shape == (-(-N // 8), K // (64 * steps), steps, 64, 8)
+              and packed8.is_contiguous() and packed8.data_ptr() % 16 == 0 and N % 8 == 0,
+              f"the packed copy does not belong to a weight of {N} x {K}")
+    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    _run("gemm_skinny8", library().ts_gemm_skinny8_bf16(
+        _ptr(out), _ptr(x), _ptr(weight if packed8 is None else packed8), M, N, K, x.stride(0), weight.stride(0),
+        out.stride(0), _code(out_dtype), int(packed8 is not None), _stream()))
+    return out
+
+
 def skinny_fuses(rows: int, k: int, norm: bool, glu: bool) -> bool:
     """Whether the kernel can apply the norm on the way in and/or the gate on the way out."""
     if not (norm or glu):
@@ -789,21 +854,35 @@ def gemm_tiled(x: torch.Tensor, weight: torch.Tensor, glu: bool = False,
     return y
 
 
+class StreamingCopies:
+    """A weight once more in the orders the weight-streaming kernels read it: `by16` for the form
+    with 16-row tiles (`pack_weight`), `by8` for the 8-row form (`pack_weight8`); either may be None."""
+
+    def __init__(self, by16: torch.Tensor | None = None, by8: torch.Tensor | None = None) -> None:
+        self.by16, self.by8 = by16, by8
+
+    def nbytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in (self.by16, self.by8) if t is not None)
+
+
 def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
-                packed: torch.Tensor | None = None) -> torch.Tensor:
-    """bfloat16 x [M, K] · weight [N, K]^T: few rows go to the weight-streaming kernel (which reads
-    `packed`, the weight in its own order, if there is one), many to the vendor matrix library."""
+                packed: StreamingCopies | None = None) -> torch.Tensor:
+    """bfloat16 x [M, K] · weight [N, K]^T: few rows go to the weight-streaming kernels (which read
+    the weight's copy in their own order from `packed`, if there is one), many to the vendor matrix
+    library."""
     _gpu(x, weight)
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "linear_bf16 takes bfloat16")
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
           f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
-    # Measured: reductions longer than 4096 leave the kernel too few workgroups, and with more than 16
-    # rows it only wins on small matrices (8M elements: a layer's qkv and o, not its gate_up or the
+    streams = x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0
+    if streams and skinny8_takes(x.shape[0], weight.shape[0], x.shape[1]):
+        return gemm_skinny8(x, weight, out_dtype, None if packed is None else packed.by8)
+    # Measured: reductions longer than 4096 leave the 16-row kernel too few workgroups, and with more than
+    # 16 rows it only wins on small matrices (8M elements: a layer's qkv and o, not its gate_up or the
     # head); the library streams the rest faster.
-    if (skinny_takes(x.shape[0], x.shape[1]) and x.shape[1] <= 4096
-            and (x.shape[0] <= SKINNY_FUSED_ROWS or weight.numel() <= SKINNY_WIDE_ELEMENTS)
-            and x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
-        return gemm_skinny(x, weight, out_dtype, packed=packed)[0]
+    if (streams and skinny_takes(x.shape[0], x.shape[1]) and x.shape[1] <= 4096
+            and (x.shape[0] <= SKINNY_FUSED_ROWS or weight.numel() <= SKINNY_WIDE_ELEMENTS)):
+        return gemm_skinny(x, weight, out_dtype, packed=None if packed is None else packed.by16)[0]
     # (float32: the 32-bit sums themselves, as the weight-streaming kernel gives them for few rows, so
     # that a row's logits are rounded the same way whatever the number of rows beside it)
     _need(out_dtype in (torch.bfloat16, torch.float32), f"bfloat16 products come out as bfloat16 or float32, not {out_dtype}")

@@ -37,8 +37,8 @@ class Attention(Mixer):
         self.window = window
         self.qkv: torch.Tensor | None = None
         self.o: torch.Tensor | None = None
-        self.qkv_packed: torch.Tensor | None = None
-        self.o_packed: torch.Tensor | None = None
+        self.qkv_packed: hip.StreamingCopies | None = None
+        self.o_packed: hip.StreamingCopies | None = None
 
     @property
     def q_size(self) -> int:
@@ -50,13 +50,14 @@ class Attention(Mixer):
 
     def keep_streaming_copies(self) -> int:
         self.qkv_packed, self.o_packed = streaming_copy(self.qkv), streaming_copy(self.o)
-        return sum(t.numel() * t.element_size() for t in (self.qkv_packed, self.o_packed) if t is not None)
+        return sum(c.nbytes() for c in (self.qkv_packed, self.o_packed) if c is not None)
 
     def _project_fused(self, x, table, positions, slots, k_store, v_store) -> torch.Tensor | None:
         """Projection, rotation and cache write in one kernel where a step is small enough for the
         weight-streaming kernel; None where it is not."""
         d = x if isinstance(x, DeferredNorm) else None
         rows = d.x if d is not None else x
+        by16 = None if self.qkv_packed is None else self.qkv_packed.by16
         if not (rows.is_cuda and hip.qkv_rope_fuses(rows, self.qkv, self.head_dim, k_store)):
             return None
         if d is not None and not (hip.qkv_rope_fuses(rows, self.qkv, self.head_dim, k_store, norm=True)
@@ -65,10 +66,10 @@ class Attention(Mixer):
             rows, d = d.materialize(), None      # the norm by its own kernel, the rest in one
         if d is None:
             return hip.qkv_rope_store(rows, self.qkv, table, positions, slots, k_store, v_store, self.num_heads,
-                                      self.num_kv_heads, self.head_dim, packed=self.qkv_packed)[0]
+                                      self.num_kv_heads, self.head_dim, packed=by16)[0]
         q, d.residual_out = hip.qkv_rope_store(rows, self.qkv, table, positions, slots, k_store, v_store, self.num_heads,
                                                self.num_kv_heads, self.head_dim, residual=d.residual,
-                                               norm_weight=d.weight, eps=d.eps, packed=self.qkv_packed)
+                                               norm_weight=d.weight, eps=d.eps, packed=by16)
         return q
 
     def param_specs(self) -> dict[str, ParamSpec]:

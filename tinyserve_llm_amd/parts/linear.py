@@ -37,33 +37,36 @@ def _streams(x: torch.Tensor, weight: torch.Tensor) -> bool:
             and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
 
 
-def streaming_copy(weight: torch.Tensor) -> torch.Tensor | None:
-    """The weight once more in the order the weight-streaming kernel reads it, for a part to keep
-    beside the weight and hand to `linear` (decode steps read it, steps with many rows read the
-    weight itself through the library); None where that kernel would never take the weight."""
-    if (weight.is_cuda and weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous()
-            and hip.skinny_takes(1, weight.shape[1]) and weight.shape[1] <= 4096):
-        return hip.pack_weight(weight)
-    return None
+def streaming_copy(weight: torch.Tensor) -> hip.StreamingCopies | None:
+    """The weight once more in the orders the weight-streaming kernels read it, for a part to keep
+    beside the weight and hand to `linear` (decode steps read the copies, steps with many rows read
+    the weight itself through the library); None where those kernels would never take the weight."""
+    if not (weight.is_cuda and weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous()):
+        return None
+    n, k = weight.shape
+    by16 = hip.pack_weight(weight) if hip.skinny_takes(1, k) and k <= 4096 else None
+    by8 = hip.pack_weight8(weight) if hip.skinny8_takes(1, n, k) and n % 8 == 0 else None
+    return hip.StreamingCopies(by16, by8) if by16 is not None or by8 is not None else None
 
 
 def linear(x: torch.Tensor | DeferredNorm, weight: torch.Tensor, out_dtype: torch.dtype | None = None,
-           glu: bool = False, packed: torch.Tensor | None = None) -> torch.Tensor:
+           glu: bool = False, packed: hip.StreamingCopies | None = None) -> torch.Tensor:
     """x · Wᵀ; with `glu`, W holds gate rows then up rows and silu(gate) * up comes back.
     `packed` is `streaming_copy(weight)` if the part keeps one."""
+    by16 = None if packed is None else packed.by16
     if isinstance(x, DeferredNorm):
         d = x
         if (out_dtype in (None, torch.bfloat16) and _streams(d.x, weight) and d.weight.dtype == torch.bfloat16
                 and (d.residual is None or d.residual.is_contiguous())
                 and hip.skinny_fuses(d.x.shape[0], weight.shape[1], True, glu) and (not glu or weight.shape[0] % 32 == 0)):
             y, d.residual_out = hip.gemm_skinny(d.x, weight, residual=d.residual, norm_weight=d.weight, eps=d.eps, glu=glu,
-                                                packed=packed)
+                                                packed=by16)
             return y
         x = d.materialize()
     if glu:
         if (out_dtype in (None, torch.bfloat16) and _streams(x, weight) and weight.shape[0] % 32 == 0
                 and hip.skinny_fuses(x.shape[0], weight.shape[1], False, True)):
-            return hip.gemm_skinny(x, weight, glu=True, packed=packed)[0]
+            return hip.gemm_skinny(x, weight, glu=True, packed=by16)[0]
         if (out_dtype in (None, torch.bfloat16) and hip.many_rows_products() == "tiled" and x.is_cuda
                 and hip.tiled_takes(x, weight, glu=True)):
             return hip.gemm_tiled(x, weight, glu=True)

@@ -21,8 +21,8 @@ class GatedMLP(FeedForward):
         self.intermediate_size = intermediate_size
         self.gate_up: torch.Tensor | None = None
         self.down: torch.Tensor | None = None
-        self.gate_up_packed: torch.Tensor | None = None
-        self.down_packed: torch.Tensor | None = None
+        self.gate_up_packed = None       # `streaming_copy` of each weight, if the model keeps them
+        self.down_packed = None
 
     def param_specs(self) -> dict[str, ParamSpec]:
         return {"gate_up": ParamSpec((2 * self.intermediate_size, self.hidden_size)),
@@ -30,7 +30,7 @@ class GatedMLP(FeedForward):
 
     def keep_streaming_copies(self) -> int:
         self.gate_up_packed, self.down_packed = streaming_copy(self.gate_up), streaming_copy(self.down)
-        return sum(t.numel() * t.element_size() for t in (self.gate_up_packed, self.down_packed) if t is not None)
+        return sum(c.nbytes() for c in (self.gate_up_packed, self.down_packed) if c is not None)
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         return linear(linear(x, self.gate_up, glu=True, packed=self.gate_up_packed), self.down, packed=self.down_packed)
