@@ -519,6 +519,27 @@ def test_weight_streaming_gemm_and_its_fused_inputs(m, n, k):
         torch.testing.assert_close(out.double().cpu(), want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
 
 
+@pytest.mark.parametrize("m", [17, 32, 33, 48, 64])
+@pytest.mark.parametrize("n,k", [(16384, 2048), (2048, 2048), (320, 768), (6144, 1024)])
+def test_gate_on_the_way_out_for_up_to_64_rows(m, n, k):
+    """silu(gate) * up straight from the gate|up product for two and four blocks of 16 rows of x,
+    against the product in 64-bit followed by the gate; a row among many equals the row alone."""
+    g = gen(m + n + k)
+    w = (torch.randn(n, k, generator=g) * 0.05).bfloat16().to(dev())
+    x = torch.randn(m, k, generator=g).bfloat16().to(dev())
+    assert hip().skinny_fuses(m, k, False, True) and not hip().skinny_fuses(m, k, True, True)
+    out, _ = hip().gemm_skinny(x, w, glu=True)
+    want = P.silu_mul(x.double().cpu() @ w.double().cpu().T)
+    assert out.shape == (m, n // 2) and out.dtype == torch.bfloat16
+    torch.testing.assert_close(out.double().cpu(), want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
+    alone, _ = hip().gemm_skinny(x[m - 1:].contiguous(), w, glu=True)
+    assert torch.equal(alone[0], out[m - 1])
+    from tinyserve_llm_amd.parts.linear import linear
+    assert torch.equal(linear(x, w, glu=True), out), "the part's projection takes this path"
+    with pytest.raises(hip().KernelError):
+        hip().gemm_skinny(x.repeat(4, 1)[:65].contiguous(), w, glu=True)
+
+
 def test_weight_streaming_gemm_refuses_what_it_cannot_take():
     x = torch.zeros(33, 2048, dtype=torch.bfloat16, device=dev())
     w = torch.zeros(64, 2048, dtype=torch.bfloat16, device=dev())
@@ -629,7 +650,9 @@ def test_several_draws_may_read_one_row_of_logits():
 
 
 @pytest.mark.parametrize("nh,nkv,hd,K,M,page", [(32, 8, 64, 2048, 8, 64), (6, 2, 96, 768, 5, 16), (4, 4, 128, 256, 16, 8),
-                                                 (3, 1, 32, 1280, 1, 32), (24, 8, 128, 3072, 8, 64), (8, 2, 128, 4096, 3, 32)])
+                                                 (3, 1, 32, 1280, 1, 32), (24, 8, 128, 3072, 8, 64), (8, 2, 128, 4096, 3, 32),
+                                                 (32, 8, 64, 2048, 24, 64), (32, 8, 64, 2048, 64, 64), (6, 2, 96, 768, 40, 16),
+                                                 (3, 1, 32, 1280, 33, 32)])
 @pytest.mark.parametrize("norm", [False, True])
 @pytest.mark.parametrize("rotate", [True, False])
 def test_fused_projection_rotation_and_cache_write(nh, nkv, hd, K, M, page, norm, rotate):
@@ -658,10 +681,11 @@ def test_fused_projection_rotation_and_cache_write(nh, nkv, hd, K, M, page, norm
         xn, res_want = hip().rmsnorm(x, nw, 1e-5, res)
     else:
         xn, res_want = x, None
-    qkv = hip().gemm_skinny(xn, w)[0]
+    from tinyserve_llm_amd.parts.linear import linear
+    qkv = linear(xn, w)
     q_want = hip().rope_store(qkv, table, positions, slots, kp1.permute(0, 2, 1, 3), vp1.permute(0, 3, 1, 2), nh, nkv, hd)
     assert hip().qkv_rope_fuses(x, w, hd, kp2.permute(0, 2, 1, 3))
-    if norm and K > 2048:            # the norm rides along only up to 2048; a part runs it by itself beyond
+    if norm and (K > 2048 or M > 16):   # the norm rides along only up to 2048 and 16 rows; a part runs it by itself beyond
         assert not hip().qkv_rope_fuses(x, w, hd, kp2.permute(0, 2, 1, 3), norm=True)
         with pytest.raises(hip().KernelError, match="qkv_rope_store takes"):
             hip().qkv_rope_store(x, w, table, positions, slots, kp2.permute(0, 2, 1, 3), vp2.permute(0, 3, 1, 2),
@@ -703,15 +727,17 @@ def test_fused_projection_rotation_and_cache_write(nh, nkv, hd, K, M, page, norm
 
 
 def test_fused_projection_refuses_what_it_cannot_serve():
-    x = torch.zeros(17, 256, dtype=torch.bfloat16, device=dev())
+    x = torch.zeros(65, 256, dtype=torch.bfloat16, device=dev())
     w = torch.zeros(3 * 64, 256, dtype=torch.bfloat16, device=dev())
-    assert not hip().qkv_rope_fuses(x, w, 64, None), "17 rows"
+    assert hip().qkv_rope_fuses(x[:64], w, 64, None) and not hip().qkv_rope_fuses(x, w, 64, None), "65 rows"
+    assert not hip().qkv_rope_fuses(x[:17], w, 64, None, norm=True), "17 rows with the norm"
+    assert not hip().qkv_rope_fuses(torch.zeros(17, 2304, dtype=torch.bfloat16, device=dev()), w, 64, None), "17 rows over more than 2048"
     assert not hip().qkv_rope_fuses(x[:4], w, 48, None), "head_dim 48"
     assert not hip().qkv_rope_fuses(torch.zeros(4, 4352, dtype=torch.bfloat16, device=dev()), w, 64, None), "K beyond 4096"
     assert not hip().qkv_rope_fuses(torch.zeros(4, 2304, dtype=torch.bfloat16, device=dev()), w, 64, None, norm=True), \
         "K beyond 2048 with the norm"
     with pytest.raises(hip().KernelError, match="qkv_rope_store takes"):
-        hip().qkv_rope_store(x, w, None, torch.zeros(17, dtype=torch.int32, device=dev()), None, None, None, 1, 1, 64)
+        hip().qkv_rope_store(x, w, None, torch.zeros(65, dtype=torch.int32, device=dev()), None, None, None, 1, 1, 64)
 
 
 @pytest.mark.parametrize("heads,kv,hd,page", [(32, 8, 64, 256), (8, 2, 128, 64), (3, 1, 32, 24)])

@@ -93,7 +93,8 @@ gemm_skinny_kernel(const SkinnyArgs a) {
   constexpr bool GLU = EPI == EPI_GLU, ROPE = EPI == EPI_ROPE, PAIRS = EPI != EPI_NONE;
   static_assert(MODE == MODE_PLAIN || CB == 1, "the fused norm serves one block of rows");
   static_assert(!PAIRS || RT % 2 == 0, "gate and up tiles, and the halves of a head, come in pairs");
-  constexpr int SK_XBATCH = (CB == 2 && MAXT > 512) ? 4 : 8;   // steps of x fetched at a time
+  // steps of x fetched at a time: fewer where more blocks of x, more row tiles of W or a larger workgroup leave fewer registers
+  constexpr int SK_XBATCH = CB >= 4 ? 4 : (CB == 2 && (MAXT > 512 || RT >= 4)) ? 4 : 8;
   extern __shared__ __align__(16) float smem[];
   const int nwaves = blockDim.x / TS_WAVE;
   float* part = smem;                                   // [nwaves][RT][CB][256]
@@ -342,12 +343,18 @@ static int sk_dispatch(const SkinnyArgs& a, hipStream_t stream) {
   if (a.K % (steps * SK_KSTEP) || a.K / (steps * SK_KSTEP) > 16) return TS_BAD_SHAPE;
   const int nwaves = a.K / (steps * SK_KSTEP);
   const int cb = (a.M + 15) / 16;
-  if ((MODE == MODE_NORM || GLU) && cb != 1) return TS_BAD_SHAPE;
+  if (MODE == MODE_NORM && cb != 1) return TS_BAD_SHAPE;
   const int ncols = GLU ? a.N / 2 : a.N;
 #define SK_GO(RT, CB, ST) return sk_launch<RT, CB, ST, MODE, GLU, OUT>(a, stream)
   if constexpr (MODE == MODE_NORM || GLU != 0) {
     // the instances that hold x + res or four row tiles need the registers of a workgroup of 8 waves
     if (steps != 8) return TS_BAD_SHAPE;
+    if constexpr (MODE == MODE_PLAIN && GLU != 0) {
+      // the gate for 17 to 64 rows of x: two or four blocks of rows against the same registers of W
+      if (cb > 1 && nwaves > 8) return TS_BAD_SHAPE;
+      if (cb == 2) { if (ncols >= 4096) SK_GO(4, 2, 8); else SK_GO(2, 2, 8); }
+      if (cb > 2) SK_GO(2, 4, 8);
+    }
     if (nwaves <= 8) {
       if (ncols >= 4096 * (GLU ? 1 : 2)) SK_GO(4, 1, 8);
       if (GLU || ncols >= 4096) SK_GO(2, 1, 8);
@@ -470,13 +477,14 @@ extern "C" int ts_gemm_skinny8_bf16(void* y, const void* x, const void* w, int M
 
 // mode: 0 plain, 1 residual + RMSNorm on the way in (M <= 16, K in steps of 256 up to 2048). glu: W holds
 // gate rows then up rows, y is [M, N / 2] = silu(gate) * up (M <= 16, K up to 4096, 2048 with the norm). out_dtype: 1 bfloat16, 0 float
-// (plain only). packed: w holds the matrix in the kernel's own order (see the loads of W), ldw is unused. Requires M <= 32, K a multiple of 256 (up to 4096) or of 512 (up to 8192), contiguous
+// (plain only). packed: w holds the matrix in the kernel's own order (see the loads of W), ldw is unused. Requires M <= 32 (the gate
+// alone: M <= 64 for K up to 2048), K a multiple of 256 (up to 4096) or of 512 (up to 8192), contiguous
 // 16-byte aligned rows; mode 1 takes x, res, res_out as dense [M, K].
 extern "C" int ts_gemm_skinny_bf16(void* y, const void* x, const void* w, const void* res, const void* nw,
                                    void* res_out, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldy,
                                    float eps, int mode, int glu, int out_dtype, int packed, hipStream_t stream) {
   if (M <= 0 || N <= 0) return TS_OK;
-  if (M > 32 || K <= 0 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ldy < (glu ? N / 2 : N)) return TS_BAD_SHAPE;
+  if (M > (glu && mode == MODE_PLAIN ? 64 : 32) || K <= 0 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ldy < (glu ? N / 2 : N)) return TS_BAD_SHAPE;
   if (glu && (N % 2 || (N / 2) % 16)) return TS_BAD_SHAPE;
   if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)res | (uintptr_t)nw | (uintptr_t)res_out) & 15) return TS_BAD_SHAPE;
   if (mode == MODE_NORM && (!nw || (res && !res_out))) return TS_BAD_SHAPE;
@@ -497,8 +505,8 @@ extern "C" int ts_gemm_skinny_bf16(void* y, const void* x, const void* w, const 
 // The qkv projection of an attention layer with the rotation and the cache write on the way out:
 // q_out [M, nh * hd] gets the rotated queries, the rotated keys and the values go to the slots
 // `slots[m]` of the pages (see SkinnyArgs); w is [(nh + 2 nkv) * hd, K]. mode as above. Requires
-// M <= 16, hd a multiple of 32, K a multiple of 256 up to 4096 (2048 with the norm), 8-byte aligned
-// cache strides.
+// M <= 16 (without the norm: M <= 64 for K up to 2048), hd a multiple of 32, K a multiple of 256 up to 4096
+// (2048 with the norm), 8-byte aligned cache strides.
 extern "C" int ts_gemm_skinny_rope_bf16(void* q_out, const void* x, const void* w, const void* res, const void* nw,
                                         void* res_out, int M, int K, int64_t ldx, int64_t ldw, float eps, int mode,
                                         int packed, const float* cos_sin, const int32_t* positions, const int32_t* slots,
@@ -506,7 +514,7 @@ extern "C" int ts_gemm_skinny_rope_bf16(void* q_out, const void* x, const void* 
                                         int page_size, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vs,
                                         int64_t vh, int64_t vd, hipStream_t stream) {
   if (M <= 0) return TS_OK;
-  if (M > 16 || K <= 0 || K % 256 || K / 256 > (mode == MODE_NORM ? 8 : 16) || ldx % 8 || ldw % 8 || ldx < K || ldw < K) return TS_BAD_SHAPE;
+  if (M > (mode == MODE_PLAIN && K <= 2048 ? 64 : 16) || K <= 0 || K % 256 || K / 256 > (mode == MODE_NORM ? 8 : 16) || ldx % 8 || ldw % 8 || ldx < K || ldw < K) return TS_BAD_SHAPE;
   if (nh <= 0 || nkv < 0 || hd <= 0 || hd % 32 || page_size <= 0) return TS_BAD_SHAPE;
   if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)res | (uintptr_t)nw | (uintptr_t)res_out | (uintptr_t)q_out) & 15)
     return TS_BAD_SHAPE;
@@ -520,6 +528,8 @@ extern "C" int ts_gemm_skinny_rope_bf16(void* q_out, const void* x, const void* 
   a.cos_sin = cos_sin; a.positions = positions; a.slots = slots; a.q_out = (bf16_t*)q_out;
   a.k_cache = (bf16_t*)k_cache; a.v_cache = (bf16_t*)v_cache; a.nh = nh; a.nkv = nkv; a.hd = hd; a.rotate = rotate;
   a.page_size = page_size; a.kp = kp; a.ks = ks; a.kh = kh; a.vp = vp; a.vs = vs; a.vh = vh; a.vd = vd;
+  if (mode == MODE_PLAIN && M > 32) return sk_launch<2, 4, 8, MODE_PLAIN, EPI_ROPE, bf16_t>(a, stream);
+  if (mode == MODE_PLAIN && M > 16) return sk_launch<2, 2, 8, MODE_PLAIN, EPI_ROPE, bf16_t>(a, stream);
   if (mode == MODE_PLAIN) return sk_launch<2, 1, 8, MODE_PLAIN, EPI_ROPE, bf16_t>(a, stream);
   if (mode == MODE_NORM) return sk_launch<2, 1, 8, MODE_NORM, EPI_ROPE, bf16_t>(a, stream);
   return TS_BAD_SHAPE;

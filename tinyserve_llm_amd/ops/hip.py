@@ -605,7 +605,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 
 
 SKINNY_MAX_ROWS = 32
-SKINNY_FUSED_ROWS = 16       # the fused norm and the gated epilogue serve one 16-row block of x
+SKINNY_FUSED_ROWS = 16       # the fused norm serves one 16-row block of x,
+SKINNY_EPILOGUE_ROWS = 64    # the gate and the rotation on the way out up to four (for reductions up to 2048)
 SKINNY_WIDE_ELEMENTS = 8 << 20   # largest matrix that `linear_bf16` gives the kernel with 17 to 32 rows
 
 
@@ -704,7 +705,11 @@ def skinny_fuses(rows: int, k: int, norm: bool, glu: bool) -> bool:
     """Whether the kernel can apply the norm on the way in and/or the gate on the way out."""
     if not (norm or glu):
         return skinny_takes(rows, k)
-    return rows <= SKINNY_FUSED_ROWS and k % 256 == 0 and k // 256 <= (8 if norm else 16)
+    if k % 256:
+        return False
+    if norm or rows <= SKINNY_FUSED_ROWS:
+        return rows <= SKINNY_FUSED_ROWS and k // 256 <= (8 if norm else 16)
+    return rows <= SKINNY_EPILOGUE_ROWS and k // 256 <= 8
 
 
 def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, *,
@@ -722,8 +727,8 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     N = weight.shape[0]
     norm = norm_weight is not None
     _need(skinny_fuses(M, K, norm, glu),
-          f"gemm_skinny takes up to {SKINNY_MAX_ROWS} rows ({SKINNY_FUSED_ROWS} when fused) and K in steps of 256 up to "
-          "4096 (2048 with the norm) or of 512 up to 8192")
+          f"gemm_skinny takes up to {SKINNY_MAX_ROWS} rows ({SKINNY_FUSED_ROWS} with the norm, {SKINNY_EPILOGUE_ROWS} with the gate alone "
+          "over up to 2048) and K in steps of 256 up to 4096 (2048 with the norm) or of 512 up to 8192")
     _need(x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0,
           "rows must be contiguous and 16-byte aligned")
     _need(not glu or (N % 32 == 0), "gate and up rows come in whole 16-row tiles")
@@ -754,7 +759,9 @@ def qkv_rope_fuses(x: torch.Tensor, weight: torch.Tensor, head_dim: int, k_cache
     """Whether `qkv_rope_store` serves these operands: few bfloat16 rows, a reduction of up to 4096 in
     steps of 256 (2048 with the norm on the way in), heads of a multiple of 32 dimensions, keys whose
     strides allow 8-byte stores."""
-    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.dim() == 2 and x.shape[0] <= SKINNY_FUSED_ROWS
+    rows_ok = (x.dim() == 2 and (x.shape[0] <= SKINNY_FUSED_ROWS
+                                 or (not norm and x.shape[0] <= SKINNY_EPILOGUE_ROWS and x.shape[1] <= 2048)))
+    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and rows_ok
             and x.shape[1] % 256 == 0 and x.shape[1] // 256 <= (8 if norm else 16) and head_dim % 32 == 0
             and x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0
             and (k_cache is None or (all(st % 4 == 0 for st in k_cache.stride()[:3]) and k_cache.data_ptr() % 8 == 0)))
@@ -771,7 +778,8 @@ def qkv_rope_store(x: torch.Tensor, weight: torch.Tensor, cos_sin: torch.Tensor 
     With `packed` (= pack_weight(weight)) the kernel reads that copy."""
     _gpu(x, weight, cos_sin, positions, slots, k_cache, v_cache, residual, norm_weight)
     _need(qkv_rope_fuses(x, weight, head_dim, k_cache, norm_weight is not None),
-          "qkv_rope_store takes up to 16 bfloat16 rows, K in steps of 256 up to 4096 (2048 with the norm), head_dim in steps of 32")
+          "qkv_rope_store takes up to 16 bfloat16 rows (64 over up to 2048 without the norm), K in steps of 256 up to 4096 "
+          "(2048 with the norm), head_dim in steps of 32")
     M, K = x.shape
     _need(weight.shape == ((num_heads + 2 * num_kv_heads) * head_dim, K), f"weight {tuple(weight.shape)} for "
           f"{num_heads}+2x{num_kv_heads} heads of {head_dim} over {K}")
