@@ -378,7 +378,7 @@ def test_streaming_copies_of_the_weights_change_nothing(tmp_path):
         llm = LLM(str(tmp_path), sc, CacheConfig(block_size=16), dtype=torch.bfloat16, num_blocks=60, seed=2,
                   keep_streaming_copies=keep)
         mixer, ff = llm.model.layers[0].mixer, llm.model.layers[0].feed_forward
-        assert (mixer.qkv_packed is not None) == keep and (mixer.o_packed is not None) == keep
+        assert (mixer.qkv_rope_packed is not None) == keep and (mixer.o_packed is not None) == keep
         assert (ff.gate_up_packed is not None) == keep and (ff.down_packed is not None) == keep
         outs.append([r.token_ids for r in llm.generate(prompts, SamplingParams(max_tokens=10, temperature=0.7, ignore_eos=True))])
     assert outs[0] == outs[1]

@@ -919,7 +919,7 @@ def test_fused_projection_reads_the_packed_copy_to_the_same_result():
     positions = torch.randint(0, 64, (M,), generator=g, dtype=torch.int32).to(dev())
     slots = torch.randperm(4 * page, generator=g)[:M].to(torch.int32).to(dev())
     outs = []
-    for packed in (None, hip().pack_weight(w)):
+    for packed in (None, hip().pack_weight_rope(w, hd)):
         kp = torch.zeros(4, nkv, page, hd, dtype=torch.bfloat16, device=dev())
         vp = torch.zeros(4, nkv, hd, page, dtype=torch.bfloat16, device=dev())
         q, _ = hip().qkv_rope_store(x, w, table, positions, slots, kp.permute(0, 2, 1, 3), vp.permute(0, 3, 1, 2),

@@ -15,8 +15,10 @@
 //              T(x + res) as the new residual
 //   EPI_GLU    W = [gate rows | up rows]; a workgroup takes matching rows of both and writes
 //              silu(gate) * up, y being [M, N / 2]
-//   EPI_ROPE   W = [q heads | k heads | v heads] of head_dim columns each; a workgroup takes 16
-//              columns of the first half of a head and the 16 that rotate with them, rounds the
+//   EPI_ROPE   W = [q heads | k heads | v heads] of head_dim columns each; a 16-row tile holds 8
+//              columns of the first half of a head (matrix rows r < 8) and the 8 that rotate with
+//              them (rows r >= 8: head_dim / 2 further on), so a workgroup of one tile has both
+//              halves of a rotation and a matrix of 3,072 columns gives 192 workgroups; it rounds the
 //              products as y would hold them, rotates q and k by the token's position, and writes q
 //              to its own tensor and k and v into their cache slots: y itself is never stored
 #include "common.h"
@@ -92,7 +94,7 @@ __global__ void __launch_bounds__(MAXT)
 gemm_skinny_kernel(const SkinnyArgs a) {
   constexpr bool GLU = EPI == EPI_GLU, ROPE = EPI == EPI_ROPE, PAIRS = EPI != EPI_NONE;
   static_assert(MODE == MODE_PLAIN || CB == 1, "the fused norm serves one block of rows");
-  static_assert(!PAIRS || RT % 2 == 0, "gate and up tiles, and the halves of a head, come in pairs");
+  static_assert(!GLU || RT % 2 == 0, "gate and up tiles come in pairs");
   // steps of x fetched at a time: fewer where more blocks of x, more row tiles of W or a larger workgroup leave fewer registers
   constexpr int SK_XBATCH = CB >= 4 ? 4 : (CB == 2 && (MAXT > 512 || RT >= 4)) ? 4 : 8;
   extern __shared__ __align__(16) float smem[];
@@ -102,9 +104,9 @@ gemm_skinny_kernel(const SkinnyArgs a) {
   const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
   // GLU: tiles 0 .. RT/2-1 are gate rows n0 + 16 t, tiles RT/2 .. RT-1 the up rows N/2 below them.
-  // ROPE: tiles 0 .. RT/2-1 are 16-row blocks of first halves of heads (block j of the matrix: head
-  // j / (hd / 32), rows 16 (j % (hd / 32)) of it), tiles RT/2 .. RT-1 the rows hd / 2 below them.
-  constexpr int OT = PAIRS ? RT / 2 : RT;               // 16-column tiles of the output per workgroup
+  // ROPE: tile j of the matrix holds rows 8 (j % (hd / 16)) .. + 7 of head j / (hd / 16) in its rows
+  // r < 8 and the rows hd / 2 below them in its rows r >= 8.
+  constexpr int OT = GLU ? RT / 2 : RT;                 // 16-column tiles of the output per workgroup
   const int n0 = blockIdx.x * 16 * OT;
   const int half = a.N / 2;
   const int kbeg = wave * STEPS * SK_KSTEP + 8 * g;     // this lane's first k
@@ -144,15 +146,15 @@ gemm_skinny_kernel(const SkinnyArgs a) {
     int n = GLU ? (t < OT ? n0 + t * 16 + r : half + n0 + (t - OT) * 16 + r) : n0 + t * 16 + r;
     int limit = GLU ? (t < OT ? half : a.N) : a.N;
     if (ROPE) {
-      const int per_head = a.hd / 32, j = blockIdx.x * OT + (t < OT ? t : t - OT);
-      n = (j / per_head) * a.hd + 16 * (j % per_head) + (t < OT ? 0 : a.hd / 2) + r;
+      const int per_head = a.hd / 16, j = blockIdx.x * RT + t;
+      n = (j / per_head) * a.hd + 8 * (j % per_head) + (r & 7) + (r >> 3) * (a.hd / 2);
       limit = a.N;
     }
     if (a.packed) {
       // W in 1 KB blocks [16-row tile][32-wide k step][lane][8 k]: one load of a wave is one
       // contiguous kilobyte and a wave's slice of a tile a contiguous run of them (rows past N are
       // zeros in the last tile; tiles past the last are computed from it and not stored)
-      int tile_n = (n - r) / 16;
+      int tile_n = ROPE ? blockIdx.x * RT + t : (n - r) / 16;   // (ROPE: the packed copy holds the tiles as described above)
       const int last = (a.N - 1) / 16;
       if (tile_n > last) tile_n = last;
       const bf16_t* wblk = a.w + (((int64_t)tile_n * (a.K / SK_KSTEP) + (int64_t)wave * STEPS) * 64 + lane) * 8;
@@ -240,10 +242,12 @@ gemm_skinny_kernel(const SkinnyArgs a) {
   // part[.][t][b][m_local * 16 + n_local]: a thread sums 4 consecutive n of one m over the waves in order
   OUT* y = (OUT*)a.y;
   const int ncols = GLU ? half : a.N;
-  for (int idx = threadIdx.x; idx < OT * CB * 64; idx += blockDim.x) {
-    const int tile = idx >> 6, e = idx & 63;
+  // ROPE: a tile gives 8 columns of a head's first half (n_local 0 .. 7) and their partners (n_local 8 .. 15): 32 items of 4
+  constexpr int PER_TILE = ROPE ? 32 : 64;
+  for (int idx = threadIdx.x; idx < OT * CB * PER_TILE; idx += blockDim.x) {
+    const int tile = idx / PER_TILE, e = idx - tile * PER_TILE;
     const int t = tile / CB, b = tile - t * CB;
-    const int ml = e >> 2, nl = (e & 3) * 4;
+    const int ml = ROPE ? e >> 1 : e >> 2, nl = ROPE ? (e & 1) * 4 : (e & 3) * 4;
     const int m = b * 16 + ml, n = n0 + t * 16 + nl;
     if (m >= a.M) continue;
     float s[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
@@ -252,7 +256,7 @@ gemm_skinny_kernel(const SkinnyArgs a) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) s[j] += p[j];
       if (PAIRS) {
-        const float* pu = part + (((size_t)wv * RT + t + OT) * CB + b) * 256 + ml * 16 + nl;
+        const float* pu = ROPE ? p + 8 : part + (((size_t)wv * RT + t + OT) * CB + b) * 256 + ml * 16 + nl;
 #pragma unroll
         for (int j = 0; j < 4; ++j) u[j] += pu[j];
       }
@@ -265,8 +269,8 @@ gemm_skinny_kernel(const SkinnyArgs a) {
       for (int j = 0; j < 4; ++j) { s[j] *= inv; u[j] *= inv; }
     }
     if (ROPE) {
-      const int per_head = a.hd / 32, jb = blockIdx.x * OT + t, hdh = a.hd / 2;
-      const int head = jb / per_head, d0 = 16 * (jb % per_head) + nl;   // d0 .. d0 + 3 of the head's first half
+      const int per_head = a.hd / 16, jb = blockIdx.x * RT + t, hdh = a.hd / 2;
+      const int head = jb / per_head, d0 = 8 * (jb % per_head) + nl;    // d0 .. d0 + 3 of the head's first half
       if (head >= a.nh + 2 * a.nkv) continue;
       float y1[4], y2[4];
 #pragma unroll
@@ -320,8 +324,8 @@ template <int RT, int CB, int STEPS, int MODE, int GLU, typename OUT>
 static int sk_launch(const SkinnyArgs& a, hipStream_t stream) {
   const int nwaves = a.K / (STEPS * SK_KSTEP);
   const size_t smem = sizeof(float) * ((size_t)nwaves * RT * CB * 256 + (size_t)nwaves * 16);
-  constexpr int OT = GLU != EPI_NONE ? RT / 2 : RT;
-  const int ncols = GLU != EPI_NONE ? a.N / 2 : a.N;    // EPI_ROPE: the first halves of all heads
+  constexpr int OT = GLU == EPI_GLU ? RT / 2 : RT;
+  const int ncols = GLU == EPI_GLU ? a.N / 2 : a.N;     // (EPI_ROPE: a 16-row tile of the matrix per 8 columns and their partners)
   dim3 grid((ncols + 16 * OT - 1) / (16 * OT)), block(nwaves * TS_WAVE);
   if (nwaves <= 8) {
     gemm_skinny_kernel<RT, CB, STEPS, MODE, GLU, 512, OUT><<<grid, block, smem, stream>>>(a);
@@ -528,9 +532,9 @@ extern "C" int ts_gemm_skinny_rope_bf16(void* q_out, const void* x, const void* 
   a.cos_sin = cos_sin; a.positions = positions; a.slots = slots; a.q_out = (bf16_t*)q_out;
   a.k_cache = (bf16_t*)k_cache; a.v_cache = (bf16_t*)v_cache; a.nh = nh; a.nkv = nkv; a.hd = hd; a.rotate = rotate;
   a.page_size = page_size; a.kp = kp; a.ks = ks; a.kh = kh; a.vp = vp; a.vs = vs; a.vh = vh; a.vd = vd;
-  if (mode == MODE_PLAIN && M > 32) return sk_launch<2, 4, 8, MODE_PLAIN, EPI_ROPE, bf16_t>(a, stream);
-  if (mode == MODE_PLAIN && M > 16) return sk_launch<2, 2, 8, MODE_PLAIN, EPI_ROPE, bf16_t>(a, stream);
-  if (mode == MODE_PLAIN) return sk_launch<2, 1, 8, MODE_PLAIN, EPI_ROPE, bf16_t>(a, stream);
-  if (mode == MODE_NORM) return sk_launch<2, 1, 8, MODE_NORM, EPI_ROPE, bf16_t>(a, stream);
+  if (mode == MODE_PLAIN && M > 32) return sk_launch<1, 4, 8, MODE_PLAIN, EPI_ROPE, bf16_t>(a, stream);
+  if (mode == MODE_PLAIN && M > 16) return sk_launch<1, 2, 8, MODE_PLAIN, EPI_ROPE, bf16_t>(a, stream);
+  if (mode == MODE_PLAIN) return sk_launch<1, 1, 8, MODE_PLAIN, EPI_ROPE, bf16_t>(a, stream);
+  if (mode == MODE_NORM) return sk_launch<1, 1, 8, MODE_NORM, EPI_ROPE, bf16_t>(a, stream);
   return TS_BAD_SHAPE;
 }

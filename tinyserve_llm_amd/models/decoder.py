@@ -13,7 +13,7 @@ from tinyserve_llm_amd.ops import hip
 from tinyserve_llm_amd.parts import base
 from tinyserve_llm_amd.parts.base import KVSpec, LayerMemory, ParamSpec, StateSpec, StepContext
 from tinyserve_llm_amd.parts.block import Layer
-from tinyserve_llm_amd.parts.linear import linear
+from tinyserve_llm_amd.parts.linear import linear, streaming_copy
 
 
 @dataclass(frozen=True)
@@ -46,6 +46,7 @@ class DecoderModel:
                                    for name, ps in spec.position_encodings.items()}
         self.embed: torch.Tensor | None = None
         self.head: torch.Tensor | None = None
+        self.head_packed = None                  # `streaming_copy` of the head, if the model keeps them
         self.dtype: torch.dtype | None = None
         self.device: torch.device | None = None
         self._check_order()
@@ -126,8 +127,11 @@ class DecoderModel:
 
     def keep_streaming_copies(self) -> int:
         """Lets every part of every layer keep its weights once more in a decode kernel's reading
-        order; returns the bytes that takes."""
-        return sum(part.keep_streaming_copies() for layer in self.layers for part in layer.parts().values())
+        order, and keeps the head's (a step reads the whole vocabulary matrix once whatever its
+        size: at the 1B sizes a fifth of a decode step's bytes); returns the bytes that takes."""
+        self.head_packed = streaming_copy(self.head)
+        own = 0 if self.head_packed is None else self.head_packed.nbytes()
+        return own + sum(part.keep_streaming_copies() for layer in self.layers for part in layer.parts().values())
 
     # ---- one step ----------------------------------------------------------------------------
     def forward(self, ctx: StepContext, memory: list[LayerMemory]) -> tuple[torch.Tensor, torch.Tensor | None]:
@@ -147,4 +151,4 @@ class DecoderModel:
         """float32 logits [len(rows), vocab] at the wanted rows only: the final norm and the
         vocabulary projection touch no other row (tinyserve_llm/engine/model_runner.py:125-127)."""
         normed, _ = self.final_norm(hidden, residual, rows)
-        return linear(normed, self.head, out_dtype=torch.float32)
+        return linear(normed, self.head, out_dtype=torch.float32, packed=self.head_packed)

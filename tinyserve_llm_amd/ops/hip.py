@@ -629,6 +629,19 @@ def pack_weight(weight: torch.Tensor) -> torch.Tensor:
     return padded.view(tiles, 16, k // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(tiles, k // 32, 64, 8)
 
 
+def pack_weight_rope(weight: torch.Tensor, head_dim: int) -> torch.Tensor:
+    """A copy of a fused q|k|v weight [heads * head_dim, K] in the order `qkv_rope_store` reads it:
+    `pack_weight` of the matrix with its rows regrouped so that a 16-row tile holds 8 rows of the first
+    half of a head and, below them, the 8 rows that rotate with them (head_dim / 2 further on)."""
+    _gpu(weight)
+    _need(weight.dim() == 2 and head_dim % 16 == 0 and weight.shape[0] % head_dim == 0,
+          "pack_weight_rope takes [heads * head_dim, K] with head_dim a multiple of 16")
+    heads, half = weight.shape[0] // head_dim, head_dim // 2
+    # [head, half (0: first, 1: second), block of 8, row] -> [head, block, half, row]
+    regrouped = weight.view(heads, 2, half // 8, 8, weight.shape[1]).permute(0, 2, 1, 3, 4).reshape(weight.shape)
+    return pack_weight(regrouped)
+
+
 def _check_packed(packed: torch.Tensor | None, weight: torch.Tensor) -> None:
     if packed is not None:
         n, k = weight.shape
@@ -775,7 +788,7 @@ def qkv_rope_store(x: torch.Tensor, weight: torch.Tensor, cos_sin: torch.Tensor 
     """`rope_store(f(x) · weight^T, ...)` in one kernel for few rows of x: the projection is never
     stored, q [tokens, nh, hd] comes back rotated, rotated k and v go to their cache slots. With
     `norm_weight`, f = RMSNorm(x + residual) * norm_weight and x + residual is the second result.
-    With `packed` (= pack_weight(weight)) the kernel reads that copy."""
+    With `packed` (= pack_weight_rope(weight, head_dim)) the kernel reads that copy."""
     _gpu(x, weight, cos_sin, positions, slots, k_cache, v_cache, residual, norm_weight)
     _need(qkv_rope_fuses(x, weight, head_dim, k_cache, norm_weight is not None),
           "qkv_rope_store takes up to 16 bfloat16 rows (64 over up to 2048 without the norm), K in steps of 256 up to 4096 "

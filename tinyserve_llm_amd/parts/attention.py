@@ -38,6 +38,7 @@ class Attention(Mixer):
         self.qkv: torch.Tensor | None = None
         self.o: torch.Tensor | None = None
         self.qkv_packed: hip.StreamingCopies | None = None
+        self.qkv_rope_packed: torch.Tensor | None = None     # for the one-kernel path: `hip.pack_weight_rope`
         self.o_packed: hip.StreamingCopies | None = None
 
     @property
@@ -50,14 +51,19 @@ class Attention(Mixer):
 
     def keep_streaming_copies(self) -> int:
         self.qkv_packed, self.o_packed = streaming_copy(self.qkv), streaming_copy(self.o)
-        return sum(c.nbytes() for c in (self.qkv_packed, self.o_packed) if c is not None)
+        if self.qkv_packed is not None and self.qkv_packed.by16 is not None and self.head_dim % 32 == 0:
+            self.qkv_rope_packed = hip.pack_weight_rope(self.qkv, self.head_dim)
+            if self.hidden_size <= 2048:
+                self.qkv_packed = None           # every step that would stream the plain copy takes the one-kernel path
+        copies = sum(c.nbytes() for c in (self.qkv_packed, self.o_packed) if c is not None)
+        return copies + (0 if self.qkv_rope_packed is None else self.qkv_rope_packed.numel() * 2)
 
     def _project_fused(self, x, table, positions, slots, k_store, v_store) -> torch.Tensor | None:
         """Projection, rotation and cache write in one kernel where a step is small enough for the
         weight-streaming kernel; None where it is not."""
         d = x if isinstance(x, DeferredNorm) else None
         rows = d.x if d is not None else x
-        by16 = None if self.qkv_packed is None else self.qkv_packed.by16
+        by16 = self.qkv_rope_packed
         if not (rows.is_cuda and hip.qkv_rope_fuses(rows, self.qkv, self.head_dim, k_store)):
             return None
         if d is not None and not (hip.qkv_rope_fuses(rows, self.qkv, self.head_dim, k_store, norm=True)
