@@ -208,8 +208,8 @@ def toy_spec(hidden=48, vocab=97, mean_mixer="toy_running_mean"):
     norm = PartSpec("rmsnorm", dict(hidden_size=hidden, eps=1e-5))
     mlp = PartSpec("gated_mlp", dict(hidden_size=hidden, intermediate_size=64))
     attn = PartSpec("attention", dict(hidden_size=hidden, num_heads=3, num_kv_heads=1, head_dim=16, position=None))
-    layers = [LayerSpec(PartSpec(mean_mixer, dict(hidden_size=hidden)), mlp, norm, norm),
-              LayerSpec(attn, PartSpec("toy_routed", dict(hidden_size=hidden, experts=3)), norm, norm)]
+    layers = [LayerSpec.pre_norm(PartSpec(mean_mixer, dict(hidden_size=hidden)), mlp, norm, norm),
+              LayerSpec.pre_norm(attn, PartSpec("toy_routed", dict(hidden_size=hidden, experts=3)), norm, norm)]
     return ModelSpec(architecture="Toy", vocab_size=vocab, hidden_size=hidden, max_position=128, layers=layers,
                      order=[LayerRun(0), LayerRun(1), LayerRun(0)], final_norm=norm,
                      position_encodings={"learned": PartSpec("toy_learned", dict(hidden_size=hidden, max_position=128))},
@@ -345,7 +345,7 @@ def test_a_layer_can_read_another_layers_cache():
     from tinyserve_llm_amd.weights.random_init import random_params
     hidden = 32
     norm = PartSpec("rmsnorm", dict(hidden_size=hidden, eps=1e-5))
-    layer = LayerSpec(PartSpec("attention", dict(hidden_size=hidden, num_heads=2, num_kv_heads=2, head_dim=16, position=None)),
+    layer = LayerSpec.pre_norm(PartSpec("attention", dict(hidden_size=hidden, num_heads=2, num_kv_heads=2, head_dim=16, position=None)),
                       PartSpec("gated_mlp", dict(hidden_size=hidden, intermediate_size=48)), norm, norm)
     spec = ModelSpec("Toy2", 50, hidden, 64, [layer, layer], [LayerRun(0), LayerRun(1, cache=0, store=False)], norm,
                      tie_word_embeddings=True)
@@ -394,7 +394,97 @@ def test_bad_orders_are_refused_when_the_model_is_built():
     spec.order = [LayerRun(1, store=False)]
     with pytest.raises(ValueError, match="neither owns"):
         DecoderModel(spec)
-    spec.layers[1] = spec.layers[1].__class__(spec.layers[1].mixer.__class__("no_such_mixer", {}), spec.layers[1].feed_forward,
-                                              spec.layers[1].mixer_norm, spec.layers[1].ff_norm)
+    from dataclasses import replace
+    from tinyserve_llm_amd.parts.base import PartSpec
+    spec.order = [LayerRun(0), LayerRun(1)]
+    good = spec.layers[1]
+    spec.layers[1] = replace(good, mixer=PartSpec("no_such_mixer", {}))
     with pytest.raises(KeyError, match="no mixer named"):
         DecoderModel(spec)
+    spec.layers[1] = replace(good, norms={"mixer_norm": good.norms["mixer_norm"]})
+    with pytest.raises(KeyError, match=r"asks for the norms \['ff_norm'\]"):
+        DecoderModel(spec)
+    spec.layers[1] = replace(good, block="no_such_block")
+    with pytest.raises(KeyError, match="no block arrangement"):
+        DecoderModel(spec)
+
+
+def test_another_block_arrangement_another_embedding_and_another_head():
+    """Parts of the kinds the built-in model has one of each, defined here: a block that runs mixer and
+    feed-forward side by side from one norm and normalises each branch again on the way out (three
+    norms under names of its own), an embedding that scales its rows, and a head that caps its
+    logits. They are registered, named in a model description, built, bound to random weights and
+    stepped in portions through the unchanged framework, against the same model written out plainly."""
+    from tinyserve_llm_amd.engine.interface import build_cache
+    from tinyserve_llm_amd.engine.runner import ModelRunner, StepEntry
+    from tinyserve_llm_amd.models.decoder import DecoderModel
+    from tinyserve_llm_amd.models.spec import LayerRun, LayerSpec, ModelSpec
+    from tinyserve_llm_amd.parts.base import Embedding, Head, ParamSpec, PartSpec, register
+    from tinyserve_llm_amd.parts.block import uses_norms
+    from tinyserve_llm_amd.weights.random_init import random_params
+
+    @register("block", "toy_side_by_side")
+    @uses_norms("in_norm", "mixer_out_norm", "ff_out_norm")
+    def side_by_side(layer, hidden, residual, ctx, mem):
+        x, stream = layer.norms["in_norm"](hidden, residual)               # (norm(h), h) with h = hidden + residual
+        a, _ = layer.norms["mixer_out_norm"](layer.mixer.forward(x, ctx, mem))
+        b, _ = layer.norms["ff_out_norm"](layer.feed_forward.forward(x, ctx))
+        return a + b, stream
+
+    @register("embedding", "toy_scaled")
+    class Scaled(Embedding):
+        def __init__(self, vocab_size, hidden_size, scale):
+            self.vocab_size, self.hidden_size, self.scale = vocab_size, hidden_size, scale
+
+        def param_specs(self):
+            return {"rows": ParamSpec((self.vocab_size, self.hidden_size), init=(0.0, 0.3))}
+
+        def forward(self, ctx):
+            return self.rows[ctx.token_ids.long()] * self.scale
+
+    @register("head", "toy_capped")
+    class Capped(Head):
+        def __init__(self, vocab_size, hidden_size, cap):
+            self.vocab_size, self.hidden_size, self.cap = vocab_size, hidden_size, cap
+
+        def param_specs(self):
+            return {"w": ParamSpec((self.vocab_size, self.hidden_size), init=(0.0, 0.5))}
+
+        def forward(self, rows):
+            return self.cap * torch.tanh((rows.float() @ self.w.float().T) / self.cap)
+
+    hidden, vocab = 32, 61
+    norm = PartSpec("rmsnorm", dict(hidden_size=hidden, eps=1e-6))
+    layer = LayerSpec(PartSpec("attention", dict(hidden_size=hidden, num_heads=2, num_kv_heads=1, head_dim=16, position=None)),
+                      PartSpec("gated_mlp", dict(hidden_size=hidden, intermediate_size=48)),
+                      {"in_norm": norm, "mixer_out_norm": norm, "ff_out_norm": norm}, block="toy_side_by_side")
+    spec = ModelSpec("Toy3", vocab, hidden, 64, [layer, layer], [LayerRun(0), LayerRun(1)], norm,
+                     embedding=PartSpec("toy_scaled", dict(vocab_size=vocab, hidden_size=hidden, scale=2.5)),
+                     head=PartSpec("toy_capped", dict(vocab_size=vocab, hidden_size=hidden, cap=3.0)))
+    model = DecoderModel(spec)
+    assert sorted(n for n in model.param_specs() if n.startswith("layers.0.") and "norm" in n) == [
+        "layers.0.ff_out_norm.weight", "layers.0.in_norm.weight", "layers.0.mixer_out_norm.weight"]
+    assert "embed.rows" in model.param_specs() and "head.w" in model.param_specs() and not model.graph_safe()
+    params = random_params(model, 8, torch.float32, "cpu")
+    model.bind({k: v.to(DEV) for k, v in params.items()}, torch.float32, torch.device(DEV))
+    p = {k: v.double() for k, v in params.items()}
+    ids = [4, 9, 33, 2, 17, 8, 40, 60, 0]
+    n = len(ids)
+    h = p["embed.rows"][torch.tensor(ids)] * 2.5
+    for i in range(2):
+        w = lambda name: p[f"layers.{i}.{name}"]
+        x = P.rms_norm(h, w("in_norm.weight"), 1e-6)
+        qkv = x @ w("mixer.qkv").T
+        attn = P.causal_attention(qkv[:, :32].reshape(n, 2, 16), qkv[:, 32:48].reshape(n, 1, 16), qkv[:, 48:].reshape(n, 1, 16))
+        a = P.rms_norm(attn.reshape(n, 32) @ w("mixer.o").T, w("mixer_out_norm.weight"), 1e-6)
+        b = P.rms_norm(P.silu_mul(x @ w("ff.gate_up").T) @ w("ff.down").T, w("ff_out_norm.weight"), 1e-6)
+        h = h + a + b
+    want = 3.0 * torch.tanh((P.rms_norm(h, p["final_norm.weight"], 1e-6) @ p["head.w"].T) / 3.0)
+    storage, manager = build_cache(model, 8, 4, torch.float32, DEV, num_state_slots=2)
+    runner = ModelRunner(model, storage, manager)
+    manager.allocate(0, ids[:6])
+    first = runner.step([StepEntry(0, ids[:6], 0, list(range(6)))])
+    manager.commit(0, 6)
+    manager.append_slots(0, ids[6:])
+    rest = runner.step([StepEntry(0, ids[6:], 6, [0, 1, 2])])
+    torch.testing.assert_close(torch.cat([first, rest]).double().cpu(), want, rtol=1e-4, atol=1e-5)

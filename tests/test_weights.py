@@ -107,3 +107,51 @@ def test_stored_types_are_kept_in_the_file(tmp_path):
     write_random_model(str(tmp_path), TINY_A, 0, torch.float32)
     with safe_open(str(tmp_path / "model.safetensors"), "pt", "cpu") as f:
         assert f.get_tensor("model.norm.weight").dtype == torch.float32
+
+
+def test_destinations_slice_columns_transpose_and_fill_stacks(tmp_path):
+    """What a checkpoint table can say beyond rows: a tensor may land in a column range, in one
+    matrix of a stacked parameter, or transposed; wrong shapes are reported in the checkpoint's own
+    orientation, and the random-weights mode writes the same tensors back out."""
+    import torch
+    from safetensors.torch import save_file
+    from tinyserve_llm_amd.models.decoder import DecoderModel
+    from tinyserve_llm_amd.models.spec import Destination, LayerRun, LayerSpec, ModelSpec
+    from tinyserve_llm_amd.parts.base import FeedForward, ParamSpec, PartSpec, register
+    from tinyserve_llm_amd.weights.loader import WeightsError, load_params
+    from tinyserve_llm_amd.weights.random_init import checkpoint_tensors, random_params
+
+    @register("feed_forward", "toy_stacked")
+    class Stacked(FeedForward):
+        def __init__(self, hidden_size, experts):
+            self.hidden_size, self.experts = hidden_size, experts
+
+        def param_specs(self):
+            return {"w": ParamSpec((self.experts, self.hidden_size, self.hidden_size)),
+                    "wide": ParamSpec((self.hidden_size, 3 * self.hidden_size))}
+
+    h = 8
+    norm = PartSpec("rmsnorm", dict(hidden_size=h, eps=1e-5))
+    layer = LayerSpec.pre_norm(PartSpec("attention", dict(hidden_size=h, num_heads=1, num_kv_heads=1, head_dim=16)),
+                               PartSpec("toy_stacked", dict(hidden_size=h, experts=2)), norm, norm)
+    table = {"emb": Destination("embed.weight"), "n0": Destination("layers.0.mixer_norm.weight"),
+             "n1": Destination("layers.0.ff_norm.weight"), "nf": Destination("final_norm.weight"),
+             "qkv": Destination("layers.0.mixer.qkv"), "o_t": Destination("layers.0.mixer.o", transpose=True),
+             "e0": Destination("layers.0.ff.w", index=(0,)), "e1_t": Destination("layers.0.ff.w", index=(1,), transpose=True),
+             "left": Destination("layers.0.ff.wide", col=0, cols=h), "right": Destination("layers.0.ff.wide", col=h, cols=2 * h)}
+    spec = ModelSpec("ToyW", 20, h, 32, [layer], [LayerRun(0)], norm, tie_word_embeddings=True, checkpoint=table,
+                     position_encodings={"rope": PartSpec("rope", dict(head_dim=16, max_position=32, theta=10000.0))})
+    model = DecoderModel(spec)
+    params = random_params(model, 1, torch.float32)
+    tensors = checkpoint_tensors(model, params)
+    assert tensors["o_t"].shape == (16, h) and tensors["e1_t"].shape == (h, h) and tensors["right"].shape == (h, 2 * h)
+    assert torch.equal(tensors["o_t"], params["layers.0.mixer.o"].t()) and torch.equal(tensors["e0"], params["layers.0.ff.w"][0])
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    loaded = load_params(model, str(tmp_path), torch.float32, "cpu")
+    assert all(torch.equal(loaded[k], params[k]) for k in params)
+    tensors["o_t"] = tensors["o_t"].t().contiguous()          # stored the model's way round: not what the table says
+    del tensors["left"]
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    with pytest.raises(WeightsError) as e:
+        load_params(model, str(tmp_path), torch.float32, "cpu")
+    assert e.value.missing == ["left"] and e.value.wrong_shape == [f"o_t: checkpoint [{h}, 16], model [16, {h}]"]

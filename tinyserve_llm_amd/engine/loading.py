@@ -43,13 +43,15 @@ def streaming_copies(model: DecoderModel, policy: bool | None, device: torch.dev
 
 
 def _bound_tensors(model: DecoderModel):
-    for layer in model.layers:
-        for part in layer.parts().values():
-            for name in part.param_specs():
-                t = getattr(part, name, None)
-                if isinstance(t, torch.Tensor):
-                    yield t
-    yield model.embed
+    """Every parameter tensor the model's parts hold (a tied head's is the embedding's: counted once)."""
+    seen: set[int] = set()
+    parts = [p for layer in model.layers for p in layer.parts().values()] + [model.embedding, model.head, model.final_norm]
+    for part in parts:
+        for name in part.param_specs():
+            t = getattr(part, name, None)
+            if isinstance(t, torch.Tensor) and t.data_ptr() not in seen:
+                seen.add(t.data_ptr())
+                yield t
 
 
 def load_model(folder: str, dtype: str | torch.dtype = torch.bfloat16, device: str | torch.device = "cuda:0",

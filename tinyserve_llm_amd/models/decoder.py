@@ -9,11 +9,9 @@ from dataclasses import dataclass
 import torch
 
 from tinyserve_llm_amd.models.spec import ModelSpec
-from tinyserve_llm_amd.ops import hip
 from tinyserve_llm_amd.parts import base
-from tinyserve_llm_amd.parts.base import KVSpec, LayerMemory, ParamSpec, StateSpec, StepContext
+from tinyserve_llm_amd.parts.base import KVSpec, LayerMemory, ParamSpec, PartSpec, StateSpec, StepContext
 from tinyserve_llm_amd.parts.block import Layer
-from tinyserve_llm_amd.parts.linear import linear, streaming_copy
 
 
 @dataclass(frozen=True)
@@ -36,17 +34,20 @@ class DecoderModel:
         self.layers: list[Layer] = []
         for ls in spec.layers:
             # one LayerSpec object listed at several indices still gives one set of weights per index
-            self.layers.append(Layer(
-                mixer=base.make("mixer", ls.mixer), feed_forward=base.make("feed_forward", ls.feed_forward),
-                mixer_norm=base.make("norm", ls.mixer_norm), ff_norm=base.make("norm", ls.ff_norm), block=ls.block))
             if ls.block not in base.BLOCKS:
                 raise KeyError(f"no block arrangement named {ls.block!r}; registered: {sorted(base.BLOCKS)}")
+            lacking = [n for n in getattr(base.BLOCKS[ls.block], "norm_names", ()) if n not in ls.norms]
+            if lacking:
+                raise KeyError(f"block arrangement {ls.block!r} asks for the norms {lacking}; the layer names {sorted(ls.norms)}")
+            self.layers.append(Layer(
+                mixer=base.make("mixer", ls.mixer), feed_forward=base.make("feed_forward", ls.feed_forward),
+                norms={name: base.make("norm", ps) for name, ps in ls.norms.items()}, block=ls.block))
         self.final_norm = base.make("norm", spec.final_norm)
         self.position_encodings = {name: base.make("position_encoding", ps)
                                    for name, ps in spec.position_encodings.items()}
-        self.embed: torch.Tensor | None = None
-        self.head: torch.Tensor | None = None
-        self.head_packed = None                  # `streaming_copy` of the head, if the model keeps them
+        sizes = dict(vocab_size=spec.vocab_size, hidden_size=spec.hidden_size, init=spec.embedding_init)
+        self.embedding = base.make("embedding", spec.embedding or PartSpec("table", sizes))
+        self.head = base.make("head", spec.head or PartSpec("projection", dict(sizes, tied=spec.tie_word_embeddings)))
         self.dtype: torch.dtype | None = None
         self.device: torch.device | None = None
         self._check_order()
@@ -88,13 +89,12 @@ class DecoderModel:
     def graph_safe(self) -> bool:
         """True if every part may be recorded into a HIP graph (see Part.graph_safe)."""
         parts = [p for layer in self.layers for p in layer.parts().values()]
-        parts += [self.final_norm, *self.position_encodings.values()]
+        parts += [self.final_norm, self.embedding, self.head, *self.position_encodings.values()]
         return all(getattr(p, "graph_safe", False) for p in parts)
 
     # ---- parameters --------------------------------------------------------------------------
     def param_specs(self) -> dict[str, ParamSpec]:
-        s = self.spec
-        out: dict[str, ParamSpec] = {"embed.weight": ParamSpec((s.vocab_size, s.hidden_size), init=s.embedding_init)}
+        out: dict[str, ParamSpec] = {f"embed.{pname}": ps for pname, ps in self.embedding.param_specs().items()}
         for i, layer in enumerate(self.layers):
             for part_name, part in layer.parts().items():
                 for pname, ps in part.param_specs().items():
@@ -104,8 +104,8 @@ class DecoderModel:
                 out[f"positions.{name}.{pname}"] = ps
         for pname, ps in self.final_norm.param_specs().items():
             out[f"final_norm.{pname}"] = ps
-        if not s.tie_word_embeddings:
-            out["head.weight"] = ParamSpec((s.vocab_size, s.hidden_size), init=s.embedding_init)
+        for pname, ps in self.head.param_specs().items():
+            out[f"head.{pname}"] = ps
         return out
 
     def bind(self, params: dict[str, torch.Tensor], dtype: torch.dtype, device: torch.device) -> None:
@@ -115,8 +115,10 @@ class DecoderModel:
         for name, tensor in params.items():
             owner, _, pname = name.rpartition(".")
             grouped.setdefault(owner, {})[pname] = tensor
-        self.embed = params["embed.weight"]
-        self.head = self.embed if self.spec.tie_word_embeddings else params["head.weight"]
+        self.embedding.bind(grouped.get("embed", {}))
+        self.head.bind(grouped.get("head", {}))
+        if self.spec.tie_word_embeddings:
+            self.head.tie(self.embedding.table())
         for i, layer in enumerate(self.layers):
             for part_name, part in layer.parts().items():
                 part.bind(grouped.get(f"layers.{i}.{part_name}", {}))
@@ -127,18 +129,16 @@ class DecoderModel:
 
     def keep_streaming_copies(self) -> int:
         """Lets every part of every layer keep its weights once more in a decode kernel's reading
-        order, and keeps the head's (a step reads the whole vocabulary matrix once whatever its
-        size: at the 1B sizes a fifth of a decode step's bytes); returns the bytes that takes."""
-        self.head_packed = streaming_copy(self.head)
-        own = 0 if self.head_packed is None else self.head_packed.nbytes()
-        return own + sum(part.keep_streaming_copies() for layer in self.layers for part in layer.parts().values())
+        order, and the head likewise; returns the bytes that takes."""
+        return self.head.keep_streaming_copies() + sum(part.keep_streaming_copies() for layer in self.layers
+                                                       for part in layer.parts().values())
 
     # ---- one step ----------------------------------------------------------------------------
     def forward(self, ctx: StepContext, memory: list[LayerMemory]) -> tuple[torch.Tensor, torch.Tensor | None]:
         """Runs the step's tokens through every entry of the order; returns the last feed-forward
         output and the residual stream, whose sum the final norm takes."""
         ctx.position_encodings = self.position_encodings
-        hidden = hip.embedding(self.embed, ctx.token_ids)
+        hidden = self.embedding.forward(ctx)
         for enc in self.position_encodings.values():
             hidden = enc.on_embedding(hidden, ctx)
         residual = None
@@ -151,4 +151,4 @@ class DecoderModel:
         """float32 logits [len(rows), vocab] at the wanted rows only: the final norm and the
         vocabulary projection touch no other row (tinyserve_llm/engine/model_runner.py:125-127)."""
         normed, _ = self.final_norm(hidden, residual, rows)
-        return linear(normed, self.head, out_dtype=torch.float32, packed=self.head_packed)
+        return self.head.forward(normed)

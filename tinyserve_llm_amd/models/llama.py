@@ -19,13 +19,13 @@ def llama_spec(config: LlamaConfig) -> ModelSpec:
     rope = PartSpec("rope", dict(head_dim=c.head_dim, max_position=c.max_position_embeddings,
                                  theta=c.rope_theta, scaling=scaling))
     norm = PartSpec("rmsnorm", dict(hidden_size=c.hidden_size, eps=c.rms_norm_eps))
-    layer = LayerSpec(
+    layer = LayerSpec.pre_norm(
         mixer=PartSpec("attention", dict(hidden_size=c.hidden_size, num_heads=c.num_attention_heads,
                                          num_kv_heads=c.num_key_value_heads, head_dim=c.head_dim,
                                          position="rope")),
         feed_forward=PartSpec("gated_mlp", dict(hidden_size=c.hidden_size, intermediate_size=c.intermediate_size,
                                                 activation="silu")),
-        mixer_norm=norm, ff_norm=norm, block="pre_norm")
+        mixer_norm=norm, ff_norm=norm)
     n = c.num_hidden_layers
     ckpt: dict[str, Destination] = {"model.embed_tokens.weight": Destination("embed.weight"),
                                     "model.norm.weight": Destination("final_norm.weight")}

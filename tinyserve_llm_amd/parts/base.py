@@ -1,7 +1,8 @@
 """What a part of a layer is, and the registries that a configuration picks parts from.
 
-A layer is assembled from four parts (a mixer, a feed-forward, two norms) in an arrangement
-(a block); position encodings are shared parts that mixers refer to by name. Each part is built
+A layer is assembled from a mixer, a feed-forward and the norms its arrangement (a block) names;
+position encodings are shared parts that mixers refer to by name; an embedding and a head stand
+at the two ends of the model. Each part is built
 from explicit sizes and constants, declares the parameters it needs, receives them once, and then
 works on flat batches of tokens. No part knows which model or which layer it is in.
 
@@ -162,16 +163,40 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
+class Embedding(Part):
+    """Token ids to the first hidden rows [tokens, hidden]."""
+
+    def forward(self, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+    def table(self) -> torch.Tensor | None:
+        """The [vocab, hidden] matrix a tied head may share, or None if there is none to share."""
+        return None
+
+
+class Head(Part):
+    """The final (already normalised) rows to float32 logits [rows, vocab]."""
+
+    def tie(self, table: torch.Tensor) -> None:
+        """Called instead of handing the head a weight of its own when the model ties it to the embedding."""
+        raise NotImplementedError(f"{type(self).__name__} cannot be tied to the embedding")
+
+    def forward(self, rows: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
 # ---- registries -----------------------------------------------------------------------------
 
 MIXERS: dict[str, Callable[..., Mixer]] = {}
 FEED_FORWARDS: dict[str, Callable[..., FeedForward]] = {}
 NORMS: dict[str, Callable[..., Norm]] = {}
 POSITION_ENCODINGS: dict[str, Callable[..., PositionEncoding]] = {}
+EMBEDDINGS: dict[str, Callable[..., Embedding]] = {}
+HEADS: dict[str, Callable[..., Head]] = {}
 BLOCKS: dict[str, Callable[..., Any]] = {}
 
 _TABLES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS,
-           "position_encoding": POSITION_ENCODINGS, "block": BLOCKS}
+           "position_encoding": POSITION_ENCODINGS, "embedding": EMBEDDINGS, "head": HEADS, "block": BLOCKS}
 
 
 def register(family: str, name: str) -> Callable:

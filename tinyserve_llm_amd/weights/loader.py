@@ -2,7 +2,8 @@
 
 Files are `model*.safetensors` in sorted order (tinyserve_llm/model/loader.py:33-35). Each
 checkpoint tensor goes to the destination the architecture's table names for it (a whole
-parameter or a row slice of a fused one, loader.py:49-60). Everything that is wrong with a
+parameter, a row or column slice of a fused one, one matrix of a stack, possibly transposed;
+the reference knows whole parameters and row slices, loader.py:49-60). Everything that is wrong with a
 checkpoint is collected and raised once: tensors the model needs and did not get ("did not
 fill", loader.py:63-70), tensors it has no place for, and shapes that do not fit.
 """
@@ -52,7 +53,7 @@ def load_params(model: DecoderModel, folder: str, dtype: torch.dtype, device: to
     specs = model.param_specs()
     host: dict[str, torch.Tensor] = {
         name: torch.empty(ps.shape, dtype=storage_dtype(ps, dtype)) for name, ps in specs.items()}
-    filled: dict[str, int] = {name: 0 for name in specs}       # rows written per parameter
+    filled: dict[str, int] = {name: 0 for name in specs}       # elements written per parameter
     seen: set[str] = set()
     unexpected: list[str] = []
     wrong: list[str] = []
@@ -70,18 +71,18 @@ def load_params(model: DecoderModel, folder: str, dtype: torch.dtype, device: to
                     wrong.append(f"{name}: present in more than one file")
                     continue
                 seen.add(name)
-                target = host[dest.param]
-                rows = dest.rows if dest.rows is not None else target.shape[0]
-                want = (rows, *target.shape[1:])
+                place = dest.view(host[dest.param])          # what of the parameter this tensor fills
+                want = tuple(reversed(place.shape)) if dest.transpose else tuple(place.shape)
                 got = tuple(f.get_slice(name).get_shape())
                 if got != want:
                     wrong.append(f"{name}: checkpoint {list(got)}, model {list(want)}")
                     continue
-                target.narrow(0, dest.row, rows).copy_(f.get_tensor(name))
-                filled[dest.param] += rows
+                tensor = f.get_tensor(name)
+                place.copy_(tensor.t() if dest.transpose else tensor)
+                filled[dest.param] += place.numel()
     missing = sorted(n for n, d in spec.checkpoint.items() if n not in seen)
     # a parameter no checkpoint name maps to cannot be filled at all: that is a bug of the table
-    unmapped = sorted(p for p, n in filled.items() if n != specs[p].shape[0]
+    unmapped = sorted(p for p, n in filled.items() if n != host[p].numel()
                       and not any(d.param == p for d in spec.checkpoint.values()))
     if unmapped:
         missing += [f"{p} (no checkpoint name maps to it)" for p in unmapped]

@@ -39,10 +39,8 @@ def checkpoint_tensors(model: DecoderModel, params: dict[str, torch.Tensor]) -> 
     """Parameters split back into the tensors of a checkpoint, by the architecture's table."""
     out = {}
     for name, dest in model.spec.checkpoint.items():
-        t = params[dest.param]
-        if dest.rows is not None:
-            t = t.narrow(0, dest.row, dest.rows)
-        out[name] = t.detach().cpu().contiguous().clone()
+        t = dest.view(params[dest.param])
+        out[name] = (t.t() if dest.transpose else t).detach().cpu().contiguous().clone()
     return out
 
 
