@@ -113,6 +113,28 @@ def test_prompt_portions_then_decoding_side_by_side(case, dtype):
           f"{len(got)} rows; logits have standard deviation {spread:.3f}")
 
 
+def test_bfloat16_fed_whole_and_fed_singly_at_real_sizes(case):
+    """At these widths a step of up to 16 rows has its norms inside the projection kernels (the operand
+    (x + residual) * weight rounded once, the row's scale applied to the finished sums) and a larger
+    step runs them as kernels of their own (rounded before the weight, as the reference does); the
+    attention kernels differ as well. The same request fed whole and fed token by token therefore
+    goes through different roundings in every layer: the two must stay as close to each other as each
+    is held to the plain model."""
+    from tinyserve_llm_amd.engine.replay import Replay
+    folder, prompts, rows = case
+    p = prompts[0]
+    tail = list(range(len(p) - DECODED, len(p)))
+    rep = Replay(folder, "bfloat16", 1024)
+    whole = rep.step([{"id": "w", "tokens": p, "want": tail}], ["w"])
+    rep.step([{"id": "s", "tokens": p[:tail[0]], "want": []}], [])
+    single = torch.cat([rep.step([{"id": "s", "tokens": [p[pos]], "want": [0]}], []) for pos in tail])
+    spread = float(torch.stack(list(rows.values())).std())
+    diff = (whole - single).double()
+    rms, worst = float(diff.pow(2).mean().sqrt()), float(diff.abs().max())
+    print(f"fed whole against fed singly: root mean square {rms:.3e}, worst {worst:.3e}, spread {spread:.3f}")
+    assert 0.0 < rms <= BF16_RMS * spread and worst <= BF16_WORST * spread
+
+
 def test_a_recorded_batch_of_forty_at_the_1b_sizes(tmp_path):
     """Forty requests decode together through recorded steps at the 1B layer sizes: above 32 rows the
     projections are the matrix library's, with the candidate that was fastest when the step was

@@ -9,6 +9,7 @@ from __future__ import annotations
 import pytest
 import torch
 
+from tests.helpers import prompt
 from tests.plain import llama as P
 
 pytestmark = pytest.mark.gpu
@@ -488,3 +489,83 @@ def test_another_block_arrangement_another_embedding_and_another_head():
     manager.append_slots(0, ids[6:])
     rest = runner.step([StepEntry(0, ids[6:], 6, [0, 1, 2])])
     torch.testing.assert_close(torch.cat([first, rest]).double().cpu(), want, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_layer_that_reads_a_window_gives_its_pages_back_while_the_engine_steps(dtype):
+    """Two layers, one that keeps every key and one that only ever reads the last 10 positions (no
+    multiple of the page of 4): the windowed layer has a page space of its own, whose pages go back
+    as the window passes them and are taken again by the other request. Portions, single tokens and
+    a second request on the same few pages, against attention with the same window written plainly."""
+    from tinyserve_llm_amd.engine.interface import build_cache
+    from tinyserve_llm_amd.engine.runner import ModelRunner, StepEntry
+    from tinyserve_llm_amd.models.decoder import DecoderModel
+    from tinyserve_llm_amd.models.spec import LayerRun, LayerSpec, ModelSpec
+    from tinyserve_llm_amd.parts.base import PartSpec
+    from tinyserve_llm_amd.weights.random_init import random_params
+    hidden, window, page = 32, 10, 4
+    norm = PartSpec("rmsnorm", dict(hidden_size=hidden, eps=1e-5))
+    mlp = PartSpec("gated_mlp", dict(hidden_size=hidden, intermediate_size=48))
+    def attn(w):
+        return PartSpec("attention", dict(hidden_size=hidden, num_heads=2, num_kv_heads=1, head_dim=16, position="rope", window=w))
+    rope = PartSpec("rope", dict(head_dim=16, max_position=96, theta=10000.0))
+    spec = ModelSpec("ToyWindow", 50, hidden, 96, [LayerSpec.pre_norm(attn(0), mlp, norm, norm), LayerSpec.pre_norm(attn(window), mlp, norm, norm)],
+                     [LayerRun(0), LayerRun(1)], norm, position_encodings={"rope": rope}, tie_word_embeddings=True)
+    model = DecoderModel(spec)
+    params = random_params(model, 6, dtype, "cpu")
+    model.bind({k: v.to(DEV) for k, v in params.items()}, dtype, torch.device(DEV))
+    p = {k: v.double() for k, v in params.items()}
+    storage, manager = build_cache(model, [24, 8], page, dtype, DEV, num_state_slots=2)    # 8 pages for the window: two requests cannot keep all theirs
+    assert [s.window for s in storage.spaces] == [0, window] and not manager.caching
+    runner = ModelRunner(model, storage, manager)
+
+    def plain(ids):
+        n = len(ids)
+        cos, sin = P.rope_tables(16, 10000.0, None, 96, n, torch.float64)
+        h = p["embed.weight"][torch.tensor(ids)]
+        for i, w in enumerate((0, window)):
+            x = P.rms_norm(h, p[f"layers.{i}.mixer_norm.weight"], 1e-5)
+            qkv = x @ p[f"layers.{i}.mixer.qkv"].T
+            q, k = P.apply_rope(qkv[:, :32].reshape(n, 2, 16), cos, sin), P.apply_rope(qkv[:, 32:48].reshape(n, 1, 16), cos, sin)
+            o = P.causal_attention(q, k, qkv[:, 48:].reshape(n, 1, 16), window=w)
+            h = h + o.reshape(n, 32) @ p[f"layers.{i}.mixer.o"].T
+            x = P.rms_norm(h, p[f"layers.{i}.ff_norm.weight"], 1e-5)
+            h = h + P.silu_mul(x @ p[f"layers.{i}.ff.gate_up"].T) @ p[f"layers.{i}.ff.down"].T
+        return P.rms_norm(h, p["final_norm.weight"], 1e-5) @ p["embed.weight"].T
+
+    a, b = prompt(1, 41, 50), prompt(2, 23, 50)
+    want = {0: plain(a), 1: plain(b)}
+    got, fed = {}, {0: 0, 1: 0}
+
+    def step(entries):
+        batch = []
+        for r, n in entries:
+            ids = (a, b)[r][fed[r]:fed[r] + n]
+            (manager.allocate(r, ids) if fed[r] == 0 else manager.append_slots(r, ids))
+            batch.append(StepEntry(r, ids, fed[r], [0, n - 1] if n > 1 else [0]))
+        logits = runner.step(batch)
+        row = 0
+        for (r, n), e in zip(entries, batch):
+            for wpos in e.want:
+                got[(r, fed[r] + wpos)] = logits[row]
+                row += 1
+            manager.commit(r, n)
+            fed[r] += n
+
+    step([(0, 13)])
+    step([(0, 2), (1, 9)])
+    for _ in range(6):
+        step([(0, 1), (1, 1)])
+    step([(0, 5), (1, 3)])
+    step([(0, 6), (1, 5)])
+    assert manager.stats().window_frees > 0 and fed[1] == len(b)
+    while fed[0] < len(a):
+        step([(0, 1)])
+    assert manager.block_table(0, 1)[0] < 0 and manager.block_table(0, 0)[0] >= 0, "only the windowed space lets go of old pages"
+    tol = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=3e-2, atol=3e-2)
+    for (r, pos), row in got.items():
+        torch.testing.assert_close(row.double().cpu(), want[r][pos], msg=lambda m: f"request {r} position {pos}: {m}", **tol)
+    assert len(got) >= 30
+    manager.release(0)
+    manager.release(1)
+    assert manager.num_available_blocks(1) == 8 and manager.num_available_blocks(0) == 24

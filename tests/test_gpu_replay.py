@@ -171,6 +171,34 @@ def test_mixed_requests_on_few_pages(case, dtype):
     assert rep.manager.num_available_blocks() == rep.manager.num_blocks
 
 
+def test_bfloat16_logits_of_one_token_at_a_time_stay_with_those_of_the_whole_prompt(case):
+    """In bfloat16 a step of up to 16 rows applies the norm inside the projection kernels (the operand
+    is (x + residual) * weight rounded once, the row's scale multiplies the finished sums), a larger
+    step runs the norm as a kernel of its own (rounded before the weight, as the reference does), and
+    attention takes the split-key kernel or the tile kernel: the same request fed whole and fed token
+    by token goes through different roundings at every layer. Both are held to the plain model
+    elsewhere; here they are held to each other, at the last 32 positions, where token-by-token
+    feeding has gone through its own roundings the longest."""
+    name, folder, config, prompts, oracles = case
+    worst = 0.0
+    for r, p in enumerate(prompts):
+        if len(p) < 40:
+            continue
+        rep = replayer(folder, "bfloat16", 512)
+        tail = list(range(len(p) - 32, len(p)))
+        whole = rep.step([{"id": "w", "tokens": p, "want": tail}], ["w"])
+        rep.step([{"id": "s", "tokens": p[:len(p) - 32], "want": []}], [])
+        single = torch.cat([rep.step([{"id": "s", "tokens": [p[pos]], "want": [0]}], []) for pos in tail])
+        diff = float((whole - single).abs().max())
+        worst = max(worst, diff)
+        assert diff <= TOL["bfloat16"]["atol"], f"request {r}: fed whole and fed singly differ by {diff:.3e}"
+        for got in (whole, single):       # and neither has drifted from the plain model
+            torch.testing.assert_close(got.double().cpu(), oracles["bfloat16"][r][tail[0]:], **TOL["bfloat16"])
+    print(f"worst difference between the two ways of feeding: {worst:.3e}")
+    if name == "B":      # (configuration A's head size of 16 goes to the one kernel that serves every step alike)
+        assert worst > 0.0, "the two ways take different attention kernels; equal results would mean one of them did not run"
+
+
 def test_float32_logits_do_not_depend_on_the_cut(case):
     """In float32 every kernel fixes the order of its sums per row, so logits are bit-equal
     however the tokens were cut into steps and whatever else was in the batch."""
