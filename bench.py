@@ -137,6 +137,9 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=None)
     ap.add_argument("--shape", default="1b", choices=sorted(SHAPES), help="layer sizes of the decode and prefill steps")
+    ap.add_argument("--context", type=int, default=PROMPT_LEN,
+                    help="tokens of every prompt: the decode steps start from contexts of this length, and the prefill "
+                         "is of this many tokens (the headline numbers are quoted at the default)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--points", default="1,64", help="further decode batch sizes (comma-separated; '' for none)")
     ap.add_argument("--no-prefill", action="store_true")
@@ -180,19 +183,22 @@ def main() -> int:
     weight_bytes = (args.layers * layer_weights + c.vocab_size * c.hidden_size) * itemsize   # the head; the embedding reads rows
     kv_bytes_per_token = 2 * args.layers * c.kv_size * itemsize
 
+    prompt_len = args.context
+    max_model_len = max(MAX_MODEL_LEN, prompt_len + 1024)
+
     def engine(batch: int, steps: int) -> LLM:
-        pages = batch * (MAX_MODEL_LEN // PAGE) + 2
-        sc = SchedulerConfig(max_model_len=MAX_MODEL_LEN, max_num_seqs=max(batch, 1),
-                             max_num_batched_tokens=max(PROMPT_LEN, batch + 1) + batch, watermark=0.0)
+        pages = batch * -(-max_model_len // PAGE) + 2
+        sc = SchedulerConfig(max_model_len=max_model_len, max_num_seqs=max(batch, 1),
+                             max_num_batched_tokens=max(prompt_len, batch + 1) + batch, watermark=0.0)
         return LLM(None, sc, CacheConfig(block_size=PAGE, caching=False), dtype=dtype, num_blocks=pages, seed=0,
                    model=model)
 
     def decode(batch: int, steps: int, warmup: int) -> tuple[float, float]:
         """(seconds for `steps` decode steps, mean context length over them)."""
         llm = engine(batch, steps + warmup)
-        sp = SamplingParams(max_tokens=MAX_MODEL_LEN - PROMPT_LEN, temperature=0.0, ignore_eos=True)
+        sp = SamplingParams(max_tokens=max_model_len - prompt_len, temperature=0.0, ignore_eos=True)
         for _ in range(batch):
-            llm.add_request([rng.randrange(c.vocab_size) for _ in range(PROMPT_LEN)], sp)
+            llm.add_request([rng.randrange(c.vocab_size) for _ in range(prompt_len)], sp)
         while any(s.in_prefill or not s.output_token_ids for s in llm.scheduler.running + llm.scheduler.waiting):
             llm.step()
         for _ in range(warmup):
@@ -213,7 +219,7 @@ def main() -> int:
         sp = SamplingParams(max_tokens=1, temperature=0.0, ignore_eos=True)
         times = []
         for r in range(reps + 1):
-            llm.add_request([rng.randrange(c.vocab_size) for _ in range(PROMPT_LEN)], sp)
+            llm.add_request([rng.randrange(c.vocab_size) for _ in range(prompt_len)], sp)
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             llm.step()
@@ -225,7 +231,7 @@ def main() -> int:
 
     def prefill_record() -> dict:
         t = prefill()
-        T = PROMPT_LEN
+        T = prompt_len
         linear_flops = 2 * T * args.layers * layer_weights + 2 * c.vocab_size * c.hidden_size
         attn_flops = args.layers * 4 * c.q_size * T * (T + 1) / 2
         return {"value": T / t, "tokens": T, "ms": 1e3 * t, "frac": (linear_flops + attn_flops) / t / PEAK_FLOPS[args.dtype]}
@@ -239,14 +245,14 @@ def main() -> int:
     step_bytes = weight_bytes + args.batch * mean_ctx * kv_bytes_per_token
     achieved = step_bytes / (seconds / args.steps)
     record = {
-        "metric": f"decode tok/s at batch {args.batch} ({sizes['model']}, 2,048-token contexts)",
+        "metric": f"decode tok/s at batch {args.batch} ({sizes['model']}, {prompt_len:,}-token contexts)",
         "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": 1e3 * seconds / args.steps, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": args.dtype, "data": "synthetic uniform token ids, random weights N(0,0.02)",
         "config": {"model": sizes["model"], "layers": args.layers, "layers_full": full_layers,
                    "hidden": c.hidden_size, "heads": c.num_attention_heads, "kv_heads": c.num_key_value_heads,
                    "head_dim": c.head_dim, "intermediate": c.intermediate_size, "vocab": c.vocab_size,
-                   "global_batch": args.batch, "prompt_len": PROMPT_LEN, "seq_len": MAX_MODEL_LEN,
+                   "global_batch": args.batch, "prompt_len": prompt_len, "seq_len": max_model_len,
                    "page_size": PAGE, "parallelism": "single-gpu"},
         "roofline": {"bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_BYTES_PER_S / 1e9, "unit": "GB/s",
                      "frac": achieved / HBM_BYTES_PER_S},

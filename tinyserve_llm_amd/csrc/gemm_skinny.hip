@@ -396,6 +396,18 @@ gemm_skinny8_kernel(const SkinnyArgs a) {
   const int r = lane & 15, g = lane >> 4, row = r & 7, half = r >> 3;
   const int n0 = blockIdx.x * 8;
   const int kbeg = wave * (2 * STEPS * SK_KSTEP) + half * (STEPS * SK_KSTEP) + 8 * g;   // this lane's first k
+  // x first where the registers allow it (workgroups of up to 8 waves): it is small and comes from the
+  // cache, loads return in the order they were issued, and so the products start the moment W is there;
+  // a larger workgroup has half the registers and fetches x in batches after W instead
+  constexpr bool X_FIRST = MAXT <= 512;
+  constexpr int XB = X_FIRST ? STEPS : (STEPS < 8 ? STEPS : 8);
+  const bf16_t* xrow = a.x + (int64_t)(row < a.M ? row : 0) * a.ldx + kbeg;   // rows past M repeat row 0 and are not stored
+  uint4 xb[XB];
+  if (X_FIRST) {
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) xb[s] = *(const uint4*)(xrow + s * SK_KSTEP);
+    __builtin_amdgcn_sched_barrier(0);
+  }
   uint4 wreg[STEPS];
   if (a.packed) {
     const bf16_t* blk = a.w + ((((int64_t)blockIdx.x * nwaves + wave) * STEPS) * 64 + lane) * 8;
@@ -408,17 +420,19 @@ gemm_skinny8_kernel(const SkinnyArgs a) {
     for (int s = 0; s < STEPS; ++s) wreg[s] = *(const uint4*)(wrow + s * SK_KSTEP);
   }
   __builtin_amdgcn_sched_barrier(0);                    // all of W's loads are in flight before anything waits
-  const bf16_t* xrow = a.x + (int64_t)(row < a.M ? row : 0) * a.ldx + kbeg;   // rows past M repeat row 0 and are not stored
   float4_t acc = {0.f, 0.f, 0.f, 0.f};
-  constexpr int XB = STEPS < 8 ? STEPS : 8;
+  if (X_FIRST) {
 #pragma unroll
-  for (int s0 = 0; s0 < STEPS; s0 += XB) {
-    uint4 xb[XB];
+    for (int s = 0; s < STEPS; ++s) acc = sk_mfma(wreg[s], xb[s], acc);
+  } else {
 #pragma unroll
-    for (int s = 0; s < XB; ++s) xb[s] = *(const uint4*)(xrow + (s0 + s) * SK_KSTEP);
-    __builtin_amdgcn_sched_barrier(0);
+    for (int s0 = 0; s0 < STEPS; s0 += XB) {
 #pragma unroll
-    for (int s = 0; s < XB; ++s) acc = sk_mfma(wreg[s0 + s], xb[s], acc);
+      for (int s = 0; s < XB; ++s) xb[s] = *(const uint4*)(xrow + (s0 + s) * SK_KSTEP);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < XB; ++s) acc = sk_mfma(wreg[s0 + s], xb[s], acc);
+    }
   }
   // acc[j] = D[4 g + j][r]: W row (4 g + j) & 7 of half (4 g + j) >> 3 times x row r & 7 of half r >> 3
 #pragma unroll

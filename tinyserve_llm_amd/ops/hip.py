@@ -651,7 +651,8 @@ def _check_packed(packed: torch.Tensor | None, weight: torch.Tensor) -> None:
 
 
 SKINNY8_MAX_ROWS = 8          # rows of x that the 8-row form of the weight-streaming kernel takes
-SKINNY8_MAX_WIDTH = 4096      # widest matrix it is chosen for where the 16-row form would serve as well
+SKINNY8_FEW_ROWS = 4          # up to this many rows it is chosen for a matrix of any width,
+SKINNY8_FULL_WIDTH = 2048     # with more rows only up to this width (a workgroup per compute unit)
 
 
 def skinny8_steps(k: int) -> int:
@@ -664,10 +665,15 @@ def skinny8_steps(k: int) -> int:
 
 
 def skinny8_takes(rows: int, n: int, k: int) -> bool:
-    """Whether `linear_bf16` gives the product to the 8-row form: at most 8 rows of x, and a matrix
-    narrow enough that 16-row tiles would leave compute units idle, or a reduction too long for them."""
+    """Whether `linear_bf16` gives the product to the 8-row form. Every workgroup reads all rows of x
+    for its 8 rows of W, twice as much of x per byte of W as the 16-row form: with 8 rows of x and a
+    matrix of 3,072 or 4,096 rows the compute units' reads of x out of the second-level cache weigh
+    as much as W itself, and the 16-row form or the library is faster (decode steps at the 3B and 8B
+    layer sizes, batch 8: 2.59 against 2.67 ms and 4.39 against 4.55; at batch 1 the 8-row form wins
+    at every width). So: few rows of x at any width, more rows only where the 8-row tiles are what
+    gives every compute unit a workgroup."""
     return (rows <= SKINNY8_MAX_ROWS and skinny8_steps(k) > 0
-            and (n <= SKINNY8_MAX_WIDTH or not (skinny_takes(rows, k) and k <= 4096)))
+            and (rows <= SKINNY8_FEW_ROWS or n <= SKINNY8_FULL_WIDTH))
 
 
 def pack_weight8(weight: torch.Tensor) -> torch.Tensor:

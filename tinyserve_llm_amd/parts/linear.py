@@ -45,7 +45,7 @@ def streaming_copy(weight: torch.Tensor) -> hip.StreamingCopies | None:
         return None
     n, k = weight.shape
     by16 = hip.pack_weight(weight) if hip.skinny_takes(1, k) and k <= 4096 else None
-    by8 = hip.pack_weight8(weight) if hip.skinny8_takes(1, n, k) and n % 8 == 0 else None
+    by8 = hip.pack_weight8(weight) if hip.skinny8_takes(1, n, k) and n % 8 == 0 else None     # (one row: the widest reach of that form)
     return hip.StreamingCopies(by16, by8) if by16 is not None or by8 is not None else None
 
 
