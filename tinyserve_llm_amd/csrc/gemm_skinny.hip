@@ -21,49 +21,7 @@
 //              halves of a rotation and a matrix of 3,072 columns gives 192 workgroups; it rounds the
 //              products as y would hold them, rotates q and k by the token's position, and writes q
 //              to its own tensor and k and v into their cache slots: y itself is never stored
-#include "common.h"
-
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float float4_t __attribute__((ext_vector_type(4)));
-
-#define SK_KSTEP 32      // k covered by one MFMA: lane group g holds k = 8 g .. 8 g + 7
-#define MODE_PLAIN 0
-#define MODE_NORM 1
-#define EPI_NONE 0
-#define EPI_GLU 1
-#define EPI_ROPE 2
-
-// acc + A · B over 32 k: lane (r, g) gives k = 8 g .. 8 g + 7 of row r of A and of column r of B
-static __device__ __forceinline__ float4_t sk_mfma(const uint4& a, const uint4& b, float4_t acc) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
-}
-
-static __device__ __forceinline__ void sk_unpack(const uint4& v, float* f) {
-  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    f[2 * i] = __uint_as_float(w[i] << 16);
-    f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
-  }
-}
-// round to nearest even; the values here are finite sums and products of finite activations
-static __device__ __forceinline__ uint32_t sk_round(float f) {
-  const uint32_t u = __float_as_uint(f);
-  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-}
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-typedef float float2_t __attribute__((ext_vector_type(2)));
-// eight floats to eight bfloat16, round to nearest even, by the hardware's packed conversion
-static __device__ __forceinline__ uint4 sk_pack(const float* f) {
-  uint32_t w[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-    w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector((float2_t){f[2 * i], f[2 * i + 1]}, bf16x2_t));
-  return make_uint4(w[0], w[1], w[2], w[3]);
-}
-static __device__ __forceinline__ float sk_silu(float g) {
-  return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896340736f * g));
-}
+#include "skinny_ops.h"
 
 struct SkinnyArgs {
   const bf16_t* x;      // [M, K] (MODE_GATE: [M, 2K])

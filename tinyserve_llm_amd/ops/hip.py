@@ -681,10 +681,10 @@ def pack_weight8(weight: torch.Tensor) -> torch.Tensor:
     [N / 8 tiles, waves, steps, 64 lanes, 8], lane r + 16 g holding row 8 tile + r % 8 at
     k = 64 steps wave + 32 steps (r // 8) + 32 step + 8 g .. + 7; rows past N are zeros."""
     _gpu(weight)
-    _need(weight.dtype == torch.bfloat16 and weight.dim() == 2 and skinny8_steps(weight.shape[1]) > 0,
-          "pack_weight8 takes bfloat16 [N, K] with a K that the 8-row form serves")
+    _need(weight.dtype == torch.bfloat16 and weight.dim() == 2, "pack_weight8 takes bfloat16 [N, K]")
     n, k = weight.shape
     steps = skinny8_steps(k)
+    _need(steps > 0, f"the 8-row form does not take a reduction of {k}")
     waves, tiles = k // (64 * steps), -(-n // 8)
     padded = weight if n == 8 * tiles else torch.cat([weight, weight.new_zeros(8 * tiles - n, k)])
     # [tile, row, wave, half, step, g, 8] -> [tile, wave, step, g, half, row, 8]
