@@ -911,6 +911,32 @@ def test_eight_row_form_of_the_weight_streaming_gemm(m, n, k):
         hip().gemm_skinny8(torch.cat([x, x])[:9].contiguous(), w)
 
 
+@pytest.mark.parametrize("m", [17, 33, 50, 64])
+@pytest.mark.parametrize("n,k", [(8192, 1024), (16384, 2048), (9152, 3072)])
+def test_wide_product_for_a_few_dozen_rows(m, n, k):
+    """The kernel that shares x among 64 rows of W through LDS, against 64-bit products: plain (bfloat16
+    and 32-bit sums) and with the gate; each row's result does not depend on the rows beside it."""
+    g = gen(m + n + k)
+    x = torch.randn(m, k, generator=g).bfloat16().to(dev())
+    w = (torch.randn(n, k, generator=g) * k ** -0.5).bfloat16().to(dev())
+    packed = hip().pack_weight(w)
+    want = x.double().cpu() @ w.double().cpu().T
+    y32, _ = hip().gemm_rows64(x, packed, torch.float32)
+    torch.testing.assert_close(y32.double().cpu(), want, rtol=1e-4, atol=1e-4 * float(want.abs().max()))
+    y16, none = hip().gemm_rows64(x, packed)
+    assert none is None and torch.equal(y16, y32.bfloat16())
+    if n % 128 == 0:
+        gate = P.silu_mul(want)
+        yg, _ = hip().gemm_rows64(x, packed, glu=True)
+        assert yg.shape == (m, n // 2)
+        torch.testing.assert_close(yg.double().cpu(), gate, rtol=2e-2, atol=2e-2 * float(gate.abs().max()))
+    alone, _ = hip().gemm_rows64(x[m - 1:].contiguous(), packed, torch.float32)
+    assert torch.equal(alone[0], y32[m - 1])
+    assert hip().rows64_takes(max(m, 33), n, k) and not hip().rows64_takes(65, n, k) and not hip().rows64_takes(40, n, k + 512)
+    with pytest.raises(hip().KernelError):
+        hip().gemm_rows64(torch.cat([x, x, x, x])[:65].contiguous(), packed)
+
+
 def test_fused_projection_reads_the_packed_copy_to_the_same_result():
     g = gen(77)
     nh, nkv, hd, K, M, page = 6, 2, 64, 1024, 7, 16

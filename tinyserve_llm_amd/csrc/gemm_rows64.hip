@@ -1,0 +1,240 @@
+// y[M, N] = e(f(x)[M, K] · W[N, K]^T) in bfloat16 for 17 to 64 rows of x and a wide W (the gate|up
+// projection of a decode step of a few dozen requests), where time should go to reading W once.
+//
+// With so many rows the weight-streaming kernel of gemm_skinny.hip reads x from the second-level cache
+// once per 32 rows of W, which is twice the bytes of W itself. Here a workgroup owns 64 rows of W and
+// splits the work between two kinds of wave:
+//   four compute waves, one 16-row tile of W each over the whole of K: the tile streams from memory
+//   straight into MFMA operands, 32 steps of 32 k under way at any time (a step's register is asked for
+//   again as soon as it has been used), and the four 16-row blocks of x come out of LDS;
+//   four staging waves, which bring x into LDS in chunks of 256 k, in the order the lanes read it, one
+//   chunk ahead of the compute waves (two buffers, a barrier per chunk). Their loads are few and hit the
+//   cache; in waves of their own they do not queue behind the loads of W (a wave's loads come back in
+//   the order it asked).
+// What precedes and follows the product rides along as in gemm_skinny.hip, operation for operation:
+//   NORM  the staging waves add the residual, write the new residual (workgroup 0), sum the squares in
+//         32 bits and put T((x + res) * nw) into LDS; the row's scale multiplies the finished sums
+//   GLU   W = [gate rows | up rows]: waves 0 and 1 take two gate tiles, waves 2 and 3 the up tiles
+//         N / 2 rows below them, and y [M, N / 2] = silu(gate) * up
+// W comes as the 16-row packed copy ([N / 16 tiles][K / 32 steps][64 lanes][8]); K is a multiple of
+// 1,024. A row of x meets W's k in ascending order in one accumulator, whatever the other rows are.
+#include <type_traits>
+#include "skinny_ops.h"
+
+#define R64_CHUNK_STEPS 8         // 32-wide k steps per chunk of x in LDS
+#define R64_RING 32               // steps of W a compute wave has under way (four chunks)
+#define R64_STAGE_STEPS (R64_CHUNK_STEPS / 4)   // steps of a chunk that one staging wave brings
+
+struct Rows64Args {
+  const bf16_t* x;       // [M, K], row stride ldx
+  const bf16_t* res;     // NORM: residual [M, K] or null
+  const bf16_t* nw;      // NORM: norm weight [K]
+  bf16_t* res_out;       // NORM with res: new residual [M, K]
+  const bf16_t* w16;     // W [N, K], packed
+  void* y;               // [M, N] (GLU: [M, N / 2]), row stride ldy
+  int M, N, K;
+  int64_t ldx, ldy;
+  float eps;
+};
+
+// What a staging wave has asked for of one chunk: its steps of x for the four blocks of rows, and with
+// the norm the residual's and the weight's.
+template <bool NORM>
+struct Rows64Staged {
+  uint4 x[R64_STAGE_STEPS][4], res[NORM ? R64_STAGE_STEPS : 1][4], nw[NORM ? R64_STAGE_STEPS : 1];
+};
+
+template <bool NORM, bool GLU, typename OUT>
+__global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
+  // x as the B operands of the matrix instruction: [buffer][step][block of 16 rows][lane], lane r + 16 g
+  // holding k = 8 g .. 8 g + 7 of row r
+  __shared__ uint4 xs[2][R64_CHUNK_STEPS][4][TS_WAVE];
+  __shared__ float ssq[4][64];                           // NORM: the staging waves' shares of the rows' sums of squares
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TS_WAVE), lane = threadIdx.x & (TS_WAVE - 1);
+  const int r = lane & 15, g = lane >> 4;
+  const int nsteps = a.K / SK_KSTEP, nchunks = nsteps / R64_CHUNK_STEPS;   // (a multiple of 4)
+
+  if (wave >= 4) {
+    // ---- staging waves: wave sw brings steps 2 sw and 2 sw + 1 of every chunk, all four blocks of
+    // rows. It asks for the next chunk before it works on this one, so that a chunk costs the compute
+    // waves a barrier and not a trip to the cache.
+    const int sw = wave - 4;
+    const bool has_res = NORM && a.res != nullptr;
+    float sq[4] = {0.f, 0.f, 0.f, 0.f};                  // this lane's share of rows 16 b + r
+    bool ok[4];
+    int64_t xoff[4], roff[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      ok[b] = 16 * b + r < a.M;                          // rows past M read row 0 and count as zeros
+      xoff[b] = (int64_t)(ok[b] ? 16 * b + r : 0) * a.ldx + 8 * g;
+      roff[b] = (int64_t)(ok[b] ? 16 * b + r : 0) * a.K + 8 * g;
+    }
+    auto ask = [&](int c, Rows64Staged<NORM>& t) {
+      const int k0 = (c * R64_CHUNK_STEPS + R64_STAGE_STEPS * sw) * SK_KSTEP;   // first k of this wave's steps
+#pragma unroll
+      for (int s = 0; s < R64_STAGE_STEPS; ++s) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) t.x[s][b] = *(const uint4*)(a.x + xoff[b] + k0 + s * SK_KSTEP);
+        if (NORM) {
+          t.nw[s] = *(const uint4*)(a.nw + k0 + s * SK_KSTEP + 8 * g);
+          // (a missing residual reads x again: the same loads on every path)
+#pragma unroll
+          for (int b = 0; b < 4; ++b)
+            t.res[s][b] = *(const uint4*)((has_res ? a.res + roff[b] : a.x + xoff[b]) + k0 + s * SK_KSTEP);
+        }
+      }
+    };
+    auto put = [&](int c, const Rows64Staged<NORM>& t) {
+      const int k0 = (c * R64_CHUNK_STEPS + R64_STAGE_STEPS * sw) * SK_KSTEP;
+#pragma unroll
+      for (int s = 0; s < R64_STAGE_STEPS; ++s)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          uint4 v = ok[b] ? t.x[s][b] : make_uint4(0, 0, 0, 0);
+          if (NORM) {
+            float xv[8], rv[8], nv[8];
+            sk_unpack(t.x[s][b], xv);
+            sk_unpack(t.res[s][b], rv);
+            sk_unpack(t.nw[s], nv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) xv[i] = ok[b] ? xv[i] + (has_res ? rv[i] : 0.f) : 0.f;
+            if (has_res && blockIdx.x == 0 && ok[b]) *(uint4*)(a.res_out + roff[b] + k0 + s * SK_KSTEP) = sk_pack(xv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+              sq[b] = fmaf(xv[i], xv[i], sq[b]);
+              xv[i] *= nv[i];
+            }
+            v = sk_pack(xv);
+          }
+          xs[c & 1][R64_STAGE_STEPS * sw + s][b][lane] = v;
+        }
+    };
+    Rows64Staged<NORM> A, B;
+    ask(0, A);
+    for (int c = 0; c < nchunks; c += 2) {
+      ask(c + 1, B);
+      put(c, A);
+      __syncthreads();          // chunk c is there (and chunk c - 1 has been used: its buffer is the next one's)
+      ask(min(c + 2, nchunks - 1), A);   // (past the end: the last chunk again, and nobody uses it)
+      put(c + 1, B);
+      __syncthreads();
+    }
+    if (NORM) {
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        sq[b] += __shfl_xor(sq[b], 16, TS_WAVE);
+        sq[b] += __shfl_xor(sq[b], 32, TS_WAVE);
+        if (g == 0) ssq[sw][16 * b + r] = sq[b];
+      }
+    }
+    __syncthreads();            // the compute waves' last chunk
+    __syncthreads();            // the squares are there
+    return;
+  }
+
+  // ---- compute waves
+  const int tile = GLU ? (wave < 2 ? 2 * blockIdx.x + wave : a.N / 32 + 2 * blockIdx.x + (wave - 2)) : 4 * blockIdx.x + wave;
+  const bf16_t* wp = a.w16 + ((int64_t)tile * nsteps * 64 + lane) * 8;      // step s at wp + 512 s
+  uint4 wr[R64_RING];
+  // (in this order and no other: the ring is used oldest first, and a wait is for the oldest load only if the
+  // compiler sees the first loads come in the order of their use)
+#pragma unroll
+  for (int s = 0; s < R64_RING; ++s) {
+    wr[s] = *(const uint4*)(wp + (int64_t)s * 512);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  float4_t acc[4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) acc[b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+  __syncthreads();              // chunk 0 is there
+  // 32 steps at a time, each register of the ring asked for again once it has been used; the last 32 ask for nothing
+  auto ring = [&](int base, auto more) {
+#pragma unroll
+    for (int h = 0; h < R64_RING / R64_CHUNK_STEPS; ++h) {
+      // a chunk in four pairs of steps: the next pair's operands leave LDS while this pair's products
+      // run (left to itself the compiler reads two operands, waits, multiplies, and so on)
+      constexpr int PAIRS = R64_CHUNK_STEPS / 2;
+      uint4 xb[2][2][4];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) xb[0][i][b] = xs[h & 1][i][b][lane];
+#pragma unroll
+      for (int q = 0; q < PAIRS; ++q) {
+        if (q + 1 < PAIRS) {
+#pragma unroll
+          for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int b = 0; b < 4; ++b) xb[(q + 1) & 1][i][b] = xs[h & 1][2 * (q + 1) + i][b][lane];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const int sl = R64_CHUNK_STEPS * h + 2 * q + i;
+#pragma unroll
+          for (int b = 0; b < 4; ++b) acc[b] = sk_mfma(wr[sl], xb[q & 1][i][b], acc[b]);
+          if (decltype(more)::value) wr[sl] = *(const uint4*)(wp + (int64_t)(base + R64_RING + sl) * 512);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      __syncthreads();
+    }
+  };
+  int base = 0;
+  for (; base + R64_RING < nsteps; base += R64_RING) ring(base, std::true_type{});
+  ring(base, std::false_type{});
+  // acc[b][j] = sum over k of W[row 16 tile + 4 g + j, k] * f(x)[16 b + r, k]
+  float4_t* ex = (float4_t*)&xs[0][0][0][0];             // [2 up waves][4 blocks][lane]; every read of x is behind the last barrier
+  if (GLU && wave >= 2) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) ex[((wave - 2) * 4 + b) * TS_WAVE + lane] = acc[b];
+  }
+  __syncthreads();
+  if (GLU && wave >= 2) return;
+  OUT* y = (OUT*)a.y;
+  const int n0 = GLU ? (2 * blockIdx.x + wave) * 16 + 4 * g : tile * 16 + 4 * g;
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int m = 16 * b + r;
+    if (m >= a.M) continue;
+    float inv = 1.0f;
+    if (NORM) inv = 1.0f / sqrtf((ssq[0][m] + ssq[1][m] + ssq[2][m] + ssq[3][m]) / (float)a.K + a.eps);
+    float4_t u = {0.f, 0.f, 0.f, 0.f};
+    if (GLU) u = ex[(wave * 4 + b) * TS_WAVE + lane];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float s = acc[b][j] * inv;
+      Num<OUT>::st(y + (int64_t)m * a.ldy + n0 + j, GLU ? sk_silu(s) * (u[j] * inv) : s);
+    }
+  }
+}
+
+template <bool NORM, bool GLU, typename OUT>
+static int r64_launch(const Rows64Args& a, hipStream_t stream) {
+  const int grid = a.N / 64;                             // 64 rows of W per workgroup
+  gemm_rows64_kernel<NORM, GLU, OUT><<<grid, 512, 0, stream>>>(a);
+  return ts_check_launch();
+}
+
+// x [M <= 64, K] (row stride ldx), w16: W [N, K] as its 16-row packed copy, y [M, N] or, with glu, [M, N / 2]
+// (row stride ldy; out_f32: 32-bit sums instead of bfloat16). norm_weight non-null: the residual (may be
+// null) and RMSNorm on the way in, res_out the new residual. N a multiple of 64, K of 1,024.
+extern "C" int ts_gemm_rows64_bf16(void* y, const void* x, const void* w16, const void* res, const void* norm_weight,
+                                   void* res_out, int M, int N, int K, int64_t ldx, int64_t ldy, float eps, int glu,
+                                   int out_f32, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return TS_OK;
+  if (M > 64 || N % 64 || K <= 0 || K % 1024 || ldx < K || (ldx % 8) || !y || !x || !w16) return TS_BAD_SHAPE;
+  if ((((uintptr_t)x) | ((uintptr_t)w16) | ((uintptr_t)res) | ((uintptr_t)norm_weight) | ((uintptr_t)res_out)) & 15) return TS_BAD_SHAPE;
+  if (res && (!norm_weight || !res_out)) return TS_BAD_SHAPE;
+  if (glu && out_f32) return TS_BAD_SHAPE;
+  Rows64Args a = {(const bf16_t*)x, (const bf16_t*)res, (const bf16_t*)norm_weight, (bf16_t*)res_out, (const bf16_t*)w16, y,
+                  M, N, K, ldx, ldy, eps};
+  if (norm_weight) {
+    if (glu) return r64_launch<true, true, bf16_t>(a, stream);
+    if (out_f32) return r64_launch<true, false, float>(a, stream);
+    return r64_launch<true, false, bf16_t>(a, stream);
+  }
+  if (glu) return r64_launch<false, true, bf16_t>(a, stream);
+  if (out_f32) return r64_launch<false, false, float>(a, stream);
+  return r64_launch<false, false, bf16_t>(a, stream);
+}
