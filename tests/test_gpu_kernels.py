@@ -921,16 +921,15 @@ def test_wide_product_for_a_few_dozen_rows(m, n, k):
     w = (torch.randn(n, k, generator=g) * k ** -0.5).bfloat16().to(dev())
     packed = hip().pack_weight(w)
     want = x.double().cpu() @ w.double().cpu().T
-    y32, _ = hip().gemm_rows64(x, packed, torch.float32)
+    y32 = hip().gemm_rows64(x, packed, torch.float32)
     torch.testing.assert_close(y32.double().cpu(), want, rtol=1e-4, atol=1e-4 * float(want.abs().max()))
-    y16, none = hip().gemm_rows64(x, packed)
-    assert none is None and torch.equal(y16, y32.bfloat16())
+    assert torch.equal(hip().gemm_rows64(x, packed), y32.bfloat16())
     if n % 128 == 0:
         gate = P.silu_mul(want)
-        yg, _ = hip().gemm_rows64(x, packed, glu=True)
+        yg = hip().gemm_rows64(x, packed, glu=True)
         assert yg.shape == (m, n // 2)
         torch.testing.assert_close(yg.double().cpu(), gate, rtol=2e-2, atol=2e-2 * float(gate.abs().max()))
-    alone, _ = hip().gemm_rows64(x[m - 1:].contiguous(), packed, torch.float32)
+    alone = hip().gemm_rows64(x[m - 1:].contiguous(), packed, torch.float32)
     assert torch.equal(alone[0], y32[m - 1])
     assert hip().rows64_takes(max(m, 33), n, k) and not hip().rows64_takes(65, n, k) and not hip().rows64_takes(40, n, k + 512)
     with pytest.raises(hip().KernelError):

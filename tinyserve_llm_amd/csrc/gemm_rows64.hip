@@ -11,11 +11,11 @@
 //   chunk ahead of the compute waves (two buffers, a barrier per chunk). Their loads are few and hit the
 //   cache; in waves of their own they do not queue behind the loads of W (a wave's loads come back in
 //   the order it asked).
-// What precedes and follows the product rides along as in gemm_skinny.hip, operation for operation:
-//   NORM  the staging waves add the residual, write the new residual (workgroup 0), sum the squares in
-//         32 bits and put T((x + res) * nw) into LDS; the row's scale multiplies the finished sums
+// The gate can ride along as in gemm_skinny.hip:
 //   GLU   W = [gate rows | up rows]: waves 0 and 1 take two gate tiles, waves 2 and 3 the up tiles
 //         N / 2 rows below them, and y [M, N / 2] = silu(gate) * up
+// (The norm on the way in, which every workgroup would have to repeat for all of x, was tried in the
+// staging waves and costs more than the norm kernel it saves: 37 µs against 21 + 7 at 64 rows.)
 // W comes as the 16-row packed copy ([N / 16 tiles][K / 32 steps][64 lanes][8]); K is a multiple of
 // 1,024. A row of x meets W's k in ascending order in one accumulator, whatever the other rows are.
 #include <type_traits>
@@ -27,89 +27,47 @@
 
 struct Rows64Args {
   const bf16_t* x;       // [M, K], row stride ldx
-  const bf16_t* res;     // NORM: residual [M, K] or null
-  const bf16_t* nw;      // NORM: norm weight [K]
-  bf16_t* res_out;       // NORM with res: new residual [M, K]
   const bf16_t* w16;     // W [N, K], packed
   void* y;               // [M, N] (GLU: [M, N / 2]), row stride ldy
   int M, N, K;
   int64_t ldx, ldy;
-  float eps;
 };
 
-// What a staging wave has asked for of one chunk: its steps of x for the four blocks of rows, and with
-// the norm the residual's and the weight's.
-template <bool NORM>
-struct Rows64Staged {
-  uint4 x[R64_STAGE_STEPS][4], res[NORM ? R64_STAGE_STEPS : 1][4], nw[NORM ? R64_STAGE_STEPS : 1];
-};
-
-template <bool NORM, bool GLU, typename OUT>
+template <bool GLU, typename OUT>
 __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
   // x as the B operands of the matrix instruction: [buffer][step][block of 16 rows][lane], lane r + 16 g
   // holding k = 8 g .. 8 g + 7 of row r
   __shared__ uint4 xs[2][R64_CHUNK_STEPS][4][TS_WAVE];
-  __shared__ float ssq[4][64];                           // NORM: the staging waves' shares of the rows' sums of squares
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TS_WAVE), lane = threadIdx.x & (TS_WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
   const int nsteps = a.K / SK_KSTEP, nchunks = nsteps / R64_CHUNK_STEPS;   // (a multiple of 4)
 
   if (wave >= 4) {
     // ---- staging waves: wave sw brings steps 2 sw and 2 sw + 1 of every chunk, all four blocks of
-    // rows. It asks for the next chunk before it works on this one, so that a chunk costs the compute
-    // waves a barrier and not a trip to the cache.
+    // rows. It asks for the next chunk before it puts this one into LDS, so that a chunk costs the
+    // compute waves a barrier and not a trip to the cache.
     const int sw = wave - 4;
-    const bool has_res = NORM && a.res != nullptr;
-    float sq[4] = {0.f, 0.f, 0.f, 0.f};                  // this lane's share of rows 16 b + r
     bool ok[4];
-    int64_t xoff[4], roff[4];
+    int64_t xoff[4];
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       ok[b] = 16 * b + r < a.M;                          // rows past M read row 0 and count as zeros
       xoff[b] = (int64_t)(ok[b] ? 16 * b + r : 0) * a.ldx + 8 * g;
-      roff[b] = (int64_t)(ok[b] ? 16 * b + r : 0) * a.K + 8 * g;
     }
-    auto ask = [&](int c, Rows64Staged<NORM>& t) {
+    auto ask = [&](int c, uint4 (&t)[R64_STAGE_STEPS][4]) {
       const int k0 = (c * R64_CHUNK_STEPS + R64_STAGE_STEPS * sw) * SK_KSTEP;   // first k of this wave's steps
-#pragma unroll
-      for (int s = 0; s < R64_STAGE_STEPS; ++s) {
-#pragma unroll
-        for (int b = 0; b < 4; ++b) t.x[s][b] = *(const uint4*)(a.x + xoff[b] + k0 + s * SK_KSTEP);
-        if (NORM) {
-          t.nw[s] = *(const uint4*)(a.nw + k0 + s * SK_KSTEP + 8 * g);
-          // (a missing residual reads x again: the same loads on every path)
-#pragma unroll
-          for (int b = 0; b < 4; ++b)
-            t.res[s][b] = *(const uint4*)((has_res ? a.res + roff[b] : a.x + xoff[b]) + k0 + s * SK_KSTEP);
-        }
-      }
-    };
-    auto put = [&](int c, const Rows64Staged<NORM>& t) {
-      const int k0 = (c * R64_CHUNK_STEPS + R64_STAGE_STEPS * sw) * SK_KSTEP;
 #pragma unroll
       for (int s = 0; s < R64_STAGE_STEPS; ++s)
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-          uint4 v = ok[b] ? t.x[s][b] : make_uint4(0, 0, 0, 0);
-          if (NORM) {
-            float xv[8], rv[8], nv[8];
-            sk_unpack(t.x[s][b], xv);
-            sk_unpack(t.res[s][b], rv);
-            sk_unpack(t.nw[s], nv);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) xv[i] = ok[b] ? xv[i] + (has_res ? rv[i] : 0.f) : 0.f;
-            if (has_res && blockIdx.x == 0 && ok[b]) *(uint4*)(a.res_out + roff[b] + k0 + s * SK_KSTEP) = sk_pack(xv);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-              sq[b] = fmaf(xv[i], xv[i], sq[b]);
-              xv[i] *= nv[i];
-            }
-            v = sk_pack(xv);
-          }
-          xs[c & 1][R64_STAGE_STEPS * sw + s][b][lane] = v;
-        }
+        for (int b = 0; b < 4; ++b) t[s][b] = *(const uint4*)(a.x + xoff[b] + k0 + s * SK_KSTEP);
     };
-    Rows64Staged<NORM> A, B;
+    auto put = [&](int c, const uint4 (&t)[R64_STAGE_STEPS][4]) {
+#pragma unroll
+      for (int s = 0; s < R64_STAGE_STEPS; ++s)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) xs[c & 1][R64_STAGE_STEPS * sw + s][b][lane] = ok[b] ? t[s][b] : make_uint4(0, 0, 0, 0);
+    };
+    uint4 A[R64_STAGE_STEPS][4], B[R64_STAGE_STEPS][4];
     ask(0, A);
     for (int c = 0; c < nchunks; c += 2) {
       ask(c + 1, B);
@@ -119,16 +77,8 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
       put(c + 1, B);
       __syncthreads();
     }
-    if (NORM) {
-#pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        sq[b] += __shfl_xor(sq[b], 16, TS_WAVE);
-        sq[b] += __shfl_xor(sq[b], 32, TS_WAVE);
-        if (g == 0) ssq[sw][16 * b + r] = sq[b];
-      }
-    }
     __syncthreads();            // the compute waves' last chunk
-    __syncthreads();            // the squares are there
+    if (GLU) __syncthreads();   // their exchange
     return;
   }
 
@@ -183,58 +133,45 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
   int base = 0;
   for (; base + R64_RING < nsteps; base += R64_RING) ring(base, std::true_type{});
   ring(base, std::false_type{});
-  // acc[b][j] = sum over k of W[row 16 tile + 4 g + j, k] * f(x)[16 b + r, k]
+  // acc[b][j] = sum over k of W[row 16 tile + 4 g + j, k] * x[16 b + r, k]
   float4_t* ex = (float4_t*)&xs[0][0][0][0];             // [2 up waves][4 blocks][lane]; every read of x is behind the last barrier
-  if (GLU && wave >= 2) {
+  if (GLU) {
+    if (wave >= 2) {
 #pragma unroll
-    for (int b = 0; b < 4; ++b) ex[((wave - 2) * 4 + b) * TS_WAVE + lane] = acc[b];
+      for (int b = 0; b < 4; ++b) ex[((wave - 2) * 4 + b) * TS_WAVE + lane] = acc[b];
+    }
+    __syncthreads();
+    if (wave >= 2) return;
   }
-  __syncthreads();
-  if (GLU && wave >= 2) return;
   OUT* y = (OUT*)a.y;
   const int n0 = GLU ? (2 * blockIdx.x + wave) * 16 + 4 * g : tile * 16 + 4 * g;
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
     const int m = 16 * b + r;
     if (m >= a.M) continue;
-    float inv = 1.0f;
-    if (NORM) inv = 1.0f / sqrtf((ssq[0][m] + ssq[1][m] + ssq[2][m] + ssq[3][m]) / (float)a.K + a.eps);
     float4_t u = {0.f, 0.f, 0.f, 0.f};
     if (GLU) u = ex[(wave * 4 + b) * TS_WAVE + lane];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float s = acc[b][j] * inv;
-      Num<OUT>::st(y + (int64_t)m * a.ldy + n0 + j, GLU ? sk_silu(s) * (u[j] * inv) : s);
-    }
+    for (int j = 0; j < 4; ++j) Num<OUT>::st(y + (int64_t)m * a.ldy + n0 + j, GLU ? sk_silu(acc[b][j]) * u[j] : acc[b][j]);
   }
 }
 
-template <bool NORM, bool GLU, typename OUT>
+template <bool GLU, typename OUT>
 static int r64_launch(const Rows64Args& a, hipStream_t stream) {
-  const int grid = a.N / 64;                             // 64 rows of W per workgroup
-  gemm_rows64_kernel<NORM, GLU, OUT><<<grid, 512, 0, stream>>>(a);
+  gemm_rows64_kernel<GLU, OUT><<<a.N / 64, 512, 0, stream>>>(a);   // 64 rows of W per workgroup
   return ts_check_launch();
 }
 
 // x [M <= 64, K] (row stride ldx), w16: W [N, K] as its 16-row packed copy, y [M, N] or, with glu, [M, N / 2]
-// (row stride ldy; out_f32: 32-bit sums instead of bfloat16). norm_weight non-null: the residual (may be
-// null) and RMSNorm on the way in, res_out the new residual. N a multiple of 64, K of 1,024.
-extern "C" int ts_gemm_rows64_bf16(void* y, const void* x, const void* w16, const void* res, const void* norm_weight,
-                                   void* res_out, int M, int N, int K, int64_t ldx, int64_t ldy, float eps, int glu,
-                                   int out_f32, hipStream_t stream) {
+// (row stride ldy; out_f32: 32-bit sums instead of bfloat16). N a multiple of 64 (128 with glu), K of 1,024.
+extern "C" int ts_gemm_rows64_bf16(void* y, const void* x, const void* w16, int M, int N, int K, int64_t ldx, int64_t ldy,
+                                   int glu, int out_f32, hipStream_t stream) {
   if (M <= 0 || N <= 0) return TS_OK;
-  if (M > 64 || N % 64 || K <= 0 || K % 1024 || ldx < K || (ldx % 8) || !y || !x || !w16) return TS_BAD_SHAPE;
-  if ((((uintptr_t)x) | ((uintptr_t)w16) | ((uintptr_t)res) | ((uintptr_t)norm_weight) | ((uintptr_t)res_out)) & 15) return TS_BAD_SHAPE;
-  if (res && (!norm_weight || !res_out)) return TS_BAD_SHAPE;
+  if (M > 64 || N % (glu ? 128 : 64) || K <= 0 || K % 1024 || ldx < K || (ldx % 8) || !y || !x || !w16) return TS_BAD_SHAPE;
+  if ((((uintptr_t)x) | ((uintptr_t)w16)) & 15) return TS_BAD_SHAPE;
   if (glu && out_f32) return TS_BAD_SHAPE;
-  Rows64Args a = {(const bf16_t*)x, (const bf16_t*)res, (const bf16_t*)norm_weight, (bf16_t*)res_out, (const bf16_t*)w16, y,
-                  M, N, K, ldx, ldy, eps};
-  if (norm_weight) {
-    if (glu) return r64_launch<true, true, bf16_t>(a, stream);
-    if (out_f32) return r64_launch<true, false, float>(a, stream);
-    return r64_launch<true, false, bf16_t>(a, stream);
-  }
-  if (glu) return r64_launch<false, true, bf16_t>(a, stream);
-  if (out_f32) return r64_launch<false, false, float>(a, stream);
-  return r64_launch<false, false, bf16_t>(a, stream);
+  Rows64Args a = {(const bf16_t*)x, (const bf16_t*)w16, y, M, N, K, ldx, ldy};
+  if (glu) return r64_launch<true, bf16_t>(a, stream);
+  if (out_f32) return r64_launch<false, float>(a, stream);
+  return r64_launch<false, bf16_t>(a, stream);
 }

@@ -63,7 +63,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, i, i, i, i, p, p, p],
         "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p],
         "ts_gemm_skinny8_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
-        "ts_gemm_rows64_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, f, i, i, p],
+        "ts_gemm_rows64_bf16": [p, p, p, i, i, i, i64, i64, i, i, p],
         "ts_gemm_skinny_rope_bf16": [p, p, p, p, p, p, i, i, i64, i64, f, i, i, p, p, p, p, p, i, i, i, i, i, i64, i64, i64,
                                      i64, i64, i64, i64, p],
     }
@@ -786,39 +786,25 @@ def rows64_takes(rows: int, n: int, k: int) -> bool:
 
 
 def gemm_rows64(x: torch.Tensor, packed: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, *,
-                residual: torch.Tensor | None = None, norm_weight: torch.Tensor | None = None, eps: float = 0.0,
-                glu: bool = False) -> tuple[torch.Tensor, torch.Tensor | None]:
-    """bfloat16 e(f(x) [M <= 64, K] · W [N, K]^T) for a wide W given as `packed` = pack_weight(W), by
-    the kernel that shares x among 64 rows of W through LDS (gemm_rows64.hip). `norm_weight`,
-    `residual`, `glu` and the two results as in `gemm_skinny`."""
-    _gpu(x, packed, residual, norm_weight)
+                glu: bool = False) -> torch.Tensor:
+    """bfloat16 e(x [M <= 64, K] · W [N, K]^T) for a wide W given as `packed` = pack_weight(W), by the
+    kernel that shares x among 64 rows of W through LDS (gemm_rows64.hip). With `glu`, W holds gate
+    rows then up rows and the result is silu(gate) * up, [M, N / 2]."""
+    _gpu(x, packed)
     _need(x.dtype == torch.bfloat16 and packed.dtype == torch.bfloat16 and x.dim() == 2 and packed.dim() == 4
           and packed.shape[2:] == (64, 8) and packed.is_contiguous(), "gemm_rows64 takes bfloat16 x [M, K] and pack_weight(W)")
     M, K = x.shape
     N = packed.shape[0] * 16
     _need(packed.shape[1] * 32 == K, f"the packed copy is of a weight over {packed.shape[1] * 32}, x is over {K}")
-    _need(1 <= M <= ROWS64_MAX_ROWS and N % 64 == 0 and K % 1024 == 0,
-          f"gemm_rows64 takes up to {ROWS64_MAX_ROWS} rows, N in steps of 64 and K in steps of 1024, not {M} x {K} against {N}")
+    _need(1 <= M <= ROWS64_MAX_ROWS and N % (128 if glu else 64) == 0 and K % 1024 == 0,
+          f"gemm_rows64 takes up to {ROWS64_MAX_ROWS} rows, N in steps of 64 (128 with the gate) and K in steps of 1024, "
+          f"not {M} x {K} against {N}")
     _need(x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0, "rows of x must be dense and 16-byte aligned")
-    norm = norm_weight is not None
-    res_out = None
-    if norm:
-        _need(norm_weight.dtype == torch.bfloat16 and norm_weight.shape == (K,) and norm_weight.is_contiguous(),
-              "the norm weight must be bfloat16 [K]")
-        if residual is not None:
-            _need(residual.shape == x.shape and residual.dtype == x.dtype and residual.is_contiguous(),
-                  "residual must match the input")
-            res_out = torch.empty_like(residual)
-        else:
-            res_out = x
-    else:
-        _need(residual is None, "a residual comes with a norm weight")
     _need(out_dtype == torch.bfloat16 or (out_dtype == torch.float32 and not glu), "32-bit output comes without the gate")
     out = torch.empty((M, N // 2 if glu else N), dtype=out_dtype, device=x.device)
     _run("gemm_rows64", library().ts_gemm_rows64_bf16(
-        _ptr(out), _ptr(x), _ptr(packed), _ptr(residual), _ptr(norm_weight), _ptr(res_out) if residual is not None else None,
-        M, N, K, x.stride(0), out.stride(0), float(eps), int(glu), int(out_dtype == torch.float32), _stream()))
-    return out, res_out
+        _ptr(out), _ptr(x), _ptr(packed), M, N, K, x.stride(0), out.stride(0), int(glu), int(out_dtype == torch.float32), _stream()))
+    return out
 
 
 def qkv_rope_fuses(x: torch.Tensor, weight: torch.Tensor, head_dim: int, k_cache: torch.Tensor | None,
@@ -963,7 +949,7 @@ def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     _need(out_dtype in (torch.bfloat16, torch.float32), f"bfloat16 products come out as bfloat16 or float32, not {out_dtype}")
     if (streams and packed is not None and packed.by16 is not None
             and rows64_takes(x.shape[0], weight.shape[0], x.shape[1])):
-        return gemm_rows64(x, packed.by16, out_dtype)[0]
+        return gemm_rows64(x, packed.by16, out_dtype)
     if _many_rows == "tiled" and tiled_takes(x, weight):
         return gemm_tiled(x, weight, out_dtype=out_dtype)
     return gemm_library(x, weight, out_dtype)

@@ -65,8 +65,8 @@ def linear(x: torch.Tensor | DeferredNorm, weight: torch.Tensor, out_dtype: torc
         x = d.materialize()
     if glu:
         if (out_dtype in (None, torch.bfloat16) and by16 is not None and _streams(x, weight)
-                and hip.rows64_takes(x.shape[0], weight.shape[0], weight.shape[1])):
-            return hip.gemm_rows64(x, by16, glu=True)[0]
+                and hip.rows64_takes(x.shape[0], weight.shape[0], weight.shape[1]) and weight.shape[0] % 128 == 0):
+            return hip.gemm_rows64(x, by16, glu=True)
         if (out_dtype in (None, torch.bfloat16) and _streams(x, weight) and weight.shape[0] % 32 == 0
                 and hip.skinny_fuses(x.shape[0], weight.shape[1], False, True)):
             return hip.gemm_skinny(x, weight, glu=True, packed=by16)[0]
