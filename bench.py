@@ -147,6 +147,9 @@ def main() -> int:
                     help="'prefill': time the 2,048-token prefill alone and print its record (for profiling)")
     ap.add_argument("--scenario", default=None, choices=sorted(SCENARIOS),
                     help="run a whole workload through LLM.generate instead of the decode step")
+    ap.add_argument("--peaks", action="store_true",
+                    help="measure what a kernel that only reads memory and a loop of matrix instructions reach on "
+                         "this GPU, print them beside the published peaks and exit")
     ap.add_argument("--many-rows-products", default="library", choices=["library", "tiled"],
                     help="bfloat16 products of many rows: the vendor's library, or the engine's own tiled kernel")
     args = ap.parse_args()
@@ -156,6 +159,13 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
         return 2
+    if args.peaks:
+        from tinyserve_llm_amd.ops import hip
+        measured = hip.measure_peaks()
+        print(json.dumps({"peaks": {"read": {"measured": measured["read_GBps"], "published": HBM_BYTES_PER_S / 1e9, "unit": "GB/s"},
+                                    "mfma_bf16": {"measured": measured["mfma_bf16_TFLOPs"], "published": PEAK_FLOPS["bf16"] / 1e12,
+                                                  "unit": "TFLOP/s"}}}))
+        return 0
     if args.scenario:
         return scenario(args.scenario, args.layers, args.dtype)
     sizes = SHAPES[args.shape]

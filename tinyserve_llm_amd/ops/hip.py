@@ -64,6 +64,8 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p],
         "ts_gemm_skinny8_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_gemm_rows64_bf16": [p, p, p, i, i, i, i64, i64, i, i, p],
+        "ts_peak_read": [p, ctypes.c_size_t, p, i, p],
+        "ts_peak_mfma": [p, i, i, p],
         "ts_gemm_skinny_rope_bf16": [p, p, p, p, p, p, i, i, i64, i64, f, i, i, p, p, p, p, p, i, i, i, i, i, i64, i64, i64,
                                      i64, i64, i64, i64, p],
     }
@@ -995,3 +997,30 @@ def gemm_library(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype =
             int(sweep is not None),
             _ptr(sweep), 0 if sweep is None else sweep.numel(), _stream()))
     return y
+
+
+def measure_peaks(read_bytes: int = 2 << 30, repeats: int = 5) -> dict[str, float]:
+    """What this GPU reaches in a kernel that only reads `read_bytes` of memory once (GB/s) and in a
+    loop of bfloat16 matrix instructions on registers (TFLOP/s): the best of `repeats` timed runs
+    each (peaks.hip)."""
+    data = torch.empty(read_bytes // 4, dtype=torch.int32, device="cuda").fill_(1)
+    sink = torch.zeros(1 << 16, dtype=torch.float32, device="cuda")
+    cus = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def best(launch) -> float:
+        times = []
+        for _ in range(repeats + 1):
+            begin.record()
+            launch()
+            end.record()
+            end.synchronize()
+            times.append(begin.elapsed_time(end))
+        return min(times[1:]) * 1e-3
+
+    groups, iters = 16 * cus, 1 << 14
+    read_s = best(lambda: _run("peak_read", library().ts_peak_read(_ptr(data), data.numel() * 4, _ptr(sink), 8 * cus, _stream())))
+    mfma_s = best(lambda: _run("peak_mfma", library().ts_peak_mfma(_ptr(sink), iters, groups, _stream())))
+    return {"read_GBps": data.numel() * 4 / read_s / 1e9,
+            "mfma_bf16_TFLOPs": groups * 4 * iters * 4 * 2 * 16 * 16 * 32 / mfma_s / 1e12}
+
