@@ -78,16 +78,18 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, fl
       TS_USE(A, kb);
     }
   } else if (kb < kend) {
+    // (the next step is asked for on every path, this step again where there is none: with a load that
+    // may or may not have been issued the compiler waits for all of them before it uses any)
     KVTile<HD> A, B;
     TS_LOAD(A, kb);
     while (true) {
       const bool more_b = kb + stride < kend;
-      if (more_b) TS_LOAD(B, kb + stride);
+      TS_LOAD(B, more_b ? kb + stride : kb);
       TS_USE(A, kb);
       if (!more_b) break;
       kb += stride;
       const bool more_a = kb + stride < kend;
-      if (more_a) TS_LOAD(A, kb + stride);
+      TS_LOAD(A, more_a ? kb + stride : kb);
       TS_USE(B, kb);
       if (!more_a) break;
       kb += stride;

@@ -48,6 +48,7 @@ static __device__ __forceinline__ int wave_index() { return __builtin_amdgcn_rea
 template <int HD> struct KVTile {
   uint4 k[2][HD / 32];   // two 16-key tiles as A operands: row i of tile tau is key kb + 8 (i / 4) + 4 tau + i % 4
   uint4 v[HD / 16];      // transposed values: keys kb + 8 g .. + 7 of dimension 16 db + r
+  bool vok;              // whether any of this lane's eight keys of v is visible (else v may hold anything and counts as zeros)
 };
 
 // Exchanges between the four lanes (r, g = 0..3) that share a row, by the register swaps of the
@@ -66,8 +67,11 @@ static __device__ __forceinline__ float row_sum(float x) {
   return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
-// Loads the 32-key step at kb (a multiple of 32) of one request's pages into operand registers;
-// keys outside [lo, pos] read as zeros.
+// Asks for the 32-key step at kb (a multiple of 32, kb <= pos) of one request's pages, straight into
+// operand registers. Every lane loads, whatever its keys, from an address inside the request's pages
+// (that of a visible key where its own is not), by the same instructions on every path: the compiler
+// can then count the loads under way and wait for a step's own only, while the next step's are in
+// flight. Keys outside [lo, pos] are masked by the softmax; values outside count as zeros (`vok`).
 template <int HD>
 static __device__ __forceinline__ void load_tile(KVTile<HD>& T, int kb, int r, int g, int lo, int pos, int kvh,
                                                  const int32_t* __restrict__ table, const PageMath pm,
@@ -75,49 +79,36 @@ static __device__ __forceinline__ void load_tile(KVTile<HD>& T, int kb, int r, i
                                                  int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vh,
                                                  int64_t vd) {
   constexpr int NC = HD / 32, NDB = HD / 16;
+  int64_t koff[2], voff;      // (offsets, not pointers: the loads below are then plainly loads from the two caches)
   if (pm.whole_steps()) {
     // one page for the whole step: its base addresses are scalars, the lanes add fixed offsets
+    // (the page is the request's since kb <= pos, and all its slots are memory of the pool)
     const int pg = pm.page(kb);
     const int64_t page = table[pg];
     const int slot = pm.slot(kb, pg);
-    const bf16_t* kbase = k_cache + page * kp + (int64_t)slot * ks + (int64_t)kvh * kh;
-    const bf16_t* vbase = v_cache + page * vp + slot + (int64_t)kvh * vh;
-    const bool inner = kb >= lo && kb + 31 <= pos;
+    const int64_t kbase = page * kp + (int64_t)slot * ks + (int64_t)kvh * kh;
+#pragma unroll
+    for (int tau = 0; tau < 2; ++tau) koff[tau] = kbase + (int64_t)(8 * (r >> 2) + 4 * tau + (r & 3)) * ks + 8 * g;
+    voff = page * vp + slot + (int64_t)kvh * vh + 8 * g + (int64_t)r * vd;
+  } else {
 #pragma unroll
     for (int tau = 0; tau < 2; ++tau) {
-      const int koff = 8 * (r >> 2) + 4 * tau + (r & 3);
-      const bf16_t* kr = kbase + (int64_t)koff * ks + 8 * g;
-      const bool ok = inner || (kb + koff <= pos && kb + koff >= lo);
-#pragma unroll
-      for (int c = 0; c < NC; ++c) T.k[tau][c] = ok ? *(const uint4*)(kr + 32 * c) : make_uint4(0, 0, 0, 0);
-    }
-    const bf16_t* vr = vbase + 8 * g + (int64_t)r * vd;
-    const bool vok = inner || (kb + 8 * g <= pos && kb + 8 * g + 7 >= lo);
-#pragma unroll
-    for (int db = 0; db < NDB; ++db) T.v[db] = vok ? *(const uint4*)(vr + (int64_t)(16 * db) * vd) : make_uint4(0, 0, 0, 0);
-    return;
-  }
-#pragma unroll
-  for (int tau = 0; tau < 2; ++tau) {
-    const int key = kb + 8 * (r >> 2) + 4 * tau + (r & 3);
-#pragma unroll
-    for (int c = 0; c < NC; ++c) T.k[tau][c] = make_uint4(0, 0, 0, 0);
-    if (key <= pos && key >= lo) {
+      const int key = min(max(kb + 8 * (r >> 2) + 4 * tau + (r & 3), lo), pos);     // a visible key, for the address
       const int pg = pm.page(key);
-      const bf16_t* kr = k_cache + (int64_t)table[pg] * kp + (int64_t)pm.slot(key, pg) * ks + (int64_t)kvh * kh + 8 * g;
-#pragma unroll
-      for (int c = 0; c < NC; ++c) T.k[tau][c] = *(const uint4*)(kr + 32 * c);
+      koff[tau] = (int64_t)table[pg] * kp + (int64_t)pm.slot(key, pg) * ks + (int64_t)kvh * kh + 8 * g;
     }
-  }
-  const int vkey = kb + 8 * g;      // page sizes are multiples of 8: the 8 keys share a page
-#pragma unroll
-  for (int db = 0; db < NDB; ++db) T.v[db] = make_uint4(0, 0, 0, 0);
-  if (vkey <= pos && vkey + 7 >= lo) {
+    // page sizes are multiples of 8: the 8 keys share a page
+    const int vkey = (kb + 8 * g <= pos && kb + 8 * g + 7 >= lo) ? kb + 8 * g : (pos & ~7);
     const int pg = pm.page(vkey);
-    const bf16_t* vr = v_cache + (int64_t)table[pg] * vp + pm.slot(vkey, pg) + (int64_t)kvh * vh + (int64_t)r * vd;
-#pragma unroll
-    for (int db = 0; db < NDB; ++db) T.v[db] = *(const uint4*)(vr + (int64_t)(16 * db) * vd);
+    voff = (int64_t)table[pg] * vp + pm.slot(vkey, pg) + (int64_t)kvh * vh + (int64_t)r * vd;
   }
+  T.vok = kb + 8 * g <= pos && kb + 8 * g + 7 >= lo;
+#pragma unroll
+  for (int tau = 0; tau < 2; ++tau)
+#pragma unroll
+    for (int c = 0; c < NC; ++c) T.k[tau][c] = *(const uint4*)(k_cache + koff[tau] + 32 * c);
+#pragma unroll
+  for (int db = 0; db < NDB; ++db) T.v[db] = *(const uint4*)(v_cache + voff + (int64_t)(16 * db) * vd);
 }
 
 #define TS_LAZY_MAX 8.0f     // a row's reference maximum is raised when a score exceeds it by more than this (log2 units)
@@ -182,7 +173,7 @@ static __device__ __forceinline__ void use_tile(const KVTile<HD>& T, int kb, int
   const uint4 pa = make_uint4(pack_bf16(p[0][0], p[0][1]), pack_bf16(p[0][2], p[0][3]), pack_bf16(p[1][0], p[1][1]),
                               pack_bf16(p[1][2], p[1][3]));
 #pragma unroll
-  for (int db = 0; db < NDB; ++db) o[db] = mfma32(pa, T.v[db], o[db]);
+  for (int db = 0; db < NDB; ++db) o[db] = mfma32(pa, (MASKED && !T.vok) ? make_uint4(0, 0, 0, 0) : T.v[db], o[db]);
 }
 
 // The same, choosing the variant: `pmin` and `lomax` are the smallest position and the largest

@@ -215,6 +215,7 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
       for (int c = 0; c < NC; ++c) { T.k[0][c] = stage[buf][c][lane]; T.k[1][c] = stage[buf][NC + c][lane]; }
 #pragma unroll
       for (int db = 0; db < NDB; ++db) T.v[db] = stage[buf][2 * NC + db][lane];
+      T.vok = true;                          // (what lies outside the range went into LDS as zeros)
       if (kb + 32 < kend) put(buf ^ 1);      // the other buffer was last read before the previous barrier
       if (kb + 64 < kend) fetch(kb + 64);
 #pragma unroll
