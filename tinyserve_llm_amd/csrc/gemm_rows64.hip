@@ -5,7 +5,7 @@
 // once per 32 rows of W, which is twice the bytes of W itself. Here a workgroup owns 64 rows of W and
 // splits the work between two kinds of wave:
 //   four compute waves, one 16-row tile of W each over the whole of K: the tile streams from memory
-//   straight into MFMA operands, 32 steps of 32 k under way at any time (a step's register is asked for
+//   straight into MFMA operands, 16 steps of 32 k under way at any time (a step's register is asked for
 //   again as soon as it has been used), and the four 16-row blocks of x come out of LDS;
 //   four staging waves, which bring x into LDS in chunks of 256 k, in the order the lanes read it, one
 //   chunk ahead of the compute waves (two buffers, a barrier per chunk). Their loads are few and hit the
@@ -22,7 +22,8 @@
 #include "skinny_ops.h"
 
 #define R64_CHUNK_STEPS 8         // 32-wide k steps per chunk of x in LDS
-#define R64_RING 32               // steps of W a compute wave has under way (four chunks)
+#define R64_RING 16               // steps of W a compute wave has under way (two chunks): with 32 the chip had 32 MB under way and
+                                  // every load, x's among them, came back some 5 us later (the gate|up product of 64 rows 20.7 us, 19.7 with 16)
 #define R64_STAGE_STEPS (R64_CHUNK_STEPS / 4)   // steps of a chunk that one staging wave brings
 
 struct Rows64Args {
@@ -97,7 +98,7 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
 #pragma unroll
   for (int b = 0; b < 4; ++b) acc[b] = (float4_t){0.f, 0.f, 0.f, 0.f};
   __syncthreads();              // chunk 0 is there
-  // 32 steps at a time, each register of the ring asked for again once it has been used; the last 32 ask for nothing
+  // a turn of the ring at a time, each register asked for again once it has been used; the last turn asks for nothing
   auto ring = [&](int base, auto more) {
 #pragma unroll
     for (int h = 0; h < R64_RING / R64_CHUNK_STEPS; ++h) {
@@ -108,14 +109,14 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int b = 0; b < 4; ++b) xb[0][i][b] = xs[h & 1][i][b][lane];
+        for (int b = 0; b < 4; ++b) xb[0][i][b] = xs[(base / R64_CHUNK_STEPS + h) & 1][i][b][lane];
 #pragma unroll
       for (int q = 0; q < PAIRS; ++q) {
         if (q + 1 < PAIRS) {
 #pragma unroll
           for (int i = 0; i < 2; ++i)
 #pragma unroll
-            for (int b = 0; b < 4; ++b) xb[(q + 1) & 1][i][b] = xs[h & 1][2 * (q + 1) + i][b][lane];
+            for (int b = 0; b < 4; ++b) xb[(q + 1) & 1][i][b] = xs[(base / R64_CHUNK_STEPS + h) & 1][2 * (q + 1) + i][b][lane];
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
