@@ -81,3 +81,23 @@ def test_decode_plan_divides_the_context_into_32_key_steps_per_wave():
     assert hip.decode_plan(31, 8, 4, 128, 8192) == (8192, 4)       # 248 workgroups are as good as 256
     assert hip.decode_plan(24, 8, 4, 64, 2304) == (2304, 8)        # and so are 192
     assert hip.decode_plan(80, 8, 4, 64, 2304) == (256, 8)         # 640 of 768 are not
+
+
+def test_which_kernel_takes_a_projection_of_few_rows():
+    """The row counts and shapes at which the 8-row form, the shared-x kernel and their fused
+    epilogues are chosen (the thresholds are measured; this pins what the parts rely on)."""
+    # 8-row form: up to 4 rows at any width, up to 8 rows for matrices of up to 2,048 rows; K in waves of 64 steps
+    assert hip.skinny8_takes(1, 128256, 2048) and hip.skinny8_takes(4, 16384, 2048) and hip.skinny8_takes(8, 2048, 8192)
+    assert not hip.skinny8_takes(8, 16384, 2048) and not hip.skinny8_takes(9, 2048, 2048) and not hip.skinny8_takes(1, 2048, 2000)
+    for k in (256, 2048, 8192, 14336, 16384):
+        steps = hip.skinny8_steps(k)
+        assert steps in (4, 8, 16) and k % (64 * steps) == 0 and k // (64 * steps) <= 16
+    assert hip.skinny8_steps(100) == 0
+    # shared-x kernel: 33 to 64 rows against at least 8,192 rows of W in steps of 64, K in steps of 1,024
+    assert hip.rows64_takes(33, 16384, 2048) and hip.rows64_takes(64, 128256, 2048) and hip.rows64_takes(40, 8192, 3072)
+    for rows, n, k in ((32, 16384, 2048), (65, 16384, 2048), (40, 4096, 2048), (40, 8200, 2048), (40, 16384, 2560)):
+        assert not hip.rows64_takes(rows, n, k)
+    # the fused norm serves one block of 16 rows; the gate alone up to 64 rows over reductions of up to 2,048
+    assert hip.skinny_fuses(16, 2048, True, True) and not hip.skinny_fuses(17, 2048, True, True)
+    assert hip.skinny_fuses(64, 2048, False, True) and not hip.skinny_fuses(65, 2048, False, True)
+    assert not hip.skinny_fuses(40, 4096, False, True)
