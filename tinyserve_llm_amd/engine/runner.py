@@ -357,13 +357,15 @@ class DecodeGraphs:
         draw_temps = dev_i32[start + 2 * size:start + 3 * size].view(torch.float32)
         # once without capture: libraries set up their workspaces, the kernel library loads, and
         # the matrix library's candidates for this batch size are timed and the fastest kept
-        side = torch.cuda.Stream(device=r.device)
-        side.wait_stream(torch.cuda.current_stream(r.device))
         # (this run and the first replay feed the same tokens: keys and values land in the same slots
         # twice, which changes nothing, but a mixer's state would take the step twice, so the state
-        # slots are put back as they were)
+        # slots are put back as they were. The copies are queued on the current stream before the
+        # side stream is told to wait for it: the side stream's run, which writes the slots, then
+        # starts after the copies have been taken.)
         states = r.storage.state_tensors()
         before = [t.clone() for t in states]
+        side = torch.cuda.Stream(device=r.device)
+        side.wait_stream(torch.cuda.current_stream(r.device))
         with hip.library_tuning(), torch.cuda.stream(side):      # (the sweep buffer belongs to the current stream)
             hidden, residual = r.model.forward(ctx, r.memory)
             hip.sample(r.model.logits(hidden, residual, rows), draw_temps, draw_keys, self.seed)
