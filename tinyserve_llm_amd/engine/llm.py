@@ -47,6 +47,20 @@ class Completion:
     first_token_time: float
     finish_time: float
 
+    @classmethod
+    def of(cls, output: RequestOutput, tokenizer=None) -> "Completion":
+        """A finished request as its caller sees it: the samples' tokens in fork order (and their
+        text, if there is a tokenizer), the time of the first token of any sample and of the last
+        sample's end (llm_engine.py:170-185)."""
+        first = output.sequences[0]
+        samples = [list(seq.output_token_ids) for seq in output.sequences]
+        return cls(
+            output.request_id, list(first.prompt_token_ids), samples,
+            None if tokenizer is None else [tokenizer.decode(ids, skip_special_tokens=True) for ids in samples],
+            [seq.finish_reason for seq in output.sequences], first.arrival_time,
+            min(seq.first_token_time for seq in output.sequences),
+            max(seq.finish_time for seq in output.sequences))
+
 
 class LLM:
     def __init__(
@@ -246,22 +260,16 @@ class LLM:
 
     def generate(self, prompts: list[str] | list[list[int]],
                  params: SamplingParams | list[SamplingParams] = SamplingParams()) -> list[Completion]:
-        """Runs the prompts to completion; results in prompt order."""
-        params = params if isinstance(params, list) else [params] * len(prompts)
-        order = [self.add_request(p, sp) for p, sp in zip(prompts, params, strict=True)]
-        done: dict[int, RequestOutput] = {}
+        """Queues every prompt (one `SamplingParams` for all, or one each), steps the engine until
+        both queues are empty, and returns the completions in the order of the prompts
+        (llm_engine.py:159-168)."""
+        each = params if isinstance(params, list) else [params] * len(prompts)
+        if len(each) != len(prompts):
+            raise ValueError(f"{len(prompts)} prompts but {len(each)} sampling parameters")
+        place = {self.add_request(prompt, sp): i for i, (prompt, sp) in enumerate(zip(prompts, each))}
+        results: list[Completion | None] = [None] * len(prompts)
         while self.scheduler.has_unfinished():
-            for output in self.step():
-                done[output.request_id] = output
-        return [self._completion(done[r]) for r in order]
-
-    def _completion(self, output: RequestOutput) -> Completion:
-        seqs = output.sequences
-        token_ids = [list(s.output_token_ids) for s in seqs]
-        texts = None
-        if self.tokenizer is not None:
-            texts = [self.tokenizer.decode(t, skip_special_tokens=True) for t in token_ids]
-        return Completion(
-            request_id=output.request_id, prompt_token_ids=list(seqs[0].prompt_token_ids), token_ids=token_ids,
-            texts=texts, finish_reasons=[s.finish_reason for s in seqs], arrival_time=seqs[0].arrival_time,
-            first_token_time=min(s.first_token_time for s in seqs), finish_time=max(s.finish_time for s in seqs))
+            for finished in self.step():
+                if finished.request_id in place:          # (requests queued through add_request run along)
+                    results[place[finished.request_id]] = Completion.of(finished, self.tokenizer)
+        return results

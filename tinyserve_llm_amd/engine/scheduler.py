@@ -26,7 +26,8 @@ from __future__ import annotations
 import itertools
 import math
 import operator
-from dataclasses import dataclass, replace
+from collections import Counter
+from dataclasses import dataclass
 from typing import Literal, NamedTuple
 
 from tinyserve_llm_amd.cache.manager import AdmissionCost, KVCacheManager
@@ -78,6 +79,17 @@ class ScheduledSeq(NamedTuple):
 _START = operator.attrgetter("start")
 
 
+class _Offer(NamedTuple):
+    """The terms of one admission: the sequence's tokens, how many of the uncached ones the step
+    would feed, the pages that takes in every page space, the share of the sequence found in the
+    cache, and the samples it will split off at its first token."""
+    tokens: list[int]
+    feed: int
+    per_space: list[int]
+    hit: float
+    forks: int
+
+
 class RequestOutput(NamedTuple):
     request_id: int
     sequences: list[Sequence]
@@ -93,7 +105,7 @@ class Scheduler:
         self.watermark_blocks = math.ceil(config.watermark * kv.num_blocks)
         self._seq_ids = itertools.count()
         self._request_ids = itertools.count()
-        self.counters = SchedulerStats()
+        self.tally: Counter[str] = Counter()       # the running totals of `SchedulerStats`, by field name
 
     def has_unfinished(self) -> bool:
         return bool(self.waiting or self.running)
@@ -193,13 +205,13 @@ class Scheduler:
                 victim = self._lowest_unscheduled(now, exclude=seq, gone=gone)
                 if victim is None:
                     break
-                self._preempt(victim)
+                self._send_back(victim)
                 gone.add(victim.seq_id)
                 if victim in mine:
                     mine.remove(victim)
                 fits = self.kv.try_append_one(seq.seq_id, tokens[0]) if one else self.kv.can_append(seq.seq_id, len(tokens))
             if not fits:
-                self._preempt(seq)
+                self._send_back(seq)
                 gone.add(seq.seq_id)
                 break
             if not one:
@@ -208,9 +220,9 @@ class Scheduler:
             samples = 1
             if want_prefill:
                 samples = 0 if not final else (seq.params.n if seq.awaits_first_token() else 1)
-                self.counters.prefill_tokens += len(tokens)
+                self.tally["prefill_tokens"] += len(tokens)
             else:
-                self.counters.decode_tokens += 1
+                self.tally["decode_tokens"] += 1
             seq.in_step = True
             scheduled.append(ScheduledSeq(seq, tokens, samples, seq.num_computed))
             budget -= len(tokens)
@@ -221,70 +233,74 @@ class Scheduler:
                 and not s.in_step]
         return min(pool, key=lambda s: self._score(s.admission_hit, s, now), default=None)
 
-    def _preempt(self, seq: Sequence) -> None:
-        """Pages go back (staying in the prefix cache while nobody needs them); the sequence
-        waits again with its outputs and its original arrival time (scheduler.py:152-158)."""
-        self.kv.release(seq.seq_id)
-        seq.status = SequenceStatus.WAITING
-        seq.num_preemptions += 1
-        seq.num_computed = 0
-        seq.prefill_target = 0
-        self.counters.preemptions += 1
+    def _send_back(self, seq: Sequence) -> None:
+        """Preemption (scheduler.py:152-158): the sequence leaves the running list for the end of the
+        waiting queue, keeping its outputs and its place in time; its pages go back to the manager,
+        where they stay findable by prefix while nobody needs them."""
         self.running.remove(seq)
+        self.kv.release(seq.seq_id)
+        seq.back_to_waiting()
         self.waiting.append(seq)
+        self.tally["preemptions"] += 1
 
     def _owed_forks(self) -> int:
         """Sequences that running requests will still split off when their prompts end."""
         return sum(s.params.n - 1 for s in self.running if s.awaits_first_token())
 
+    def _offer(self, seq: Sequence, budget: int) -> "_Offer":
+        """What admitting `seq` now would feed and take, priced against the cache as it is at this
+        moment (an admission made a moment ago may have evicted pages an older price counted on)."""
+        tokens = seq.all_token_ids
+        whole = self.kv.calculate_admission_cost(tokens)
+        feed = self._chunk(whole.prefill_tokens, budget)
+        return _Offer(tokens, feed, self.kv.calculate_admission_cost(tokens, feed).per_space,
+                      self._hit(len(tokens), whole), seq.params.n - 1 if seq.awaits_first_token() else 0)
+
+    def _room_for(self, offer: "_Offer", owed: int) -> bool:
+        """Seats: the sequence and every sample it or an earlier admission still owes. Pages: its own,
+        one per owed sample (the copy of a shared last page), and the watermark."""
+        seats = len(self.running) + owed + offer.forks + 1
+        return (offer.feed >= 1 and seats <= self.config.max_num_seqs
+                and self.kv.fits(offer.per_space, owed + offer.forks + self.watermark_blocks))
+
+    def _seat(self, seq: Sequence, offer: "_Offer") -> ScheduledSeq:
+        """Makes the admission: pages reserved for the first portion, the books updated."""
+        took = self.kv.allocate(seq.seq_id, offer.tokens, offer.feed)
+        assert took is not None, "the price was taken a moment ago"
+        cached = self.kv.num_cached_tokens(seq.seq_id)
+        fed = offer.tokens[cached:cached + offer.feed]
+        self.tally["readmissions" if seq.num_preemptions else "admissions"] += 1
+        self.tally["cached_tokens"] += cached
+        self.tally["prefill_tokens"] += len(fed)
+        seq.start_running(offer.hit, target=len(offer.tokens), computed=cached)
+        self.running.append(seq)
+        ends_prompt = cached + len(fed) >= len(offer.tokens)
+        return ScheduledSeq(seq, fed, (offer.forks + 1) if ends_prompt else 0, cached)
+
     def _admit(self, now: float, budget: int) -> list[ScheduledSeq]:
-        """Admits waiting sequences, best score first, within the token budget, the sequence cap
-        and the watermark. A candidate that does not fit is skipped, unless it has waited
-        `max_skip_wait`: then admission stops so that what frees up goes to it
-        (scheduler.py:160-204)."""
-        admitted: list[ScheduledSeq] = []
-        owed = self._owed_forks()                # kept up to date as groups are admitted below
-        if budget <= 0 or not self.waiting or len(self.running) + owed + 1 > self.config.max_num_seqs:
-            return admitted                      # no one can be admitted: nothing to rank
-        for seq, _ in self._ranked_waiting(now):
+        """New admissions of a step (the policy of scheduler.py:160-204, over portions): waiting
+        sequences are offered a seat in the order of their scores; one that has no room is passed
+        over, except that one which has waited `max_skip_wait` ends the round, so that what frees up
+        next goes to it and not to smaller requests behind it."""
+        seated: list[ScheduledSeq] = []
+        owed = self._owed_forks()
+        if not self.waiting or len(self.running) + owed >= self.config.max_num_seqs:
+            return seated                        # nobody to admit or no seat: no ranking needed
+        for seq, _ in (self._ranked_waiting(now) if budget > 0 else ()):
+            offer = self._offer(seq, budget)
+            if not self._room_for(offer, owed):
+                if now - seq.arrival_time < self.config.max_skip_wait:
+                    continue
+                break
+            entry = self._seat(seq, offer)
+            seated.append(entry)
+            owed += offer.forks
+            budget -= len(entry.token_ids)
             if budget <= 0:
                 break
-            tokens = seq.all_token_ids
-            whole = self.kv.calculate_admission_cost(tokens)      # fresh: earlier admissions may have evicted
-            feed = self._chunk(whole.prefill_tokens, budget)
-            cost = self.kv.calculate_admission_cost(tokens, feed)
-            hit = self._hit(len(tokens), whole)
-            forks = seq.params.n - 1 if seq.awaits_first_token() else 0
-            fits = (feed >= 1
-                    and len(self.running) + owed + 1 + forks <= self.config.max_num_seqs
-                    and self.kv.fits(cost.per_space, owed + forks + self.watermark_blocks))
-            if not fits:
-                if now - seq.arrival_time >= self.config.max_skip_wait:
-                    break
-                continue
-            assert self.kv.allocate(seq.seq_id, tokens, feed) is not None
-            cached = self.kv.num_cached_tokens(seq.seq_id)
-            fed = tokens[cached:cached + feed]
-            if seq.num_preemptions:
-                self.counters.readmissions += 1
-            else:
-                self.counters.admissions += 1
-            self.counters.cached_tokens += cached
-            self.counters.prefill_tokens += len(fed)
-            budget -= len(fed)
-            seq.status = SequenceStatus.RUNNING
-            seq.admission_hit = hit
-            seq.prefill_target = len(tokens)
-            seq.num_computed = cached
-            final = cached + len(fed) >= len(tokens)
-            samples = 0 if not final else (seq.params.n if forks else 1)
-            self.running.append(seq)
-            owed += forks
-            seq.in_step = True
-            admitted.append(ScheduledSeq(seq, fed, samples, cached))
-        if admitted:
+        if seated:
             self.waiting = [s for s in self.waiting if s.status is SequenceStatus.WAITING]
-        return admitted
+        return seated
 
     # ---- after the model ran ----------------------------------------------------------------
     def _split_off(self, first: Sequence, how_many: int) -> list[Sequence]:
@@ -387,4 +403,5 @@ class Scheduler:
         return self._retire(ended), [b for b in ahead or () if b.seq.seq_id in fed_ahead]
 
     def stats(self) -> SchedulerStats:
-        return replace(self.counters, num_waiting=len(self.waiting), num_running=len(self.running))
+        """The totals so far and the lengths of the two queues as they are now."""
+        return SchedulerStats(num_waiting=len(self.waiting), num_running=len(self.running), **self.tally)

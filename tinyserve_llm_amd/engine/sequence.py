@@ -81,5 +81,16 @@ class Sequence:
                         status=self.status, sample_index=sample_index, admission_hit=self.admission_hit,
                         prefill_target=self.prefill_target, num_computed=self.num_computed)
 
+    def start_running(self, hit: float, target: int, computed: int) -> None:
+        """Admitted: `computed` of its first `target` tokens were found in the cache."""
+        self.status, self.admission_hit = SequenceStatus.RUNNING, hit
+        self.prefill_target, self.num_computed, self.in_step = target, computed, True
+
+    def back_to_waiting(self) -> None:
+        """Preempted: nothing of it is in the cache any more; outputs and arrival time stay."""
+        self.status = SequenceStatus.WAITING
+        self.num_preemptions += 1
+        self.prefill_target = self.num_computed = 0
+
     def finish(self, reason: Literal["eos", "length"], now: float) -> None:
         self.status, self.finish_reason, self.finish_time = SequenceStatus.FINISHED, reason, now
