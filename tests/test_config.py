@@ -98,3 +98,44 @@ def test_spec_holds_every_size_from_the_config():
     assert "lm_head.weight" not in spec.checkpoint and spec.optional == ("lm_head.weight",)
     d = spec.checkpoint["model.layers.3.self_attn.v_proj.weight"]
     assert (d.param, d.row, d.rows) == ("layers.3.mixer.qkv", 2048 + 512, 512)
+
+
+def test_an_architecture_is_found_by_its_configurations_type_and_written_from_its_fields(tmp_path):
+    """A configuration class needs `from_dict` only: the registry finds the architecture of a typed
+    configuration by the class `config_from_dict` belongs to and writes config.json from the
+    fields, adding the keys by which the folder is resolved again."""
+    import json
+    from dataclasses import dataclass
+
+    from tinyserve_llm_amd.models import registry
+
+    @dataclass(frozen=True)
+    class Small:
+        width: int
+        depth: int = 2
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(int(raw["width"]), int(raw.get("depth", 2)))
+
+    arch = registry.Architecture("SmallForCausalLM", ("small",), Small.from_dict, lambda c: None)
+    assert arch.owns(Small(8)) and not arch.owns(object())
+    assert arch.to_dict(Small(8, 3)) == dict(width=8, depth=3, architectures=["SmallForCausalLM"], model_type="small")
+    registry.register_architecture(arch)
+    try:
+        assert registry.architecture_of(Small(8)) is arch
+        registry.write_config(str(tmp_path), Small(8, 5))
+        with open(tmp_path / "config.json") as f:
+            assert json.load(f)["depth"] == 5
+        found, config = registry.read_config(str(tmp_path))
+        assert found is arch and config == Small(8, 5)
+    finally:
+        del registry.ARCHITECTURES["SmallForCausalLM"]
+    import pytest as _pytest
+    with _pytest.raises(NotImplementedError, match="Small"):
+        registry.architecture_of(Small(8))
+    # the Llama configuration goes out in the Hub's spelling, by its own writer
+    from tests.helpers import TINY_B
+    llama = registry.architecture_of(TINY_B)
+    assert llama.name == "LlamaForCausalLM" and llama.to_dict(TINY_B)["rope_scaling"]["rope_type"] == "llama3"
+    assert llama.config_from_dict(llama.to_dict(TINY_B)) == TINY_B

@@ -569,3 +569,101 @@ def test_random_workloads_generate_the_same_under_every_engine_setting(case, fol
         outs.append([(c.token_ids, c.finish_reasons) for c in llm.generate(prompts, params)])
         assert caching or llm.manager.num_available_blocks() == llm.manager.num_blocks, "pages leaked"
     assert outs[1] == outs[0] and outs[2] == outs[0] and outs[3] == outs[0]
+
+
+def test_recorded_steps_are_bounded_and_dropping_them_changes_nothing(folder_b):
+    """At most `max_decode_graphs` recorded steps are kept, the one replayed longest ago goes first,
+    and their own buffers stay inside the budget; walking many (batch size, context) keys twice
+    leaves the device's memory where the first walk left it, and an engine that keeps only three
+    graphs generates what an engine without graphs does."""
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+    sc = SchedulerConfig(max_model_len=320, max_num_seqs=40, max_num_batched_tokens=160, max_prefill_chunk=32)
+    llm = LLM(folder_b, sc, CacheConfig(block_size=16), dtype=torch.float32, num_blocks=400, seed=5, max_decode_graphs=6,
+              record_decode_steps=[3, (9, 100)])
+    graphs = llm.runner.graphs
+    assert list(graphs.graphs) == [(3, 32), (16, 16)], "recorded at start: 320 positions reach 512 in pages of 16; 9 requests in 16 rows"
+    keys = [(batch, context) for context in (60, 300) for batch in (1, 2, 3, 4, 5, 6, 7, 8, 9, 17, 25, 33)]
+    held = []
+    for walk in range(2):
+        for batch, context in keys:
+            key = graphs.record(batch, context)
+            assert key in graphs.graphs and len(graphs.graphs) <= 6 and list(graphs.graphs)[-1] == key
+            assert graphs.memory_held() <= graphs.memory_budget
+        torch.cuda.synchronize()
+        held.append(torch.cuda.memory_allocated())
+    assert graphs.recorded >= 2 * len(keys) - 6 and graphs.dropped == graphs.recorded - 6, (graphs.recorded, graphs.dropped)
+    assert held[1] <= held[0], f"the second walk took more memory: {held}"
+    # a budget of bytes: graphs of 40 rows hold 40 x 384 logits each; room for two of them
+    tight = LLM(folder_b, sc, CacheConfig(block_size=16), dtype=torch.float32, num_blocks=400, seed=5,
+                decode_graph_memory=2 * 40 * 384 * 4 + 4096)
+    for context in (10, 300, 10, 300):
+        tight.runner.graphs.record(40, context)
+        tight.runner.graphs.record(33, context)       # the same graph: 40 rows
+        tight.runner.graphs.record(1, context)
+    assert tight.runner.graphs.memory_held() <= tight.runner.graphs.memory_budget and tight.runner.graphs.dropped > 0
+    prompts = [prompt(70 + i, 3 + 5 * i, 384) for i in range(11)]
+    params = [SamplingParams(max_tokens=3 + 2 * (i % 6), temperature=0.7 if i % 3 == 0 else 0.0, ignore_eos=True) for i in range(11)]
+    outs = []
+    for cap in (3, None):
+        one = LLM(folder_b, sc, CacheConfig(block_size=16), dtype=torch.float32, num_blocks=400, seed=5,
+                  decode_graphs=cap is not None, max_decode_graphs=cap or 64)
+        outs.append([r.token_ids for r in one.generate(prompts, params)])
+        if cap:
+            assert one.runner.graphs.dropped > 0 and len(one.runner.graphs.graphs) <= cap
+    assert outs[0] == outs[1]
+
+
+def test_drawn_tokens_say_when_the_graph_has_overwritten_them(folder_a):
+    """The tokens of a replayed step stay on the device until the graph's next replay and in one of
+    two landing places on the host until the replay after that; a result held longer refuses to be
+    read instead of handing out another step's tokens."""
+    from tinyserve_llm_amd.engine.runner import DrawnTokens, StepEntry, StepError
+    llm = engine(folder_a)
+    m, r = llm.manager, llm.runner
+    ids = prompt(3, 9, 256)
+    m.allocate(0, ids)
+    r.step([StepEntry(0, ids, 0, [])])
+    m.commit(0, len(ids))
+    held = []
+    for k in range(3):
+        m.append_slots(0, [5 + k])
+        held.append(r.step_sample([StepEntry(0, [5 + k], len(ids) + k, [0])], [0.0], [k], llm.seed))
+        m.commit(0, 1)
+    assert all(isinstance(h, DrawnTokens) for h in held)
+    assert len(held[2].tolist()) == 1 and len(held[1].tolist()) == 1 and held[2].on_device.shape == (1,)
+    with pytest.raises(StepError, match="replayed twice"):
+        held[0].tolist()
+    with pytest.raises(StepError, match="replayed since"):
+        held[1].on_device
+    m.release(0)
+
+
+def test_without_library_timing_two_processes_draw_the_same_bfloat16_tokens(tmp_path):
+    """Steps of more than 64 requests take their projections from the vendor's matrix library. With
+    its candidates timed, which of them serves a shape may differ from run to run; with the timing
+    off (`--no-library-timing`) every shape keeps the library's first candidate, the record says
+    so, and two processes generate the same tokens."""
+    from tinyserve_llm_amd.config import LlamaConfig
+    from tinyserve_llm_amd.weights.random_init import write_random_model
+    config = LlamaConfig(vocab_size=300, hidden_size=256, intermediate_size=512, num_hidden_layers=2,
+                         num_attention_heads=4, num_key_value_heads=2, head_dim=64, max_position_embeddings=256,
+                         rms_norm_eps=1e-5, rope_theta=10000.0, rope_scaling=None, tie_word_embeddings=True, eos_token_id=299)
+    folder = write_random_model(str(tmp_path / "m"), config, 6, torch.bfloat16)
+    records = []
+    for run in range(2):
+        out = str(tmp_path / f"r{run}.json")
+        cmd = [sys.executable, "-m", "tinyserve_llm_amd.generate", "--model", folder, "--prompt-lengths",
+               ",".join(str(3 + i % 11) for i in range(80)), "--max-tokens", "6", "--temperature", "0.8", "--ignore-eos",
+               "--block-size", "16", "--num-blocks", "400", "--max-model-len", "96", "--max-num-seqs", "96",
+               "--max-num-batched-tokens", "512", "--no-library-timing", "--out", out]
+        r = subprocess.run(cmd, cwd=ROOT, capture_output=True, text=True, timeout=300)
+        assert r.returncode == 0, r.stderr[-2000:]
+        with open(out) as f:
+            records.append(json.load(f))
+    a, b = records
+    assert a["library_choices"] and all(c["chosen"] == "first" for c in a["library_choices"]), a["library_choices"]
+    assert any(c["rows"] > 64 for c in a["library_choices"]), "a step of many requests went through the library"
+    assert a["library_choices"] == b["library_choices"]
+    assert [c["token_ids"] for c in a["completions"]] == [c["token_ids"] for c in b["completions"]]

@@ -569,3 +569,80 @@ def test_a_layer_that_reads_a_window_gives_its_pages_back_while_the_engine_steps
     manager.release(0)
     manager.release(1)
     assert manager.num_available_blocks(1) == 8 and manager.num_available_blocks(0) == 24
+
+
+def test_a_whole_architecture_is_a_config_with_from_dict_a_spec_and_one_registration(tmp_path, capsys):
+    """A new architecture brings a configuration class with nothing but `from_dict`, a function from
+    it to a ModelSpec, and one registration. The random-weights mode (on the device and as a
+    folder), the loader, the entry point and the command line then run it as they are: they find
+    the architecture by the configuration's type and write its config.json from its fields."""
+    import json
+    import os
+    from dataclasses import dataclass
+
+    from safetensors import safe_open
+
+    from tinyserve_llm_amd import generate
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.loading import load_model, random_model
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+    from tinyserve_llm_amd.models.decoder import DecoderModel
+    from tinyserve_llm_amd.models.registry import Architecture, read_config, register_architecture
+    from tinyserve_llm_amd.models.spec import Destination
+    from tinyserve_llm_amd.weights.random_init import write_random_model
+    register_toy_parts()
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        vocab: int
+        width: int
+        mean_mixer: str
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(int(raw["vocab"]), int(raw["width"]), str(raw["mean_mixer"]))
+
+    def spec_of(c: ToyConfig):
+        spec = toy_spec(hidden=c.width, vocab=c.vocab, mean_mixer=c.mean_mixer)
+        spec.checkpoint = {f"toy.{name}": Destination(name) for name in DecoderModel(spec).param_specs()
+                           if not name.startswith("head.")}
+        return spec
+
+    register_architecture(Architecture("ToyForCausalLM", ("toy",), ToyConfig.from_dict, spec_of))
+    cfg = ToyConfig(vocab=97, width=48, mean_mixer="toy_running_mean_on_device")
+    folder = write_random_model(str(tmp_path / "toy"), cfg, 3, torch.float32)
+    with open(os.path.join(folder, "config.json")) as f:
+        raw = json.load(f)
+    assert raw == dict(vocab=97, width=48, mean_mixer="toy_running_mean_on_device", architectures=["ToyForCausalLM"],
+                       model_type="toy")
+    assert read_config(folder)[1] == cfg
+    model, config = load_model(folder, torch.float32, DEV)
+    assert config == cfg and model.spec.architecture == "Toy"
+    with safe_open(os.path.join(folder, "model.safetensors"), "pt", "cpu") as f:
+        p = {k[len("toy."):]: f.get_tensor(k).double() for k in f.keys()}
+
+    def plain_greedy(ids, n):
+        ids, out = list(ids), []
+        for _ in range(n):
+            out.append(int(toy_plain(p, ids)[-1].argmax()))
+            ids.append(out[-1])
+        return out
+
+    prompts = [[3, 50, 7, 7, 96, 1], [9, 8, 7]]
+    sc = SchedulerConfig(max_model_len=64, max_num_seqs=4, max_num_batched_tokens=24, max_prefill_chunk=5)
+    sp = SamplingParams(max_tokens=6, temperature=0.0, ignore_eos=True)
+    got = LLM(folder, sc, CacheConfig(block_size=4), dtype=torch.float32, num_blocks=24).generate(prompts, sp)
+    assert [r.token_ids[0] for r in got] == [plain_greedy(q, 6) for q in prompts]
+    drawn = random_model(cfg, 3, torch.float32, DEV)
+    again = LLM(None, sc, CacheConfig(block_size=4), model=drawn, num_blocks=24).generate(prompts, sp)
+    assert all(len(r.token_ids[0]) == 6 for r in again)
+    out = str(tmp_path / "record.json")
+    rc = generate.main(["--random-config", os.path.join(folder, "config.json"), "--random-seed", "3", "--dtype", "float32",
+                        "--prompt-ids", "3,50,7,7,96,1", "--max-tokens", "6", "--temperature", "0", "--ignore-eos",
+                        "--block-size", "4", "--num-blocks", "24", "--max-model-len", "64", "--max-num-seqs", "4",
+                        "--max-num-batched-tokens", "24", "--out", out])
+    assert rc == 0
+    with open(out) as f:
+        record = json.load(f)
+    assert record["completions"][0]["token_ids"] == [again[0].token_ids[0]], "the same seed on the device draws the same weights"

@@ -48,6 +48,7 @@ struct LtPlan {
   hipblasLtMatmulAlgo_t algo;
   size_t workspace = 0;
   bool tuned = false;
+  bool chosen = false;       // picked among borrowed algorithms by timing
   // algorithms picked for neighbouring row counts that also serve this shape, until one of them
   // or `algo` has been chosen by timing
   int borrowed = 0;
@@ -63,6 +64,9 @@ struct LtDevice {
 
 std::mutex lt_mutex;
 LtDevice lt_devices[LT_MAX_DEVICES];
+// Whether candidates may be timed at all. Off: every shape keeps the heuristic's first candidate,
+// so that two processes round a product the same way (candidates differ in the order of their sums).
+bool lt_timing = true;
 
 // The first of the library's candidates for these layouts that fits the workspace (they come best
 // first, whatever workspace they want). Shapes that a recorded decode step may hold take a candidate
@@ -203,6 +207,7 @@ void lt_tune(LtDevice& dev, LtPlan& plan, void* y, const void* x, const void* w,
 void lt_choose(LtDevice& dev, LtPlan& plan, void* y, const void* x, const void* w, hipStream_t stream) {
   const int candidates = plan.borrowed + 1;
   plan.borrowed = 0;
+  plan.chosen = true;
   hipEvent_t begin = nullptr, end = nullptr;
   if (hipEventCreate(&begin) != hipSuccess || hipEventCreate(&end) != hipSuccess) {
     if (begin) hipEventDestroy(begin);
@@ -262,6 +267,39 @@ extern "C" int ts_gemm_library_init() {
   return lt_device() ? TS_OK : TS_LAUNCH_FAILED;
 }
 
+// Switches the timing of candidates on or off for the process (see lt_timing); returns what it was.
+extern "C" int ts_gemm_library_timing(int on) {
+  std::lock_guard<std::mutex> guard(lt_mutex);
+  const int was = lt_timing;
+  lt_timing = on != 0;
+  return was;
+}
+
+// The algorithm kept for every shape met so far on the current device, as rows of six numbers:
+// M, N, K, 32-bit output or not, how it was chosen (0 the heuristic's first candidate, 1 the fastest
+// of the timed candidates, 2 still to be chosen among borrowed ones) and the library's index of the
+// solution. Writes at most `capacity` rows; returns how many shapes there are.
+extern "C" int ts_gemm_library_choices(int64_t* rows, int capacity) {
+  std::lock_guard<std::mutex> guard(lt_mutex);
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= LT_MAX_DEVICES) return 0;
+  int n = 0;
+  for (auto& kv : lt_devices[device].plans) {
+    if (!kv.second.desc) continue;
+    if (n < capacity && rows) {
+      int64_t* r = rows + 6 * n;
+      r[0] = std::get<0>(kv.first);
+      r[1] = std::get<1>(kv.first);
+      r[2] = std::get<2>(kv.first);
+      r[3] = std::get<6>(kv.first);
+      r[4] = kv.second.borrowed ? 2 : (kv.second.tuned || kv.second.chosen ? 1 : 0);
+      r[5] = hipblaslt_ext::getIndexFromAlgo(kv.second.algo);
+    }
+    ++n;
+  }
+  return n;
+}
+
 // x, w bfloat16; y bfloat16, or float32 if out_f32 (the 32-bit sums as they are, not rounded to
 // bfloat16 on the way); rows of x, w and y are ldx, ldw, ldy elements apart (each at least the row's
 // length). The stream may be one that is being captured into a graph (after ts_gemm_library_init).
@@ -278,12 +316,12 @@ extern "C" int ts_gemm_library_bf16(void* y, const void* x, const void* w, int M
   if (!dev) return TS_LAUNCH_FAILED;
   LtPlan* plan = lt_plan(*dev, M, N, K, ldx, ldw, ldy, out_f32 != 0);
   if (!plan) return TS_BAD_SHAPE;
-  if (tune && !plan->tuned && M >= LT_TUNE_MIN_ROWS && M <= LT_TUNE_MAX_ROWS) {
+  if (lt_timing && tune && !plan->tuned && M >= LT_TUNE_MIN_ROWS && M <= LT_TUNE_MAX_ROWS) {
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone)
       lt_tune(*dev, *plan, y, x, w, flush, flush_bytes, stream);
   }
-  if (plan->borrowed) {
+  if (lt_timing && plan->borrowed) {
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone)
       lt_choose(*dev, *plan, y, x, w, stream);

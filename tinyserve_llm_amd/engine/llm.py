@@ -9,14 +9,14 @@ import logging
 import os
 import time
 from dataclasses import dataclass, replace
-from typing import Literal
+from typing import Literal, Sequence
 
 import torch
 
 from tinyserve_llm_amd.engine.interface import CacheConfig, CacheStats, build_cache, bytes_per_page
 from tinyserve_llm_amd.engine.loading import as_dtype, load_model, random_model, require_gpu
 from tinyserve_llm_amd.models.decoder import DecoderModel
-from tinyserve_llm_amd.engine.runner import ModelRunner, StepEntry
+from tinyserve_llm_amd.engine.runner import DecodeGraphs, ModelRunner, StepEntry
 from tinyserve_llm_amd.engine.scheduler import (PENDING, RequestOutput, ScheduledSeq, Scheduler, SchedulerConfig,
                                                 SchedulerStats)
 from tinyserve_llm_amd.engine.sequence import SamplingParams
@@ -79,6 +79,10 @@ class LLM:
             decode_graphs: bool = True,              # replay decode steps from HIP graphs
             run_ahead: bool = True,                  # schedule and pack the next decode step while this one runs
             keep_streaming_copies: bool | None = None,   # layer weights once more in the decode kernels' order; None: if memory is ample
+            max_decode_graphs: int = DecodeGraphs.MAX_GRAPHS,         # recorded decode steps kept at most (least recently replayed out),
+            decode_graph_memory: int = DecodeGraphs.MEMORY_BUDGET,    # and the bytes their own buffers may take
+            record_decode_steps: Sequence[int | tuple[int, int]] = (),   # batch sizes (or (batch size, context)) to record now, not at first use
+            time_library: bool = True,               # time the matrix library's candidates when a step is recorded (faster; roundings may differ between runs)
     ) -> None:
         self.device = require_gpu(cache_config.device if cache_config.device != "cuda" else "cuda:0")
         self.dtype = as_dtype(dtype)
@@ -93,7 +97,7 @@ class LLM:
                 raise ValueError("give a model folder or random_weights=(config, seed)")
             self.model, self.config = load_model(model_path, self.dtype, self.device, keep_streaming_copies)
         spec = self.model.spec
-        if scheduler_config.max_model_len > spec.max_position:
+        if spec.max_position is not None and scheduler_config.max_model_len > spec.max_position:
             raise ValueError(f"max_model_len {scheduler_config.max_model_len} exceeds the model's "
                              f"{spec.max_position} positions")
         self.tokenizer = None
@@ -106,15 +110,25 @@ class LLM:
         if scheduler_config.eos_token_id == -1:
             scheduler_config = replace(scheduler_config, eos_token_id=self._eos_token_id())
         self.seed = 0 if seed is None else seed
+        graphs_on = decode_graphs and self.model.graph_safe()
+        if not time_library:
+            from tinyserve_llm_amd.ops import hip
+            hip.library_timing(False)                # (for the process: also the choice among three for steps of many rows)
         if num_blocks is None:
-            num_blocks = self._size_from_free_memory(scheduler_config, cache_config, gpu_memory_utilization)
+            num_blocks = self._size_from_free_memory(scheduler_config, cache_config, gpu_memory_utilization,
+                                                     decode_graph_memory if graphs_on else 0)
         self.storage, self.manager = build_cache(self.model, num_blocks, cache_config.block_size, self.dtype, self.device,
                                                  num_state_slots=scheduler_config.max_num_seqs,
                                                  caching=cache_config.caching)
         self.scheduler = Scheduler(scheduler_config, self.manager)
         self.runner = ModelRunner(self.model, self.storage, self.manager)
-        if decode_graphs:
-            self.runner.enable_decode_graphs(scheduler_config.max_model_len, scheduler_config.max_num_seqs, self.seed)
+        if graphs_on:
+            self.runner.enable_decode_graphs(scheduler_config.max_model_len, scheduler_config.max_num_seqs, self.seed,
+                                             max_graphs=max_decode_graphs, memory_budget=decode_graph_memory,
+                                             time_library=time_library)
+            for wanted in record_decode_steps:
+                batch, context = wanted if isinstance(wanted, tuple) else (wanted, scheduler_config.max_model_len)
+                self.runner.graphs.record(batch, context)
         self.run_ahead = run_ahead
         self._ahead: tuple | None = None             # (what is left of the step scheduled ahead, its launch or None, its rows)
         self.steps: list[StepRecord] = []
@@ -125,15 +139,18 @@ class LLM:
             return self.tokenizer.eos_token_id
         return self.model.spec.eos_token_id
 
-    def _size_from_free_memory(self, sc: SchedulerConfig, cc: CacheConfig, utilisation: float) -> int:
-        """Pages from what the GPU has left under the utilisation limit, after setting aside the
-        activations of a worst-case step (llm_engine.py:112-140 measures them with a trial step;
-        here they are bounded from the model's widths)."""
+    def _size_from_free_memory(self, sc: SchedulerConfig, cc: CacheConfig, utilisation: float, graph_memory: int) -> int:
+        """Pages from what the GPU has left under the utilisation limit, after setting aside what is
+        allocated later: the activations of a worst-case step (llm_engine.py:112-140 measures them
+        with a trial step; here the parts say how wide they get), the matrix library's workspace and
+        the buffer its timing sweeps, and the recorded decode steps' own buffers (`graph_memory`,
+        which `DecodeGraphs` holds itself to)."""
+        from tinyserve_llm_amd.ops import hip
         free, total = torch.cuda.mem_get_info(self.device)
-        widest = max([self.model.spec.hidden_size] + [p.shape[0] for n, p in self.model.param_specs().items()
-                                                        if n.startswith("layers.") and len(p.shape) == 2])
+        widest = self.model.widest_activation()
         act = sc.max_num_batched_tokens * widest * 4 * 6 + sc.max_num_seqs * self.model.spec.vocab_size * 4 * 2
-        budget = total * utilisation - (total - free) - act
+        later = act + graph_memory + hip.LIBRARY_WORKSPACE_BYTES + hip.LIBRARY_TUNING_SWEEP_BYTES
+        budget = total * utilisation - (total - free) - later
         per_page = max(1, bytes_per_page(self.model, cc.block_size, self.dtype))
         pages = int(budget // per_page)
         most_useful = sc.max_num_seqs * (-(-sc.max_model_len // cc.block_size) + 1) + 8

@@ -6,7 +6,7 @@ import torch
 
 from tinyserve_llm_amd import models  # noqa: F401  (registers the architectures)
 from tinyserve_llm_amd.models.decoder import DecoderModel
-from tinyserve_llm_amd.models.registry import read_config, resolve
+from tinyserve_llm_amd.models.registry import architecture_of, read_config
 from tinyserve_llm_amd.weights.loader import load_params
 from tinyserve_llm_amd.weights.random_init import random_params
 
@@ -72,7 +72,7 @@ def random_model(config, seed: int, dtype: str | torch.dtype = torch.bfloat16,
     """A model of `config` with weights drawn on the device from `seed` (no files)."""
     device = require_gpu(device)
     dtype = as_dtype(dtype)
-    arch = resolve(config.to_dict())
+    arch = architecture_of(config)
     model = DecoderModel(arch.build_spec(config))
     model.bind(random_params(model, seed, dtype, device), dtype, device)
     streaming_copies(model, keep_streaming_copies, device)

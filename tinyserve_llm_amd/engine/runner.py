@@ -10,8 +10,10 @@ logits [wanted, vocab] in the order of the entries and of their `want` lists.
 
 from __future__ import annotations
 
+import contextlib
 import gc
 import struct
+import sys
 import weakref
 from array import array
 from typing import NamedTuple, Sequence
@@ -58,7 +60,7 @@ class ModelRunner:
         if not entries:
             raise StepError("a step needs at least one entry")
         ps = self.storage.page_size
-        vocab, max_pos = self.model.spec.vocab_size, self.model.spec.max_position
+        vocab, max_pos = self.model.spec.vocab_size, self.model.spec.max_position or sys.maxsize
         num_spaces = len(self.storage.spaces)
         ids: list[int] = []
         positions: list[int] = []
@@ -150,16 +152,16 @@ class ModelRunner:
         """`_pack` for steps whose entries all feed one token and want its logits: the same checks
         and the same layout, without the per-token loops."""
         ps = self.storage.page_size
-        vocab, max_pos = self.model.spec.vocab_size, self.model.spec.max_position
+        vocab, max_pos = self.model.spec.vocab_size, self.model.spec.max_position or sys.maxsize
         num_spaces = len(self.storage.spaces)
         S, n = max(pad_to, len(entries)), len(entries)
         ids = [e.tokens[0] for e in entries]
         starts = [e.start for e in entries]
         if len({e.seq_id for e in entries}) != n:
             raise StepError("a request appears twice in one step")
-        if min(ids) < 0 or max(ids) >= vocab:
+        if n and (min(ids) < 0 or max(ids) >= vocab):
             raise StepError(f"a token id outside the vocabulary of {vocab}")
-        if min(starts) < 0 or max(starts) >= max_pos:
+        if n and (min(starts) < 0 or max(starts) >= max_pos):
             raise StepError(f"a position outside the model's {max_pos}")
         pad = S - n
         slots = [self.view.state_slot(e.seq_id) for e in entries]
@@ -264,14 +266,17 @@ class ModelRunner:
         `feed` named take their ids. Returns the drawn tokens as `DrawnTokens`."""
         return self.graphs.launch(prepared, drawn_before=drawn_before)
 
-    def enable_decode_graphs(self, max_context: int, max_batch: int, seed: int = 0) -> bool:
+    def enable_decode_graphs(self, max_context: int, max_batch: int, seed: int = 0, *, max_graphs: int = 0,
+                             memory_budget: int = 0, time_library: bool = True) -> bool:
         """Decode steps (every entry one token whose logits are wanted) are then replayed from HIP
         graphs, one per batch size, instead of being launched kernel by kernel. Only for models
-        whose parts all declare `graph_safe`. `seed` is the one the graphs' draws use. Returns
-        whether graphs are on."""
+        whose parts all declare `graph_safe`. `seed` is the one the graphs' draws use; `max_graphs`
+        and `memory_budget` bound what is kept (0: `DecodeGraphs`' defaults); `time_library` as in
+        `DecodeGraphs`. Returns whether graphs are on."""
         if not self.model.graph_safe():
             return False
-        self.graphs = DecodeGraphs(self, max_context, max_batch, seed)
+        self.graphs = DecodeGraphs(self, max_context, max_batch, seed, max_graphs=max_graphs or DecodeGraphs.MAX_GRAPHS,
+                                   memory_budget=memory_budget or DecodeGraphs.MEMORY_BUDGET, time_library=time_library)
         return True
 
 
@@ -281,10 +286,26 @@ class DrawnTokens:
     copy on its way to pinned host memory. `tolist()` waits for that copy alone, not for what was
     started on the device after it."""
 
-    def __init__(self, on_device: torch.Tensor, host: torch.Tensor, landed: torch.cuda.Event, n: int) -> None:
-        self.on_device, self.host, self.landed, self.n = on_device, host, landed, n
+    def __init__(self, on_device: torch.Tensor, host: torch.Tensor, landed: torch.cuda.Event, n: int,
+                 kept: list | None = None) -> None:
+        self._on_device, self.host, self.landed, self.n = on_device, host, landed, n
+        # the graph these tokens came from and the number of its replay that drew them: the graph's
+        # next replay overwrites them on the device, the one after that their landing place on the host
+        self._kept, self._replay = kept, kept[8] if kept is not None else 0
+
+    def _replays_since(self) -> int:
+        return 0 if self._kept is None else self._kept[8] - self._replay
+
+    @property
+    def on_device(self) -> torch.Tensor:
+        if self._replays_since() >= 1:
+            raise StepError("these tokens are gone from the device: the graph that drew them has been replayed since")
+        return self._on_device
 
     def tolist(self) -> list[int]:
+        if self._replays_since() >= 2:
+            raise StepError("these tokens are gone: the graph that drew them has been replayed twice since, and its "
+                            "two landing places on the host take turns")
         self.landed.synchronize()
         return self.host[:self.n].tolist()
 
@@ -296,9 +317,19 @@ class DecodeGraphs:
     of the block tables, and with it the attention kernels' grids. A graph's inputs live in one
     fixed device buffer that every replay overwrites with one copy from pinned host memory: the
     step's integers, then the draws' keys and temperatures. A graph ends with the logits and with
-    the tokens drawn from them; a caller that only wants logits ignores the tokens."""
+    the tokens drawn from them; a caller that only wants logits ignores the tokens.
 
-    def __init__(self, runner: ModelRunner, max_context: int, max_batch: int, seed: int = 0) -> None:
+    What is kept is bounded: at most `max_graphs` graphs whose own buffers (the logits above all:
+    batch size x vocabulary x 4 bytes each) add up to at most `memory_budget` bytes; beyond either,
+    the graph replayed longest ago is dropped (and recorded again if its key comes back). The engine
+    sets the budget aside when it sizes the cache pool. `record` makes a graph ahead of its first
+    use, so that no request waits for a recording."""
+
+    MAX_GRAPHS = 64
+    MEMORY_BUDGET = 2 << 30
+
+    def __init__(self, runner: ModelRunner, max_context: int, max_batch: int, seed: int = 0, *,
+                 max_graphs: int = MAX_GRAPHS, memory_budget: int = MEMORY_BUDGET, time_library: bool = True) -> None:
         self.runner = weakref.proxy(runner)     # (the runner owns the graphs: no cycle, so a dropped engine's memory is freed at once)
         self.page_size = runner.storage.page_size
         self.num_spaces = len(runner.storage.spaces)
@@ -306,7 +337,14 @@ class DecodeGraphs:
         self.max_context = max_context
         self.max_batch = max_batch
         self.can_pad = not runner.model.state_plan()
-        self.graphs: dict[int, tuple] = {}
+        self.graphs: dict[tuple[int, int], list] = {}      # (batch size, table width) -> kept graph, oldest replay first
+        self.max_graphs = max(2, max_graphs)      # (the step before and the step being started may be of two graphs)
+        self.memory_budget = memory_budget
+        self.recorded = 0                 # graphs recorded so far, dropped ones included
+        self.dropped = 0
+        # Whether the matrix library's candidates for a batch size are timed when its step is recorded
+        # (faster steps; which candidate wins may differ between two runs, and with it the rounding).
+        self.time_library = time_library
         self.pool = None
         self.seed = seed                  # of the draws the graphs hold
         from tinyserve_llm_amd.ops import hip
@@ -366,7 +404,8 @@ class DecodeGraphs:
         before = [t.clone() for t in states]
         side = torch.cuda.Stream(device=r.device)
         side.wait_stream(torch.cuda.current_stream(r.device))
-        with hip.library_tuning(), torch.cuda.stream(side):      # (the sweep buffer belongs to the current stream)
+        tuning = hip.library_tuning() if self.time_library else contextlib.nullcontext()
+        with tuning, torch.cuda.stream(side):      # (the sweep buffer belongs to the current stream)
             hidden, residual = r.model.forward(ctx, r.memory)
             hip.sample(r.model.logits(hidden, residual, rows), draw_temps, draw_keys, self.seed)
         torch.cuda.current_stream(r.device).wait_stream(side)
@@ -386,7 +425,56 @@ class DecodeGraphs:
         # the drawn tokens travel to the host through two pinned buffers in turn: a step may be
         # started before the tokens of the step before it have been read
         landing = [(torch.empty(size, dtype=torch.int32, pin_memory=True), torch.cuda.Event()) for _ in range(2)]
-        return [graph, host_i32, dev_i32, logits, tokens, torch.cuda.Event(), landing, 0]
+        return [graph, host_i32, dev_i32, logits, tokens, torch.cuda.Event(), landing, 0, 0]    # (.., turn, replays)
+
+    @staticmethod
+    def _bytes_of(kept: list) -> int:
+        """What a kept graph holds on the device for itself: its inputs, logits and tokens (the
+        activations between them lie in the pool that all graphs share)."""
+        return sum(t.numel() * t.element_size() for t in (kept[2], kept[3], kept[4]))
+
+    def memory_held(self) -> int:
+        return sum(self._bytes_of(k) for k in self.graphs.values())
+
+    def _make_room(self, incoming: int) -> None:
+        """Drops the graphs replayed longest ago until one more of `incoming` bytes fits both bounds."""
+        while self.graphs and (len(self.graphs) >= self.max_graphs
+                               or (len(self.graphs) >= 2 and self.memory_held() + incoming > self.memory_budget)):
+            oldest = next(iter(self.graphs))
+            # its last replay may still be running, and its tokens on their way to the host
+            torch.cuda.current_stream(self.runner.device).synchronize()
+            del self.graphs[oldest]
+            self.dropped += 1
+
+    def _kept(self, key: tuple[int, int], words: torch.Tensor, start: int, dims, host) -> list:
+        """The graph for `key`, recorded now if it is not kept; it becomes the most recently used."""
+        kept = self.graphs.pop(key, None)
+        if kept is None:
+            vocab = self.runner.model.spec.vocab_size
+            self._make_room(key[0] * vocab * 4 + 4 * len(words) + 4 * key[0])
+            kept = self._capture(key[0], words, start, dims, host)
+            self.recorded += 1
+        self.graphs[key] = kept
+        return kept
+
+    def record(self, batch_size: int, context: int) -> tuple[int, int]:
+        """Records the graph that serves `batch_size` requests whose longest context is `context`
+        positions, ahead of its first use, from a step of idle rows (position 0, page 0, nothing
+        written). Returns the graph's key."""
+        if not 1 <= batch_size <= self.max_batch or not 1 <= context <= self.max_context:
+            raise StepError(f"no recorded step serves {batch_size} requests of {context} positions "
+                            f"(up to {self.max_batch} of {self.max_context})")
+        size, width = self._size(batch_size), self._width(context)
+        if (size, width) not in self.graphs:
+            flat, dims, host = self.runner._pack_decode([], [width] * self.num_spaces, pad_to=size)
+            words, start = self._with_draws(flat, size, None)
+            self._kept((size, width), words, start, dims, host)
+        return size, width
+
+    def _width(self, longest: int) -> int:
+        """Pages per block table of the graph that serves contexts up to `longest` positions."""
+        reach = min(-(-longest // self.bucket) * self.bucket, -(-self.max_context // self.bucket) * self.bucket)
+        return -(-reach // self.page_size)
 
     @staticmethod
     def _record(graph, pool, body):
@@ -409,9 +497,7 @@ class DecodeGraphs:
         if feed is not None and (len(feed) != len(entries) or min(feed) < -1):
             raise StepError("one source row (or -1) per entry")
         size = self._size(len(entries))
-        longest = max(e.start + 1 for e in entries)
-        reach = min(-(-longest // self.bucket) * self.bucket, -(-self.max_context // self.bucket) * self.bucket)
-        width = -(-reach // self.page_size)
+        width = self._width(max(e.start + 1 for e in entries))
         flat, dims, host = self.runner._pack_decode(entries, [width] * self.num_spaces, pad_to=size)
         words, start = self._with_draws(flat, size, draws, feed)
         return (size, width), words, start, dims, host, len(entries), draws is not None, feed is not None and max(feed) >= 0
@@ -425,11 +511,8 @@ class DecodeGraphs:
         key, words, start, dims, host, n, drawn, fed = prepared
         if fed and drawn_before is None:
             raise StepError("the step takes ids from the step before, whose tokens were not given")
-        if key not in self.graphs:
-            self.graphs[key] = self._capture(key[0], words, start, dims, host)
-            # the capture recorded the step without running it: the replay below runs it
-        kept = self.graphs[key]
-        graph, host_i32, dev_i32, logits, tokens, uploaded, landing, turn = kept
+        kept = self._kept(key, words, start, dims, host)    # (a recording does not run the step: the replay below does)
+        graph, host_i32, dev_i32, logits, tokens, uploaded, landing, turn, _ = kept
         uploaded.synchronize()                  # the last upload from the pinned words has long been made
         host_i32.copy_(words)
         dev_i32.copy_(host_i32, non_blocking=True)
@@ -439,6 +522,7 @@ class DecodeGraphs:
             before = drawn_before.on_device if isinstance(drawn_before, DrawnTokens) else drawn_before
             hip.feed_tokens(dev_i32[:n], before.contiguous(), dev_i32[start + 3 * size:start + 3 * size + n])
         graph.replay()
+        kept[8] += 1
         if not drawn:
             return logits[:n]
         host_tokens, landed = landing[turn]
@@ -449,7 +533,7 @@ class DecodeGraphs:
         # tokens anew, comes after both on the stream.
         host_tokens[:n].copy_(tokens[:n], non_blocking=True)
         landed.record()
-        return DrawnTokens(tokens[:n], host_tokens, landed, n)
+        return DrawnTokens(tokens[:n], host_tokens, landed, n, kept)
 
     def run(self, entries: Sequence[StepEntry], draws=None) -> torch.Tensor:
         """Replays the step's graph. Without `draws` the logits [entries, vocab] come back; with

@@ -48,8 +48,18 @@ def parse_args(argv=None) -> argparse.Namespace:
     p.add_argument("--device", default="cuda")
     p.add_argument("--many-rows-products", choices=["library", "tiled"], default="library",
                    help="bfloat16 products of many rows: the vendor's matrix library, or the engine's own tiled kernel (slower)")
+    p.add_argument("--no-library-timing", action="store_true",
+                   help="keep the matrix library's first candidate for every shape instead of timing candidates: "
+                        "two runs then round every product alike")
     p.add_argument("--out", help="write the JSON record here as well as printing a summary")
     return p.parse_args(argv)
+
+
+def _library_choices() -> list:
+    """Which of the matrix library's algorithms served which shape in this run (bfloat16 roundings
+    follow from them)."""
+    from tinyserve_llm_amd.ops import hip
+    return hip.library_choices()
 
 
 def main(argv=None) -> int:
@@ -74,7 +84,8 @@ def main(argv=None) -> int:
         from tinyserve_llm_amd.ops import hip
         hip.many_rows_products(args.many_rows_products)
     llm = LLM(args.model, sc, cc, dtype=args.dtype, num_blocks=args.num_blocks,
-              gpu_memory_utilization=args.gpu_memory_utilization, seed=args.seed, random_weights=random_weights)
+              gpu_memory_utilization=args.gpu_memory_utilization, seed=args.seed, random_weights=random_weights,
+              time_library=not args.no_library_timing)
     vocab = llm.model.spec.vocab_size
     prompts: list = list(args.prompt)
     prompts += [[int(t) for t in ids.split(",") if t.strip()] for ids in args.prompt_ids]
@@ -107,7 +118,7 @@ def main(argv=None) -> int:
         "temperature": args.temperature, "seed": args.seed, "n": args.n, "max_tokens": args.max_tokens,
         "device": torch.cuda.get_device_name(), "torch": torch.__version__, "started": started,
         "seconds": seconds, "output_tokens": out_tokens, "output_tokens_per_second": out_tokens / seconds,
-        "steps": len(llm.steps), "scheduler_stats": asdict(stats), "cache_stats": asdict(llm.manager.stats()),
+        "steps": len(llm.steps), "library_choices": _library_choices(), "scheduler_stats": asdict(stats), "cache_stats": asdict(llm.manager.stats()),
         "completions": [{"request_id": r.request_id, "prompt_token_ids": r.prompt_token_ids, "token_ids": r.token_ids,
                          "texts": r.texts, "finish_reasons": r.finish_reasons} for r in results],
     }

@@ -127,6 +127,11 @@ class DecoderModel:
             enc.prepare(device)
         self.final_norm.bind(grouped.get("final_norm", {}))
 
+    def widest_activation(self) -> int:
+        """Elements per token of the widest tensor any layer makes (the parts say: `Part.widest_activation`)."""
+        return max([self.spec.hidden_size] + [part.widest_activation() for layer in self.layers
+                                              for part in layer.parts().values()])
+
     def keep_streaming_copies(self) -> int:
         """Lets every part of every layer keep its weights once more in a decode kernel's reading
         order, and the head likewise; returns the bytes that takes."""

@@ -56,4 +56,4 @@ def llama_spec(config: LlamaConfig) -> ModelSpec:
 
 LLAMA = register_architecture(Architecture(
     name="LlamaForCausalLM", model_types=("llama",), config_from_dict=LlamaConfig.from_dict,
-    build_spec=llama_spec))
+    build_spec=llama_spec, config_to_dict=LlamaConfig.to_dict))

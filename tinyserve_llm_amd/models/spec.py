@@ -69,7 +69,7 @@ class ModelSpec:
     architecture: str
     vocab_size: int
     hidden_size: int
-    max_position: int
+    max_position: int | None          # None: the model's parts set no limit to a request's length
     layers: list[LayerSpec]
     order: list[LayerRun]
     final_norm: PartSpec

@@ -60,6 +60,8 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_gemm_library_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p, ctypes.c_size_t, p],
         "ts_gemm_tiled_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_gemm_library_init": [],
+        "ts_gemm_library_timing": [i],
+        "ts_gemm_library_choices": [p, i],
         "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, i, i, i, i, p, p, p],
         "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p],
         "ts_gemm_skinny8_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
@@ -609,7 +611,10 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 
 SKINNY_MAX_ROWS = 32
 SKINNY_FUSED_ROWS = 16       # the fused norm serves one 16-row block of x,
-SKINNY_EPILOGUE_ROWS = 64    # the gate and the rotation on the way out up to four (for reductions up to 2048)
+SKINNY_EPILOGUE_ROWS = 64    # the gate and the rotation on the way out up to four,
+SKINNY_EPILOGUE_WIDE_K = 2048    # for reductions up to this
+SKINNY_NORM_MAX_K = 2048     # longest reduction with the norm on the way in,
+SKINNY_EPILOGUE_MAX_K = 4096     # and with the gate or the rotation on the way out
 SKINNY_WIDE_ELEMENTS = 8 << 20   # largest matrix that `linear_bf16` gives the kernel with 17 to 32 rows
 
 
@@ -730,8 +735,8 @@ def skinny_fuses(rows: int, k: int, norm: bool, glu: bool) -> bool:
     if k % 256:
         return False
     if norm or rows <= SKINNY_FUSED_ROWS:
-        return rows <= SKINNY_FUSED_ROWS and k // 256 <= (8 if norm else 16)
-    return rows <= SKINNY_EPILOGUE_ROWS and k // 256 <= 8
+        return rows <= SKINNY_FUSED_ROWS and k <= (SKINNY_NORM_MAX_K if norm else SKINNY_EPILOGUE_MAX_K)
+    return rows <= SKINNY_EPILOGUE_ROWS and k <= SKINNY_EPILOGUE_WIDE_K
 
 
 def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, *,
@@ -809,15 +814,24 @@ def gemm_rows64(x: torch.Tensor, packed: torch.Tensor, out_dtype: torch.dtype = 
     return out
 
 
+def qkv_rope_max_rows(k: int, norm: bool = False) -> int:
+    """Most rows of x that `qkv_rope_store` takes over a reduction of `k`, with or without the norm
+    on the way in; 0 if it does not take the reduction at all."""
+    if k % 256 or k > (SKINNY_NORM_MAX_K if norm else SKINNY_EPILOGUE_MAX_K):
+        return 0
+    return SKINNY_EPILOGUE_ROWS if not norm and k <= SKINNY_EPILOGUE_WIDE_K else SKINNY_FUSED_ROWS
+
+
+STREAMING_MAX_ROWS = 64      # most rows of x for which `linear_bf16` reads a weight's streaming copy
+
+
 def qkv_rope_fuses(x: torch.Tensor, weight: torch.Tensor, head_dim: int, k_cache: torch.Tensor | None,
                    norm: bool = False) -> bool:
     """Whether `qkv_rope_store` serves these operands: few bfloat16 rows, a reduction of up to 4096 in
     steps of 256 (2048 with the norm on the way in), heads of a multiple of 32 dimensions, keys whose
     strides allow 8-byte stores."""
-    rows_ok = (x.dim() == 2 and (x.shape[0] <= SKINNY_FUSED_ROWS
-                                 or (not norm and x.shape[0] <= SKINNY_EPILOGUE_ROWS and x.shape[1] <= 2048)))
-    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and rows_ok
-            and x.shape[1] % 256 == 0 and x.shape[1] // 256 <= (8 if norm else 16) and head_dim % 32 == 0
+    rows_ok = x.dim() == 2 and x.shape[0] <= qkv_rope_max_rows(x.shape[1], norm)
+    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and rows_ok and head_dim % 32 == 0
             and x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0
             and (k_cache is None or (all(st % 4 == 0 for st in k_cache.stride()[:3]) and k_cache.data_ptr() % 8 == 0)))
 
@@ -963,6 +977,33 @@ def gemm_library_init() -> None:
     _run("gemm_library_init", library().ts_gemm_library_init())
 
 
+def library_timing(on: bool | None = None) -> bool:
+    """Whether the matrix library's candidates may be timed and the fastest kept (`library_tuning`, and
+    the choice among three for row counts beyond 256 that are no multiple of 256). With it off every
+    shape keeps the library's first candidate, so two processes round every product alike: candidates
+    sum in different orders, and which of them is fastest may differ from run to run. Sets it for the
+    process if `on` is given (shapes already chosen keep their choice); returns what it was."""
+    lib = library()
+    was = lib.ts_gemm_library_timing(1)
+    lib.ts_gemm_library_timing(int(was if on is None else on))
+    return bool(was)
+
+
+def library_choices() -> list[dict[str, int | str]]:
+    """The algorithm kept for every shape the matrix library has served on the current device:
+    rows, columns, reduction, whether the output is 32-bit, how it was chosen ("first": the library's
+    first candidate; "timed": the fastest of those timed; "open": still to be timed) and the
+    library's index of the solution. A record of them tells two runs' roundings apart."""
+    lib = library()
+    n = lib.ts_gemm_library_choices(None, 0)
+    buf = (ctypes.c_int64 * (6 * max(n, 1)))()
+    n = min(n, lib.ts_gemm_library_choices(buf, n))
+    how = ("first", "timed", "open")
+    return [dict(rows=buf[6 * r], columns=buf[6 * r + 1], reduction=buf[6 * r + 2], out_float32=bool(buf[6 * r + 3]),
+                 chosen=how[buf[6 * r + 4]], solution=buf[6 * r + 5]) for r in range(n)]
+
+
+LIBRARY_WORKSPACE_BYTES = 128 << 20       # what gemm_library.hip allocates once per device for the library
 LIBRARY_TUNING_SWEEP_BYTES = 320 << 20    # overwritten between timed runs: more than the caches hold (256 MB)
 _library_tuning: torch.Tensor | None = None
 

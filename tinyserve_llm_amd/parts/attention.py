@@ -4,8 +4,9 @@ tinyserve_llm/engine/model_runner.py:100-108, tinyserve_llm/attention/torch_page
 One fused projection gives q | k | v; q and k are rotated by the named position encoding; k and v
 of the step's tokens are written to their cache slots; then every token attends, causally, over
 the cache pages of its request (its own key included), and the output projection follows.
-For steps of up to 16 tokens projection, rotation and cache write are one kernel
-(`hip.qkv_rope_store`), which also takes a deferred norm; larger steps run them one after the other.
+For steps of few tokens (`hip.qkv_rope_max_rows` says how many for the layer's width) projection,
+rotation and cache write are one kernel (`hip.qkv_rope_store`), which also takes a deferred norm
+where it reaches; larger steps run them one after the other.
 """
 
 from __future__ import annotations
@@ -53,7 +54,7 @@ class Attention(Mixer):
         self.qkv_packed, self.o_packed = streaming_copy(self.qkv), streaming_copy(self.o)
         if self.qkv_packed is not None and self.qkv_packed.by16 is not None and self.head_dim % 32 == 0:
             self.qkv_rope_packed = hip.pack_weight_rope(self.qkv, self.head_dim)
-            if self.hidden_size <= 2048:
+            if hip.qkv_rope_max_rows(self.hidden_size) >= hip.STREAMING_MAX_ROWS:
                 self.qkv_packed = None           # every step that would stream the plain copy takes the one-kernel path
         copies = sum(c.nbytes() for c in (self.qkv_packed, self.o_packed) if c is not None)
         return copies + (0 if self.qkv_rope_packed is None else self.qkv_rope_packed.numel() * 2)

@@ -108,6 +108,12 @@ class Part:
         for name, tensor in params.items():
             setattr(self, name, tensor)
 
+    def widest_activation(self) -> int:
+        """Elements per token of the widest tensor the part makes on its way: the engine sets memory
+        aside for a step's activations by it. The default is the most rows of any of the part's
+        matrices (a projection's output; the last two dimensions of stacked matrices count)."""
+        return max((ps.shape[-2] for ps in self.param_specs().values() if len(ps.shape) >= 2), default=0)
+
     def keep_streaming_copies(self) -> int:
         """Optionally keeps second copies of weights in the order a decode kernel reads them
         (`parts.linear.streaming_copy`), to hand to `linear(..., packed=)`; returns the bytes they

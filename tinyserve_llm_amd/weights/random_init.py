@@ -15,7 +15,7 @@ import torch
 from safetensors.torch import save_file
 
 from tinyserve_llm_amd.models.decoder import DecoderModel
-from tinyserve_llm_amd.models.registry import resolve
+from tinyserve_llm_amd.models.registry import architecture_of, write_config
 from tinyserve_llm_amd.weights.loader import storage_dtype
 
 
@@ -47,11 +47,8 @@ def checkpoint_tensors(model: DecoderModel, params: dict[str, torch.Tensor]) -> 
 def write_random_model(folder: str, config, seed: int, dtype: torch.dtype = torch.bfloat16) -> str:
     """Writes `folder`/config.json and `folder`/model.safetensors for `config` (a typed
     configuration of a registered architecture) with weights drawn from `seed`."""
-    raw = config.to_dict()
-    arch = resolve(raw)
-    model = DecoderModel(arch.build_spec(config))
-    os.makedirs(folder, exist_ok=True)
-    config.save(folder)
+    model = DecoderModel(architecture_of(config).build_spec(config))
+    write_config(folder, config)
     params = random_params(model, seed, dtype, "cpu")
     save_file(checkpoint_tensors(model, params), os.path.join(folder, "model.safetensors"))
     return folder
