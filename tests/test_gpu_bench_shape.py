@@ -170,35 +170,165 @@ def folder_1b(tmp_path_factory):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_the_benchmarks_own_regime_against_the_plain_model(folder_1b, dtype):
-    """What bench.py times, checked: eight requests of 2,048 tokens (eight full pages of 256 each)
-    decode sixteen tokens through `LLM.generate`, set up as bench.py sets its engine up: decode steps
-    replayed from a graph whose block tables are nine pages wide (the bucket above 2,048 positions),
-    the host one step ahead, the split-key attention kernel over 2,049 to 2,064 keys that cross into
-    a ninth page. Every token against the plain model run whole over the same history: in float32
-    it is the plain model's choice; in bfloat16 it lies within a small gap of it."""
+@pytest.mark.parametrize("batch", [8, 64])
+def test_the_benchmarks_own_regime_against_the_plain_model(folder_1b, dtype, batch, monkeypatch):
+    """What bench.py times, checked, at both of its batch sizes beyond one: requests of 2,048 tokens
+    (eight full pages of 256 each) decode sixteen tokens through `LLM.generate`, set up as bench.py
+    sets its engine up: decode steps replayed from a graph whose block tables are nine pages wide
+    (the bucket above 2,048 positions), the host one step ahead, attention over 2,049 to 2,064 keys
+    that cross into a ninth page. Eight requests take the split-key attention kernel and the
+    weight-streaming projections; sixty-four take one workgroup per (request, key/value head) over
+    the whole context, the shared-x kernel for the gate|up projection and the head, and this
+    repository's or the library's kernels for the rest, and the test sees that they did. Every token
+    of some of the requests against the plain model run whole over the same history: in float32 it is
+    the plain model's choice; in bfloat16 it lies within a small gap of it."""
     from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
     from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
     from tinyserve_llm_amd.engine.sequence import SamplingParams
-    batch, length, decoded, page = 8, 2048, 16, 256
+    from tinyserve_llm_amd.ops import hip
+    length, decoded, page = 2048, 16, 256
     prompts = [prompt(900 + i, length, CONFIG.vocab_size) for i in range(batch)]
-    sc = SchedulerConfig(max_model_len=4096, max_num_seqs=batch, max_num_batched_tokens=length + batch, watermark=0.0)
+    plans, rows64 = [], []
+    plan, shared_x = hip.decode_plan, hip.gemm_rows64
+
+    def seen_plan(num_tokens, nkv, group, hd, capacity):
+        plans.append(((num_tokens, capacity), plan(num_tokens, nkv, group, hd, capacity)))
+        return plans[-1][1]
+
+    def seen_rows64(x, packed, *a, **kw):
+        rows64.append((x.shape[0], packed.shape[0] * 16))
+        return shared_x(x, packed, *a, **kw)
+
+    monkeypatch.setattr(hip, "decode_plan", seen_plan)
+    monkeypatch.setattr(hip, "gemm_rows64", seen_rows64)
+    # prompts first, one a step under the token budget; once the last one is in, all decode together
+    sc = SchedulerConfig(max_model_len=4096, max_num_seqs=batch, max_num_batched_tokens=length + batch, watermark=0.0,
+                         step_mode="prefill_first")
     llm = LLM(folder_1b, sc, CacheConfig(block_size=page, caching=False), dtype=torch.float32 if dtype == "float32" else torch.bfloat16,
-              num_blocks=batch * (4096 // page) + 2, seed=0)
+              num_blocks=batch * 9 + 2, seed=0)
     outs = [c.token_ids[0] for c in llm.generate(prompts, SamplingParams(max_tokens=decoded, temperature=0.0, ignore_eos=True))]
-    assert (batch, 9) in llm.runner.graphs.graphs, "the decode steps ran as the graph of eight requests over nine pages"
-    # (a prompt a step is admitted under the token budget; once the last one is in, all eight decode together)
-    assert sum(s.num_tokens == s.num_seqs == batch for s in llm.steps) >= 5
+    assert (batch, 9) in llm.runner.graphs.graphs, f"the decode steps ran as the graph of {batch} requests over nine pages"
+    assert sum(s.num_tokens == s.num_seqs == batch for s in llm.steps) == decoded - 1
+    if dtype == "bfloat16":
+        assert ((batch, 9 * page), hip.decode_plan(batch, 8, 4, 64, 9 * page)) in plans
+        if batch == 64:
+            assert plan(64, 8, 4, 64, 9 * page) == (9 * page, 8), "a workgroup walks the whole context: nothing is combined"
+            assert (64, 2 * 8192) in rows64 and (64, CONFIG.vocab_size) in rows64, f"gate|up and the head by the shared-x kernel: {rows64}"
+        else:
+            assert plan(8, 8, 4, 64, 9 * page)[0] < 9 * page and not rows64, "eight requests: keys in chunks, combined afterwards"
     plain = PlainLlama(folder_1b, torch.float64)
     head = plain.w["model.embed_tokens.weight"]
-    for p, tokens in list(zip(prompts, outs))[:batch if dtype == "float32" else 4]:
+    some = [0, 1, batch // 2, batch - 1] if batch > 8 or dtype == "bfloat16" else range(batch)
+    for r in some:
+        p, tokens = prompts[r], outs[r]
         logits = plain.hidden_states(p + tokens[:-1])[length - 1:] @ head.T
         best = logits.max(-1)
         if dtype == "float32":
             close = torch.topk(logits, 2).values
             for i, tok in enumerate(tokens):
                 assert tok == int(best.indices[i]) or float(close[i, 0] - close[i, 1]) < 2e-4, \
-                    f"token {i}: {tok}, the plain model chooses {int(best.indices[i])}"
+                    f"request {r} token {i}: {tok}, the plain model chooses {int(best.indices[i])}"
         else:
             gaps = best.values - logits[torch.arange(decoded), torch.tensor(tokens)]
-            assert float(gaps.max()) <= 0.05 * float(logits.std()), f"a token far from the best: gaps {gaps.tolist()}"
+            assert float(gaps.max()) <= 0.05 * float(logits.std()), f"request {r}: a token far from the best: gaps {gaps.tolist()}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prefix_hits_partial_page_copies_and_forks_at_pages_of_256(folder_1b, dtype):
+    """The cache at the page size and widths the benchmarks use: a prompt of 350 tokens leaves a full
+    page and a part of a second one; two prompts that share its first 300 tokens find them (the
+    whole first page, and 44 slots of the second copied into a page of their own: the transposed
+    value layout of a 256-slot page goes through `copy_slots` here); one of them is drawn twice at a
+    temperature, so the two samples share the prompt's pages until they write and then copy the last
+    one; an unrelated long prompt then needs more pages than were never used, so pages that were kept
+    for reuse are taken back; and the first prompt, fed again, finds its prefix in what is left. The
+    matrix-core kernels read the copied pages. Every drawn token against the plain model run whole on
+    the same history (the race under the kernel's own noise: the winner in float32, within a small
+    gap of it in bfloat16)."""
+    from tests.test_gpu_generate import race_scores
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+    vocab, seed, t, n_out = CONFIG.vocab_size, 4, 0.7, 6
+    common = prompt(60, 300, vocab)
+    first, second, third = common + prompt(61, 50, vocab), common + prompt(62, 40, vocab), common + prompt(63, 30, vocab)
+    other = prompt(64, 1000, vocab)
+    assert len({first[300], second[300], third[300]}) == 3, "the prompts part right after the common prefix"
+    sc = SchedulerConfig(max_model_len=1024, max_num_seqs=4, max_num_batched_tokens=2048, watermark=0.0)
+    llm = LLM(folder_1b, sc, CacheConfig(block_size=256), dtype=torch.float32 if dtype == "float32" else torch.bfloat16,
+              num_blocks=8, seed=seed)
+
+    def run(*requests):
+        params = [SamplingParams(max_tokens=n_out, temperature=t, n=n, ignore_eos=True) for _, n in requests]
+        ids = [llm.add_request(p, sp) for (p, _), sp in zip(requests, params)]
+        done = {}
+        while llm.scheduler.has_unfinished():
+            for out in llm.step():
+                done[out.request_id] = out
+        return [(rid, p, done[rid].sequences) for rid, (p, _) in zip(ids, requests)]
+
+    judged = run((first, 1))
+    assert llm.scheduler.stats().cached_tokens == 0
+    judged += run((second, 2), (third, 1))
+    st, cache = llm.scheduler.stats(), llm.manager.stats()
+    assert st.cached_tokens == 600, "both found the 300 tokens they share with the first prompt"
+    assert cache.partial_copies >= 2 and cache.cow_copies >= 1, cache
+    run((other, 1))
+    assert llm.manager.stats().evictions >= 1, "pages kept for reuse were taken back"
+    again = run((first, 1))
+    assert llm.scheduler.stats().cached_tokens >= 600 + 256, "the first page, at least, was still there"
+    judged += again
+    plain = PlainLlama(folder_1b, torch.float64)
+    head = plain.w["model.embed_tokens.weight"]
+    checked = 0
+    for rid, p, sequences in judged:
+        for seq in sequences:
+            tokens = seq.output_token_ids
+            assert len(tokens) == n_out
+            logits = plain.hidden_states(list(p) + tokens[:-1])[len(p) - 1:] @ head.T
+            for i, tok in enumerate(tokens):
+                scores = race_scores(logits[i], t, seed, rid, seq.sample_index, i)
+                where = f"request {rid} sample {seq.sample_index} token {i}"
+                if dtype == "float32":
+                    top = torch.topk(scores, 2).values
+                    assert tok == int(scores.argmax()) or float(top[0] - top[1]) < 2e-4, \
+                        f"{where}: drew {tok}, the race's winner is {int(scores.argmax())}"
+                else:
+                    assert float(scores.max() - scores[tok]) <= 0.08, f"{where}: {float(scores.max() - scores[tok])}"
+                checked += 1
+    assert checked == 5 * n_out
+    two = judged[1][2]
+    assert len(two) == 2 and two[0].output_token_ids != two[1].output_token_ids
+    assert llm.manager.stats().blocks_in_use == 0
+
+
+def test_float32_logits_at_the_1b_widths_do_not_depend_on_the_cut(folder_1b):
+    """In 32-bit every sum is taken in an order that depends on the position alone: the logits of a
+    300-token prompt fed whole, in portions of changing size (down to two tokens, across the page's
+    edge at 256, beside another request's tokens) and with its last 32 tokens fed one by one are
+    the same bits, at the widths of the 1B shape as at the tiny ones."""
+    from tinyserve_llm_amd.engine.replay import Replay
+    ids, beside = prompt(70, 300, CONFIG.vocab_size), prompt(71, 90, CONFIG.vocab_size)
+    wanted = [0, 1, 7, 63, 64, 127, 128, 200, 254, 255, 256, 257, 268, 269, 299]
+    rep = Replay(folder_1b, "float32", 1024)
+    whole = rep.step([{"id": "w", "tokens": ids, "want": wanted}], ["w"])
+    got = {}
+    fed, other = 0, 0
+    for k, n in enumerate([2, 5, 57, 64, 3, 124, 2, 11, 32]):
+        entries = [{"id": "p", "tokens": ids[fed:fed + n], "want": [w - fed for w in wanted if fed <= w < fed + n]}]
+        if k in (2, 3, 5, 7):                # another request's portion, or its single token, in the same step
+            m = 40 if k == 2 else 1
+            entries.insert(k % 2, {"id": "o", "tokens": beside[other:other + m], "want": []})
+            other += m
+        out = rep.step(entries, [])
+        for row, w in zip(out, [w for w in wanted if fed <= w < fed + n]):
+            got[w] = row
+        fed += n
+    assert fed == 300 and sorted(got) == wanted
+    for i, w in enumerate(wanted):
+        assert torch.equal(got[w], whole[i]), f"position {w}: fed in portions {float((got[w] - whole[i]).abs().max()):.3e} off"
+    rep.step([{"id": "s", "tokens": ids[:268], "want": []}], ["p", "o"])
+    for pos in range(268, 300):
+        row = rep.step([{"id": "s", "tokens": [ids[pos]], "want": [0]}], ["s"] if pos == 299 else [])[0]
+        if pos in wanted:
+            assert torch.equal(row, whole[wanted.index(pos)]), f"position {pos}, fed singly"
