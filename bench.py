@@ -6,6 +6,12 @@ A "step" is one decode step of the whole engine (scheduler, step function, kerne
 batch 8 with 2,048-token contexts that grow while decoding. Prints ONE JSON line. The same line
 carries the 2,048-token prefill, the decode step's HBM roofline, and decode at batch 1 and 64.
 
+    python bench.py --kernel-classes [--batch B]
+
+times the kernels of one decode step class by class (qkv, attention, o, gate|up, down, norms, head,
+sampling) with events around each launch of an eager step, and prints the bytes each class has to
+read, its time and its rate beside the step's total, as one JSON line.
+
     python bench.py --scenario requests-3b | chunked-8b [--layers L]
 
 runs a whole workload through `LLM.generate` instead and prints one JSON line of its own: many
@@ -129,6 +135,110 @@ def scenario(name: str, layers: int | None, dtype_name: str) -> int:
     return 0
 
 
+def kernel_classes(llm, config, batch: int, reps: int = 5) -> dict:
+    """Times one decode step's kernels by class. An eager step (no graph) is run once with every
+    launch of the engine's kernel module noted down with its operands; then each class's launches
+    (one per layer, with that layer's own weights) are recorded into a graph of their own, and the
+    graph is replayed between two events after a sweep of the caches: a class's time is its kernels
+    and the dispatches between them, as a recorded decode step sees them. Its bytes are what it has
+    to read once (weights, or the keys and values of the live requests). The best of `reps` replays."""
+    import torch
+
+    from tinyserve_llm_amd.ops import hip
+
+    c = config
+    item = 2 if llm.dtype == torch.bfloat16 else 4
+    by_shape = {(c.q_size + 2 * c.kv_size, c.hidden_size): "qkv", (c.hidden_size, c.q_size): "o",
+                (2 * c.intermediate_size, c.hidden_size): "gate_up", (c.hidden_size, c.intermediate_size): "down",
+                (c.vocab_size, c.hidden_size): "head"}
+    calls: dict[str, list] = {}
+
+    def note(klass, nbytes, inner, a, kw):
+        calls.setdefault(klass, []).append((nbytes, inner, a, kw))
+        return inner(*a, **kw)
+
+    def product(name, weight_of):
+        inner = getattr(hip, name)
+
+        def noted(*a, **kw):
+            w = weight_of(*a, **kw)
+            if w.dim() == 4:                                   # a streaming copy: [N / 16, K / 32, 64, 8]
+                shape = (w.shape[0] * 16, w.shape[1] * 32)
+            elif w.dim() == 5:                                 # the 8-row form's: [N / 8, waves, steps, 64, 8]
+                shape = (w.shape[0] * 8, w.shape[1] * w.shape[2] * 64)
+            else:
+                shape = tuple(w.shape)
+            # (a copy's rows are padded to whole tiles)
+            klass = next((v for k, v in by_shape.items() if k[1] == shape[1] and 0 <= shape[0] - k[0] < 16), f"product {shape}")
+            return note(klass, shape[0] * shape[1] * item, inner, a, kw)
+        return noted
+
+    def other(name, klass, nbytes_of=lambda *a, **kw: 0):
+        inner = getattr(hip, name)
+        return lambda *a, **kw: note(klass, nbytes_of(*a, **kw), inner, a, kw)
+
+    live = sum(s.num_tokens for s in llm.scheduler.running)
+    kv_layer = live * 2 * c.kv_size * item
+    patched = {
+        "gemm_skinny": product("gemm_skinny", lambda x, w, *a, **kw: w),
+        "gemm_skinny8": product("gemm_skinny8", lambda x, w, *a, **kw: w),
+        "gemm_rows64": product("gemm_rows64", lambda x, packed, *a, **kw: packed),
+        "gemm_library": product("gemm_library", lambda x, w, *a, **kw: w),
+        "gemm_exact": product("gemm_exact", lambda x, w, *a, **kw: w),
+        "qkv_rope_store": product("qkv_rope_store", lambda x, w, *a, **kw: w),
+        "paged_attention_decode": other("paged_attention_decode", "attention", lambda *a, **kw: kv_layer),
+        "paged_attention_wave": other("paged_attention_wave", "attention", lambda *a, **kw: kv_layer),
+        "rmsnorm": other("rmsnorm", "norm"), "rope_store": other("rope_store", "rotation and cache write"),
+        "silu_mul": other("silu_mul", "gate"), "sample": other("sample", "sampling"), "embedding": other("embedding", "embedding"),
+    }
+    kept = {name: getattr(hip, name) for name in patched}
+    graphs, llm.runner.graphs, ahead = llm.runner.graphs, None, llm.run_ahead
+    llm.run_ahead = False
+    try:
+        llm.step()                                         # (closes the step that was started ahead, starts none)
+        for name, fn in patched.items():
+            setattr(hip, name, fn)
+        llm.step()
+        torch.cuda.synchronize()
+    finally:
+        for name, fn in kept.items():
+            setattr(hip, name, fn)
+        llm.runner.graphs, llm.run_ahead = graphs, ahead
+    sweep = torch.zeros(128 << 20, dtype=torch.int32, device="cuda")       # 512 MB: more than the caches hold
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    classes: dict[str, dict] = {}
+    tiny = torch.zeros(64, dtype=torch.int32, device="cuda")
+    calls = {"(a graph of one small kernel)": [(0, lambda: tiny.add_(1), (), {})], **calls}
+    overhead = 0.0
+    with torch.inference_mode():                          # (the step's tensors were made under it)
+        for klass, noted in calls.items():
+            for _, inner, a, kw in noted:                      # once outside a recording (libraries set themselves up)
+                inner(*a, **kw)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                outs = [inner(*a, **kw) for _, inner, a, kw in noted]
+            times = []
+            for _ in range(reps + 1):
+                sweep.sum()                                    # read, not written: the caches hold nothing of the weights, and nothing dirty
+                begin.record()
+                graph.replay()
+                end.record()
+                end.synchronize()
+                times.append(1e3 * begin.elapsed_time(end))
+            del outs, graph
+            us, nbytes = min(times[1:]) - overhead, sum(n for n, *_ in noted)
+            if klass.startswith("("):
+                overhead = us                                  # what a replay costs before its first kernel's work: taken off every class
+                continue
+            classes[klass] = {"launches": len(noted), "bytes": nbytes, "us": us, "us_per_launch": us / len(noted),
+                              "GBps": nbytes / us / 1e3, "frac_of_hbm": nbytes / us * 1e6 / HBM_BYTES_PER_S}
+    total = {"bytes": sum(r["bytes"] for r in classes.values()), "us": sum(r["us"] for r in classes.values())}
+    total["GBps"] = total["bytes"] / total["us"] / 1e3
+    return {"batch": batch, "live_tokens": live, "classes": dict(sorted(classes.items(), key=lambda kv: -kv[1]["us"])),
+            "all_classes": total, "replay_overhead_us": overhead}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -147,6 +257,8 @@ def main() -> int:
                     help="'prefill': time the 2,048-token prefill alone and print its record (for profiling)")
     ap.add_argument("--scenario", default=None, choices=sorted(SCENARIOS),
                     help="run a whole workload through LLM.generate instead of the decode step")
+    ap.add_argument("--kernel-classes", action="store_true",
+                    help="time one decode step's kernels class by class (bytes, microseconds, GB/s) and exit")
     ap.add_argument("--peaks", action="store_true",
                     help="measure what a kernel that only reads memory and a loop of matrix instructions reach on "
                          "this GPU, print them beside the published peaks and exit")
@@ -203,8 +315,9 @@ def main() -> int:
         return LLM(None, sc, CacheConfig(block_size=PAGE, caching=False), dtype=dtype, num_blocks=pages, seed=0,
                    model=model)
 
-    def decode(batch: int, steps: int, warmup: int) -> tuple[float, float]:
-        """(seconds for `steps` decode steps, mean context length over them)."""
+    def decode(batch: int, steps: int, warmup: int, classes: bool = False):
+        """(seconds for `steps` decode steps, mean context length over them); with `classes`, the
+        kernel classes of one such step instead."""
         llm = engine(batch, steps + warmup)
         sp = SamplingParams(max_tokens=max_model_len - prompt_len, temperature=0.0, ignore_eos=True)
         for _ in range(batch):
@@ -214,6 +327,8 @@ def main() -> int:
         for _ in range(warmup):
             llm.step()
         assert len(llm.scheduler.running) == batch and not llm.scheduler.waiting
+        if classes:
+            return kernel_classes(llm, c, batch)
         ctx0 = llm.scheduler.running[0].num_tokens
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -249,6 +364,15 @@ def main() -> int:
     if args.only == "prefill":
         print(json.dumps({"prefill": prefill_record()}))
         return 0
+    if args.kernel_classes:
+        print(json.dumps({"kernel_classes": decode(args.batch, 1, args.warmup, classes=True),
+                          "config": {"model": sizes["model"], "layers": args.layers, "context": prompt_len, "dtype": args.dtype}}))
+        return 0
+
+    from tinyserve_llm_amd.ops import hip
+    measured = hip.measure_peaks()       # what this box gives a kernel that only reads, and a loop of matrix instructions
+    read_peak = measured["read_GBps"] * 1e9
+    mfma_peak = measured["mfma_bf16_TFLOPs"] * 1e12 if args.dtype == "bf16" else None
 
     seconds, mean_ctx = decode(args.batch, args.steps, args.warmup)
     value = args.batch * args.steps / seconds
@@ -265,17 +389,25 @@ def main() -> int:
                    "global_batch": args.batch, "prompt_len": prompt_len, "seq_len": max_model_len,
                    "page_size": PAGE, "parallelism": "single-gpu"},
         "roofline": {"bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_BYTES_PER_S / 1e9, "unit": "GB/s",
-                     "frac": achieved / HBM_BYTES_PER_S},
+                     "frac": achieved / HBM_BYTES_PER_S, "measured_peak": read_peak / 1e9,
+                     "frac_of_measured": achieved / read_peak},
     }
     if not args.no_prefill:
         record["prefill"] = prefill_record()
-    points = {}
+        if mfma_peak:
+            record["prefill"]["measured_peak_tflops"] = mfma_peak / 1e12
+            record["prefill"]["frac_of_measured"] = record["prefill"]["frac"] * PEAK_FLOPS[args.dtype] / mfma_peak
+    points, detail = {}, {}
     for b in [int(x) for x in args.points.split(",") if x.strip()]:
         k = max(16, min(args.steps, 64))
-        s, _ = decode(b, k, 4)
+        s, ctx = decode(b, k, 4)
         points[f"decode_b{b}"] = b * k / s
+        rate = (weight_bytes + b * ctx * kv_bytes_per_token) / (s / k)
+        detail[f"decode_b{b}"] = {"tok_s": b * k / s, "ms_per_step": 1e3 * s / k, "frac": rate / HBM_BYTES_PER_S,
+                                  "frac_of_measured": rate / read_peak}
     if points:
         record["points"] = points
+        record["points_detail"] = detail
     print(json.dumps(record))
     return 0
 

@@ -541,13 +541,144 @@ def test_gate_on_the_way_out_for_up_to_64_rows(m, n, k):
 
 
 def test_weight_streaming_gemm_refuses_what_it_cannot_take():
-    x = torch.zeros(33, 2048, dtype=torch.bfloat16, device=dev())
-    w = torch.zeros(64, 2048, dtype=torch.bfloat16, device=dev())
-    assert not hip().skinny_takes(33, 2048) and not hip().skinny_takes(8, 96) and not hip().skinny_takes(8, 14336)
+    x = torch.zeros(33, 2304, dtype=torch.bfloat16, device=dev())
+    w = torch.zeros(64, 2304, dtype=torch.bfloat16, device=dev())
+    assert hip().skinny_takes(33, 2048) and hip().skinny_takes(64, 256), "33 to 64 rows over reductions of up to 2048"
+    assert not hip().skinny_takes(33, 2304) and not hip().skinny_takes(65, 2048)
+    assert not hip().skinny_takes(8, 96) and not hip().skinny_takes(8, 14336)
     with pytest.raises(hip().KernelError, match="rows"):
         hip().gemm_skinny(x, w)
     from tinyserve_llm_amd.parts.linear import linear
     assert linear(x, w).shape == (33, 64), "the vendor library takes what the skinny kernel does not"
+
+
+@pytest.mark.parametrize("m", [33, 48, 64])
+@pytest.mark.parametrize("n,k", [(2048, 2048), (3072, 1024), (130, 768), (8200, 256)])
+def test_weight_streaming_gemm_for_33_to_64_rows(m, n, k):
+    """Three and four blocks of 16 rows of x against one tile of W a workgroup, x asked for before W."""
+    g = gen(m + n + k)
+    w = (torch.randn(n, k, generator=g) * 0.05).bfloat16().to(dev())
+    x = torch.randn(m, k, generator=g).bfloat16().to(dev())
+    want = x.double().cpu() @ w.double().cpu().T
+    for packed in (None, hip().pack_weight(w)):
+        out, _ = hip().gemm_skinny(x, w, packed=packed)
+        assert out.shape == (m, n) and out.dtype == torch.bfloat16
+        torch.testing.assert_close(out.double().cpu(), want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
+    alone, _ = hip().gemm_skinny(x[m - 1:].contiguous(), w)
+    assert torch.equal(alone[0], out[m - 1]), "a row's result does not depend on the other rows"
+
+
+def bf(t):
+    """Rounded to bfloat16 and back to 64-bit."""
+    return t.float().bfloat16().double()
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 2048, 2048), (8, 2048, 8192), (5, 264, 512), (3, 44, 256), (8, 3072, 1024),     # the 8-row form
+                                   (16, 2048, 2048), (9, 130, 768), (23, 992, 512), (32, 2048, 4096), (12, 8224, 256),  # 16-row tiles
+                                   (48, 2048, 2048), (64, 3072, 1024), (33, 72, 512)])                                  # four blocks of x
+@pytest.mark.parametrize("with_residual", [True, False])
+def test_projection_that_finishes_into_a_residual_sum_and_a_norm(m, n, k, with_residual):
+    """`next_norm=`: the projection leaves T(T(y) + res), T((T(y) + res) * nw) and the rows' sums of
+    squares in parts, against the same steps in 64-bit with the storage type's roundings; then the
+    projections that take the prepared operand (plain, gated, into the rotation and the cache, and
+    the shared-x kernel) against their own definition on exactly these operands, and the whole chain
+    against norm(y + res) * nw followed by the product without any rounding."""
+    g = gen(m * 3 + n + k)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * k ** -0.5).bfloat16()
+    res = torch.randn(m, n, generator=g).bfloat16() if with_residual else None
+    nw = (1 + 0.1 * torch.randn(n, generator=g)).bfloat16()
+    eps = 1e-5
+    xd, wd, nwd = x.to(dev()), w.to(dev()), nw.to(dev())
+    def finish(rows, residual):
+        # (`linear_bf16` leaves 33 to 64 rows to the library; the kernel takes them when asked directly)
+        request = (None if residual is None else residual.to(dev()), nwd)
+        if hip().next_norm_fuses(rows, wd):
+            return hip().linear_bf16(rows, wd, next_norm=request)
+        return hip().gemm_skinny(rows, wd, next_norm=request)[0]
+
+    assert hip().next_norm_fuses(xd, wd) == (m <= 32)
+    prepared = finish(xd, res)
+    assert isinstance(prepared, hip().PreparedNorm)
+    y = x.double() @ w.double().T
+    t = bf(y) + (res.double() if with_residual else 0)
+    # (a product that lies next to a rounding boundary may round the other way than 64-bit does)
+    torch.testing.assert_close(prepared.summed.double().cpu(), bf(t), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(prepared.operand.double().cpu(), bf(t * nw.double()), rtol=2e-2, atol=2e-2)
+    assert prepared.squares.dtype == torch.float32 and prepared.squares.shape[0] == m
+    torch.testing.assert_close(prepared.squares.sum(1).double().cpu(), t.pow(2).sum(1), rtol=1e-2, atol=1e-3)
+    # every part is the sum of squares of its own columns: 8 a part in the 8-row form, else 16
+    width = 8 if hip().skinny8_takes(m, n, k) else 16
+    assert prepared.squares.shape[1] >= -(-n // width)
+    own = prepared.summed.float()      # (within a rounding of t)
+    parts = torch.stack([own[:, i:i + width].pow(2).sum(1) for i in range(0, n, width)], 1)
+    torch.testing.assert_close(prepared.squares[:, :parts.shape[1]].cpu(), parts.cpu(), rtol=3e-2, atol=1e-3)
+    assert float(prepared.squares[:, parts.shape[1]:].abs().sum()) == 0.0, "tiles past the last column count nothing"
+    alone = finish(xd[m - 1:].contiguous(), None if res is None else res[m - 1:])
+    if hip().skinny8_takes(m, n, k) == hip().skinny8_takes(1, n, k):
+        assert torch.equal(alone.summed[0], prepared.summed[m - 1]) and torch.equal(alone.operand[0], prepared.operand[m - 1])
+    # ---- what takes the prepared operand: K of the next projection is this one's N
+    scale = torch.rsqrt(prepared.squares.double().cpu().sum(1, keepdim=True) / n + eps)
+    operand = prepared.operand.double().cpu()
+    truth_in = t * torch.rsqrt(t.pow(2).mean(1, keepdim=True) + eps) * nw.double()          # no rounding
+    if n % 256 == 0 and n <= 4096:
+        for n2, glu in ((2 * 320, True), (264, False), (16384 if n <= 2048 else 512, True)):
+            if not (hip().skinny_fuses(m, n, False, True) if glu else hip().skinny_takes(m, n)):
+                continue
+            w2 = (torch.randn(n2, n, generator=g) * n ** -0.5).bfloat16()
+            out, _ = hip().gemm_skinny(prepared.operand, w2.to(dev()), glu=glu, squares=prepared.squares, eps=eps)
+            want = (operand @ w2.double().T) * scale
+            truth = truth_in @ w2.double().T
+            if glu:
+                want, truth = P.silu_mul(want), P.silu_mul(truth)
+            torch.testing.assert_close(out.double().cpu(), want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
+            torch.testing.assert_close(out.double().cpu(), truth, rtol=4e-2, atol=4e-2 * float(truth.abs().max()))
+    if n % 1024 == 0 and m > 32:
+        for glu in (False, True):
+            w2 = (torch.randn(8192, n, generator=g) * n ** -0.5).bfloat16().to(dev())
+            out = hip().gemm_rows64(prepared.operand, hip().pack_weight(w2), glu=glu, squares=prepared.squares, eps=eps)
+            want = (operand @ w2.double().cpu().T) * scale
+            want = P.silu_mul(want) if glu else want
+            torch.testing.assert_close(out.double().cpu(), want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
+    if hip().qkv_rope_fuses(prepared.operand, torch.empty(1, n, dtype=torch.bfloat16, device=dev()), 64, None):
+        nh, nkv, hd = 3, 1, 64
+        w2 = (torch.randn((nh + 2 * nkv) * hd, n, generator=g) * n ** -0.5).bfloat16().to(dev())
+        table = torch.randn(32, hd, generator=g).to(dev())
+        positions = torch.randint(0, 32, (m,), generator=g, dtype=torch.int32).to(dev())
+        slots = torch.randperm(128, generator=g)[:m].to(torch.int32).to(dev())
+        kp = [torch.zeros(4, nkv, 32, hd, dtype=torch.bfloat16, device=dev()) for _ in range(2)]
+        vp = [torch.zeros(4, nkv, hd, 32, dtype=torch.bfloat16, device=dev()) for _ in range(2)]
+        q, _ = hip().qkv_rope_store(prepared.operand, w2, table, positions, slots, kp[0].permute(0, 2, 1, 3),
+                                    vp[0].permute(0, 3, 1, 2), nh, nkv, hd, eps=eps, squares=prepared.squares)
+        # the same through the separate kernels: the norm applied to the operand first
+        normed = (operand * scale).bfloat16().to(dev())
+        q_want = hip().rope_store(hip().linear_bf16(normed, w2), table, positions, slots, kp[1].permute(0, 2, 1, 3),
+                                  vp[1].permute(0, 3, 1, 2), nh, nkv, hd)
+        torch.testing.assert_close(q.double(), q_want.double(), rtol=3e-2, atol=3e-2 * float(q_want.abs().max()))
+        torch.testing.assert_close(kp[0].double(), kp[1].double(), rtol=3e-2, atol=3e-2 * float(kp[1].abs().max()))
+        torch.testing.assert_close(vp[0].double(), vp[1].double(), rtol=3e-2, atol=3e-2 * float(vp[1].abs().max()))
+        assert torch.equal(kp[0] == 0, kp[1] == 0), "the same slots are written"
+
+
+def test_a_prepared_norm_is_refused_where_no_kernel_leaves_one():
+    x = torch.zeros(70, 512, dtype=torch.bfloat16, device=dev())
+    w = torch.zeros(64, 512, dtype=torch.bfloat16, device=dev())
+    nw = torch.ones(64, dtype=torch.bfloat16, device=dev())
+    assert not hip().next_norm_fuses(x, w), "70 rows go to the vendor's library"
+    with pytest.raises(hip().KernelError, match="prepared norm"):
+        hip().linear_bf16(x, w, next_norm=(None, nw))
+    with pytest.raises(hip().KernelError, match="next norm's weight"):
+        hip().linear_bf16(x[:8].contiguous(), w, next_norm=(None, nw[:32].contiguous()))
+    with pytest.raises(hip().KernelError, match="residual"):
+        hip().linear_bf16(x[:8].contiguous(), w, next_norm=(x[:8, :32], nw))
+    with pytest.raises(hip().KernelError, match="sums of squares"):
+        hip().gemm_skinny(x[:8].contiguous(), w, squares=torch.zeros(7, 4, device=dev()), eps=1e-5)
+    from tinyserve_llm_amd.parts.linear import DeferredNorm, NormRequest, linear
+    d = linear(x, w, then=NormRequest(nw, 1e-5, None))
+    assert isinstance(d, DeferredNorm) and d.prepared is None and d.x.shape == (70, 64), "left to the next projection"
+    d8 = linear(x[:8].contiguous(), w, then=NormRequest(nw, 1e-5, None))
+    assert d8.prepared is not None and d8.residual_out is d8.prepared.summed
+    assert d8.materialize().shape == (8, 64)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

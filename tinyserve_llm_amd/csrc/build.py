@@ -28,6 +28,10 @@ FLAGS = [
     # matrix-core results stay in ordinary vector registers: the softmax and the epilogues work on
     # them with vector instructions, and copies to and from the accumulation registers cost more
     "-mllvm", "-amdgpu-mfma-vgpr-form=1",
+    # the first kernel arguments arrive in scalar registers with the wave instead of being loaded
+    # by its first instructions: a decode step is a hundred short kernels, each of which would
+    # otherwise start with a trip to memory for its arguments
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-Wno-unused-command-line-argument", "-Wno-unknown-attributes",
 ]
 

@@ -32,6 +32,12 @@ struct Rows64Args {
   void* y;               // [M, N] (GLU: [M, N / 2]), row stride ldy
   int M, N, K;
   int64_t ldx, ldy;
+  // the norm on the way in, prepared by the kernel that made x (see MODE_PREP in gemm_skinny.hip): x is
+  // the operand as it stands and a row's scale rsqrt(sum of its ssq_parts parts / K + eps) multiplies
+  // its finished sums; null: no scale
+  const float* ssq_in;
+  int ssq_parts;
+  float eps;
 };
 
 template <bool GLU, typename OUT>
@@ -39,6 +45,7 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
   // x as the B operands of the matrix instruction: [buffer][step][block of 16 rows][lane], lane r + 16 g
   // holding k = 8 g .. 8 g + 7 of row r
   __shared__ uint4 xs[2][R64_CHUNK_STEPS][4][TS_WAVE];
+  __shared__ float row_scale[64];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TS_WAVE), lane = threadIdx.x & (TS_WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
   const int nsteps = a.K / SK_KSTEP, nchunks = nsteps / R64_CHUNK_STEPS;   // (a multiple of 4)
@@ -70,6 +77,25 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
     };
     uint4 A[R64_STAGE_STEPS][4], B[R64_STAGE_STEPS][4];
     ask(0, A);
+    // the rows' scales, rows 16 sw .. 16 sw + 15 in this wave: a lane every 64th part (all sixteen rows' loads
+    // under way together), then the lanes in a fixed tree
+    if (a.ssq_in) {
+      float sums[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sums[i] = 0.f;
+      for (int q = lane; q < a.ssq_parts; q += TS_WAVE) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int m = 16 * sw + i;
+          sums[i] += m < a.M ? a.ssq_in[(int64_t)m * a.ssq_parts + q] : 0.f;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float total = wave_sum(sums[i]);
+        if (lane == 0) row_scale[16 * sw + i] = 1.0f / sqrtf(total / (float)a.K + a.eps);
+      }
+    }
     for (int c = 0; c < nchunks; c += 2) {
       ask(c + 1, B);
       put(c, A);
@@ -152,6 +178,11 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
     if (m >= a.M) continue;
     float4_t u = {0.f, 0.f, 0.f, 0.f};
     if (GLU) u = ex[(wave * 4 + b) * TS_WAVE + lane];
+    if (a.ssq_in) {                                  // (the same for every thread)
+      const float scale = row_scale[m];
+      acc[b] *= scale;
+      u *= scale;
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) Num<OUT>::st(y + (int64_t)m * a.ldy + n0 + j, GLU ? sk_silu(acc[b][j]) * u[j] : acc[b][j]);
   }
@@ -165,13 +196,16 @@ static int r64_launch(const Rows64Args& a, hipStream_t stream) {
 
 // x [M <= 64, K] (row stride ldx), w16: W [N, K] as its 16-row packed copy, y [M, N] or, with glu, [M, N / 2]
 // (row stride ldy; out_f32: 32-bit sums instead of bfloat16). N a multiple of 64 (128 with glu), K of 1,024.
+// ssq_in [M, ssq_parts] and eps: the prepared norm's scale per row (null: none).
 extern "C" int ts_gemm_rows64_bf16(void* y, const void* x, const void* w16, int M, int N, int K, int64_t ldx, int64_t ldy,
-                                   int glu, int out_f32, hipStream_t stream) {
+                                   int glu, int out_f32, const void* ssq_in, int ssq_parts, float eps, hipStream_t stream) {
   if (M <= 0 || N <= 0) return TS_OK;
   if (M > 64 || N % (glu ? 128 : 64) || K <= 0 || K % 1024 || ldx < K || (ldx % 8) || !y || !x || !w16) return TS_BAD_SHAPE;
+  if (ldy < (glu ? N / 2 : N) || (((uintptr_t)y) & (out_f32 ? 3 : 1))) return TS_BAD_SHAPE;
   if ((((uintptr_t)x) | ((uintptr_t)w16)) & 15) return TS_BAD_SHAPE;
   if (glu && out_f32) return TS_BAD_SHAPE;
-  Rows64Args a = {(const bf16_t*)x, (const bf16_t*)w16, y, M, N, K, ldx, ldy};
+  if (ssq_in && (ssq_parts <= 0 || (((uintptr_t)ssq_in) & 3))) return TS_BAD_SHAPE;
+  Rows64Args a = {(const bf16_t*)x, (const bf16_t*)w16, y, M, N, K, ldx, ldy, (const float*)ssq_in, ssq_parts, eps};
   if (glu) return r64_launch<true, bf16_t>(a, stream);
   if (out_f32) return r64_launch<false, float>(a, stream);
   return r64_launch<false, bf16_t>(a, stream);

@@ -13,6 +13,14 @@
 //              (the separate norm kernel rounds (x + res) * scale first and the product with nw
 //              again: the same value up to the rounding of the storage type); workgroup 0 also writes
 //              T(x + res) as the new residual
+//   MODE_PREP  the norm on the way in, half done already by the kernel that made x (EPI_NEXT below):
+//              x is the operand T((h + res) * nw) as it stands, and the row's scale comes from the
+//              partial sums of squares that kernel left, one per row and column tile, added up in
+//              the tiles' order; any number of 16-row blocks of x
+//   EPI_NEXT   what follows a projection whose result goes into a residual sum and a norm: with
+//              t = T(y) + res, the kernel writes T(t) as the new residual, T(t * nw) as the next
+//              projection's operand and, per row and 16-column tile (8 in the 8-row form), the sum of
+//              t^2 over the tile's columns; y itself is not stored
 //   EPI_GLU    W = [gate rows | up rows]; a workgroup takes matching rows of both and writes
 //              silu(gate) * up, y being [M, N / 2]
 //   EPI_ROPE   W = [q heads | k heads | v heads] of head_dim columns each; a 16-row tile holds 8
@@ -33,6 +41,15 @@ struct SkinnyArgs {
   int M, N, K, packed;
   int64_t ldx, ldw, ldy;
   float eps;
+  // MODE_PREP: sums of squares [M, ssq_parts] of the rows of h + res, in parts (K is their width)
+  const float* ssq_in;
+  int ssq_parts;
+  // EPI_NEXT: res [M, N] or null, next norm's weight [N], outputs [M, N] dense and [M, tiles of the grid]
+  const bf16_t* next_res;
+  const bf16_t* next_nw;
+  bf16_t* next_res_out;
+  bf16_t* next_op;
+  float* ssq_out;
   // EPI_ROPE: N = (nh + 2 nkv) * hd; cos_sin [max_pos, hd] 32-bit, [cos | sin] halves; slot -1 stores nothing.
   // key element: page * kp + offset * ks + head * kh + d; value element: page * vp + offset * vs + head * vh + d * vd
   const float* cos_sin;
@@ -50,15 +67,15 @@ struct SkinnyArgs {
 template <int RT, int CB, int STEPS, int MODE, int EPI, int MAXT, typename OUT>
 __global__ void __launch_bounds__(MAXT)
 gemm_skinny_kernel(const SkinnyArgs a) {
-  constexpr bool GLU = EPI == EPI_GLU, ROPE = EPI == EPI_ROPE, PAIRS = EPI != EPI_NONE;
-  static_assert(MODE == MODE_PLAIN || CB == 1, "the fused norm serves one block of rows");
+  constexpr bool GLU = EPI == EPI_GLU, ROPE = EPI == EPI_ROPE, PAIRS = GLU || ROPE, NEXT = EPI == EPI_NEXT;
+  static_assert(MODE != MODE_NORM || CB == 1, "the fused norm serves one block of rows");
   static_assert(!GLU || RT % 2 == 0, "gate and up tiles come in pairs");
   // steps of x fetched at a time: fewer where more blocks of x, more row tiles of W or a larger workgroup leave fewer registers
   constexpr int SK_XBATCH = CB >= 4 ? 4 : (CB == 2 && (MAXT > 512 || RT >= 4)) ? 4 : 8;
   extern __shared__ __align__(16) float smem[];
   const int nwaves = blockDim.x / TS_WAVE;
   float* part = smem;                                   // [nwaves][RT][CB][256]
-  float* ssq = smem + (size_t)nwaves * RT * CB * 256;   // [nwaves][16]
+  float* ssq = smem + (size_t)nwaves * RT * CB * 256;   // MODE_NORM: [nwaves][16]; MODE_PREP: [CB][nwaves][16]
   const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
   // GLU: tiles 0 .. RT/2-1 are gate rows n0 + 16 t, tiles RT/2 .. RT-1 the up rows N/2 below them.
@@ -97,6 +114,20 @@ gemm_skinny_kernel(const SkinnyArgs a) {
     __builtin_amdgcn_sched_barrier(0);                  // the compiler keeps these loads ahead of W's
   }
 
+  // ---- MODE_PLAIN with room in the registers: all of this wave's x is asked for before W. It is
+  // small and comes from the cache, loads come back in the order they were issued, and so the products
+  // can start the moment W has arrived; asked for after W, every batch of x would wait behind all of W
+  // and then for its own trip to the cache.
+  constexpr bool X_FIRST = MODE != MODE_NORM && MAXT <= 512 && (CB * STEPS + RT * STEPS) <= 48;
+  uint4 xall[X_FIRST ? CB : 1][X_FIRST ? STEPS : 1];
+  if constexpr (X_FIRST) {
+#pragma unroll
+    for (int b = 0; b < CB; ++b)
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) xall[b][s] = *(const uint4*)(xrow[b] + s * SK_KSTEP);   // rows past M repeat row 0 and are not stored
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
   // ---- every load of this wave's slice of W, at once
   uint4 wreg[RT][STEPS];
 #pragma unroll
@@ -128,6 +159,51 @@ gemm_skinny_kernel(const SkinnyArgs a) {
   // all of W's loads are in flight before anything waits: left to itself the compiler interleaves
   // them with the products to save registers, and the matrix no longer streams at memory speed
   __builtin_amdgcn_sched_barrier(0);
+
+  // ---- MODE_PREP: the rows' sums of squares, from the parts the kernel before left. The parts of a
+  // row are dealt out in runs to the 4 x nwaves lanes that hold the row (lane (r, g) of wave w adds up
+  // run 4 w + g of row 16 b + r), and the runs' sums meet in LDS as the waves' squares do in MODE_NORM.
+  // The parts are asked for here, right behind W (whose addresses are in registers when the wave
+  // starts, while the address of the parts has to be fetched first: asked for ahead of W they would
+  // hold W back), and added up after the products. (Runs longer than the registers set aside hold,
+  // as short reductions with their few waves have, are fetched and added after the products.)
+  constexpr int PREP_VECS = 2;                          // 16-byte pieces of a run that a lane holds
+  float4 pv[MODE == MODE_PREP ? CB : 1][MODE == MODE_PREP ? PREP_VECS : 1];
+  // parts of a row per lane, in whole pieces of four
+  const int prep_run = MODE == MODE_PREP ? (a.ssq_parts + 16 * nwaves - 1) / (16 * nwaves) * 4 : 0;
+  const bool prep_early = MODE == MODE_PREP && prep_run <= 4 * PREP_VECS && a.ssq_parts % 4 == 0;
+  if constexpr (MODE == MODE_PREP) {
+    if (prep_early) {
+      const int first = (4 * wave + g) * prep_run;
+#pragma unroll
+      for (int b = 0; b < CB; ++b)
+#pragma unroll
+        for (int i = 0; i < PREP_VECS; ++i)
+          pv[b][i] = (xok[b] && 4 * i < prep_run && first + 4 * i < a.ssq_parts)
+                         ? *(const float4*)(a.ssq_in + (int64_t)(16 * b + r) * a.ssq_parts + first + 4 * i)
+                         : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  // ---- EPI_NEXT: the residual and the next norm's weight of the four columns this thread will finish
+  // are asked for right behind W (where every thread finishes at most one item and the columns are
+  // whole), so that the way out does not wait for a trip to the cache
+  constexpr int NEXT_ITEMS = (EPI == EPI_GLU ? RT / 2 : RT) * CB * 64;
+  const bool next_early = NEXT && NEXT_ITEMS <= (int)blockDim.x && a.N % 4 == 0;
+  uint2 pre_res = make_uint2(0, 0), pre_nw = make_uint2(0, 0);
+  if constexpr (NEXT) {
+    if (next_early && (int)threadIdx.x < NEXT_ITEMS) {
+      const int tile = threadIdx.x / 64, e = threadIdx.x - tile * 64;
+      const int t = tile / CB, b = tile - t * CB, m = b * 16 + (e >> 2), n = n0 + t * 16 + (e & 3) * 4;
+      if (m < a.M && n < a.N) {
+        pre_nw = *(const uint2*)(a.next_nw + n);
+        if (a.next_res) pre_res = *(const uint2*)(a.next_res + (int64_t)m * a.N + n);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
 
   float4_t acc[RT][CB];
 #pragma unroll
@@ -170,6 +246,13 @@ gemm_skinny_kernel(const SkinnyArgs a) {
     sq += __shfl_xor(sq, 16, TS_WAVE);
     sq += __shfl_xor(sq, 32, TS_WAVE);
     if (g == 0) ssq[wave * 16 + r] = sq;
+  } else if constexpr (X_FIRST) {
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+      for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int b = 0; b < CB; ++b) acc[t][b] = sk_mfma(wreg[t][s], xall[b][s], acc[t][b]);
   } else {
     // ---- x in batches of steps, then the products
 #pragma unroll
@@ -189,6 +272,22 @@ gemm_skinny_kernel(const SkinnyArgs a) {
           for (int b = 0; b < CB; ++b) acc[t][b] = sk_mfma(wreg[t][s0 + s], xb[b][s], acc[t][b]);
     }
   }
+  if constexpr (MODE == MODE_PREP) {
+    const int first = (4 * wave + g) * prep_run;
+#pragma unroll
+    for (int b = 0; b < CB; ++b) {
+      float run = 0.f;
+      if (prep_early) {
+#pragma unroll
+        for (int i = 0; i < PREP_VECS; ++i) run += (pv[b][i].x + pv[b][i].y) + (pv[b][i].z + pv[b][i].w);
+      } else if (xok[b]) {
+        for (int i = first; i < first + prep_run && i < a.ssq_parts; ++i) run += a.ssq_in[(int64_t)(16 * b + r) * a.ssq_parts + i];
+      }
+      run += __shfl_xor(run, 16, TS_WAVE);
+      run += __shfl_xor(run, 32, TS_WAVE);
+      if (g == 0) ssq[(b * nwaves + wave) * 16 + r] = run;
+    }
+  }
   // acc[t][b][j] = sum over this wave's k of W[row 16 t + 4 g + j of the workgroup, k] * f(x)[16 b + r, k]
 #pragma unroll
   for (int t = 0; t < RT; ++t)
@@ -199,6 +298,7 @@ gemm_skinny_kernel(const SkinnyArgs a) {
   __syncthreads();
   // part[.][t][b][m_local * 16 + n_local]: a thread sums 4 consecutive n of one m over the waves in order
   OUT* y = (OUT*)a.y;
+  const float inv_k = 1.0f / (float)a.K;
   const int ncols = GLU ? half : a.N;
   // ROPE: a tile gives 8 columns of a head's first half (n_local 0 .. 7) and their partners (n_local 8 .. 15): 32 items of 4
   constexpr int PER_TILE = ROPE ? 32 : 64;
@@ -219,10 +319,10 @@ gemm_skinny_kernel(const SkinnyArgs a) {
         for (int j = 0; j < 4; ++j) u[j] += pu[j];
       }
     }
-    if (MODE == MODE_NORM) {                              // the row's scale, from every wave's squares
+    if (MODE != MODE_PLAIN) {                             // the row's scale, from every wave's squares (MODE_PREP: from the row's total)
       float total = 0.f;
-      for (int wv = 0; wv < nwaves; ++wv) total += ssq[wv * 16 + ml];
-      const float inv = 1.0f / sqrtf(total / (float)a.K + a.eps);
+      for (int wv = 0; wv < nwaves; ++wv) total += ssq[((MODE == MODE_PREP ? b : 0) * nwaves + wv) * 16 + ml];
+      const float inv = __builtin_amdgcn_rsqf(total * inv_k + a.eps);   // (the hardware's reciprocal square root: within a rounding)
 #pragma unroll
       for (int j = 0; j < 4; ++j) { s[j] *= inv; u[j] *= inv; }
     }
@@ -272,6 +372,40 @@ gemm_skinny_kernel(const SkinnyArgs a) {
       }
       continue;
     }
+    if constexpr (NEXT) {
+      // t = T(y) + res; the new residual T(t), the next operand T(t * nw), and the tile's share of the row's
+      // sum of t^2: the four threads that hold a row's 16 columns of a tile are neighbours in a wave
+      float sq = 0.f, tv[4], ov[4];
+      const uint32_t early_res[2] = {pre_res.x, pre_res.y}, early_nw[2] = {pre_nw.x, pre_nw.y};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const bool in = n + j < a.N;
+        const int64_t at = (int64_t)m * a.N + (in ? n + j : 0);
+        // (fetched at the start where that was possible: the low half of a word is the even column)
+        const float rj = next_early ? __uint_as_float((early_res[j >> 1] >> (16 * (j & 1))) << 16)
+                                    : (a.next_res ? bf2f(a.next_res[at]) : 0.f);
+        const float nj = next_early ? __uint_as_float((early_nw[j >> 1] >> (16 * (j & 1))) << 16) : bf2f(a.next_nw[in ? n + j : 0]);
+        const float sum = __uint_as_float(sk_round(s[j]) << 16) + rj;
+        tv[j] = sum;
+        ov[j] = sum * nj;
+        sq = in ? fmaf(sum, sum, sq) : sq;
+      }
+      sq += __shfl_xor(sq, 1, TS_WAVE);
+      sq += __shfl_xor(sq, 2, TS_WAVE);
+      if (!(e & 3)) a.ssq_out[(int64_t)m * gridDim.x * OT + (int64_t)blockIdx.x * OT + t] = sq;
+      if (a.N % 4 == 0 && n + 3 < a.N) {
+        *(uint2*)(a.next_res_out + (int64_t)m * a.N + n) = make_uint2(sk_round(tv[0]) | (sk_round(tv[1]) << 16), sk_round(tv[2]) | (sk_round(tv[3]) << 16));
+        *(uint2*)(a.next_op + (int64_t)m * a.N + n) = make_uint2(sk_round(ov[0]) | (sk_round(ov[1]) << 16), sk_round(ov[2]) | (sk_round(ov[3]) << 16));
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (n + j < a.N) {
+            a.next_res_out[(int64_t)m * a.N + n + j] = (bf16_t)sk_round(tv[j]);
+            a.next_op[(int64_t)m * a.N + n + j] = (bf16_t)sk_round(ov[j]);
+          }
+      }
+      continue;
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       if (n + j < ncols) Num<OUT>::st(y + (int64_t)m * a.ldy + n + j, GLU ? sk_silu(s[j]) * u[j] : s[j]);
@@ -281,7 +415,7 @@ gemm_skinny_kernel(const SkinnyArgs a) {
 template <int RT, int CB, int STEPS, int MODE, int GLU, typename OUT>
 static int sk_launch(const SkinnyArgs& a, hipStream_t stream) {
   const int nwaves = a.K / (STEPS * SK_KSTEP);
-  const size_t smem = sizeof(float) * ((size_t)nwaves * RT * CB * 256 + (size_t)nwaves * 16);
+  const size_t smem = sizeof(float) * ((size_t)nwaves * RT * CB * 256 + (size_t)nwaves * 16 * CB);
   constexpr int OT = GLU == EPI_GLU ? RT / 2 : RT;
   const int ncols = GLU == EPI_GLU ? a.N / 2 : a.N;     // (EPI_ROPE: a 16-row tile of the matrix per 8 columns and their partners)
   dim3 grid((ncols + 16 * OT - 1) / (16 * OT)), block(nwaves * TS_WAVE);
@@ -289,7 +423,7 @@ static int sk_launch(const SkinnyArgs& a, hipStream_t stream) {
     gemm_skinny_kernel<RT, CB, STEPS, MODE, GLU, 512, OUT><<<grid, block, smem, stream>>>(a);
   } else {
     // a workgroup of 16 waves has 128 registers a lane: one or two row tiles, and no fused norm
-    if constexpr (MODE == MODE_PLAIN && (RT == 1 || (RT == 2 && CB == 1)))
+    if constexpr (MODE != MODE_NORM && (RT == 1 || (RT == 2 && CB == 1)))
       gemm_skinny_kernel<RT, CB, STEPS, MODE, GLU, 1024, OUT><<<grid, block, smem, stream>>>(a);
     else return TS_BAD_SHAPE;
   }
@@ -299,19 +433,20 @@ static int sk_launch(const SkinnyArgs& a, hipStream_t stream) {
 // Picks the instance: slices of 256 k while that needs at most 16 waves, else slices of 512; more
 // rows of W per workgroup for wide matrices once that still leaves a workgroup per compute unit
 // (fewer workgroups repeat less of the work on x).
-template <int MODE, int GLU, typename OUT>
+template <int MODE, int EPI, typename OUT>
 static int sk_dispatch(const SkinnyArgs& a, hipStream_t stream) {
+  constexpr bool GLU = EPI == EPI_GLU, NORM = MODE == MODE_NORM;
   const int steps = (a.K % 256 == 0 && a.K / 256 <= 16) ? 8 : 16;
   if (a.K % (steps * SK_KSTEP) || a.K / (steps * SK_KSTEP) > 16) return TS_BAD_SHAPE;
   const int nwaves = a.K / (steps * SK_KSTEP);
   const int cb = (a.M + 15) / 16;
-  if (MODE == MODE_NORM && cb != 1) return TS_BAD_SHAPE;
+  if (NORM && cb != 1) return TS_BAD_SHAPE;
   const int ncols = GLU ? a.N / 2 : a.N;
-#define SK_GO(RT, CB, ST) return sk_launch<RT, CB, ST, MODE, GLU, OUT>(a, stream)
-  if constexpr (MODE == MODE_NORM || GLU != 0) {
+#define SK_GO(RT, CB, ST) return sk_launch<RT, CB, ST, MODE, EPI, OUT>(a, stream)
+  if constexpr (NORM || GLU) {
     // the instances that hold x + res or four row tiles need the registers of a workgroup of 8 waves
     if (steps != 8) return TS_BAD_SHAPE;
-    if constexpr (MODE == MODE_PLAIN && GLU != 0) {
+    if constexpr (!NORM && GLU) {
       // the gate for 17 to 64 rows of x: two or four blocks of rows against the same registers of W
       if (cb > 1 && nwaves > 8) return TS_BAD_SHAPE;
       if (cb == 2) { if (ncols >= 4096) SK_GO(4, 2, 8); else SK_GO(2, 2, 8); }
@@ -321,10 +456,14 @@ static int sk_dispatch(const SkinnyArgs& a, hipStream_t stream) {
       if (ncols >= 4096 * (GLU ? 1 : 2)) SK_GO(4, 1, 8);
       if (GLU || ncols >= 4096) SK_GO(2, 1, 8);
     }
-    if constexpr (GLU == 0) SK_GO(1, 1, 8);
-    if constexpr (MODE == MODE_PLAIN) SK_GO(2, 1, 8);   // the gate alone, in a workgroup of up to 16 waves
+    if constexpr (!GLU) SK_GO(1, 1, 8);
+    if constexpr (!NORM) SK_GO(2, 1, 8);                // the gate alone, in a workgroup of up to 16 waves
     return TS_BAD_SHAPE;
   } else {
+    if (cb > 2) {                                       // 33 to 64 rows of x: reductions of up to 2048 in 8 waves
+      if (steps == 8 && nwaves <= 8) SK_GO(1, 4, 8);
+      return TS_BAD_SHAPE;
+    }
     const bool two = a.N >= 8192 && (nwaves <= 8 || cb == 1);
     if (steps == 8) {
       if (two) { if (cb == 1) SK_GO(2, 1, 8); else SK_GO(2, 2, 8); }
@@ -345,7 +484,7 @@ static int sk_dispatch(const SkinnyArgs& a, hipStream_t stream) {
 // gives 256 workgroups, one per compute unit, and a reduction of 8,192 fits the 8 waves of one
 // workgroup (a wave covers 64 STEPS of k), where the 16-row form needs 16 waves on half the chip.
 // packed: W in the order of these loads, [N / 8 tiles][waves][STEPS][lane][8] (see hip.pack_weight8).
-template <int STEPS, int MAXT, typename OUT>
+template <int STEPS, int MAXT, typename OUT, bool NEXT = false>
 __global__ void __launch_bounds__(MAXT)
 gemm_skinny8_kernel(const SkinnyArgs a) {
   extern __shared__ __align__(16) float smem[];         // [nwaves][256]
@@ -378,6 +517,16 @@ gemm_skinny8_kernel(const SkinnyArgs a) {
     for (int s = 0; s < STEPS; ++s) wreg[s] = *(const uint4*)(wrow + s * SK_KSTEP);
   }
   __builtin_amdgcn_sched_barrier(0);                    // all of W's loads are in flight before anything waits
+  // EPI_NEXT: the residual and the next norm's weight of the element this thread will finish, asked for right behind W
+  bf16_t pre_res = 0, pre_nw = 0;
+  if constexpr (NEXT) {
+    const int m = threadIdx.x >> 3, n = n0 + (threadIdx.x & 7);
+    if (threadIdx.x < 64 && m < a.M && n < a.N) {
+      pre_nw = a.next_nw[n];
+      if (a.next_res) pre_res = a.next_res[(int64_t)m * a.N + n];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
   float4_t acc = {0.f, 0.f, 0.f, 0.f};
   if (X_FIRST) {
 #pragma unroll
@@ -402,7 +551,29 @@ gemm_skinny8_kernel(const SkinnyArgs a) {
   for (int wv = 0; wv < nwaves; ++wv)                    // waves in order, within a wave the lower half of k first
     sum += smem[wv * 256 + m * 16 + nl] + smem[wv * 256 + (m + 8) * 16 + nl + 8];
   const int n = n0 + nl;
-  if constexpr (sizeof(OUT) == 4) {
+  if constexpr (NEXT) {
+    // EPI_NEXT (see the top of the file): the eight threads of a row hold the tile's eight columns
+    const bool in = m < a.M && n < a.N;
+    const float t = __uint_as_float(sk_round(sum) << 16) + bf2f(pre_res);
+    float sq = in ? t * t : 0.f;
+    sq += __shfl_xor(sq, 1, TS_WAVE);
+    sq += __shfl_xor(sq, 2, TS_WAVE);
+    sq += __shfl_xor(sq, 4, TS_WAVE);
+    if (nl == 0 && m < a.M) a.ssq_out[(int64_t)m * gridDim.x + blockIdx.x] = sq;
+    const uint32_t res_mine = sk_round(t), op_mine = sk_round(t * bf2f(pre_nw));
+    const uint32_t res_next = __shfl_down(res_mine, 1, TS_WAVE), op_next = __shfl_down(op_mine, 1, TS_WAVE);
+    if (m < a.M && !(nl & 1)) {
+      bf16_t* r_dst = a.next_res_out + (int64_t)m * a.N + n;
+      bf16_t* o_dst = a.next_op + (int64_t)m * a.N + n;
+      if (n + 1 < a.N && !((((uintptr_t)r_dst) | ((uintptr_t)o_dst)) & 3)) {
+        *(uint32_t*)r_dst = res_mine | (res_next << 16);
+        *(uint32_t*)o_dst = op_mine | (op_next << 16);
+      } else {
+        if (n < a.N) { r_dst[0] = (bf16_t)res_mine; o_dst[0] = (bf16_t)op_mine; }
+        if (n + 1 < a.N) { r_dst[1] = (bf16_t)res_next; o_dst[1] = (bf16_t)op_next; }
+      }
+    }
+  } else if constexpr (sizeof(OUT) == 4) {
     if (m < a.M && n < a.N) ((float*)a.y)[(int64_t)m * a.ldy + n] = sum;
   } else {
     const uint32_t mine = sk_round(sum), next = __shfl_down(mine, 1, TS_WAVE);
@@ -417,7 +588,7 @@ gemm_skinny8_kernel(const SkinnyArgs a) {
   }
 }
 
-template <typename OUT>
+template <typename OUT, bool NEXT = false>
 static int sk8_dispatch(const SkinnyArgs& a, hipStream_t stream) {
   // a wave covers 64 STEPS of k; 8 waves where the reduction allows it, never more than 16
   int steps = 0;
@@ -428,54 +599,100 @@ static int sk8_dispatch(const SkinnyArgs& a, hipStream_t stream) {
   const int nwaves = a.K / (64 * steps);
   dim3 grid((a.N + 7) / 8), block(nwaves * TS_WAVE);
   const size_t smem = sizeof(float) * 256 * nwaves;
-  if (steps == 4) gemm_skinny8_kernel<4, 512, OUT><<<grid, block, smem, stream>>>(a);
-  else if (steps == 8) gemm_skinny8_kernel<8, 512, OUT><<<grid, block, smem, stream>>>(a);
-  else if (nwaves <= 8) gemm_skinny8_kernel<16, 512, OUT><<<grid, block, smem, stream>>>(a);
-  else gemm_skinny8_kernel<16, 1024, OUT><<<grid, block, smem, stream>>>(a);
+  if (steps == 4) gemm_skinny8_kernel<4, 512, OUT, NEXT><<<grid, block, smem, stream>>>(a);
+  else if (steps == 8) gemm_skinny8_kernel<8, 512, OUT, NEXT><<<grid, block, smem, stream>>>(a);
+  else if (nwaves <= 8) gemm_skinny8_kernel<16, 512, OUT, NEXT><<<grid, block, smem, stream>>>(a);
+  else gemm_skinny8_kernel<16, 1024, OUT, NEXT><<<grid, block, smem, stream>>>(a);
   return ts_check_launch();
+}
+
+// The operands of EPI_NEXT, checked: the next norm's weight [N], the outputs [M, N] dense (the new residual
+// and the next operand) and [M, parts] (sums of squares), an optional residual [M, N].
+static bool sk_next_ok(const void* next_res, const void* next_nw, const void* next_res_out, const void* next_op,
+                       const void* ssq_out) {
+  if (!next_nw || !next_res_out || !next_op || !ssq_out) return false;
+  return !((((uintptr_t)next_res) | ((uintptr_t)next_nw) | ((uintptr_t)next_res_out) | ((uintptr_t)next_op)) & 1) &&
+         !(((uintptr_t)ssq_out) & 3);
 }
 
 // y [M <= 8, N] = x · W^T by the 8-row form above: K a multiple of 256 up to 8,192 or of 1,024 up to
 // 16,384; contiguous 16-byte aligned rows. out_dtype: 1 bfloat16, 0 float. packed: w is
-// hip.pack_weight8(W) for this K, ldw unused, N a multiple of 8.
+// hip.pack_weight8(W) for this K, ldw unused, N a multiple of 8. With next_nw (EPI_NEXT; bfloat16 only)
+// y is not written: next_res_out, next_op [M, N] and ssq_out [M, (N + 7) / 8] are.
 extern "C" int ts_gemm_skinny8_bf16(void* y, const void* x, const void* w, int M, int N, int K, int64_t ldx, int64_t ldw,
-                                    int64_t ldy, int out_dtype, int packed, hipStream_t stream) {
+                                    int64_t ldy, int out_dtype, int packed, const void* next_res, const void* next_nw,
+                                    void* next_res_out, void* next_op, void* ssq_out, hipStream_t stream) {
   if (M <= 0 || N <= 0) return TS_OK;
-  if (M > 8 || K <= 0 || ldx % 8 || ldx < K || ldy < N || (!packed && (ldw % 8 || ldw < K)) || (packed && N % 8)) return TS_BAD_SHAPE;
-  if (((uintptr_t)x | (uintptr_t)w) & 15 || !y) return TS_BAD_SHAPE;
+  if (M > 8 || K <= 0 || ldx % 8 || ldx < K || (!packed && (ldw % 8 || ldw < K)) || (packed && N % 8)) return TS_BAD_SHAPE;
+  if (((uintptr_t)x | (uintptr_t)w) & 15) return TS_BAD_SHAPE;
   SkinnyArgs a = {};
   a.x = (const bf16_t*)x; a.w = (const bf16_t*)w; a.y = y; a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldw = ldw; a.ldy = ldy;
   a.packed = packed;
+  if (next_nw) {
+    if (out_dtype != 1 || !sk_next_ok(next_res, next_nw, next_res_out, next_op, ssq_out)) return TS_BAD_SHAPE;
+    a.next_res = (const bf16_t*)next_res; a.next_nw = (const bf16_t*)next_nw; a.next_res_out = (bf16_t*)next_res_out;
+    a.next_op = (bf16_t*)next_op; a.ssq_out = (float*)ssq_out;
+    return sk8_dispatch<bf16_t, true>(a, stream);
+  }
+  if (!y || ldy < N) return TS_BAD_SHAPE;
   if (out_dtype == 1) return sk8_dispatch<bf16_t>(a, stream);
   if (out_dtype == 0) return sk8_dispatch<float>(a, stream);
   return TS_BAD_DTYPE;
 }
 
-// mode: 0 plain, 1 residual + RMSNorm on the way in (M <= 16, K in steps of 256 up to 2048). glu: W holds
-// gate rows then up rows, y is [M, N / 2] = silu(gate) * up (M <= 16, K up to 4096, 2048 with the norm). out_dtype: 1 bfloat16, 0 float
-// (plain only). packed: w holds the matrix in the kernel's own order (see the loads of W), ldw is unused. Requires M <= 32 (the gate
-// alone: M <= 64 for K up to 2048), K a multiple of 256 (up to 4096) or of 512 (up to 8192), contiguous
-// 16-byte aligned rows; mode 1 takes x, res, res_out as dense [M, K].
+// mode: 0 plain, 1 residual + RMSNorm on the way in (M <= 16, K in steps of 256 up to 2048), 2 the norm
+// prepared by the kernel before (x is the operand as it stands; ssq_in [M, ssq_parts] the parts of the rows'
+// sums of squares; eps). glu: W holds gate rows then up rows, y is [M, N / 2] = silu(gate) * up (M <= 16,
+// K up to 4096, 2048 with the norm; without the norm of mode 1 M <= 64 for K up to 2048). out_dtype: 1 bfloat16,
+// 0 float (plain only). packed: w holds the matrix in the kernel's own order (see the loads of W), ldw is
+// unused. Requires M <= 32 (M <= 64 for K up to 2048 in 8 waves), K a multiple of 256 (up to 4096) or of 512
+// (up to 8192), contiguous 16-byte aligned rows; mode 1 takes x, res, res_out as dense [M, K].
+// With next_nw (EPI_NEXT; modes 0 and 2 without glu, bfloat16) y is not written: next_res_out, next_op
+// [M, N] and ssq_out [M, tiles] are, tiles being the 16-column tiles the grid covers (ts_skinny_tiles).
 extern "C" int ts_gemm_skinny_bf16(void* y, const void* x, const void* w, const void* res, const void* nw,
                                    void* res_out, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldy,
-                                   float eps, int mode, int glu, int out_dtype, int packed, hipStream_t stream) {
+                                   float eps, int mode, int glu, int out_dtype, int packed, const void* ssq_in,
+                                   int ssq_parts, const void* next_res, const void* next_nw, void* next_res_out,
+                                   void* next_op, void* ssq_out, hipStream_t stream) {
   if (M <= 0 || N <= 0) return TS_OK;
-  if (M > (glu && mode == MODE_PLAIN ? 64 : 32) || K <= 0 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ldy < (glu ? N / 2 : N)) return TS_BAD_SHAPE;
+  const bool wide = mode != MODE_NORM && K <= 2048 && K % 256 == 0;        // 33 to 64 rows: see sk_dispatch
+  if (M > (wide ? 64 : 32) || K <= 0 || ldx % 8 || ldw % 8 || ldx < K || ldw < K) return TS_BAD_SHAPE;
   if (glu && (N % 2 || (N / 2) % 16)) return TS_BAD_SHAPE;
   if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)res | (uintptr_t)nw | (uintptr_t)res_out) & 15) return TS_BAD_SHAPE;
   if (mode == MODE_NORM && (!nw || (res && !res_out))) return TS_BAD_SHAPE;
+  if (mode == MODE_PREP && (!ssq_in || ssq_parts <= 0 || (((uintptr_t)ssq_in) & 3))) return TS_BAD_SHAPE;
   SkinnyArgs a = {};
   a.x = (const bf16_t*)x; a.res = (const bf16_t*)res; a.nw = (const bf16_t*)nw; a.res_out = (bf16_t*)res_out;
   a.w = (const bf16_t*)w; a.y = y; a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldw = ldw; a.ldy = ldy; a.eps = eps; a.packed = packed;
+  a.ssq_in = (const float*)ssq_in; a.ssq_parts = ssq_parts;
+  if (next_nw) {
+    if (glu || out_dtype != 1 || mode == MODE_NORM || !sk_next_ok(next_res, next_nw, next_res_out, next_op, ssq_out)) return TS_BAD_SHAPE;
+    a.next_res = (const bf16_t*)next_res; a.next_nw = (const bf16_t*)next_nw; a.next_res_out = (bf16_t*)next_res_out;
+    a.next_op = (bf16_t*)next_op; a.ssq_out = (float*)ssq_out;
+    if (mode == MODE_PLAIN) return sk_dispatch<MODE_PLAIN, EPI_NEXT, bf16_t>(a, stream);
+    return sk_dispatch<MODE_PREP, EPI_NEXT, bf16_t>(a, stream);
+  }
+  if (!y || ldy < (glu ? N / 2 : N)) return TS_BAD_SHAPE;
   if (out_dtype == 1) {
-    if (mode == MODE_PLAIN && !glu) return sk_dispatch<MODE_PLAIN, 0, bf16_t>(a, stream);
-    if (mode == MODE_PLAIN && glu) return sk_dispatch<MODE_PLAIN, 1, bf16_t>(a, stream);
-    if (mode == MODE_NORM && !glu) return sk_dispatch<MODE_NORM, 0, bf16_t>(a, stream);
-    if (mode == MODE_NORM && glu) return sk_dispatch<MODE_NORM, 1, bf16_t>(a, stream);
+    if (mode == MODE_PLAIN && !glu) return sk_dispatch<MODE_PLAIN, EPI_NONE, bf16_t>(a, stream);
+    if (mode == MODE_PLAIN && glu) return sk_dispatch<MODE_PLAIN, EPI_GLU, bf16_t>(a, stream);
+    if (mode == MODE_NORM && !glu) return sk_dispatch<MODE_NORM, EPI_NONE, bf16_t>(a, stream);
+    if (mode == MODE_NORM && glu) return sk_dispatch<MODE_NORM, EPI_GLU, bf16_t>(a, stream);
+    if (mode == MODE_PREP && !glu) return sk_dispatch<MODE_PREP, EPI_NONE, bf16_t>(a, stream);
+    if (mode == MODE_PREP && glu) return sk_dispatch<MODE_PREP, EPI_GLU, bf16_t>(a, stream);
     return TS_BAD_SHAPE;
   }
-  if (out_dtype == 0 && mode == MODE_PLAIN && !glu) return sk_dispatch<MODE_PLAIN, 0, float>(a, stream);
+  if (out_dtype == 0 && mode == MODE_PLAIN && !glu) return sk_dispatch<MODE_PLAIN, EPI_NONE, float>(a, stream);
   return TS_BAD_DTYPE;
+}
+
+// The 16-column tiles that ts_gemm_skinny_bf16's grid covers for a matrix of N rows over K with M rows of x: the
+// second dimension of ssq_out. (The workgroups own one, two or four tiles; the last may reach past N.)
+extern "C" int ts_skinny_tiles(int M, int N, int K) {
+  const int steps = (K % 256 == 0 && K / 256 <= 16) ? 8 : 16;
+  const int nwaves = K / (steps * SK_KSTEP), cb = (M + 15) / 16;
+  const int rt = (cb <= 2 && N >= 8192 && (nwaves <= 8 || cb == 1) && steps == 8) ? 2 : 1;
+  return (N + 16 * rt - 1) / (16 * rt) * rt;
 }
 
 // The qkv projection of an attention layer with the rotation and the cache write on the way out:
@@ -488,9 +705,10 @@ extern "C" int ts_gemm_skinny_rope_bf16(void* q_out, const void* x, const void* 
                                         int packed, const float* cos_sin, const int32_t* positions, const int32_t* slots,
                                         void* k_cache, void* v_cache, int nh, int nkv, int hd, int rotate,
                                         int page_size, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vs,
-                                        int64_t vh, int64_t vd, hipStream_t stream) {
+                                        int64_t vh, int64_t vd, const void* ssq_in, int ssq_parts, hipStream_t stream) {
   if (M <= 0) return TS_OK;
-  if (M > (mode == MODE_PLAIN && K <= 2048 ? 64 : 16) || K <= 0 || K % 256 || K / 256 > (mode == MODE_NORM ? 8 : 16) || ldx % 8 || ldw % 8 || ldx < K || ldw < K) return TS_BAD_SHAPE;
+  if (mode == MODE_PREP && (!ssq_in || ssq_parts <= 0 || (((uintptr_t)ssq_in) & 3))) return TS_BAD_SHAPE;
+  if (M > (mode != MODE_NORM && K <= 2048 ? 64 : 16) || K <= 0 || K % 256 || K / 256 > (mode == MODE_NORM ? 8 : 16) || ldx % 8 || ldw % 8 || ldx < K || ldw < K) return TS_BAD_SHAPE;
   if (nh <= 0 || nkv < 0 || hd <= 0 || hd % 32 || page_size <= 0) return TS_BAD_SHAPE;
   if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)res | (uintptr_t)nw | (uintptr_t)res_out | (uintptr_t)q_out) & 15)
     return TS_BAD_SHAPE;
@@ -504,6 +722,10 @@ extern "C" int ts_gemm_skinny_rope_bf16(void* q_out, const void* x, const void* 
   a.cos_sin = cos_sin; a.positions = positions; a.slots = slots; a.q_out = (bf16_t*)q_out;
   a.k_cache = (bf16_t*)k_cache; a.v_cache = (bf16_t*)v_cache; a.nh = nh; a.nkv = nkv; a.hd = hd; a.rotate = rotate;
   a.page_size = page_size; a.kp = kp; a.ks = ks; a.kh = kh; a.vp = vp; a.vs = vs; a.vh = vh; a.vd = vd;
+  a.ssq_in = (const float*)ssq_in; a.ssq_parts = ssq_parts;
+  if (mode == MODE_PREP && M > 32) return sk_launch<1, 4, 8, MODE_PREP, EPI_ROPE, bf16_t>(a, stream);
+  if (mode == MODE_PREP && M > 16) return sk_launch<1, 2, 8, MODE_PREP, EPI_ROPE, bf16_t>(a, stream);
+  if (mode == MODE_PREP) return sk_launch<1, 1, 8, MODE_PREP, EPI_ROPE, bf16_t>(a, stream);
   if (mode == MODE_PLAIN && M > 32) return sk_launch<1, 4, 8, MODE_PLAIN, EPI_ROPE, bf16_t>(a, stream);
   if (mode == MODE_PLAIN && M > 16) return sk_launch<1, 2, 8, MODE_PLAIN, EPI_ROPE, bf16_t>(a, stream);
   if (mode == MODE_PLAIN) return sk_launch<1, 1, 8, MODE_PLAIN, EPI_ROPE, bf16_t>(a, stream);

@@ -9,9 +9,11 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 #define SK_KSTEP 32      // k covered by one MFMA: lane group g holds k = 8 g .. 8 g + 7
 #define MODE_PLAIN 0
 #define MODE_NORM 1
+#define MODE_PREP 2
 #define EPI_NONE 0
 #define EPI_GLU 1
 #define EPI_ROPE 2
+#define EPI_NEXT 3
 
 // acc + A · B over 32 k: lane (r, g) gives k = 8 g .. 8 g + 7 of row r of A and of column r of B
 static __device__ __forceinline__ float4_t sk_mfma(const uint4& a, const uint4& b, float4_t acc) {

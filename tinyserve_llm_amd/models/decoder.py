@@ -11,7 +11,7 @@ import torch
 from tinyserve_llm_amd.models.spec import ModelSpec
 from tinyserve_llm_amd.parts import base
 from tinyserve_llm_amd.parts.base import KVSpec, LayerMemory, ParamSpec, PartSpec, StateSpec, StepContext
-from tinyserve_llm_amd.parts.block import Layer
+from tinyserve_llm_amd.parts.block import Layer, first_norm_of
 
 
 @dataclass(frozen=True)
@@ -147,9 +147,17 @@ class DecoderModel:
         for enc in self.position_encodings.values():
             hidden = enc.on_embedding(hidden, ctx)
         residual = None
-        for run, mem in zip(self.spec.order, memory):
+        order = self.spec.order
+        for i, (run, mem) in enumerate(zip(order, memory)):
             layer = self.layers[run.layer]
-            hidden, residual = base.BLOCKS[layer.block](layer, hidden, residual, ctx, mem)
+            block = base.BLOCKS[layer.block]
+            if getattr(block, "first_norm", None) is None:
+                hidden, residual = block(layer, hidden, residual, ctx, mem)
+                continue
+            # the norm the next run starts with, which this one's last projection may finish into
+            # (after the last run comes the final norm, which picks rows: it takes plain tensors)
+            following = first_norm_of(self.layers[order[i + 1].layer]) if i + 1 < len(order) else None
+            hidden, residual = block(layer, hidden, residual, ctx, mem, following=following)
         return hidden, residual
 
     def logits(self, hidden: torch.Tensor, residual: torch.Tensor | None, rows: torch.Tensor) -> torch.Tensor:

@@ -63,13 +63,14 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_gemm_library_timing": [i],
         "ts_gemm_library_choices": [p, i],
         "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, i, i, i, i, p, p, p],
-        "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p],
-        "ts_gemm_skinny8_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
-        "ts_gemm_rows64_bf16": [p, p, p, i, i, i, i64, i64, i, i, p],
+        "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p, i, p, p, p, p, p, p],
+        "ts_gemm_skinny8_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p, p, p, p, p, p],
+        "ts_gemm_rows64_bf16": [p, p, p, i, i, i, i64, i64, i, i, p, i, f, p],
+        "ts_skinny_tiles": [i, i, i],
         "ts_peak_read": [p, ctypes.c_size_t, p, i, p],
         "ts_peak_mfma": [p, i, i, p],
         "ts_gemm_skinny_rope_bf16": [p, p, p, p, p, p, i, i, i64, i64, f, i, i, p, p, p, p, p, i, i, i, i, i, i64, i64, i64,
-                                     i64, i64, i64, i64, p],
+                                     i64, i64, i64, i64, p, i, p],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -619,8 +620,47 @@ SKINNY_WIDE_ELEMENTS = 8 << 20   # largest matrix that `linear_bf16` gives the k
 
 
 def skinny_takes(rows: int, k: int) -> bool:
-    """Whether the weight-streaming kernel serves `rows` rows of x over a reduction of `k`."""
-    return rows <= SKINNY_MAX_ROWS and ((k % 256 == 0 and k // 256 <= 16) or (k % 512 == 0 and k // 512 <= 16))
+    """Whether the weight-streaming kernel serves `rows` rows of x over a reduction of `k` (33 to 64
+    rows: reductions of up to 2048 in steps of 256, which fit a workgroup of 8 waves)."""
+    if rows > SKINNY_MAX_ROWS:
+        return rows <= SKINNY_EPILOGUE_ROWS and k % 256 == 0 and k <= SKINNY_EPILOGUE_WIDE_K
+    return (k % 256 == 0 and k // 256 <= 16) or (k % 512 == 0 and k // 512 <= 16)
+
+
+class PreparedNorm:
+    """A residual sum and the first half of the norm that follows it, as the projection before them
+    leaves them (`next_norm=` of the weight-streaming kernels): `summed` = T(T(y) + residual), the new
+    residual [M, N]; `operand` = T((T(y) + residual) * weight), what the next projection multiplies;
+    `squares` [M, parts] float32, whose row sums are the rows' sums of squares of T(y) + residual. The
+    projection that takes `operand` multiplies its finished sums by rsqrt(sum(squares) / N + eps)
+    (`squares=`, `eps=` of the same kernels): together that is norm(y + residual) * weight."""
+
+    __slots__ = ("summed", "operand", "squares")
+
+    def __init__(self, summed: torch.Tensor, operand: torch.Tensor, squares: torch.Tensor) -> None:
+        self.summed, self.operand, self.squares = summed, operand, squares
+
+
+def _next_norm_outputs(x: torch.Tensor, n: int, parts: int, next_norm) -> tuple[PreparedNorm, torch.Tensor | None, torch.Tensor]:
+    """Checks `next_norm` = (residual or None, weight) for a product [M, n] and makes its outputs."""
+    residual, weight = next_norm
+    _gpu(residual, weight)
+    M = x.shape[0]
+    _need(weight.dtype == torch.bfloat16 and weight.shape == (n,) and weight.is_contiguous(), f"the next norm's weight must be bfloat16 [{n}]")
+    if residual is not None:
+        _need(residual.dtype == torch.bfloat16 and residual.shape == (M, n) and residual.is_contiguous(),
+              f"the residual must be bfloat16 [{M}, {n}]")
+    out = PreparedNorm(torch.empty((M, n), dtype=torch.bfloat16, device=x.device),
+                       torch.empty((M, n), dtype=torch.bfloat16, device=x.device),
+                       torch.empty((M, parts), dtype=torch.float32, device=x.device))
+    return out, residual, weight
+
+
+def _check_squares(squares: torch.Tensor | None, rows: int) -> None:
+    if squares is not None:
+        _gpu(squares)
+        _need(squares.dtype == torch.float32 and squares.dim() == 2 and squares.shape[0] == rows and squares.shape[1] >= 1
+              and squares.is_contiguous(), f"the sums of squares must be contiguous float32 [{rows}, parts]")
 
 
 def pack_weight(weight: torch.Tensor) -> torch.Tensor:
@@ -701,10 +741,12 @@ def pack_weight8(weight: torch.Tensor) -> torch.Tensor:
 
 
 def gemm_skinny8(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
-                 packed8: torch.Tensor | None = None) -> torch.Tensor:
+                 packed8: torch.Tensor | None = None, next_norm=None) -> "torch.Tensor | PreparedNorm":
     """bfloat16 x [M <= 8, K] · weight [N, K]^T by the weight-streaming kernel's 8-row form (a matrix
     instruction multiplies 8 rows of W by 8 rows of x over 64 k; a workgroup owns 8 rows of W).
-    With `packed8` (= pack_weight8(weight)) the kernel reads that copy."""
+    With `packed8` (= pack_weight8(weight)) the kernel reads that copy. With `next_norm` =
+    (residual or None, weight of the norm that follows) the product is not stored: a `PreparedNorm`
+    comes back."""
     _gpu(x, weight, packed8)
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "gemm_skinny8 takes bfloat16")
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
@@ -721,15 +763,24 @@ def gemm_skinny8(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype =
         _need(packed8.dtype == torch.bfloat16 and packed8.shape == (-(-N // 8), K // (64 * steps), steps, 64, 8)
               and packed8.is_contiguous() and packed8.data_ptr() % 16 == 0 and N % 8 == 0,
               f"the packed copy does not belong to a weight of {N} x {K}")
+    if next_norm is not None:
+        _need(out_dtype == torch.bfloat16, "a prepared norm comes with bfloat16")
+        prepared, residual, nw = _next_norm_outputs(x, N, -(-N // 8), next_norm)
+        _run("gemm_skinny8", library().ts_gemm_skinny8_bf16(
+            None, _ptr(x), _ptr(weight if packed8 is None else packed8), M, N, K, x.stride(0), weight.stride(0), N, 1,
+            int(packed8 is not None), _ptr(residual), _ptr(nw), _ptr(prepared.summed), _ptr(prepared.operand),
+            _ptr(prepared.squares), _stream()))
+        return prepared
     out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     _run("gemm_skinny8", library().ts_gemm_skinny8_bf16(
         _ptr(out), _ptr(x), _ptr(weight if packed8 is None else packed8), M, N, K, x.stride(0), weight.stride(0),
-        out.stride(0), _code(out_dtype), int(packed8 is not None), _stream()))
+        out.stride(0), _code(out_dtype), int(packed8 is not None), None, None, None, None, None, _stream()))
     return out
 
 
 def skinny_fuses(rows: int, k: int, norm: bool, glu: bool) -> bool:
-    """Whether the kernel can apply the norm on the way in and/or the gate on the way out."""
+    """Whether the kernel can apply the norm on the way in and/or the gate on the way out (a norm
+    that the kernel before has prepared counts as none: it is a scale on the way out)."""
     if not (norm or glu):
         return skinny_takes(rows, k)
     if k % 256:
@@ -741,11 +792,15 @@ def skinny_fuses(rows: int, k: int, norm: bool, glu: bool) -> bool:
 
 def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, *,
                 residual: torch.Tensor | None = None, norm_weight: torch.Tensor | None = None, eps: float = 0.0,
-                glu: bool = False, packed: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor | None]:
-    """bfloat16 e(f(x) [M <= 32, K] · weight [N, K]^T) by the weight-streaming MFMA kernel.
-    With `norm_weight`: f = RMSNorm(x + residual) * norm_weight, and x + residual comes back as the
-    second result. With `glu`: weight holds gate rows then up rows and the result is
-    silu(gate) * up, [M, N / 2]. With `packed` (= pack_weight(weight)) the kernel reads that copy."""
+                glu: bool = False, packed: torch.Tensor | None = None, squares: torch.Tensor | None = None,
+                next_norm=None) -> "tuple[torch.Tensor | PreparedNorm, torch.Tensor | None]":
+    """bfloat16 e(f(x) [M <= 32, K] · weight [N, K]^T) by the weight-streaming MFMA kernel (up to 64
+    rows over reductions of up to 2048). With `norm_weight`: f = RMSNorm(x + residual) * norm_weight,
+    and x + residual comes back as the second result. With `squares` (and `eps`): x is the operand of
+    a `PreparedNorm` and `squares` its sums of squares; the rows' scales multiply the finished sums.
+    With `glu`: weight holds gate rows then up rows and the result is silu(gate) * up, [M, N / 2].
+    With `packed` (= pack_weight(weight)) the kernel reads that copy. With `next_norm` = (residual or
+    None, weight of the norm that follows) the first result is a `PreparedNorm` instead of the product."""
     _gpu(x, weight, residual, norm_weight)
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "gemm_skinny takes bfloat16")
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
@@ -760,6 +815,18 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
           "rows must be contiguous and 16-byte aligned")
     _need(not glu or (N % 32 == 0), "gate and up rows come in whole 16-row tiles")
     _check_packed(packed, weight)
+    _check_squares(squares, M)
+    _need(squares is None or not norm, "a norm is either prepared by the kernel before or made here")
+    mode = 1 if norm else 2 if squares is not None else 0
+    if next_norm is not None:
+        _need(not glu and not norm and out_dtype == torch.bfloat16, "a prepared norm follows a plain bfloat16 product")
+        prepared, nres, nw = _next_norm_outputs(x, N, library().ts_skinny_tiles(M, N, K), next_norm)
+        _run("gemm_skinny", library().ts_gemm_skinny_bf16(
+            None, _ptr(x), _ptr(weight if packed is None else packed), None, None, None, M, N, K, x.stride(0),
+            weight.stride(0), N, float(eps), mode, 0, 1, int(packed is not None), _ptr(squares),
+            0 if squares is None else squares.shape[1], _ptr(nres), _ptr(nw), _ptr(prepared.summed), _ptr(prepared.operand),
+            _ptr(prepared.squares), _stream()))
+        return prepared, None
     res_out = None
     if norm:
         _need(norm_weight.dtype == torch.bfloat16 and norm_weight.shape == (K,) and norm_weight.is_contiguous(),
@@ -777,7 +844,8 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     _run("gemm_skinny", library().ts_gemm_skinny_bf16(
         _ptr(out), _ptr(x), _ptr(weight if packed is None else packed), _ptr(residual), _ptr(norm_weight),
         _ptr(res_out) if residual is not None else None, M, N, K, x.stride(0), weight.stride(0), out.stride(0),
-        float(eps), int(norm), int(glu), _code(out_dtype), int(packed is not None), _stream()))
+        float(eps), mode, int(glu), _code(out_dtype), int(packed is not None), _ptr(squares),
+        0 if squares is None else squares.shape[1], None, None, None, None, None, _stream()))
     return out, res_out
 
 
@@ -793,10 +861,11 @@ def rows64_takes(rows: int, n: int, k: int) -> bool:
 
 
 def gemm_rows64(x: torch.Tensor, packed: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, *,
-                glu: bool = False) -> torch.Tensor:
+                glu: bool = False, squares: torch.Tensor | None = None, eps: float = 0.0) -> torch.Tensor:
     """bfloat16 e(x [M <= 64, K] · W [N, K]^T) for a wide W given as `packed` = pack_weight(W), by the
     kernel that shares x among 64 rows of W through LDS (gemm_rows64.hip). With `glu`, W holds gate
-    rows then up rows and the result is silu(gate) * up, [M, N / 2]."""
+    rows then up rows and the result is silu(gate) * up, [M, N / 2]. With `squares` (and `eps`) x is
+    the operand of a `PreparedNorm` and the rows' scales multiply the finished sums."""
     _gpu(x, packed)
     _need(x.dtype == torch.bfloat16 and packed.dtype == torch.bfloat16 and x.dim() == 2 and packed.dim() == 4
           and packed.shape[2:] == (64, 8) and packed.is_contiguous(), "gemm_rows64 takes bfloat16 x [M, K] and pack_weight(W)")
@@ -808,9 +877,11 @@ def gemm_rows64(x: torch.Tensor, packed: torch.Tensor, out_dtype: torch.dtype = 
           f"not {M} x {K} against {N}")
     _need(x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0, "rows of x must be dense and 16-byte aligned")
     _need(out_dtype == torch.bfloat16 or (out_dtype == torch.float32 and not glu), "32-bit output comes without the gate")
+    _check_squares(squares, M)
     out = torch.empty((M, N // 2 if glu else N), dtype=out_dtype, device=x.device)
     _run("gemm_rows64", library().ts_gemm_rows64_bf16(
-        _ptr(out), _ptr(x), _ptr(packed), M, N, K, x.stride(0), out.stride(0), int(glu), int(out_dtype == torch.float32), _stream()))
+        _ptr(out), _ptr(x), _ptr(packed), M, N, K, x.stride(0), out.stride(0), int(glu), int(out_dtype == torch.float32),
+        _ptr(squares), 0 if squares is None else squares.shape[1], float(eps), _stream()))
     return out
 
 
@@ -839,13 +910,17 @@ def qkv_rope_fuses(x: torch.Tensor, weight: torch.Tensor, head_dim: int, k_cache
 def qkv_rope_store(x: torch.Tensor, weight: torch.Tensor, cos_sin: torch.Tensor | None, positions: torch.Tensor,
                    slots: torch.Tensor | None, k_cache: torch.Tensor | None, v_cache: torch.Tensor | None,
                    num_heads: int, num_kv_heads: int, head_dim: int, *, residual: torch.Tensor | None = None,
-                   norm_weight: torch.Tensor | None = None, eps: float = 0.0, packed: torch.Tensor | None = None
-                   ) -> tuple[torch.Tensor, torch.Tensor | None]:
+                   norm_weight: torch.Tensor | None = None, eps: float = 0.0, packed: torch.Tensor | None = None,
+                   squares: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor | None]:
     """`rope_store(f(x) · weight^T, ...)` in one kernel for few rows of x: the projection is never
     stored, q [tokens, nh, hd] comes back rotated, rotated k and v go to their cache slots. With
     `norm_weight`, f = RMSNorm(x + residual) * norm_weight and x + residual is the second result.
-    With `packed` (= pack_weight_rope(weight, head_dim)) the kernel reads that copy."""
+    With `squares` (and `eps`) x is the operand of a `PreparedNorm` instead, and the rows' scales
+    multiply the finished sums. With `packed` (= pack_weight_rope(weight, head_dim)) the kernel reads
+    that copy."""
     _gpu(x, weight, cos_sin, positions, slots, k_cache, v_cache, residual, norm_weight)
+    _check_squares(squares, x.shape[0])
+    _need(squares is None or norm_weight is None, "a norm is either prepared by the kernel before or made here")
     _need(qkv_rope_fuses(x, weight, head_dim, k_cache, norm_weight is not None),
           "qkv_rope_store takes up to 16 bfloat16 rows (64 over up to 2048 without the norm), K in steps of 256 up to 4096 "
           "(2048 with the norm), head_dim in steps of 32")
@@ -880,9 +955,10 @@ def qkv_rope_store(x: torch.Tensor, weight: torch.Tensor, cos_sin: torch.Tensor 
     q = torch.empty((M, num_heads, head_dim), dtype=x.dtype, device=x.device)
     _run("qkv_rope_store", library().ts_gemm_skinny_rope_bf16(
         _ptr(q), _ptr(x), _ptr(weight if packed is None else packed), _ptr(residual), _ptr(norm_weight),
-        _ptr(res_out) if residual is not None else None, M, K, x.stride(0), weight.stride(0), float(eps), int(norm),
+        _ptr(res_out) if residual is not None else None, M, K, x.stride(0), weight.stride(0), float(eps),
+        1 if norm else 2 if squares is not None else 0,
         int(packed is not None), _ptr(cos_sin), _ptr(positions), _ptr(slots), _ptr(k_cache), _ptr(v_cache), num_heads, num_kv_heads, head_dim,
-        int(cos_sin is not None), page_size, *kst, *vst, _stream()))
+        int(cos_sin is not None), page_size, *kst, *vst, _ptr(squares), 0 if squares is None else squares.shape[1], _stream()))
     return q, res_out
 
 
@@ -942,24 +1018,39 @@ class StreamingCopies:
         return sum(t.numel() * t.element_size() for t in (self.by16, self.by8) if t is not None)
 
 
+def next_norm_fuses(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether `linear_bf16(x, weight, next_norm=...)` has a kernel that leaves a `PreparedNorm`."""
+    if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.is_cuda and x.dim() == 2 and weight.dim() == 2
+            and x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
+        return False
+    rows, (n, k) = x.shape[0], weight.shape
+    return skinny8_takes(rows, n, k) or _skinny_serves(rows, n, k)
+
+
+def _skinny_serves(rows: int, n: int, k: int) -> bool:
+    """Whether `linear_bf16` gives a plain product to the 16-row weight-streaming kernel. Measured:
+    reductions longer than 4096 leave it too few workgroups, and with more than 16 rows it only wins
+    on small matrices (8M elements: a layer's qkv and o, not its gate_up or the head); the library
+    streams the rest faster."""
+    return (rows <= SKINNY_MAX_ROWS and skinny_takes(rows, k) and k <= 4096
+            and (rows <= SKINNY_FUSED_ROWS or n * k <= SKINNY_WIDE_ELEMENTS))
+
+
 def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
-                packed: StreamingCopies | None = None) -> torch.Tensor:
+                packed: StreamingCopies | None = None, next_norm=None) -> "torch.Tensor | PreparedNorm":
     """bfloat16 x [M, K] · weight [N, K]^T: few rows go to the weight-streaming kernels (which read
     the weight's copy in their own order from `packed`, if there is one), many to the vendor matrix
-    library."""
+    library. With `next_norm` (where `next_norm_fuses` says so) a `PreparedNorm` comes back."""
     _gpu(x, weight)
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "linear_bf16 takes bfloat16")
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
           f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
     streams = x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0
     if streams and skinny8_takes(x.shape[0], weight.shape[0], x.shape[1]):
-        return gemm_skinny8(x, weight, out_dtype, None if packed is None else packed.by8)
-    # Measured: reductions longer than 4096 leave the 16-row kernel too few workgroups, and with more than
-    # 16 rows it only wins on small matrices (8M elements: a layer's qkv and o, not its gate_up or the
-    # head); the library streams the rest faster.
-    if (streams and skinny_takes(x.shape[0], x.shape[1]) and x.shape[1] <= 4096
-            and (x.shape[0] <= SKINNY_FUSED_ROWS or weight.numel() <= SKINNY_WIDE_ELEMENTS)):
-        return gemm_skinny(x, weight, out_dtype, packed=None if packed is None else packed.by16)[0]
+        return gemm_skinny8(x, weight, out_dtype, None if packed is None else packed.by8, next_norm=next_norm)
+    if streams and _skinny_serves(x.shape[0], weight.shape[0], x.shape[1]):
+        return gemm_skinny(x, weight, out_dtype, packed=None if packed is None else packed.by16, next_norm=next_norm)[0]
+    _need(next_norm is None, "no kernel leaves a prepared norm for this product (ask next_norm_fuses first)")
     # (float32: the 32-bit sums themselves, as the weight-streaming kernel gives them for few rows, so
     # that a row's logits are rounded the same way whatever the number of rows beside it)
     _need(out_dtype in (torch.bfloat16, torch.float32), f"bfloat16 products come out as bfloat16 or float32, not {out_dtype}")

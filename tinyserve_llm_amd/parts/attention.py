@@ -22,6 +22,7 @@ from tinyserve_llm_amd.parts.linear import DeferredNorm, linear, streaming_copy
 class Attention(Mixer):
     graph_safe = True
     takes_deferred_norm = True
+    finishes_into_norm = True
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position: str | None = "rope", scale: float | None = None, window: int = 0) -> None:
@@ -63,8 +64,14 @@ class Attention(Mixer):
         """Projection, rotation and cache write in one kernel where a step is small enough for the
         weight-streaming kernel; None where it is not."""
         d = x if isinstance(x, DeferredNorm) else None
-        rows = d.x if d is not None else x
         by16 = self.qkv_rope_packed
+        if d is not None and d.prepared is not None:     # the norm's first half is done: its operand, then a scale per row
+            rows = d.prepared.operand
+            if not hip.qkv_rope_fuses(rows, self.qkv, self.head_dim, k_store):
+                return None
+            return hip.qkv_rope_store(rows, self.qkv, table, positions, slots, k_store, v_store, self.num_heads,
+                                      self.num_kv_heads, self.head_dim, eps=d.eps, packed=by16, squares=d.prepared.squares)[0]
+        rows = d.x if d is not None else x
         if not (rows.is_cuda and hip.qkv_rope_fuses(rows, self.qkv, self.head_dim, k_store)):
             return None
         if d is not None and not (hip.qkv_rope_fuses(rows, self.qkv, self.head_dim, k_store, norm=True)
@@ -86,7 +93,7 @@ class Attention(Mixer):
     def kv_spec(self) -> KVSpec:
         return KVSpec(self.num_kv_heads, self.head_dim, self.window)
 
-    def forward(self, x: torch.Tensor, ctx: StepContext, mem: LayerMemory) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, ctx: StepContext, mem: LayerMemory, then=None) -> torch.Tensor:
         table = ctx.position_encodings[self.position].rotary_table() if self.position else None
         slots = ctx.slot_mapping[mem.space] if mem.store else None
         k_store, v_store = (mem.k_cache, mem.v_cache) if mem.store else (None, None)
@@ -96,4 +103,4 @@ class Attention(Mixer):
             q = hip.rope_store(qkv, table, ctx.positions, slots, k_store, v_store, self.num_heads, self.num_kv_heads,
                                self.head_dim)
         o = hip.paged_attention(q, mem.k_cache, mem.v_cache, ctx, mem.space, self.scale, self.window)
-        return linear(o.view(ctx.num_tokens, self.q_size), self.o, packed=self.o_packed)
+        return linear(o.view(ctx.num_tokens, self.q_size), self.o, packed=self.o_packed, then=then)

@@ -133,6 +133,18 @@ class Norm(Part):
         then holds `residual_out`. None (the default): this norm is always computed by itself."""
         return None
 
+    def request(self, residual=None):
+        """Optionally the norm as a request to the part before it, if that part declares
+        `finishes_into_norm`: the part hands the request to its last projection (`then=`) and returns
+        what comes back, this norm deferred with its first half done. `residual` is the stream the
+        part's output is added to (a tensor, None, or a deferred norm that will hold it). None (the
+        default): this norm takes plain tensors only."""
+        return None
+
+    def made_for(self, pending) -> bool:
+        """Whether `pending` is this very norm in deferred form."""
+        return False
+
 
 class PositionEncoding(Part):
     def prepare(self, device: torch.device) -> None:
@@ -151,6 +163,9 @@ class Mixer(Part):
     # True if forward() passes x to exactly one `linear()` call and uses it nowhere else, so that a
     # norm may hand it over deferred (see Norm.defer)
     takes_deferred_norm = False
+    # True if forward() takes `then=` (a request of the norm that follows: Norm.request), hands it to
+    # the `linear()` call that makes its result, and returns what that call returns
+    finishes_into_norm = False
 
     def kv_spec(self) -> KVSpec | None:
         return None
@@ -164,6 +179,7 @@ class Mixer(Part):
 
 class FeedForward(Part):
     takes_deferred_norm = False    # as for Mixer
+    finishes_into_norm = False     # as for Mixer
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         raise NotImplementedError

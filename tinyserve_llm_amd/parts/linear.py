@@ -8,7 +8,10 @@ many, as the reference uses a vendor library for every projection (or, if
 With few rows a step's time goes to launching kernels and to waiting for memory, so what
 precedes or follows a projection can ride along with it: a norm may hand its input over as a
 `DeferredNorm` and the projection applies residual add and normalisation while it reads x; a
-gated feed-forward may ask for silu(gate) * up straight out of the gate|up projection. Where the
+gated feed-forward may ask for silu(gate) * up straight out of the gate|up projection; and a
+projection whose result goes into a residual sum and a norm may be asked to finish into them
+(`then=`, a `NormRequest`): it then leaves the sum, the next projection's operand and the rows'
+sums of squares, and what comes back is again a `DeferredNorm`, half done already. Where the
 fused kernel does not serve the shape, the same calls run the separate kernels.
 """
 
@@ -21,15 +24,38 @@ from tinyserve_llm_amd.ops import hip
 
 class DeferredNorm:
     """norm(x + residual) * weight, not yet computed: the first projection that takes it either
-    fuses it or materialises it. Either way `residual_out` then holds x + residual."""
+    fuses it or materialises it. Either way `residual_out` then holds x + residual. With `prepared`
+    (what the projection that made x has left: `hip.PreparedNorm`) the sum is there already and
+    `x`, `residual` are not given."""
 
-    def __init__(self, x: torch.Tensor, residual: torch.Tensor | None, weight: torch.Tensor, eps: float) -> None:
-        self.x, self.residual, self.weight, self.eps = x, residual, weight, eps
-        self.residual_out: torch.Tensor | None = None
+    def __init__(self, x: torch.Tensor | None, residual: torch.Tensor | None, weight: torch.Tensor, eps: float,
+                 prepared: hip.PreparedNorm | None = None) -> None:
+        self.x, self.residual, self.weight, self.eps, self.prepared = x, residual, weight, eps, prepared
+        self.residual_out: torch.Tensor | None = None if prepared is None else prepared.summed
+
+    @property
+    def rows(self) -> int:
+        return (self.x if self.prepared is None else self.prepared.operand).shape[0]
 
     def materialize(self) -> torch.Tensor:
+        if self.prepared is not None:
+            return hip.rmsnorm(self.prepared.summed, self.weight, self.eps, want_residual=False)[0]
         out, self.residual_out = hip.rmsnorm(self.x, self.weight, self.eps, self.residual)
         return out
+
+
+class NormRequest:
+    """Asks a projection to finish into the residual sum and the norm that follow it: `weight` and
+    `eps` are that norm's, `residual` the stream its input is added to: a tensor, None, or a
+    `DeferredNorm` whose `residual_out` is the stream once its projection has run (the norm before
+    the part that holds this projection, fused into that part's first projection)."""
+
+    def __init__(self, weight: torch.Tensor, eps: float, residual: "torch.Tensor | DeferredNorm | None") -> None:
+        self.weight, self.eps, self._residual = weight, eps, residual
+
+    def residual(self) -> torch.Tensor | None:
+        r = self._residual
+        return r.residual_out if isinstance(r, DeferredNorm) else r
 
 
 def _streams(x: torch.Tensor, weight: torch.Tensor) -> bool:
@@ -50,10 +76,34 @@ def streaming_copy(weight: torch.Tensor) -> hip.StreamingCopies | None:
 
 
 def linear(x: torch.Tensor | DeferredNorm, weight: torch.Tensor, out_dtype: torch.dtype | None = None,
-           glu: bool = False, packed: hip.StreamingCopies | None = None) -> torch.Tensor:
+           glu: bool = False, packed: hip.StreamingCopies | None = None,
+           then: NormRequest | None = None) -> "torch.Tensor | DeferredNorm":
     """x · Wᵀ; with `glu`, W holds gate rows then up rows and silu(gate) * up comes back.
-    `packed` is `streaming_copy(weight)` if the part keeps one."""
+    `packed` is `streaming_copy(weight)` if the part keeps one. With `then` the result is the
+    `DeferredNorm` of that request: norm(x · Wᵀ + residual) * weight, prepared by this projection's
+    kernel where it can be, left to the next projection otherwise."""
+    if then is not None:
+        if glu:
+            raise ValueError("a gated projection does not finish into a norm")
+        residual = then.residual()
+        if isinstance(x, DeferredNorm):
+            x = x.materialize()
+        if (out_dtype in (None, torch.bfloat16) and then.weight.dtype == torch.bfloat16 and hip.next_norm_fuses(x, weight)
+                and (residual is None or (residual.is_contiguous() and residual.dtype == torch.bfloat16))):
+            prepared = hip.linear_bf16(x, weight, torch.bfloat16, packed, next_norm=(residual, then.weight))
+            return DeferredNorm(None, None, then.weight, then.eps, prepared)
+        return DeferredNorm(linear(x, weight, out_dtype, packed=packed), residual, then.weight, then.eps)
     by16 = None if packed is None else packed.by16
+    if isinstance(x, DeferredNorm) and x.prepared is not None:
+        d, op = x, x.prepared.operand
+        if out_dtype in (None, torch.bfloat16) and _streams(op, weight) and not (glu and weight.shape[0] % 32):
+            rows, (n, k) = op.shape[0], weight.shape
+            wide = by16 is not None and hip.rows64_takes(rows, n, k) and n % (128 if glu else 64) == 0
+            if wide:
+                return hip.gemm_rows64(op, by16, glu=glu, squares=d.prepared.squares, eps=d.eps)
+            if (hip.skinny_fuses(rows, k, False, True) if glu else hip._skinny_serves(rows, n, k)):
+                return hip.gemm_skinny(op, weight, glu=glu, packed=by16, squares=d.prepared.squares, eps=d.eps)[0]
+        x = d.materialize()
     if isinstance(x, DeferredNorm):
         d = x
         if (out_dtype in (None, torch.bfloat16) and _streams(d.x, weight) and d.weight.dtype == torch.bfloat16

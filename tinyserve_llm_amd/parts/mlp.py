@@ -13,6 +13,7 @@ from tinyserve_llm_amd.parts.linear import linear, streaming_copy
 class GatedMLP(FeedForward):
     graph_safe = True
     takes_deferred_norm = True
+    finishes_into_norm = True
 
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu") -> None:
         if activation != "silu":
@@ -32,5 +33,6 @@ class GatedMLP(FeedForward):
         self.gate_up_packed, self.down_packed = streaming_copy(self.gate_up), streaming_copy(self.down)
         return sum(c.nbytes() for c in (self.gate_up_packed, self.down_packed) if c is not None)
 
-    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
-        return linear(linear(x, self.gate_up, glu=True, packed=self.gate_up_packed), self.down, packed=self.down_packed)
+    def forward(self, x: torch.Tensor, ctx: StepContext, then=None) -> torch.Tensor:
+        return linear(linear(x, self.gate_up, glu=True, packed=self.gate_up_packed), self.down, packed=self.down_packed,
+                      then=then)

@@ -11,7 +11,7 @@ import torch
 
 from tinyserve_llm_amd.ops import hip
 from tinyserve_llm_amd.parts.base import Norm, ParamSpec, register
-from tinyserve_llm_amd.parts.linear import DeferredNorm
+from tinyserve_llm_amd.parts.linear import DeferredNorm, NormRequest
 
 
 @register("norm", "rmsnorm")
@@ -32,3 +32,11 @@ class RMSNorm(Norm):
     def defer(self, x, residual=None) -> DeferredNorm:
         """The same norm as an operand that the next projection may fuse."""
         return DeferredNorm(x, residual, self.weight, self.eps)
+
+    def request(self, residual=None) -> NormRequest:
+        """The same norm as a request to the projection before it (`linear(..., then=)`)."""
+        return NormRequest(self.weight, self.eps, residual)
+
+    def made_for(self, pending) -> bool:
+        """Whether `pending` is this norm, deferred (by `defer` or through `request`)."""
+        return isinstance(pending, DeferredNorm) and pending.weight is self.weight and pending.eps == self.eps
