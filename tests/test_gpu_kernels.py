@@ -121,6 +121,45 @@ def test_rope_and_cache_write_on_a_strided_layer_view(dtype):
     assert torch.equal(k_pool[3, 2, 0].cpu(), qkv[0, nh * hd:(nh + nkv) * hd].view(nkv, hd))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hd,rot,T", [(48, 16, 8), (64, 32, 40), (40, 6, 3), (128, 64, 17)])
+def test_rotation_of_the_leading_part_of_a_head(dtype, hd, rot, T):
+    """A table narrower than the head turns the first `rot` dimensions (j with j + rot / 2) and lets
+    the rest pass, in q and in the keys that are written; the sixteen-byte path and the one element
+    at a time (widths of 6 and 34 have no whole pieces)."""
+    nh, nkv, page = 3, 1, 8
+    g = gen(hd + rot)
+    qkv = torch.randn(T, (nh + 2 * nkv) * hd, generator=g).to(dtype)
+    positions = torch.randint(0, 64, (T,), generator=g, dtype=torch.int32)
+    slots = torch.randperm(48, generator=g)[:T].to(torch.int32)
+    cos, sin = P.rope_tables(rot, 10000.0, None, 64, 64, torch.float64)
+    table = torch.cat((cos, sin), -1).float()
+    k_pool = torch.zeros(6, page, nkv, hd, dtype=dtype, device=dev())
+    v_pool = torch.zeros_like(k_pool)
+    q = hip().rope_store(qkv.to(dev()), table.to(dev()), positions.to(dev()), slots.to(dev()), k_pool, v_pool, nh, nkv, hd)
+    x = qkv.double()
+    qs, ks = x[:, :nh * hd].view(T, nh, hd), x[:, nh * hd:(nh + nkv) * hd].view(T, nkv, hd)
+    pos = positions.long()
+
+    def turned(t):
+        return torch.cat((P.apply_rope(t[..., :rot], cos[pos], sin[pos]), t[..., rot:]), -1)
+
+    torch.testing.assert_close(q.double().cpu(), turned(qs), **tol(dtype))
+    assert torch.equal(q[..., rot:].cpu(), qkv[:, :nh * hd].view(T, nh, hd)[..., rot:]), "what does not turn passes bit for bit"
+    kr = turned(ks)
+    for t in range(T):
+        b, o = int(slots[t]) // page, int(slots[t]) % page
+        torch.testing.assert_close(k_pool[b, o].double().cpu(), kr[t], **tol(dtype))
+        assert torch.equal(v_pool[b, o].cpu(), qkv[t, (nh + nkv) * hd:].view(nkv, hd))
+    with pytest.raises(hip().KernelError, match="rotation table"):
+        hip().rope_store(qkv.to(dev()), torch.zeros(64, hd + 2, device=dev()), positions.to(dev()), None, None, None, nh, nkv, hd)
+    w = torch.zeros((nh + 2 * nkv) * hd, 256, dtype=torch.bfloat16, device=dev())
+    xs = torch.zeros(4, 256, dtype=torch.bfloat16, device=dev())
+    if hd % 32 == 0:
+        assert hip().qkv_rope_fuses(xs, w, hd, None) and not hip().qkv_rope_fuses(xs, w, hd, None, table=table.to(dev())), \
+            "the one-kernel path turns whole heads only: a part leaves this table to the separate kernels"
+
+
 def scattered(k, v, table, page, pages, dtype, layers=2, layer=1):
     """A pool full of junk with k/v of positions 0.. written to the pages `table` names."""
     g = gen(9)
@@ -259,12 +298,21 @@ def test_split_key_decode_attention(heads, kv, hd, page, chunk, waves):
 @pytest.mark.parametrize("heads,kv,hd,page", [(3, 1, 32, 16), (6, 2, 96, 8), (32, 8, 64, 256), (5, 5, 128, 32),
                                               (16, 1, 128, 64), (14, 2, 64, 24), (12, 6, 32, 16), (32, 16, 64, 64),
                                               (8, 4, 96, 32), (24, 12, 32, 8)])
-@pytest.mark.parametrize("row_tiles", [1, 2, 4])
-def test_matrix_core_prefill_attention(heads, kv, hd, page, row_tiles):
+@pytest.mark.parametrize("row_tiles,waves", [(1, 4), (2, 4), (4, 4), (1, 8), (2, 8)])
+def test_matrix_core_prefill_attention(heads, kv, hd, page, row_tiles, waves):
     """A packed step of three requests on shared pools: a whole prompt, a portion over a cached
     prefix, and single decoded tokens; tiles never cross a request. Once for each number of row
-    tiles that a wave of the kernel may hold."""
+    tiles that a wave of the kernel may hold, in workgroups of four and of eight waves."""
     dtype = torch.bfloat16
+    if waves == 8 and hd not in (64, 128):
+        q0 = torch.zeros(4, heads, hd, dtype=dtype, device=dev())
+        kc0 = torch.zeros(1, kv, page, hd, dtype=dtype, device=dev()).permute(0, 2, 1, 3)
+        vc0 = torch.zeros(1, kv, hd, page, dtype=dtype, device=dev()).permute(0, 3, 1, 2)
+        z = torch.zeros(4, dtype=torch.int32, device=dev())
+        with pytest.raises(hip().KernelError, match="waves"):
+            hip().paged_attention_prefill(q0, kc0, vc0, z[:1].view(1, 1), z, z, torch.tensor([[0, 4]], dtype=torch.int32, device=dev()),
+                                          1.0, waves=8)
+        return
     g = gen(hd * 3 + page)
     lens = [150, 77, 300]                       # keys each request has after the step
     fed = [150, 9, 1]                           # tokens of each in the step
@@ -291,21 +339,21 @@ def test_matrix_core_prefill_attention(heads, kv, hd, page, row_tiles):
     seq_of = sum(([i] * fed[i] for i in range(3)), [])
     positions = sum((list(range(lens[i] - fed[i], lens[i])) for i in range(3)), [])
     cu = [0, fed[0], fed[0] + fed[1], sum(fed)]
-    per_tile = row_tiles * hip().PREFILL_WAVES * (16 // (heads // kv))
+    per_tile = row_tiles * waves * (16 // (heads // kv))
     flat = hip().attention_tiles(cu, [lens[i] - fed[i] for i in range(3)], per_tile)
     assert all(flat[2 * i + 1] <= per_tile for i in range(len(flat) // 2))
     assert sum(flat[1::2]) == sum(fed) and len(flat) // 2 == sum(-(-f // per_tile) for f in fed)
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev())
     kc, vc = kp.to(dev()).permute(0, 2, 1, 3), vp.to(dev()).permute(0, 3, 1, 2)
     out = hip().paged_attention_prefill(q_step.to(dev()), kc, vc, i32(padded), i32(seq_of), i32(positions),
-                                        i32(flat).view(-1, 2), hd ** -0.5, tile_tokens=per_tile)
+                                        i32(flat).view(-1, 2), hd ** -0.5, tile_tokens=per_tile, waves=waves)
     want = torch.cat([P.causal_attention(q_all[i].double(), k_all[i].double(), v_all[i].double())[lens[i] - fed[i]:]
                       for i in range(3)])
     torch.testing.assert_close(out.double().cpu(), want, **tol(dtype))
     wave = run_attention(q_step, kc, vc, padded, seq_of, positions, hd ** -0.5)
     torch.testing.assert_close(out.float(), wave.float(), **tol(dtype))
     win = hip().paged_attention_prefill(q_step.to(dev()), kc, vc, i32(padded), i32(seq_of), i32(positions),
-                                        i32(flat).view(-1, 2), hd ** -0.5, window=40, tile_tokens=per_tile)
+                                        i32(flat).view(-1, 2), hd ** -0.5, window=40, tile_tokens=per_tile, waves=waves)
     want = torch.cat([P.causal_attention(q_all[i].double(), k_all[i].double(), v_all[i].double(), window=40)[lens[i] - fed[i]:]
                       for i in range(3)])
     torch.testing.assert_close(win.double().cpu(), want, **tol(dtype))

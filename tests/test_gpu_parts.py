@@ -119,6 +119,35 @@ def test_gated_mlp_part(dtype):
         GatedMLP(8, 8, activation="gelu")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_part_with_a_rotation_of_part_of_the_head(dtype):
+    """The attention part with a position encoding that turns 32 of a head's 64 dimensions: a step
+    of a few tokens, which would take the one-kernel projection if heads turned whole, and a longer
+    one, both against the plain formulas with the rotation applied to the leading part."""
+    from tinyserve_llm_amd.parts.attention import Attention
+    from tinyserve_llm_amd.parts.rope import Rope
+    hidden, nh, nkv, hd, rot, page = 256, 4, 2, 64, 32, 16
+    part = Attention(hidden_size=hidden, num_heads=nh, num_kv_heads=nkv, head_dim=hd, position="rope")
+    w = bound(part, dtype, 3)
+    rope = Rope(head_dim=hd, max_position=128, theta=10000.0, rotary_dim=rot)
+    rope.prepare(torch.device(DEV))
+    assert rope.rotary_table().shape == (128, rot)
+    from tinyserve_llm_amd.parts.base import LayerMemory
+    for n in (5, 70):
+        x = (torch.randn(n, hidden, generator=torch.Generator().manual_seed(n)) * 0.5).to(dtype)
+        pages = -(-n // page)
+        kc = torch.zeros(pages, nkv, page, hd, dtype=dtype, device=DEV).permute(0, 2, 1, 3)
+        vc = torch.zeros(pages, nkv, hd, page, dtype=dtype, device=DEV).permute(0, 3, 1, 2)
+        ctx = context([n], [0], page, [list(range(pages))], {"rope": rope})
+        out = part.forward(x.to(DEV), ctx, LayerMemory(k_cache=kc, v_cache=vc))
+        cos, sin = P.rope_tables(rot, 10000.0, None, 128, n, torch.float64)
+        qkv = x.double() @ w["qkv"].T
+        q, k, v = qkv[:, :nh * hd].view(n, nh, hd), qkv[:, nh * hd:(nh + nkv) * hd].view(n, nkv, hd), qkv[:, (nh + nkv) * hd:].view(n, nkv, hd)
+        turn = lambda t: torch.cat((P.apply_rope(t[..., :rot], cos, sin), t[..., rot:]), -1)
+        want = P.causal_attention(turn(q), turn(k), v).reshape(n, nh * hd) @ w["o"].T
+        torch.testing.assert_close(out.double().cpu(), want, **tol(dtype))
+
+
 # ---- parts from outside the framework --------------------------------------------------------------
 
 def register_toy_parts():

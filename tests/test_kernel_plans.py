@@ -40,6 +40,11 @@ def test_prefill_tile_tokens_keeps_the_chip_busy():
     assert hip.prefill_tile_tokens(4096, 8, 4, 64, mean_keys=4096) == 64      # four: small heads, a long walk
     assert hip.prefill_tile_tokens(16384, 8, 4, 128, mean_keys=8192) == 32    # large heads stop at two
     assert hip.prefill_tile_tokens(10, 1, 16, 32) == 4
+    # eight waves a workgroup where four would hold two row tiles each and the walk is short
+    assert hip.prefill_waves(32, 4, 64, mean_keys=1024.5) == 8 and hip.prefill_waves(32, 4, 128, mean_keys=1024.5) == 8
+    assert hip.prefill_waves(32, 4, 64, mean_keys=4096.0) == 4, "a long walk: the doubled reads of LDS cost more"
+    assert hip.prefill_waves(16, 4, 64, mean_keys=256.0) == 4 and hip.prefill_waves(64, 4, 64, mean_keys=100.0) == 4
+    assert hip.prefill_waves(40, 3, 96, mean_keys=500.0) == 4, "twelve registers a step do not go round eight waves"
     for tokens, nkv, group in ((100, 2, 3), (5000, 4, 8), (100000, 8, 1)):
         per_wave = hip.PREFILL_WAVES * (16 // group)
         assert hip.prefill_tile_tokens(tokens, nkv, group, 64, 5000.0) in (per_wave, 2 * per_wave, 4 * per_wave)

@@ -6,12 +6,15 @@
 // m follows the row's running maximum lazily: it is raised (and the sums rescaled) only when a score
 // exceeds it by more than 2^8, so that most steps need no exchange between lanes; P stays below 2^8,
 // the sums are 32-bit, and a row's m depends on that row's scores alone. Each lane sums the P of its
-// own keys; the four lanes of a row add theirs up once, at the end (`row_sum`).
+// own keys; the four lanes of a row add theirs up once, at the end (`row_sum`). Or, where the vector
+// unit is what bounds the kernel (prompt portions), the matrix cores sum P as well: one more product,
+// of P with a matrix of ones, gives every row's sum in the layout of the output rows.
 // The result layout of the first product is the operand layout of the second, so P never leaves
 // its registers. Keys are read as 16-byte pieces of their rows; values are read from pages that
 // hold them transposed ([head_dim, page_size] per head), so that the consecutive keys an operand
 // needs lie side by side in memory.
 #pragma once
+#include <type_traits>
 #include "common.h"
 
 typedef float float4_t __attribute__((ext_vector_type(4)));
@@ -113,23 +116,31 @@ static __device__ __forceinline__ void load_tile(KVTile<HD>& T, int kb, int r, i
 
 #define TS_LAZY_MAX 8.0f     // a row's reference maximum is raised when a score exceeds it by more than this (log2 units)
 
-// One 32-key step of the online softmax for the 16 rows that `qreg` holds (lane r = row r of the
-// score tile; output row 4 g + j). `m` is the row's reference maximum in units of log2 (the same in
-// the row's four lanes), `l` this lane's share of the row's sum. scale2 > 0.
-// MASKED: rows mask the keys beyond their position and before their window; without it every key
-// of the step is visible to every row (the caller has checked).
-template <int HD, bool MASKED>
-static __device__ __forceinline__ void use_tile(const KVTile<HD>& T, int kb, int r, int g, int lo, int pos,
-                                                const uint4 (&qreg)[HD / 32], float scale2, float& m, float& l,
-                                                float4_t (&o)[HD / 16]) {
-  constexpr int NC = HD / 32, NDB = HD / 16;
-  float4_t s[2];
+// The scores of one 32-key step for the 16 rows that `qreg` holds: s[tau][j] = key kb + 8 g + 4 tau + j
+// against row r (lane r = row r of the score tile), not yet scaled.
+template <int HD>
+static __device__ __forceinline__ void tile_scores(const uint4 (&k)[2][HD / 32], const uint4 (&qreg)[HD / 32], float4_t (&s)[2]) {
 #pragma unroll
   for (int tau = 0; tau < 2; ++tau) {
     s[tau] = (float4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int c = 0; c < NC; ++c) s[tau] = mfma32(T.k[tau][c], qreg[c], s[tau]);
+    for (int c = 0; c < HD / 32; ++c) s[tau] = mfma32(k[tau][c], qreg[c], s[tau]);
   }
+}
+
+// The rest of the step: the online softmax of the scores `s` and the products with the values `v`
+// (output row 4 g + j). `m` is the row's reference maximum in units of log2 (the same in the row's four
+// lanes). `l`, a float: this lane's share of the row's sum; a float4_t: the sums of the output rows
+// 4 g + j, made by the matrix cores from the rounded P that the output is made of. scale2 > 0.
+// MASKED: rows mask the keys beyond their position and before their window (`vok`: whether any of
+// this lane's eight keys of v is visible); without it every key of the step is visible to every row
+// (the caller has checked).
+template <int HD, bool MASKED, typename L>
+static __device__ __forceinline__ void tile_softmax_values(float4_t (&s)[2], const uint4 (&v)[HD / 16], bool vok, int kb, int r,
+                                                           int g, int lo, int pos, float scale2, float& m, L& l,
+                                                           float4_t (&o)[HD / 16]) {
+  constexpr int NDB = HD / 16;
+  constexpr bool SUMS_BY_MFMA = std::is_same<L, float4_t>::value;
   // this lane: row r, keys kb + 8 g + 4 tau + j
   float mloc = -INFINITY;
 #pragma unroll
@@ -150,11 +161,12 @@ static __device__ __forceinline__ void use_tile(const KVTile<HD>& T, int kb, int
     const bool mine = ((hit >> r) & 0x0001000100010001ull) != 0;   // a lane of this lane's row
     const float m_new = mine ? fmaxf(m, mrow) : m;                 // finite where it changes
     const float alpha = m_new == m ? 1.0f : fast_exp2(m - m_new);
-    l *= alpha;
+    if constexpr (!SUMS_BY_MFMA) l *= alpha;
     // output row 4 g + j belongs to score row 4 g + j, whose alpha lane 4 g + j holds
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const float aj = __shfl(alpha, 4 * g + j, TS_WAVE);
+      if constexpr (SUMS_BY_MFMA) l[j] *= aj;
 #pragma unroll
       for (int db = 0; db < NDB; ++db) o[db][j] *= aj;
     }
@@ -167,13 +179,27 @@ static __device__ __forceinline__ void use_tile(const KVTile<HD>& T, int kb, int
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       p[tau][j] = fast_exp2(fmaf(s[tau][j], scale2, neg_m));
-      l += p[tau][j];
+      if constexpr (!SUMS_BY_MFMA) l += p[tau][j];
     }
   // this lane's eight keys kb + 8 g .. + 7, in the order the value registers hold them
   const uint4 pa = make_uint4(pack_bf16(p[0][0], p[0][1]), pack_bf16(p[0][2], p[0][3]), pack_bf16(p[1][0], p[1][1]),
                               pack_bf16(p[1][2], p[1][3]));
 #pragma unroll
-  for (int db = 0; db < NDB; ++db) o[db] = mfma32(pa, (MASKED && !T.vok) ? make_uint4(0, 0, 0, 0) : T.v[db], o[db]);
+  for (int db = 0; db < NDB; ++db) o[db] = mfma32(pa, (MASKED && !vok) ? make_uint4(0, 0, 0, 0) : v[db], o[db]);
+  if constexpr (SUMS_BY_MFMA) {
+    const uint32_t ones = 0x3f803f80u;                 // 1.0 twice (a masked key's P is 0 already)
+    l = mfma32(pa, make_uint4(ones, ones, ones, ones), l);
+  }
+}
+
+// One 32-key step whole: the scores, then the softmax and the values.
+template <int HD, bool MASKED, typename L>
+static __device__ __forceinline__ void use_tile(const KVTile<HD>& T, int kb, int r, int g, int lo, int pos,
+                                                const uint4 (&qreg)[HD / 32], float scale2, float& m, L& l,
+                                                float4_t (&o)[HD / 16]) {
+  float4_t s[2];
+  tile_scores<HD>(T.k, qreg, s);
+  tile_softmax_values<HD, MASKED, L>(s, T.v, T.vok, kb, r, g, lo, pos, scale2, m, l, o);
 }
 
 // The same, choosing the variant: `pmin` and `lomax` are the smallest position and the largest
@@ -182,8 +208,8 @@ template <int HD>
 static __device__ __forceinline__ void use_tile_auto(const KVTile<HD>& T, int kb, int r, int g, int lo, int pos,
                                                      int pmin, int lomax, const uint4 (&qreg)[HD / 32], float scale2,
                                                      float& m, float& l, float4_t (&o)[HD / 16]) {
-  if (kb + 31 <= pmin && kb >= lomax) use_tile<HD, false>(T, kb, r, g, lo, pos, qreg, scale2, m, l, o);
-  else use_tile<HD, true>(T, kb, r, g, lo, pos, qreg, scale2, m, l, o);
+  if (kb + 31 <= pmin && kb >= lomax) use_tile<HD, false, float>(T, kb, r, g, lo, pos, qreg, scale2, m, l, o);
+  else use_tile<HD, true, float>(T, kb, r, g, lo, pos, qreg, scale2, m, l, o);
 }
 
 // out[t, h, :] from the chunks' partial results part_o [tokens, nh, num_splits, hd] and part_ml

@@ -23,15 +23,19 @@
 #include <type_traits>
 #include "attention_mfma.h"
 
-#define PRE_WAVES 4
+#define PRE_MAX_WAVES 8
 
 template <int HD>
 struct PrefillLds {
   uint4 stage[2][HD / 8][TS_WAVE];   // two steps of operand registers, [register][lane]
-  int range[4][PRE_WAVES];
+  int range[4][PRE_MAX_WAVES];
 };
 
-template <int HD, int RT>
+// PRE_WAVES: 4, or 8 (heads of 64 or 128 dimensions): the same tokens a workgroup in tiles half as
+// large a wave, so that a step's vector work is spread over twice the waves; the longest tiles of a
+// short prompt, which run alone at the end, then take a shorter step (2,048 tokens at head size 64:
+// 48.9 µs against 51.3; over long contexts the doubled reads of LDS cost more than that gains).
+template <int HD, int RT, int PRE_WAVES>
 static __device__ __forceinline__ void
 prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
              const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
@@ -123,11 +127,12 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
   }
 
   uint4 qreg[RT][NC];
-  float m[RT], l[RT];
+  float m[RT];
+  float4_t l[RT];                 // the sums of the output rows 4 g + i, made by the matrix cores
   float4_t o[RT][NDB];
 #pragma unroll
   for (int j = 0; j < RT; ++j) {
-    m[j] = -INFINITY; l[j] = 0.f;
+    m[j] = -INFINITY; l[j] = (float4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int c = 0; c < NC; ++c) qreg[j][c] = make_uint4(0, 0, 0, 0);
     if (tk[j] >= 0) {
@@ -139,10 +144,14 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
     for (int db = 0; db < NDB; ++db) o[j][db] = (float4_t){0.f, 0.f, 0.f, 0.f};
   }
 
-  // This wave's quarter of a step's operand registers: waves 0 and 1 the two 16-key tiles of K
-  // (NC registers each), waves 2 and 3 half of the NDB registers of V each (NDB = 2 NC).
-  uint4 fetched[NC];
+  // This wave's share of a step's operand registers, PER of the 4 NC: register q < 2 NC is piece q % NC
+  // of the 16-key tile q / NC of K, register 2 NC + db is dimension block db of V.
+  constexpr int PER = 4 * NC / PRE_WAVES;
+  static_assert(PER >= 1 && PER * PRE_WAVES == 4 * NC, "the waves share a step's operand registers evenly");
+  uint4 fetched[PER];
   const bool whole = pm.whole_steps();
+  const bool loads_k = wave * PER < 2 * NC;           // (a wave's registers are all of K or all of V)
+  const int tau = (wave * PER) / NC, c0 = (wave * PER) % NC, db0 = wave * PER - 2 * NC;
   auto fetch = [&](int kb) {
     if (whole) {
       // one page for the whole step: its base addresses are scalars, the lanes add fixed offsets
@@ -153,49 +162,49 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
       const bf16_t* src;              // this lane's first piece; the others follow at a fixed stride
       int64_t stride;
       bool ok;
-      if (wave < 2) {
-        const int koff = 8 * (r >> 2) + 4 * wave + (r & 3);
-        src = k_cache + page * kp + (int64_t)slot * ks + (int64_t)kvh * kh + (int64_t)koff * ks + 8 * g;
+      if (loads_k) {
+        const int koff = 8 * (r >> 2) + 4 * tau + (r & 3);
+        src = k_cache + page * kp + (int64_t)slot * ks + (int64_t)kvh * kh + (int64_t)koff * ks + 8 * g + 32 * c0;
         stride = 32;
         ok = kb + koff <= whi && kb + koff >= wlo;
       } else {
-        src = v_cache + page * vp + slot + (int64_t)kvh * vh + 8 * g + (int64_t)((wave - 2) * NC * 16 + r) * vd;
+        src = v_cache + page * vp + slot + (int64_t)kvh * vh + 8 * g + (int64_t)(db0 * 16 + r) * vd;
         stride = 16 * vd;
         ok = kb + 8 * g <= whi && kb + 8 * g + 7 >= wlo;
       }
       if (inner) {                    // nearly every step: nothing to leave out, nothing to clear
 #pragma unroll
-        for (int c = 0; c < NC; ++c) fetched[c] = *(const uint4*)(src + c * stride);
+        for (int c = 0; c < PER; ++c) fetched[c] = *(const uint4*)(src + c * stride);
       } else {
 #pragma unroll
-        for (int c = 0; c < NC; ++c) fetched[c] = ok ? *(const uint4*)(src + c * stride) : make_uint4(0, 0, 0, 0);
+        for (int c = 0; c < PER; ++c) fetched[c] = ok ? *(const uint4*)(src + c * stride) : make_uint4(0, 0, 0, 0);
       }
       return;
     }
 #pragma unroll
-    for (int c = 0; c < NC; ++c) fetched[c] = make_uint4(0, 0, 0, 0);
-    if (wave < 2) {
-      const int key = kb + 8 * (r >> 2) + 4 * wave + (r & 3);
+    for (int c = 0; c < PER; ++c) fetched[c] = make_uint4(0, 0, 0, 0);
+    if (loads_k) {
+      const int key = kb + 8 * (r >> 2) + 4 * tau + (r & 3);
       if (key <= whi && key >= wlo) {
         const int pg = pm.page(key);
-        const bf16_t* kr = k_cache + (int64_t)table[pg] * kp + (int64_t)pm.slot(key, pg) * ks + (int64_t)kvh * kh + 8 * g;
+        const bf16_t* kr = k_cache + (int64_t)table[pg] * kp + (int64_t)pm.slot(key, pg) * ks + (int64_t)kvh * kh + 8 * g + 32 * c0;
 #pragma unroll
-        for (int c = 0; c < NC; ++c) fetched[c] = *(const uint4*)(kr + 32 * c);
+        for (int c = 0; c < PER; ++c) fetched[c] = *(const uint4*)(kr + 32 * c);
       }
     } else {
       const int vkey = kb + 8 * g;
       if (vkey <= whi && vkey + 7 >= wlo) {
         const int pg = pm.page(vkey);
         const bf16_t* vr = v_cache + (int64_t)table[pg] * vp + pm.slot(vkey, pg) + (int64_t)kvh * vh +
-                           (int64_t)((wave - 2) * NC * 16 + r) * vd;
+                           (int64_t)(db0 * 16 + r) * vd;
 #pragma unroll
-        for (int c = 0; c < NC; ++c) fetched[c] = *(const uint4*)(vr + (int64_t)(16 * c) * vd);
+        for (int c = 0; c < PER; ++c) fetched[c] = *(const uint4*)(vr + (int64_t)(16 * c) * vd);
       }
     }
   };
   auto put = [&](int buf) {
 #pragma unroll
-    for (int c = 0; c < NC; ++c) stage[buf][wave * NC + c][lane] = fetched[c];
+    for (int c = 0; c < PER; ++c) stage[buf][wave * PER + c][lane] = fetched[c];
   };
 
   const int kbeg = wlo & ~31;
@@ -223,9 +232,9 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
         if constexpr (decltype(masked)::value) {
           // a step wholly beyond the tile's last position, or wholly before all its windows, has nothing for it
           if (kb <= tile_pmax[j] && kb + 31 >= tile_lomin[j])
-            use_tile<HD, true>(T, kb, r, g, lo[j], pos[j], qreg[j], scale2, m[j], l[j], o[j]);
+            use_tile<HD, true, float4_t>(T, kb, r, g, lo[j], pos[j], qreg[j], scale2, m[j], l[j], o[j]);
         } else {
-          use_tile<HD, false>(T, kb, r, g, lo[j], pos[j], qreg[j], scale2, m[j], l[j], o[j]);
+          use_tile<HD, false, float4_t>(T, kb, r, g, lo[j], pos[j], qreg[j], scale2, m[j], l[j], o[j]);
         }
       }
       __syncthreads();
@@ -240,16 +249,13 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
     walk(full_lo, full_hi, std::false_type{});
     walk(full_hi, kend, std::true_type{});
   }
-  // output row 4 g + i of row tile j: its token and head; its sum sits in lane 4 g + i
-  float lsum[RT];
-#pragma unroll
-  for (int j = 0; j < RT; ++j) lsum[j] = row_sum(l[j]);
+  // output row 4 g + i of row tile j: its token and head, and its sum
 #pragma unroll
   for (int j = 0; j < RT; ++j)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int row = 4 * g + i;
-      const float lj = __shfl(lsum[j], row, TS_WAVE);
+      const float lj = l[j][i];
       const int rtk = (wave * RT + j) * tpt + row / G, rhh = row % G;
       if (num_splits > 1) {
         // the chunk's share of the row, not normalised: sums, and the reference maximum they are relative to
@@ -271,7 +277,7 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
     }
 }
 
-template <int HD, int RT>
+template <int HD, int RT, int PRE_WAVES>
 __global__ void __launch_bounds__(PRE_WAVES * TS_WAVE)
 attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
                          const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables,
@@ -288,21 +294,22 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
   if (item >= num_tiles * heads_per_group) return;
   const int tile = num_tiles - 1 - item / heads_per_group;
   const int kvh = (die / dies_per_group) * heads_per_group + item % heads_per_group;
-  prefill_tile<HD, RT>(lds, tile, kvh, out, q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, nh,
+  prefill_tile<HD, RT, PRE_WAVES>(lds, tile, kvh, out, q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, nh,
                        G, page_size, page_shift, kp, ks, kh, vp, vh, vd, max_blocks, scale2, window, part_o, part_ml,
                        num_splits, chunk, blockIdx.y);
 }
 
 // Keys: rows dense in head_dim, strides kp/ks/kh (page, slot, head). Values: transposed pages,
 // slot stride 1, strides vp/vh/vd (page, head, dimension). tile_tokens: the most tokens a listed
-// tile holds, 4 RT (16 / G) for RT of 1, 2 or 4. num_splits > 1: chunk (a multiple of 32; the last chunk
+// tile holds, waves x RT (16 / G) for RT of 1, 2 or 4 row tiles a wave and 4 waves, or 8 waves with one or two
+// (heads of 64 or 128 dimensions). num_splits > 1: chunk (a multiple of 32; the last chunk
 // takes every key from its start on) and the float workspaces part_o [num_tokens, nh, num_splits, hd] and
 // part_ml [num_tokens, nh, num_splits, 2]; every token from first_token on must then be in a tile (the ones
 // before it keep what `out` held).
 extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* k_cache, const void* v_cache,
                                           const int32_t* block_tables, const int32_t* seq_of_token,
                                           const int32_t* positions, const int32_t* tiles, int num_tiles,
-                                          int tile_tokens, int nh, int nkv, int hd, int page_size, int64_t kp,
+                                          int tile_tokens, int waves, int nh, int nkv, int hd, int page_size, int64_t kp,
                                           int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
                                           float scale, int window, int first_token, int num_tokens, int num_splits,
                                           int chunk, float* part_o, float* part_ml, hipStream_t stream) {
@@ -313,8 +320,9 @@ extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* 
   if (nkv <= 0 || nh % nkv || page_size <= 0 || page_size % 8 || max_blocks <= 0) return TS_BAD_SHAPE;
   const int G = nh / nkv;
   if (G > 16) return TS_BAD_SHAPE;
-  const int per_wave = PRE_WAVES * (16 / G);
-  if (tile_tokens != per_wave && tile_tokens != 2 * per_wave && tile_tokens != 4 * per_wave) return TS_BAD_SHAPE;
+  if (waves != 4 && !(waves == 8 && (hd == 64 || hd == 128))) return TS_BAD_SHAPE;
+  const int per_wave = waves * (16 / G);
+  if (tile_tokens != per_wave && tile_tokens != 2 * per_wave && !(tile_tokens == 4 * per_wave && waves == 4)) return TS_BAD_SHAPE;
   const int rt = tile_tokens / per_wave;
   if ((kp % 8) || (ks % 8) || (kh % 8) || (vp % 8) || (vh % 8) || (vd % 8)) return TS_BAD_SHAPE;
   if ((((uintptr_t)q) | ((uintptr_t)k_cache) | ((uintptr_t)v_cache)) & 15) return TS_BAD_SHAPE;
@@ -329,22 +337,33 @@ extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* 
   const int64_t turns = ((int64_t)num_tiles * heads_per_group + dies_per_group - 1) / dies_per_group;
   if (turns * 8 > 0x7fffffff) return TS_BAD_SHAPE;
   dim3 grid((unsigned)(8 * turns), num_splits);
-#define TS_PRE(HH, RR)                                                                                          \
-  attn_prefill_mfma_kernel<HH, RR><<<grid, PRE_WAVES * TS_WAVE, 0, stream>>>(                                   \
+#define TS_PRE_W(HH, RR, WW)                                                                                    \
+  attn_prefill_mfma_kernel<HH, RR, WW><<<grid, WW * TS_WAVE, 0, stream>>>(                                      \
       (bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,             \
       seq_of_token, positions, tiles, num_tiles, nh, G, dies_per_group, heads_per_group, page_size, page_shift, kp,  \
       ks, kh, vp, vh, vd, max_blocks, scale * 1.44269504088896340736f, window, part_o, part_ml, num_splits, chunk)
 #define TS_PRE_RT(HH)                                                                                           \
-  if (rt == 1) TS_PRE(HH, 1); else if (rt == 2) TS_PRE(HH, 2); else TS_PRE(HH, 4)
-  switch (hd) {
-    case 32: TS_PRE_RT(32); break;
-    case 64: TS_PRE_RT(64); break;
-    case 96: TS_PRE_RT(96); break;
-    case 128: TS_PRE_RT(128); break;
-    default: return TS_BAD_SHAPE;
+  if (rt == 1) TS_PRE_W(HH, 1, 4); else if (rt == 2) TS_PRE_W(HH, 2, 4); else TS_PRE_W(HH, 4, 4)
+#define TS_PRE_RT8(HH)                                                                                          \
+  if (rt == 1) TS_PRE_W(HH, 1, 8); else TS_PRE_W(HH, 2, 8)
+  if (waves == 8) {
+    switch (hd) {
+      case 64: TS_PRE_RT8(64); break;
+      case 128: TS_PRE_RT8(128); break;
+      default: return TS_BAD_SHAPE;       // (96: twelve registers a step do not go round eight waves)
+    }
+  } else {
+    switch (hd) {
+      case 32: TS_PRE_RT(32); break;
+      case 64: TS_PRE_RT(64); break;
+      case 96: TS_PRE_RT(96); break;
+      case 128: TS_PRE_RT(128); break;
+      default: return TS_BAD_SHAPE;
+    }
   }
+#undef TS_PRE_RT8
 #undef TS_PRE_RT
-#undef TS_PRE
+#undef TS_PRE_W
   const int rc = ts_check_launch();
   if (rc || num_splits == 1) return rc;
   const int64_t skip = (int64_t)first_token * nh;     // rows of the tokens before the first listed one

@@ -195,8 +195,9 @@ extern "C" int ts_rmsnorm(void* out, void* res_out, const void* x, const void* r
 }
 
 // ------------------------------------------------------------------------------------------
-// Rotate-half RoPE on q and k from a 32-bit [max_pos, head_dim] table ([cos | sin] halves),
-// fused with the scatter of rotated k and of v into their cache slots.
+// Rotate-half RoPE on q and k from a 32-bit [max_pos, rot] table ([cos | sin] halves), fused with the
+// scatter of rotated k and of v into their cache slots. rot <= head_dim is the rotated width: dimension
+// j < rot / 2 of a head turns with dimension j + rot / 2, the dimensions from rot on pass as they are.
 //   qkv   [T, (nh + 2*nkv) * hd]   one token's q heads, then k heads, then v heads
 //   q_out [T, nh * hd]
 //   key element address:   page * kp + offset * ks + head * kh + d          (d dense)
@@ -215,12 +216,12 @@ template <typename T>
 __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
                                   const T* __restrict__ qkv, const float* __restrict__ cos_sin,
                                   const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
-                                  int num_tokens, int nh, int nkv, int hd, int rotate, int page_size, int64_t kp,
+                                  int num_tokens, int nh, int nkv, int hd, int rot, int rotate, int page_size, int64_t kp,
                                   int64_t ks, int64_t kh, int64_t vp, int64_t vs, int64_t vh, int64_t vd, int vec, int vtile,
                                   int v_slices) {
   const int t0 = blockIdx.x * ROPE_TOK;
   const int nt = num_tokens - t0 < ROPE_TOK ? num_tokens - t0 : ROPE_TOK;
-  const int half = hd / 2;
+  const int half = rot / 2, rest = hd - rot;          // pairs that turn, and dimensions that pass
   // v_slices > 0: the last v_slices of the gridDim.y slices write the values, the others rotate q
   // and k (the two are independent chains of loads and stores: side by side they take half the
   // time); v_slices == 0: every workgroup does its slice of both
@@ -235,28 +236,30 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
   const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
   auto page_of = [&](int slot) { return page_shift >= 0 ? slot >> page_shift : slot / page_size; };
   const int row = (nh + 2 * nkv) * hd;
-  const int qpairs = nh * half, kpairs = nkv * half;
-  // q and k pairs of every token of the group: this workgroup's slice of them
+  const int per_head_items = half + rest;             // a pair or a passing dimension each
+  const int qpairs = nh * per_head_items, kpairs = nkv * per_head_items;
+  // q and k items of every token of the group: this workgroup's slice of them
   const int npairs = nt * (qpairs + kpairs);
   constexpr int V = 16 / sizeof(T);
   if (!do_qk) {
   } else if (vec) {
-    // 16 bytes of each half of a head at a time
-    const int per_head = half / V;
+    // 16 bytes of each half of a head's rotated part at a time, then 16 bytes of what passes
+    const int turning = half / V, per_head = turning + rest / V;
     const int npieces = nt * (nh + nkv) * per_head;
     const int pbeg = (int)((int64_t)npieces * by / ny), pend = (int)((int64_t)npieces * (by + 1) / ny);
     for (int i = pbeg + threadIdx.x; i < pend; i += blockDim.x) {
       const int tl = i / ((nh + nkv) * per_head), e = i - tl * ((nh + nkv) * per_head);
       const int t = t0 + tl;
-      const int h = e / per_head, j = (e - h * per_head) * V;
-      const bool is_k = h >= nh;
+      const int h = e / per_head, piece = e - h * per_head;
+      const bool is_k = h >= nh, passes = piece >= turning;
+      const int j = passes ? rot + (piece - turning) * V : piece * V;
       if (is_k && (!k_cache || slots[t] < 0)) continue;
       const T* src = qkv + (int64_t)t * row + h * hd;      // k heads follow the q heads in a row
       float x1[V], x2[V];
       Pack16<T>::ld(src + j, x1);
-      Pack16<T>::ld(src + j + half, x2);
-      if (rotate) {
-        const float* cs = cos_sin + (int64_t)positions[t] * hd;
+      if (!passes) Pack16<T>::ld(src + j + half, x2);
+      if (rotate && !passes) {
+        const float* cs = cos_sin + (int64_t)positions[t] * rot;
 #pragma unroll
         for (int k = 0; k < V; ++k) {
           const float c = cs[j + k], sn = cs[half + j + k];
@@ -273,7 +276,7 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
         dst = q_out + ((int64_t)t * nh + h) * hd;
       }
       Pack16<T>::st(dst + j, x1);
-      Pack16<T>::st(dst + j + half, x2);
+      if (!passes) Pack16<T>::st(dst + j + half, x2);
     }
   } else {
   const int pbeg = (int)((int64_t)npairs * by / ny), pend = (int)((int64_t)npairs * (by + 1) / ny);
@@ -282,13 +285,15 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
     const int t = t0 + tl;
     const bool is_k = e >= qpairs;
     const int pe = is_k ? e - qpairs : e;
-    const int h = pe / half, j = pe - h * half;
+    const int h = pe / per_head_items, item = pe - h * per_head_items;
+    const bool passes = item >= half;
+    const int j = passes ? rot + (item - half) : item;
     const T* src = qkv + (int64_t)t * row + (is_k ? nh * hd : 0) + h * hd;
     if (is_k && (!k_cache || slots[t] < 0)) continue;
-    const float x1 = Num<T>::ld(src + j), x2 = Num<T>::ld(src + j + half);
+    const float x1 = Num<T>::ld(src + j), x2 = passes ? 0.f : Num<T>::ld(src + j + half);
     float y1 = x1, y2 = x2;
-    if (rotate) {
-      const float* cs = cos_sin + (int64_t)positions[t] * hd;
+    if (rotate && !passes) {
+      const float* cs = cos_sin + (int64_t)positions[t] * rot;
       const float c = cs[j], sn = cs[half + j];
       y1 = x1 * c - x2 * sn;
       y2 = x2 * c + x1 * sn;
@@ -301,7 +306,7 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
       dst = q_out + ((int64_t)t * nh + h) * hd;
     }
     Num<T>::st(dst + j, y1);
-    Num<T>::st(dst + j + half, y2);
+    if (!passes) Num<T>::st(dst + j + half, y2);
   }
   }
   if (!k_cache || !do_v) return;
@@ -385,10 +390,11 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
 
 extern "C" int ts_rope_store(void* q_out, void* k_cache, void* v_cache, const void* qkv, const float* cos_sin,
                              const int32_t* positions, const int32_t* slots, int num_tokens, int nh, int nkv,
-                             int hd, int rotate, int page_size, int64_t kp, int64_t ks, int64_t kh, int64_t vp,
+                             int hd, int rot, int rotate, int page_size, int64_t kp, int64_t ks, int64_t kh, int64_t vp,
                              int64_t vs, int64_t vh, int64_t vd, int dtype, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
-  if (hd % 2 || nh <= 0 || nkv < 0 || page_size <= 0) return TS_BAD_SHAPE;
+  if (hd <= 0 || rot % 2 || rot < 0 || rot > hd || nh <= 0 || nkv < 0 || page_size <= 0) return TS_BAD_SHAPE;
+  if (!rotate) rot = hd - hd % 2;                     // (nothing turns: the split into pairs is free)
   const int groups = (num_tokens + ROPE_TOK - 1) / ROPE_TOK;
   int slices = 2048 / groups;                       // enough workgroups to hide the loads' latency
   if (slices < 1) slices = 1;
@@ -397,7 +403,7 @@ extern "C" int ts_rope_store(void* q_out, void* k_cache, void* v_cache, const vo
   // 16-byte pieces need halves of whole pieces and aligned rows everywhere
   const int per16 = dtype == 0 ? 4 : 8;
   const int row = (nh + 2 * nkv) * hd;
-  const int vec = (hd / 2) % per16 == 0 && row % per16 == 0 && kp % per16 == 0 && ks % per16 == 0 && kh % per16 == 0 &&
+  const int vec = (rot / 2) % per16 == 0 && (hd - rot) % per16 == 0 && hd % per16 == 0 && row % per16 == 0 && kp % per16 == 0 && ks % per16 == 0 && kh % per16 == 0 &&
                   ((((uintptr_t)q_out) | ((uintptr_t)k_cache) | ((uintptr_t)qkv)) & 15) == 0;
   // values through LDS: bfloat16 steps of several tokens into transposed pages (slot stride 1) whose
   // 8-slot pieces are 16-byte aligned
@@ -412,11 +418,11 @@ extern "C" int ts_rope_store(void* q_out, void* k_cache, void* v_cache, const vo
   if (dtype == 0)
     rope_store_kernel<float><<<blocks, 256, 0, stream>>>((float*)q_out, (float*)k_cache, (float*)v_cache,
                                                          (const float*)qkv, cos_sin, positions, slots, num_tokens, nh,
-                                                         nkv, hd, rotate, page_size, kp, ks, kh, vp, vs, vh, vd, vec, 0, 0);
+                                                         nkv, hd, rot, rotate, page_size, kp, ks, kh, vp, vs, vh, vd, vec, 0, 0);
   else if (dtype == 1)
     rope_store_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache,
                                                           (const bf16_t*)qkv, cos_sin, positions, slots, num_tokens,
-                                                          nh, nkv, hd, rotate, page_size, kp, ks, kh, vp, vs, vh, vd, vec, vtile, v_slices);
+                                                          nh, nkv, hd, rot, rotate, page_size, kp, ks, kh, vp, vs, vh, vd, vec, vtile, v_slices);
   else
     return TS_BAD_DTYPE;
   return ts_check_launch();

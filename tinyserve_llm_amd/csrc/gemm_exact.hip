@@ -65,6 +65,42 @@ gemm_exact_kernel(TC* __restrict__ C, const TA* __restrict__ A, const TW* __rest
   }
 }
 
+// The same sums for few rows of A (decode steps): a 64-row tile would be mostly empty and a narrow W would
+// make a few dozen workgroups. Here a workgroup owns 16 rows of W, a thread one element of C, and the
+// element's sum runs over k in the same ascending order with the same fused multiply-adds, so it is
+// the same 32 bits as the tiled kernel gives.
+#define GR_BN 16
+#define GR_BM 16
+#define GR_BK 64
+
+template <typename TA, typename TW, typename TC>
+__global__ void __launch_bounds__(256)
+gemm_exact_rows_kernel(TC* __restrict__ C, const TA* __restrict__ A, const TW* __restrict__ W, int M, int N, int K,
+                       int64_t lda, int64_t ldw, int64_t ldc) {
+  __shared__ float As[GR_BM][GR_BK + 4];
+  __shared__ float Ws[GR_BN][GR_BK + 4];
+  const int tid = threadIdx.x;
+  const int n0 = blockIdx.x * GR_BN, m0 = blockIdx.y * GR_BM;
+  const int tx = tid & 15, ty = tid >> 4;     // this thread's element: row m0 + ty of A, row n0 + tx of W
+  const int lr = tid >> 4, lk = (tid & 15) * 4;   // loading: row lr of the tile, 4 consecutive k from lk
+  float acc = 0.f;
+  for (int k0 = 0; k0 < K; k0 += GR_BK) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int k = k0 + lk + i;
+      As[lr][lk + i] = (k < K && m0 + lr < M) ? Num<TA>::ld(A + (int64_t)(m0 + lr) * lda + k) : 0.f;
+      Ws[lr][lk + i] = (k < K && n0 + lr < N) ? Num<TW>::ld(W + (int64_t)(n0 + lr) * ldw + k) : 0.f;
+    }
+    __syncthreads();
+    // (the sum stops at K: no products of the tile's padding are added)
+    const int kn = K - k0 < GR_BK ? K - k0 : GR_BK;
+    for (int k = 0; k < kn; ++k) acc = fmaf(As[ty][k], Ws[tx][k], acc);
+    __syncthreads();
+  }
+  const int m = m0 + ty, n = n0 + tx;
+  if (m < M && n < N) Num<TC>::st(C + (int64_t)m * ldc + n, acc);
+}
+
 // in_dtype: storage of A and W; out_dtype: storage of C (0 float, 1 bfloat16).
 extern "C" int ts_gemm_exact(void* C, const void* A, const void* W, int M, int N, int K, int64_t lda, int64_t ldw,
                              int64_t ldc, int in_dtype, int out_dtype, hipStream_t stream) {
@@ -72,6 +108,21 @@ extern "C" int ts_gemm_exact(void* C, const void* A, const void* W, int M, int N
   if (K <= 0 || lda < K || ldw < K || ldc < N) return TS_BAD_SHAPE;
   dim3 grid((N + GE_BN - 1) / GE_BN, (M + GE_BM - 1) / GE_BM), block(256);
   if (grid.y > 65535) return TS_BAD_SHAPE;
+  if (M <= 2 * GR_BM) {                     // few rows: an element a thread
+    dim3 rgrid((N + GR_BN - 1) / GR_BN, (M + GR_BM - 1) / GR_BM);
+    if (in_dtype == 0 && out_dtype == 0)
+      gemm_exact_rows_kernel<float, float, float><<<rgrid, block, 0, stream>>>((float*)C, (const float*)A, (const float*)W,
+                                                                               M, N, K, lda, ldw, ldc);
+    else if (in_dtype == 1 && out_dtype == 1)
+      gemm_exact_rows_kernel<bf16_t, bf16_t, bf16_t><<<rgrid, block, 0, stream>>>((bf16_t*)C, (const bf16_t*)A,
+                                                                                  (const bf16_t*)W, M, N, K, lda, ldw, ldc);
+    else if (in_dtype == 1 && out_dtype == 0)
+      gemm_exact_rows_kernel<bf16_t, bf16_t, float><<<rgrid, block, 0, stream>>>((float*)C, (const bf16_t*)A,
+                                                                                 (const bf16_t*)W, M, N, K, lda, ldw, ldc);
+    else
+      return TS_BAD_DTYPE;
+    return ts_check_launch();
+  }
   if (in_dtype == 0 && out_dtype == 0)
     gemm_exact_kernel<float, float, float><<<grid, block, 0, stream>>>((float*)C, (const float*)A, (const float*)W, M,
                                                                        N, K, lda, ldw, ldc);

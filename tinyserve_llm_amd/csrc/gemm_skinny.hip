@@ -412,12 +412,26 @@ gemm_skinny_kernel(const SkinnyArgs a) {
   }
 }
 
+// The LDS a workgroup may ask for on the current device (asked of the runtime once per device).
+static size_t sk_lds_limit() {
+  static int limit[16] = {0};
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 16) return 65536;
+  if (!limit[device]) {
+    int v = 0;
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, device) != hipSuccess || v <= 0) v = 65536;
+    limit[device] = v;
+  }
+  return (size_t)limit[device];
+}
+
 template <int RT, int CB, int STEPS, int MODE, int GLU, typename OUT>
 static int sk_launch(const SkinnyArgs& a, hipStream_t stream) {
   const int nwaves = a.K / (STEPS * SK_KSTEP);
   const size_t smem = sizeof(float) * ((size_t)nwaves * RT * CB * 256 + (size_t)nwaves * 16 * CB);
   constexpr int OT = GLU == EPI_GLU ? RT / 2 : RT;
   const int ncols = GLU == EPI_GLU ? a.N / 2 : a.N;     // (EPI_ROPE: a 16-row tile of the matrix per 8 columns and their partners)
+  if (smem > sk_lds_limit()) return TS_BAD_SHAPE;       // (the largest instances ask for a little more than 64 KB)
   dim3 grid((ncols + 16 * OT - 1) / (16 * OT)), block(nwaves * TS_WAVE);
   if (nwaves <= 8) {
     gemm_skinny_kernel<RT, CB, STEPS, MODE, GLU, 512, OUT><<<grid, block, smem, stream>>>(a);

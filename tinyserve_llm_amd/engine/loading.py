@@ -2,6 +2,8 @@
 
 from __future__ import annotations
 
+import logging
+
 import torch
 
 from tinyserve_llm_amd import models  # noqa: F401  (registers the architectures)
@@ -9,6 +11,8 @@ from tinyserve_llm_amd.models.decoder import DecoderModel
 from tinyserve_llm_amd.models.registry import architecture_of, read_config
 from tinyserve_llm_amd.weights.loader import load_params
 from tinyserve_llm_amd.weights.random_init import random_params
+
+logger = logging.getLogger(__name__)
 
 DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
 
@@ -32,14 +36,25 @@ def require_gpu(device: str | torch.device) -> torch.device:
     return device
 
 
+STREAMING_COPIES_AT_MOST = 2.0     # times the weights' own bytes: a weight keeps at most one copy per kernel form
+STREAMING_COPIES_SHARE = 0.25      # of the free memory that the weights' copies may take at most
+
+
 def streaming_copies(model: DecoderModel, policy: bool | None, device: torch.device) -> int:
-    """Second copies of layer weights in the decode kernels' reading order (about a sixth faster
-    to stream, for 60 % more weight memory at the 1B shape). `policy` None: only if the model's own
-    weights take less than a fifth of the memory that is still free."""
+    """Second copies of the weights in the decode kernels' reading orders (about a sixth faster to
+    stream). A weight keeps up to one copy per kernel form that can take it (16-row tiles, 8-row
+    tiles, and for q|k|v the tiles regrouped for the rotation), so the copies come to between one and
+    two times the weights' own bytes (1.7 times at the Llama 3.2 1B shape). `policy` None: made only
+    if twice the weights' bytes are less than a quarter of the memory that is still free, which
+    leaves the cache pool what it had; the bytes taken are logged. Returns the bytes taken."""
     if policy is None:
         own = sum(p.numel() * p.element_size() for p in _bound_tensors(model))
-        policy = model.dtype == torch.bfloat16 and own < torch.cuda.mem_get_info(device)[0] / 5
-    return model.keep_streaming_copies() if policy else 0
+        free = torch.cuda.mem_get_info(device)[0]
+        policy = model.dtype == torch.bfloat16 and STREAMING_COPIES_AT_MOST * own < STREAMING_COPIES_SHARE * free
+    taken = model.keep_streaming_copies() if policy else 0
+    if taken:
+        logger.info("streaming copies of the weights: %.2f GB beside the weights' own bytes", taken / 1e9)
+    return taken
 
 
 def _bound_tensors(model: DecoderModel):

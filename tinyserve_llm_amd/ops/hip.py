@@ -46,7 +46,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     sig = {
         "ts_embedding": [p, p, p, i, i, i, p],
         "ts_rmsnorm": [p, p, p, p, p, p, i, i, f, i, i, p],
-        "ts_rope_store": [p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i64, i, p],
+        "ts_rope_store": [p, p, p, p, p, p, p, i, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i64, i, p],
         "ts_silu_mul": [p, p, i, i, i, p],
         "ts_copy_slots": [p, i64, i64, i64, i, i, p],
         "ts_paged_attention_wave": [p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i64, i, f, i, i, p],
@@ -62,7 +62,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_gemm_library_init": [],
         "ts_gemm_library_timing": [i],
         "ts_gemm_library_choices": [p, i],
-        "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, i, i, i, i, p, p, p],
+        "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, i, i, i, i, p, p, p],
         "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p, i, p, p, p, p, p, p],
         "ts_gemm_skinny8_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p, p, p, p, p, p],
         "ts_gemm_rows64_bf16": [p, p, p, i, i, i, i64, i64, i, i, p, i, f, p],
@@ -161,16 +161,20 @@ def rope_store(qkv: torch.Tensor, cos_sin: torch.Tensor | None, positions: torch
     """Rotates q and k of `qkv` [tokens, (nh + 2 nkv) hd] by the table rows of `positions`, returns q
     [tokens, nh, hd] and writes rotated k and v to the cache slots. `k_cache`/`v_cache` are one
     layer's view [pages, page_size, nkv, hd] (may be strided over pages and slots); None = no write.
-    `cos_sin` None = no rotation."""
+    `cos_sin` None = no rotation; a table narrower than head_dim ([positions, rot], rot even) turns
+    the first rot dimensions of every head (j with j + rot / 2) and lets the others pass."""
     _gpu(qkv, cos_sin, positions, slots, k_cache, v_cache)
     T = qkv.shape[0]
     row = (num_heads + 2 * num_kv_heads) * head_dim
     _need(qkv.dim() == 2 and qkv.shape[1] == row and qkv.is_contiguous(), f"qkv must be contiguous [tokens, {row}]")
     _need(positions.dtype == torch.int32 and positions.shape == (T,) and positions.is_contiguous(),
           "positions must be int32 [tokens]")
+    rot = head_dim
     if cos_sin is not None:
-        _need(cos_sin.dtype == torch.float32 and cos_sin.dim() == 2 and cos_sin.shape[1] == head_dim
-              and cos_sin.is_contiguous(), "the rotation table must be float32 [positions, head_dim]")
+        _need(cos_sin.dtype == torch.float32 and cos_sin.dim() == 2 and cos_sin.is_contiguous()
+              and 2 <= cos_sin.shape[1] <= head_dim and cos_sin.shape[1] % 2 == 0,
+              f"the rotation table must be float32 [positions, an even width up to head_dim {head_dim}]")
+        rot = cos_sin.shape[1]
     page_size, kst, vst = 1, (0, 0, 0), (0, 0, 0, 0)
     if k_cache is not None:
         _need(v_cache is not None and slots is not None, "a cache write needs k, v and the slots")
@@ -180,7 +184,7 @@ def rope_store(qkv: torch.Tensor, cos_sin: torch.Tensor | None, positions: torch
     q = torch.empty((T, num_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
     _run("rope_store", library().ts_rope_store(
         _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(qkv), _ptr(cos_sin), _ptr(positions), _ptr(slots), T, num_heads,
-        num_kv_heads, head_dim, int(cos_sin is not None), page_size, *kst, *vst, _code(qkv.dtype), _stream()))
+        num_kv_heads, head_dim, rot, int(cos_sin is not None), page_size, *kst, *vst, _code(qkv.dtype), _stream()))
     return q
 
 
@@ -488,6 +492,23 @@ def prefill_tile_tokens(num_tokens: int, nkv: int, group: int, head_dim: int, me
     return per_wave
 
 
+PREFILL_EIGHT_WAVES_MEAN_KEYS = 1536    # a shorter walk than this on average takes workgroups of eight waves,
+PREFILL_EIGHT_WAVES_HEAD_DIMS = (64, 128)   # for the head sizes whose registers of a step go round eight waves
+
+
+def prefill_waves(tile_tokens: int, group: int, head_dim: int, mean_keys: float) -> int:
+    """Waves of a workgroup of the prefill kernel for tiles of `tile_tokens` tokens: 4, or 8 where a
+    wave of four would hold two row tiles and the walk is short. The longest tiles of a prompt run
+    alone at the end, a step after a step; with eight waves a wave holds one row tile and a step takes
+    it less time (2,048 tokens from position 0 at head size 64: 48.5 µs against 50.1, head size 128:
+    60.6 against 64.6), but every wave reads the step's keys and values out of LDS, which costs more
+    than that over long walks (8,192 tokens: 467 µs against 373)."""
+    two_a_wave = tile_tokens == 2 * PREFILL_WAVES * (16 // group)
+    if two_a_wave and head_dim in PREFILL_EIGHT_WAVES_HEAD_DIMS and 0.0 < mean_keys < PREFILL_EIGHT_WAVES_MEAN_KEYS:
+        return 2 * PREFILL_WAVES
+    return PREFILL_WAVES
+
+
 PREFILL_SPLIT_BELOW_WORKGROUPS = 384    # a step whose tiles make fewer workgroups than this may cut its keys into chunks
 PREFILL_SPLIT_TARGET_WORKGROUPS = 512   # so that about this many workgroups walk them,
 PREFILL_SPLIT_MIN_CHUNK = 512           # each at least this many keys
@@ -532,7 +553,7 @@ def attention_tiles(cu_seqlens: list[int], starts: list[int], tokens_per_tile: i
 def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                             seq_of_token: torch.Tensor, positions: torch.Tensor, tiles: torch.Tensor, scale: float,
                             window: int = 0, tile_tokens: int | None = None, out: torch.Tensor | None = None,
-                            num_splits: int = 1, chunk: int = 0, first_token: int = 0) -> torch.Tensor:
+                            num_splits: int = 1, chunk: int = 0, first_token: int = 0, waves: int = PREFILL_WAVES) -> torch.Tensor:
     """Attention of a packed step on the matrix cores (bfloat16, values in transposed pages).
     `tiles` int32 [num_tiles, 2] lists (first token, token count <= tile_tokens) per workgroup,
     every tile inside one request and inside the step (the caller built the list from the step's
@@ -556,9 +577,12 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         _need(t.dtype == torch.int32 and t.shape == (T,) and t.is_contiguous(), f"{name} must be int32 [tokens]")
     _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 2 and tiles.is_contiguous(),
           "tiles must be contiguous int32 [tiles, 2]")
-    per_wave = PREFILL_WAVES * (16 // (nh // nkv))
+    _need(waves == PREFILL_WAVES or (waves == 2 * PREFILL_WAVES and hd in (64, 128)),
+          f"workgroups of {PREFILL_WAVES} waves, or of {2 * PREFILL_WAVES} for heads of 64 or 128 dimensions")
+    per_wave = waves * (16 // (nh // nkv))
     tile_tokens = tile_tokens or per_wave
-    _need(tile_tokens in (per_wave, 2 * per_wave, 4 * per_wave), f"tiles of {tile_tokens} tokens; {per_wave}, twice or four times that")
+    _need(tile_tokens in (per_wave, 2 * per_wave) or (tile_tokens == 4 * per_wave and waves == PREFILL_WAVES),
+          f"tiles of {tile_tokens} tokens; {per_wave}, twice or (4 waves) four times that")
     out = _out_like(q, out)
     part_o = part_ml = None
     if num_splits > 1:
@@ -568,7 +592,7 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         part_ml = torch.empty((T, nh, num_splits, 2), dtype=torch.float32, device=q.device)
     _run("paged_attention_prefill", library().ts_paged_attention_prefill(
         _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_of_token), _ptr(positions),
-        _ptr(tiles), tiles.shape[0], tile_tokens, nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3], v_cache.stride(0),
+        _ptr(tiles), tiles.shape[0], tile_tokens, waves, nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3], v_cache.stride(0),
         v_cache.stride(2), v_cache.stride(3), block_tables.shape[1], float(scale), int(window), first_token, T,
         num_splits, chunk, _ptr(part_o), _ptr(part_ml), _stream()))
     return out
@@ -592,8 +616,9 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             lead += 1
         nkv = k_cache.shape[2]
         walked = sum((cu[i + 1] - cu[i]) * (ctx.host_starts[i] + (cu[i + 1] - cu[i] + 1) / 2) for i in range(lead, len(cu) - 1))
-        tile_tokens = prefill_tile_tokens(q.shape[0] - lead, nkv, q.shape[1] // nkv, q.shape[2],
-                                          walked / max(1, q.shape[0] - lead))
+        mean_keys = walked / max(1, q.shape[0] - lead)
+        tile_tokens = prefill_tile_tokens(q.shape[0] - lead, nkv, q.shape[1] // nkv, q.shape[2], mean_keys)
+        waves = prefill_waves(tile_tokens, q.shape[1] // nkv, q.shape[2], mean_keys)
         tiles = ctx.scratch.get(("attention_tiles", tile_tokens, lead))
         if tiles is None:
             flat = attention_tiles(cu, ctx.host_starts, tile_tokens, lead)
@@ -606,7 +631,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         splits, chunk = prefill_splits(tiles.shape[0] * nkv, max(ctx.host_context_lens[lead:], default=0))
         return paged_attention_prefill(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, tiles, scale,
                                        window, tile_tokens=tile_tokens, out=out, num_splits=splits, chunk=chunk,
-                                       first_token=cu[lead])
+                                       first_token=cu[lead], waves=waves)
     return paged_attention_wave(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, window)
 
 
@@ -897,11 +922,11 @@ STREAMING_MAX_ROWS = 64      # most rows of x for which `linear_bf16` reads a we
 
 
 def qkv_rope_fuses(x: torch.Tensor, weight: torch.Tensor, head_dim: int, k_cache: torch.Tensor | None,
-                   norm: bool = False) -> bool:
+                   norm: bool = False, table: torch.Tensor | None = None) -> bool:
     """Whether `qkv_rope_store` serves these operands: few bfloat16 rows, a reduction of up to 4096 in
-    steps of 256 (2048 with the norm on the way in), heads of a multiple of 32 dimensions, keys whose
-    strides allow 8-byte stores."""
-    rows_ok = x.dim() == 2 and x.shape[0] <= qkv_rope_max_rows(x.shape[1], norm)
+    steps of 256 (2048 with the norm on the way in), heads of a multiple of 32 dimensions that turn
+    whole (`table`, if given, as wide as a head), keys whose strides allow 8-byte stores."""
+    rows_ok = x.dim() == 2 and x.shape[0] <= qkv_rope_max_rows(x.shape[1], norm) and (table is None or table.shape[1] == head_dim)
     return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and rows_ok and head_dim % 32 == 0
             and x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0
             and (k_cache is None or (all(st % 4 == 0 for st in k_cache.stride()[:3]) and k_cache.data_ptr() % 8 == 0)))

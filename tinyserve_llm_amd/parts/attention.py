@@ -67,12 +67,12 @@ class Attention(Mixer):
         by16 = self.qkv_rope_packed
         if d is not None and d.prepared is not None:     # the norm's first half is done: its operand, then a scale per row
             rows = d.prepared.operand
-            if not hip.qkv_rope_fuses(rows, self.qkv, self.head_dim, k_store):
+            if not hip.qkv_rope_fuses(rows, self.qkv, self.head_dim, k_store, table=table):
                 return None
             return hip.qkv_rope_store(rows, self.qkv, table, positions, slots, k_store, v_store, self.num_heads,
                                       self.num_kv_heads, self.head_dim, eps=d.eps, packed=by16, squares=d.prepared.squares)[0]
         rows = d.x if d is not None else x
-        if not (rows.is_cuda and hip.qkv_rope_fuses(rows, self.qkv, self.head_dim, k_store)):
+        if not (rows.is_cuda and hip.qkv_rope_fuses(rows, self.qkv, self.head_dim, k_store, table=table)):
             return None
         if d is not None and not (hip.qkv_rope_fuses(rows, self.qkv, self.head_dim, k_store, norm=True)
                                   and d.weight.dtype == torch.bfloat16

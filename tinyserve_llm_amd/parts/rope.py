@@ -33,12 +33,20 @@ def inverse_frequencies(head_dim: int, theta: float, scaling: dict | None, max_p
 class Rope(PositionEncoding):
     graph_safe = True
 
-    def __init__(self, head_dim: int, max_position: int, theta: float, scaling: dict | None = None) -> None:
+    def __init__(self, head_dim: int, max_position: int, theta: float, scaling: dict | None = None,
+                 rotary_dim: int | None = None) -> None:
+        """`rotary_dim` (even, up to head_dim; default: all of it): the leading dimensions of a head
+        that turn, dimension j with j + rotary_dim / 2; the table is that wide and the rest of a head
+        passes unchanged (the Llama models turn whole heads)."""
+        rotary_dim = head_dim if rotary_dim is None else rotary_dim
+        if rotary_dim % 2 or not 2 <= rotary_dim <= head_dim:
+            raise ValueError(f"rotary_dim {rotary_dim}: an even number from 2 to head_dim {head_dim}")
         self.head_dim = head_dim
+        self.rotary_dim = rotary_dim
         self.max_position = max_position
         self.theta = theta
         self.scaling = scaling
-        self.inv_freq = inverse_frequencies(head_dim, theta, scaling, max_position)
+        self.inv_freq = inverse_frequencies(rotary_dim, theta, scaling, max_position)
         self.cos_sin: torch.Tensor | None = None
 
     def host_table(self) -> torch.Tensor:
