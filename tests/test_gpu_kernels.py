@@ -1115,6 +1115,59 @@ def test_wide_product_for_a_few_dozen_rows(m, n, k):
         hip().gemm_rows64(torch.cat([x, x, x, x])[:65].contiguous(), packed)
 
 
+@pytest.mark.parametrize("m", [17, 40, 64])
+@pytest.mark.parametrize("n,k,slices", [(2048, 2048, 4), (2048, 8192, 8), (3072, 3072, 6), (192, 1536, 3), (4096, 14336, 4),
+                                        (2048, 512, 1)])
+def test_narrow_product_in_slices_of_its_reduction(m, n, k, slices):
+    """The shared-x kernel with the reduction cut into slices and the kernel that adds the parts, against
+    64-bit products: the plain product, and the product finished into the residual sum, the next
+    operand and the rows' sums of squares. A row's result does not depend on the rows beside it."""
+    g = gen(m + n + k)
+    x = torch.randn(m, k, generator=g).bfloat16().to(dev())
+    w = (torch.randn(n, k, generator=g) * k ** -0.5).bfloat16().to(dev())
+    packed = hip().pack_weight(w)
+    want = x.double().cpu() @ w.double().cpu().T
+    y = hip().gemm_rows64_sliced(x, packed, slices)
+    assert y.dtype == torch.bfloat16 and y.shape == (m, n)
+    torch.testing.assert_close(y.double().cpu(), want, rtol=1e-2, atol=1e-2 * float(want.abs().max()))
+    assert torch.equal(hip().gemm_rows64_sliced(x[m - 1:].contiguous(), packed, slices)[0], y[m - 1])
+    res = torch.randn(m, n, generator=g).bfloat16().to(dev())
+    nw = (1 + 0.1 * torch.randn(n, generator=g)).bfloat16().to(dev())
+    for residual in (res, None):
+        prepared = hip().gemm_rows64_sliced(x, packed, slices, next_norm=(residual, nw))
+        t = y.double().cpu() + (0 if residual is None else residual.double().cpu())        # T(y) + res
+        assert torch.equal(prepared.summed.cpu(), t.float().bfloat16())
+        assert torch.equal(prepared.operand.cpu(), (t.float() * nw.float().cpu()).bfloat16())
+        assert prepared.squares.shape == (m, 1), "a row's sum of squares comes whole"
+        torch.testing.assert_close(prepared.squares.double().cpu(), t.pow(2).sum(1, keepdim=True), rtol=1e-5, atol=1e-6)
+    with pytest.raises(hip().KernelError):
+        hip().gemm_rows64_sliced(x, packed, slices * 2 if k % (1024 * slices) else 5 if (k // 512) % 5 else 7)
+    with pytest.raises(hip().KernelError):
+        hip().gemm_rows64_sliced(torch.cat([x] * 4)[:65].contiguous(), packed, slices)
+
+
+def test_which_narrow_products_are_cut_into_slices():
+    from tinyserve_llm_amd.parts.linear import linear, streaming_copy, NormRequest, DeferredNorm
+    assert hip().rows64_slices(64, 2048, 2048) == 4 and hip().rows64_slices(33, 2048, 8192) == 8
+    assert hip().rows64_slices(48, 3072, 3072) == 6 and hip().rows64_slices(64, 4096, 14336) == 4
+    assert hip().rows64_slices(16, 2048, 8192) == 0 and hip().rows64_slices(65, 2048, 8192) == 0
+    assert hip().rows64_slices(64, 16384, 2048) == 0, "a wide weight gives every compute unit a workgroup as it is"
+    assert hip().rows64_slices(64, 2048, 2304) == 0 and hip().rows64_slices(64, 2000, 2048) == 0
+    g = gen(5)
+    for m, n, k in ((64, 2048, 8192), (40, 2048, 2048), (24, 2048, 8192)):
+        x = torch.randn(m, k, generator=g).bfloat16().to(dev())
+        w = (torch.randn(n, k, generator=g) * k ** -0.5).bfloat16().to(dev())
+        copies = streaming_copy(w)
+        assert copies is not None and copies.by16 is not None
+        y = linear(x, w, packed=copies)
+        assert torch.equal(y, hip().gemm_rows64_sliced(x, copies.by16, hip().rows64_slices(m, n, k))), "the parts' projections take this path"
+        nw = torch.ones(n, dtype=torch.bfloat16, device=dev())
+        d = linear(x, w, packed=copies, then=NormRequest(nw, 1e-5, None))
+        assert isinstance(d, DeferredNorm) and d.prepared is not None and torch.equal(d.prepared.summed, y)
+        d = linear(x, w, then=NormRequest(nw, 1e-5, None))
+        assert d.prepared is None, "without the packed copy the library multiplies and the norm is a kernel of its own"
+
+
 def test_fused_projection_reads_the_packed_copy_to_the_same_result():
     g = gen(77)
     nh, nkv, hd, K, M, page = 6, 2, 64, 1024, 7, 16

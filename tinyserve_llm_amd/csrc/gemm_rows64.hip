@@ -18,6 +18,15 @@
 // staging waves and costs more than the norm kernel it saves: 37 µs against 21 + 7 at 64 rows.)
 // W comes as the 16-row packed copy ([N / 16 tiles][K / 32 steps][64 lanes][8]); K is a multiple of
 // 1,024. A row of x meets W's k in ascending order in one accumulator, whatever the other rows are.
+//
+// A narrow W (the o and down projections: 2,048 to 4,096 rows) has too few 64-row tiles to give every
+// compute unit a workgroup, so its reduction may be cut into slices (the grid's second dimension): the
+// workgroup of slice s multiplies k = s K / slices .. (s + 1) K / slices and leaves its 32-bit sums in
+// part s of y [slices][M][N]. rows64_finish_kernel then adds a column's parts in ascending order
+// (always the same order: the result does not depend on which workgroup finished first) and either
+// stores the product or finishes it into the residual sum and the norm that follow it, as EPI_NEXT of
+// gemm_skinny.hip does: the new residual, the next projection's operand and the rows' sums of squares
+// (whole: a workgroup of that kernel takes a row).
 #include <type_traits>
 #include "skinny_ops.h"
 
@@ -38,6 +47,7 @@ struct Rows64Args {
   const float* ssq_in;
   int ssq_parts;
   float eps;
+  int slices;            // the reduction in this many slices (gridDim.y); more than one: y is float [slices][M][ldy]
 };
 
 template <bool GLU, typename OUT>
@@ -45,10 +55,11 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
   // x as the B operands of the matrix instruction: [buffer][step][block of 16 rows][lane], lane r + 16 g
   // holding k = 8 g .. 8 g + 7 of row r
   __shared__ uint4 xs[2][R64_CHUNK_STEPS][4][TS_WAVE];
-  __shared__ float row_scale[64];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TS_WAVE), lane = threadIdx.x & (TS_WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
-  const int nsteps = a.K / SK_KSTEP, nchunks = nsteps / R64_CHUNK_STEPS;   // (a multiple of 4)
+  const int slice = blockIdx.y;
+  const int nsteps = a.K / SK_KSTEP / a.slices, nchunks = nsteps / R64_CHUNK_STEPS;   // (steps: a multiple of the ring, chunks: even)
+  const int64_t kfirst = (int64_t)slice * nsteps * SK_KSTEP;                  // the slice's first k
 
   if (wave >= 4) {
     // ---- staging waves: wave sw brings steps 2 sw and 2 sw + 1 of every chunk, all four blocks of
@@ -60,7 +71,7 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       ok[b] = 16 * b + r < a.M;                          // rows past M read row 0 and count as zeros
-      xoff[b] = (int64_t)(ok[b] ? 16 * b + r : 0) * a.ldx + 8 * g;
+      xoff[b] = (int64_t)(ok[b] ? 16 * b + r : 0) * a.ldx + kfirst + 8 * g;
     }
     auto ask = [&](int c, uint4 (&t)[R64_STAGE_STEPS][4]) {
       const int k0 = (c * R64_CHUNK_STEPS + R64_STAGE_STEPS * sw) * SK_KSTEP;   // first k of this wave's steps
@@ -77,25 +88,6 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
     };
     uint4 A[R64_STAGE_STEPS][4], B[R64_STAGE_STEPS][4];
     ask(0, A);
-    // the rows' scales, rows 16 sw .. 16 sw + 15 in this wave: a lane every 64th part (all sixteen rows' loads
-    // under way together), then the lanes in a fixed tree
-    if (a.ssq_in) {
-      float sums[16];
-#pragma unroll
-      for (int i = 0; i < 16; ++i) sums[i] = 0.f;
-      for (int q = lane; q < a.ssq_parts; q += TS_WAVE) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int m = 16 * sw + i;
-          sums[i] += m < a.M ? a.ssq_in[(int64_t)m * a.ssq_parts + q] : 0.f;
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const float total = wave_sum(sums[i]);
-        if (lane == 0) row_scale[16 * sw + i] = 1.0f / sqrtf(total / (float)a.K + a.eps);
-      }
-    }
     for (int c = 0; c < nchunks; c += 2) {
       ask(c + 1, B);
       put(c, A);
@@ -111,7 +103,7 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
 
   // ---- compute waves
   const int tile = GLU ? (wave < 2 ? 2 * blockIdx.x + wave : a.N / 32 + 2 * blockIdx.x + (wave - 2)) : 4 * blockIdx.x + wave;
-  const bf16_t* wp = a.w16 + ((int64_t)tile * nsteps * 64 + lane) * 8;      // step s at wp + 512 s
+  const bf16_t* wp = a.w16 + (((int64_t)tile * a.slices + slice) * nsteps * 64 + lane) * 8;      // the slice's step s at wp + 512 s
   uint4 wr[R64_RING];
   // (in this order and no other: the ring is used oldest first, and a wait is for the oldest load only if the
   // compiler sees the first loads come in the order of their use)
@@ -123,6 +115,22 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
   float4_t acc[4];
 #pragma unroll
   for (int b = 0; b < 4; ++b) acc[b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+  // the scales of this lane's rows: the parts of a row's sum of squares in ascending order. The wait is for
+  // loads that come back behind the ring's first turn, which the first products wait for anyway (in the
+  // staging waves a wait for the parts held the second chunk's request back by a trip to memory).
+  float scale[4] = {1.f, 1.f, 1.f, 1.f};
+  if (a.ssq_in) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int m = 16 * b + r;
+      float total = 0.f;
+      if (m < a.M) {
+        total = a.ssq_in[(int64_t)m * a.ssq_parts];
+        for (int q = 1; q < a.ssq_parts; ++q) total += a.ssq_in[(int64_t)m * a.ssq_parts + q];
+      }
+      scale[b] = 1.0f / sqrtf(total / (float)a.K + a.eps);
+    }
+  }
   __syncthreads();              // chunk 0 is there
   // a turn of the ring at a time, each register asked for again once it has been used; the last turn asks for nothing
   auto ring = [&](int base, auto more) {
@@ -170,7 +178,7 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
     __syncthreads();
     if (wave >= 2) return;
   }
-  OUT* y = (OUT*)a.y;
+  OUT* y = (OUT*)a.y + (int64_t)slice * a.M * a.ldy;
   const int n0 = GLU ? (2 * blockIdx.x + wave) * 16 + 4 * g : tile * 16 + 4 * g;
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
@@ -178,11 +186,8 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
     if (m >= a.M) continue;
     float4_t u = {0.f, 0.f, 0.f, 0.f};
     if (GLU) u = ex[(wave * 4 + b) * TS_WAVE + lane];
-    if (a.ssq_in) {                                  // (the same for every thread)
-      const float scale = row_scale[m];
-      acc[b] *= scale;
-      u *= scale;
-    }
+    acc[b] *= scale[b];
+    u *= scale[b];
 #pragma unroll
     for (int j = 0; j < 4; ++j) Num<OUT>::st(y + (int64_t)m * a.ldy + n0 + j, GLU ? sk_silu(acc[b][j]) * u[j] : acc[b][j]);
   }
@@ -190,8 +195,13 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
 
 template <bool GLU, typename OUT>
 static int r64_launch(const Rows64Args& a, hipStream_t stream) {
-  gemm_rows64_kernel<GLU, OUT><<<a.N / 64, 512, 0, stream>>>(a);   // 64 rows of W per workgroup
+  gemm_rows64_kernel<GLU, OUT><<<dim3(a.N / 64, a.slices), 512, 0, stream>>>(a);   // 64 rows of W per workgroup
   return ts_check_launch();
+}
+
+static bool r64_operands_ok(const void* x, const void* w16, int M, int N, int K, int64_t ldx) {
+  if (M > 64 || K <= 0 || ldx < K || (ldx % 8) || !x || !w16) return false;
+  return !((((uintptr_t)x) | ((uintptr_t)w16)) & 15);
 }
 
 // x [M <= 64, K] (row stride ldx), w16: W [N, K] as its 16-row packed copy, y [M, N] or, with glu, [M, N / 2]
@@ -200,13 +210,114 @@ static int r64_launch(const Rows64Args& a, hipStream_t stream) {
 extern "C" int ts_gemm_rows64_bf16(void* y, const void* x, const void* w16, int M, int N, int K, int64_t ldx, int64_t ldy,
                                    int glu, int out_f32, const void* ssq_in, int ssq_parts, float eps, hipStream_t stream) {
   if (M <= 0 || N <= 0) return TS_OK;
-  if (M > 64 || N % (glu ? 128 : 64) || K <= 0 || K % 1024 || ldx < K || (ldx % 8) || !y || !x || !w16) return TS_BAD_SHAPE;
+  if (N % (glu ? 128 : 64) || K % 1024 || !y || !r64_operands_ok(x, w16, M, N, K, ldx)) return TS_BAD_SHAPE;
   if (ldy < (glu ? N / 2 : N) || (((uintptr_t)y) & (out_f32 ? 3 : 1))) return TS_BAD_SHAPE;
-  if ((((uintptr_t)x) | ((uintptr_t)w16)) & 15) return TS_BAD_SHAPE;
   if (glu && out_f32) return TS_BAD_SHAPE;
   if (ssq_in && (ssq_parts <= 0 || (((uintptr_t)ssq_in) & 3))) return TS_BAD_SHAPE;
-  Rows64Args a = {(const bf16_t*)x, (const bf16_t*)w16, y, M, N, K, ldx, ldy, (const float*)ssq_in, ssq_parts, eps};
+  Rows64Args a = {(const bf16_t*)x, (const bf16_t*)w16, y, M, N, K, ldx, ldy, (const float*)ssq_in, ssq_parts, eps, 1};
   if (glu) return r64_launch<true, bf16_t>(a, stream);
   if (out_f32) return r64_launch<false, float>(a, stream);
   return r64_launch<false, bf16_t>(a, stream);
+}
+
+// ---- a product in slices of its reduction, and what finishes it
+
+#define R64_FINISH_THREADS 1024   // a workgroup of the finishing kernel takes a row, a thread four neighbouring columns at a time
+
+struct Rows64FinishArgs {
+  const float* parts;    // [slices][M][N]
+  int slices, M, N;
+  bf16_t* y;             // the product [M, N] (not NEXT)
+  // NEXT: t = T(y) + res; res_out = T(t), op = T(t * nw), ssq_out [M] the rows' sums of t^2
+  const bf16_t* res;     // [M, N] or null
+  const bf16_t* nw;      // [N]
+  bf16_t* res_out;
+  bf16_t* op;
+  float* ssq_out;
+};
+
+// A workgroup per row: a thread adds the parts of four neighbouring columns, first slice first, then of the
+// four columns 4,096 further on, and so on. The row's sum of squares: a thread's own columns in ascending
+// order, the lanes of a wave in a fixed tree, the waves in ascending order.
+template <bool NEXT>
+__global__ void __launch_bounds__(R64_FINISH_THREADS) rows64_finish_kernel(const Rows64FinishArgs a) {
+  __shared__ float wave_sq[R64_FINISH_THREADS / TS_WAVE];
+  const int m = blockIdx.x;
+  float sq = 0.f;
+  for (int n = 4 * threadIdx.x; n < a.N; n += 4 * blockDim.x) {      // (N is a multiple of 64)
+    const int64_t at = (int64_t)m * a.N + n;
+    uint2 res = make_uint2(0, 0), nw = make_uint2(0, 0);
+    if (NEXT) {
+      nw = *(const uint2*)(a.nw + n);
+      if (a.res) res = *(const uint2*)(a.res + at);
+    }
+    // four slices' parts asked for together, added first slice first
+    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int s0 = 0; s0 < a.slices; s0 += 4) {
+      float4 p[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        p[j] = s0 + j < a.slices ? *(const float4*)(a.parts + (int64_t)(s0 + j) * a.M * a.N + at) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (s0 + j == 0) { sum = p[0]; continue; }        // (not 0 + p: a sum of -0 stays -0)
+        if (s0 + j < a.slices) { sum.x += p[j].x; sum.y += p[j].y; sum.z += p[j].z; sum.w += p[j].w; }
+      }
+    }
+    const float s4[4] = {sum.x, sum.y, sum.z, sum.w};
+    if (!NEXT) {
+      *(uint2*)(a.y + at) = make_uint2(sk_round(s4[0]) | (sk_round(s4[1]) << 16), sk_round(s4[2]) | (sk_round(s4[3]) << 16));
+      continue;
+    }
+    const uint32_t rw[2] = {res.x, res.y}, ww[2] = {nw.x, nw.y};
+    float tv[4], ov[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {                           // (the low half of a word is the even column)
+      const float rj = __uint_as_float((rw[j >> 1] >> (16 * (j & 1))) << 16);
+      const float nj = __uint_as_float((ww[j >> 1] >> (16 * (j & 1))) << 16);
+      const float t = __uint_as_float(sk_round(s4[j]) << 16) + rj;
+      tv[j] = t;
+      ov[j] = t * nj;
+      sq = fmaf(t, t, sq);
+    }
+    *(uint2*)(a.res_out + at) = make_uint2(sk_round(tv[0]) | (sk_round(tv[1]) << 16), sk_round(tv[2]) | (sk_round(tv[3]) << 16));
+    *(uint2*)(a.op + at) = make_uint2(sk_round(ov[0]) | (sk_round(ov[1]) << 16), sk_round(ov[2]) | (sk_round(ov[3]) << 16));
+  }
+  if (!NEXT) return;
+  sq = wave_sum(sq);
+  if ((threadIdx.x & (TS_WAVE - 1)) == 0) wave_sq[threadIdx.x / TS_WAVE] = sq;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < R64_FINISH_THREADS / TS_WAVE; ++w) total += w < (int)blockDim.x / TS_WAVE ? wave_sq[w] : 0.f;
+    a.ssq_out[m] = total;
+  }
+}
+
+// The same product with the reduction cut into `slices` (K / slices a multiple of 512), for a W of few rows:
+// parts [slices][M][N] float is scratch that the call fills and reads. With next_nw the product is not stored:
+// next_res_out, next_op [M, N] and ssq_out [M] (the rows' whole sums of squares: one part) are (next_res [M, N] or null is
+// added first); without it y [M, N] bfloat16 is.
+extern "C" int ts_gemm_rows64_sliced_bf16(void* y, void* parts, const void* x, const void* w16, int M, int N, int K, int64_t ldx,
+                                          int slices, const void* next_res, const void* next_nw, void* next_res_out,
+                                          void* next_op, void* ssq_out, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return TS_OK;
+  if (N % 64 || slices < 1 || slices > 64 || K % (512 * slices) || !parts || !r64_operands_ok(x, w16, M, N, K, ldx)) return TS_BAD_SHAPE;
+  if (((uintptr_t)parts) & 15) return TS_BAD_SHAPE;
+  Rows64FinishArgs f = {(const float*)parts, slices, M, N, (bf16_t*)y, (const bf16_t*)next_res, (const bf16_t*)next_nw,
+                        (bf16_t*)next_res_out, (bf16_t*)next_op, (float*)ssq_out};
+  if (next_nw) {
+    if (!next_res_out || !next_op || !ssq_out || (((uintptr_t)ssq_out) & 3)) return TS_BAD_SHAPE;
+    if ((((uintptr_t)next_res) | ((uintptr_t)next_nw) | ((uintptr_t)next_res_out) | ((uintptr_t)next_op)) & 7) return TS_BAD_SHAPE;
+  } else if (!y || (((uintptr_t)y) & 7)) {
+    return TS_BAD_SHAPE;
+  }
+  Rows64Args a = {(const bf16_t*)x, (const bf16_t*)w16, parts, M, N, K, ldx, (int64_t)N, nullptr, 0, 0.f, slices};
+  const int rc = r64_launch<false, float>(a, stream);
+  if (rc != TS_OK) return rc;
+  const int threads = N / 4 >= R64_FINISH_THREADS ? R64_FINISH_THREADS : (N / 4 + TS_WAVE - 1) / TS_WAVE * TS_WAVE;
+  if (next_nw) rows64_finish_kernel<true><<<M, threads, 0, stream>>>(f);
+  else rows64_finish_kernel<false><<<M, threads, 0, stream>>>(f);
+  return ts_check_launch();
 }

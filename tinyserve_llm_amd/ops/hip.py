@@ -66,6 +66,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p, i, p, p, p, p, p, p],
         "ts_gemm_skinny8_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p, p, p, p, p, p],
         "ts_gemm_rows64_bf16": [p, p, p, i, i, i, i64, i64, i, i, p, i, f, p],
+        "ts_gemm_rows64_sliced_bf16": [p, p, p, p, i, i, i, i64, i, p, p, p, p, p, p],
         "ts_skinny_tiles": [i, i, i],
         "ts_peak_read": [p, ctypes.c_size_t, p, i, p],
         "ts_peak_mfma": [p, i, i, p],
@@ -910,6 +911,51 @@ def gemm_rows64(x: torch.Tensor, packed: torch.Tensor, out_dtype: torch.dtype = 
     return out
 
 
+ROWS64_SLICE_K = 512           # a slice of the reduction is a multiple of this (one turn of a compute wave's ring of W)
+ROWS64_SLICED_MIN_ROWS = 17    # fewer rows: the 16-row weight-streaming kernel, whose workgroups reduce over all of k themselves
+ROWS64_WORKGROUPS = 192        # workgroups from which the chip's 256 compute units count as filled
+
+
+def rows64_slices(rows: int, n: int, k: int) -> int:
+    """Slices of the reduction that `gemm_rows64_sliced` cuts a product of `rows` rows of x against a
+    narrow weight [n, k] into: the fewest that give every compute unit a workgroup of 64 rows of W
+    (else the most the reduction allows); 0 where the kernel does not serve the shape or the weight
+    is wide enough for `gemm_rows64` itself."""
+    if not (ROWS64_SLICED_MIN_ROWS <= rows <= ROWS64_MAX_ROWS) or n % 64 or n >= ROWS64_MIN_WIDTH or k % ROWS64_SLICE_K:
+        return 0
+    fits = [s for s in range(1, 17) if (k // ROWS64_SLICE_K) % s == 0]
+    enough = [s for s in fits if (n // 64) * s >= ROWS64_WORKGROUPS]
+    return enough[0] if enough else fits[-1]
+
+
+def gemm_rows64_sliced(x: torch.Tensor, packed: torch.Tensor, slices: int, next_norm=None) -> "torch.Tensor | PreparedNorm":
+    """bfloat16 x [M <= 64, K] · W [N, K]^T for a narrow W given as `packed` = pack_weight(W): the
+    shared-x kernel with the reduction in `slices` slices (K / slices a multiple of 512), whose 32-bit
+    parts a second kernel adds in ascending order. With `next_norm` = (residual or None, weight of the
+    norm that follows) the product is not stored: a `PreparedNorm` comes back."""
+    _gpu(x, packed)
+    _need(x.dtype == torch.bfloat16 and packed.dtype == torch.bfloat16 and x.dim() == 2 and packed.dim() == 4
+          and packed.shape[2:] == (64, 8) and packed.is_contiguous(), "gemm_rows64_sliced takes bfloat16 x [M, K] and pack_weight(W)")
+    M, K = x.shape
+    N = packed.shape[0] * 16
+    _need(packed.shape[1] * 32 == K, f"the packed copy is of a weight over {packed.shape[1] * 32}, x is over {K}")
+    _need(1 <= M <= ROWS64_MAX_ROWS and N % 64 == 0 and 1 <= slices <= 64 and K % (ROWS64_SLICE_K * slices) == 0,
+          f"gemm_rows64_sliced takes up to {ROWS64_MAX_ROWS} rows, N in steps of 64 and slices of K that are multiples of "
+          f"{ROWS64_SLICE_K}, not {M} x {K} against {N} in {slices}")
+    _need(x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0, "rows of x must be dense and 16-byte aligned")
+    parts = torch.empty((slices, M, N), dtype=torch.float32, device=x.device)
+    if next_norm is not None:
+        prepared, residual, nw = _next_norm_outputs(x, N, 1, next_norm)
+        _run("gemm_rows64_sliced", library().ts_gemm_rows64_sliced_bf16(
+            None, _ptr(parts), _ptr(x), _ptr(packed), M, N, K, x.stride(0), slices, _ptr(residual), _ptr(nw),
+            _ptr(prepared.summed), _ptr(prepared.operand), _ptr(prepared.squares), _stream()))
+        return prepared
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    _run("gemm_rows64_sliced", library().ts_gemm_rows64_sliced_bf16(
+        _ptr(out), _ptr(parts), _ptr(x), _ptr(packed), M, N, K, x.stride(0), slices, None, None, None, None, None, _stream()))
+    return out
+
+
 def qkv_rope_max_rows(k: int, norm: bool = False) -> int:
     """Most rows of x that `qkv_rope_store` takes over a reduction of `k`, with or without the norm
     on the way in; 0 if it does not take the reduction at all."""
@@ -1043,13 +1089,20 @@ class StreamingCopies:
         return sum(t.numel() * t.element_size() for t in (self.by16, self.by8) if t is not None)
 
 
-def next_norm_fuses(x: torch.Tensor, weight: torch.Tensor) -> bool:
+def next_norm_fuses(x: torch.Tensor, weight: torch.Tensor, packed: "StreamingCopies | None" = None) -> bool:
     """Whether `linear_bf16(x, weight, next_norm=...)` has a kernel that leaves a `PreparedNorm`."""
     if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.is_cuda and x.dim() == 2 and weight.dim() == 2
             and x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
         return False
     rows, (n, k) = x.shape[0], weight.shape
-    return skinny8_takes(rows, n, k) or _skinny_serves(rows, n, k)
+    return skinny8_takes(rows, n, k) or _skinny_serves(rows, n, k) or _sliced_serves(rows, n, k, packed) > 0
+
+
+def _sliced_serves(rows: int, n: int, k: int, packed: "StreamingCopies | None") -> int:
+    """The slices in which `linear_bf16` gives a product to `gemm_rows64_sliced` (0: it does not)."""
+    if packed is None or packed.by16 is None or skinny8_takes(rows, n, k) or _skinny_serves(rows, n, k):
+        return 0
+    return rows64_slices(rows, n, k)
 
 
 def _skinny_serves(rows: int, n: int, k: int) -> bool:
@@ -1075,6 +1128,9 @@ def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
         return gemm_skinny8(x, weight, out_dtype, None if packed is None else packed.by8, next_norm=next_norm)
     if streams and _skinny_serves(x.shape[0], weight.shape[0], x.shape[1]):
         return gemm_skinny(x, weight, out_dtype, packed=None if packed is None else packed.by16, next_norm=next_norm)[0]
+    slices = _sliced_serves(x.shape[0], weight.shape[0], x.shape[1], packed) if streams and out_dtype == torch.bfloat16 else 0
+    if slices:
+        return gemm_rows64_sliced(x, packed.by16, slices, next_norm=next_norm)
     _need(next_norm is None, "no kernel leaves a prepared norm for this product (ask next_norm_fuses first)")
     # (float32: the 32-bit sums themselves, as the weight-streaming kernel gives them for few rows, so
     # that a row's logits are rounded the same way whatever the number of rows beside it)

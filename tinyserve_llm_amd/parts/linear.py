@@ -70,7 +70,7 @@ def streaming_copy(weight: torch.Tensor) -> hip.StreamingCopies | None:
     if not (weight.is_cuda and weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous()):
         return None
     n, k = weight.shape
-    by16 = hip.pack_weight(weight) if hip.skinny_takes(1, k) and k <= 4096 else None
+    by16 = hip.pack_weight(weight) if (hip.skinny_takes(1, k) and k <= 4096) or hip.rows64_slices(hip.ROWS64_MAX_ROWS, n, k) else None
     by8 = hip.pack_weight8(weight) if hip.skinny8_takes(1, n, k) and n % 8 == 0 else None     # (one row: the widest reach of that form)
     return hip.StreamingCopies(by16, by8) if by16 is not None or by8 is not None else None
 
@@ -88,7 +88,7 @@ def linear(x: torch.Tensor | DeferredNorm, weight: torch.Tensor, out_dtype: torc
         residual = then.residual()
         if isinstance(x, DeferredNorm):
             x = x.materialize()
-        if (out_dtype in (None, torch.bfloat16) and then.weight.dtype == torch.bfloat16 and hip.next_norm_fuses(x, weight)
+        if (out_dtype in (None, torch.bfloat16) and then.weight.dtype == torch.bfloat16 and hip.next_norm_fuses(x, weight, packed)
                 and (residual is None or (residual.is_contiguous() and residual.dtype == torch.bfloat16))):
             prepared = hip.linear_bf16(x, weight, torch.bfloat16, packed, next_norm=(residual, then.weight))
             return DeferredNorm(None, None, then.weight, then.eps, prepared)
