@@ -1115,7 +1115,7 @@ def test_wide_product_for_a_few_dozen_rows(m, n, k):
         hip().gemm_rows64(torch.cat([x, x, x, x])[:65].contiguous(), packed)
 
 
-@pytest.mark.parametrize("m", [17, 40, 64])
+@pytest.mark.parametrize("m", [5, 17, 40, 64])
 @pytest.mark.parametrize("n,k,slices", [(2048, 2048, 4), (2048, 8192, 8), (3072, 3072, 6), (192, 1536, 3), (4096, 14336, 4),
                                         (2048, 512, 1)])
 def test_narrow_product_in_slices_of_its_reduction(m, n, k, slices):
@@ -1143,18 +1143,18 @@ def test_narrow_product_in_slices_of_its_reduction(m, n, k, slices):
     with pytest.raises(hip().KernelError):
         hip().gemm_rows64_sliced(x, packed, slices * 2 if k % (1024 * slices) else 5 if (k // 512) % 5 else 7)
     with pytest.raises(hip().KernelError):
-        hip().gemm_rows64_sliced(torch.cat([x] * 4)[:65].contiguous(), packed, slices)
+        hip().gemm_rows64_sliced(x[:1].expand(65, k).contiguous(), packed, slices)
 
 
 def test_which_narrow_products_are_cut_into_slices():
     from tinyserve_llm_amd.parts.linear import linear, streaming_copy, NormRequest, DeferredNorm
     assert hip().rows64_slices(64, 2048, 2048) == 4 and hip().rows64_slices(33, 2048, 8192) == 8
     assert hip().rows64_slices(48, 3072, 3072) == 6 and hip().rows64_slices(64, 4096, 14336) == 4
-    assert hip().rows64_slices(16, 2048, 8192) == 0 and hip().rows64_slices(65, 2048, 8192) == 0
+    assert hip().rows64_slices(4, 2048, 8192) == 0 and hip().rows64_slices(65, 2048, 8192) == 0 and hip().rows64_slices(9, 2048, 8192) == 8
     assert hip().rows64_slices(64, 16384, 2048) == 0, "a wide weight gives every compute unit a workgroup as it is"
     assert hip().rows64_slices(64, 2048, 2304) == 0 and hip().rows64_slices(64, 2000, 2048) == 0
     g = gen(5)
-    for m, n, k in ((64, 2048, 8192), (40, 2048, 2048), (24, 2048, 8192)):
+    for m, n, k in ((64, 2048, 8192), (40, 2048, 2048), (24, 2048, 8192), (9, 2048, 8192), (8, 3072, 8192)):
         x = torch.randn(m, k, generator=g).bfloat16().to(dev())
         w = (torch.randn(n, k, generator=g) * k ** -0.5).bfloat16().to(dev())
         copies = streaming_copy(w)

@@ -23,8 +23,9 @@ LENGTHS = {"A": [5, 17, 33, 100], "B": [1, 40, 70, 129]}
 
 # float32 engine against the float64 oracle: only the engine's own 32-bit rounding separates them.
 # bfloat16 engine against the float64 oracle on bfloat16-rounded weights: activations are rounded
-# to 8 bits of mantissa a few dozen times on the way to a logit.
-TOL = {"float32": dict(atol=5e-6, rtol=1e-5), "bfloat16": dict(atol=1.5e-2, rtol=2e-2)}
+# to 8 bits of mantissa a few dozen times on the way to a logit. The worst logit is off by 2.6e-3 to
+# 4.9e-3 in every way of feeding (the logits' spread is 0.16); the bound is twice that.
+TOL = {"float32": dict(atol=5e-6, rtol=1e-5), "bfloat16": dict(atol=1e-2, rtol=0.0)}
 
 
 @pytest.fixture(scope="module", params=["A", "B"])

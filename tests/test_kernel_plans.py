@@ -106,3 +106,22 @@ def test_which_kernel_takes_a_projection_of_few_rows():
     assert hip.skinny_fuses(16, 2048, True, True) and not hip.skinny_fuses(17, 2048, True, True)
     assert hip.skinny_fuses(64, 2048, False, True) and not hip.skinny_fuses(65, 2048, False, True)
     assert not hip.skinny_fuses(40, 4096, False, True)
+
+
+def test_which_narrow_products_have_their_reduction_cut_into_slices():
+    """The shared-x kernel with the reduction in slices: for weights too narrow to give every compute
+    unit a workgroup of 64 rows; the fewest slices (multiples of 512 of k) that reach 192 workgroups."""
+    assert hip.rows64_slices(64, 2048, 2048) == 4 and hip.rows64_slices(33, 2048, 8192) == 8 and hip.rows64_slices(9, 2048, 8192) == 8
+    assert hip.rows64_slices(48, 3072, 3072) == 6 and hip.rows64_slices(8, 3072, 8192) == 4 and hip.rows64_slices(64, 4096, 14336) == 4
+    for rows, n, k in ((4, 2048, 8192), (65, 2048, 8192), (64, 16384, 2048), (64, 2048, 2304), (64, 2000, 2048)):
+        assert hip.rows64_slices(rows, n, k) == 0
+    for n, k in ((64, 512), (2048, 8192), (3072, 3072), (4096, 14336), (4096, 4096)):
+        s = hip.rows64_slices(40, n, k)
+        assert 1 <= s <= 16 and k % (512 * s) == 0
+        fewer = [t for t in range(1, s) if (k // 512) % t == 0]
+        assert all((n // 64) * t < 192 for t in fewer), "a smaller number of slices would have filled the chip"
+    # where the weight-streaming kernels serve a shape they come first: the o projection of up to 32 rows
+    copies = hip.StreamingCopies(by16=object())
+    assert hip._sliced_serves(32, 2048, 2048, copies) == 0 and hip._sliced_serves(33, 2048, 2048, copies) == 4
+    assert hip._sliced_serves(8, 2048, 8192, copies) == 0 and hip._sliced_serves(9, 2048, 8192, copies) == 8
+    assert hip._sliced_serves(40, 2048, 8192, None) == 0, "no packed copy: the library"

@@ -912,7 +912,7 @@ def gemm_rows64(x: torch.Tensor, packed: torch.Tensor, out_dtype: torch.dtype = 
 
 
 ROWS64_SLICE_K = 512           # a slice of the reduction is a multiple of this (one turn of a compute wave's ring of W)
-ROWS64_SLICED_MIN_ROWS = 17    # fewer rows: the 16-row weight-streaming kernel, whose workgroups reduce over all of k themselves
+ROWS64_SLICED_MIN_ROWS = 5     # (fewer rows are the 8-row form's at any width; where the weight-streaming kernels serve a shape, they come first)
 ROWS64_WORKGROUPS = 192        # workgroups from which the chip's 256 compute units count as filled
 
 
@@ -920,7 +920,10 @@ def rows64_slices(rows: int, n: int, k: int) -> int:
     """Slices of the reduction that `gemm_rows64_sliced` cuts a product of `rows` rows of x against a
     narrow weight [n, k] into: the fewest that give every compute unit a workgroup of 64 rows of W
     (else the most the reduction allows); 0 where the kernel does not serve the shape or the weight
-    is wide enough for `gemm_rows64` itself."""
+    is wide enough for `gemm_rows64` itself. Measured with the finishing kernel, against the library
+    followed by the norm kernel, for a down projection over 8,192 (14,336 at the widest): 9 rows 12.9
+    against 15.5 µs at a width of 2,048, 15.8 against 18.5 at 3,072, 27.0 against 31.1 at 4,096; 32 rows
+    14.1 against 18.9, 17.3 against 21.6, 27.5 against 38.3; 64 rows 15.5 against 22.0 + 7 at 2,048."""
     if not (ROWS64_SLICED_MIN_ROWS <= rows <= ROWS64_MAX_ROWS) or n % 64 or n >= ROWS64_MIN_WIDTH or k % ROWS64_SLICE_K:
         return 0
     fits = [s for s in range(1, 17) if (k // ROWS64_SLICE_K) % s == 0]
