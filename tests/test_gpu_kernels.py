@@ -905,6 +905,69 @@ def test_fused_projection_rotation_and_cache_write(nh, nkv, hd, K, M, page, norm
     assert torch.equal(q_only, q)
 
 
+@pytest.mark.parametrize("nh,nkv,hd,K,M,page,slices,prepared", [
+    (32, 8, 64, 2048, 64, 256, 4, True), (32, 8, 64, 2048, 33, 16, 4, False), (24, 8, 128, 3072, 20, 32, 3, True),
+    (24, 8, 128, 3072, 40, 32, 3, True), (4, 2, 128, 4096, 64, 16, 2, False),
+    (6, 2, 32, 512, 48, 8, 1, True), (5, 3, 96, 1024, 17, 24, 2, False)])
+def test_projection_in_slices_with_rotation_and_cache_write(nh, nkv, hd, K, M, page, slices, prepared):
+    """The qkv projection with its reduction in slices and the kernel that adds the parts, rotates and
+    writes the cache, against projection then rope_store and against the chain in 64-bit: q, every written
+    slot of k and v, and the slots it must not touch. With `prepared`, x is a prepared norm's operand and
+    the rows' scales multiply the finished sums."""
+    g = gen(nh * 11 + K + M)
+    N = (nh + 2 * nkv) * hd
+    if N % 64:
+        with pytest.raises(hip().KernelError):
+            hip().qkv_rope_store_sliced(torch.zeros(M, K, dtype=torch.bfloat16, device=dev()),
+                                        torch.zeros(-(-N // 16), K // 32, 64, 8, dtype=torch.bfloat16, device=dev()), slices, None,
+                                        torch.zeros(M, dtype=torch.int32, device=dev()), None, None, None, nh, nkv, hd)
+        return
+    x = (torch.randn(M, K, generator=g) * 0.5).bfloat16().to(dev())
+    w = (torch.randn(N, K, generator=g) * K ** -0.5).bfloat16().to(dev())
+    squares = (torch.rand(M, 3, generator=g) * K / 3 + 1).to(dev()) if prepared else None
+    table = torch.randn(64, hd, generator=g).to(dev())
+    positions = torch.randint(0, 64, (M,), generator=g, dtype=torch.int32).to(dev())
+    pages = -(-2 * M // page) + 1
+    perm = torch.randperm(pages * page, generator=g)[:M].to(torch.int32)
+    perm[1] = -1
+    slots = perm.to(dev())
+    def pools():
+        return (torch.full((pages, nkv, page, hd), 7.0, dtype=torch.bfloat16, device=dev()),
+                torch.full((pages, nkv, hd, page), 7.0, dtype=torch.bfloat16, device=dev()))
+    (kp1, vp1), (kp2, vp2) = pools(), pools()
+    scale = torch.rsqrt(squares.double().cpu().sum(1, keepdim=True) / K + 1e-5) if prepared else 1.0
+    y64 = (x.double().cpu() @ w.double().cpu().T) * scale
+    q_want = hip().rope_store(y64.float().bfloat16().to(dev()), table, positions, slots, kp1.permute(0, 2, 1, 3), vp1.permute(0, 3, 1, 2),
+                              nh, nkv, hd)
+    takes = hip().qkv_rope_sliced_slices(x, w, hd, kp2.permute(0, 2, 1, 3), table)
+    assert (takes > 0) == (M >= 33 and not hip().qkv_rope_fuses(x, w, hd, kp2.permute(0, 2, 1, 3))), "where the parts choose this path"
+    q = hip().qkv_rope_store_sliced(x, hip().pack_weight_rope(w, hd), slices, table, positions, slots, kp2.permute(0, 2, 1, 3),
+                                    vp2.permute(0, 3, 1, 2), nh, nkv, hd, eps=1e-5, squares=squares)
+    t64 = y64.view(M, nh + 2 * nkv, hd).clone()
+    cs = table.double().cpu()[positions.cpu().long()]
+    c, sn = cs[:, None, :hd // 2], cs[:, None, hd // 2:]
+    a, b = t64[:, :nh + nkv, :hd // 2].clone(), t64[:, :nh + nkv, hd // 2:].clone()
+    t64[:, :nh + nkv, :hd // 2], t64[:, :nh + nkv, hd // 2:] = a * c - b * sn, b * c + a * sn
+    live = (slots >= 0).cpu()
+    pg, off = (slots.cpu().long() // page)[live], (slots.cpu().long() % page)[live]
+    def written(kp, vp):
+        return kp.double().cpu()[pg, :, off, :], vp.double().cpu()[pg, :, :, off]
+    (k_one, v_one), (k_seq, v_seq) = written(kp2, vp2), written(kp1, vp1)
+    for name, one, seq, truth in (("q", q.double().cpu(), q_want.double().cpu(), t64[:, :nh]),
+                                  ("k", k_one, k_seq, t64[live][:, nh:nh + nkv]), ("v", v_one, v_seq, t64[live][:, nh + nkv:])):
+        e_one, e_seq = (one - truth).abs(), (seq - truth).abs()
+        assert float(e_seq.max()) <= 3e-2 * max(1.0, float(truth.abs().max())), f"{name}: the separate kernels are off"
+        assert float(e_one.max()) <= 1.25 * float(e_seq.max()) + 1e-3, f"{name}: worst error {float(e_one.max())} vs {float(e_seq.max())}"
+        assert float(e_one.pow(2).mean().sqrt()) <= 1.1 * float(e_seq.pow(2).mean().sqrt()) + 1e-4, f"{name}: mean error"
+    assert torch.equal(kp2 == 7.0, kp1 == 7.0) and torch.equal(vp2 == 7.0, vp1 == 7.0), "the same places are written"
+    q_only = hip().qkv_rope_store_sliced(x, hip().pack_weight_rope(w, hd), slices, table, positions, None, None, None, nh, nkv, hd,
+                                         eps=1e-5, squares=squares)
+    assert torch.equal(q_only, q)
+    alone = hip().qkv_rope_store_sliced(x[M - 1:].contiguous(), hip().pack_weight_rope(w, hd), slices, table, positions[M - 1:].contiguous(),
+                                        None, None, None, nh, nkv, hd, eps=1e-5, squares=None if squares is None else squares[M - 1:].contiguous())
+    assert torch.equal(alone[0], q[M - 1]), "a row's result does not depend on the rows beside it"
+
+
 def test_fused_projection_refuses_what_it_cannot_serve():
     x = torch.zeros(65, 256, dtype=torch.bfloat16, device=dev())
     w = torch.zeros(3 * 64, 256, dtype=torch.bfloat16, device=dev())

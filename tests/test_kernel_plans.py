@@ -125,3 +125,5 @@ def test_which_narrow_products_have_their_reduction_cut_into_slices():
     assert hip._sliced_serves(32, 2048, 2048, copies) == 0 and hip._sliced_serves(33, 2048, 2048, copies) == 4
     assert hip._sliced_serves(8, 2048, 8192, copies) == 0 and hip._sliced_serves(9, 2048, 8192, copies) == 8
     assert hip._sliced_serves(40, 2048, 8192, None) == 0, "no packed copy: the library"
+    assert hip._sliced_serves(24, 5120, 3072, copies) == 3 and hip._sliced_serves(24, 5120, 3072, copies, finishing=False) == 0
+    assert hip._sliced_serves(24, 4096, 14336, copies, finishing=False) == 4

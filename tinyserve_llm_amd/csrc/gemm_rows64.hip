@@ -321,3 +321,139 @@ extern "C" int ts_gemm_rows64_sliced_bf16(void* y, void* parts, const void* x, c
   else rows64_finish_kernel<false><<<M, threads, 0, stream>>>(f);
   return ts_check_launch();
 }
+
+// ---- the qkv projection in slices, finished into the rotation and the cache write
+
+struct Rows64RopeArgs {
+  const float* parts;    // [slices][M][N], columns in the order of hip.pack_weight_rope: a 16-column tile holds 8
+                         // dimensions of a head's first half and, behind them, the 8 that rotate with them
+  int slices, M, N, K;
+  const float* ssq_in;   // a prepared norm's sums of squares [M, ssq_parts], or null
+  int ssq_parts;
+  float eps;
+  const float* cos_sin;  // [positions, hd] 32-bit, [cos | sin] halves
+  const int32_t* positions;
+  const int32_t* slots;
+  bf16_t* q_out;         // [M, nh * hd]
+  bf16_t* k_cache;       // null: this layer owns no cache, only q is produced
+  bf16_t* v_cache;
+  int nh, nkv, hd, rotate, page_size;
+  int64_t kp, ks, kh, vp, vs, vh, vd;   // key element: page * kp + offset * ks + head * kh + d; value: page * vp + offset * vs + head * vh + d * vd
+};
+
+// A workgroup per token: a thread adds the parts of four columns of a head's first half and of the four
+// that rotate with them, first slice first, scales them by the prepared norm's rsqrt(mean square + eps),
+// rounds them as the product would be stored, turns q and k by the token's position and writes q to
+// q_out, k and v to the token's slot: what EPI_ROPE of gemm_skinny.hip does with its own sums.
+__global__ void __launch_bounds__(R64_FINISH_THREADS) rows64_finish_rope_kernel(const Rows64RopeArgs a) {
+  __shared__ float wave_sq[R64_FINISH_THREADS / TS_WAVE];
+  const int m = blockIdx.x;
+  float inv = 1.0f;
+  if (a.ssq_in) {
+    float v = 0.f;
+    for (int q = threadIdx.x; q < a.ssq_parts; q += blockDim.x) v += a.ssq_in[(int64_t)m * a.ssq_parts + q];
+    v = wave_sum(v);
+    if ((threadIdx.x & (TS_WAVE - 1)) == 0) wave_sq[threadIdx.x / TS_WAVE] = v;
+    __syncthreads();
+    float total = 0.f;
+    for (int w = 0; w < (int)blockDim.x / TS_WAVE; ++w) total += wave_sq[w];
+    inv = __builtin_amdgcn_rsqf(total / (float)a.K + a.eps);
+  }
+  const int per_head = a.hd / 16, hdh = a.hd / 2;
+  for (int idx = threadIdx.x; idx < a.N / 8; idx += blockDim.x) {
+    const int jb = idx >> 1, nl = (idx & 1) * 4;            // the tile, and which four of its first eight columns
+    const int64_t at = (int64_t)m * a.N + 16 * jb + nl;
+    float4 s4 = make_float4(0.f, 0.f, 0.f, 0.f), u4 = s4;
+    for (int s0 = 0; s0 < a.slices; s0 += 4) {
+      float4 p[4], pu[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const bool in = s0 + j < a.slices;
+        const float* src = a.parts + (int64_t)(s0 + j) * a.M * a.N + at;
+        p[j] = in ? *(const float4*)src : make_float4(0.f, 0.f, 0.f, 0.f);
+        pu[j] = in ? *(const float4*)(src + 8) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (s0 + j == 0) { s4 = p[0]; u4 = pu[0]; continue; }
+        if (s0 + j < a.slices) {
+          s4.x += p[j].x; s4.y += p[j].y; s4.z += p[j].z; s4.w += p[j].w;
+          u4.x += pu[j].x; u4.y += pu[j].y; u4.z += pu[j].z; u4.w += pu[j].w;
+        }
+      }
+    }
+    const float s[4] = {s4.x * inv, s4.y * inv, s4.z * inv, s4.w * inv}, u[4] = {u4.x * inv, u4.y * inv, u4.z * inv, u4.w * inv};
+    const int head = jb / per_head, d0 = 8 * (jb % per_head) + nl;      // d0 .. d0 + 3 of the head's first half
+    float y1[4], y2[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {                         // as the product would be stored
+      y1[j] = __uint_as_float(sk_round(s[j]) << 16);
+      y2[j] = __uint_as_float(sk_round(u[j]) << 16);
+    }
+    if (a.rotate && head < a.nh + a.nkv) {
+      const float* cs = a.cos_sin + (int64_t)a.positions[m] * a.hd + d0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float c = cs[j], sn = cs[hdh + j];
+        const float r1 = y1[j] * c - y2[j] * sn, r2 = y2[j] * c + y1[j] * sn;
+        y1[j] = r1;
+        y2[j] = r2;
+      }
+    }
+    const uint2 o1 = make_uint2(sk_round(y1[0]) | (sk_round(y1[1]) << 16), sk_round(y1[2]) | (sk_round(y1[3]) << 16));
+    const uint2 o2 = make_uint2(sk_round(y2[0]) | (sk_round(y2[1]) << 16), sk_round(y2[2]) | (sk_round(y2[3]) << 16));
+    if (head < a.nh) {
+      bf16_t* dst = a.q_out + ((int64_t)m * a.nh + head) * a.hd + d0;
+      *(uint2*)dst = o1;
+      *(uint2*)(dst + hdh) = o2;
+      continue;
+    }
+    const int64_t slot = a.slots ? a.slots[m] : -1;
+    if (!a.k_cache || slot < 0) continue;
+    const int64_t page = slot / a.page_size, off = slot - page * a.page_size;
+    if (head < a.nh + a.nkv) {
+      bf16_t* dst = a.k_cache + page * a.kp + off * a.ks + (int64_t)(head - a.nh) * a.kh + d0;
+      *(uint2*)dst = o1;
+      *(uint2*)(dst + hdh) = o2;
+    } else {
+      bf16_t* dst = a.v_cache + page * a.vp + off * a.vs + (int64_t)(head - a.nh - a.nkv) * a.vh + (int64_t)d0 * a.vd;
+      const uint32_t w1[2] = {o1.x, o1.y}, w2[2] = {o2.x, o2.y};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        dst[(int64_t)j * a.vd] = (bf16_t)(w1[j >> 1] >> (16 * (j & 1)));
+        dst[(int64_t)(hdh + j) * a.vd] = (bf16_t)(w2[j >> 1] >> (16 * (j & 1)));
+      }
+    }
+  }
+}
+
+// The qkv projection of an attention layer for up to 64 rows of x with the reduction in `slices`
+// (K / slices a multiple of 512): w16 is hip.pack_weight_rope of W [(nh + 2 nkv) * hd, K], parts
+// [slices][M][N] float scratch. q_out [M, nh * hd] gets the rotated queries, the rotated keys and the
+// values go to the slots `slots[m]` of the pages (slot -1 stores nothing; k_cache null: only q).
+// ssq_in [M, ssq_parts] and eps: the prepared norm's scale per row (null: none). hd a multiple of 32,
+// (nh + 2 nkv) * hd a multiple of 64, 8-byte aligned key strides.
+extern "C" int ts_gemm_rows64_sliced_rope_bf16(void* q_out, void* parts, const void* x, const void* w16, int M, int K,
+                                               int64_t ldx, int slices, const void* ssq_in, int ssq_parts, float eps,
+                                               const float* cos_sin, const int32_t* positions, const int32_t* slots,
+                                               void* k_cache, void* v_cache, int nh, int nkv, int hd, int rotate,
+                                               int page_size, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vs,
+                                               int64_t vh, int64_t vd, hipStream_t stream) {
+  if (M <= 0) return TS_OK;
+  if (nh <= 0 || nkv < 0 || hd <= 0 || hd % 32 || page_size <= 0) return TS_BAD_SHAPE;
+  const int N = (nh + 2 * nkv) * hd;
+  if (N % 64 || slices < 1 || slices > 64 || K % (512 * slices) || !parts || !q_out || !r64_operands_ok(x, w16, M, N, K, ldx)) return TS_BAD_SHAPE;
+  if ((((uintptr_t)parts) & 15) || (((uintptr_t)q_out) & 7)) return TS_BAD_SHAPE;
+  if (ssq_in && (ssq_parts <= 0 || (((uintptr_t)ssq_in) & 3))) return TS_BAD_SHAPE;
+  if (rotate && (!cos_sin || !positions)) return TS_BAD_SHAPE;
+  if (k_cache && (!v_cache || !slots || (kp % 4) || (ks % 4) || (kh % 4) || (((uintptr_t)k_cache) & 7))) return TS_BAD_SHAPE;
+  Rows64Args a = {(const bf16_t*)x, (const bf16_t*)w16, parts, M, N, K, ldx, (int64_t)N, nullptr, 0, 0.f, slices};
+  const int rc = r64_launch<false, float>(a, stream);
+  if (rc != TS_OK) return rc;
+  Rows64RopeArgs f = {(const float*)parts, slices, M, N, K, (const float*)ssq_in, ssq_parts, eps, cos_sin, positions, slots,
+                      (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv, hd, rotate, page_size,
+                      kp, ks, kh, vp, vs, vh, vd};
+  const int threads = N / 8 >= R64_FINISH_THREADS ? R64_FINISH_THREADS : (N / 8 + TS_WAVE - 1) / TS_WAVE * TS_WAVE;
+  rows64_finish_rope_kernel<<<M, threads, 0, stream>>>(f);
+  return ts_check_launch();
+}

@@ -67,6 +67,8 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_gemm_skinny8_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p, p, p, p, p, p],
         "ts_gemm_rows64_bf16": [p, p, p, i, i, i, i64, i64, i, i, p, i, f, p],
         "ts_gemm_rows64_sliced_bf16": [p, p, p, p, i, i, i, i64, i, p, p, p, p, p, p],
+        "ts_gemm_rows64_sliced_rope_bf16": [p, p, p, p, i, i, i64, i, p, i, f, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64,
+                                            i64, i64, p],
         "ts_skinny_tiles": [i, i, i],
         "ts_peak_read": [p, ctypes.c_size_t, p, i, p],
         "ts_peak_mfma": [p, i, i, p],
@@ -1036,6 +1038,69 @@ def qkv_rope_store(x: torch.Tensor, weight: torch.Tensor, cos_sin: torch.Tensor 
     return q, res_out
 
 
+QKV_SLICED_MIN_ROWS = 33       # fewer rows: the library and the rotation kernel are as fast
+
+
+def qkv_rope_sliced_slices(x: torch.Tensor, weight: torch.Tensor, head_dim: int, k_cache: torch.Tensor | None,
+                           table: torch.Tensor | None = None) -> int:
+    """Slices in which `qkv_rope_store_sliced` should serve these operands; 0 if it should not: 33 to
+    64 bfloat16 rows over a reduction that `qkv_rope_store` does not take with so many rows (where it
+    does, it is the faster one: 64 rows over 2,048 against 3,072 columns 12.2 µs, 12.7 in slices), heads
+    of a multiple of 32 dimensions that turn whole, a width in steps of 64, a reduction in steps of
+    512. Measured against the library followed by the rotation kernel at 64 rows: 16.3 against 20.8 µs
+    over 3,072 against 5,120 columns, 22.0 against 21.4 over 4,096 against 6,144."""
+    if not (x.dim() == 2 and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and head_dim % 32 == 0
+            and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+            and (table is None or table.shape[1] == head_dim)
+            and (k_cache is None or (all(st % 4 == 0 for st in k_cache.stride()[:3]) and k_cache.data_ptr() % 8 == 0))):
+        return 0
+    rows, (n, k) = x.shape[0], weight.shape
+    if not (QKV_SLICED_MIN_ROWS <= rows <= ROWS64_MAX_ROWS) or rows <= qkv_rope_max_rows(k) or n % 64 or k % ROWS64_SLICE_K:
+        return 0
+    fits = [s for s in range(1, 17) if (k // ROWS64_SLICE_K) % s == 0]
+    enough = [s for s in fits if (n // 64) * s >= ROWS64_WORKGROUPS]
+    return enough[0] if enough else fits[-1]
+
+
+def qkv_rope_store_sliced(x: torch.Tensor, packed_rope: torch.Tensor, slices: int, cos_sin: torch.Tensor | None,
+                          positions: torch.Tensor, slots: torch.Tensor | None, k_cache: torch.Tensor | None,
+                          v_cache: torch.Tensor | None, num_heads: int, num_kv_heads: int, head_dim: int, *,
+                          eps: float = 0.0, squares: torch.Tensor | None = None) -> torch.Tensor:
+    """`qkv_rope_store` for 17 to 64 rows by the shared-x kernel with the reduction in `slices` and a
+    second kernel that adds the parts, rotates and writes the cache: q [tokens, nh, hd] comes back.
+    `packed_rope` = pack_weight_rope(weight, head_dim). With `squares` (and `eps`) x is the operand of
+    a `PreparedNorm` and the rows' scales multiply the finished sums."""
+    _gpu(x, packed_rope, cos_sin, positions, slots, k_cache, v_cache)
+    _check_squares(squares, x.shape[0])
+    M, K = x.shape
+    N = (num_heads + 2 * num_kv_heads) * head_dim
+    _need(x.dtype == torch.bfloat16 and packed_rope.dtype == torch.bfloat16 and packed_rope.dim() == 4
+          and packed_rope.shape == (N // 16, K // 32, 64, 8) and packed_rope.is_contiguous() and packed_rope.data_ptr() % 16 == 0,
+          f"qkv_rope_store_sliced takes bfloat16 x [M, K] and pack_weight_rope of a weight [{N}, {K}]")
+    _need(1 <= M <= ROWS64_MAX_ROWS and N % 64 == 0 and head_dim % 32 == 0 and 1 <= slices <= 64 and K % (ROWS64_SLICE_K * slices) == 0,
+          f"qkv_rope_store_sliced takes up to {ROWS64_MAX_ROWS} rows, a width in steps of 64, heads in steps of 32 and slices of K that "
+          f"are multiples of {ROWS64_SLICE_K}, not {M} x {K} against {N} in {slices}")
+    _need(x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0, "rows of x must be dense and 16-byte aligned")
+    _need(positions.dtype == torch.int32 and positions.shape == (M,) and positions.is_contiguous(), "positions must be int32 [tokens]")
+    if cos_sin is not None:
+        _need(cos_sin.dtype == torch.float32 and cos_sin.dim() == 2 and cos_sin.shape[1] == head_dim
+              and cos_sin.is_contiguous(), "the rotation table must be float32 [positions, head_dim]")
+    page_size, kst, vst = 1, (0, 0, 0), (0, 0, 0, 0)
+    if k_cache is not None:
+        _need(v_cache is not None and slots is not None, "a cache write needs k, v and the slots")
+        _need(slots.dtype == torch.int32 and slots.shape == (M,) and slots.is_contiguous(), "slots must be int32 [tokens]")
+        _check_cache(k_cache, v_cache, x.dtype, num_kv_heads, head_dim)
+        _need(all(st % 4 == 0 for st in k_cache.stride()[:3]) and k_cache.data_ptr() % 8 == 0, "key strides must allow 8-byte stores")
+        page_size, kst, vst = k_cache.shape[1], k_cache.stride()[:3], v_cache.stride()
+    parts = torch.empty((slices, M, N), dtype=torch.float32, device=x.device)
+    q = torch.empty((M, num_heads, head_dim), dtype=x.dtype, device=x.device)
+    _run("qkv_rope_store_sliced", library().ts_gemm_rows64_sliced_rope_bf16(
+        _ptr(q), _ptr(parts), _ptr(x), _ptr(packed_rope), M, K, x.stride(0), slices, _ptr(squares),
+        0 if squares is None else squares.shape[1], float(eps), _ptr(cos_sin), _ptr(positions), _ptr(slots), _ptr(k_cache),
+        _ptr(v_cache), num_heads, num_kv_heads, head_dim, int(cos_sin is not None), page_size, *kst, *vst, _stream()))
+    return q
+
+
 MANY_ROWS_PRODUCTS = ("library", "tiled")
 _many_rows = "library"
 
@@ -1101,9 +1166,17 @@ def next_norm_fuses(x: torch.Tensor, weight: torch.Tensor, packed: "StreamingCop
     return skinny8_takes(rows, n, k) or _skinny_serves(rows, n, k) or _sliced_serves(rows, n, k, packed) > 0
 
 
-def _sliced_serves(rows: int, n: int, k: int, packed: "StreamingCopies | None") -> int:
-    """The slices in which `linear_bf16` gives a product to `gemm_rows64_sliced` (0: it does not)."""
+ROWS64_PLAIN_MAX_WIDTH = 4096  # widest product that takes the sliced kernel when nothing rides on its finishing kernel
+
+
+def _sliced_serves(rows: int, n: int, k: int, packed: "StreamingCopies | None", finishing: bool = True) -> int:
+    """The slices in which `linear_bf16` gives a product to `gemm_rows64_sliced` (0: it does not).
+    `finishing`: the second kernel also makes the residual sum and the next norm's first half, and
+    so saves a kernel; without that the parts' trip through memory only pays for narrow products (32
+    rows against a weight of 5,120 x 3,072: 14.5 µs, the library 11)."""
     if packed is None or packed.by16 is None or skinny8_takes(rows, n, k) or _skinny_serves(rows, n, k):
+        return 0
+    if not finishing and n > ROWS64_PLAIN_MAX_WIDTH:
         return 0
     return rows64_slices(rows, n, k)
 
@@ -1131,7 +1204,8 @@ def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
         return gemm_skinny8(x, weight, out_dtype, None if packed is None else packed.by8, next_norm=next_norm)
     if streams and _skinny_serves(x.shape[0], weight.shape[0], x.shape[1]):
         return gemm_skinny(x, weight, out_dtype, packed=None if packed is None else packed.by16, next_norm=next_norm)[0]
-    slices = _sliced_serves(x.shape[0], weight.shape[0], x.shape[1], packed) if streams and out_dtype == torch.bfloat16 else 0
+    slices = (_sliced_serves(x.shape[0], weight.shape[0], x.shape[1], packed, next_norm is not None)
+              if streams and out_dtype == torch.bfloat16 else 0)
     if slices:
         return gemm_rows64_sliced(x, packed.by16, slices, next_norm=next_norm)
     _need(next_norm is None, "no kernel leaves a prepared norm for this product (ask next_norm_fuses first)")

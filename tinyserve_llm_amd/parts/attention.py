@@ -62,18 +62,29 @@ class Attention(Mixer):
 
     def _project_fused(self, x, table, positions, slots, k_store, v_store) -> torch.Tensor | None:
         """Projection, rotation and cache write in one kernel where a step is small enough for the
-        weight-streaming kernel; None where it is not."""
+        weight-streaming kernel (in two, with the reduction in slices, for a few dozen rows over a
+        reduction that kernel does not take); None where neither serves."""
         d = x if isinstance(x, DeferredNorm) else None
         by16 = self.qkv_rope_packed
         if d is not None and d.prepared is not None:     # the norm's first half is done: its operand, then a scale per row
             rows = d.prepared.operand
             if not hip.qkv_rope_fuses(rows, self.qkv, self.head_dim, k_store, table=table):
-                return None
+                slices = 0 if by16 is None else hip.qkv_rope_sliced_slices(rows, self.qkv, self.head_dim, k_store, table)
+                if not slices:
+                    return None
+                return hip.qkv_rope_store_sliced(rows, by16, slices, table, positions, slots, k_store, v_store, self.num_heads,
+                                                 self.num_kv_heads, self.head_dim, eps=d.eps, squares=d.prepared.squares)
             return hip.qkv_rope_store(rows, self.qkv, table, positions, slots, k_store, v_store, self.num_heads,
                                       self.num_kv_heads, self.head_dim, eps=d.eps, packed=by16, squares=d.prepared.squares)[0]
         rows = d.x if d is not None else x
         if not (rows.is_cuda and hip.qkv_rope_fuses(rows, self.qkv, self.head_dim, k_store, table=table)):
-            return None
+            slices = 0 if by16 is None or not rows.is_cuda else hip.qkv_rope_sliced_slices(rows, self.qkv, self.head_dim, k_store, table)
+            if not slices:
+                return None
+            if d is not None:
+                rows = d.materialize()           # the norm by its own kernel
+            return hip.qkv_rope_store_sliced(rows, by16, slices, table, positions, slots, k_store, v_store, self.num_heads,
+                                             self.num_kv_heads, self.head_dim)
         if d is not None and not (hip.qkv_rope_fuses(rows, self.qkv, self.head_dim, k_store, norm=True)
                                   and d.weight.dtype == torch.bfloat16
                                   and (d.residual is None or d.residual.is_contiguous())):
