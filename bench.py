@@ -183,6 +183,8 @@ def kernel_classes(llm, config, batch: int, reps: int = 5) -> dict:
         "gemm_skinny": product("gemm_skinny", lambda x, w, *a, **kw: w),
         "gemm_skinny8": product("gemm_skinny8", lambda x, w, *a, **kw: w),
         "gemm_rows64": product("gemm_rows64", lambda x, packed, *a, **kw: packed),
+        "gemm_rows64_sliced": product("gemm_rows64_sliced", lambda x, packed, *a, **kw: packed),
+        "qkv_rope_store_sliced": product("qkv_rope_store_sliced", lambda x, packed, *a, **kw: packed),
         "gemm_library": product("gemm_library", lambda x, w, *a, **kw: w),
         "gemm_exact": product("gemm_exact", lambda x, w, *a, **kw: w),
         "qkv_rope_store": product("qkv_rope_store", lambda x, w, *a, **kw: w),
@@ -227,7 +229,7 @@ def kernel_classes(llm, config, batch: int, reps: int = 5) -> dict:
                 end.synchronize()
                 times.append(1e3 * begin.elapsed_time(end))
             del outs, graph
-            us, nbytes = min(times[1:]) - overhead, sum(n for n, *_ in noted)
+            us, nbytes = max(min(times[1:]) - overhead, 1e-3), sum(n for n, *_ in noted)     # (a class of one tiny kernel may cost no more than the replay itself)
             if klass.startswith("("):
                 overhead = us                                  # what a replay costs before its first kernel's work: taken off every class
                 continue

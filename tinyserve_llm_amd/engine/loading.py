@@ -44,7 +44,8 @@ def streaming_copies(model: DecoderModel, policy: bool | None, device: torch.dev
     """Second copies of the weights in the decode kernels' reading orders (about a sixth faster to
     stream). A weight keeps up to one copy per kernel form that can take it (16-row tiles, 8-row
     tiles, and for q|k|v the tiles regrouped for the rotation), so the copies come to between one and
-    two times the weights' own bytes (1.7 times at the Llama 3.2 1B shape). `policy` None: made only
+    two times the weights' own bytes (1.9 times at the Llama 3.2 1B shape: every projection but q|k|v
+    keeps both tile forms). `policy` None: made only
     if twice the weights' bytes are less than a quarter of the memory that is still free, which
     leaves the cache pool what it had; the bytes taken are logged. Returns the bytes taken."""
     if policy is None:
