@@ -179,8 +179,8 @@ def test_the_benchmarks_own_regime_against_the_plain_model(folder_1b, dtype, bat
     (the bucket above 2,048 positions), the host one step ahead, attention over 2,049 to 2,064 keys
     that cross into a ninth page. Eight requests take the split-key attention kernel and the
     weight-streaming projections; sixty-four take one workgroup per (request, key/value head) over
-    the whole context, the shared-x kernel for the gate|up projection and the head, and this
-    repository's or the library's kernels for the rest, and the test sees that they did. Every token
+    the whole context, the shared-x kernel for the gate|up projection and the head, and the same kernel
+    with the reduction in slices for the o and down projections, and the test sees that they did. Every token
     of some of the requests against the plain model run whole over the same history: in float32 it is
     the plain model's choice; in bfloat16 it lies within a small gap of it."""
     from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
@@ -189,8 +189,8 @@ def test_the_benchmarks_own_regime_against_the_plain_model(folder_1b, dtype, bat
     from tinyserve_llm_amd.ops import hip
     length, decoded, page = 2048, 16, 256
     prompts = [prompt(900 + i, length, CONFIG.vocab_size) for i in range(batch)]
-    plans, rows64 = [], []
-    plan, shared_x = hip.decode_plan, hip.gemm_rows64
+    plans, rows64, sliced = [], [], []
+    plan, shared_x, in_slices = hip.decode_plan, hip.gemm_rows64, hip.gemm_rows64_sliced
 
     def seen_plan(num_tokens, nkv, group, hd, capacity):
         plans.append(((num_tokens, capacity), plan(num_tokens, nkv, group, hd, capacity)))
@@ -200,8 +200,13 @@ def test_the_benchmarks_own_regime_against_the_plain_model(folder_1b, dtype, bat
         rows64.append((x.shape[0], packed.shape[0] * 16))
         return shared_x(x, packed, *a, **kw)
 
+    def seen_sliced(x, packed, slices, next_norm=None):
+        sliced.append((x.shape[0], packed.shape[0] * 16, x.shape[1], slices, next_norm is not None))
+        return in_slices(x, packed, slices, next_norm=next_norm)
+
     monkeypatch.setattr(hip, "decode_plan", seen_plan)
     monkeypatch.setattr(hip, "gemm_rows64", seen_rows64)
+    monkeypatch.setattr(hip, "gemm_rows64_sliced", seen_sliced)
     # prompts first, one a step under the token budget; once the last one is in, all decode together
     sc = SchedulerConfig(max_model_len=4096, max_num_seqs=batch, max_num_batched_tokens=length + batch, watermark=0.0,
                          step_mode="prefill_first")
@@ -215,8 +220,10 @@ def test_the_benchmarks_own_regime_against_the_plain_model(folder_1b, dtype, bat
         if batch == 64:
             assert plan(64, 8, 4, 64, 9 * page) == (9 * page, 8), "a workgroup walks the whole context: nothing is combined"
             assert (64, 2 * 8192) in rows64 and (64, CONFIG.vocab_size) in rows64, f"gate|up and the head by the shared-x kernel: {rows64}"
+            assert (64, 2048, 2048, 4, True) in sliced and (64, 2048, 8192, 8, True) in sliced, \
+                f"o and down in slices of their reductions, finished into the norms that follow them: {set(sliced)}"
         else:
-            assert plan(8, 8, 4, 64, 9 * page)[0] < 9 * page and not rows64, "eight requests: keys in chunks, combined afterwards"
+            assert plan(8, 8, 4, 64, 9 * page)[0] < 9 * page and not rows64 and not sliced, "eight requests: keys in chunks, combined afterwards"
     plain = PlainLlama(folder_1b, torch.float64)
     head = plain.w["model.embed_tokens.weight"]
     some = [0, 1, batch // 2, batch - 1] if batch > 8 or dtype == "bfloat16" else range(batch)
