@@ -1202,6 +1202,7 @@ def test_narrow_product_in_slices_of_its_reduction(m, n, k, slices):
         assert torch.equal(prepared.summed.cpu(), t.float().bfloat16())
         assert torch.equal(prepared.operand.cpu(), (t.float() * nw.float().cpu()).bfloat16())
         assert prepared.squares.shape == (m, 1), "a row's sum of squares comes whole"
+        assert prepared.operand.stride() == (n + hip().OPERAND_ROW_SKEW, 1), "the operand's rows lie a little further apart than they are long"
         torch.testing.assert_close(prepared.squares.double().cpu(), t.pow(2).sum(1, keepdim=True), rtol=1e-5, atol=1e-6)
     with pytest.raises(hip().KernelError):
         hip().gemm_rows64_sliced(x, packed, slices * 2 if k % (1024 * slices) else 5 if (k // 512) % 5 else 7)

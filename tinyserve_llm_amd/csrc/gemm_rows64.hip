@@ -232,8 +232,9 @@ struct Rows64FinishArgs {
   const bf16_t* res;     // [M, N] or null
   const bf16_t* nw;      // [N]
   bf16_t* res_out;
-  bf16_t* op;
+  bf16_t* op;            // rows ld_op apart
   float* ssq_out;
+  int64_t ld_op;
 };
 
 // A workgroup per row: a thread adds the parts of four neighbouring columns, first slice first, then of the
@@ -281,7 +282,7 @@ __global__ void __launch_bounds__(R64_FINISH_THREADS) rows64_finish_kernel(const
       sq = fmaf(t, t, sq);
     }
     *(uint2*)(a.res_out + at) = make_uint2(sk_round(tv[0]) | (sk_round(tv[1]) << 16), sk_round(tv[2]) | (sk_round(tv[3]) << 16));
-    *(uint2*)(a.op + at) = make_uint2(sk_round(ov[0]) | (sk_round(ov[1]) << 16), sk_round(ov[2]) | (sk_round(ov[3]) << 16));
+    *(uint2*)(a.op + (int64_t)m * a.ld_op + n) = make_uint2(sk_round(ov[0]) | (sk_round(ov[1]) << 16), sk_round(ov[2]) | (sk_round(ov[3]) << 16));
   }
   if (!NEXT) return;
   sq = wave_sum(sq);
@@ -297,18 +298,18 @@ __global__ void __launch_bounds__(R64_FINISH_THREADS) rows64_finish_kernel(const
 
 // The same product with the reduction cut into `slices` (K / slices a multiple of 512), for a W of few rows:
 // parts [slices][M][N] float is scratch that the call fills and reads. With next_nw the product is not stored:
-// next_res_out, next_op [M, N] and ssq_out [M] (the rows' whole sums of squares: one part) are (next_res [M, N] or null is
-// added first); without it y [M, N] bfloat16 is.
+// next_res_out [M, N], next_op [M, N] with rows ld_op apart (a multiple of 4, at least N) and ssq_out [M] (the rows'
+// whole sums of squares: one part) are (next_res [M, N] or null is added first); without it y [M, N] bfloat16 is.
 extern "C" int ts_gemm_rows64_sliced_bf16(void* y, void* parts, const void* x, const void* w16, int M, int N, int K, int64_t ldx,
                                           int slices, const void* next_res, const void* next_nw, void* next_res_out,
-                                          void* next_op, void* ssq_out, hipStream_t stream) {
+                                          void* next_op, void* ssq_out, int64_t ld_op, hipStream_t stream) {
   if (M <= 0 || N <= 0) return TS_OK;
   if (N % 64 || slices < 1 || slices > 64 || K % (512 * slices) || !parts || !r64_operands_ok(x, w16, M, N, K, ldx)) return TS_BAD_SHAPE;
   if (((uintptr_t)parts) & 15) return TS_BAD_SHAPE;
   Rows64FinishArgs f = {(const float*)parts, slices, M, N, (bf16_t*)y, (const bf16_t*)next_res, (const bf16_t*)next_nw,
-                        (bf16_t*)next_res_out, (bf16_t*)next_op, (float*)ssq_out};
+                        (bf16_t*)next_res_out, (bf16_t*)next_op, (float*)ssq_out, ld_op};
   if (next_nw) {
-    if (!next_res_out || !next_op || !ssq_out || (((uintptr_t)ssq_out) & 3)) return TS_BAD_SHAPE;
+    if (!next_res_out || !next_op || !ssq_out || (((uintptr_t)ssq_out) & 3) || ld_op < N || ld_op % 4) return TS_BAD_SHAPE;
     if ((((uintptr_t)next_res) | ((uintptr_t)next_nw) | ((uintptr_t)next_res_out) | ((uintptr_t)next_op)) & 7) return TS_BAD_SHAPE;
   } else if (!y || (((uintptr_t)y) & 7)) {
     return TS_BAD_SHAPE;

@@ -66,7 +66,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p, i, p, p, p, p, p, p],
         "ts_gemm_skinny8_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p, p, p, p, p, p],
         "ts_gemm_rows64_bf16": [p, p, p, i, i, i, i64, i64, i, i, p, i, f, p],
-        "ts_gemm_rows64_sliced_bf16": [p, p, p, p, i, i, i, i64, i, p, p, p, p, p, p],
+        "ts_gemm_rows64_sliced_bf16": [p, p, p, p, i, i, i, i64, i, p, p, p, p, p, i64, p],
         "ts_gemm_rows64_sliced_rope_bf16": [p, p, p, p, i, i, i64, i, p, i, f, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64,
                                             i64, i64, p],
         "ts_skinny_tiles": [i, i, i],
@@ -669,8 +669,15 @@ class PreparedNorm:
         self.summed, self.operand, self.squares = summed, operand, squares
 
 
-def _next_norm_outputs(x: torch.Tensor, n: int, parts: int, next_norm) -> tuple[PreparedNorm, torch.Tensor | None, torch.Tensor]:
-    """Checks `next_norm` = (residual or None, weight) for a product [M, n] and makes its outputs."""
+OPERAND_ROW_SKEW = 8      # elements between the rows of an operand made for kernels that read 16 rows of x side by side
+
+
+def _next_norm_outputs(x: torch.Tensor, n: int, parts: int, next_norm, skew: int = 0) -> tuple[PreparedNorm, torch.Tensor | None, torch.Tensor]:
+    """Checks `next_norm` = (residual or None, weight) for a product [M, n] and makes its outputs.
+    `skew`: the operand's rows lie n + skew elements apart. (The kernels that take it read the same
+    64 bytes of 16 rows with one instruction; rows a power of two apart are slow to fetch that way:
+    64 rows over 2,048 against the q|k|v weight 12.0 µs, 10.2 with rows 16 bytes further apart, against
+    the gate|up weight 20.4 and 18.9.)"""
     residual, weight = next_norm
     _gpu(residual, weight)
     M = x.shape[0]
@@ -679,7 +686,7 @@ def _next_norm_outputs(x: torch.Tensor, n: int, parts: int, next_norm) -> tuple[
         _need(residual.dtype == torch.bfloat16 and residual.shape == (M, n) and residual.is_contiguous(),
               f"the residual must be bfloat16 [{M}, {n}]")
     out = PreparedNorm(torch.empty((M, n), dtype=torch.bfloat16, device=x.device),
-                       torch.empty((M, n), dtype=torch.bfloat16, device=x.device),
+                       torch.empty((M, n + skew), dtype=torch.bfloat16, device=x.device)[:, :n],
                        torch.empty((M, parts), dtype=torch.float32, device=x.device))
     return out, residual, weight
 
@@ -839,8 +846,8 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     _need(skinny_fuses(M, K, norm, glu),
           f"gemm_skinny takes up to {SKINNY_MAX_ROWS} rows ({SKINNY_FUSED_ROWS} with the norm, {SKINNY_EPILOGUE_ROWS} with the gate alone "
           "over up to 2048) and K in steps of 256 up to 4096 (2048 with the norm) or of 512 up to 8192")
-    _need(x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0,
-          "rows must be contiguous and 16-byte aligned")
+    _need((x.is_contiguous() if norm else _dense_rows(x)) and weight.is_contiguous() and x.data_ptr() % 16 == 0
+          and weight.data_ptr() % 16 == 0, "rows must be dense and 16-byte aligned (contiguous with the norm on the way in)")
     _need(not glu or (N % 32 == 0), "gate and up rows come in whole 16-row tiles")
     _check_packed(packed, weight)
     _check_squares(squares, M)
@@ -950,15 +957,21 @@ def gemm_rows64_sliced(x: torch.Tensor, packed: torch.Tensor, slices: int, next_
     _need(x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0, "rows of x must be dense and 16-byte aligned")
     parts = torch.empty((slices, M, N), dtype=torch.float32, device=x.device)
     if next_norm is not None:
-        prepared, residual, nw = _next_norm_outputs(x, N, 1, next_norm)
+        prepared, residual, nw = _next_norm_outputs(x, N, 1, next_norm, skew=OPERAND_ROW_SKEW)
         _run("gemm_rows64_sliced", library().ts_gemm_rows64_sliced_bf16(
             None, _ptr(parts), _ptr(x), _ptr(packed), M, N, K, x.stride(0), slices, _ptr(residual), _ptr(nw),
-            _ptr(prepared.summed), _ptr(prepared.operand), _ptr(prepared.squares), _stream()))
+            _ptr(prepared.summed), _ptr(prepared.operand), _ptr(prepared.squares), prepared.operand.stride(0), _stream()))
         return prepared
     out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
     _run("gemm_rows64_sliced", library().ts_gemm_rows64_sliced_bf16(
-        _ptr(out), _ptr(parts), _ptr(x), _ptr(packed), M, N, K, x.stride(0), slices, None, None, None, None, None, _stream()))
+        _ptr(out), _ptr(parts), _ptr(x), _ptr(packed), M, N, K, x.stride(0), slices, None, None, None, None, None, 0, _stream()))
     return out
+
+
+def _dense_rows(x: torch.Tensor) -> bool:
+    """Whether the rows of a matrix are dense and begin at multiples of 16 bytes (they may lie further
+    apart than they are long)."""
+    return x.dim() == 2 and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.stride(0) >= x.shape[1]
 
 
 def qkv_rope_max_rows(k: int, norm: bool = False) -> int:
@@ -979,7 +992,8 @@ def qkv_rope_fuses(x: torch.Tensor, weight: torch.Tensor, head_dim: int, k_cache
     whole (`table`, if given, as wide as a head), keys whose strides allow 8-byte stores."""
     rows_ok = x.dim() == 2 and x.shape[0] <= qkv_rope_max_rows(x.shape[1], norm) and (table is None or table.shape[1] == head_dim)
     return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and rows_ok and head_dim % 32 == 0
-            and x.is_contiguous() and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0
+            and (x.is_contiguous() if norm else _dense_rows(x)) and weight.is_contiguous() and x.data_ptr() % 16 == 0
+            and weight.data_ptr() % 16 == 0
             and (k_cache is None or (all(st % 4 == 0 for st in k_cache.stride()[:3]) and k_cache.data_ptr() % 8 == 0)))
 
 

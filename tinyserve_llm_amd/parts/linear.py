@@ -58,8 +58,11 @@ class NormRequest:
         return r.residual_out if isinstance(r, DeferredNorm) else r
 
 
-def _streams(x: torch.Tensor, weight: torch.Tensor) -> bool:
-    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.is_cuda and x.is_contiguous()
+def _streams(x: torch.Tensor, weight: torch.Tensor, dense_rows: bool = False) -> bool:
+    """Whether the weight-streaming kernels take these operands; `dense_rows`: x need not be
+    contiguous as long as its rows are (a prepared norm's operand, whose rows may lie further apart)."""
+    rows_ok = (x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.stride(0) >= x.shape[1]) if dense_rows and x.dim() == 2 else x.is_contiguous()
+    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.is_cuda and rows_ok
             and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
 
 
@@ -96,7 +99,7 @@ def linear(x: torch.Tensor | DeferredNorm, weight: torch.Tensor, out_dtype: torc
     by16 = None if packed is None else packed.by16
     if isinstance(x, DeferredNorm) and x.prepared is not None:
         d, op = x, x.prepared.operand
-        if out_dtype in (None, torch.bfloat16) and _streams(op, weight) and not (glu and weight.shape[0] % 32):
+        if out_dtype in (None, torch.bfloat16) and _streams(op, weight, dense_rows=True) and not (glu and weight.shape[0] % 32):
             rows, (n, k) = op.shape[0], weight.shape
             wide = by16 is not None and hip.rows64_takes(rows, n, k) and n % (128 if glu else 64) == 0
             if wide:
