@@ -403,6 +403,53 @@ def test_split_key_decode_window_and_far_key():
         assert torch.allclose(out[0, 0].float().cpu(), v[target, 0].to(dtype).float(), rtol=1e-2, atol=1e-2) == seen
 
 
+@pytest.mark.parametrize("page,pool_page", [(256, 32), (64, 32), (128, 64), (48, 8)])
+def test_block_tables_may_count_in_longer_pages_than_the_pools_are_cut_into(page, pool_page):
+    """An entry of a block table may stand for several consecutive pages of the pools (the engine's
+    bfloat16 pools are cut into pages of 32 slots whatever page size the manager counts in): the
+    three attention kernels read the same keys either way, and give the same result bit for bit."""
+    dtype = torch.bfloat16
+    n, heads, kv, hd = 600, 8, 2, 64
+    per = page // pool_page
+    if per & (per - 1):
+        with pytest.raises(hip().KernelError, match="power of two"):
+            hip().paged_attention_wave(torch.zeros(1, heads, hd, dtype=dtype, device=dev()),
+                                       torch.zeros(6, pool_page, kv, hd, dtype=dtype, device=dev()),
+                                       torch.zeros(6, pool_page, kv, hd, dtype=dtype, device=dev()),
+                                       torch.zeros(1, 1, dtype=torch.int32, device=dev()), torch.zeros(1, dtype=torch.int32, device=dev()),
+                                       torch.zeros(1, dtype=torch.int32, device=dev()), 1.0, pages_per_entry=per)
+        return
+    g = gen(page + pool_page)
+    q = torch.randn(n, heads, hd, generator=g).to(dtype)
+    k, v = torch.randn(n, kv, hd, generator=g).to(dtype), torch.randn(n, kv, hd, generator=g).to(dtype)
+    pages = -(-n // page) + 2
+    table = torch.randperm(pages, generator=g)[:-(-n // page)].tolist()
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev())
+    kc, vc = engine_layout(k, v, table, page, pages, dtype)                       # pools in pages of `page`
+    # the same slots in pools of `pool_page`: page p of the table is the pool's pages p * per + j
+    fine = [table[e] * per + j for e in range(len(table)) for j in range(per)]
+    kf, vf = engine_layout(k, v, fine, pool_page, pages * per, dtype)
+    rows = [0, 31, 32, pool_page, page - 1, page, 333, 599]
+    qd, tables, seqs, positions = q[rows].to(dev()), i32([table]), i32([0] * len(rows)), i32(rows)
+    want = P.causal_attention(q.double(), k.double(), v.double())[rows]
+    for run in (lambda kc, vc, **kw: hip().paged_attention_wave(qd, kc, vc, tables, seqs, positions, hd ** -0.5, **kw),
+                lambda kc, vc, **kw: hip().paged_attention_decode(qd, kc, vc, tables, seqs, positions, hd ** -0.5, chunk=256, waves=8, **kw),
+                lambda kc, vc, **kw: hip().paged_attention_decode(qd, kc, vc, tables, seqs, positions, hd ** -0.5, window=100, **kw)):
+        coarse, sub = run(kc, vc), run(kf, vf, pages_per_entry=per)
+        assert torch.equal(coarse, sub)
+    torch.testing.assert_close(hip().paged_attention_decode(qd, kf, vf, tables, seqs, positions, hd ** -0.5, pages_per_entry=per).double().cpu(),
+                               want, **tol(dtype))
+    # a whole prompt through the tile kernel
+    tile_tokens = 4 * (16 // (heads // kv))
+    tiles = i32(hip().attention_tiles([0, n], [0], tile_tokens)).view(-1, 2)
+    every = i32(list(range(n)))
+    whole = lambda kc, vc, **kw: hip().paged_attention_prefill(q.to(dev()), kc, vc, tables, i32([0] * n), every, tiles, hd ** -0.5,
+                                                               tile_tokens=tile_tokens, **kw)
+    coarse, sub = whole(kc, vc), whole(kf, vf, pages_per_entry=per)
+    assert torch.equal(coarse, sub)
+    torch.testing.assert_close(sub.double().cpu(), P.causal_attention(q.double(), k.double(), v.double()), **tol(dtype))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_wave_kernel_reads_the_engine_layout(dtype):
     n, heads, kv, hd, page = 100, 6, 3, 48, 16

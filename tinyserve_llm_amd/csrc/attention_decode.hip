@@ -28,7 +28,7 @@ __global__ void __launch_bounds__(DEC_WAVES_FOR(HD, ONE) * TS_WAVE)
 attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
                         const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
                         const int32_t* __restrict__ block_tables, const int32_t* __restrict__ seq_of_token,
-                        const int32_t* __restrict__ positions, int nh, int G, int page_size, int page_shift,
+                        const int32_t* __restrict__ positions, int nh, int G, int page_size, int page_shift, int page_run,
                         int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
                         int num_splits, int chunk, float scale2, int window) {
   constexpr int NC = HD / 32;    // 32-dimension pieces of a key row (one 16-byte load per lane each)
@@ -47,7 +47,7 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, fl
   const int k0 = split * chunk;
   if (k0 > pos || k0 + chunk <= lo) return;     // nothing of this chunk is visible
   const int32_t* table = block_tables + (int64_t)seq_of_token[t] * max_blocks;
-  const PageMath pm{page_size, page_shift};
+  const PageMath pm{page_size, page_shift, page_run};
 
   uint4 qreg[NC];
 #pragma unroll
@@ -182,15 +182,16 @@ int ts_launch_attention_combine(void* out, const float* part_o, const float* par
 // of a token combine its chunks inside the first kernel was tried and is slower: on a GPU of several
 // dies the device-scope fences it needs write back and invalidate each die's L2.) Keys: rows dense in
 // head_dim, strides kp/ks/kh (page, slot, head). Values: transposed pages, slot stride 1, strides
-// vp/vh/vd (page, head, dimension).
+// vp/vh/vd (page, head, dimension). An entry of block_tables names 2^page_run consecutive pages of page_size
+// keys (entry e: the pages e 2^page_run + j); max_blocks is the tables' width in entries.
 extern "C" int ts_paged_attention_decode(void* out, float* part_o, float* part_ml, const void* q, const void* k_cache,
                                          const void* v_cache, const int32_t* block_tables,
                                          const int32_t* seq_of_token, const int32_t* positions, int num_tokens, int nh,
                                          int nkv, int hd, int page_size, int64_t kp, int64_t ks, int64_t kh,
                                          int64_t vp, int64_t vh, int64_t vd, int max_blocks, int num_splits, int chunk,
-                                         int waves, float scale, int window, hipStream_t stream) {
+                                         int waves, float scale, int window, int page_run, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
-  if (nkv <= 0 || nh % nkv || page_size <= 0 || page_size % 8 || max_blocks <= 0 || num_splits <= 0)
+  if (nkv <= 0 || nh % nkv || page_size <= 0 || page_size % 8 || max_blocks <= 0 || num_splits <= 0 || page_run < 0 || page_run > 16)
     return TS_BAD_SHAPE;
   if (waves < 1 || waves > DEC_WAVES_FOR(hd, chunk == 32 * waves) || chunk <= 0 || chunk % (32 * waves) || num_splits > COMBINE_MAX_SPLITS)
     return TS_BAD_SHAPE;
@@ -212,7 +213,7 @@ extern "C" int ts_paged_attention_decode(void* out, float* part_o, float* part_m
 #define TS_DEC1(HH, ON)                                                                                         \
   attn_decode_mfma_kernel<HH, ON><<<grid, waves * TS_WAVE, smem, stream>>>(                                 \
       (bf16_t*)out, part_o, part_ml, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,          \
-      block_tables, seq_of_token, positions, nh, G, page_size, page_shift, kp, ks, kh, vp, vh, vd, max_blocks,  \
+      block_tables, seq_of_token, positions, nh, G, page_size, page_shift, page_run, kp, ks, kh, vp, vh, vd, max_blocks,  \
       num_splits, chunk, scale * 1.44269504088896340736f, window)
 #define TS_DEC(HH) if (chunk == 32 * waves) TS_DEC1(HH, true); else TS_DEC1(HH, false)
   switch (hd) {

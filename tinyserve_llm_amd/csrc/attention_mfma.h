@@ -36,10 +36,16 @@ static __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
 // (scale * log2 e) is all the softmax needs besides it
 static __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-struct PageMath {   // key -> (page index in the table, slot inside the page)
+struct PageMath {   // key -> (page index in the request, slot inside the page)
   int size, shift;  // shift >= 0: the page size is 2^shift
+  int run = 0;      // an entry of a request's page table names 2^run consecutive pages of the pool: entry e the pages
+                    // e 2^run .. e 2^run + 2^run - 1 (the pools may be cut into shorter pages than the tables count in)
   __device__ __forceinline__ int page(int key) const { return shift >= 0 ? key >> shift : key / size; }
   __device__ __forceinline__ int slot(int key, int pg) const { return key - pg * size; }
+  // the pool's page that is page pg of the request whose table this is
+  __device__ __forceinline__ int64_t pool_page(const int32_t* __restrict__ table, int pg) const {
+    return ((int64_t)table[pg >> run] << run) + (pg & ((1 << run) - 1));
+  }
   // pages of a multiple of 32 keys: a 32-key step (kb a multiple of 32) lies inside one page, and
   // its table entry is one scalar lookup for the whole wave
   __device__ __forceinline__ bool whole_steps() const { return (size & 31) == 0; }
@@ -87,7 +93,7 @@ static __device__ __forceinline__ void load_tile(KVTile<HD>& T, int kb, int r, i
     // one page for the whole step: its base addresses are scalars, the lanes add fixed offsets
     // (the page is the request's since kb <= pos, and all its slots are memory of the pool)
     const int pg = pm.page(kb);
-    const int64_t page = table[pg];
+    const int64_t page = pm.pool_page(table, pg);
     const int slot = pm.slot(kb, pg);
     const int64_t kbase = page * kp + (int64_t)slot * ks + (int64_t)kvh * kh;
 #pragma unroll
@@ -98,12 +104,12 @@ static __device__ __forceinline__ void load_tile(KVTile<HD>& T, int kb, int r, i
     for (int tau = 0; tau < 2; ++tau) {
       const int key = min(max(kb + 8 * (r >> 2) + 4 * tau + (r & 3), lo), pos);     // a visible key, for the address
       const int pg = pm.page(key);
-      koff[tau] = (int64_t)table[pg] * kp + (int64_t)pm.slot(key, pg) * ks + (int64_t)kvh * kh + 8 * g;
+      koff[tau] = pm.pool_page(table, pg) * kp + (int64_t)pm.slot(key, pg) * ks + (int64_t)kvh * kh + 8 * g;
     }
     // page sizes are multiples of 8: the 8 keys share a page
     const int vkey = (kb + 8 * g <= pos && kb + 8 * g + 7 >= lo) ? kb + 8 * g : (pos & ~7);
     const int pg = pm.page(vkey);
-    voff = (int64_t)table[pg] * vp + pm.slot(vkey, pg) + (int64_t)kvh * vh + (int64_t)r * vd;
+    voff = pm.pool_page(table, pg) * vp + pm.slot(vkey, pg) + (int64_t)kvh * vh + (int64_t)r * vd;
   }
   T.vok = kb + 8 * g <= pos && kb + 8 * g + 7 >= lo;
 #pragma unroll

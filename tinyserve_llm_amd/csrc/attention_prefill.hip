@@ -41,7 +41,7 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
              const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
              const int32_t* __restrict__ block_tables, const int32_t* __restrict__ seq_of_token,
              const int32_t* __restrict__ positions, const int32_t* __restrict__ tiles, int nh, int G, int page_size,
-             int page_shift, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
+             int page_shift, int page_run, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
              float scale2, int window, float* __restrict__ part_o, float* __restrict__ part_ml, int num_splits,
              int chunk, int split) {
   constexpr int NC = HD / 32, NDB = HD / 16;   // operand registers of a 32-key step: 2 NC of K, NDB of V
@@ -51,7 +51,7 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
   const int r = lane & 15, g = lane >> 4;
   const int t0 = tiles[2 * tile], ntok = tiles[2 * tile + 1];
   const int32_t* table = block_tables + (int64_t)seq_of_token[t0] * max_blocks;
-  const PageMath pm{page_size, page_shift};
+  const PageMath pm{page_size, page_shift, page_run};
   const int tpt = 16 / G;                                   // tokens per row tile
 
   // lane r carries row r of each of its wave's score tiles: token tk[j], head r % G of the group
@@ -156,7 +156,7 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
     if (whole) {
       // one page for the whole step: its base addresses are scalars, the lanes add fixed offsets
       const int pg = pm.page(kb);
-      const int64_t page = table[pg];
+      const int64_t page = pm.pool_page(table, pg);
       const int slot = pm.slot(kb, pg);
       const bool inner = kb >= wlo && kb + 31 <= whi;
       const bf16_t* src;              // this lane's first piece; the others follow at a fixed stride
@@ -187,7 +187,7 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
       const int key = kb + 8 * (r >> 2) + 4 * tau + (r & 3);
       if (key <= whi && key >= wlo) {
         const int pg = pm.page(key);
-        const bf16_t* kr = k_cache + (int64_t)table[pg] * kp + (int64_t)pm.slot(key, pg) * ks + (int64_t)kvh * kh + 8 * g + 32 * c0;
+        const bf16_t* kr = k_cache + pm.pool_page(table, pg) * kp + (int64_t)pm.slot(key, pg) * ks + (int64_t)kvh * kh + 8 * g + 32 * c0;
 #pragma unroll
         for (int c = 0; c < PER; ++c) fetched[c] = *(const uint4*)(kr + 32 * c);
       }
@@ -195,7 +195,7 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
       const int vkey = kb + 8 * g;
       if (vkey <= whi && vkey + 7 >= wlo) {
         const int pg = pm.page(vkey);
-        const bf16_t* vr = v_cache + (int64_t)table[pg] * vp + pm.slot(vkey, pg) + (int64_t)kvh * vh +
+        const bf16_t* vr = v_cache + pm.pool_page(table, pg) * vp + pm.slot(vkey, pg) + (int64_t)kvh * vh +
                            (int64_t)(db0 * 16 + r) * vd;
 #pragma unroll
         for (int c = 0; c < PER; ++c) fetched[c] = *(const uint4*)(vr + (int64_t)(16 * c) * vd);
@@ -283,7 +283,7 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
                          const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables,
                          const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ positions,
                          const int32_t* __restrict__ tiles, int num_tiles, int nh, int G, int dies_per_group,
-                         int heads_per_group, int page_size, int page_shift, int64_t kp, int64_t ks, int64_t kh,
+                         int heads_per_group, int page_size, int page_shift, int page_run, int64_t kp, int64_t ks, int64_t kh,
                          int64_t vp, int64_t vh, int64_t vd, int max_blocks, float scale2, int window,
                          float* __restrict__ part_o, float* __restrict__ part_ml, int num_splits, int chunk) {
   __shared__ PrefillLds<HD> lds;
@@ -295,7 +295,7 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
   const int tile = num_tiles - 1 - item / heads_per_group;
   const int kvh = (die / dies_per_group) * heads_per_group + item % heads_per_group;
   prefill_tile<HD, RT, PRE_WAVES>(lds, tile, kvh, out, q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, nh,
-                       G, page_size, page_shift, kp, ks, kh, vp, vh, vd, max_blocks, scale2, window, part_o, part_ml,
+                       G, page_size, page_shift, page_run, kp, ks, kh, vp, vh, vd, max_blocks, scale2, window, part_o, part_ml,
                        num_splits, chunk, blockIdx.y);
 }
 
@@ -305,19 +305,19 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
 // (heads of 64 or 128 dimensions). num_splits > 1: chunk (a multiple of 32; the last chunk
 // takes every key from its start on) and the float workspaces part_o [num_tokens, nh, num_splits, hd] and
 // part_ml [num_tokens, nh, num_splits, 2]; every token from first_token on must then be in a tile (the ones
-// before it keep what `out` held).
+// before it keep what `out` held). An entry of block_tables names 2^page_run consecutive pages of page_size keys.
 extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* k_cache, const void* v_cache,
                                           const int32_t* block_tables, const int32_t* seq_of_token,
                                           const int32_t* positions, const int32_t* tiles, int num_tiles,
                                           int tile_tokens, int waves, int nh, int nkv, int hd, int page_size, int64_t kp,
                                           int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
                                           float scale, int window, int first_token, int num_tokens, int num_splits,
-                                          int chunk, float* part_o, float* part_ml, hipStream_t stream) {
+                                          int chunk, float* part_o, float* part_ml, int page_run, hipStream_t stream) {
   if (num_tiles <= 0) return TS_OK;
   if (num_splits < 1 || num_splits > 65535) return TS_BAD_SHAPE;
   if (num_splits > 1 && (chunk <= 0 || chunk % 32 || !part_o || !part_ml || first_token < 0 || num_tokens <= first_token))
     return TS_BAD_SHAPE;
-  if (nkv <= 0 || nh % nkv || page_size <= 0 || page_size % 8 || max_blocks <= 0) return TS_BAD_SHAPE;
+  if (nkv <= 0 || nh % nkv || page_size <= 0 || page_size % 8 || max_blocks <= 0 || page_run < 0 || page_run > 16) return TS_BAD_SHAPE;
   const int G = nh / nkv;
   if (G > 16) return TS_BAD_SHAPE;
   if (waves != 4 && !(waves == 8 && (hd == 64 || hd == 128))) return TS_BAD_SHAPE;
@@ -340,7 +340,7 @@ extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* 
 #define TS_PRE_W(HH, RR, WW)                                                                                    \
   attn_prefill_mfma_kernel<HH, RR, WW><<<grid, WW * TS_WAVE, 0, stream>>>(                                      \
       (bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,             \
-      seq_of_token, positions, tiles, num_tiles, nh, G, dies_per_group, heads_per_group, page_size, page_shift, kp,  \
+      seq_of_token, positions, tiles, num_tiles, nh, G, dies_per_group, heads_per_group, page_size, page_shift, page_run, kp,  \
       ks, kh, vp, vh, vd, max_blocks, scale * 1.44269504088896340736f, window, part_o, part_ml, num_splits, chunk)
 #define TS_PRE_RT(HH)                                                                                           \
   if (rt == 1) TS_PRE_W(HH, 1, 4); else if (rt == 2) TS_PRE_W(HH, 2, 4); else TS_PRE_W(HH, 4, 4)

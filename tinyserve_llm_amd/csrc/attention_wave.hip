@@ -39,7 +39,7 @@ paged_attention_wave_kernel(T* __restrict__ out, const T* __restrict__ q, const 
                             const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ positions,
                             int num_tokens, int nh, int nkv, int hd, int page_size, int64_t page_stride,
                             int64_t slot_stride, int64_t head_stride, int64_t vp, int64_t vs, int64_t vh, int64_t vd,
-                            int max_blocks, float scale, int window) {
+                            int max_blocks, float scale, int window, int page_run) {
   __shared__ float q_s[ATT_WAVES][ATT_MAX_HD];
   __shared__ float p_s[ATT_WAVES][TS_WAVE];
   __shared__ int64_t row_s[ATT_WAVES][TS_WAVE];   // element offset of each key's value row
@@ -64,10 +64,11 @@ paged_attention_wave_kernel(T* __restrict__ out, const T* __restrict__ q, const 
     float s = -INFINITY;
     int64_t rowoff = 0;
     if (valid) {
-      const int page = table[key / page_size];
-      const int slot = key % page_size;
-      rowoff = (int64_t)page * vp + (int64_t)slot * vs + (int64_t)kvh * vh;
-      const T* kr = k_cache + (int64_t)page * page_stride + (int64_t)slot * slot_stride + (int64_t)kvh * head_stride;
+      // (an entry of the table names 2^page_run consecutive pages of the pool)
+      const int pg = key / page_size, slot = key % page_size;
+      const int64_t page = ((int64_t)table[pg >> page_run] << page_run) + (pg & ((1 << page_run) - 1));
+      rowoff = page * vp + (int64_t)slot * vs + (int64_t)kvh * vh;
+      const T* kr = k_cache + page * page_stride + (int64_t)slot * slot_stride + (int64_t)kvh * head_stride;
       float dot = 0.f;
       for (int d = 0; d < hd; d += Vec<T>::N) {
         float kv[Vec<T>::N];
@@ -112,9 +113,9 @@ extern "C" int ts_paged_attention_wave(void* out, const void* q, const void* k_c
                                        const int32_t* positions, int num_tokens, int nh, int nkv, int hd,
                                        int page_size, int64_t page_stride, int64_t slot_stride, int64_t head_stride,
                                        int64_t vp, int64_t vs, int64_t vh, int64_t vd, int max_blocks, float scale,
-                                       int window, int dtype, hipStream_t stream) {
+                                       int window, int dtype, int page_run, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
-  if (hd % 16 || hd > ATT_MAX_HD || hd <= 0 || nkv <= 0 || nh % nkv || page_size <= 0 || max_blocks <= 0)
+  if (hd % 16 || hd > ATT_MAX_HD || hd <= 0 || nkv <= 0 || nh % nkv || page_size <= 0 || max_blocks <= 0 || page_run < 0 || page_run > 16)
     return TS_BAD_SHAPE;
   // 16-byte key loads need 16-byte aligned rows
   const int64_t elem = dtype == 0 ? 4 : 2;
@@ -127,12 +128,12 @@ extern "C" int ts_paged_attention_wave(void* out, const void* q, const void* k_c
     paged_attention_wave_kernel<float><<<grid, block, 0, stream>>>(
         (float*)out, (const float*)q, (const float*)k_cache, (const float*)v_cache, block_tables, seq_of_token,
         positions, num_tokens, nh, nkv, hd, page_size, page_stride, slot_stride, head_stride, vp, vs, vh, vd, max_blocks,
-        scale, window);
+        scale, window, page_run);
   else if (dtype == 1)
     paged_attention_wave_kernel<bf16_t><<<grid, block, 0, stream>>>(
         (bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, seq_of_token,
         positions, num_tokens, nh, nkv, hd, page_size, page_stride, slot_stride, head_stride, vp, vs, vh, vd, max_blocks,
-        scale, window);
+        scale, window, page_run);
   else
     return TS_BAD_DTYPE;
   return ts_check_launch();

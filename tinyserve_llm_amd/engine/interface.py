@@ -52,7 +52,10 @@ class StepMemory(Protocol):
 
     def layer_cache(self, owner: int) -> tuple[torch.Tensor, torch.Tensor, int]:
         """(keys, values, page space) of the cache that run `owner` of the model's order owns, both
-        addressed [pages, page_size, kv_heads, head_dim]."""
+        addressed [pages, slots of a page, kv_heads, head_dim]. The views' pages may be shorter than
+        `page_size` (a whole number of them to a page, laid out one after the other): slot numbers, which
+        count in `page_size`, address the same memory either way, and readers that go through block
+        tables learn the ratio from the step's context (`StepContext.page_size`)."""
 
     def state(self, run: int) -> torch.Tensor | None: ...
 

@@ -208,7 +208,7 @@ class ModelRunner:
             num_tokens=T, num_seqs=S, token_ids=cut(T), positions=cut(T), seq_of_token=cut(T), cu_seqlens=cut(S + 1),
             context_lens=cut(S), state_slots=cut(S), slot_mapping=[], block_tables=[],
             host_cu_seqlens=host["cu"], host_starts=host["starts"], host_context_lens=host["ctx_lens"],
-            host_state_slots=host["slots"])
+            host_state_slots=host["slots"], page_size=self.storage.page_size)
         row_t = cut(R)
         for sp in range(len(widths)):
             ctx.block_tables.append(packed[offsets[sp]:offsets[sp] + S * widths[sp]].view(S, widths[sp]))

@@ -49,9 +49,9 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_rope_store": [p, p, p, p, p, p, p, i, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i64, i, p],
         "ts_silu_mul": [p, p, i, i, i, p],
         "ts_copy_slots": [p, i64, i64, i64, i, i, p],
-        "ts_paged_attention_wave": [p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i64, i, f, i, i, p],
+        "ts_paged_attention_wave": [p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i64, i, f, i, i, i, p],
         "ts_paged_attention_decode": [p, p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, i, i, i, f,
-                                      i, p],
+                                      i, i, p],
         "ts_gemm_exact": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_sample": [p, p, p, p, p, p, u64, i, i, i64, p],
         "ts_sample_static": [p, p, p, p, u64, i, i, i64, p],
@@ -62,7 +62,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_gemm_library_init": [],
         "ts_gemm_library_timing": [i],
         "ts_gemm_library_choices": [p, i],
-        "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, i, i, i, i, p, p, p],
+        "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, i, i, i, i, p, p, i, p],
         "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p, i, p, p, p, p, p, p],
         "ts_gemm_skinny8_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p, p, p, p, p, p],
         "ts_gemm_rows64_bf16": [p, p, p, i, i, i, i64, i64, i, i, p, i, f, p],
@@ -212,11 +212,20 @@ def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, dtype: torch.dtyp
           "key rows must be 16-byte aligned")
 
 
+def _page_run(pages_per_entry: int) -> int:
+    """log2 of the pool pages that one entry of a block table names (a power of two)."""
+    _need(pages_per_entry >= 1 and pages_per_entry & (pages_per_entry - 1) == 0 and pages_per_entry <= 65536,
+          f"an entry of a block table names a power of two of pages, not {pages_per_entry}")
+    return pages_per_entry.bit_length() - 1
+
+
 def paged_attention_wave(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                          block_tables: torch.Tensor, seq_of_token: torch.Tensor, positions: torch.Tensor,
-                         scale: float, window: int = 0) -> torch.Tensor:
+                         scale: float, window: int = 0, pages_per_entry: int = 1) -> torch.Tensor:
     """Attention of each token (at its position, causal, optionally windowed) over the cache
-    pages that its request's row of `block_tables` names."""
+    pages that its request's row of `block_tables` names. `pages_per_entry` (a power of two): an
+    entry e of a block table stands for that many consecutive pages of the cache, e * n + j (the
+    pools may be cut into shorter pages than the tables count in)."""
     _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions)
     _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
     T, nh, hd = q.shape
@@ -232,7 +241,7 @@ def paged_attention_wave(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.
     _run("paged_attention_wave", library().ts_paged_attention_wave(
         _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_of_token), _ptr(positions),
         T, nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3], *v_cache.stride(),
-        block_tables.shape[1], float(scale), int(window), _code(q.dtype), _stream()))
+        block_tables.shape[1], float(scale), int(window), _code(q.dtype), _page_run(pages_per_entry), _stream()))
     return out
 
 
@@ -333,10 +342,11 @@ def decode_kernel_takes(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
 def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                            seq_of_token: torch.Tensor, positions: torch.Tensor, scale: float, window: int = 0,
                            chunk: int | None = None, waves: int | None = None,
-                           out: torch.Tensor | None = None) -> torch.Tensor:
+                           out: torch.Tensor | None = None, pages_per_entry: int = 1) -> torch.Tensor:
     """Split-key attention on the matrix cores for tokens that each bring one query (bfloat16,
     values in transposed pages). Every position in `positions` must lie inside the pages its row
-    of `block_tables` has (checked by the caller on the host). `out`, if given, receives the result."""
+    of `block_tables` has (checked by the caller on the host). `out`, if given, receives the result.
+    `pages_per_entry`: as for `paged_attention_wave`."""
     _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions)
     _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
     T, nh, hd = q.shape
@@ -350,7 +360,7 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     for name, t in (("seq_of_token", seq_of_token), ("positions", positions)):
         _need(t.dtype == torch.int32 and t.shape == (T,) and t.is_contiguous(), f"{name} must be int32 [tokens]")
     _need(T <= MAX_DECODE_TOKENS, f"the decode kernel takes up to {MAX_DECODE_TOKENS} tokens a launch")
-    capacity = block_tables.shape[1] * k_cache.shape[1]
+    capacity = block_tables.shape[1] * pages_per_entry * k_cache.shape[1]
     if chunk is None:
         chunk, waves = decode_plan(T, nkv, nh // nkv, hd, capacity)
     waves = waves or 4
@@ -367,7 +377,7 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
         _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
         _ptr(seq_of_token), _ptr(positions), T, nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3],
         v_cache.stride(0), v_cache.stride(2), v_cache.stride(3), block_tables.shape[1], splits, chunk, waves,
-        float(scale), int(window), _stream()))
+        float(scale), int(window), _page_run(pages_per_entry), _stream()))
     return out
 
 
@@ -556,7 +566,8 @@ def attention_tiles(cu_seqlens: list[int], starts: list[int], tokens_per_tile: i
 def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                             seq_of_token: torch.Tensor, positions: torch.Tensor, tiles: torch.Tensor, scale: float,
                             window: int = 0, tile_tokens: int | None = None, out: torch.Tensor | None = None,
-                            num_splits: int = 1, chunk: int = 0, first_token: int = 0, waves: int = PREFILL_WAVES) -> torch.Tensor:
+                            num_splits: int = 1, chunk: int = 0, first_token: int = 0, waves: int = PREFILL_WAVES,
+                            pages_per_entry: int = 1) -> torch.Tensor:
     """Attention of a packed step on the matrix cores (bfloat16, values in transposed pages).
     `tiles` int32 [num_tiles, 2] lists (first token, token count <= tile_tokens) per workgroup,
     every tile inside one request and inside the step (the caller built the list from the step's
@@ -597,7 +608,7 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_of_token), _ptr(positions),
         _ptr(tiles), tiles.shape[0], tile_tokens, waves, nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3], v_cache.stride(0),
         v_cache.stride(2), v_cache.stride(3), block_tables.shape[1], float(scale), int(window), first_token, T,
-        num_splits, chunk, _ptr(part_o), _ptr(part_ml), _stream()))
+        num_splits, chunk, _ptr(part_o), _ptr(part_ml), _page_run(pages_per_entry), _stream()))
     return out
 
 
@@ -607,11 +618,16 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     float32 always takes the one-wave-per-row kernel, whose sums do not depend on the batch;
     bfloat16 takes the matrix-core kernels where they serve the shape."""
     tables = ctx.block_tables[space]
+    # (the tables count in pages of ctx.page_size tokens; the pools may be cut into shorter ones)
+    table_page = getattr(ctx, "page_size", 0) or k_cache.shape[1]
+    _need(table_page % k_cache.shape[1] == 0, f"block tables in pages of {table_page} over a cache in pages of {k_cache.shape[1]}")
+    per_entry = table_page // k_cache.shape[1]
     if decode_kernel_takes(q, k_cache, v_cache):
-        capacity = tables.shape[1] * k_cache.shape[1]
+        capacity = tables.shape[1] * table_page
         decode_ok = -(-capacity // 1024) <= MAX_DECODE_SPLITS and q.shape[0] <= MAX_DECODE_TOKENS
         if ctx.max_query_len == 1 and decode_ok:
-            return paged_attention_decode(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, window)
+            return paged_attention_decode(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, window,
+                                          pages_per_entry=per_entry)
         # the one-token requests that lead the step go to the split-key kernel, the rest to the tiles
         cu = ctx.host_cu_seqlens
         lead = 0
@@ -630,12 +646,13 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         out = torch.empty_like(q)
         if lead:
             paged_attention_decode(q[:lead], k_cache, v_cache, tables, ctx.seq_of_token[:lead], ctx.positions[:lead],
-                                   scale, window, out=out[:lead])
+                                   scale, window, out=out[:lead], pages_per_entry=per_entry)
         splits, chunk = prefill_splits(tiles.shape[0] * nkv, max(ctx.host_context_lens[lead:], default=0))
         return paged_attention_prefill(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, tiles, scale,
                                        window, tile_tokens=tile_tokens, out=out, num_splits=splits, chunk=chunk,
-                                       first_token=cu[lead], waves=waves)
-    return paged_attention_wave(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, window)
+                                       first_token=cu[lead], waves=waves, pages_per_entry=per_entry)
+    return paged_attention_wave(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, window,
+                                pages_per_entry=per_entry)
 
 
 SKINNY_MAX_ROWS = 32

@@ -77,13 +77,15 @@ class StepContext:
     context_lens: torch.Tensor            # [S] int32, keys of each request after this step's writes
     state_slots: torch.Tensor             # [S] int32
     slot_mapping: list[torch.Tensor]      # per space: [T] int32, page * page_size + offset
-    block_tables: list[torch.Tensor]      # per space: [S, max_pages] int32
+    block_tables: list[torch.Tensor]      # per space: [S, max_pages] int32, in pages of `page_size` tokens
     host_cu_seqlens: list[int] = field(default_factory=list)
     host_starts: list[int] = field(default_factory=list)      # first position fed, per request
     host_context_lens: list[int] = field(default_factory=list)
     host_state_slots: list[int] = field(default_factory=list)
     position_encodings: dict[str, "PositionEncoding"] = field(default_factory=dict)
     scratch: dict = field(default_factory=dict)     # what parts derive from a step once and share
+    page_size: int = 0                    # tokens per entry of the block tables (0: a page of the cache views; the pools may
+                                          # be cut into shorter pages, entry e then standing for the consecutive pages e n + j)
 
     @property
     def max_query_len(self) -> int:
