@@ -576,7 +576,8 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     With `num_splits` > 1 every tile's keys are walked in that many chunks of `chunk` keys (a
     multiple of 32; the last takes every key from its start on) by workgroups of their own, and the
     chunks are combined afterwards: for steps of few tokens over long contexts, which have too few
-    tiles to fill the chip. The tiles must then list every token from `first_token` on."""
+    tiles to fill the chip. The tiles must then list every token from `first_token` on.
+    `pages_per_entry`: as for `paged_attention_wave`."""
     _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles)
     _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
     T, nh, hd = q.shape
