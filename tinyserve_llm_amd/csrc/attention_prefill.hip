@@ -25,17 +25,23 @@
 
 #define PRE_MAX_WAVES 8
 
+// Where the steps of a walk lie (whole steps only: pages of a multiple of 32 keys): a ring of PRE_PLACES steps, refilled
+// by halves, that holds for step i what its page and slot add to a lane's fixed place in the keys' pool and in the
+// values'. The walk reads a step's entry instead of looking its page up and multiplying.
+#define PRE_PLACES 256
 template <int HD>
 struct PrefillLds {
   uint4 stage[2][HD / 8][TS_WAVE];   // two steps of operand registers, [register][lane]
   int range[4][PRE_MAX_WAVES];
+  int64_t place[2][PRE_PLACES];      // [keys | values][step mod PRE_PLACES], in elements
 };
 
 // PRE_WAVES: 4, or 8 (heads of 64 or 128 dimensions): the same tokens a workgroup in tiles half as
 // large a wave, so that a step's vector work is spread over twice the waves; the longest tiles of a
 // short prompt, which run alone at the end, then take a shorter step (2,048 tokens at head size 64:
 // 48.9 µs against 51.3; over long contexts the doubled reads of LDS cost more than that gains).
-template <int HD, int RT, int PRE_WAVES>
+// WHOLE: a page holds a multiple of 32 keys, so that every step lies in one page.
+template <int HD, int RT, int PRE_WAVES, bool WHOLE>
 static __device__ __forceinline__ void
 prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
              const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
@@ -149,36 +155,46 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
   constexpr int PER = 4 * NC / PRE_WAVES;
   static_assert(PER >= 1 && PER * PRE_WAVES == 4 * NC, "the waves share a step's operand registers evenly");
   uint4 fetched[PER];
-  const bool whole = pm.whole_steps();
   const bool loads_k = wave * PER < 2 * NC;           // (a wave's registers are all of K or all of V)
   const int tau = (wave * PER) / NC, c0 = (wave * PER) % NC, db0 = wave * PER - 2 * NC;
-  auto fetch = [&](int kb) {
-    if (whole) {
-      // one page for the whole step: its base addresses are scalars, the lanes add fixed offsets
+  const int kbeg = wlo & ~31;
+  const int kend = whi + 1;
+  // Whole steps: a lane's pieces lie at the same places of every page, so what the lane adds to a step's
+  // place is worked out once, and the steps' places come from the ring in LDS.
+  const int koff = 8 * (r >> 2) + 4 * tau + (r & 3);
+  const bf16_t* const lane_base = loads_k ? k_cache + ((int64_t)kvh * kh + (int64_t)koff * ks + 8 * g + 32 * c0)
+                                          : v_cache + ((int64_t)kvh * vh + 8 * g + (int64_t)(db0 * 16 + r) * vd);
+  const int64_t piece = loads_k ? 32 : 16 * vd;
+  const int lane_first = loads_k ? koff : 8 * g, lane_last = loads_k ? koff : 8 * g + 7;   // the keys a piece holds
+  const int64_t* const places = lds.place[loads_k ? 0 : 1];
+  // the places of the walk's steps first .. first + count - 1 go into the ring (steps beyond the last one: the
+  // last one's, whose page is the request's as well)
+  auto fill_places = [&](int first, int count) {
+    for (int i = threadIdx.x; i < count; i += PRE_WAVES * TS_WAVE) {
+      const int kb = min(kbeg + 32 * (first + i), whi & ~31);
       const int pg = pm.page(kb);
       const int64_t page = pm.pool_page(table, pg);
       const int slot = pm.slot(kb, pg);
-      const bool inner = kb >= wlo && kb + 31 <= whi;
-      const bf16_t* src;              // this lane's first piece; the others follow at a fixed stride
-      int64_t stride;
-      bool ok;
-      if (loads_k) {
-        const int koff = 8 * (r >> 2) + 4 * tau + (r & 3);
-        src = k_cache + page * kp + (int64_t)slot * ks + (int64_t)kvh * kh + (int64_t)koff * ks + 8 * g + 32 * c0;
-        stride = 32;
-        ok = kb + koff <= whi && kb + koff >= wlo;
-      } else {
-        src = v_cache + page * vp + slot + (int64_t)kvh * vh + 8 * g + (int64_t)(db0 * 16 + r) * vd;
-        stride = 16 * vd;
-        ok = kb + 8 * g <= whi && kb + 8 * g + 7 >= wlo;
-      }
-      if (inner) {                    // nearly every step: nothing to leave out, nothing to clear
+      lds.place[0][(first + i) & (PRE_PLACES - 1)] = page * kp + (int64_t)slot * ks;
+      lds.place[1][(first + i) & (PRE_PLACES - 1)] = page * vp + slot;
+    }
+  };
+  auto place_of = [&](int kb) { return places[((kb - kbeg) >> 5) & (PRE_PLACES - 1)]; };
+  // asks for the step at kb, which lies at `place` (whole steps; kb may lie beyond the walk: nothing is loaded then)
+  auto fetch_at = [&](int kb, int64_t place) {
+    const bf16_t* src = lane_base + place;
+    if (kb >= wlo && kb + 31 <= whi) {              // nearly every step: nothing to leave out, nothing to clear
 #pragma unroll
-        for (int c = 0; c < PER; ++c) fetched[c] = *(const uint4*)(src + c * stride);
-      } else {
+      for (int c = 0; c < PER; ++c) fetched[c] = *(const uint4*)(src + c * piece);
+    } else {
+      const bool ok = kb + lane_first <= whi && kb + lane_last >= wlo;
 #pragma unroll
-        for (int c = 0; c < PER; ++c) fetched[c] = ok ? *(const uint4*)(src + c * stride) : make_uint4(0, 0, 0, 0);
-      }
+      for (int c = 0; c < PER; ++c) fetched[c] = ok ? *(const uint4*)(src + c * piece) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto fetch = [&](int kb) {
+    if constexpr (WHOLE) {
+      fetch_at(kb, place_of(kb));
       return;
     }
 #pragma unroll
@@ -207,8 +223,6 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
     for (int c = 0; c < PER; ++c) stage[buf][wave * PER + c][lane] = fetched[c];
   };
 
-  const int kbeg = wlo & ~31;
-  const int kend = whi + 1;
   // The walk has three stretches: steps that some row sees in part (before the last window start),
   // steps that every row of the workgroup sees whole, and the steps around the rows' own positions.
   // The middle one, nearly all of a long walk, runs without masks and without the test whether a
@@ -217,16 +231,32 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
   const int full_lo = min(max((wfull_lo + 31) & ~31, kbeg), kend);
   const int full_hi = min(max(wfull_hi == 0x7fffffff ? 0 : ((wfull_hi + 1) & ~31), full_lo), kend);
   int buf = 0;
+  int64_t place_next = 0;                    // whole steps: the place of the step two ahead, read a step early
   auto walk = [&](int from, int to, auto masked) {
     for (int kb = from; kb < to; kb += 32, buf ^= 1) {
+      int64_t place_now = 0;
+      if constexpr (WHOLE) {
+        // every half turn of the ring the half that the walk has left behind takes the places of the steps
+        // a turn ahead (first read half a turn from now, many barriers later)
+        const int step = (kb - kbeg) >> 5;
+        if ((step & (PRE_PLACES / 2 - 1)) == 0 && step) fill_places(step + PRE_PLACES / 2, PRE_PLACES / 2);
+        place_now = place_next;
+        place_next = place_of(kb + 96);
+      }
       KVTile<HD> T;
 #pragma unroll
       for (int c = 0; c < NC; ++c) { T.k[0][c] = stage[buf][c][lane]; T.k[1][c] = stage[buf][NC + c][lane]; }
 #pragma unroll
       for (int db = 0; db < NDB; ++db) T.v[db] = stage[buf][2 * NC + db][lane];
       T.vok = true;                          // (what lies outside the range went into LDS as zeros)
-      if (kb + 32 < kend) put(buf ^ 1);      // the other buffer was last read before the previous barrier
-      if (kb + 64 < kend) fetch(kb + 64);
+      if constexpr (WHOLE) {
+        // (no tests for the walk's end: past it zeros are put where nobody reads, and nothing is asked for)
+        put(buf ^ 1);                        // the other buffer was last read before the previous barrier
+        fetch_at(kb + 64, place_now);
+      } else {
+        if (kb + 32 < kend) put(buf ^ 1);
+        if (kb + 64 < kend) fetch(kb + 64);
+      }
 #pragma unroll
       for (int j = 0; j < RT; ++j) {
         if constexpr (decltype(masked)::value) {
@@ -241,6 +271,11 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
     }
   };
   if (kbeg < kend) {                         // uniform over the workgroup
+    if constexpr (WHOLE) {
+      fill_places(0, PRE_PLACES);
+      __syncthreads();
+      place_next = place_of(kbeg + 64);
+    }
     fetch(kbeg);
     put(0);
     if (kbeg + 32 < kend) fetch(kbeg + 32);
@@ -277,7 +312,7 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
     }
 }
 
-template <int HD, int RT, int PRE_WAVES>
+template <int HD, int RT, int PRE_WAVES, bool WHOLE>
 __global__ void __launch_bounds__(PRE_WAVES * TS_WAVE)
 attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
                          const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables,
@@ -294,7 +329,7 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
   if (item >= num_tiles * heads_per_group) return;
   const int tile = num_tiles - 1 - item / heads_per_group;
   const int kvh = (die / dies_per_group) * heads_per_group + item % heads_per_group;
-  prefill_tile<HD, RT, PRE_WAVES>(lds, tile, kvh, out, q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, nh,
+  prefill_tile<HD, RT, PRE_WAVES, WHOLE>(lds, tile, kvh, out, q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, nh,
                        G, page_size, page_shift, page_run, kp, ks, kh, vp, vh, vd, max_blocks, scale2, window, part_o, part_ml,
                        num_splits, chunk, blockIdx.y);
 }
@@ -338,7 +373,9 @@ extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* 
   if (turns * 8 > 0x7fffffff) return TS_BAD_SHAPE;
   dim3 grid((unsigned)(8 * turns), num_splits);
 #define TS_PRE_W(HH, RR, WW)                                                                                    \
-  attn_prefill_mfma_kernel<HH, RR, WW><<<grid, WW * TS_WAVE, 0, stream>>>(                                      \
+  if (page_size % 32 == 0) TS_PRE_P(HH, RR, WW, true); else TS_PRE_P(HH, RR, WW, false)
+#define TS_PRE_P(HH, RR, WW, PP)                                                                                \
+  attn_prefill_mfma_kernel<HH, RR, WW, PP><<<grid, WW * TS_WAVE, 0, stream>>>(                                  \
       (bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,             \
       seq_of_token, positions, tiles, num_tiles, nh, G, dies_per_group, heads_per_group, page_size, page_shift, page_run, kp,  \
       ks, kh, vp, vh, vd, max_blocks, scale * 1.44269504088896340736f, window, part_o, part_ml, num_splits, chunk)
@@ -364,6 +401,7 @@ extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* 
 #undef TS_PRE_RT8
 #undef TS_PRE_RT
 #undef TS_PRE_W
+#undef TS_PRE_P
   const int rc = ts_check_launch();
   if (rc || num_splits == 1) return rc;
   const int64_t skip = (int64_t)first_token * nh;     // rows of the tokens before the first listed one
