@@ -47,16 +47,15 @@ extern "C" int ts_embedding(void* out, const void* table, const int32_t* ids, in
 template <typename T> struct Pack16;   // a 16-byte piece of a row as floats
 template <> struct Pack16<float> {
   static constexpr int N = 4;
-  static __device__ __forceinline__ void ld(const float* p, float* f) {
-    const float4 v = *(const float4*)p;
-    f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+  static __device__ __forceinline__ void unpack(const uint4 v, float* f) {
+    f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y); f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
   }
+  static __device__ __forceinline__ void ld(const float* p, float* f) { unpack(*(const uint4*)p, f); }
   static __device__ __forceinline__ void st(float* p, const float* f) { *(float4*)p = make_float4(f[0], f[1], f[2], f[3]); }
 };
 template <> struct Pack16<bf16_t> {
   static constexpr int N = 8;
-  static __device__ __forceinline__ void ld(const bf16_t* p, float* f) {
-    const uint4 v = *(const uint4*)p;
+  static __device__ __forceinline__ void unpack(const uint4 v, float* f) {
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -64,6 +63,7 @@ template <> struct Pack16<bf16_t> {
       f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
     }
   }
+  static __device__ __forceinline__ void ld(const bf16_t* p, float* f) { unpack(*(const uint4*)p, f); }
   static __device__ __forceinline__ void st(bf16_t* p, const float* f) {
     uint32_t w[4];
 #pragma unroll
@@ -122,15 +122,29 @@ rmsnorm_row_kernel(T* __restrict__ out, T* __restrict__ res_out, const T* __rest
   const T* rr = res ? res + src * hidden : nullptr;
   const int pieces = hidden / N;
   float v[NORM_MAX_CHUNKS][N];
+  // everything the thread reads is asked for at once, the weights' pieces too, which are used only after the
+  // barrier (without a residual the row is asked for twice, the second time from the cache: no test stands
+  // between the loads that would make one wait for the other)
+  uint4 xraw[NORM_MAX_CHUNKS], rraw[NORM_MAX_CHUNKS], wraw[NORM_MAX_CHUNKS];
+  const T* rsrc = rr ? rr : xr;
+#pragma unroll
+  for (int c = 0; c < NORM_MAX_CHUNKS; ++c) {
+    const int i = threadIdx.x + c * NORM_THREADS;
+    if (i < pieces) {
+      xraw[c] = *(const uint4*)(xr + (int64_t)i * N);
+      rraw[c] = *(const uint4*)(rsrc + (int64_t)i * N);
+      wraw[c] = *(const uint4*)(w + (int64_t)i * N);
+    }
+  }
   float acc = 0.f;
 #pragma unroll
   for (int c = 0; c < NORM_MAX_CHUNKS; ++c) {
     const int i = threadIdx.x + c * NORM_THREADS;
     if (i < pieces) {
-      Pack16<T>::ld(xr + (int64_t)i * N, v[c]);
+      Pack16<T>::unpack(xraw[c], v[c]);
       if (rr) {
         float t[N];
-        Pack16<T>::ld(rr + (int64_t)i * N, t);
+        Pack16<T>::unpack(rraw[c], t);
 #pragma unroll
         for (int k = 0; k < N; ++k) v[c][k] += t[k];
       }
@@ -153,7 +167,7 @@ rmsnorm_row_kernel(T* __restrict__ out, T* __restrict__ res_out, const T* __rest
     if (i < pieces) {
       if (rorow) Pack16<T>::st(rorow + (int64_t)i * N, v[c]);
       float wv[N];
-      Pack16<T>::ld(w + (int64_t)i * N, wv);
+      Pack16<T>::unpack(wraw[c], wv);
 #pragma unroll
       for (int k = 0; k < N; ++k) v[c][k] = Num<T>::round(v[c][k] * inv) * wv[k];
       Pack16<T>::st(orow + (int64_t)i * N, v[c]);
@@ -253,24 +267,35 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
       const int h = e / per_head, piece = e - h * per_head;
       const bool is_k = h >= nh, passes = piece >= turning;
       const int j = passes ? rot + (piece - turning) * V : piece * V;
-      if (is_k && (!k_cache || slots[t] < 0)) continue;
+      if (is_k && !k_cache) continue;
+      // the token's slot and position and both pieces are asked for together (a piece that passes asks for
+      // itself twice), then the table's rows for the position: two trips to memory, not four
       const T* src = qkv + (int64_t)t * row + h * hd;      // k heads follow the q heads in a row
+      const int slot = k_cache ? slots[t] : 0, position = positions[t];
+      const uint4 raw1 = *(const uint4*)(src + j), raw2 = *(const uint4*)(src + (passes ? j : j + half));
       float x1[V], x2[V];
-      Pack16<T>::ld(src + j, x1);
-      if (!passes) Pack16<T>::ld(src + j + half, x2);
+      Pack16<T>::unpack(raw1, x1);
+      Pack16<T>::unpack(raw2, x2);
       if (rotate && !passes) {
-        const float* cs = cos_sin + (int64_t)positions[t] * rot;
+        const float* cs = cos_sin + (int64_t)position * rot + j;      // (16-byte aligned: rot and j are multiples of V)
+        float c[V], sn[V];
+#pragma unroll
+        for (int k = 0; k < V; k += 4) {
+          const float4 cv = *(const float4*)(cs + k), sv = *(const float4*)(cs + half + k);
+          c[k] = cv.x; c[k + 1] = cv.y; c[k + 2] = cv.z; c[k + 3] = cv.w;
+          sn[k] = sv.x; sn[k + 1] = sv.y; sn[k + 2] = sv.z; sn[k + 3] = sv.w;
+        }
 #pragma unroll
         for (int k = 0; k < V; ++k) {
-          const float c = cs[j + k], sn = cs[half + j + k];
-          const float y1 = x1[k] * c - x2[k] * sn, y2 = x2[k] * c + x1[k] * sn;
+          const float y1 = x1[k] * c[k] - x2[k] * sn[k], y2 = x2[k] * c[k] + x1[k] * sn[k];
           x1[k] = y1;
           x2[k] = y2;
         }
       }
+      if (is_k && slot < 0) continue;
       T* dst;
       if (is_k) {
-        const int slot = slots[t], pg = page_of(slot);
+        const int pg = page_of(slot);
         dst = k_cache + (int64_t)pg * kp + (int64_t)(slot - pg * page_size) * ks + (int64_t)(h - nh) * kh;
       } else {
         dst = q_out + ((int64_t)t * nh + h) * hd;
@@ -399,12 +424,15 @@ extern "C" int ts_rope_store(void* q_out, void* k_cache, void* v_cache, const vo
   int slices = 2048 / groups;                       // enough workgroups to hide the loads' latency
   if (slices < 1) slices = 1;
   if (slices > 32) slices = 32;
+  // (no more slices than give each of a workgroup's threads a piece of q or k)
+  const int group_pieces = ROPE_TOK * (nh + nkv) * ((hd + (dtype == 0 ? 4 : 8) - 1) / (dtype == 0 ? 4 : 8)) / 2;
+  if (slices > (group_pieces + 255) / 256) slices = (group_pieces + 255) / 256;
   dim3 blocks(groups, slices);
   // 16-byte pieces need halves of whole pieces and aligned rows everywhere
   const int per16 = dtype == 0 ? 4 : 8;
   const int row = (nh + 2 * nkv) * hd;
   const int vec = (rot / 2) % per16 == 0 && (hd - rot) % per16 == 0 && hd % per16 == 0 && row % per16 == 0 && kp % per16 == 0 && ks % per16 == 0 && kh % per16 == 0 &&
-                  ((((uintptr_t)q_out) | ((uintptr_t)k_cache) | ((uintptr_t)qkv)) & 15) == 0;
+                  ((((uintptr_t)q_out) | ((uintptr_t)k_cache) | ((uintptr_t)qkv) | ((uintptr_t)cos_sin)) & 15) == 0;
   // values through LDS: bfloat16 steps of several tokens into transposed pages (slot stride 1) whose
   // 8-slot pieces are 16-byte aligned
   const int vtile = dtype == 1 && num_tokens >= 8 && v_cache && vs == 1 && row % 8 == 0 && ((nh + nkv) * hd) % 8 == 0 &&
@@ -431,6 +459,19 @@ extern "C" int ts_rope_store(void* q_out, void* k_cache, void* v_cache, const vo
 // ------------------------------------------------------------------------------------------
 // SiLU gate: out[t, i] = silu(gu[t, i]) * gu[t, inter + i]  (gate in the first half of a row)
 // ------------------------------------------------------------------------------------------
+// silu(g) for a result that is stored in 32 bits: the library's exponential and a true division. For bfloat16
+// results the hardware's 2^x and reciprocal, each good to a unit in the last place of 32 bits (what the
+// projections' gate epilogue uses): a piece of 8 elements costs a fifth of the instructions.
+template <typename T> struct Gate;
+template <> struct Gate<float> {
+  static __device__ __forceinline__ float silu(float g) { return g / (1.0f + expf(-g)); }
+};
+template <> struct Gate<bf16_t> {
+  static __device__ __forceinline__ float silu(float g) {
+    return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896340736f * g));
+  }
+};
+
 template <typename T>
 __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, int64_t total, int inter) {
   for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
@@ -439,26 +480,38 @@ __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, i
     const int i = (int)(idx - t * inter);
     const float g = Num<T>::ld(gu + t * 2 * inter + i);
     const float u = Num<T>::ld(gu + t * 2 * inter + inter + i);
-    const float a = g / (1.0f + expf(-g));
-    Num<T>::st(out + idx, a * u);
+    Num<T>::st(out + idx, Gate<T>::silu(g) * u);
   }
 }
 
-// 16 bytes of gate and of up per thread; for widths that are whole numbers of such pieces
+// 16 bytes of gate and of up at a time, SILU_PIECES such pieces a thread (a workgroup's threads side by side in
+// each), all of them asked for before the first is used; for widths that are whole numbers of pieces. A workgroup
+// works on one token (blockIdx.x) and on 256 SILU_PIECES pieces of its row (blockIdx.y): nothing is divided.
+#define SILU_PIECES 4
 template <typename T>
-__global__ void silu_mul_vec_kernel(T* __restrict__ out, const T* __restrict__ gu, int64_t pieces, int inter) {
+__global__ void __launch_bounds__(256)
+silu_mul_vec_kernel(T* __restrict__ out, const T* __restrict__ gu, int inter) {
   constexpr int N = Pack16<T>::N;
   const int per_row = inter / N;
-  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < pieces;
-       idx += (int64_t)gridDim.x * blockDim.x) {
-    const int64_t t = idx / per_row;
-    const int i = (int)(idx - t * per_row) * N;
-    float g[N], u[N];
-    Pack16<T>::ld(gu + t * 2 * inter + i, g);
-    Pack16<T>::ld(gu + t * 2 * inter + inter + i, u);
+  const T* row = gu + (int64_t)blockIdx.x * 2 * inter;
+  T* orow = out + (int64_t)blockIdx.x * inter;
+  const int first = blockIdx.y * (256 * SILU_PIECES) + threadIdx.x;
+  uint4 graw[SILU_PIECES], uraw[SILU_PIECES];
 #pragma unroll
-    for (int k = 0; k < N; ++k) g[k] = g[k] / (1.0f + expf(-g[k])) * u[k];
-    Pack16<T>::st(out + t * inter + i, g);
+  for (int p = 0; p < SILU_PIECES; ++p) {
+    // (a piece past the row's end is its last piece once more: loads without a test between them all go out at once)
+    const int i = min(first + p * 256, per_row - 1) * N;
+    graw[p] = *(const uint4*)(row + i);
+    uraw[p] = *(const uint4*)(row + inter + i);
+  }
+#pragma unroll
+  for (int p = 0; p < SILU_PIECES; ++p) {
+    float g[N], u[N];
+    Pack16<T>::unpack(graw[p], g);
+    Pack16<T>::unpack(uraw[p], u);
+#pragma unroll
+    for (int k = 0; k < N; ++k) g[k] = Gate<T>::silu(g[k]) * u[k];
+    if (first + p * 256 < per_row) Pack16<T>::st(orow + (int64_t)(first + p * 256) * N, g);
   }
 }
 
@@ -468,13 +521,13 @@ extern "C" int ts_silu_mul(void* out, const void* gu, int num_tokens, int inter,
   if (dtype != 0 && dtype != 1) return TS_BAD_DTYPE;
   const int per16 = dtype == 0 ? 4 : 8;
   if (inter % per16 == 0 && ((((uintptr_t)out) | ((uintptr_t)gu)) & 15) == 0) {
-    const int64_t pieces = total / per16;
-    int64_t blocks = (pieces + 255) / 256;
-    if (blocks > 16384) blocks = 16384;
+    const int chunks = (inter / per16 + 256 * SILU_PIECES - 1) / (256 * SILU_PIECES);
+    if (chunks > 65535) return TS_BAD_SHAPE;
+    const dim3 blocks(num_tokens, chunks);
     if (dtype == 0)
-      silu_mul_vec_kernel<float><<<(int)blocks, 256, 0, stream>>>((float*)out, (const float*)gu, pieces, inter);
+      silu_mul_vec_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)gu, inter);
     else
-      silu_mul_vec_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, pieces, inter);
+      silu_mul_vec_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, inter);
     return ts_check_launch();
   }
   int64_t blocks = (total + 255) / 256;
