@@ -7,10 +7,14 @@
 //   four compute waves, one 16-row tile of W each over the whole of K: the tile streams from memory
 //   straight into MFMA operands, 16 steps of 32 k under way at any time (a step's register is asked for
 //   again as soon as it has been used), and the four 16-row blocks of x come out of LDS;
-//   four staging waves, which bring x into LDS in chunks of 256 k, in the order the lanes read it, one
-//   chunk ahead of the compute waves (two buffers, a barrier per chunk). Their loads are few and hit the
-//   cache; in waves of their own they do not queue behind the loads of W (a wave's loads come back in
-//   the order it asked).
+//   four staging waves, which bring x into LDS in chunks of 256 k, one chunk ahead of the compute waves
+//   (two buffers, a barrier per chunk). A staging wave takes a block of 16 rows, and each of its loads
+//   512 contiguous bytes of two rows (an instruction that gathered 64 bytes of each of 16 rows, the
+//   order in which the matrix instruction wants them, cost the gate|up product of 64 rows 1.7 of 20 us
+//   and 7.5 of 62 at the 8B widths); the pieces go into LDS where the compute lanes look for them, with
+//   the place inside a block of 16 rows turned by the piece's step and part of k so that neither the
+//   writes nor the reads meet in a bank. Their loads hit the cache; in waves of their own they do not
+//   queue behind the loads of W (a wave's loads come back in the order it asked).
 // The gate can ride along as in gemm_skinny.hip:
 //   GLU   W = [gate rows | up rows]: waves 0 and 1 take two gate tiles, waves 2 and 3 the up tiles
 //         N / 2 rows below them, and y [M, N / 2] = silu(gate) * up
@@ -33,7 +37,11 @@
 #define R64_CHUNK_STEPS 8         // 32-wide k steps per chunk of x in LDS
 #define R64_RING 16               // steps of W a compute wave has under way (two chunks): with 32 the chip had 32 MB under way and
                                   // every load, x's among them, came back some 5 us later (the gate|up product of 64 rows 20.7 us, 19.7 with 16)
-#define R64_STAGE_STEPS (R64_CHUNK_STEPS / 4)   // steps of a chunk that one staging wave brings
+#define R64_STAGE_LOADS 8          // loads of a staging wave per chunk: two rows of its block each
+// where in a block's [64] the piece of row r (of 16), step s, k = 8 g .. 8 g + 7 lies: the 16 pieces that the lanes of a
+// staging wave's load write side by side (one row, 4 steps x 4 g) land in 16 different places, and a compute
+// wave's 64 lanes (16 rows x 4 g of one step) read 64 different places
+static __device__ __forceinline__ int r64_place(int r, int s, int g) { return (r ^ ((g + 4 * s) & 15)) + 16 * g; }
 
 struct Rows64Args {
   const bf16_t* x;       // [M, K], row stride ldx
@@ -62,31 +70,32 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
   const int64_t kfirst = (int64_t)slice * nsteps * SK_KSTEP;                  // the slice's first k
 
   if (wave >= 4) {
-    // ---- staging waves: wave sw brings steps 2 sw and 2 sw + 1 of every chunk, all four blocks of
-    // rows. It asks for the next chunk before it puts this one into LDS, so that a chunk costs the
-    // compute waves a barrier and not a trip to the cache.
-    const int sw = wave - 4;
-    bool ok[4];
-    int64_t xoff[4];
+    // ---- staging waves: wave sw brings block sw of 16 rows, all the steps of every chunk. It asks for
+    // the next chunk before it puts this one into LDS, so that a chunk costs the compute waves a barrier
+    // and not a trip to the cache.
+    const int sw = wave - 4;                              // this wave's block of 16 rows
+    const int half = lane >> 5, kl = lane & 31;           // the row of a load's two, and the piece of its 256 k
+    bool ok[R64_STAGE_LOADS];
+    int64_t xoff[R64_STAGE_LOADS];
+    int slot[R64_STAGE_LOADS];
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      ok[b] = 16 * b + r < a.M;                          // rows past M read row 0 and count as zeros
-      xoff[b] = (int64_t)(ok[b] ? 16 * b + r : 0) * a.ldx + kfirst + 8 * g;
+    for (int j = 0; j < R64_STAGE_LOADS; ++j) {
+      const int r = 2 * j + half, m = 16 * sw + r;
+      ok[j] = m < a.M;                                    // rows past M read row 0 and count as zeros
+      xoff[j] = (int64_t)(ok[j] ? m : 0) * a.ldx + kfirst + 8 * kl;
+      slot[j] = ((kl >> 2) * 4 + sw) * TS_WAVE + r64_place(r, kl >> 2, kl & 3);      // in a buffer's [step][block][64]
     }
-    auto ask = [&](int c, uint4 (&t)[R64_STAGE_STEPS][4]) {
-      const int k0 = (c * R64_CHUNK_STEPS + R64_STAGE_STEPS * sw) * SK_KSTEP;   // first k of this wave's steps
+    auto ask = [&](int c, uint4 (&t)[R64_STAGE_LOADS]) {
+      const int k0 = c * R64_CHUNK_STEPS * SK_KSTEP;      // first k of the chunk
 #pragma unroll
-      for (int s = 0; s < R64_STAGE_STEPS; ++s)
-#pragma unroll
-        for (int b = 0; b < 4; ++b) t[s][b] = *(const uint4*)(a.x + xoff[b] + k0 + s * SK_KSTEP);
+      for (int j = 0; j < R64_STAGE_LOADS; ++j) t[j] = *(const uint4*)(a.x + xoff[j] + k0);
     };
-    auto put = [&](int c, const uint4 (&t)[R64_STAGE_STEPS][4]) {
+    auto put = [&](int c, const uint4 (&t)[R64_STAGE_LOADS]) {
+      uint4* buf = &xs[c & 1][0][0][0];
 #pragma unroll
-      for (int s = 0; s < R64_STAGE_STEPS; ++s)
-#pragma unroll
-        for (int b = 0; b < 4; ++b) xs[c & 1][R64_STAGE_STEPS * sw + s][b][lane] = ok[b] ? t[s][b] : make_uint4(0, 0, 0, 0);
+      for (int j = 0; j < R64_STAGE_LOADS; ++j) buf[slot[j]] = ok[j] ? t[j] : make_uint4(0, 0, 0, 0);
     };
-    uint4 A[R64_STAGE_STEPS][4], B[R64_STAGE_STEPS][4];
+    uint4 A[R64_STAGE_LOADS], B[R64_STAGE_LOADS];
     ask(0, A);
     for (int c = 0; c < nchunks; c += 2) {
       ask(c + 1, B);
@@ -115,6 +124,9 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
   float4_t acc[4];
 #pragma unroll
   for (int b = 0; b < 4; ++b) acc[b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+  int at[4];                    // where this lane's piece of a step lies in a block, by the step's last two bits
+#pragma unroll
+  for (int i = 0; i < 4; ++i) at[i] = r64_place(r, i, g);
   // the scales of this lane's rows: the parts of a row's sum of squares in ascending order. The wait is for
   // loads that come back behind the ring's first turn, which the first products wait for anyway (in the
   // staging waves a wait for the parts held the second chunk's request back by a trip to memory).
@@ -143,14 +155,14 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int b = 0; b < 4; ++b) xb[0][i][b] = xs[(base / R64_CHUNK_STEPS + h) & 1][i][b][lane];
+        for (int b = 0; b < 4; ++b) xb[0][i][b] = xs[(base / R64_CHUNK_STEPS + h) & 1][i][b][at[i & 3]];
 #pragma unroll
       for (int q = 0; q < PAIRS; ++q) {
         if (q + 1 < PAIRS) {
 #pragma unroll
           for (int i = 0; i < 2; ++i)
 #pragma unroll
-            for (int b = 0; b < 4; ++b) xb[(q + 1) & 1][i][b] = xs[(base / R64_CHUNK_STEPS + h) & 1][2 * (q + 1) + i][b][lane];
+            for (int b = 0; b < 4; ++b) xb[(q + 1) & 1][i][b] = xs[(base / R64_CHUNK_STEPS + h) & 1][2 * (q + 1) + i][b][at[(2 * (q + 1) + i) & 3]];
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
