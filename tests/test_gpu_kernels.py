@@ -1200,6 +1200,88 @@ def test_eight_row_form_of_the_weight_streaming_gemm(m, n, k):
         hip().gemm_skinny8(torch.cat([x, x])[:9].contiguous(), w)
 
 
+@pytest.mark.parametrize("m", [1, 3, 8])
+@pytest.mark.parametrize("k", [1024, 2048, 4096, 8192])
+def test_rows_in_the_order_the_eight_row_form_reads_them(m, k):
+    """Up to 8 rows packed lane by lane for the 8-row form: the packing and its inverse, the place of one
+    piece spelled out, and the product from packed rows bit for bit the product from the matrix, stored or
+    finished into the next norm. The lanes of the rows that are not there are filled with NaN: no row
+    that is there may see them."""
+    H = hip()
+    g = gen(7 * m + k)
+    steps = H.skinny8_steps(k)
+    x = torch.randn(m, k, generator=g).bfloat16().to(dev())
+    px = H.pack_rows8(x, steps)
+    assert px.shape == (m, k) and px.data.shape == (k // (64 * steps), steps, 64, 8)
+    assert torch.equal(px.rows(), x)
+    row, wave, half, step, part = m - 1, k // (64 * steps) - 1, 1, steps - 2, 3
+    at = 64 * steps * wave + 32 * steps * half + 32 * step + 8 * part
+    assert torch.equal(px.data[wave, step, row + 8 * half + 16 * part], x[row, at:at + 8])
+    lanes = px.data.view(-1, steps, 4, 2, 8, 8)
+    lanes[:, :, :, :, m:] = float("nan")
+    n = 2048
+    w = (torch.randn(n, k, generator=g) * 0.05).bfloat16().to(dev())
+    assert H.rows8_reader_steps(m, w) == steps
+    for packed8 in (None, H.pack_weight8(w)):
+        assert torch.equal(H.gemm_skinny8(px, w, packed8=packed8), H.gemm_skinny8(x, w, packed8=packed8))
+        assert torch.equal(H.gemm_skinny8(px, w, torch.float32, packed8=packed8), H.gemm_skinny8(x, w, torch.float32, packed8=packed8))
+    res = torch.randn(m, n, generator=g).bfloat16().to(dev())
+    nw = (1 + 0.1 * torch.randn(n, generator=g)).bfloat16().to(dev())
+    a, b = H.gemm_skinny8(px, w, next_norm=(res, nw)), H.gemm_skinny8(x, w, next_norm=(res, nw))
+    assert torch.equal(a.summed, b.summed) and torch.equal(a.operand, b.operand) and torch.equal(a.squares, b.squares)
+    assert torch.equal(H.linear_bf16(px, w), H.gemm_skinny8(x, w))
+    with pytest.raises(H.KernelError, match="steps"):
+        H.gemm_skinny8(H.PackedRows8(px.data, m, k, 4 if steps != 4 else 8), w)
+    wide = (torch.randn(4096, k, generator=g) * 0.05).bfloat16().to(dev())
+    assert H.rows8_reader_steps(m, wide) == steps and H.rows8_reader_steps(9, wide) == 0
+    assert torch.equal(H.linear_bf16(px, wide), H.gemm_skinny8(x, wide)), "packed rows go to the 8-row form at any width"
+
+
+@pytest.mark.parametrize("m", [2, 5, 8])
+@pytest.mark.parametrize("inter,k", [(8192, 2048), (1024, 512), (4096, 1024)])
+def test_gated_product_handed_on_in_the_eight_row_forms_order(m, inter, k):
+    """The gate|up projection of a few rows leaves silu(gate) * up in the order the down projection's kernel
+    reads it: the same numbers as the matrix it otherwise leaves, with the norm on the way in, prepared by the
+    kernel before, or absent; and through `linear` the two projections give what they give without it."""
+    H = hip()
+    from tinyserve_llm_amd.parts.linear import DeferredNorm, NormRequest, linear, streaming_copy
+    g = gen(m + inter + k)
+    gate_up = (torch.randn(2 * inter, k, generator=g) * k ** -0.5).bfloat16().to(dev())
+    down = (torch.randn(k, inter, generator=g) * inter ** -0.5).bfloat16().to(dev())
+    x = torch.randn(m, k, generator=g).bfloat16().to(dev())
+    steps = H.rows8_reader_steps(m, down)
+    assert steps == H.skinny8_steps(inter) > 0
+    plain = H.gemm_skinny(x, gate_up, glu=True)[0]
+    packed = H.gemm_skinny(x, gate_up, glu=True, pack8_steps=steps)[0]
+    assert isinstance(packed, H.PackedRows8) and packed.shape == (m, inter) and packed.steps == steps
+    assert torch.equal(packed.rows(), plain)
+    sq = (x.float() ** 2).sum(1, keepdim=True)
+    assert torch.equal(H.gemm_skinny(x, gate_up, glu=True, squares=sq, eps=1e-5, pack8_steps=steps)[0].rows(),
+                       H.gemm_skinny(x, gate_up, glu=True, squares=sq, eps=1e-5)[0])
+    if H.skinny_fuses(m, k, True, True):
+        nw = (1 + 0.1 * torch.randn(k, generator=g)).bfloat16().to(dev())
+        assert torch.equal(H.gemm_skinny(x, gate_up, norm_weight=nw, eps=1e-5, glu=True, pack8_steps=steps)[0].rows(),
+                           H.gemm_skinny(x, gate_up, norm_weight=nw, eps=1e-5, glu=True)[0])
+    with pytest.raises(H.KernelError, match="packed rows"):
+        H.gemm_skinny(x, gate_up, pack8_steps=steps)
+    # through the parts' projections: handed on packed, and not
+    res = torch.randn(m, k, generator=g).bfloat16().to(dev())
+    nw2 = (1 + 0.1 * torch.randn(k, generator=g)).bfloat16().to(dev())
+    copies = streaming_copy(gate_up), streaming_copy(down)
+    handed = linear(x, gate_up, glu=True, packed=copies[0], feeds=down)
+    assert isinstance(handed, H.PackedRows8)
+    kept = linear(x, gate_up, glu=True, packed=copies[0])
+    assert torch.equal(linear(handed, down, packed=copies[1]), linear(kept, down, packed=copies[1]))
+    a = linear(handed, down, packed=copies[1], then=NormRequest(nw2, 1e-5, res))
+    b = linear(kept, down, packed=copies[1], then=NormRequest(nw2, 1e-5, res))
+    assert isinstance(a, DeferredNorm) and a.prepared is not None
+    assert torch.equal(a.prepared.summed, b.prepared.summed) and torch.equal(a.prepared.operand, b.prepared.operand)
+    # a reader it was not made for gets the matrix
+    other = torch.zeros(64, inter, dtype=torch.bfloat16, device=dev())
+    assert linear(handed, other).shape == (m, 64)
+    assert not isinstance(linear(x[:1], gate_up, glu=True, packed=copies[0], feeds=down), H.PackedRows8), "one row is handed on as it is"
+
+
 @pytest.mark.parametrize("m", [17, 33, 50, 64])
 @pytest.mark.parametrize("n,k", [(8192, 1024), (16384, 2048), (9152, 3072)])
 def test_wide_product_for_a_few_dozen_rows(m, n, k):

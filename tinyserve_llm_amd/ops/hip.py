@@ -63,8 +63,8 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_gemm_library_timing": [i],
         "ts_gemm_library_choices": [p, i],
         "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, i, i, i, i, p, p, i, p],
-        "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p, i, p, p, p, p, p, p],
-        "ts_gemm_skinny8_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p, p, p, p, p, p],
+        "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p, i, p, p, p, p, p, i, p],
+        "ts_gemm_skinny8_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p, p, p, p, p, i, p],
         "ts_gemm_rows64_bf16": [p, p, p, i, i, i, i64, i64, i, i, p, i, f, p],
         "ts_gemm_rows64_sliced_bf16": [p, p, p, p, i, i, i, i64, i, p, p, p, p, p, i64, p],
         "ts_gemm_rows64_sliced_rope_bf16": [p, p, p, p, i, i, i64, i, p, i, f, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64,
@@ -699,15 +699,16 @@ def _gated_output(rows: int, width: int, device) -> torch.Tensor:
     return torch.empty((rows, width + skew), dtype=torch.bfloat16, device=device)[:, :width]
 
 
-def _next_norm_outputs(x: torch.Tensor, n: int, parts: int, next_norm, skew: int = 0) -> tuple[PreparedNorm, torch.Tensor | None, torch.Tensor]:
+def _next_norm_outputs(x: torch.Tensor, n: int, parts: int, next_norm, skew: int = 0,
+                       rows: int | None = None) -> tuple[PreparedNorm, torch.Tensor | None, torch.Tensor]:
     """Checks `next_norm` = (residual or None, weight) for a product [M, n] and makes its outputs.
     `skew`: the operand's rows lie n + skew elements apart. (The kernels that take it read the same
     64 bytes of 16 rows with one instruction; rows a power of two apart are slow to fetch that way:
     64 rows over 2,048 against the q|k|v weight 12.0 µs, 10.2 with rows 16 bytes further apart, against
-    the gate|up weight 20.4 and 18.9.)"""
+    the gate|up weight 20.4 and 18.9.) `rows`: the product's rows where x is not [M, K] itself."""
     residual, weight = next_norm
     _gpu(residual, weight)
-    M = x.shape[0]
+    M = x.shape[0] if rows is None else rows
     _need(weight.dtype == torch.bfloat16 and weight.shape == (n,) and weight.is_contiguous(), f"the next norm's weight must be bfloat16 [{n}]")
     if residual is not None:
         _need(residual.dtype == torch.bfloat16 and residual.shape == (M, n) and residual.is_contiguous(),
@@ -786,6 +787,52 @@ def skinny8_takes(rows: int, n: int, k: int) -> bool:
             and (rows <= SKINNY8_FEW_ROWS or n <= SKINNY8_FULL_WIDTH))
 
 
+class PackedRows8:
+    """Up to 8 rows of a bfloat16 matrix [rows, k] in the order the lanes of the 8-row form read their
+    x, for a reader of `steps` steps a wave: `data` [k / (64 steps), steps, 64, 8], lane r + 16 g of
+    (wave, step) holding row r % 8 at k = 64 steps wave + 32 steps (r // 8) + 32 step + 8 g .. + 7.
+    The kernel then loads contiguous kilobytes instead of 64 bytes of each row in two places (the
+    down projection of 8 rows over 8,192: 10.8 -> 9.2 µs). Lanes of rows past `rows` hold anything.
+    What makes it (`gemm_skinny` with `pack8_steps`) and what reads it (`gemm_skinny8`) are chosen
+    together by `linear`; nothing else takes it but `rows()`."""
+
+    def __init__(self, data: torch.Tensor, rows: int, k: int, steps: int) -> None:
+        self.data, self.num_rows, self.k, self.steps = data, rows, k, steps
+
+    @property
+    def shape(self) -> tuple[int, int]:
+        return (self.num_rows, self.k)
+
+    def rows(self) -> torch.Tensor:
+        """The matrix [rows, k] itself (a copy), for tests and for readers that take no packed operand."""
+        waves = self.k // (64 * self.steps)
+        # [wave, step, g, half, row, 8] -> [row, wave, half, step, g, 8]
+        return (self.data.view(waves, self.steps, 4, 2, 8, 8).permute(4, 0, 3, 1, 2, 5).reshape(8, self.k)[:self.num_rows]
+                .contiguous())
+
+
+def rows8_reader_steps(rows: int, weight: torch.Tensor) -> int:
+    """The steps of the `PackedRows8` that `linear_bf16` takes as the operand of a product of `rows`
+    rows by `weight`; 0: that product does not go to the 8-row form, its operand stays a matrix.
+    From packed rows the 8-row form is the fastest at every width (8 rows against the down weight of
+    3,072 x 8,192: 14.1 µs, 16.2 from a matrix by the 16-row form; 4,096 x 14,336: 26.0 against 26.6),
+    also where `skinny8_takes` leaves a matrix of so many rows to other kernels."""
+    if not (weight.is_cuda and weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous()
+            and weight.data_ptr() % 16 == 0):
+        return 0
+    return skinny8_steps(weight.shape[1]) if rows <= SKINNY8_MAX_ROWS else 0
+
+
+def pack_rows8(x: torch.Tensor, steps: int) -> PackedRows8:
+    """`x` [rows <= 8, k] as a `PackedRows8` for a reader of `steps` steps (rows past the last are zeros)."""
+    _need(x.dim() == 2 and x.dtype == torch.bfloat16 and x.shape[0] <= 8 and steps in (4, 8, 16) and x.shape[1] % (64 * steps) == 0,
+          "pack_rows8 takes bfloat16 [rows <= 8, k], k in whole waves of 64 steps")
+    rows, k = x.shape
+    full = x if rows == 8 else torch.cat([x, x.new_zeros(8 - rows, k)])
+    data = full.view(8, k // (64 * steps), 2, steps, 4, 8).permute(1, 3, 4, 2, 0, 5).contiguous().view(k // (64 * steps), steps, 64, 8)
+    return PackedRows8(data, rows, k, steps)
+
+
 def pack_weight8(weight: torch.Tensor) -> torch.Tensor:
     """A copy of bfloat16 `weight` [N, K] in the order the 8-row form reads it:
     [N / 8 tiles, waves, steps, 64 lanes, 8], lane r + 16 g holding row 8 tile + r % 8 at
@@ -802,24 +849,29 @@ def pack_weight8(weight: torch.Tensor) -> torch.Tensor:
             .view(tiles, waves, steps, 64, 8))
 
 
-def gemm_skinny8(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
+def gemm_skinny8(x: "torch.Tensor | PackedRows8", weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
                  packed8: torch.Tensor | None = None, next_norm=None) -> "torch.Tensor | PreparedNorm":
     """bfloat16 x [M <= 8, K] · weight [N, K]^T by the weight-streaming kernel's 8-row form (a matrix
     instruction multiplies 8 rows of W by 8 rows of x over 64 k; a workgroup owns 8 rows of W).
-    With `packed8` (= pack_weight8(weight)) the kernel reads that copy. With `next_norm` =
-    (residual or None, weight of the norm that follows) the product is not stored: a `PreparedNorm`
-    comes back."""
-    _gpu(x, weight, packed8)
-    _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "gemm_skinny8 takes bfloat16")
-    _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
+    x may come as a `PackedRows8` made for this K. With `packed8` (= pack_weight8(weight)) the kernel
+    reads that copy. With `next_norm` = (residual or None, weight of the norm that follows) the product
+    is not stored: a `PreparedNorm` comes back."""
+    x_packed = isinstance(x, PackedRows8)
+    xt = x.data if x_packed else x
+    _gpu(xt, weight, packed8)
+    _need(xt.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "gemm_skinny8 takes bfloat16")
+    _need(len(x.shape) == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
           f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
     M, K = x.shape
     N = weight.shape[0]
     steps = skinny8_steps(K)
     _need(M <= SKINNY8_MAX_ROWS and steps > 0, f"gemm_skinny8 takes up to {SKINNY8_MAX_ROWS} rows and K in steps of 256 up to "
           "8192 or of 1024 up to 16384")
-    _need(_dense_rows(x) and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0,
+    if x_packed:
+        _need(x.steps == steps and xt.is_contiguous() and xt.numel() == 8 * K, f"the packed rows were made for a reader of {x.steps} steps, not {steps}")
+    _need((x_packed or _dense_rows(xt)) and weight.is_contiguous() and xt.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0,
           "rows must be dense and 16-byte aligned")
+    ldx = K if x_packed else xt.stride(0)
     _need(out_dtype in (torch.bfloat16, torch.float32), "the result is bfloat16 or float32")
     if packed8 is not None:
         _need(packed8.dtype == torch.bfloat16 and packed8.shape == (-(-N // 8), K // (64 * steps), steps, 64, 8)
@@ -827,16 +879,16 @@ def gemm_skinny8(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype =
               f"the packed copy does not belong to a weight of {N} x {K}")
     if next_norm is not None:
         _need(out_dtype == torch.bfloat16, "a prepared norm comes with bfloat16")
-        prepared, residual, nw = _next_norm_outputs(x, N, -(-N // 8), next_norm)
+        prepared, residual, nw = _next_norm_outputs(xt, N, -(-N // 8), next_norm, rows=M)
         _run("gemm_skinny8", library().ts_gemm_skinny8_bf16(
-            None, _ptr(x), _ptr(weight if packed8 is None else packed8), M, N, K, x.stride(0), weight.stride(0), N, 1,
+            None, _ptr(xt), _ptr(weight if packed8 is None else packed8), M, N, K, ldx, weight.stride(0), N, 1,
             int(packed8 is not None), _ptr(residual), _ptr(nw), _ptr(prepared.summed), _ptr(prepared.operand),
-            _ptr(prepared.squares), _stream()))
+            _ptr(prepared.squares), int(x_packed), _stream()))
         return prepared
-    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    out = torch.empty((M, N), dtype=out_dtype, device=xt.device)
     _run("gemm_skinny8", library().ts_gemm_skinny8_bf16(
-        _ptr(out), _ptr(x), _ptr(weight if packed8 is None else packed8), M, N, K, x.stride(0), weight.stride(0),
-        out.stride(0), _code(out_dtype), int(packed8 is not None), None, None, None, None, None, _stream()))
+        _ptr(out), _ptr(xt), _ptr(weight if packed8 is None else packed8), M, N, K, ldx, weight.stride(0),
+        out.stride(0), _code(out_dtype), int(packed8 is not None), None, None, None, None, None, int(x_packed), _stream()))
     return out
 
 
@@ -855,14 +907,16 @@ def skinny_fuses(rows: int, k: int, norm: bool, glu: bool) -> bool:
 def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, *,
                 residual: torch.Tensor | None = None, norm_weight: torch.Tensor | None = None, eps: float = 0.0,
                 glu: bool = False, packed: torch.Tensor | None = None, squares: torch.Tensor | None = None,
-                next_norm=None) -> "tuple[torch.Tensor | PreparedNorm, torch.Tensor | None]":
+                next_norm=None, pack8_steps: int = 0) -> "tuple[torch.Tensor | PreparedNorm | PackedRows8, torch.Tensor | None]":
     """bfloat16 e(f(x) [M <= 32, K] · weight [N, K]^T) by the weight-streaming MFMA kernel (up to 64
     rows over reductions of up to 2048). With `norm_weight`: f = RMSNorm(x + residual) * norm_weight,
     and x + residual comes back as the second result. With `squares` (and `eps`): x is the operand of
     a `PreparedNorm` and `squares` its sums of squares; the rows' scales multiply the finished sums.
     With `glu`: weight holds gate rows then up rows and the result is silu(gate) * up, [M, N / 2].
     With `packed` (= pack_weight(weight)) the kernel reads that copy. With `next_norm` = (residual or
-    None, weight of the norm that follows) the first result is a `PreparedNorm` instead of the product."""
+    None, weight of the norm that follows) the first result is a `PreparedNorm` instead of the product.
+    With `pack8_steps` (and `glu`, up to 8 rows) the gated product comes back as a `PackedRows8` for a
+    reader of that many steps."""
     _gpu(x, weight, residual, norm_weight)
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "gemm_skinny takes bfloat16")
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
@@ -887,7 +941,7 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
             None, _ptr(x), _ptr(weight if packed is None else packed), None, None, None, M, N, K, x.stride(0),
             weight.stride(0), N, float(eps), mode, 0, 1, int(packed is not None), _ptr(squares),
             0 if squares is None else squares.shape[1], _ptr(nres), _ptr(nw), _ptr(prepared.summed), _ptr(prepared.operand),
-            _ptr(prepared.squares), _stream()))
+            _ptr(prepared.squares), 0, _stream()))
         return prepared, None
     res_out = None
     if norm:
@@ -902,13 +956,20 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     else:
         _need(residual is None, "a residual comes with a norm weight")
     _need(out_dtype == torch.bfloat16 or not (norm or glu), "float32 output comes with the plain product only")
-    out = _gated_output(M, N // 2, x.device) if glu else torch.empty((M, N), dtype=out_dtype, device=x.device)
+    if pack8_steps:
+        _need(glu and M <= 8 and pack8_steps in (4, 8, 16) and (N // 2) % (64 * pack8_steps) == 0,
+              "packed rows come from a gated product of up to 8 rows whose width is whole waves of the reader")
+        out = torch.empty(((N // 2) // (64 * pack8_steps), pack8_steps, 64, 8), dtype=torch.bfloat16, device=x.device)
+        ldy = N // 2
+    else:
+        out = _gated_output(M, N // 2, x.device) if glu else torch.empty((M, N), dtype=out_dtype, device=x.device)
+        ldy = out.stride(0)
     _run("gemm_skinny", library().ts_gemm_skinny_bf16(
         _ptr(out), _ptr(x), _ptr(weight if packed is None else packed), _ptr(residual), _ptr(norm_weight),
-        _ptr(res_out) if residual is not None else None, M, N, K, x.stride(0), weight.stride(0), out.stride(0),
+        _ptr(res_out) if residual is not None else None, M, N, K, x.stride(0), weight.stride(0), ldy,
         float(eps), mode, int(glu), _code(out_dtype), int(packed is not None), _ptr(squares),
-        0 if squares is None else squares.shape[1], None, None, None, None, None, _stream()))
-    return out, res_out
+        0 if squares is None else squares.shape[1], None, None, None, None, None, int(pack8_steps), _stream()))
+    return (PackedRows8(out, M, N // 2, pack8_steps) if pack8_steps else out), res_out
 
 
 ROWS64_MIN_ROWS = 33         # fewer rows are the weight-streaming kernel's (gemm_skinny: 32 rows 16.6 µs against 17.7 here,
@@ -1198,8 +1259,10 @@ class StreamingCopies:
         return sum(t.numel() * t.element_size() for t in (self.by16, self.by8) if t is not None)
 
 
-def next_norm_fuses(x: torch.Tensor, weight: torch.Tensor, packed: "StreamingCopies | None" = None) -> bool:
+def next_norm_fuses(x: "torch.Tensor | PackedRows8", weight: torch.Tensor, packed: "StreamingCopies | None" = None) -> bool:
     """Whether `linear_bf16(x, weight, next_norm=...)` has a kernel that leaves a `PreparedNorm`."""
+    if isinstance(x, PackedRows8):          # (made for the 8-row form, which does)
+        return True
     if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.is_cuda and x.dim() == 2 and weight.dim() == 2
             and _dense_rows(x) and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
         return False
@@ -1236,6 +1299,9 @@ def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     """bfloat16 x [M, K] · weight [N, K]^T: few rows go to the weight-streaming kernels (which read
     the weight's copy in their own order from `packed`, if there is one), many to the vendor matrix
     library. With `next_norm` (where `next_norm_fuses` says so) a `PreparedNorm` comes back."""
+    if isinstance(x, PackedRows8):
+        _need(rows8_reader_steps(x.shape[0], weight) == x.steps, "packed rows go to the projection they were made for")
+        return gemm_skinny8(x, weight, out_dtype, None if packed is None else packed.by8, next_norm=next_norm)
     _gpu(x, weight)
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "linear_bf16 takes bfloat16")
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],

@@ -78,13 +78,23 @@ def streaming_copy(weight: torch.Tensor) -> hip.StreamingCopies | None:
     return hip.StreamingCopies(by16, by8) if by16 is not None or by8 is not None else None
 
 
-def linear(x: torch.Tensor | DeferredNorm, weight: torch.Tensor, out_dtype: torch.dtype | None = None,
+PACKED_ROWS_MIN = 2      # rows from which a gated product is handed on in the 8-row form's order (one row is read whole anyway)
+
+
+def linear(x: "torch.Tensor | DeferredNorm | hip.PackedRows8", weight: torch.Tensor, out_dtype: torch.dtype | None = None,
            glu: bool = False, packed: hip.StreamingCopies | None = None,
-           then: NormRequest | None = None) -> "torch.Tensor | DeferredNorm":
+           then: NormRequest | None = None, feeds: torch.Tensor | None = None) -> "torch.Tensor | DeferredNorm | hip.PackedRows8":
     """x · Wᵀ; with `glu`, W holds gate rows then up rows and silu(gate) * up comes back.
     `packed` is `streaming_copy(weight)` if the part keeps one. With `then` the result is the
     `DeferredNorm` of that request: norm(x · Wᵀ + residual) * weight, prepared by this projection's
-    kernel where it can be, left to the next projection otherwise."""
+    kernel where it can be, left to the next projection otherwise. `feeds` (with `glu`): the weight of
+    the projection that alone reads this product; where that projection's kernel reads its operand
+    faster in an order of its own, the product comes back in that order (a `hip.PackedRows8`), to be
+    handed to `linear` with that weight and to nothing else."""
+    if isinstance(x, hip.PackedRows8) and (glu or hip.rows8_reader_steps(x.shape[0], weight) != x.steps):
+        x = x.rows()
+    if isinstance(x, hip.PackedRows8) and then is None:
+        return hip.linear_bf16(x, weight, out_dtype or torch.bfloat16, packed)
     if then is not None:
         if glu:
             raise ValueError("a gated projection does not finish into a norm")
@@ -97,6 +107,10 @@ def linear(x: torch.Tensor | DeferredNorm, weight: torch.Tensor, out_dtype: torc
             return DeferredNorm(None, None, then.weight, then.eps, prepared)
         return DeferredNorm(linear(x, weight, out_dtype, packed=packed), residual, then.weight, then.eps)
     by16 = None if packed is None else packed.by16
+    rows = x.rows if isinstance(x, DeferredNorm) else x.shape[0]
+    pack8 = hip.rows8_reader_steps(rows, feeds) if glu and feeds is not None and PACKED_ROWS_MIN <= rows <= 8 else 0
+    if pack8 and (weight.shape[0] // 2) % (64 * pack8):
+        pack8 = 0
     if isinstance(x, DeferredNorm) and x.prepared is not None:
         d, op = x, x.prepared.operand
         if out_dtype in (None, torch.bfloat16) and _streams(op, weight, dense_rows=True) and not (glu and weight.shape[0] % 32):
@@ -105,7 +119,8 @@ def linear(x: torch.Tensor | DeferredNorm, weight: torch.Tensor, out_dtype: torc
             if wide:
                 return hip.gemm_rows64(op, by16, glu=glu, squares=d.prepared.squares, eps=d.eps)
             if (hip.skinny_fuses(rows, k, False, True) if glu else hip._skinny_serves(rows, n, k)):
-                return hip.gemm_skinny(op, weight, glu=glu, packed=by16, squares=d.prepared.squares, eps=d.eps)[0]
+                return hip.gemm_skinny(op, weight, glu=glu, packed=by16, squares=d.prepared.squares, eps=d.eps,
+                                       pack8_steps=pack8 if glu else 0)[0]
         x = d.materialize()
     if isinstance(x, DeferredNorm):
         d = x
@@ -113,7 +128,7 @@ def linear(x: torch.Tensor | DeferredNorm, weight: torch.Tensor, out_dtype: torc
                 and (d.residual is None or d.residual.is_contiguous())
                 and hip.skinny_fuses(d.x.shape[0], weight.shape[1], True, glu) and (not glu or weight.shape[0] % 32 == 0)):
             y, d.residual_out = hip.gemm_skinny(d.x, weight, residual=d.residual, norm_weight=d.weight, eps=d.eps, glu=glu,
-                                                packed=by16)
+                                                packed=by16, pack8_steps=pack8 if glu else 0)
             return y
         x = d.materialize()
     if glu:
@@ -122,7 +137,7 @@ def linear(x: torch.Tensor | DeferredNorm, weight: torch.Tensor, out_dtype: torc
             return hip.gemm_rows64(x, by16, glu=True)
         if (out_dtype in (None, torch.bfloat16) and _streams(x, weight) and weight.shape[0] % 32 == 0
                 and hip.skinny_fuses(x.shape[0], weight.shape[1], False, True)):
-            return hip.gemm_skinny(x, weight, glu=True, packed=by16)[0]
+            return hip.gemm_skinny(x, weight, glu=True, packed=by16, pack8_steps=pack8)[0]
         if (out_dtype in (None, torch.bfloat16) and hip.many_rows_products() == "tiled" and x.is_cuda
                 and hip.tiled_takes(x, weight, glu=True)):
             return hip.gemm_tiled(x, weight, glu=True)

@@ -34,5 +34,5 @@ class GatedMLP(FeedForward):
         return sum(c.nbytes() for c in (self.gate_up_packed, self.down_packed) if c is not None)
 
     def forward(self, x: torch.Tensor, ctx: StepContext, then=None) -> torch.Tensor:
-        return linear(linear(x, self.gate_up, glu=True, packed=self.gate_up_packed), self.down, packed=self.down_packed,
-                      then=then)
+        gated = linear(x, self.gate_up, glu=True, packed=self.gate_up_packed, feeds=self.down)
+        return linear(gated, self.down, packed=self.down_packed, then=then)
