@@ -38,10 +38,6 @@
 #define R64_RING 16               // steps of W a compute wave has under way (two chunks): with 32 the chip had 32 MB under way and
                                   // every load, x's among them, came back some 5 us later (the gate|up product of 64 rows 20.7 us, 19.7 with 16)
 #define R64_STAGE_LOADS 8          // loads of a staging wave per chunk: two rows of its block each
-// where in a block's [64] the piece of row r (of 16), step s, k = 8 g .. 8 g + 7 lies: the 16 pieces that the lanes of a
-// staging wave's load write side by side (one row, 4 steps x 4 g) land in 16 different places, and a compute
-// wave's 64 lanes (16 rows x 4 g of one step) read 64 different places
-static __device__ __forceinline__ int r64_place(int r, int s, int g) { return (r ^ ((g + 4 * s) & 15)) + 16 * g; }
 
 struct Rows64Args {
   const bf16_t* x;       // [M, K], row stride ldx
@@ -83,7 +79,7 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
       const int r = 2 * j + half, m = 16 * sw + r;
       ok[j] = m < a.M;                                    // rows past M read row 0 and count as zeros
       xoff[j] = (int64_t)(ok[j] ? m : 0) * a.ldx + kfirst + 8 * kl;
-      slot[j] = ((kl >> 2) * 4 + sw) * TS_WAVE + r64_place(r, kl >> 2, kl & 3);      // in a buffer's [step][block][64]
+      slot[j] = ((kl >> 2) * 4 + sw) * TS_WAVE + sk_place(r, kl >> 2, kl & 3);      // in a buffer's [step][block][64]
     }
     auto ask = [&](int c, uint4 (&t)[R64_STAGE_LOADS]) {
       const int k0 = c * R64_CHUNK_STEPS * SK_KSTEP;      // first k of the chunk
@@ -126,7 +122,7 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
   for (int b = 0; b < 4; ++b) acc[b] = (float4_t){0.f, 0.f, 0.f, 0.f};
   int at[4];                    // where this lane's piece of a step lies in a block, by the step's last two bits
 #pragma unroll
-  for (int i = 0; i < 4; ++i) at[i] = r64_place(r, i, g);
+  for (int i = 0; i < 4; ++i) at[i] = sk_place(r, i, g);
   // the scales of this lane's rows: the parts of a row's sum of squares in ascending order. The wait is for
   // loads that come back behind the ring's first turn, which the first products wait for anyway (in the
   // staging waves a wait for the parts held the second chunk's request back by a trip to memory).

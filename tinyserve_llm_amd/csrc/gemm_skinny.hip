@@ -125,8 +125,27 @@ gemm_skinny_kernel(const SkinnyArgs a) {
   // can start the moment W has arrived; asked for after W, every batch of x would wait behind all of W
   // and then for its own trip to the cache.
   constexpr bool X_FIRST = MODE != MODE_NORM && MAXT <= 512 && (CB * STEPS + RT * STEPS) <= 48;
+  // ---- with more than one block of rows the loads of x outnumber W's, and a load that gathers 64 bytes of each
+  // of 16 rows costs far more than one of long pieces (q|k|v of 64 rows: 10.9 us, 8.0 with contiguous loads):
+  // the wave then fetches its slice of a block's rows whole (STEPS 64 bytes of a row side by side, 64 / (4 STEPS)
+  // rows a load) and turns them into operand order through LDS once W's loads are out (sk_place). (Not where a
+  // wave has more row tiles of W than blocks of x: the gate|up product of 24 rows, 4 tiles against 2 blocks, takes
+  // 16.7 us that way and 16.5 as it is.)
+  constexpr bool X_TURNED = X_FIRST && CB >= 2 && CB >= RT;
+  constexpr int X_LANES = 4 * STEPS <= TS_WAVE ? 4 * STEPS : TS_WAVE;     // lanes that share a row of such a load
+  static_assert(!X_TURNED || 4 * STEPS <= TS_WAVE, "a wave's slice of a row is at most a kilobyte");
   uint4 xall[X_FIRST ? CB : 1][X_FIRST ? STEPS : 1];
-  if constexpr (X_FIRST) {
+  if constexpr (X_TURNED) {
+    const int lr = lane / X_LANES, piece = lane % X_LANES;
+#pragma unroll
+    for (int b = 0; b < CB; ++b)
+#pragma unroll
+      for (int j = 0; j < STEPS; ++j) {
+        const int m = b * 16 + j * (TS_WAVE / X_LANES) + lr;              // rows past M repeat row 0 and are not stored
+        xall[b][j] = *(const uint4*)(a.x + (int64_t)(m < a.M ? m : 0) * a.ldx + wave * STEPS * SK_KSTEP + 8 * piece);
+      }
+    __builtin_amdgcn_sched_barrier(0);
+  } else if constexpr (X_FIRST) {
 #pragma unroll
     for (int b = 0; b < CB; ++b)
 #pragma unroll
@@ -210,6 +229,21 @@ gemm_skinny_kernel(const SkinnyArgs a) {
     __builtin_amdgcn_sched_barrier(0);
   }
 
+
+  if constexpr (X_TURNED) {
+    // a block at a time through this wave's STEPS kilobytes (a wave's LDS operations keep their order)
+    uint4* turn = (uint4*)smem + (size_t)wave * STEPS * TS_WAVE;
+    const int lr = lane / X_LANES, piece = lane % X_LANES;
+#pragma unroll
+    for (int b = 0; b < CB; ++b) {
+#pragma unroll
+      for (int j = 0; j < STEPS; ++j)
+        turn[(piece >> 2) * TS_WAVE + sk_place(j * (TS_WAVE / X_LANES) + lr, piece >> 2, piece & 3)] = xall[b][j];
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) xall[b][s] = turn[s * TS_WAVE + sk_place(r, s, g)];
+    }
+    __syncthreads();            // the kilobytes are the waves' partial sums from here on
+  }
 
   float4_t acc[RT][CB];
 #pragma unroll
@@ -446,7 +480,10 @@ static size_t sk_lds_limit() {
 template <int RT, int CB, int STEPS, int MODE, int GLU, typename OUT>
 static int sk_launch(const SkinnyArgs& a, hipStream_t stream) {
   const int nwaves = a.K / (STEPS * SK_KSTEP);
-  const size_t smem = sizeof(float) * ((size_t)nwaves * RT * CB * 256 + (size_t)nwaves * 16 * CB);
+  size_t smem = sizeof(float) * ((size_t)nwaves * RT * CB * 256 + (size_t)nwaves * 16 * CB);
+  // (the kilobytes through which a wave turns its rows of x, where it does: X_TURNED of the kernel)
+  if (CB >= 2 && CB >= RT && MODE != MODE_NORM && nwaves <= 8 && (CB * STEPS + RT * STEPS) <= 48 && smem < (size_t)nwaves * STEPS * 1024)
+    smem = (size_t)nwaves * STEPS * 1024;
   constexpr int OT = GLU == EPI_GLU ? RT / 2 : RT;
   const int ncols = GLU == EPI_GLU ? a.N / 2 : a.N;     // (EPI_ROPE: a 16-row tile of the matrix per 8 columns and their partners)
   if (smem > sk_lds_limit()) return TS_BAD_SHAPE;       // (the largest instances ask for a little more than 64 KB)

@@ -43,6 +43,13 @@ static __device__ __forceinline__ uint4 sk_pack(const float* f) {
     w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector((float2_t){f[2 * i], f[2 * i + 1]}, bf16x2_t));
   return make_uint4(w[0], w[1], w[2], w[3]);
 }
+// Rows of x fetched in long pieces (a load takes 256 bytes or more of a row, not 64 bytes of each of 16 rows) reach the
+// order the matrix instruction wants through LDS. Where in a block's [64] places of 16 bytes the piece of row r (of
+// 16), step s, k = 8 g .. 8 g + 7 lies: the 16 pieces that neighbouring lanes of such a load write (one row, 4 steps
+// x 4 g) land in 16 different places, and the 64 lanes of a reading wave (16 rows x 4 g of one step) read 64
+// different places, so neither meets in a bank.
+static __device__ __forceinline__ int sk_place(int r, int s, int g) { return (r ^ ((g + 4 * s) & 15)) + 16 * g; }
+
 static __device__ __forceinline__ float sk_silu(float g) {
   return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896340736f * g));
 }
