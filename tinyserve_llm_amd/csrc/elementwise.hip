@@ -342,6 +342,7 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
     // page where their slots are consecutive, aligned and inside one page
     __shared__ T tile[ROPE_TOK][ROPE_VTILE];
     __shared__ int base_slot[ROPE_TOK / 8];          // first slot of each run of 8 tokens, or -1: no fast path
+    __shared__ int slot_of[ROPE_TOK];                // the group's slots (tokens that are not there: -1), fetched once
     constexpr int VP = 16 / sizeof(T);                // elements of a 16-byte piece
     static_assert(VP == 8 || sizeof(T) == 4, "runs of 8 tokens are pieces of bfloat16");
     if (threadIdx.x < ROPE_TOK / 8) {
@@ -358,6 +359,10 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
         if (!ok) s0 = -1;
       }
       base_slot[threadIdx.x] = s0;
+    }
+    if (threadIdx.x >= 64 && threadIdx.x < 64 + ROPE_TOK) {
+      const int tl = threadIdx.x - 64;
+      slot_of[tl] = tl < nt ? slots[t0 + tl] : -1;
     }
     const int ebeg = (int)((int64_t)(vel / VP) * by / ny) * VP;
     const int eend = (int)((int64_t)(vel / VP) * (by + 1) / ny) * VP;
@@ -384,10 +389,11 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
             *(uint4*)(v_cache + (int64_t)pg * vp + (s0 - pg * page_size) + (int64_t)h * vh + (int64_t)d * vd) =
                 make_uint4(w[0], w[1], w[2], w[3]);
           } else {
+            // (tokens of different requests, one slot each: eight stores that wait for nothing but LDS)
+#pragma unroll
             for (int k = 0; k < 8; ++k) {
               const int tl = 8 * run + k;
-              if (tl >= nt) break;
-              const int slot = slots[t0 + tl];
+              const int slot = slot_of[tl];
               if (slot < 0) continue;
               const int pg = page_of(slot);
               v_cache[(int64_t)pg * vp + (int64_t)(slot - pg * page_size) * vs + (int64_t)h * vh + (int64_t)d * vd] = tile[tl][el];
