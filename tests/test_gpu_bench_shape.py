@@ -170,8 +170,7 @@ def folder_1b(tmp_path_factory):
     return folder
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("batch", [8, 64])
+@pytest.mark.parametrize("batch,dtype", [(8, "float32"), (8, "bfloat16"), (64, "float32"), (64, "bfloat16"), (96, "bfloat16")])
 def test_the_benchmarks_own_regime_against_the_plain_model(folder_1b, dtype, batch, monkeypatch):
     """What bench.py times, checked, at both of its batch sizes beyond one: requests of 2,048 tokens
     (eight full pages of 256 each) decode sixteen tokens through `LLM.generate`, set up as bench.py
@@ -180,7 +179,8 @@ def test_the_benchmarks_own_regime_against_the_plain_model(folder_1b, dtype, bat
     that cross into a ninth page. Eight requests take the split-key attention kernel and the
     weight-streaming projections; sixty-four take one workgroup per (request, key/value head) over
     the whole context, the shared-x kernel for the gate|up projection and the head, and the same kernel
-    with the reduction in slices for the o and down projections, and the test sees that they did. Every token
+    with the reduction in slices for the o and down projections, and the test sees that they did; ninety-six
+    the same kernels with eight blocks of rows in LDS instead of four (the head is the library's then). Every token
     of some of the requests against the plain model run whole over the same history: in float32 it is
     the plain model's choice; in bfloat16 it lies within a small gap of it."""
     from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
@@ -222,6 +222,9 @@ def test_the_benchmarks_own_regime_against_the_plain_model(folder_1b, dtype, bat
             assert (64, 2 * 8192) in rows64 and (64, CONFIG.vocab_size) in rows64, f"gate|up and the head by the shared-x kernel: {rows64}"
             assert (64, 2048, 2048, 4, True) in sliced and (64, 2048, 8192, 8, True) in sliced, \
                 f"o and down in slices of their reductions, finished into the norms that follow them: {set(sliced)}"
+        elif batch == 96:
+            assert (96, 2 * 8192) in rows64 and (96, CONFIG.vocab_size) not in rows64, f"gate|up by the shared-x kernel, the head by the library: {rows64}"
+            assert {(96, 2048, 2048, 4, True), (96, 2048, 8192, 8, True)} <= set(sliced), f"o and down in slices: {set(sliced)}"
         else:
             assert plan(8, 8, 4, 64, 9 * page)[0] < 9 * page and not rows64 and not sliced, "eight requests: keys in chunks, combined afterwards"
     plain = PlainLlama(folder_1b, torch.float64)

@@ -954,7 +954,8 @@ def test_fused_projection_rotation_and_cache_write(nh, nkv, hd, K, M, page, norm
 
 @pytest.mark.parametrize("nh,nkv,hd,K,M,page,slices,prepared", [
     (32, 8, 64, 2048, 64, 256, 4, True), (32, 8, 64, 2048, 33, 16, 4, False), (24, 8, 128, 3072, 20, 32, 3, True),
-    (24, 8, 128, 3072, 40, 32, 3, True), (4, 2, 128, 4096, 64, 16, 2, False),
+    (24, 8, 128, 3072, 40, 32, 3, True), (4, 2, 128, 4096, 64, 16, 2, False), (32, 8, 64, 2048, 128, 32, 4, True),
+    (24, 8, 128, 3072, 90, 16, 3, False),
     (6, 2, 32, 512, 48, 8, 1, True), (5, 3, 96, 1024, 17, 24, 2, False)])
 def test_projection_in_slices_with_rotation_and_cache_write(nh, nkv, hd, K, M, page, slices, prepared):
     """The qkv projection with its reduction in slices and the kernel that adds the parts, rotates and
@@ -1282,11 +1283,12 @@ def test_gated_product_handed_on_in_the_eight_row_forms_order(m, inter, k):
     assert not isinstance(linear(x[:1], gate_up, glu=True, packed=copies[0], feeds=down), H.PackedRows8), "one row is handed on as it is"
 
 
-@pytest.mark.parametrize("m", [17, 33, 50, 64])
+@pytest.mark.parametrize("m", [17, 33, 50, 64, 65, 100, 128])
 @pytest.mark.parametrize("n,k", [(8192, 1024), (16384, 2048), (9152, 3072)])
 def test_wide_product_for_a_few_dozen_rows(m, n, k):
     """The kernel that shares x among 64 rows of W through LDS, against 64-bit products: plain (bfloat16
-    and 32-bit sums) and with the gate; each row's result does not depend on the rows beside it."""
+    and 32-bit sums) and with the gate; each row's result does not depend on the rows beside it. Up to 64
+    rows lie in four blocks of 16 in LDS, up to 128 in eight."""
     g = gen(m + n + k)
     x = torch.randn(m, k, generator=g).bfloat16().to(dev())
     w = (torch.randn(n, k, generator=g) * k ** -0.5).bfloat16().to(dev())
@@ -1302,12 +1304,14 @@ def test_wide_product_for_a_few_dozen_rows(m, n, k):
         torch.testing.assert_close(yg.double().cpu(), gate, rtol=2e-2, atol=2e-2 * float(gate.abs().max()))
     alone = hip().gemm_rows64(x[m - 1:].contiguous(), packed, torch.float32)
     assert torch.equal(alone[0], y32[m - 1])
-    assert hip().rows64_takes(max(m, 33), n, k) and not hip().rows64_takes(65, n, k) and not hip().rows64_takes(40, n, k + 512)
+    assert hip().rows64_takes(max(m, 33), n, k, glu=True) and not hip().rows64_takes(40, n, k + 512)
+    assert hip().rows64_takes(64, n, k) and not hip().rows64_takes(65, n, k), "a plain product of more than 64 rows is the library's"
+    assert hip().rows64_takes(128, n, k, glu=True) and not hip().rows64_takes(129, n, k, glu=True)
     with pytest.raises(hip().KernelError):
-        hip().gemm_rows64(torch.cat([x, x, x, x])[:65].contiguous(), packed)
+        hip().gemm_rows64(x[:1].expand(129, k).contiguous(), packed)
 
 
-@pytest.mark.parametrize("m", [5, 17, 40, 64])
+@pytest.mark.parametrize("m", [5, 17, 40, 64, 77, 128])
 @pytest.mark.parametrize("n,k,slices", [(2048, 2048, 4), (2048, 8192, 8), (3072, 3072, 6), (192, 1536, 3), (4096, 14336, 4),
                                         (2048, 512, 1)])
 def test_narrow_product_in_slices_of_its_reduction(m, n, k, slices):
@@ -1336,14 +1340,14 @@ def test_narrow_product_in_slices_of_its_reduction(m, n, k, slices):
     with pytest.raises(hip().KernelError):
         hip().gemm_rows64_sliced(x, packed, slices * 2 if k % (1024 * slices) else 5 if (k // 512) % 5 else 7)
     with pytest.raises(hip().KernelError):
-        hip().gemm_rows64_sliced(x[:1].expand(65, k).contiguous(), packed, slices)
+        hip().gemm_rows64_sliced(x[:1].expand(129, k).contiguous(), packed, slices)
 
 
 def test_which_narrow_products_are_cut_into_slices():
     from tinyserve_llm_amd.parts.linear import linear, streaming_copy, NormRequest, DeferredNorm
     assert hip().rows64_slices(64, 2048, 2048) == 4 and hip().rows64_slices(33, 2048, 8192) == 8
     assert hip().rows64_slices(48, 3072, 3072) == 6 and hip().rows64_slices(64, 4096, 14336) == 4
-    assert hip().rows64_slices(4, 2048, 8192) == 0 and hip().rows64_slices(65, 2048, 8192) == 0 and hip().rows64_slices(9, 2048, 8192) == 8
+    assert hip().rows64_slices(4, 2048, 8192) == 0 and hip().rows64_slices(129, 2048, 8192) == 0 and hip().rows64_slices(9, 2048, 8192) == 8 and hip().rows64_slices(128, 2048, 8192) == 8
     assert hip().rows64_slices(64, 16384, 2048) == 0, "a wide weight gives every compute unit a workgroup as it is"
     assert hip().rows64_slices(64, 2048, 2304) == 0 and hip().rows64_slices(64, 2000, 2048) == 0
     g = gen(5)

@@ -98,10 +98,12 @@ def test_which_kernel_takes_a_projection_of_few_rows():
         steps = hip.skinny8_steps(k)
         assert steps in (4, 8, 16) and k % (64 * steps) == 0 and k // (64 * steps) <= 16
     assert hip.skinny8_steps(100) == 0
-    # shared-x kernel: 33 to 64 rows against at least 8,192 rows of W in steps of 64, K in steps of 1,024
+    # shared-x kernel: 33 to 64 rows (128 with the gate) against at least 8,192 rows of W in steps of 64, K in steps of 1,024
     assert hip.rows64_takes(33, 16384, 2048) and hip.rows64_takes(64, 128256, 2048) and hip.rows64_takes(40, 8192, 3072)
+    assert hip.rows64_takes(65, 16384, 2048, glu=True) and hip.rows64_takes(128, 16384, 2048, glu=True)
     for rows, n, k in ((32, 16384, 2048), (65, 16384, 2048), (40, 4096, 2048), (40, 8200, 2048), (40, 16384, 2560)):
         assert not hip.rows64_takes(rows, n, k)
+    assert not hip.rows64_takes(129, 16384, 2048, glu=True) and not hip.rows64_takes(32, 16384, 2048, glu=True)
     # the fused norm serves one block of 16 rows; the gate alone up to 64 rows over reductions of up to 2,048
     assert hip.skinny_fuses(16, 2048, True, True) and not hip.skinny_fuses(17, 2048, True, True)
     assert hip.skinny_fuses(64, 2048, False, True) and not hip.skinny_fuses(65, 2048, False, True)
@@ -113,7 +115,7 @@ def test_which_narrow_products_have_their_reduction_cut_into_slices():
     unit a workgroup of 64 rows; the fewest slices (multiples of 512 of k) that reach 192 workgroups."""
     assert hip.rows64_slices(64, 2048, 2048) == 4 and hip.rows64_slices(33, 2048, 8192) == 8 and hip.rows64_slices(9, 2048, 8192) == 8
     assert hip.rows64_slices(48, 3072, 3072) == 6 and hip.rows64_slices(8, 3072, 8192) == 4 and hip.rows64_slices(64, 4096, 14336) == 4
-    for rows, n, k in ((4, 2048, 8192), (65, 2048, 8192), (64, 16384, 2048), (64, 2048, 2304), (64, 2000, 2048)):
+    for rows, n, k in ((4, 2048, 8192), (129, 2048, 8192), (64, 16384, 2048), (64, 2048, 2304), (64, 2000, 2048)):
         assert hip.rows64_slices(rows, n, k) == 0
     for n, k in ((64, 512), (2048, 8192), (3072, 3072), (4096, 14336), (4096, 4096)):
         s = hip.rows64_slices(40, n, k)

@@ -1,4 +1,4 @@
-// y[M, N] = e(f(x)[M, K] · W[N, K]^T) in bfloat16 for 17 to 64 rows of x and a wide W (the gate|up
+// y[M, N] = e(f(x)[M, K] · W[N, K]^T) in bfloat16 for 17 to 128 rows of x and a wide W (the gate|up
 // projection of a decode step of a few dozen requests), where time should go to reading W once.
 //
 // With so many rows the weight-streaming kernel of gemm_skinny.hip reads x from the second-level cache
@@ -54,11 +54,14 @@ struct Rows64Args {
   int slices;            // the reduction in this many slices (gridDim.y); more than one: y is float [slices][M][ldy]
 };
 
-template <bool GLU, typename OUT>
+// BLOCKS: blocks of 16 rows of x, 4 (up to 64 rows) or 8 (up to 128: the compute waves then take a chunk's
+// steps one at a time instead of in pairs, for their registers' sake).
+template <bool GLU, typename OUT, int BLOCKS>
 __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
   // x as the B operands of the matrix instruction: [buffer][step][block of 16 rows][lane], lane r + 16 g
-  // holding k = 8 g .. 8 g + 7 of row r
-  __shared__ uint4 xs[2][R64_CHUNK_STEPS][4][TS_WAVE];
+  // holding k = 8 g .. 8 g + 7 of row r (turned: sk_place)
+  extern __shared__ __align__(16) uint4 xs_all[];
+  auto xs = [&](int buf, int step, int b) { return xs_all + (((size_t)buf * R64_CHUNK_STEPS + step) * BLOCKS + b) * TS_WAVE; };
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TS_WAVE), lane = threadIdx.x & (TS_WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
   const int slice = blockIdx.y;
@@ -69,29 +72,30 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
     // ---- staging waves: wave sw brings block sw of 16 rows, all the steps of every chunk. It asks for
     // the next chunk before it puts this one into LDS, so that a chunk costs the compute waves a barrier
     // and not a trip to the cache.
-    const int sw = wave - 4;                              // this wave's block of 16 rows
+    const int sw = wave - 4;                              // this wave's blocks of 16 rows: sw BLOCKS / 4 ..
+    constexpr int MINE = BLOCKS / 4, LOADS = R64_STAGE_LOADS * MINE;
     const int half = lane >> 5, kl = lane & 31;           // the row of a load's two, and the piece of its 256 k
-    bool ok[R64_STAGE_LOADS];
-    int64_t xoff[R64_STAGE_LOADS];
-    int slot[R64_STAGE_LOADS];
+    bool ok[LOADS];
+    int64_t xoff[LOADS];
+    int slot[LOADS];
 #pragma unroll
-    for (int j = 0; j < R64_STAGE_LOADS; ++j) {
-      const int r = 2 * j + half, m = 16 * sw + r;
+    for (int j = 0; j < LOADS; ++j) {
+      const int block = sw * MINE + j / R64_STAGE_LOADS, r = 2 * (j % R64_STAGE_LOADS) + half, m = 16 * block + r;
       ok[j] = m < a.M;                                    // rows past M read row 0 and count as zeros
       xoff[j] = (int64_t)(ok[j] ? m : 0) * a.ldx + kfirst + 8 * kl;
-      slot[j] = ((kl >> 2) * 4 + sw) * TS_WAVE + sk_place(r, kl >> 2, kl & 3);      // in a buffer's [step][block][64]
+      slot[j] = ((kl >> 2) * BLOCKS + block) * TS_WAVE + sk_place(r, kl >> 2, kl & 3);      // in a buffer's [step][block][64]
     }
-    auto ask = [&](int c, uint4 (&t)[R64_STAGE_LOADS]) {
+    auto ask = [&](int c, uint4 (&t)[LOADS]) {
       const int k0 = c * R64_CHUNK_STEPS * SK_KSTEP;      // first k of the chunk
 #pragma unroll
-      for (int j = 0; j < R64_STAGE_LOADS; ++j) t[j] = *(const uint4*)(a.x + xoff[j] + k0);
+      for (int j = 0; j < LOADS; ++j) t[j] = *(const uint4*)(a.x + xoff[j] + k0);
     };
-    auto put = [&](int c, const uint4 (&t)[R64_STAGE_LOADS]) {
-      uint4* buf = &xs[c & 1][0][0][0];
+    auto put = [&](int c, const uint4 (&t)[LOADS]) {
+      uint4* buf = xs(c & 1, 0, 0);
 #pragma unroll
-      for (int j = 0; j < R64_STAGE_LOADS; ++j) buf[slot[j]] = ok[j] ? t[j] : make_uint4(0, 0, 0, 0);
+      for (int j = 0; j < LOADS; ++j) buf[slot[j]] = ok[j] ? t[j] : make_uint4(0, 0, 0, 0);
     };
-    uint4 A[R64_STAGE_LOADS], B[R64_STAGE_LOADS];
+    uint4 A[LOADS], B[LOADS];
     ask(0, A);
     for (int c = 0; c < nchunks; c += 2) {
       ask(c + 1, B);
@@ -117,19 +121,21 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
     wr[s] = *(const uint4*)(wp + (int64_t)s * 512);
     __builtin_amdgcn_sched_barrier(0);
   }
-  float4_t acc[4];
+  float4_t acc[BLOCKS];
 #pragma unroll
-  for (int b = 0; b < 4; ++b) acc[b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+  for (int b = 0; b < BLOCKS; ++b) acc[b] = (float4_t){0.f, 0.f, 0.f, 0.f};
   int at[4];                    // where this lane's piece of a step lies in a block, by the step's last two bits
 #pragma unroll
   for (int i = 0; i < 4; ++i) at[i] = sk_place(r, i, g);
   // the scales of this lane's rows: the parts of a row's sum of squares in ascending order. The wait is for
   // loads that come back behind the ring's first turn, which the first products wait for anyway (in the
   // staging waves a wait for the parts held the second chunk's request back by a trip to memory).
-  float scale[4] = {1.f, 1.f, 1.f, 1.f};
+  float scale[BLOCKS];
+#pragma unroll
+  for (int b = 0; b < BLOCKS; ++b) scale[b] = 1.f;
   if (a.ssq_in) {
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
+    for (int b = 0; b < BLOCKS; ++b) {
       const int m = 16 * b + r;
       float total = 0.f;
       if (m < a.M) {
@@ -144,28 +150,30 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
   auto ring = [&](int base, auto more) {
 #pragma unroll
     for (int h = 0; h < R64_RING / R64_CHUNK_STEPS; ++h) {
-      // a chunk in four pairs of steps: the next pair's operands leave LDS while this pair's products
-      // run (left to itself the compiler reads two operands, waits, multiplies, and so on)
-      constexpr int PAIRS = R64_CHUNK_STEPS / 2;
-      uint4 xb[2][2][4];
+      // a chunk in batches of steps (pairs; single steps with 8 blocks of x): the next batch's operands leave
+      // LDS while this batch's products run (left to itself the compiler reads two operands, waits,
+      // multiplies, and so on)
+      constexpr int PER = BLOCKS == 4 ? 2 : 1, BATCHES = R64_CHUNK_STEPS / PER;
+      const int buf = (base / R64_CHUNK_STEPS + h) & 1;
+      uint4 xb[2][PER][BLOCKS];
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < PER; ++i)
 #pragma unroll
-        for (int b = 0; b < 4; ++b) xb[0][i][b] = xs[(base / R64_CHUNK_STEPS + h) & 1][i][b][at[i & 3]];
+        for (int b = 0; b < BLOCKS; ++b) xb[0][i][b] = xs(buf, i, b)[at[i & 3]];
 #pragma unroll
-      for (int q = 0; q < PAIRS; ++q) {
-        if (q + 1 < PAIRS) {
+      for (int q = 0; q < BATCHES; ++q) {
+        if (q + 1 < BATCHES) {
 #pragma unroll
-          for (int i = 0; i < 2; ++i)
+          for (int i = 0; i < PER; ++i)
 #pragma unroll
-            for (int b = 0; b < 4; ++b) xb[(q + 1) & 1][i][b] = xs[(base / R64_CHUNK_STEPS + h) & 1][2 * (q + 1) + i][b][at[(2 * (q + 1) + i) & 3]];
+            for (int b = 0; b < BLOCKS; ++b) xb[(q + 1) & 1][i][b] = xs(buf, PER * (q + 1) + i, b)[at[(PER * (q + 1) + i) & 3]];
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          const int sl = R64_CHUNK_STEPS * h + 2 * q + i;
+        for (int i = 0; i < PER; ++i) {
+          const int sl = R64_CHUNK_STEPS * h + PER * q + i;
 #pragma unroll
-          for (int b = 0; b < 4; ++b) acc[b] = sk_mfma(wr[sl], xb[q & 1][i][b], acc[b]);
+          for (int b = 0; b < BLOCKS; ++b) acc[b] = sk_mfma(wr[sl], xb[q & 1][i][b], acc[b]);
           if (decltype(more)::value) wr[sl] = *(const uint4*)(wp + (int64_t)(base + R64_RING + sl) * 512);
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -177,11 +185,11 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
   for (; base + R64_RING < nsteps; base += R64_RING) ring(base, std::true_type{});
   ring(base, std::false_type{});
   // acc[b][j] = sum over k of W[row 16 tile + 4 g + j, k] * x[16 b + r, k]
-  float4_t* ex = (float4_t*)&xs[0][0][0][0];             // [2 up waves][4 blocks][lane]; every read of x is behind the last barrier
+  float4_t* ex = (float4_t*)xs_all;                      // [2 up waves][blocks][lane]; every read of x is behind the last barrier
   if (GLU) {
     if (wave >= 2) {
 #pragma unroll
-      for (int b = 0; b < 4; ++b) ex[((wave - 2) * 4 + b) * TS_WAVE + lane] = acc[b];
+      for (int b = 0; b < BLOCKS; ++b) ex[((wave - 2) * BLOCKS + b) * TS_WAVE + lane] = acc[b];
     }
     __syncthreads();
     if (wave >= 2) return;
@@ -189,11 +197,11 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
   OUT* y = (OUT*)a.y + (int64_t)slice * a.M * a.ldy;
   const int n0 = GLU ? (2 * blockIdx.x + wave) * 16 + 4 * g : tile * 16 + 4 * g;
 #pragma unroll
-  for (int b = 0; b < 4; ++b) {
+  for (int b = 0; b < BLOCKS; ++b) {
     const int m = 16 * b + r;
     if (m >= a.M) continue;
     float4_t u = {0.f, 0.f, 0.f, 0.f};
-    if (GLU) u = ex[(wave * 4 + b) * TS_WAVE + lane];
+    if (GLU) u = ex[(wave * BLOCKS + b) * TS_WAVE + lane];
     acc[b] *= scale[b];
     u *= scale[b];
 #pragma unroll
@@ -201,18 +209,23 @@ __global__ void __launch_bounds__(512) gemm_rows64_kernel(const Rows64Args a) {
   }
 }
 
+#define R64_MAX_ROWS 128
+
 template <bool GLU, typename OUT>
 static int r64_launch(const Rows64Args& a, hipStream_t stream) {
-  gemm_rows64_kernel<GLU, OUT><<<dim3(a.N / 64, a.slices), 512, 0, stream>>>(a);   // 64 rows of W per workgroup
+  // 64 rows of W per workgroup; two buffers of a chunk of x in LDS: 64 KB for up to 64 rows, 128 KB beyond
+  const dim3 grid(a.N / 64, a.slices);
+  if (a.M <= 64) gemm_rows64_kernel<GLU, OUT, 4><<<grid, 512, 2 * R64_CHUNK_STEPS * 4 * TS_WAVE * sizeof(uint4), stream>>>(a);
+  else gemm_rows64_kernel<GLU, OUT, 8><<<grid, 512, 2 * R64_CHUNK_STEPS * 8 * TS_WAVE * sizeof(uint4), stream>>>(a);
   return ts_check_launch();
 }
 
 static bool r64_operands_ok(const void* x, const void* w16, int M, int N, int K, int64_t ldx) {
-  if (M > 64 || K <= 0 || ldx < K || (ldx % 8) || !x || !w16) return false;
+  if (M > R64_MAX_ROWS || K <= 0 || ldx < K || (ldx % 8) || !x || !w16) return false;
   return !((((uintptr_t)x) | ((uintptr_t)w16)) & 15);
 }
 
-// x [M <= 64, K] (row stride ldx), w16: W [N, K] as its 16-row packed copy, y [M, N] or, with glu, [M, N / 2]
+// x [M <= 128, K] (row stride ldx), w16: W [N, K] as its 16-row packed copy, y [M, N] or, with glu, [M, N / 2]
 // (row stride ldy; out_f32: 32-bit sums instead of bfloat16). N a multiple of 64 (128 with glu), K of 1,024.
 // ssq_in [M, ssq_parts] and eps: the prepared norm's scale per row (null: none).
 extern "C" int ts_gemm_rows64_bf16(void* y, const void* x, const void* w16, int M, int N, int K, int64_t ldx, int64_t ldy,

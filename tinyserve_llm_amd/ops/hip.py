@@ -974,18 +974,25 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
 
 ROWS64_MIN_ROWS = 33         # fewer rows are the weight-streaming kernel's (gemm_skinny: 32 rows 16.6 µs against 17.7 here,
                              # 48 rows 23.7 against 19.3, 64 rows 26.9 against 20.7 for a gate|up weight of 16,384 x 2,048),
-ROWS64_MAX_ROWS = 64         # more the matrix library's
+ROWS64_MAX_ROWS = 128        # rows of x the kernel takes (eight blocks of 16 in LDS): more are the matrix library's
+ROWS64_PLAIN_MAX_ROWS = 64   # a plain wide product (the head) of more rows is the library's too: 128 rows against the
+                             # vocabulary matrix take 147 µs here and 125 there. What rides on the kernel pays for 65 to
+                             # 128 rows: the gate (24.0 µs against 24.2 for the library and the gate kernel), and for the
+                             # narrow products in slices the finishing kernel (o 12.7 against 14.2 for the library and
+                             # the norm kernel, down 18.6 against 23.9, q|k|v with the rotation 18.1 against 20.4): a
+                             # decode step at batch 128 takes 2.99 ms instead of 3.20, at batch 96 2.47 instead of 2.76
 ROWS64_MIN_WIDTH = 8192      # rows of W from which 64 of them a workgroup still give every compute unit one
 
 
-def rows64_takes(rows: int, n: int, k: int) -> bool:
-    """Whether `gemm_rows64` is the kernel for `rows` rows of x against a weight [n, k]."""
-    return ROWS64_MIN_ROWS <= rows <= ROWS64_MAX_ROWS and n >= ROWS64_MIN_WIDTH and n % 64 == 0 and k % 1024 == 0
+def rows64_takes(rows: int, n: int, k: int, glu: bool = False) -> bool:
+    """Whether `gemm_rows64` is the kernel for `rows` rows of x against a weight [n, k] (`glu`: with the gate)."""
+    return (ROWS64_MIN_ROWS <= rows <= (ROWS64_MAX_ROWS if glu else ROWS64_PLAIN_MAX_ROWS) and n >= ROWS64_MIN_WIDTH
+            and n % 64 == 0 and k % 1024 == 0)
 
 
 def gemm_rows64(x: torch.Tensor, packed: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, *,
                 glu: bool = False, squares: torch.Tensor | None = None, eps: float = 0.0) -> torch.Tensor:
-    """bfloat16 e(x [M <= 64, K] · W [N, K]^T) for a wide W given as `packed` = pack_weight(W), by the
+    """bfloat16 e(x [M <= 128, K] · W [N, K]^T) for a wide W given as `packed` = pack_weight(W), by the
     kernel that shares x among 64 rows of W through LDS (gemm_rows64.hip). With `glu`, W holds gate
     rows then up rows and the result is silu(gate) * up, [M, N / 2]. With `squares` (and `eps`) x is
     the operand of a `PreparedNorm` and the rows' scales multiply the finished sums."""

@@ -115,7 +115,7 @@ def linear(x: "torch.Tensor | DeferredNorm | hip.PackedRows8", weight: torch.Ten
         d, op = x, x.prepared.operand
         if out_dtype in (None, torch.bfloat16) and _streams(op, weight, dense_rows=True) and not (glu and weight.shape[0] % 32):
             rows, (n, k) = op.shape[0], weight.shape
-            wide = by16 is not None and hip.rows64_takes(rows, n, k) and n % (128 if glu else 64) == 0
+            wide = by16 is not None and hip.rows64_takes(rows, n, k, glu) and n % (128 if glu else 64) == 0
             if wide:
                 return hip.gemm_rows64(op, by16, glu=glu, squares=d.prepared.squares, eps=d.eps)
             if (hip.skinny_fuses(rows, k, False, True) if glu else hip._skinny_serves(rows, n, k)):
@@ -133,7 +133,7 @@ def linear(x: "torch.Tensor | DeferredNorm | hip.PackedRows8", weight: torch.Ten
         x = d.materialize()
     if glu:
         if (out_dtype in (None, torch.bfloat16) and by16 is not None and _streams(x, weight)
-                and hip.rows64_takes(x.shape[0], weight.shape[0], weight.shape[1]) and weight.shape[0] % 128 == 0):
+                and hip.rows64_takes(x.shape[0], weight.shape[0], weight.shape[1], True) and weight.shape[0] % 128 == 0):
             return hip.gemm_rows64(x, by16, glu=True)
         if (out_dtype in (None, torch.bfloat16) and _streams(x, weight) and weight.shape[0] % 32 == 0
                 and hip.skinny_fuses(x.shape[0], weight.shape[1], False, True)):
