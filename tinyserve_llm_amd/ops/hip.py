@@ -102,9 +102,12 @@ def _code(dtype: torch.dtype) -> int:
         raise KernelError(f"kernels exist for float32 and bfloat16, not {dtype}") from None
 
 
-def _need(cond: bool, msg: str) -> None:
+def _need(cond: bool, msg) -> None:
+    """Raises `KernelError(msg)` unless `cond`. A message that formats anything comes as a function
+    that makes it: the checks run at every call of every kernel, and a step of a short prompt is
+    bound by what the host does between launches."""
     if not cond:
-        raise KernelError(msg)
+        raise KernelError(msg() if callable(msg) else msg)
 
 
 def _gpu(*tensors: torch.Tensor | None) -> None:
@@ -169,14 +172,14 @@ def rope_store(qkv: torch.Tensor, cos_sin: torch.Tensor | None, positions: torch
     _gpu(qkv, cos_sin, positions, slots, k_cache, v_cache)
     T = qkv.shape[0]
     row = (num_heads + 2 * num_kv_heads) * head_dim
-    _need(qkv.dim() == 2 and qkv.shape[1] == row and qkv.is_contiguous(), f"qkv must be contiguous [tokens, {row}]")
+    _need(qkv.dim() == 2 and qkv.shape[1] == row and qkv.is_contiguous(), lambda: f"qkv must be contiguous [tokens, {row}]")
     _need(positions.dtype == torch.int32 and positions.shape == (T,) and positions.is_contiguous(),
           "positions must be int32 [tokens]")
     rot = head_dim
     if cos_sin is not None:
         _need(cos_sin.dtype == torch.float32 and cos_sin.dim() == 2 and cos_sin.is_contiguous()
               and 2 <= cos_sin.shape[1] <= head_dim and cos_sin.shape[1] % 2 == 0,
-              f"the rotation table must be float32 [positions, an even width up to head_dim {head_dim}]")
+              lambda: f"the rotation table must be float32 [positions, an even width up to head_dim {head_dim}]")
         rot = cos_sin.shape[1]
     page_size, kst, vst = 1, (0, 0, 0), (0, 0, 0, 0)
     if k_cache is not None:
@@ -197,13 +200,13 @@ def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, dtype: torch.dtyp
     engine's pools keep a head's slots of one dimension together, i.e. pages transposed)."""
     for name, c in (("key", k_cache), ("value", v_cache)):
         _need(c.dim() == 4 and c.shape[2] == nkv and c.shape[3] == hd,
-              f"{name} cache view must be [pages, page_size, {nkv}, {hd}], got {tuple(c.shape)}")
+              lambda: f"{name} cache view must be [pages, page_size, {nkv}, {hd}], got {tuple(c.shape)}")
         _need(c.dtype == dtype, "cache and activations differ in storage type")
         # no two elements may overlap: sort the strides and check each spans the dimensions below it
         span = 1
         for stride, size in sorted(zip(c.stride(), c.shape)):
             if size > 1:
-                _need(stride >= span, f"{name} cache elements overlap")
+                _need(stride >= span, lambda: f"{name} cache elements overlap")
                 span = stride * size
     _need(k_cache.shape == v_cache.shape, "key and value caches differ in shape")
     _need(k_cache.stride(3) == 1, "head_dim must be contiguous in the key cache")
@@ -215,7 +218,7 @@ def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, dtype: torch.dtyp
 def _page_run(pages_per_entry: int) -> int:
     """log2 of the pool pages that one entry of a block table names (a power of two)."""
     _need(pages_per_entry >= 1 and pages_per_entry & (pages_per_entry - 1) == 0 and pages_per_entry <= 65536,
-          f"an entry of a block table names a power of two of pages, not {pages_per_entry}")
+          lambda: f"an entry of a block table names a power of two of pages, not {pages_per_entry}")
     return pages_per_entry.bit_length() - 1
 
 
@@ -231,12 +234,12 @@ def paged_attention_wave(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.
     T, nh, hd = q.shape
     nkv = k_cache.shape[2]
     _check_cache(k_cache, v_cache, q.dtype, nkv, hd)
-    _need(hd % 16 == 0 and hd <= 256, f"head_dim {hd} is not a multiple of 16 up to 256")
-    _need(nh % nkv == 0, f"{nh} heads do not divide into {nkv} key/value heads")
+    _need(hd % 16 == 0 and hd <= 256, lambda: f"head_dim {hd} is not a multiple of 16 up to 256")
+    _need(nh % nkv == 0, lambda: f"{nh} heads do not divide into {nkv} key/value heads")
     _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
           "block_tables must be contiguous int32 [requests, pages]")
     for name, t in (("seq_of_token", seq_of_token), ("positions", positions)):
-        _need(t.dtype == torch.int32 and t.shape == (T,) and t.is_contiguous(), f"{name} must be int32 [tokens]")
+        _need(t.dtype == torch.int32 and t.shape == (T,) and t.is_contiguous(), lambda: f"{name} must be int32 [tokens]")
     out = torch.empty_like(q)
     _run("paged_attention_wave", library().ts_paged_attention_wave(
         _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_of_token), _ptr(positions),
@@ -352,22 +355,22 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     T, nh, hd = q.shape
     nkv = k_cache.shape[2]
     _check_cache(k_cache, v_cache, q.dtype, nkv, hd)
-    _need(nh % nkv == 0, f"{nh} heads do not divide into {nkv} key/value heads")
+    _need(nh % nkv == 0, lambda: f"{nh} heads do not divide into {nkv} key/value heads")
     _need(decode_kernel_takes(q, k_cache, v_cache),
           "the decode kernel takes bfloat16, head_dim 32/64/96/128, groups of up to 16 heads, values in transposed pages")
     _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
           "block_tables must be contiguous int32 [requests, pages]")
     for name, t in (("seq_of_token", seq_of_token), ("positions", positions)):
-        _need(t.dtype == torch.int32 and t.shape == (T,) and t.is_contiguous(), f"{name} must be int32 [tokens]")
-    _need(T <= MAX_DECODE_TOKENS, f"the decode kernel takes up to {MAX_DECODE_TOKENS} tokens a launch")
+        _need(t.dtype == torch.int32 and t.shape == (T,) and t.is_contiguous(), lambda: f"{name} must be int32 [tokens]")
+    _need(T <= MAX_DECODE_TOKENS, lambda: f"the decode kernel takes up to {MAX_DECODE_TOKENS} tokens a launch")
     capacity = block_tables.shape[1] * pages_per_entry * k_cache.shape[1]
     if chunk is None:
         chunk, waves = decode_plan(T, nkv, nh // nkv, hd, capacity)
     waves = waves or 4
     splits = -(-capacity // chunk)
     _need(1 <= waves <= decode_waves(hd, chunk == 32 * waves) and chunk % (32 * waves) == 0 and splits <= MAX_DECODE_SPLITS,
-          f"chunk {chunk} in {waves} waves over {capacity} positions")
-    _need(4 * (32 * waves + waves * (nh // nkv) * hd) <= 65536, f"{waves} waves of {nh // nkv} heads exceed the LDS of a workgroup")
+          lambda: f"chunk {chunk} in {waves} waves over {capacity} positions")
+    _need(4 * (32 * waves + waves * (nh // nkv) * hd) <= 65536, lambda: f"{waves} waves of {nh // nkv} heads exceed the LDS of a workgroup")
     part_o = part_ml = None
     if splits > 1:
         part_o = torch.empty((T, nh, splits, hd), dtype=torch.float32, device=q.device)
@@ -384,7 +387,7 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
 def gemm_exact(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
     """a [M, K] · w [N, K]^T with 32-bit multiply-adds in ascending k."""
     _gpu(a, w)
-    _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], f"shapes {tuple(a.shape)} x {tuple(w.shape)}^T")
+    _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], lambda: f"shapes {tuple(a.shape)} x {tuple(w.shape)}^T")
     _need(a.dtype == w.dtype, "activations and weights differ in storage type")
     _need(a.stride(1) == 1 and w.stride(1) == 1, "rows must be contiguous")
     out_dtype = out_dtype or a.dtype
@@ -416,8 +419,8 @@ def copy_slots(pool: torch.Tensor, src: int, dst: int, num_slots: int, slot_dim:
     _need(pool.is_contiguous() and 1 <= slot_dim < pool.dim(), "pool must be contiguous, pages first")
     _need(pool.element_size() % 2 == 0, "pool elements must be 2 or 4 bytes")
     pages, page_size = pool.shape[0], pool.shape[slot_dim]
-    _need(0 <= src < pages and 0 <= dst < pages and src != dst, f"pages {src}->{dst} outside 0..{pages - 1}")
-    _need(0 <= num_slots <= page_size, f"{num_slots} slots do not fit a page of {page_size}")
+    _need(0 <= src < pages and 0 <= dst < pages and src != dst, lambda: f"pages {src}->{dst} outside 0..{pages - 1}")
+    _need(0 <= num_slots <= page_size, lambda: f"{num_slots} slots do not fit a page of {page_size}")
     runs = 1
     for n in pool.shape[1:slot_dim]:
         runs *= n
@@ -583,26 +586,26 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     T, nh, hd = q.shape
     nkv = k_cache.shape[2]
     _check_cache(k_cache, v_cache, q.dtype, nkv, hd)
-    _need(nh % nkv == 0, f"{nh} heads do not divide into {nkv} key/value heads")
+    _need(nh % nkv == 0, lambda: f"{nh} heads do not divide into {nkv} key/value heads")
     _need(decode_kernel_takes(q, k_cache, v_cache),
           "the prefill kernel takes bfloat16, head_dim 32/64/96/128, groups of up to 16 heads, values in transposed pages")
     _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
           "block_tables must be contiguous int32 [requests, pages]")
     for name, t in (("seq_of_token", seq_of_token), ("positions", positions)):
-        _need(t.dtype == torch.int32 and t.shape == (T,) and t.is_contiguous(), f"{name} must be int32 [tokens]")
+        _need(t.dtype == torch.int32 and t.shape == (T,) and t.is_contiguous(), lambda: f"{name} must be int32 [tokens]")
     _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 2 and tiles.is_contiguous(),
           "tiles must be contiguous int32 [tiles, 2]")
     _need(waves == PREFILL_WAVES or (waves == 2 * PREFILL_WAVES and hd in (64, 128)),
-          f"workgroups of {PREFILL_WAVES} waves, or of {2 * PREFILL_WAVES} for heads of 64 or 128 dimensions")
+          lambda: f"workgroups of {PREFILL_WAVES} waves, or of {2 * PREFILL_WAVES} for heads of 64 or 128 dimensions")
     per_wave = waves * (16 // (nh // nkv))
     tile_tokens = tile_tokens or per_wave
     _need(tile_tokens in (per_wave, 2 * per_wave) or (tile_tokens == 4 * per_wave and waves == PREFILL_WAVES),
-          f"tiles of {tile_tokens} tokens; {per_wave}, twice or (4 waves) four times that")
+          lambda: f"tiles of {tile_tokens} tokens; {per_wave}, twice or (4 waves) four times that")
     out = _out_like(q, out)
     part_o = part_ml = None
     if num_splits > 1:
         _need(chunk > 0 and chunk % 32 == 0 and 0 <= first_token < T, "chunks of a multiple of 32 keys, from a token of the step on")
-        _need(num_splits <= MAX_DECODE_SPLITS, f"at most {MAX_DECODE_SPLITS} chunks")
+        _need(num_splits <= MAX_DECODE_SPLITS, lambda: f"at most {MAX_DECODE_SPLITS} chunks")
         part_o = torch.empty((T, nh, num_splits, hd), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T, nh, num_splits, 2), dtype=torch.float32, device=q.device)
     _run("paged_attention_prefill", library().ts_paged_attention_prefill(
@@ -621,7 +624,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     tables = ctx.block_tables[space]
     # (the tables count in pages of ctx.page_size tokens; the pools may be cut into shorter ones)
     table_page = getattr(ctx, "page_size", 0) or k_cache.shape[1]
-    _need(table_page % k_cache.shape[1] == 0, f"block tables in pages of {table_page} over a cache in pages of {k_cache.shape[1]}")
+    _need(table_page % k_cache.shape[1] == 0, lambda: f"block tables in pages of {table_page} over a cache in pages of {k_cache.shape[1]}")
     per_entry = table_page // k_cache.shape[1]
     if decode_kernel_takes(q, k_cache, v_cache):
         capacity = tables.shape[1] * table_page
@@ -709,10 +712,10 @@ def _next_norm_outputs(x: torch.Tensor, n: int, parts: int, next_norm, skew: int
     residual, weight = next_norm
     _gpu(residual, weight)
     M = x.shape[0] if rows is None else rows
-    _need(weight.dtype == torch.bfloat16 and weight.shape == (n,) and weight.is_contiguous(), f"the next norm's weight must be bfloat16 [{n}]")
+    _need(weight.dtype == torch.bfloat16 and weight.shape == (n,) and weight.is_contiguous(), lambda: f"the next norm's weight must be bfloat16 [{n}]")
     if residual is not None:
         _need(residual.dtype == torch.bfloat16 and residual.shape == (M, n) and residual.is_contiguous(),
-              f"the residual must be bfloat16 [{M}, {n}]")
+              lambda: f"the residual must be bfloat16 [{M}, {n}]")
     out = PreparedNorm(torch.empty((M, n), dtype=torch.bfloat16, device=x.device),
                        torch.empty((M, n + skew), dtype=torch.bfloat16, device=x.device)[:, :n],
                        torch.empty((M, parts), dtype=torch.float32, device=x.device))
@@ -723,7 +726,7 @@ def _check_squares(squares: torch.Tensor | None, rows: int) -> None:
     if squares is not None:
         _gpu(squares)
         _need(squares.dtype == torch.float32 and squares.dim() == 2 and squares.shape[0] == rows and squares.shape[1] >= 1
-              and squares.is_contiguous(), f"the sums of squares must be contiguous float32 [{rows}, parts]")
+              and squares.is_contiguous(), lambda: f"the sums of squares must be contiguous float32 [{rows}, parts]")
 
 
 def pack_weight(weight: torch.Tensor) -> torch.Tensor:
@@ -758,7 +761,7 @@ def _check_packed(packed: torch.Tensor | None, weight: torch.Tensor) -> None:
         n, k = weight.shape
         _gpu(packed)
         _need(packed.dtype == torch.bfloat16 and packed.shape == (-(-n // 16), k // 32, 64, 8) and packed.is_contiguous()
-              and packed.data_ptr() % 16 == 0, f"the packed copy does not belong to a weight of {n} x {k}")
+              and packed.data_ptr() % 16 == 0, lambda: f"the packed copy does not belong to a weight of {n} x {k}")
 
 
 SKINNY8_MAX_ROWS = 8          # rows of x that the 8-row form of the weight-streaming kernel takes
@@ -841,7 +844,7 @@ def pack_weight8(weight: torch.Tensor) -> torch.Tensor:
     _need(weight.dtype == torch.bfloat16 and weight.dim() == 2, "pack_weight8 takes bfloat16 [N, K]")
     n, k = weight.shape
     steps = skinny8_steps(k)
-    _need(steps > 0, f"the 8-row form does not take a reduction of {k}")
+    _need(steps > 0, lambda: f"the 8-row form does not take a reduction of {k}")
     waves, tiles = k // (64 * steps), -(-n // 8)
     padded = weight if n == 8 * tiles else torch.cat([weight, weight.new_zeros(8 * tiles - n, k)])
     # [tile, row, wave, half, step, g, 8] -> [tile, wave, step, g, half, row, 8]
@@ -861,14 +864,14 @@ def gemm_skinny8(x: "torch.Tensor | PackedRows8", weight: torch.Tensor, out_dtyp
     _gpu(xt, weight, packed8)
     _need(xt.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "gemm_skinny8 takes bfloat16")
     _need(len(x.shape) == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
-          f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
+          lambda: f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
     M, K = x.shape
     N = weight.shape[0]
     steps = skinny8_steps(K)
-    _need(M <= SKINNY8_MAX_ROWS and steps > 0, f"gemm_skinny8 takes up to {SKINNY8_MAX_ROWS} rows and K in steps of 256 up to "
+    _need(M <= SKINNY8_MAX_ROWS and steps > 0, lambda: f"gemm_skinny8 takes up to {SKINNY8_MAX_ROWS} rows and K in steps of 256 up to "
           "8192 or of 1024 up to 16384")
     if x_packed:
-        _need(x.steps == steps and xt.is_contiguous() and xt.numel() == 8 * K, f"the packed rows were made for a reader of {x.steps} steps, not {steps}")
+        _need(x.steps == steps and xt.is_contiguous() and xt.numel() == 8 * K, lambda: f"the packed rows were made for a reader of {x.steps} steps, not {steps}")
     _need((x_packed or _dense_rows(xt)) and weight.is_contiguous() and xt.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0,
           "rows must be dense and 16-byte aligned")
     ldx = K if x_packed else xt.stride(0)
@@ -876,7 +879,7 @@ def gemm_skinny8(x: "torch.Tensor | PackedRows8", weight: torch.Tensor, out_dtyp
     if packed8 is not None:
         _need(packed8.dtype == torch.bfloat16 and packed8.shape == (-(-N // 8), K // (64 * steps), steps, 64, 8)
               and packed8.is_contiguous() and packed8.data_ptr() % 16 == 0 and N % 8 == 0,
-              f"the packed copy does not belong to a weight of {N} x {K}")
+              lambda: f"the packed copy does not belong to a weight of {N} x {K}")
     if next_norm is not None:
         _need(out_dtype == torch.bfloat16, "a prepared norm comes with bfloat16")
         prepared, residual, nw = _next_norm_outputs(xt, N, -(-N // 8), next_norm, rows=M)
@@ -920,12 +923,12 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     _gpu(x, weight, residual, norm_weight)
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "gemm_skinny takes bfloat16")
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
-          f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
+          lambda: f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
     M, K = x.shape
     N = weight.shape[0]
     norm = norm_weight is not None
     _need(skinny_fuses(M, K, norm, glu),
-          f"gemm_skinny takes up to {SKINNY_MAX_ROWS} rows ({SKINNY_FUSED_ROWS} with the norm, {SKINNY_EPILOGUE_ROWS} with the gate alone "
+          lambda: f"gemm_skinny takes up to {SKINNY_MAX_ROWS} rows ({SKINNY_FUSED_ROWS} with the norm, {SKINNY_EPILOGUE_ROWS} with the gate alone "
           "over up to 2048) and K in steps of 256 up to 4096 (2048 with the norm) or of 512 up to 8192")
     _need((x.is_contiguous() if norm else _dense_rows(x)) and weight.is_contiguous() and x.data_ptr() % 16 == 0
           and weight.data_ptr() % 16 == 0, "rows must be dense and 16-byte aligned (contiguous with the norm on the way in)")
@@ -1001,9 +1004,9 @@ def gemm_rows64(x: torch.Tensor, packed: torch.Tensor, out_dtype: torch.dtype = 
           and packed.shape[2:] == (64, 8) and packed.is_contiguous(), "gemm_rows64 takes bfloat16 x [M, K] and pack_weight(W)")
     M, K = x.shape
     N = packed.shape[0] * 16
-    _need(packed.shape[1] * 32 == K, f"the packed copy is of a weight over {packed.shape[1] * 32}, x is over {K}")
+    _need(packed.shape[1] * 32 == K, lambda: f"the packed copy is of a weight over {packed.shape[1] * 32}, x is over {K}")
     _need(1 <= M <= ROWS64_MAX_ROWS and N % (128 if glu else 64) == 0 and K % 1024 == 0,
-          f"gemm_rows64 takes up to {ROWS64_MAX_ROWS} rows, N in steps of 64 (128 with the gate) and K in steps of 1024, "
+          lambda: f"gemm_rows64 takes up to {ROWS64_MAX_ROWS} rows, N in steps of 64 (128 with the gate) and K in steps of 1024, "
           f"not {M} x {K} against {N}")
     _need(x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0, "rows of x must be dense and 16-byte aligned")
     _need(out_dtype == torch.bfloat16 or (out_dtype == torch.float32 and not glu), "32-bit output comes without the gate")
@@ -1045,9 +1048,9 @@ def gemm_rows64_sliced(x: torch.Tensor, packed: torch.Tensor, slices: int, next_
           and packed.shape[2:] == (64, 8) and packed.is_contiguous(), "gemm_rows64_sliced takes bfloat16 x [M, K] and pack_weight(W)")
     M, K = x.shape
     N = packed.shape[0] * 16
-    _need(packed.shape[1] * 32 == K, f"the packed copy is of a weight over {packed.shape[1] * 32}, x is over {K}")
+    _need(packed.shape[1] * 32 == K, lambda: f"the packed copy is of a weight over {packed.shape[1] * 32}, x is over {K}")
     _need(1 <= M <= ROWS64_MAX_ROWS and N % 64 == 0 and 1 <= slices <= 64 and K % (ROWS64_SLICE_K * slices) == 0,
-          f"gemm_rows64_sliced takes up to {ROWS64_MAX_ROWS} rows, N in steps of 64 and slices of K that are multiples of "
+          lambda: f"gemm_rows64_sliced takes up to {ROWS64_MAX_ROWS} rows, N in steps of 64 and slices of K that are multiples of "
           f"{ROWS64_SLICE_K}, not {M} x {K} against {N} in {slices}")
     _need(x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0, "rows of x must be dense and 16-byte aligned")
     parts = torch.empty((slices, M, N), dtype=torch.float32, device=x.device)
@@ -1110,7 +1113,7 @@ def qkv_rope_store(x: torch.Tensor, weight: torch.Tensor, cos_sin: torch.Tensor 
           "qkv_rope_store takes up to 16 bfloat16 rows (64 over up to 2048 without the norm), K in steps of 256 up to 4096 "
           "(2048 with the norm), head_dim in steps of 32")
     M, K = x.shape
-    _need(weight.shape == ((num_heads + 2 * num_kv_heads) * head_dim, K), f"weight {tuple(weight.shape)} for "
+    _need(weight.shape == ((num_heads + 2 * num_kv_heads) * head_dim, K), lambda: f"weight {tuple(weight.shape)} for "
           f"{num_heads}+2x{num_kv_heads} heads of {head_dim} over {K}")
     _check_packed(packed, weight)
     _need(positions.dtype == torch.int32 and positions.shape == (M,) and positions.is_contiguous(),
@@ -1185,9 +1188,9 @@ def qkv_rope_store_sliced(x: torch.Tensor, packed_rope: torch.Tensor, slices: in
     N = (num_heads + 2 * num_kv_heads) * head_dim
     _need(x.dtype == torch.bfloat16 and packed_rope.dtype == torch.bfloat16 and packed_rope.dim() == 4
           and packed_rope.shape == (N // 16, K // 32, 64, 8) and packed_rope.is_contiguous() and packed_rope.data_ptr() % 16 == 0,
-          f"qkv_rope_store_sliced takes bfloat16 x [M, K] and pack_weight_rope of a weight [{N}, {K}]")
+          lambda: f"qkv_rope_store_sliced takes bfloat16 x [M, K] and pack_weight_rope of a weight [{N}, {K}]")
     _need(1 <= M <= ROWS64_MAX_ROWS and N % 64 == 0 and head_dim % 32 == 0 and 1 <= slices <= 64 and K % (ROWS64_SLICE_K * slices) == 0,
-          f"qkv_rope_store_sliced takes up to {ROWS64_MAX_ROWS} rows, a width in steps of 64, heads in steps of 32 and slices of K that "
+          lambda: f"qkv_rope_store_sliced takes up to {ROWS64_MAX_ROWS} rows, a width in steps of 64, heads in steps of 32 and slices of K that "
           f"are multiples of {ROWS64_SLICE_K}, not {M} x {K} against {N} in {slices}")
     _need(x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0, "rows of x must be dense and 16-byte aligned")
     _need(positions.dtype == torch.int32 and positions.shape == (M,) and positions.is_contiguous(), "positions must be int32 [tokens]")
@@ -1220,7 +1223,7 @@ def many_rows_products(which: str | None = None) -> str:
     takes). Sets it if `which` is given; returns the setting. It holds for the process."""
     global _many_rows
     if which is not None:
-        _need(which in MANY_ROWS_PRODUCTS, f"products of many rows are one of {MANY_ROWS_PRODUCTS}, not {which!r}")
+        _need(which in MANY_ROWS_PRODUCTS, lambda: f"products of many rows are one of {MANY_ROWS_PRODUCTS}, not {which!r}")
         _many_rows = which
     return _many_rows
 
@@ -1240,7 +1243,7 @@ def gemm_tiled(x: torch.Tensor, weight: torch.Tensor, glu: bool = False,
     is bfloat16, or (without `glu`) the 32-bit sums themselves with `out_dtype` float32."""
     _gpu(x, weight)
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
-          f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
+          lambda: f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
     _need(tiled_takes(x, weight, glu), "the tiled kernel takes bfloat16 operands with dense, 16-byte aligned rows, a "
           "reduction that is a multiple of 64 and a width that is a multiple of 4 (8 with the gate)")
     _need(out_dtype == torch.bfloat16 or (out_dtype == torch.float32 and not glu),
@@ -1312,7 +1315,7 @@ def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     _gpu(x, weight)
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "linear_bf16 takes bfloat16")
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
-          f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
+          lambda: f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
     streams = _dense_rows(x) and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0
     if streams and skinny8_takes(x.shape[0], weight.shape[0], x.shape[1]):
         return gemm_skinny8(x, weight, out_dtype, None if packed is None else packed.by8, next_norm=next_norm)
@@ -1325,7 +1328,7 @@ def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
     _need(next_norm is None, "no kernel leaves a prepared norm for this product (ask next_norm_fuses first)")
     # (float32: the 32-bit sums themselves, as the weight-streaming kernel gives them for few rows, so
     # that a row's logits are rounded the same way whatever the number of rows beside it)
-    _need(out_dtype in (torch.bfloat16, torch.float32), f"bfloat16 products come out as bfloat16 or float32, not {out_dtype}")
+    _need(out_dtype in (torch.bfloat16, torch.float32), lambda: f"bfloat16 products come out as bfloat16 or float32, not {out_dtype}")
     if (streams and packed is not None and packed.by16 is not None
             and rows64_takes(x.shape[0], weight.shape[0], x.shape[1])):
         return gemm_rows64(x, packed.by16, out_dtype)
