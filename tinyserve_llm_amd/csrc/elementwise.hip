@@ -346,23 +346,21 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
     constexpr int VP = 16 / sizeof(T);                // elements of a 16-byte piece
     static_assert(VP == 8 || sizeof(T) == 4, "runs of 8 tokens are pieces of bfloat16");
     if (threadIdx.x < ROPE_TOK / 8) {
-      const int first = t0 + 8 * threadIdx.x;
-      int s0 = -1;
-      if (8 * threadIdx.x + 7 < nt) {
-        int sl[8];
+      // a thread per run of 8 tokens: their slots (tokens that are not there: -1), kept for the slow path, and
+      // whether they are consecutive, aligned and inside one page
+      const int first = 8 * threadIdx.x;
+      int sl[8];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) sl[k] = slots[first + k];
-        s0 = sl[0];
-        bool ok = s0 >= 0 && s0 % 8 == 0 && s0 % page_size + 7 < page_size;
+      for (int k = 0; k < 8; ++k) sl[k] = slots[t0 + min(first + k, nt - 1)];      // (no test between the loads: one trip)
 #pragma unroll
-        for (int k = 1; k < 8; ++k) ok = ok & (sl[k] == s0 + k);
-        if (!ok) s0 = -1;
-      }
-      base_slot[threadIdx.x] = s0;
-    }
-    if (threadIdx.x >= 64 && threadIdx.x < 64 + ROPE_TOK) {
-      const int tl = threadIdx.x - 64;
-      slot_of[tl] = tl < nt ? slots[t0 + tl] : -1;
+      for (int k = 0; k < 8; ++k) sl[k] = first + k < nt ? sl[k] : -1;
+      int s0 = sl[0];
+      bool ok = s0 >= 0 && s0 % 8 == 0 && s0 % page_size + 7 < page_size;
+#pragma unroll
+      for (int k = 1; k < 8; ++k) ok = ok & (sl[k] == s0 + k);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) slot_of[first + k] = sl[k];
+      base_slot[threadIdx.x] = ok ? s0 : -1;
     }
     const int ebeg = (int)((int64_t)(vel / VP) * by / ny) * VP;
     const int eend = (int)((int64_t)(vel / VP) * (by + 1) / ny) * VP;
@@ -374,12 +372,17 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
           *(uint4*)&tile[tl][e - eb] = *(const uint4*)(qkv + (int64_t)(t0 + tl) * row + (nh + nkv) * hd + e);
       }
       __syncthreads();
-      for (int el = threadIdx.x; el < ROPE_VTILE && eb + el < eend; el += blockDim.x) {
-        const int e = eb + el, h = e / hd, d = e - h * hd;
+      // (two loops, chosen by the workgroup as a whole: with the scattered stores inside the fast loop the compiler
+      // works out all sixteen tokens' pages before it looks whether it needs them)
+      bool all_runs = sizeof(T) == 2;
 #pragma unroll
-        for (int run = 0; run < ROPE_TOK / 8; ++run) {
-          const int s0 = base_slot[run];
-          if (s0 >= 0 && sizeof(T) == 2) {
+      for (int run = 0; run < ROPE_TOK / 8; ++run) all_runs = all_runs && base_slot[run] >= 0;
+      if (all_runs) {
+        for (int el = threadIdx.x; el < ROPE_VTILE && eb + el < eend; el += blockDim.x) {
+          const int e = eb + el, h = e / hd, d = e - h * hd;
+#pragma unroll
+          for (int run = 0; run < ROPE_TOK / 8; ++run) {
+            const int s0 = base_slot[run];
             uint32_t w[4];
 #pragma unroll
             for (int k = 0; k < 4; ++k)
@@ -388,16 +391,18 @@ __global__ void rope_store_kernel(T* __restrict__ q_out, T* __restrict__ k_cache
             const int pg = page_of(s0);
             *(uint4*)(v_cache + (int64_t)pg * vp + (s0 - pg * page_size) + (int64_t)h * vh + (int64_t)d * vd) =
                 make_uint4(w[0], w[1], w[2], w[3]);
-          } else {
-            // (tokens of different requests, one slot each: eight stores that wait for nothing but LDS)
+          }
+        }
+      } else {
+        // tokens of different requests, or a run that is not whole: a store per token, its slot out of LDS
+        for (int el = threadIdx.x; el < ROPE_VTILE && eb + el < eend; el += blockDim.x) {
+          const int e = eb + el, h = e / hd, d = e - h * hd;
 #pragma unroll
-            for (int k = 0; k < 8; ++k) {
-              const int tl = 8 * run + k;
-              const int slot = slot_of[tl];
-              if (slot < 0) continue;
-              const int pg = page_of(slot);
-              v_cache[(int64_t)pg * vp + (int64_t)(slot - pg * page_size) * vs + (int64_t)h * vh + (int64_t)d * vd] = tile[tl][el];
-            }
+          for (int tl = 0; tl < ROPE_TOK; ++tl) {
+            const int slot = slot_of[tl];
+            if (slot < 0) continue;
+            const int pg = page_of(slot);
+            v_cache[(int64_t)pg * vp + (int64_t)(slot - pg * page_size) * vs + (int64_t)h * vh + (int64_t)d * vd] = tile[tl][el];
           }
         }
       }
