@@ -136,31 +136,38 @@ def test_bfloat16_fed_whole_and_fed_singly_at_real_sizes(case):
     assert 0.0 < rms <= BF16_RMS * spread and worst <= BF16_WORST * spread
 
 
-def test_a_recorded_batch_of_forty_at_the_1b_sizes(tmp_path):
-    """Forty requests decode together through recorded steps at the 1B layer sizes: above 32 rows the
-    projections are the matrix library's, with the candidate that was fastest when the step was
-    recorded. The replays (a dozen, with the host's own work in between) must give the tokens of
-    eager steps, and every token must lie within the logit gap of the plain implementation's choice."""
+@pytest.mark.parametrize("shape,requests", [("1B", 40), ("3B", 40), ("8B", 40), ("1B", 100), ("3B", 100), ("8B", 100)])
+def test_a_recorded_batch_of_dozens_at_real_sizes(tmp_path, shape, requests):
+    """Forty and a hundred requests decode together through recorded steps at the three layer sizes:
+    above 32 rows the projections are the shared-x kernel's (the gate|up product whole, the narrow
+    ones with their reduction in slices and a finishing kernel that also rotates and writes the cache
+    where the one-kernel form does not reach; from 65 rows with eight blocks of rows in LDS), the head
+    of more than 64 rows the matrix library's. The replays (a dozen, with the host's own work in
+    between) must give the tokens of eager steps, and every token must lie within the logit gap of
+    the plain implementation's choice."""
     from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
     from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
     from tinyserve_llm_amd.engine.sequence import SamplingParams
+    config = SHAPES[shape]
     folder = str(tmp_path)
-    write_random_model(folder, CONFIG, 9, torch.bfloat16)
-    prompts = [prompt(700 + i, 24, CONFIG.vocab_size) for i in range(40)]
+    write_random_model(folder, config, 9, torch.bfloat16)
+    prompts = [prompt(700 + i, 24, config.vocab_size) for i in range(requests)]
     sp = SamplingParams(max_tokens=12, temperature=0.0, ignore_eos=True)
-    sc = SchedulerConfig(max_model_len=64, max_num_seqs=40, max_num_batched_tokens=1024)
+    sc = SchedulerConfig(max_model_len=64, max_num_seqs=requests, max_num_batched_tokens=4096)
     outs = []
     for graphs in (True, False):
-        llm = LLM(folder, sc, CacheConfig(block_size=16), dtype=torch.bfloat16, num_blocks=200, seed=0, decode_graphs=graphs)
+        llm = LLM(folder, sc, CacheConfig(block_size=16), dtype=torch.bfloat16, num_blocks=5 * requests, seed=0, decode_graphs=graphs)
         outs.append([c.token_ids[0] for c in llm.generate(prompts, sp)])
         if graphs:
-            assert 40 in {size for size, width in llm.runner.graphs.graphs}
+            assert -(-requests // 8) * 8 in {size for size, width in llm.runner.graphs.graphs}
+        del llm
     assert outs[0] == outs[1]
     plain = PlainLlama(folder, torch.float64)
-    for p, tokens in list(zip(prompts, outs[0]))[:3]:
+    for r in (0, 1, requests - 1):
+        p, tokens = prompts[r], outs[0][r]
         logits = plain.logits(p + tokens[:-1])[len(p) - 1:]
         gaps = logits.max(-1).values - logits[torch.arange(len(tokens)), torch.tensor(tokens)]
-        assert float(gaps.max()) <= 0.05 * float(logits.std()), f"a token far from the best: gaps {gaps.tolist()}"
+        assert float(gaps.max()) <= 0.05 * float(logits.std()), f"request {r}: a token far from the best: gaps {gaps.tolist()}"
 
 
 @pytest.fixture(scope="module")
