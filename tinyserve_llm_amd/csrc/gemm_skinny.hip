@@ -65,6 +65,7 @@ struct SkinnyArgs {
   bf16_t* k_cache;      // null: this layer owns no cache, only q is produced
   bf16_t* v_cache;
   int nh, nkv, hd, rotate, page_size;
+  int table_vec;        // cos_sin is 16-byte aligned: four of its values go in one load
   int64_t kp, ks, kh, vp, vs, vh, vd;
 };
 
@@ -229,6 +230,23 @@ gemm_skinny_kernel(const SkinnyArgs a) {
     __builtin_amdgcn_sched_barrier(0);
   }
 
+  // ---- EPI_ROPE: the position and the slot of the token this thread will finish are asked for right
+  // behind W as well, and the table's values of that position after the products, ahead of the
+  // waves' meeting, so that neither trip to the cache is made on the way out
+  constexpr int ROPE_ITEMS = RT * CB * 32;
+  const bool rope_early = ROPE && ROPE_ITEMS <= (int)blockDim.x && a.table_vec;
+  int pre_pos = 0;
+  int pre_slot = -1;
+  if constexpr (ROPE) {
+    if (rope_early && (int)threadIdx.x < ROPE_ITEMS) {
+      const int m = (threadIdx.x / 32 % CB) * 16 + ((threadIdx.x & 31) >> 1);
+      if (m < a.M) {
+        if (a.rotate) pre_pos = a.positions[m];
+        if (a.slots) pre_slot = a.slots[m];
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
 
   if constexpr (X_TURNED) {
     // a block at a time through this wave's STEPS kilobytes (a wave's LDS operations keep their order)
@@ -328,6 +346,18 @@ gemm_skinny_kernel(const SkinnyArgs a) {
       if (g == 0) ssq[(b * nwaves + wave) * 16 + r] = run;
     }
   }
+  float4 pre_cos = make_float4(1.f, 1.f, 1.f, 1.f), pre_sin = make_float4(0.f, 0.f, 0.f, 0.f);
+  if constexpr (ROPE) {
+    if (rope_early && a.rotate && (int)threadIdx.x < ROPE_ITEMS) {
+      const int per_head = a.hd / 16, jb = blockIdx.x * RT + threadIdx.x / 32 / CB;
+      if (jb / per_head < a.nh + a.nkv) {
+        const float* cs = a.cos_sin + (int64_t)pre_pos * a.hd + 8 * (jb % per_head) + (threadIdx.x & 1) * 4;
+        pre_cos = *(const float4*)cs;
+        pre_sin = *(const float4*)(cs + a.hd / 2);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
   // acc[t][b][j] = sum over this wave's k of W[row 16 t + 4 g + j of the workgroup, k] * f(x)[16 b + r, k]
 #pragma unroll
   for (int t = 0; t < RT; ++t)
@@ -377,10 +407,11 @@ gemm_skinny_kernel(const SkinnyArgs a) {
         y2[j] = __uint_as_float(sk_round(u[j]) << 16);
       }
       if (a.rotate && head < a.nh + a.nkv) {
-        const float* cs = a.cos_sin + (int64_t)a.positions[m] * a.hd + d0;
+        const float* cs = a.cos_sin + (int64_t)(rope_early ? 0 : a.positions[m]) * a.hd + d0;
+        const float ce[4] = {pre_cos.x, pre_cos.y, pre_cos.z, pre_cos.w}, se[4] = {pre_sin.x, pre_sin.y, pre_sin.z, pre_sin.w};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float c = cs[j], sn = cs[hdh + j];
+          const float c = rope_early ? ce[j] : cs[j], sn = rope_early ? se[j] : cs[hdh + j];
           const float r1 = y1[j] * c - y2[j] * sn, r2 = y2[j] * c + y1[j] * sn;
           y1[j] = r1;
           y2[j] = r2;
@@ -394,7 +425,7 @@ gemm_skinny_kernel(const SkinnyArgs a) {
         *(uint2*)(dst + hdh) = o2;
         continue;
       }
-      const int64_t slot = a.slots ? a.slots[m] : -1;
+      const int slot = rope_early ? pre_slot : a.slots ? a.slots[m] : -1;
       if (!a.k_cache || slot < 0) continue;
       const int64_t page = slot / a.page_size, off = slot - page * a.page_size;
       if (head < a.nh + a.nkv) {
@@ -799,6 +830,7 @@ extern "C" int ts_gemm_skinny_rope_bf16(void* q_out, const void* x, const void* 
   a.ldy = 0; a.eps = eps; a.packed = packed;
   a.cos_sin = cos_sin; a.positions = positions; a.slots = slots; a.q_out = (bf16_t*)q_out;
   a.k_cache = (bf16_t*)k_cache; a.v_cache = (bf16_t*)v_cache; a.nh = nh; a.nkv = nkv; a.hd = hd; a.rotate = rotate;
+  a.table_vec = !(((uintptr_t)cos_sin) & 15);
   a.page_size = page_size; a.kp = kp; a.ks = ks; a.kh = kh; a.vp = vp; a.vs = vs; a.vh = vh; a.vd = vd;
   a.ssq_in = (const float*)ssq_in; a.ssq_parts = ssq_parts;
   if (mode == MODE_PREP && M > 32) return sk_launch<1, 4, 8, MODE_PREP, EPI_ROPE, bf16_t>(a, stream);
