@@ -245,3 +245,89 @@ def test_trace_run_program(case, tmp_path):
     got = {(2, 0): torch.from_numpy(s0[0]), (2, 9): torch.from_numpy(s0[1]),
            (2, len(p) - 1): torch.from_numpy(s2[0]), (1, len(prompts[1]) - 1): torch.from_numpy(s2[1])}
     check(got, oracles["float32"], "float32")
+
+
+def drawn_configuration(rng):
+    """A configuration whose every size is drawn: head sizes in steps of 16 up to 256, any grouping, widths and
+    vocabularies that are no power of two (down to a width of 2 and a vocabulary of 2)."""
+    from tinyserve_llm_amd.config import LlamaConfig, RopeScaling
+    kv = rng.choice([1, 1, 2, 3, 4, 8])
+    scaling = None
+    if rng.random() < 0.5:
+        scaling = RopeScaling(factor=rng.choice([2.0, 8.0, 32.0]), low_freq_factor=1.0, high_freq_factor=rng.choice([2.0, 4.0]),
+                              original_max_position_embeddings=rng.choice([16, 64, 128]))
+    vocab = rng.choice([2, 17, 100, 255, 256, 333, 1001, 4099])
+    return LlamaConfig(
+        vocab_size=vocab, hidden_size=rng.choice([2, 10, 40, 64, 100, 136, 258, 520, 1024]),
+        intermediate_size=rng.choice([2, 30, 100, 128, 150, 300, 520, 1026]), num_hidden_layers=rng.choice([1, 2, 3]),
+        num_attention_heads=kv * rng.choice([1, 1, 2, 3, 4, 5, 7, 8]), num_key_value_heads=kv,
+        head_dim=rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 256]), max_position_embeddings=512,
+        rms_norm_eps=rng.choice([1e-5, 1e-6, 1e-3]), rope_theta=rng.choice([10000.0, 500000.0]), rope_scaling=scaling,
+        tie_word_embeddings=rng.random() < 0.5, eos_token_id=vocab - 1)
+
+
+def drawn_schedule(rng, prompts, pool_pages, page=64, most_live=4):
+    """Steps as in `mixed_schedule`, with everything drawn: the portions (one way of cutting a case: whole prompts,
+    all but the last 32 tokens and then single ones, portions of one to three tokens, or anything up to 100), the
+    places whose logits are wanted (none, some, not always the last) and requests left out of a step."""
+    cursors = [0] * len(prompts)
+    pages = [-(-len(p) // page) for p in prompts]
+    waiting, live, steps = list(range(len(prompts))), [], []
+    way = rng.choice(["whole", "tail", "tiny", "any"])
+    while waiting or live:
+        while waiting and len(live) < most_live and sum(pages[r] for r in live) + pages[waiting[0]] <= pool_pages:
+            live.append(waiting.pop(0))
+        entries, end = [], []
+        for r in live:
+            if len(live) > 1 and rng.random() < 0.15:
+                continue
+            left = len(prompts[r]) - cursors[r]
+            n = {"whole": left, "tail": left - 32 if left > 32 else 1, "tiny": rng.choice([1, 2, 2, 3]),
+                 "any": rng.choice([1, 1, 1, 2, 3, 7, 13, 16, 17, 31, 32, 33, 64, 65, 100])}[way]
+            n = max(1, min(n, left))
+            want = sorted(set(rng.sample(range(n), min(n, rng.choice([0, 1, 1, 2, 3]))) + ([n - 1] if rng.random() < 0.7 else [])))
+            entries.append((r, cursors[r], n, want))
+            cursors[r] += n
+            if cursors[r] == len(prompts[r]):
+                end.append(r)
+        live = [r for r in live if r not in end]
+        if entries:
+            steps.append((entries, end))
+    return steps
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_drawn_configurations_and_schedules(seed, tmp_path):
+    """Neither the sizes nor the schedule are this file's choice: a configuration, two to seven prompts of 1 to 300
+    tokens, a pool that holds the four longest, and a schedule are drawn per case, and both precisions are compared
+    with the plain model at every wanted place. The bounds are relative to the logits' spread: 2e-5 of it in
+    float32 (1.6e-6 is the worst of 7,500 such cases), 4 % in bfloat16 (0.62 % is)."""
+    import random
+
+    from tinyserve_llm_amd.weights.random_init import write_random_model
+    rng = random.Random(50000 + seed)
+    config = drawn_configuration(rng)
+    lengths = [rng.choice([1, 2, 5, 17, 33, 63, 64, 65, 100, 128, 129, 200, 257, 300]) for _ in range(rng.randint(2, 7))]
+    prompts = [[rng.randrange(config.vocab_size) for _ in range(n)] for n in lengths]
+    write_random_model(str(tmp_path), config, seed, rng.choice([torch.float32, torch.bfloat16]))
+    pool = sum(sorted((-(-n // 64) for n in lengths), reverse=True)[:4])
+    steps = drawn_schedule(rng, prompts, pool)
+    for dtype, bound in (("float32", 2e-5), ("bfloat16", 4e-2)):
+        plain = PlainLlama(str(tmp_path), torch.float64, weights_as=torch.bfloat16 if dtype == "bfloat16" else None)
+        oracle = [plain.logits(p) for p in prompts]
+        spread = max(float(o.max() - o.min()) for o in oracle)
+        rep = replayer(str(tmp_path), dtype, 64 * pool)
+        compared = 0
+        for entries, end in steps:
+            logits = rep.step([{"id": f"q{r}", "tokens": prompts[r][s:s + n], "want": w} for r, s, n, w in entries],
+                              [f"q{r}" for r in end])
+            assert logits.shape[0] == sum(len(w) for _, _, _, w in entries)
+            row = 0
+            for r, s, n, w in entries:
+                for j in w:
+                    off = float((logits[row].double().cpu() - oracle[r][s + j]).abs().max())
+                    assert off <= bound * spread, f"{dtype}, request {r}, position {s + j}: off by {off:.3e} of a spread of {spread:.3e}"
+                    row += 1
+                    compared += 1
+        assert rep.manager.num_available_blocks() == rep.manager.num_blocks, "every page came back"
+        print(f"[{dtype}] {compared} rows compared")
