@@ -237,14 +237,54 @@ gemm_skinny_kernel(const SkinnyArgs a) {
   const bool rope_early = ROPE && ROPE_ITEMS <= (int)blockDim.x && a.table_vec;
   int pre_pos = 0;
   int pre_slot = -1;
+  // (the same for what else the way out needs and the products do not give: which head and which of its
+  // dimensions this thread finishes, where its parts lie in LDS and where its values go. A wave has nothing
+  // to do while W is on its way; after the waves' meeting every instruction is waited for.)
+  int way_kind = 0;                                     // 0 nothing, 1 a query or a key (two pieces half a head apart), 2 a value
+  int way_part = 0, way_ssq = 0, way_head = 0, way_d0 = 0;
+  bf16_t* way_dst = nullptr;
+  float inv_k = 1.0f / (float)a.K;
   if constexpr (ROPE) {
     if (rope_early && (int)threadIdx.x < ROPE_ITEMS) {
-      const int m = (threadIdx.x / 32 % CB) * 16 + ((threadIdx.x & 31) >> 1);
-      if (m < a.M) {
+      const int tile = threadIdx.x / 32, t = tile / CB, b = tile - t * CB, ml = (threadIdx.x & 31) >> 1, nl = (threadIdx.x & 1) * 4;
+      const int m = b * 16 + ml;
+      const int per_head = a.hd / 16, jb = blockIdx.x * RT + t;
+      way_head = jb / per_head;
+      way_d0 = 8 * (jb % per_head) + nl;
+      way_part = (t * CB + b) * 256 + ml * 16 + nl;
+      way_ssq = (MODE == MODE_PREP ? b * nwaves : 0) * 16 + ml;
+      if (m < a.M && way_head < a.nh + 2 * a.nkv) {
         if (a.rotate) pre_pos = a.positions[m];
         if (a.slots) pre_slot = a.slots[m];
+        way_kind = way_head < a.nh + a.nkv ? 1 : 2;
+        if (way_head < a.nh) way_dst = a.q_out + ((int64_t)m * a.nh + way_head) * a.hd + way_d0;
       }
     }
+    asm volatile("" : "+v"(way_kind), "+v"(way_part), "+v"(way_ssq), "+v"(way_dst), "+v"(inv_k));
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  // ---- EPI_GLU in bfloat16, four whole columns a thread and at most one item a thread: likewise
+  constexpr int GLU_ITEMS = OT * CB * 64;
+  const bool glu_early = GLU && sizeof(OUT) == 2 && GLU_ITEMS <= (int)blockDim.x &&
+                         (a.y_pack8 || (half % 4 == 0 && a.ldy % 4 == 0 && !(((uintptr_t)a.y) & 7)));
+  if constexpr (GLU && sizeof(OUT) == 2) {
+    if (glu_early && (int)threadIdx.x < GLU_ITEMS) {
+      const int tile = threadIdx.x / 64, e = threadIdx.x & 63, t = tile / CB, b = tile - t * CB, ml = e >> 2, nl = (e & 3) * 4;
+      const int m = b * 16 + ml, n = n0 + t * 16 + nl;
+      way_part = (t * CB + b) * 256 + ml * 16 + nl;
+      way_ssq = (MODE == MODE_PREP ? b * nwaves : 0) * 16 + ml;
+      if (m < a.M && n < half) {
+        way_kind = 1;
+        if (a.y_pack8) {
+          // the four columns are four neighbouring k of the reader's lane (the host has checked the widths)
+          const int S = a.y_pack8, w = n / (64 * S), in_wave = n - w * 64 * S, hf = in_wave / (32 * S), in_half = in_wave - hf * 32 * S;
+          way_dst = (bf16_t*)a.y + (((int64_t)w * S + (in_half >> 5)) * 64 + m + 8 * hf + 16 * ((in_half & 31) >> 3)) * 8 + (n & 7);
+        } else {
+          way_dst = (bf16_t*)a.y + (int64_t)m * a.ldy + n;
+        }
+      }
+    }
+    asm volatile("" : "+v"(way_kind), "+v"(way_part), "+v"(way_ssq), "+v"(way_dst), "+v"(inv_k));
     __builtin_amdgcn_sched_barrier(0);
   }
 
@@ -348,14 +388,22 @@ gemm_skinny_kernel(const SkinnyArgs a) {
   }
   float4 pre_cos = make_float4(1.f, 1.f, 1.f, 1.f), pre_sin = make_float4(0.f, 0.f, 0.f, 0.f);
   if constexpr (ROPE) {
-    if (rope_early && a.rotate && (int)threadIdx.x < ROPE_ITEMS) {
-      const int per_head = a.hd / 16, jb = blockIdx.x * RT + threadIdx.x / 32 / CB;
-      if (jb / per_head < a.nh + a.nkv) {
-        const float* cs = a.cos_sin + (int64_t)pre_pos * a.hd + 8 * (jb % per_head) + (threadIdx.x & 1) * 4;
+    if (rope_early && way_kind) {
+      if (a.rotate && way_kind == 1) {
+        const float* cs = a.cos_sin + (int64_t)pre_pos * a.hd + way_d0;
         pre_cos = *(const float4*)cs;
         pre_sin = *(const float4*)(cs + a.hd / 2);
       }
+      if (way_head >= a.nh) {                           // a key or a value: its place in the pools, or nowhere
+        if (!a.k_cache || pre_slot < 0) way_kind = 0;
+        else {
+          const int64_t page = pre_slot / a.page_size, off = pre_slot - page * a.page_size;
+          way_dst = way_kind == 1 ? a.k_cache + page * a.kp + off * a.ks + (int64_t)(way_head - a.nh) * a.kh + way_d0
+                                  : a.v_cache + page * a.vp + off * a.vs + (int64_t)(way_head - a.nh - a.nkv) * a.vh + (int64_t)way_d0 * a.vd;
+        }
+      }
     }
+    asm volatile("" : "+v"(way_kind), "+v"(way_dst));
     __builtin_amdgcn_sched_barrier(0);
   }
   // acc[t][b][j] = sum over this wave's k of W[row 16 t + 4 g + j of the workgroup, k] * f(x)[16 b + r, k]
@@ -368,8 +416,81 @@ gemm_skinny_kernel(const SkinnyArgs a) {
   __syncthreads();
   // part[.][t][b][m_local * 16 + n_local]: a thread sums 4 consecutive n of one m over the waves in order
   OUT* y = (OUT*)a.y;
-  const float inv_k = 1.0f / (float)a.K;
   const int ncols = GLU ? half : a.N;
+  if constexpr (GLU && sizeof(OUT) == 2) {
+    if (glu_early) {                                    // every thread finishes at most one item, and has prepared it
+      if (!way_kind) return;
+      constexpr int WAVE_PARTS = RT * CB * 256, PAIR = OT * CB * 256;
+      float s[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
+      for (int wv = 0; wv < nwaves; ++wv) {
+        const float4 ps = *(const float4*)(part + wv * WAVE_PARTS + way_part), pu = *(const float4*)(part + wv * WAVE_PARTS + way_part + PAIR);
+        s[0] += ps.x; s[1] += ps.y; s[2] += ps.z; s[3] += ps.w;
+        u[0] += pu.x; u[1] += pu.y; u[2] += pu.z; u[3] += pu.w;
+      }
+      if (MODE != MODE_PLAIN) {
+        float total = 0.f;
+        for (int wv = 0; wv < nwaves; ++wv) total += ssq[way_ssq + wv * 16];
+        const float inv = __builtin_amdgcn_rsqf(total * inv_k + a.eps);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { s[j] *= inv; u[j] *= inv; }
+      }
+      float v[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = sk_silu(s[j]) * u[j];
+      if (a.y_pack8) *(uint2*)way_dst = make_uint2(sk_round(v[0]) | (sk_round(v[1]) << 16), sk_round(v[2]) | (sk_round(v[3]) << 16));
+      else *(uint2*)way_dst = make_uint2(f2bf(v[0]) | ((uint32_t)f2bf(v[1]) << 16), f2bf(v[2]) | ((uint32_t)f2bf(v[3]) << 16));
+      return;
+    }
+  }
+  if constexpr (ROPE) {
+    if (rope_early) {                                   // every thread finishes at most one item, and has prepared it
+      if (!way_kind) return;
+      constexpr int WAVE_PARTS = RT * CB * 256;
+      float s[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
+      for (int wv = 0; wv < nwaves; ++wv) {
+        const float4 ps = *(const float4*)(part + wv * WAVE_PARTS + way_part), pu = *(const float4*)(part + wv * WAVE_PARTS + way_part + 8);
+        s[0] += ps.x; s[1] += ps.y; s[2] += ps.z; s[3] += ps.w;
+        u[0] += pu.x; u[1] += pu.y; u[2] += pu.z; u[3] += pu.w;
+      }
+      if (MODE != MODE_PLAIN) {
+        float total = 0.f;
+        for (int wv = 0; wv < nwaves; ++wv) total += ssq[way_ssq + wv * 16];
+        const float inv = __builtin_amdgcn_rsqf(total * inv_k + a.eps);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { s[j] *= inv; u[j] *= inv; }
+      }
+      float y1[4], y2[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {                       // as the product would be stored
+        y1[j] = __uint_as_float(sk_round(s[j]) << 16);
+        y2[j] = __uint_as_float(sk_round(u[j]) << 16);
+      }
+      if (a.rotate && way_kind == 1) {
+        const float ce[4] = {pre_cos.x, pre_cos.y, pre_cos.z, pre_cos.w}, se[4] = {pre_sin.x, pre_sin.y, pre_sin.z, pre_sin.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float r1 = y1[j] * ce[j] - y2[j] * se[j], r2 = y2[j] * ce[j] + y1[j] * se[j];
+          y1[j] = r1;
+          y2[j] = r2;
+        }
+      }
+      const uint2 o1 = make_uint2(sk_round(y1[0]) | (sk_round(y1[1]) << 16), sk_round(y1[2]) | (sk_round(y1[3]) << 16));
+      const uint2 o2 = make_uint2(sk_round(y2[0]) | (sk_round(y2[1]) << 16), sk_round(y2[2]) | (sk_round(y2[3]) << 16));
+      const int hdh = a.hd / 2;
+      if (way_kind == 1) {
+        *(uint2*)way_dst = o1;
+        *(uint2*)(way_dst + hdh) = o2;
+      } else {
+        const uint32_t w1[2] = {o1.x, o1.y}, w2[2] = {o2.x, o2.y};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          way_dst[(int64_t)j * a.vd] = (bf16_t)(w1[j >> 1] >> (16 * (j & 1)));
+          way_dst[(int64_t)(hdh + j) * a.vd] = (bf16_t)(w2[j >> 1] >> (16 * (j & 1)));
+        }
+      }
+      return;
+    }
+  }
   // ROPE: a tile gives 8 columns of a head's first half (n_local 0 .. 7) and their partners (n_local 8 .. 15): 32 items of 4
   constexpr int PER_TILE = ROPE ? 32 : 64;
   for (int idx = threadIdx.x; idx < OT * CB * PER_TILE; idx += blockDim.x) {
@@ -407,11 +528,10 @@ gemm_skinny_kernel(const SkinnyArgs a) {
         y2[j] = __uint_as_float(sk_round(u[j]) << 16);
       }
       if (a.rotate && head < a.nh + a.nkv) {
-        const float* cs = a.cos_sin + (int64_t)(rope_early ? 0 : a.positions[m]) * a.hd + d0;
-        const float ce[4] = {pre_cos.x, pre_cos.y, pre_cos.z, pre_cos.w}, se[4] = {pre_sin.x, pre_sin.y, pre_sin.z, pre_sin.w};
+        const float* cs = a.cos_sin + (int64_t)a.positions[m] * a.hd + d0;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float c = rope_early ? ce[j] : cs[j], sn = rope_early ? se[j] : cs[hdh + j];
+          const float c = cs[j], sn = cs[hdh + j];
           const float r1 = y1[j] * c - y2[j] * sn, r2 = y2[j] * c + y1[j] * sn;
           y1[j] = r1;
           y2[j] = r2;
@@ -425,7 +545,7 @@ gemm_skinny_kernel(const SkinnyArgs a) {
         *(uint2*)(dst + hdh) = o2;
         continue;
       }
-      const int slot = rope_early ? pre_slot : a.slots ? a.slots[m] : -1;
+      const int slot = a.slots ? a.slots[m] : -1;
       if (!a.k_cache || slot < 0) continue;
       const int64_t page = slot / a.page_size, off = slot - page * a.page_size;
       if (head < a.nh + a.nkv) {
@@ -620,13 +740,24 @@ gemm_skinny8_kernel(const SkinnyArgs a) {
   }
   __builtin_amdgcn_sched_barrier(0);                    // all of W's loads are in flight before anything waits
   // EPI_NEXT: the residual and the next norm's weight of the element this thread will finish, asked for right behind W
+  // (and where its results go is worked out here, while W is on its way: after the waves' meeting every instruction is waited for)
   bf16_t pre_res = 0, pre_nw = 0;
+  bf16_t *way_res = nullptr, *way_op = nullptr;
+  float* way_sq = nullptr;
+  int way_pair = 0;                                     // 1: this thread stores its column and the next as one word; 2: singly
   if constexpr (NEXT) {
     const int m = threadIdx.x >> 3, n = n0 + (threadIdx.x & 7);
     if (threadIdx.x < 64 && m < a.M && n < a.N) {
       pre_nw = a.next_nw[n];
       if (a.next_res) pre_res = a.next_res[(int64_t)m * a.N + n];
     }
+    if (threadIdx.x < 64 && m < a.M) {
+      way_res = a.next_res_out + (int64_t)m * a.N + n;
+      way_op = a.next_op + (int64_t)m * a.N + n;
+      way_sq = a.ssq_out + (int64_t)m * gridDim.x + blockIdx.x;
+      if (!(threadIdx.x & 1)) way_pair = n + 1 < a.N && !((((uintptr_t)way_res) | ((uintptr_t)way_op)) & 3) ? 1 : 2;
+    }
+    asm volatile("" : "+v"(way_res), "+v"(way_op), "+v"(way_sq), "+v"(way_pair));
     __builtin_amdgcn_sched_barrier(0);
   }
   float4_t acc = {0.f, 0.f, 0.f, 0.f};
@@ -661,19 +792,15 @@ gemm_skinny8_kernel(const SkinnyArgs a) {
     sq += __shfl_xor(sq, 1, TS_WAVE);
     sq += __shfl_xor(sq, 2, TS_WAVE);
     sq += __shfl_xor(sq, 4, TS_WAVE);
-    if (nl == 0 && m < a.M) a.ssq_out[(int64_t)m * gridDim.x + blockIdx.x] = sq;
+    if (nl == 0 && m < a.M) *way_sq = sq;
     const uint32_t res_mine = sk_round(t), op_mine = sk_round(t * bf2f(pre_nw));
     const uint32_t res_next = __shfl_down(res_mine, 1, TS_WAVE), op_next = __shfl_down(op_mine, 1, TS_WAVE);
-    if (m < a.M && !(nl & 1)) {
-      bf16_t* r_dst = a.next_res_out + (int64_t)m * a.N + n;
-      bf16_t* o_dst = a.next_op + (int64_t)m * a.N + n;
-      if (n + 1 < a.N && !((((uintptr_t)r_dst) | ((uintptr_t)o_dst)) & 3)) {
-        *(uint32_t*)r_dst = res_mine | (res_next << 16);
-        *(uint32_t*)o_dst = op_mine | (op_next << 16);
-      } else {
-        if (n < a.N) { r_dst[0] = (bf16_t)res_mine; o_dst[0] = (bf16_t)op_mine; }
-        if (n + 1 < a.N) { r_dst[1] = (bf16_t)res_next; o_dst[1] = (bf16_t)op_next; }
-      }
+    if (way_pair == 1) {
+      *(uint32_t*)way_res = res_mine | (res_next << 16);
+      *(uint32_t*)way_op = op_mine | (op_next << 16);
+    } else if (way_pair == 2) {
+      if (n < a.N) { way_res[0] = (bf16_t)res_mine; way_op[0] = (bf16_t)op_mine; }
+      if (n + 1 < a.N) { way_res[1] = (bf16_t)res_next; way_op[1] = (bf16_t)op_next; }
     }
   } else if constexpr (sizeof(OUT) == 4) {
     if (m < a.M && n < a.N) ((float*)a.y)[(int64_t)m * a.ldy + n] = sum;
