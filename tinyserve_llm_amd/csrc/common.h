@@ -29,6 +29,21 @@ template <> struct Num<bf16_t> {
   static __device__ __forceinline__ float round(float v) { return bf2f(f2bf(v)); }
 };
 
+// A kernel's arguments lie in memory that no cache holds when the kernel starts, and the compiler fetches them
+// as the code comes to need them: a long argument block is then waited for two or three times, a trip to
+// memory each, before the first load of the operands can go out. This asks for one word of each 64 bytes of
+// the block at the very start, so that all of it arrives in one trip and every later fetch finds it in the
+// scalar cache.
+template <int BYTES>
+__device__ __forceinline__ void ts_fetch_arguments() {
+  typedef const uint32_t __attribute__((address_space(4))) * args_t;
+  const args_t block = (args_t)__builtin_amdgcn_kernarg_segment_ptr();
+  uint32_t seen = 0;
+#pragma unroll
+  for (int at = 0; at < BYTES; at += 64) seen |= block[at / 4];
+  asm volatile("" ::"s"(seen));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int off = TS_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, TS_WAVE);

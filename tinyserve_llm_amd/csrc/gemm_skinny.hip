@@ -79,6 +79,7 @@ gemm_skinny_kernel(const SkinnyArgs a) {
   static_assert(!GLU || RT % 2 == 0, "gate and up tiles come in pairs");
   // steps of x fetched at a time: fewer where more blocks of x, more row tiles of W or a larger workgroup leave fewer registers
   constexpr int SK_XBATCH = CB >= 4 ? 4 : (CB == 2 && (MAXT > 512 || RT >= 4)) ? 4 : 8;
+  ts_fetch_arguments<sizeof(SkinnyArgs)>();
   extern __shared__ __align__(16) float smem[];
   const int nwaves = blockDim.x / TS_WAVE;
   float* part = smem;                                   // [nwaves][RT][CB][256]
@@ -707,6 +708,7 @@ static int sk_dispatch(const SkinnyArgs& a, hipStream_t stream) {
 template <int STEPS, int MAXT, typename OUT, bool NEXT = false>
 __global__ void __launch_bounds__(MAXT)
 gemm_skinny8_kernel(const SkinnyArgs a) {
+  ts_fetch_arguments<sizeof(SkinnyArgs)>();
   extern __shared__ __align__(16) float smem[];         // [nwaves][256]
   const int nwaves = blockDim.x / TS_WAVE;
   const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
