@@ -33,6 +33,7 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, fl
                         int num_splits, int chunk, float scale2, int window) {
   constexpr int NC = HD / 32;    // 32-dimension pieces of a key row (one 16-byte load per lane each)
   constexpr int NDB = HD / 16;   // 16-dimension blocks of the output
+  ts_fetch_arguments<164>();     // (nine pointers, five numbers, six strides, four more numbers and the scale)
   extern __shared__ __align__(16) float smem[];
   const int nw = blockDim.x / TS_WAVE;
   float* wm = smem;                       // [waves][16]
@@ -42,11 +43,13 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, fl
   const int tid = threadIdx.x, wave = wave_index(), lane = tid & (TS_WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
   const int split = blockIdx.x, kvh = blockIdx.y, t = blockIdx.z;
-  const int pos = positions[t];
+  int pos = positions[t];
+  int seq = seq_of_token[t];                    // (asked for with the position: one trip to memory, not one after the other;
+  asm volatile("" : "+s"(pos), "+s"(seq));      //  left to itself the compiler fetches it when it has seen that the chunk is visible)
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int k0 = split * chunk;
   if (k0 > pos || k0 + chunk <= lo) return;     // nothing of this chunk is visible
-  const int32_t* table = block_tables + (int64_t)seq_of_token[t] * max_blocks;
+  const int32_t* table = block_tables + (int64_t)seq * max_blocks;
   const PageMath pm{page_size, page_shift, page_run};
 
   uint4 qreg[NC];
