@@ -289,6 +289,27 @@ gemm_skinny_kernel(const SkinnyArgs a) {
     __builtin_amdgcn_sched_barrier(0);
   }
 
+  // ---- EPI_NEXT with whole columns and at most one item a thread: likewise (way_dst the new residual's place,
+  // way_op the next operand's, way_sq the place of the tile's share of the row's squares)
+  bf16_t* way_op = nullptr;
+  float* way_sq = nullptr;
+  if constexpr (NEXT) {
+    if (next_early && (int)threadIdx.x < NEXT_ITEMS) {
+      const int tile = threadIdx.x / 64, e = threadIdx.x & 63, t = tile / CB, b = tile - t * CB, ml = e >> 2, nl = (e & 3) * 4;
+      const int m = b * 16 + ml, n = n0 + t * 16 + nl;
+      way_part = (t * CB + b) * 256 + ml * 16 + nl;
+      way_ssq = (MODE == MODE_PREP ? b * nwaves : 0) * 16 + ml;
+      if (m < a.M) {
+        way_kind = n < a.N ? 1 : 2;                     // 2: past the last column, only its zero goes into the row's squares
+        way_dst = a.next_res_out + (int64_t)m * a.N + n;
+        way_op = a.next_op + (int64_t)m * a.N + n;
+        way_sq = a.ssq_out + (int64_t)m * gridDim.x * OT + (int64_t)blockIdx.x * OT + t;
+      }
+    }
+    asm volatile("" : "+v"(way_kind), "+v"(way_part), "+v"(way_ssq), "+v"(way_dst), "+v"(way_op), "+v"(way_sq), "+v"(inv_k));
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
   if constexpr (X_TURNED) {
     // a block at a time through this wave's STEPS kilobytes (a wave's LDS operations keep their order)
     uint4* turn = (uint4*)smem + (size_t)wave * STEPS * TS_WAVE;
@@ -418,6 +439,44 @@ gemm_skinny_kernel(const SkinnyArgs a) {
   // part[.][t][b][m_local * 16 + n_local]: a thread sums 4 consecutive n of one m over the waves in order
   OUT* y = (OUT*)a.y;
   const int ncols = GLU ? half : a.N;
+  if constexpr (NEXT) {
+    if (next_early) {                                   // every thread finishes at most one item, and has prepared it
+      if ((int)threadIdx.x >= NEXT_ITEMS) return;       // (whole waves: an item's four threads stay together)
+      constexpr int WAVE_PARTS = RT * CB * 256;
+      float s[4] = {0.f, 0.f, 0.f, 0.f};
+      for (int wv = 0; wv < nwaves; ++wv) {
+        const float4 ps = *(const float4*)(part + wv * WAVE_PARTS + way_part);
+        s[0] += ps.x; s[1] += ps.y; s[2] += ps.z; s[3] += ps.w;
+      }
+      if (MODE != MODE_PLAIN) {
+        float total = 0.f;
+        for (int wv = 0; wv < nwaves; ++wv) total += ssq[way_ssq + wv * 16];
+        const float inv = __builtin_amdgcn_rsqf(total * inv_k + a.eps);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s[j] *= inv;
+      }
+      // t = T(y) + res; the new residual T(t), the next operand T(t * nw), and the tile's share of the row's sum of t^2
+      float sq = 0.f, tv[4], ov[4];
+      const uint32_t early_res[2] = {pre_res.x, pre_res.y}, early_nw[2] = {pre_nw.x, pre_nw.y};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {                       // (the low half of a word is the even column)
+        const float rj = __uint_as_float((early_res[j >> 1] >> (16 * (j & 1))) << 16);
+        const float nj = __uint_as_float((early_nw[j >> 1] >> (16 * (j & 1))) << 16);
+        const float sum = __uint_as_float(sk_round(s[j]) << 16) + rj;
+        tv[j] = sum;
+        ov[j] = sum * nj;
+        sq = way_kind == 1 ? fmaf(sum, sum, sq) : sq;
+      }
+      sq += __shfl_xor(sq, 1, TS_WAVE);
+      sq += __shfl_xor(sq, 2, TS_WAVE);
+      if (way_kind && !(threadIdx.x & 3)) *way_sq = sq;
+      if (way_kind == 1) {
+        *(uint2*)way_dst = make_uint2(sk_round(tv[0]) | (sk_round(tv[1]) << 16), sk_round(tv[2]) | (sk_round(tv[3]) << 16));
+        *(uint2*)way_op = make_uint2(sk_round(ov[0]) | (sk_round(ov[1]) << 16), sk_round(ov[2]) | (sk_round(ov[3]) << 16));
+      }
+      return;
+    }
+  }
   if constexpr (GLU && sizeof(OUT) == 2) {
     if (glu_early) {                                    // every thread finishes at most one item, and has prepared it
       if (!way_kind) return;
