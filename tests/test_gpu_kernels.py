@@ -1381,3 +1381,47 @@ def test_fused_projection_reads_the_packed_copy_to_the_same_result():
                                     nh, nkv, hd, packed=packed)
         outs.append((q, kp, vp))
     assert all(torch.equal(a, b) for a, b in zip(*outs))
+
+
+@pytest.mark.parametrize("heads,kv,hd,chunk,waves,window", [(32, 8, 64, 256, 8, 0), (32, 8, 64, 128, 4, 0), (16, 8, 128, 256, 4, 0),
+                                                             (8, 2, 32, 128, 4, 300), (16, 4, 96, 512, 4, 0), (24, 8, 64, 128, 4, 700)])
+def test_o_projection_adds_up_the_chunks_of_a_split_walk_itself(heads, kv, hd, chunk, waves, window):
+    """The decode kernel told to leave its chunks' parts uncombined, and the 8-row form that makes its x
+    from them on the way in (one token): bit for bit what the combining kernel and the 8-row form give one
+    after the other, with and without finishing into the next norm, and what the combining kernel gives
+    from the parts is what the decode kernel gives when it combines itself. Contexts that end inside
+    the first chunk, at a chunk's edge and in the last chunk; a window that hides the first chunks."""
+    dtype = torch.bfloat16
+    n, page = 2000, 32
+    g = gen(heads + hd + chunk)
+    k, v = torch.randn(n, kv, hd, generator=g).to(dtype), torch.randn(n, kv, hd, generator=g).to(dtype)
+    pages = -(-n // page)
+    table = list(range(pages - 1, -1, -1))
+    kc, vc = engine_layout(k, v, table, page, pages, dtype)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev())
+    K = heads * hd
+    w = (torch.randn(520, K, generator=g) * 0.05).to(dtype).to(dev())
+    nw = (1 + 0.1 * torch.randn(520, generator=g)).to(dtype).to(dev())
+    for pos in (5, chunk - 1, chunk, chunk + 1, 1000, 1999):
+        q = torch.randn(1, heads, hd, generator=g).to(dtype).to(dev())
+        res = torch.randn(1, 520, generator=g).to(dtype).to(dev())
+        args = (q, kc, vc, i32([table]), i32([0]), i32([pos]), hd ** -0.5, window)
+        whole = hip().paged_attention_decode(*args, chunk=chunk, waves=waves)
+        split = hip().paged_attention_decode(*args, chunk=chunk, waves=waves, leave_split=True)
+        if -(-n // chunk) > hip().SPLIT_ATTENTION_MAX_CHUNKS:
+            assert isinstance(split, torch.Tensor) and torch.equal(split, whole), "too many chunks: combined as ever"
+            continue
+        assert isinstance(split, hip().SplitAttention) and split.shape == (1, K)
+        x = split.combined()
+        assert torch.equal(x.view(1, heads, hd), whole)
+        assert hip().split_attention_fuses(1, w) == (K <= 2048)
+        if K > 2048:
+            with pytest.raises(hip().KernelError, match="parts"):
+                hip().gemm_skinny8(split, w)
+            continue
+        assert torch.equal(hip().gemm_skinny8(split, w), hip().gemm_skinny8(x, w))
+        assert torch.equal(hip().gemm_skinny8(split, w, packed8=hip().pack_weight8(w)), hip().gemm_skinny8(x, w))
+        for residual in (res, None):
+            a, b = hip().gemm_skinny8(split, w, next_norm=(residual, nw)), hip().gemm_skinny8(x, w, next_norm=(residual, nw))
+            assert torch.equal(a.summed, b.summed) and torch.equal(a.operand, b.operand) and torch.equal(a.squares, b.squares)
+    assert not hip().split_attention_fuses(2, w)

@@ -169,6 +169,15 @@ attn_decode_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ p
   }
 }
 
+// The combining kernel alone: out [tokens, nh, hd] bfloat16 from the parts that ts_paged_attention_decode leaves
+// with combine 0.
+extern "C" int ts_attention_combine(void* out, const float* part_o, const float* part_ml, const int32_t* positions,
+                                    int num_tokens, int nh, int hd, int num_splits, int chunk, int window, hipStream_t stream) {
+  if (num_tokens <= 0) return TS_OK;
+  if (!out || !part_o || !part_ml || !positions || nh <= 0 || hd <= 0 || num_splits < 1 || chunk <= 0) return TS_BAD_SHAPE;
+  return ts_launch_attention_combine(out, part_o, part_ml, positions, num_tokens, nh, hd, num_splits, chunk, window, stream);
+}
+
 // The combining kernel alone, for the prefill kernel's split walks (declared in attention_mfma.h).
 int ts_launch_attention_combine(void* out, const float* part_o, const float* part_ml, const int32_t* positions,
                                 int num_tokens, int nh, int hd, int num_splits, int chunk, int window,
@@ -192,7 +201,7 @@ extern "C" int ts_paged_attention_decode(void* out, float* part_o, float* part_m
                                          const int32_t* seq_of_token, const int32_t* positions, int num_tokens, int nh,
                                          int nkv, int hd, int page_size, int64_t kp, int64_t ks, int64_t kh,
                                          int64_t vp, int64_t vh, int64_t vd, int max_blocks, int num_splits, int chunk,
-                                         int waves, float scale, int window, int page_run, hipStream_t stream) {
+                                         int waves, float scale, int window, int page_run, int combine, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
   if (nkv <= 0 || nh % nkv || page_size <= 0 || page_size % 8 || max_blocks <= 0 || num_splits <= 0 || page_run < 0 || page_run > 16)
     return TS_BAD_SHAPE;
@@ -229,7 +238,7 @@ extern "C" int ts_paged_attention_decode(void* out, float* part_o, float* part_m
 #undef TS_DEC
 #undef TS_DEC1
   int rc = ts_check_launch();
-  if (rc || num_splits == 1) return rc;
+  if (rc || num_splits == 1 || !combine) return rc;     // (combine 0: the caller's next kernel reads the parts itself)
   attn_decode_combine_kernel<<<num_tokens * nh, TS_WAVE, 0, stream>>>((bf16_t*)out, part_o, part_ml, positions, nh, hd,
                                                                       num_splits, chunk, window);
   return ts_check_launch();

@@ -45,6 +45,11 @@ struct SkinnyArgs {
   // projection of 8 rows over 8,192: 10.8 -> 9.2 us). y_pack8 > 0: the gated product is stored that way for a
   // reader of y_pack8 steps; x_packed8: x comes that way (ldx is unused). Lanes of rows past M hold anything.
   int x_packed8, y_pack8;
+  // x_packed8 == 2: the 8-row form for one token (M = 1), x not given but made on the way in from the parts that the
+  // split-key attention kernel has left (the combining kernel's sums, bit for bit): x is the token's heads side by
+  // side, head h of it sum_s o[h, s, :] 2^(m_s - M) / sum_s l_s 2^(m_s - M) over the chunks s that hold keys it
+  // sees. Its operands travel in fields that the 8-row form leaves unused otherwise, so that the block of arguments
+  // which every kernel of this file fetches stays as short as it is (see SkinnyParts).
   int64_t ldx, ldw, ldy;
   float eps;
   // MODE_PREP: sums of squares [M, ssq_parts] of the rows of h + res, in parts (K is their width)
@@ -764,9 +769,20 @@ static int sk_dispatch(const SkinnyArgs& a, hipStream_t stream) {
 // gives 256 workgroups, one per compute unit, and a reduction of 8,192 fits the 8 waves of one
 // workgroup (a wave covers 64 STEPS of k), where the 16-row form needs 16 waves on half the chip.
 // packed: W in the order of these loads, [N / 8 tiles][waves][STEPS][lane][8] (see hip.pack_weight8).
-template <int STEPS, int MAXT, typename OUT, bool NEXT = false>
+#define SK_COMB_CHUNKS 16     // most chunks that the instance which makes its x from an attention's parts adds up
+// The operands of that instance, out of the fields they travel in.
+struct SkinnyParts {
+  const float* o;            // [K / hd heads, splits, hd]: the chunks' weighted values            (SkinnyArgs::x)
+  const float* ml;           // [heads, splits, 2]: a chunk's running maximum (log2 units) and sum   (ssq_in)
+  const int32_t* pos;        // [1]: the token's position                                            (positions)
+  int splits, chunk, window, hd;   //                                                                (nh, nkv, rotate, hd)
+  __device__ __host__ SkinnyParts(const SkinnyArgs& a)
+      : o((const float*)a.x), ml(a.ssq_in), pos(a.positions), splits(a.nh), chunk(a.nkv), window(a.rotate), hd(a.hd) {}
+};
+template <int STEPS, int MAXT, typename OUT, bool NEXT = false, bool COMB = false>
 __global__ void __launch_bounds__(MAXT)
 gemm_skinny8_kernel(const SkinnyArgs a) {
+  static_assert(!COMB || (STEPS == 4 && MAXT <= 512 && sizeof(OUT) == 2), "x from parts: a wave's 256 k of one token fit its kilobyte of LDS");
   ts_fetch_arguments<sizeof(SkinnyArgs)>();
   extern __shared__ __align__(16) float smem[];         // [nwaves][256]
   const int nwaves = blockDim.x / TS_WAVE;
@@ -783,7 +799,29 @@ gemm_skinny8_kernel(const SkinnyArgs a) {
   const bf16_t* xrow = a.x_packed8 ? a.x + ((int64_t)wave * STEPS * 64 + lane) * 8 : a.x + (int64_t)(row < a.M ? row : 0) * a.ldx + kbeg;
   const int xstep = a.x_packed8 ? 512 : SK_KSTEP;       // from a step's piece to the next step's
   uint4 xb[XB];
-  if (X_FIRST) {
+  // COMB: lane l makes the wave's k 4 l .. 4 l + 3 (they lie in one head). Every chunk's maximum, sum and four
+  // values are asked for here, ahead of W (a chunk that holds nothing the token sees reads the last that does, and
+  // counts with weight zero); they are added up once W's loads are out.
+  float2 c_ml[COMB ? SK_COMB_CHUNKS : 1];
+  float4 c_po[COMB ? SK_COMB_CHUNKS : 1];
+  int c_s0 = 0, c_s1 = 0;
+  if constexpr (COMB) {
+    const SkinnyParts parts(a);
+    const int pos = parts.pos[0];
+    const int lo = (parts.window > 0 && pos - parts.window + 1 > 0) ? pos - parts.window + 1 : 0;
+    c_s0 = min(lo / parts.chunk, parts.splits - 1);
+    c_s1 = min(pos / parts.chunk, parts.splits - 1);
+    const int k4 = wave * (2 * STEPS * SK_KSTEP) + 4 * lane, head = k4 / parts.hd, d = k4 - head * parts.hd;
+    const float* ml = parts.ml + (int64_t)head * parts.splits * 2;
+    const float* po = parts.o + (int64_t)head * parts.splits * parts.hd + d;
+#pragma unroll
+    for (int i = 0; i < SK_COMB_CHUNKS; ++i) {
+      const int c = c_s0 + i <= c_s1 ? c_s0 + i : c_s1;
+      c_ml[i] = *(const float2*)(ml + 2 * c);
+      c_po[i] = *(const float4*)(po + (int64_t)c * parts.hd);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  } else if (X_FIRST) {
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) xb[s] = *(const uint4*)(xrow + s * xstep);
     __builtin_amdgcn_sched_barrier(0);
@@ -820,6 +858,35 @@ gemm_skinny8_kernel(const SkinnyArgs a) {
     }
     asm volatile("" : "+v"(way_res), "+v"(way_op), "+v"(way_sq), "+v"(way_pair));
     __builtin_amdgcn_sched_barrier(0);
+  }
+  if constexpr (COMB) {
+    float top = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < SK_COMB_CHUNKS; ++i) top = c_s0 + i <= c_s1 ? fmaxf(top, c_ml[i].x) : top;
+    // the chunks' sums as the combining kernel's wave adds them: chunk s0 + i in lane i, lanes 8, 4, 2 and 1 apart in turn
+    float sum[SK_COMB_CHUNKS], v[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < SK_COMB_CHUNKS; ++i) {
+      const bool has = c_s0 + i <= c_s1;
+      const float w = has ? __builtin_amdgcn_exp2f(c_ml[i].x - top) : 0.f;
+      sum[i] = has ? c_ml[i].y * w : 0.f;
+      v[0] = has ? fmaf(c_po[i].x, w, v[0]) : v[0];
+      v[1] = has ? fmaf(c_po[i].y, w, v[1]) : v[1];
+      v[2] = has ? fmaf(c_po[i].z, w, v[2]) : v[2];
+      v[3] = has ? fmaf(c_po[i].w, w, v[3]) : v[3];
+    }
+#pragma unroll
+    for (int step = SK_COMB_CHUNKS / 2; step >= 1; step >>= 1)
+#pragma unroll
+      for (int i = 0; i < step; ++i) sum[i] += sum[i + step];
+    const float inv = 1.0f / sum[0];
+    // through this wave's kilobyte of LDS into operand order (a wave's LDS operations keep their order; the kilobyte
+    // is the wave's partial sums afterwards)
+    bf16_t* turn = (bf16_t*)(smem + wave * 256);
+    *(uint2*)(turn + 4 * lane) = make_uint2(f2bf(v[0] * inv) | ((uint32_t)f2bf(v[1] * inv) << 16), f2bf(v[2] * inv) | ((uint32_t)f2bf(v[3] * inv) << 16));
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s)
+      xb[s] = row == 0 ? *(const uint4*)(turn + half * (STEPS * SK_KSTEP) + s * SK_KSTEP + 8 * g) : make_uint4(0, 0, 0, 0);
   }
   float4_t acc = {0.f, 0.f, 0.f, 0.f};
   if (X_FIRST) {
@@ -889,6 +956,15 @@ static int sk8_dispatch(const SkinnyArgs& a, hipStream_t stream) {
   const int nwaves = a.K / (64 * steps);
   dim3 grid((a.N + 7) / 8), block(nwaves * TS_WAVE);
   const size_t smem = sizeof(float) * 256 * nwaves;
+  if (a.x_packed8 == 2) {
+    if constexpr (sizeof(OUT) == 2) {
+      if (steps != 4 || nwaves > 8 || a.M != 1 || SkinnyParts(a).splits > SK_COMB_CHUNKS) return TS_BAD_SHAPE;
+      gemm_skinny8_kernel<4, 512, OUT, NEXT, true><<<grid, block, smem, stream>>>(a);
+      return ts_check_launch();
+    } else {
+      return TS_BAD_SHAPE;
+    }
+  }
   if (steps == 4) gemm_skinny8_kernel<4, 512, OUT, NEXT><<<grid, block, smem, stream>>>(a);
   else if (steps == 8) gemm_skinny8_kernel<8, 512, OUT, NEXT><<<grid, block, smem, stream>>>(a);
   else if (nwaves <= 8) gemm_skinny8_kernel<16, 512, OUT, NEXT><<<grid, block, smem, stream>>>(a);
@@ -910,16 +986,32 @@ static bool sk_next_ok(const void* next_res, const void* next_nw, const void* ne
 // hip.pack_weight8(W) for this K, ldw unused, N a multiple of 8. With next_nw (EPI_NEXT; bfloat16 only)
 // y is not written: next_res_out, next_op [M, N] and ssq_out [M, (N + 7) / 8] are. x_packed8: x is given in
 // the order the lanes read it (SkinnyArgs::x_packed8; K / 8 16-byte pieces of 64 lanes, whatever M), ldx unused.
+// comb_o (x null, M = 1, bfloat16 out, K a multiple of 256 up to 2,048): x is made on the way in from the split-key
+// attention kernel's parts (SkinnyParts; comb_hd a multiple of 32 that divides K, up to 16 chunks).
 extern "C" int ts_gemm_skinny8_bf16(void* y, const void* x, const void* w, int M, int N, int K, int64_t ldx, int64_t ldw,
                                     int64_t ldy, int out_dtype, int packed, const void* next_res, const void* next_nw,
-                                    void* next_res_out, void* next_op, void* ssq_out, int x_packed8, hipStream_t stream) {
+                                    void* next_res_out, void* next_op, void* ssq_out, int x_packed8, const float* comb_o,
+                                    const float* comb_ml, const int32_t* comb_pos, int comb_splits, int comb_chunk,
+                                    int comb_window, int comb_hd, hipStream_t stream) {
   if (M <= 0 || N <= 0) return TS_OK;
+  if (comb_o) {
+    if (x || x_packed8 || M != 1 || out_dtype != 1 || !comb_ml || !comb_pos || comb_splits < 1 || comb_splits > SK_COMB_CHUNKS ||
+        comb_chunk <= 0 || comb_hd <= 0 || comb_hd % 32 || K % comb_hd || K % 256 || K > 2048 ||
+        ((((uintptr_t)comb_o) | ((uintptr_t)comb_ml)) & 15))
+      return TS_BAD_SHAPE;
+    ldx = K;
+  }
   if (M > 8 || K <= 0 || (!x_packed8 && (ldx % 8 || ldx < K)) || (!packed && (ldw % 8 || ldw < K)) || (packed && N % 8)) return TS_BAD_SHAPE;
   if (((uintptr_t)x | (uintptr_t)w) & 15) return TS_BAD_SHAPE;
   SkinnyArgs a = {};
   a.x = (const bf16_t*)x; a.w = (const bf16_t*)w; a.y = y; a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldw = ldw; a.ldy = ldy;
   a.packed = packed;
   a.x_packed8 = x_packed8 != 0;
+  if (comb_o) {                                         // (see SkinnyParts)
+    a.x_packed8 = 2;
+    a.x = (const bf16_t*)comb_o; a.ssq_in = comb_ml; a.positions = comb_pos;
+    a.nh = comb_splits; a.nkv = comb_chunk; a.rotate = comb_window; a.hd = comb_hd;
+  }
   if (next_nw) {
     if (out_dtype != 1 || !sk_next_ok(next_res, next_nw, next_res_out, next_op, ssq_out)) return TS_BAD_SHAPE;
     a.next_res = (const bf16_t*)next_res; a.next_nw = (const bf16_t*)next_nw; a.next_res_out = (bf16_t*)next_res_out;

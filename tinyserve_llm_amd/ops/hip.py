@@ -51,7 +51,8 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_copy_slots": [p, i64, i64, i64, i, i, p],
         "ts_paged_attention_wave": [p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i64, i, f, i, i, i, p],
         "ts_paged_attention_decode": [p, p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, i, i, i, f,
-                                      i, i, p],
+                                      i, i, i, p],
+        "ts_attention_combine": [p, p, p, p, i, i, i, i, i, i, p],
         "ts_gemm_exact": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_sample": [p, p, p, p, p, p, u64, i, i, i64, p],
         "ts_sample_static": [p, p, p, p, u64, i, i, i64, p],
@@ -64,7 +65,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_gemm_library_choices": [p, i],
         "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, i, i, i, i, p, p, i, p],
         "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p, i, p, p, p, p, p, i, p],
-        "ts_gemm_skinny8_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p, p, p, p, p, i, p],
+        "ts_gemm_skinny8_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p, p, p, p, p, i, p, p, p, i, i, i, i, p],
         "ts_gemm_rows64_bf16": [p, p, p, i, i, i, i64, i64, i, i, p, i, f, p],
         "ts_gemm_rows64_sliced_bf16": [p, p, p, p, i, i, i, i64, i, p, p, p, p, p, i64, p],
         "ts_gemm_rows64_sliced_rope_bf16": [p, p, p, p, i, i, i64, i, p, i, f, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64,
@@ -345,11 +346,14 @@ def decode_kernel_takes(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
 def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                            seq_of_token: torch.Tensor, positions: torch.Tensor, scale: float, window: int = 0,
                            chunk: int | None = None, waves: int | None = None,
-                           out: torch.Tensor | None = None, pages_per_entry: int = 1) -> torch.Tensor:
+                           out: torch.Tensor | None = None, pages_per_entry: int = 1,
+                           leave_split: bool = False) -> "torch.Tensor | SplitAttention":
     """Split-key attention on the matrix cores for tokens that each bring one query (bfloat16,
     values in transposed pages). Every position in `positions` must lie inside the pages its row
     of `block_tables` has (checked by the caller on the host). `out`, if given, receives the result.
-    `pages_per_entry`: as for `paged_attention_wave`."""
+    `pages_per_entry`: as for `paged_attention_wave`. `leave_split`: where the keys are walked in
+    2 to `SPLIT_ATTENTION_MAX_CHUNKS` chunks, the chunks' parts come back uncombined (a
+    `SplitAttention`), for the projection that reads them."""
     _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions)
     _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
     T, nh, hd = q.shape
@@ -375,13 +379,53 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     if splits > 1:
         part_o = torch.empty((T, nh, splits, hd), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T, nh, splits, 2), dtype=torch.float32, device=q.device)
-    out = _out_like(q, out)
+    leave_split = leave_split and out is None and 1 < splits <= SPLIT_ATTENTION_MAX_CHUNKS
+    out = None if leave_split else _out_like(q, out)
     _run("paged_attention_decode", library().ts_paged_attention_decode(
         _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
         _ptr(seq_of_token), _ptr(positions), T, nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3],
         v_cache.stride(0), v_cache.stride(2), v_cache.stride(3), block_tables.shape[1], splits, chunk, waves,
-        float(scale), int(window), _page_run(pages_per_entry), _stream()))
-    return out
+        float(scale), int(window), _page_run(pages_per_entry), int(not leave_split), _stream()))
+    return SplitAttention(part_o, part_ml, positions, chunk, int(window)) if leave_split else out
+
+
+SPLIT_ATTENTION_MAX_CHUNKS = 16    # chunks that the 8-row form adds up on its way in
+SPLIT_ATTENTION_MAX_K = 2048       # widest attention output it makes that way (a wave's 256 k through its kilobyte of LDS, 8 waves)
+
+
+class SplitAttention:
+    """What the split-key attention kernel leaves when it is told not to combine: `parts` [tokens, heads,
+    chunks, head_dim] float32, a chunk's weighted values, and `sums` [tokens, heads, chunks, 2] float32, its
+    running maximum (in units of log2) and its sum; `positions` [tokens], `chunk` keys a chunk and `window`
+    say which chunks hold keys a token sees. The attention output is sum_s parts_s 2^(m_s - M) / sum_s l_s
+    2^(m_s - M): `combined()` makes it with the combining kernel, `gemm_skinny8` makes it on its way in for a
+    single token, bit for bit the same. `linear` decides which; nothing else takes it."""
+
+    def __init__(self, parts: torch.Tensor, sums: torch.Tensor, positions: torch.Tensor, chunk: int, window: int) -> None:
+        self.parts, self.sums, self.positions, self.chunk, self.window = parts, sums, positions, chunk, window
+
+    @property
+    def shape(self) -> tuple[int, int]:
+        tokens, heads, _, hd = self.parts.shape
+        return (tokens, heads * hd)
+
+    def combined(self) -> torch.Tensor:
+        """The attention output [tokens, heads * head_dim] in bfloat16."""
+        tokens, heads, chunks, hd = self.parts.shape
+        out = torch.empty((tokens, heads * hd), dtype=torch.bfloat16, device=self.parts.device)
+        _run("attention_combine", library().ts_attention_combine(
+            _ptr(out), _ptr(self.parts), _ptr(self.sums), _ptr(self.positions), tokens, heads, hd, chunks, self.chunk,
+            self.window, _stream()))
+        return out
+
+
+def split_attention_fuses(rows: int, weight: torch.Tensor) -> bool:
+    """Whether the 8-row form multiplies `weight` by the attention output of `rows` tokens that it adds up from the
+    chunks' parts itself: one token (every workgroup of the projection adds up all of it), over a reduction of up
+    to 2,048."""
+    return (rows == 1 and weight.is_cuda and weight.dtype == torch.bfloat16 and weight.dim() == 2
+            and weight.is_contiguous() and weight.data_ptr() % 16 == 0
+            and weight.shape[1] % 256 == 0 and weight.shape[1] <= SPLIT_ATTENTION_MAX_K)
 
 
 def gemm_exact(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
@@ -617,10 +661,11 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
 
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx, space: int,
-                    scale: float, window: int = 0) -> torch.Tensor:
+                    scale: float, window: int = 0, leave_split: bool = False) -> "torch.Tensor | SplitAttention":
     """Attention of a packed step over the cache; picks the kernel for the storage type and shape.
     float32 always takes the one-wave-per-row kernel, whose sums do not depend on the batch;
-    bfloat16 takes the matrix-core kernels where they serve the shape."""
+    bfloat16 takes the matrix-core kernels where they serve the shape. `leave_split`: a step of single
+    tokens whose keys are walked in chunks may come back as a `SplitAttention` (see `paged_attention_decode`)."""
     tables = ctx.block_tables[space]
     # (the tables count in pages of ctx.page_size tokens; the pools may be cut into shorter ones)
     table_page = getattr(ctx, "page_size", 0) or k_cache.shape[1]
@@ -631,7 +676,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         decode_ok = -(-capacity // 1024) <= MAX_DECODE_SPLITS and q.shape[0] <= MAX_DECODE_TOKENS
         if ctx.max_query_len == 1 and decode_ok:
             return paged_attention_decode(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, window,
-                                          pages_per_entry=per_entry)
+                                          pages_per_entry=per_entry, leave_split=leave_split)
         # the one-token requests that lead the step go to the split-key kernel, the rest to the tiles
         cu = ctx.host_cu_seqlens
         lead = 0
@@ -852,17 +897,29 @@ def pack_weight8(weight: torch.Tensor) -> torch.Tensor:
             .view(tiles, waves, steps, 64, 8))
 
 
-def gemm_skinny8(x: "torch.Tensor | PackedRows8", weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
+def gemm_skinny8(x: "torch.Tensor | PackedRows8 | SplitAttention", weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
                  packed8: torch.Tensor | None = None, next_norm=None) -> "torch.Tensor | PreparedNorm":
     """bfloat16 x [M <= 8, K] · weight [N, K]^T by the weight-streaming kernel's 8-row form (a matrix
     instruction multiplies 8 rows of W by 8 rows of x over 64 k; a workgroup owns 8 rows of W).
     x may come as a `PackedRows8` made for this K. With `packed8` (= pack_weight8(weight)) the kernel
     reads that copy. With `next_norm` = (residual or None, weight of the norm that follows) the product
-    is not stored: a `PreparedNorm` comes back."""
+    is not stored: a `PreparedNorm` comes back. x may also be a `SplitAttention` that `split_attention_fuses`
+    allows: the kernel then adds up the chunks' parts on its way in (bfloat16 out)."""
     x_packed = isinstance(x, PackedRows8)
-    xt = x.data if x_packed else x
+    split = x if isinstance(x, SplitAttention) else None
+    xt = x.data if x_packed else x.parts if split is not None else x
     _gpu(xt, weight, packed8)
-    _need(xt.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "gemm_skinny8 takes bfloat16")
+    if split is not None:
+        _gpu(split.sums, split.positions)
+        tokens, heads, chunks, hd = split.parts.shape
+        _need(split_attention_fuses(tokens, weight) and chunks <= SPLIT_ATTENTION_MAX_CHUNKS and hd % 32 == 0
+              and out_dtype == torch.bfloat16
+              and split.parts.dtype == torch.float32 and split.parts.is_contiguous() and split.sums.is_contiguous()
+              and split.sums.shape == (tokens, heads, chunks, 2) and split.sums.dtype == torch.float32
+              and split.positions.dtype == torch.int32 and split.positions.shape == (tokens,) and split.positions.is_contiguous()
+              and split.parts.data_ptr() % 16 == 0 and split.sums.data_ptr() % 16 == 0,
+              lambda: f"gemm_skinny8 does not take these parts: {tuple(split.parts.shape)} against {tuple(weight.shape)}")
+    _need((split is not None or xt.dtype == torch.bfloat16) and weight.dtype == torch.bfloat16, "gemm_skinny8 takes bfloat16")
     _need(len(x.shape) == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
           lambda: f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T")
     M, K = x.shape
@@ -872,9 +929,12 @@ def gemm_skinny8(x: "torch.Tensor | PackedRows8", weight: torch.Tensor, out_dtyp
           "8192 or of 1024 up to 16384")
     if x_packed:
         _need(x.steps == steps and xt.is_contiguous() and xt.numel() == 8 * K, lambda: f"the packed rows were made for a reader of {x.steps} steps, not {steps}")
-    _need((x_packed or _dense_rows(xt)) and weight.is_contiguous() and xt.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0,
+    _need((x_packed or split is not None or _dense_rows(xt)) and weight.is_contiguous() and xt.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0,
           "rows must be dense and 16-byte aligned")
-    ldx = K if x_packed else xt.stride(0)
+    ldx = K if x_packed or split is not None else xt.stride(0)
+    comb = ((_ptr(split.parts), _ptr(split.sums), _ptr(split.positions), split.parts.shape[2], split.chunk, split.window,
+             split.parts.shape[3]) if split is not None else (None, None, None, 0, 0, 0, 0))
+    x_arg = None if split is not None else _ptr(xt)
     _need(out_dtype in (torch.bfloat16, torch.float32), "the result is bfloat16 or float32")
     if packed8 is not None:
         _need(packed8.dtype == torch.bfloat16 and packed8.shape == (-(-N // 8), K // (64 * steps), steps, 64, 8)
@@ -884,14 +944,14 @@ def gemm_skinny8(x: "torch.Tensor | PackedRows8", weight: torch.Tensor, out_dtyp
         _need(out_dtype == torch.bfloat16, "a prepared norm comes with bfloat16")
         prepared, residual, nw = _next_norm_outputs(xt, N, -(-N // 8), next_norm, rows=M)
         _run("gemm_skinny8", library().ts_gemm_skinny8_bf16(
-            None, _ptr(xt), _ptr(weight if packed8 is None else packed8), M, N, K, ldx, weight.stride(0), N, 1,
+            None, x_arg, _ptr(weight if packed8 is None else packed8), M, N, K, ldx, weight.stride(0), N, 1,
             int(packed8 is not None), _ptr(residual), _ptr(nw), _ptr(prepared.summed), _ptr(prepared.operand),
-            _ptr(prepared.squares), int(x_packed), _stream()))
+            _ptr(prepared.squares), int(x_packed), *comb, _stream()))
         return prepared
     out = torch.empty((M, N), dtype=out_dtype, device=xt.device)
     _run("gemm_skinny8", library().ts_gemm_skinny8_bf16(
-        _ptr(out), _ptr(xt), _ptr(weight if packed8 is None else packed8), M, N, K, ldx, weight.stride(0),
-        out.stride(0), _code(out_dtype), int(packed8 is not None), None, None, None, None, None, int(x_packed), _stream()))
+        _ptr(out), x_arg, _ptr(weight if packed8 is None else packed8), M, N, K, ldx, weight.stride(0),
+        out.stride(0), _code(out_dtype), int(packed8 is not None), None, None, None, None, None, int(x_packed), *comb, _stream()))
     return out
 
 

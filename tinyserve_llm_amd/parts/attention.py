@@ -113,5 +113,9 @@ class Attention(Mixer):
             qkv = linear(x, self.qkv, packed=self.qkv_packed)
             q = hip.rope_store(qkv, table, ctx.positions, slots, k_store, v_store, self.num_heads, self.num_kv_heads,
                                self.head_dim)
-        o = hip.paged_attention(q, mem.k_cache, mem.v_cache, ctx, mem.space, self.scale, self.window)
-        return linear(o.view(ctx.num_tokens, self.q_size), self.o, packed=self.o_packed, then=then)
+        # (a single token: the o projection adds the chunks of a split walk up itself, on its way in)
+        o = hip.paged_attention(q, mem.k_cache, mem.v_cache, ctx, mem.space, self.scale, self.window,
+                                leave_split=hip.split_attention_fuses(ctx.num_tokens, self.o))
+        if not isinstance(o, hip.SplitAttention):
+            o = o.view(ctx.num_tokens, self.q_size)
+        return linear(o, self.o, packed=self.o_packed, then=then)

@@ -81,7 +81,7 @@ def streaming_copy(weight: torch.Tensor) -> hip.StreamingCopies | None:
 PACKED_ROWS_MIN = 2      # rows from which a gated product is handed on in the 8-row form's order (one row is read whole anyway)
 
 
-def linear(x: "torch.Tensor | DeferredNorm | hip.PackedRows8", weight: torch.Tensor, out_dtype: torch.dtype | None = None,
+def linear(x: "torch.Tensor | DeferredNorm | hip.PackedRows8 | hip.SplitAttention", weight: torch.Tensor, out_dtype: torch.dtype | None = None,
            glu: bool = False, packed: hip.StreamingCopies | None = None,
            then: NormRequest | None = None, feeds: torch.Tensor | None = None) -> "torch.Tensor | DeferredNorm | hip.PackedRows8":
     """x · Wᵀ; with `glu`, W holds gate rows then up rows and silu(gate) * up comes back.
@@ -90,7 +90,20 @@ def linear(x: "torch.Tensor | DeferredNorm | hip.PackedRows8", weight: torch.Ten
     kernel where it can be, left to the next projection otherwise. `feeds` (with `glu`): the weight of
     the projection that alone reads this product; where that projection's kernel reads its operand
     faster in an order of its own, the product comes back in that order (a `hip.PackedRows8`), to be
-    handed to `linear` with that weight and to nothing else."""
+    handed to `linear` with that weight and to nothing else. x may be a `hip.SplitAttention` (an attention output
+    still in its chunks' parts): the 8-row form adds the parts up on its way in where it can, the combining
+    kernel does otherwise."""
+    if isinstance(x, hip.SplitAttention):
+        residual = then.residual() if then is not None else None
+        if (not glu and out_dtype in (None, torch.bfloat16) and hip.split_attention_fuses(x.shape[0], weight)
+                and (then is None or (then.weight.dtype == torch.bfloat16
+                                      and (residual is None or (residual.is_contiguous() and residual.dtype == torch.bfloat16))))):
+            by8 = None if packed is None else packed.by8
+            if then is None:
+                return hip.gemm_skinny8(x, weight, torch.bfloat16, by8)
+            prepared = hip.gemm_skinny8(x, weight, torch.bfloat16, by8, next_norm=(residual, then.weight))
+            return DeferredNorm(None, None, then.weight, then.eps, prepared)
+        x = x.combined()
     if isinstance(x, hip.PackedRows8) and (glu or hip.rows8_reader_steps(x.shape[0], weight) != x.steps):
         x = x.rows()
     if isinstance(x, hip.PackedRows8) and then is None:
