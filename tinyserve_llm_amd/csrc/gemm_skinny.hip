@@ -718,6 +718,9 @@ static int sk_launch(const SkinnyArgs& a, hipStream_t stream) {
 // Picks the instance: slices of 256 k while that needs at most 16 waves, else slices of 512; more
 // rows of W per workgroup for wide matrices once that still leaves a workgroup per compute unit
 // (fewer workgroups repeat less of the work on x).
+#ifndef SK_GLU_SMALL_ROWS
+#define SK_GLU_SMALL_ROWS 4
+#endif
 template <int MODE, int EPI, typename OUT>
 static int sk_dispatch(const SkinnyArgs& a, hipStream_t stream) {
   constexpr bool GLU = EPI == EPI_GLU, NORM = MODE == MODE_NORM;
@@ -738,7 +741,10 @@ static int sk_dispatch(const SkinnyArgs& a, hipStream_t stream) {
       if (cb > 2) SK_GO(2, 4, 8);
     }
     if (nwaves <= 8) {
-      if (ncols >= 4096 * (GLU ? 1 : 2)) SK_GO(4, 1, 8);
+      // (the gate for up to four rows of x: 512 workgroups of two row tiles stream faster than 256 of four, which
+      //  repeat less of the work on x with more rows: a decode step at batch 1 0.747 -> 0.741 ms, at batch 4
+      //  0.819 -> 0.816, at batch 6 0.837 -> 0.840)
+      if (ncols >= 4096 * (GLU ? (a.M <= SK_GLU_SMALL_ROWS ? 4 : 1) : 2)) SK_GO(4, 1, 8);
       if (GLU || ncols >= 4096) SK_GO(2, 1, 8);
     }
     if constexpr (!GLU) SK_GO(1, 1, 8);
